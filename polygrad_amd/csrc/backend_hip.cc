@@ -1,0 +1,241 @@
+// backend_hip: the C ABI of the backend -- the PolyBackendDesc row (lower_item /
+// execute / free_runner / get_allocator), the allocator, the runtime wrappers
+// and the render-only entry points.  Declarations and the reference interfaces
+// they replace are in include/polygrad_hip.h.
+#include <cstdlib>
+#include <cstring>
+
+#include "polygrad_hip.h"
+#include "runtime_hip.h"
+
+namespace polyhip {
+
+static RenderOptions options_from_flags(int flags) {
+  RenderOptions o;
+  if (flags & 1) o.allow_templates = false;
+  if (flags & 2) o.allow_vectorize = false;
+  if (flags & 4) o.allow_coop_reduce = false;
+  if (const char *e = getenv("POLY_HIP_NO_TEMPLATES")) if (*e == '1') o.allow_templates = false;
+  return o;
+}
+
+static bool render_root(const PolyUOp *root, const char *fn_name, int flags, RenderedKernel *rk) {
+  KernelGraph g;
+  if (!g.build(root)) { log_err("render_hip", "%s: %s", fn_name, g.error.c_str()); return false; }
+  std::string err;
+  if (!render_kernel(g, "poly_k", options_from_flags(flags), rk, &err)) {
+    log_err("render_hip", "%s: %s", fn_name, err.c_str());
+    return false;
+  }
+  return true;
+}
+
+HipRunner *runner_create(const PolyUOp *root, const char *fn_name, int flags) {
+  if (runtime_init() != 0) return nullptr;
+  HipRunner *r = new HipRunner();
+  r->name = fn_name ? fn_name : "kernel";
+  if (!render_root(root, r->name.c_str(), flags, &r->rk)) { delete r; return nullptr; }
+  r->main = program_create(r->rk.source, r->rk.entry);
+  if (!r->main) { runner_destroy(r); return nullptr; }
+  if (!r->rk.guards.empty()) {
+    r->flag = runtime_alloc(sizeof(int));
+    if (!r->flag) { runner_destroy(r); return nullptr; }
+    for (const RenderedKernel::Guard &gd : r->rk.guards) {
+      Program *p = program_create(gd.source, gd.entry);
+      if (!p) { runner_destroy(r); return nullptr; }
+      r->guards.push_back(p);
+    }
+    r->fallback = program_create(r->rk.fallback_source, r->rk.fallback_entry);
+    if (!r->fallback) { runner_destroy(r); return nullptr; }
+  }
+  size_t n = (size_t)r->rk.n_params + (size_t)r->rk.n_vars + 1;
+  r->ptr_store.resize(n);
+  r->var_store.resize(n);
+  r->arg_ptrs.resize(n);
+  return r;
+}
+
+void runner_destroy(HipRunner *r) {
+  if (!r) return;
+  if (r->main) program_destroy(r->main);
+  for (Program *p : r->guards) program_destroy(p);
+  if (r->fallback) program_destroy(r->fallback);
+  if (r->flag) runtime_free(r->flag);
+  delete r;
+}
+
+int runner_launch(HipRunner *r, void **args, int n_args) {
+  const int np = r->rk.n_params, nv = r->rk.n_vars;
+  if (n_args < np + nv) {
+    log_err("execute", "%s: expected %d args, got %d", r->name.c_str(), np + nv, n_args);
+    return -1;
+  }
+  for (int i = 0; i < np; i++) {
+    if (!args[i]) { log_err("execute", "%s: null buffer for param %d", r->name.c_str(), i); return -1; }
+    r->ptr_store[(size_t)i] = args[i];
+    r->arg_ptrs[(size_t)i] = &r->ptr_store[(size_t)i];
+  }
+  // DEFINE_VAR values arrive as pointers to host ints; kernels take them by value.
+  for (int v = 0; v < nv; v++) {
+    if (!args[np + v]) { log_err("execute", "%s: null var %d", r->name.c_str(), v); return -1; }
+    r->var_store[(size_t)v] = *(const int *)args[np + v];
+    r->arg_ptrs[(size_t)(np + v)] = &r->var_store[(size_t)v];
+  }
+  if (r->guards.empty()) return program_launch(r->main, r->arg_ptrs.data(), r->rk.launch);
+  // The guard writes *flag (1 = fast path valid, 0 = not); the fast kernel and
+  // its generic twin both launch and exactly one of them does the work.
+  r->ptr_store[(size_t)(np + nv)] = r->flag;
+  r->arg_ptrs[(size_t)(np + nv)] = &r->ptr_store[(size_t)(np + nv)];
+  for (size_t gi = 0; gi < r->guards.size(); gi++) {
+    const RenderedKernel::Guard &gd = r->rk.guards[gi];
+    std::vector<void *> gargs;
+    void *flagp = r->flag;
+    gargs.push_back(&flagp);
+    std::vector<void *> vals;
+    vals.reserve(gd.arg_params.size());
+    for (int p : gd.arg_params) vals.push_back(args[p]);
+    for (size_t i = 0; i < vals.size(); i++) gargs.push_back(&vals[i]);
+    if (program_launch(r->guards[gi], gargs.data(), gd.launch) != 0) return -1;
+  }
+  if (program_launch(r->main, r->arg_ptrs.data(), r->rk.launch) != 0) return -1;
+  return program_launch(r->fallback, r->arg_ptrs.data(), r->rk.fallback_launch);
+}
+
+}  // namespace polyhip
+
+using namespace polyhip;
+
+extern "C" {
+
+int poly_hip_init(void) { return runtime_init(); }
+int poly_hip_available(void) { return runtime_init() == 0 ? 1 : 0; }
+void *poly_hip_alloc(size_t nbytes) { return runtime_alloc(nbytes); }
+void poly_hip_free(void *p) { runtime_free(p); }
+int poly_hip_copy_htod(void *dst, const void *src, size_t n) { return runtime_copy(dst, src, n, 0); }
+int poly_hip_copy_dtoh(void *dst, const void *src, size_t n) { return runtime_copy(dst, src, n, 1); }
+int poly_hip_copy_dtod(void *dst, const void *src, size_t n) { return runtime_copy(dst, src, n, 2); }
+int poly_hip_memset(void *p, int value, size_t n) { return runtime_memset(p, value, n); }
+int poly_hip_sync(void) { return runtime_sync(); }
+void *poly_hip_stream(void) { return runtime_stream(); }
+
+struct PolyHipProgram { Program *p; };
+
+PolyHipProgram *poly_hip_compile(const char *source, const char *entry) {
+  if (!source || !entry) return nullptr;
+  Program *p = program_create(source, entry);
+  if (!p) return nullptr;
+  PolyHipProgram *h = new PolyHipProgram();
+  h->p = p;
+  return h;
+}
+
+int poly_hip_launch(PolyHipProgram *prog, void **kernel_args, int n_args, unsigned gx, unsigned gy,
+                    unsigned gz, unsigned bx, unsigned by, unsigned bz, unsigned lds_bytes) {
+  (void)n_args;
+  if (!prog) return -1;
+  LaunchSpec ls;
+  ls.grid[0] = gx; ls.grid[1] = gy; ls.grid[2] = gz;
+  ls.block[0] = bx; ls.block[1] = by; ls.block[2] = bz;
+  ls.lds_bytes = lds_bytes;
+  return program_launch(prog->p, kernel_args, ls);
+}
+
+void poly_hip_program_destroy(PolyHipProgram *prog) {
+  if (!prog) return;
+  program_destroy(prog->p);
+  delete prog;
+}
+
+// ── vtable ────────────────────────────────────────────────────────────────
+
+int poly_hip_lower_item(PolyCtx *ctx, PolyUOp *scheduled_root, const char *fn_name, PolyRunner *out) {
+  (void)ctx;  // the lowering only reads the graph; it creates no UOps
+  if (!scheduled_root || !out) return -1;
+  HipRunner *r = runner_create(scheduled_root, fn_name, 0);
+  if (!r) return -1;
+  out->kind = POLY_RUNNER_COMPILED;
+  out->handle = r;
+  out->handle_size = 0;
+  for (int i = 0; i < 3; i++) { out->grid[i] = (int)r->rk.launch.grid[i]; out->block[i] = (int)r->rk.launch.block[i]; }
+  return 0;
+}
+
+int poly_hip_execute(PolyRunner *runner, void **args, int n_args) {
+  if (!runner || !runner->handle) { log_err("execute", "runner has no handle"); return -1; }
+  return runner_launch((HipRunner *)runner->handle, args, n_args);
+}
+
+void poly_hip_free_runner(PolyRunner *runner) {
+  if (!runner || !runner->handle) return;
+  runner_destroy((HipRunner *)runner->handle);
+  runner->handle = nullptr;
+}
+
+static void *alloc_fn(size_t nbytes, void *dev_ctx) { (void)dev_ctx; return runtime_alloc(nbytes); }
+static void free_fn(void *h, void *dev_ctx) { (void)dev_ctx; runtime_free(h); }
+static int copy_in_fn(void *dst, const void *src, size_t n, void *dev_ctx) { (void)dev_ctx; return runtime_copy(dst, src, n, 0); }
+static int copy_out_fn(void *dst, const void *src, size_t n, void *dev_ctx) { (void)dev_ctx; return runtime_copy(dst, src, n, 1); }
+static int copy_between_fn(void *dst, const void *src, size_t n, void *dev_ctx) { (void)dev_ctx; return runtime_copy(dst, src, n, 2); }
+
+static const PolyAllocator kHipAllocator = {alloc_fn, free_fn, copy_in_fn, copy_out_fn, copy_between_fn, nullptr};
+const PolyAllocator *poly_hip_get_allocator(void) { return &kHipAllocator; }
+
+static const PolyBackendDesc kHipBackend = {"hip", POLY_DEVICE_HIP, false, poly_hip_lower_item,
+                                            poly_hip_execute, poly_hip_free_runner, poly_hip_get_allocator};
+const PolyBackendDesc *poly_hip_backend_desc(void) { return &kHipBackend; }
+
+// ── render-only entry points ──────────────────────────────────────────────
+
+static char *dup_string(const std::string &s) {
+  char *p = (char *)malloc(s.size() + 1);
+  if (p) memcpy(p, s.c_str(), s.size() + 1);
+  return p;
+}
+
+char *poly_hip_render(PolyUOp *scheduled_root, const char *fn_name, int flags, int *launch_out) {
+  RenderedKernel rk;
+  if (!scheduled_root || !render_root(scheduled_root, fn_name ? fn_name : "kernel", flags, &rk)) return nullptr;
+  if (launch_out) {
+    for (int i = 0; i < 3; i++) { launch_out[i] = (int)rk.launch.grid[i]; launch_out[3 + i] = (int)rk.launch.block[i]; }
+    launch_out[6] = (int)rk.launch.lds_bytes;
+  }
+  std::string all = rk.source;
+  for (const RenderedKernel::Guard &g : rk.guards) all += "\n// ---- guard ----\n" + g.source;
+  if (!rk.fallback_source.empty()) all += "\n// ---- fallback ----\n" + rk.fallback_source;
+  return dup_string(all);
+}
+
+char *poly_hip_describe(PolyUOp *scheduled_root, int flags) {
+  RenderedKernel rk;
+  if (!scheduled_root || !render_root(scheduled_root, "kernel", flags, &rk)) return nullptr;
+  static const char *const kn[] = {"elementwise", "row-reduce", "thread-reduce", "matmul-mfma", "gather", "copy"};
+  return dup_string(strf("%s: %s bytes=%.0f flops=%.0f grid=%u,%u,%u block=%u", kn[(int)rk.klass],
+                         rk.strategy.c_str(), rk.bytes, rk.flops, rk.launch.grid[0], rk.launch.grid[1],
+                         rk.launch.grid[2], rk.launch.block[0]));
+}
+
+int poly_hip_compile_check(const char *source) {
+  if (!source) return -1;
+  // A rendered bundle may hold several translation units (guard, fallback).
+  std::string all(source);
+  size_t pos = 0;
+  while (pos < all.size()) {
+    size_t next = all.find("\n// ---- ", pos);
+    std::string unit = all.substr(pos, next == std::string::npos ? std::string::npos : next - pos);
+    std::vector<char> code;
+    std::string log;
+    if (!compile_to_code_object(unit, &code, &log)) {
+      log_err("compile_check", "hiprtc: %s", log.c_str());
+      return -1;
+    }
+    if (next == std::string::npos) break;
+    pos = all.find('\n', next + 1);
+    if (pos == std::string::npos) break;
+    pos++;
+  }
+  return 0;
+}
+
+void poly_hip_free_string(char *s) { free(s); }
+
+}  // extern "C"

@@ -1,0 +1,617 @@
+// Generic lowering of a scheduled kernel to HIP C for gfx950.
+//
+// Three shapes of kernel come out of here:
+//   ELEMENTWISE   every END-closed range is flattened over the grid, fastest
+//                 varying range last in the thread id; when that range is
+//                 unit-stride in the store (and in a load) the access becomes one
+//                 128-bit (or 64-bit) vector access per thread.
+//   ROW_REDUCE    one wave (64 lanes) or one workgroup (256 lanes) per output
+//                 element; lanes stride over the flattened reduce ranges with
+//                 vector loads, then combine with DPP/ds_swizzle (+LDS across
+//                 the four waves of a workgroup).
+//   THREAD_REDUCE one thread per output element with serial reduce loops
+//                 (short reductions, or reductions this file cannot split).
+// Matmul-shaped and gather-shaped kernels are tried first in templates.cc.
+#include "render_hip.h"
+
+#include <algorithm>
+#include <cmath>
+#include <set>
+
+namespace polyhip {
+
+bool try_render_matmul(const KernelGraph &g, const std::string &fn, const RenderOptions &opt,
+                       RenderedKernel *out);
+bool try_render_gather(const KernelGraph &g, const std::string &fn, const RenderOptions &opt,
+                       RenderedKernel *out);
+
+namespace {
+
+struct Group {
+  std::vector<int> ranges;     // ordinals, outermost first (END order)
+  std::vector<int> stores;     // indices into g.stores
+};
+
+PolyOps reduce_op(const KNode &k) {
+  return k.u->arg.kind == POLY_ARG_OPS ? k.u->arg.ops : (PolyOps)k.u->arg.i;
+}
+
+// Extent of a range as a C expression (constant or symbolic) and as a number.
+struct Ext { int64_t n; std::string expr; };
+
+class Generic {
+ public:
+  Generic(const KernelGraph &g, const std::string &fn, const RenderOptions &opt)
+      : g_(g), fn_(fn), opt_(opt), em_(g) {}
+
+  bool run(RenderedKernel *out, std::string *err) {
+    if (!prepare(err)) return false;
+    std::string body;
+    bool coop = false;
+    if (!g_.reduces.empty() && opt_.allow_coop_reduce && groups_.size() == 1) coop = plan_coop();
+    if (coop) {
+      body = render_coop(out);
+    } else {
+      body = render_flat(out);
+    }
+    if (em_.failed()) { *err = em_.error(); return false; }
+    if (!error_.empty()) { *err = error_; return false; }
+    std::string prologue = opt_.exit_if_flag ? "  if (*poly_flag != 0) return;\n" : "";
+    out->source = std::string(hip_prelude()) + signature() + " {\n" + prologue + body + "}\n";
+    out->entry = fn_;
+    out->n_params = (int)g_.params.size();
+    out->n_vars = (int)g_.vars.size();
+    account(out);
+    return true;
+  }
+
+ private:
+  const KernelGraph &g_;
+  std::string fn_;
+  RenderOptions opt_;
+  Emitter em_;
+  std::vector<Group> groups_;
+  std::vector<int> top_reduces_;
+  std::string error_;
+  // coop plan
+  int coop_G_ = 0;
+  int64_t coop_R_ = 0;
+  std::vector<int> coop_ranges_;
+
+  std::string signature() const {
+    std::string s = strf("extern \"C\" __global__ void __launch_bounds__(%d) %s(", opt_.block, fn_.c_str());
+    bool first = true;
+    for (size_t i = 0; i < g_.params.size(); i++) {
+      const ParamInfo &p = g_.params[i];
+      if (!first) s += ", ";
+      first = false;
+      if (p.written) s += strf("%s* data%zu", dt_cname(p.dt), i);
+      else s += strf("const %s* __restrict__ data%zu", dt_cname(p.dt), i);
+    }
+    for (size_t i = 0; i < g_.vars.size(); i++) {
+      if (!first) s += ", ";
+      first = false;
+      s += strf("const int var%zu", i);
+    }
+    if (opt_.exit_if_flag) s += std::string(first ? "" : ", ") + "const int* __restrict__ poly_flag";
+    return s + ")";
+  }
+
+  bool prepare(std::string *err) {
+    for (const ParamInfo &p : g_.params)
+      if (p.numel >= ((int64_t)1 << 31)) { *err = "buffer with 2^31 or more elements"; return false; }
+    for (size_t si = 0; si < g_.stores.size(); si++) {
+      const StoreInfo &st = g_.stores[si];
+      bool placed = false;
+      for (Group &gr : groups_)
+        if (gr.ranges == st.ranges) { gr.stores.push_back((int)si); placed = true; break; }
+      if (!placed) { Group gr; gr.ranges = st.ranges; gr.stores.push_back((int)si); groups_.push_back(gr); }
+    }
+    // top-level reduces: not inside the source of another REDUCE
+    std::vector<char> inside(g_.nodes.size(), 0);
+    for (int i = (int)g_.nodes.size() - 1; i >= 0; i--) {
+      const KNode &k = g_.n(i);
+      bool in = inside[(size_t)i];
+      if (k.op == POLY_OP_REDUCE) inside[(size_t)k.src[0]] = 1;
+      if (in) for (int s : k.src) inside[(size_t)s] = 1;
+    }
+    for (int r : g_.reduces) if (!inside[(size_t)r]) top_reduces_.push_back(r);
+    return true;
+  }
+
+  Ext extent(int ord, Scope *s) {
+    const RangeInfo &r = g_.ranges[(size_t)ord];
+    if (r.extent >= 0) return {r.extent, strf("%lld", (long long)r.extent)};
+    return {-1, em_.emit(r.bound_node, s)};
+  }
+
+  // Orders a group's ranges fastest-first using the first store's index strides.
+  std::vector<int> fastest_first(const Group &gr) const {
+    const StoreInfo &st = g_.stores[(size_t)gr.stores[0]];
+    int li = g_.n(g_.n(st.index).src[1]).lin;
+    std::vector<std::pair<int64_t, int>> keyed;
+    int pos = 0;
+    for (auto it = gr.ranges.rbegin(); it != gr.ranges.rend(); ++it, ++pos) {
+      int64_t key = (int64_t)1 << 50;  // unknown stride: keep END order (inner = fast)
+      if (li >= 0) {
+        bool aff;
+        int64_t c = g_.lin_range_coef(g_.lins[(size_t)li], *it, &aff);
+        if (aff && c != 0) key = c < 0 ? -c : c;
+        else if (aff && c == 0) key = ((int64_t)1 << 55);
+      }
+      keyed.push_back({key * 64 + pos, *it});
+    }
+    std::sort(keyed.begin(), keyed.end());
+    std::vector<int> order;
+    for (auto &k : keyed) order.push_back(k.second);
+    return order;
+  }
+
+  // Can `lin` be accessed as a V-wide vector along range `F`?  Needs unit stride
+  // in F and every other contribution a multiple of V (keeps the natural
+  // alignment of the vector type).
+  bool vec_ok(const Lin &l, int F, int V) const {
+    if (l.c0 % V) return false;
+    bool seenF = false;
+    for (const Term &t : l.terms) {
+      const Atom &a = g_.atoms[(size_t)t.atom];
+      if (a.kind == Atom::RANGE && g_.range_ord.at(a.node) == F) {
+        if (t.coef != 1) return false;
+        seenF = true;
+      } else {
+        if (g_.atom_deps(t.atom) & ((uint64_t)1 << F)) return false;
+        if (t.coef % V) return false;
+        if (a.kind == Atom::VAR || a.kind == Atom::OPAQUE) {
+          // symbolic values: only fine when the coefficient already carries V
+        }
+      }
+    }
+    return seenF;
+  }
+
+  bool node_under(int root, std::vector<char> &mark) const {
+    // marks every node reachable from root
+    std::vector<int> st{root};
+    while (!st.empty()) {
+      int n = st.back(); st.pop_back();
+      if (mark[(size_t)n]) continue;
+      mark[(size_t)n] = 1;
+      for (int s : g_.n(n).src) st.push_back(s);
+    }
+    return true;
+  }
+
+  // Emits vector loads (hoisted out of the unrolled loop) for every LOAD under
+  // `roots` that is unit-stride along F; returns the preset nodes.
+  std::vector<int> hoist_vector_loads(const std::vector<int> &roots, int F, int V, const std::string &f0,
+                                      Scope *outer, bool skip_inside_reduce) {
+    std::vector<char> mark(g_.nodes.size(), 0);
+    for (int r : roots) node_under(r, mark);
+    std::vector<int> done;
+    for (int i = 0; i < (int)g_.nodes.size(); i++) {
+      if (!mark[(size_t)i]) continue;
+      const KNode &k = g_.n(i);
+      if (k.op != POLY_OP_LOAD) continue;
+      if (!(k.deps & ((uint64_t)1 << F))) continue;
+      // loads that also depend on ranges not bound in `outer` (nested serial
+      // reduces) stay scalar
+      if (k.deps & ~(outer->avail | ((uint64_t)1 << F))) continue;
+      (void)skip_inside_reduce;
+      const KNode &ix = g_.n(k.src[0]);
+      int li = g_.n(ix.src[1]).lin;
+      if (li < 0 || !vec_ok(g_.lins[(size_t)li], F, V)) continue;
+      if (ix.src.size() >= 3 && (g_.n(ix.src[2]).deps & ((uint64_t)1 << F))) continue;
+      if (k.guard >= 0 && (g_.n(k.guard).deps & ((uint64_t)1 << F))) continue;
+      if (dt_size(k.dt) * V > 16) continue;
+      int p = g_.param_slot(ix.src[0]);
+      em_.bind_range(F, f0);
+      std::string addr = em_.emit_lin(g_.lins[(size_t)li], outer);
+      std::string name = strf("ld%d", i);
+      std::string ld = strf("poly_vload<%s,%d>(data%d + %s)", dt_cname(k.dt), V, p, addr.c_str());
+      std::string gate;
+      if (ix.src.size() >= 3) gate = em_.emit(ix.src[2], outer);
+      if (k.guard >= 0) {
+        std::string g2 = em_.emit(k.guard, outer);
+        if (k.guard_neg) g2 = "(!" + g2 + ")";
+        gate = gate.empty() ? g2 : "(" + gate + "&&" + g2 + ")";
+      }
+      if (!gate.empty()) ld = strf("(%s ? %s : poly_vec<%s,%d>{})", gate.c_str(), ld.c_str(), dt_cname(k.dt), V);
+      outer->code.append((size_t)outer->indent * 2, ' ');
+      outer->code += strf("const poly_vec<%s,%d> %s = %s;\n", dt_cname(k.dt), V, name.c_str(), ld.c_str());
+      em_.preset(i, name + ".v[u]");
+      done.push_back(i);
+    }
+    return done;
+  }
+
+  static void line(std::string &code, int indent, const std::string &s) {
+    code.append((size_t)indent * 2, ' ');
+    code += s;
+    code += "\n";
+  }
+
+  // ── flat: one thread per (vector of) output element(s) ───────────────────
+  std::string render_flat(RenderedKernel *out) {
+    std::string body;
+    line(body, 1, "const long long gid = (long long)blockIdx.x * blockDim.x + threadIdx.x;");
+    double max_threads = 1;
+    bool dynamic = false;
+    bool any_reduce = !g_.reduces.empty();
+    std::string strat;
+    for (size_t gi = 0; gi < groups_.size(); gi++) {
+      const Group &gr = groups_[gi];
+      std::vector<int> order = fastest_first(gr);
+      Scope S0;
+      S0.indent = 2;
+      for (int r : gr.ranges) S0.avail |= (uint64_t)1 << r;
+      int V = 1;
+      int F = order.empty() ? -1 : order[0];
+      // choose a vector width from the stores of the group
+      if (opt_.allow_vectorize && !any_reduce && F >= 0 && g_.ranges[(size_t)F].extent > 0) {
+        int v0 = 8;
+        for (int si : gr.stores) {
+          const StoreInfo &st = g_.stores[(size_t)si];
+          v0 = std::min(v0, 16 / std::max(1, dt_size(g_.n(st.value).dt)));
+        }
+        for (int v = v0; v >= 2; v /= 2) {
+          bool ok = g_.ranges[(size_t)F].extent % v == 0;
+          for (int si : gr.stores) {
+            const StoreInfo &st = g_.stores[(size_t)si];
+            int li = g_.n(g_.n(st.index).src[1]).lin;
+            if (li < 0 || !vec_ok(g_.lins[(size_t)li], F, v)) ok = false;
+            if (st.gate >= 0 && (g_.n(st.gate).deps & ((uint64_t)1 << F))) ok = false;
+            if (dt_size(g_.n(st.value).dt) != dt_size(g_.n(st.param).dt)) ok = false;
+          }
+          if (ok) { V = v; break; }
+        }
+      }
+      // thread count of this group
+      std::string nthreads = "1";
+      double nthreads_n = 1;
+      std::string decomp;
+      line(decomp, 2, "long long t_ = gid;");
+      for (size_t oi = 0; oi < order.size(); oi++) {
+        int ord = order[oi];
+        Ext e = extent(ord, &S0);
+        std::string rv = strf("r%d", ord);
+        if (e.n < 0) dynamic = true;
+        if (oi == 0 && V > 1) {
+          int64_t nv = e.n / V;
+          line(decomp, 2, strf("const int %s_0 = (int)(t_ %% %lld) * %d; t_ /= %lld;", rv.c_str(), (long long)nv, V, (long long)nv));
+          nthreads += strf("*%lldll", (long long)nv);
+          nthreads_n *= (double)nv;
+        } else {
+          if (oi + 1 == order.size())
+            line(decomp, 2, strf("const int %s = (int)t_;", rv.c_str()));
+          else
+            line(decomp, 2, strf("const int %s = (int)(t_ %% %s); t_ /= %s;", rv.c_str(), e.expr.c_str(), e.expr.c_str()));
+          nthreads += "*(long long)" + e.expr;
+          nthreads_n *= e.n < 0 ? 1.0 : (double)e.n;
+          em_.bind_range(ord, rv);
+        }
+      }
+      max_threads = std::max(max_threads, nthreads_n);
+      std::string sect;
+      if (V > 1) {
+        std::string f0 = strf("r%d_0", F);
+        std::vector<int> roots;
+        for (int si : gr.stores) roots.push_back(g_.stores[(size_t)si].value);
+        Scope outer = S0;
+        outer.avail &= ~((uint64_t)1 << F);
+        outer.code.clear();
+        std::vector<int> pres = hoist_vector_loads(roots, F, V, f0, &outer, false);
+        Scope inner;
+        inner.parent = &outer;
+        inner.avail = outer.avail | ((uint64_t)1 << F);
+        inner.indent = 3;
+        em_.bind_range(F, strf("r%d", F));
+        std::string stores_code;
+        for (int si : gr.stores) {
+          const StoreInfo &st = g_.stores[(size_t)si];
+          std::string v = em_.emit(st.value, &inner);
+          line(inner.code, 3, strf("out%d.v[u] = %s;", si, v.c_str()));
+        }
+        std::string pre;
+        for (int si : gr.stores) {
+          const StoreInfo &st = g_.stores[(size_t)si];
+          line(pre, 2, strf("poly_vec<%s,%d> out%d;", dt_cname(g_.n(st.param).dt), V, si));
+        }
+        std::string post;
+        for (int si : gr.stores) {
+          const StoreInfo &st = g_.stores[(size_t)si];
+          int li = g_.n(g_.n(st.index).src[1]).lin;
+          em_.bind_range(F, f0);
+          std::string addr = em_.emit_lin(g_.lins[(size_t)li], &outer);
+          int p = g_.param_slot(st.param);
+          std::string stmt = strf("poly_vstore<%s,%d>(data%d + %s, out%d);", dt_cname(g_.n(st.param).dt), V, p, addr.c_str(), si);
+          if (st.gate >= 0) stmt = "if (" + em_.emit(st.gate, &outer) + ") " + stmt;
+          line(post, 2, stmt);
+        }
+        sect = outer.code + pre;
+        line(sect, 2, "#pragma unroll");
+        line(sect, 2, strf("for (int u = 0; u < %d; u++) {", V));
+        line(sect, 3, strf("const int r%d = %s + u;", F, f0.c_str()));
+        sect += inner.code;
+        line(sect, 2, "}");
+        sect += post;
+        for (int n : pres) em_.clear_preset(n);
+        strat += strf("flat vec%d; ", V);
+      } else {
+        for (int si : gr.stores) {
+          const StoreInfo &st = g_.stores[(size_t)si];
+          std::string v = em_.emit(st.value, &S0);
+          std::string idx = em_.emit(g_.n(st.index).src[1], &S0);
+          int p = g_.param_slot(st.param);
+          std::string stmt = strf("data%d[%s] = %s;", p, idx.c_str(), v.c_str());
+          if (st.gate >= 0) stmt = "if (" + em_.emit(st.gate, &S0) + ") " + stmt;
+          line(S0.code, 2, stmt);
+        }
+        sect = S0.code;
+        strat += any_reduce ? "thread-per-output serial reduce; " : "flat scalar; ";
+      }
+      line(body, 1, strf("if (gid < %s) {", nthreads.c_str()));
+      body += decomp + sect;
+      line(body, 1, "}");
+    }
+    if (dynamic) { error_ = "symbolic range bounds are not supported by the flat lowering yet"; return body; }
+    double blocks = std::ceil(max_threads / opt_.block);
+    if (blocks > 2147483647.0) { error_ = "grid too large"; return body; }
+    out->launch.grid[0] = (unsigned)std::max(1.0, blocks);
+    out->launch.block[0] = (unsigned)opt_.block;
+    out->klass = any_reduce ? KernelClass::THREAD_REDUCE : KernelClass::ELEMENTWISE;
+    out->strategy = strat;
+    return body;
+  }
+
+  // ── cooperative row reduction ─────────────────────────────────────────────
+  bool plan_coop() {
+    if (top_reduces_.empty()) return false;
+    const KNode &first = g_.n(top_reduces_[0]);
+    std::vector<int> rr;
+    for (size_t i = 1; i < first.src.size(); i++) rr.push_back(g_.range_ord.at(first.src[i]));
+    int64_t R = 1;
+    for (int r : rr) {
+      if (g_.ranges[(size_t)r].extent < 0) return false;
+      R *= g_.ranges[(size_t)r].extent;
+    }
+    for (int id : top_reduces_) {
+      const KNode &k = g_.n(id);
+      std::vector<int> r2;
+      for (size_t i = 1; i < k.src.size(); i++) r2.push_back(g_.range_ord.at(k.src[i]));
+      if (r2 != rr) return false;
+      if (dt_size(k.dt) != 4 && dt_size(k.dt) != 8) return false;
+      PolyOps op = reduce_op(k);
+      if (op != POLY_OP_ADD && op != POLY_OP_MAX && op != POLY_OP_MUL) return false;
+    }
+    for (int r : groups_[0].ranges) if (g_.ranges[(size_t)r].extent < 0) return false;
+    double rows = 1;
+    for (int r : groups_[0].ranges) rows *= (double)g_.ranges[(size_t)r].extent;
+    if (R < 128) return false;
+    // Long rows, or too few rows to fill the chip with one wave each: a whole
+    // workgroup per row.
+    if (R >= 4096 || (rows < 2048 && R >= 1024)) coop_G_ = 256; else coop_G_ = 64;
+    coop_R_ = R;
+    coop_ranges_ = rr;
+    return true;
+  }
+
+  std::string wave_reduce_call(PolyOps op, DT dt, const std::string &v) const {
+    if (dt == DT_F32) {
+      const char *fn = op == POLY_OP_ADD ? "poly_wave_add_f32" : op == POLY_OP_MUL ? "poly_wave_mul_f32" : "poly_wave_max_f32";
+      return strf("%s(%s)", fn, v.c_str());
+    }
+    const char *ct = dt_cname(dt);
+    std::string comb = Emitter::reduce_combine(op, dt, "a_", "b_");
+    return strf("poly_wave_reduce_any<%s>(%s, [](%s a_, %s b_) { return (%s)%s; })", ct, v.c_str(), ct, ct, ct, comb.c_str());
+  }
+
+  std::string render_coop(RenderedKernel *out) {
+    const Group &gr = groups_[0];
+    const int G = coop_G_;
+    const int rows_per_block = opt_.block / G;
+    std::vector<int> order = fastest_first(gr);
+    double rows = 1;
+    std::string body;
+    Scope S0;
+    S0.indent = 2;
+    for (int r : gr.ranges) S0.avail |= (uint64_t)1 << r;
+    if (G == 64) {
+      line(body, 1, "const int lane = threadIdx.x & 63;");
+      line(body, 1, strf("const long long row = (long long)blockIdx.x * %d + (threadIdx.x >> 6);", rows_per_block));
+    } else {
+      line(body, 1, "const int lane = threadIdx.x;");
+      line(body, 1, "const long long row = blockIdx.x;");
+    }
+    std::string decomp;
+    line(decomp, 2, "long long t_ = row;");
+    for (size_t oi = 0; oi < order.size(); oi++) {
+      int ord = order[oi];
+      int64_t e = g_.ranges[(size_t)ord].extent;
+      rows *= (double)e;
+      std::string rv = strf("r%d", ord);
+      if (oi + 1 == order.size()) line(decomp, 2, strf("const int %s = (int)t_;", rv.c_str()));
+      else line(decomp, 2, strf("const int %s = (int)(t_ %% %lld); t_ /= %lld;", rv.c_str(), (long long)e, (long long)e));
+      em_.bind_range(ord, rv);
+    }
+    // vector width along the fastest reduce range
+    int QF = coop_ranges_.back();
+    int64_t eF = g_.ranges[(size_t)QF].extent;
+    int V = 1;
+    if (opt_.allow_vectorize) {
+      int maxsz = 1;
+      std::vector<char> mark(g_.nodes.size(), 0);
+      for (int id : top_reduces_) node_under(g_.n(id).src[0], mark);
+      for (int i = 0; i < (int)g_.nodes.size(); i++)
+        if (mark[(size_t)i] && g_.n(i).op == POLY_OP_LOAD && (g_.n(i).deps & ((uint64_t)1 << QF)))
+          maxsz = std::max(maxsz, dt_size(g_.n(i).dt));
+      V = std::max(1, 16 / maxsz);
+      while (V > 1 && (eF % V != 0 || coop_R_ < (int64_t)G * V)) V /= 2;
+    }
+    // accumulators
+    std::string accs;
+    for (int id : top_reduces_) {
+      const KNode &k = g_.n(id);
+      line(accs, 2, strf("%s acc%d = %s;", dt_cname(k.dt), id, Emitter::reduce_identity(reduce_op(k), k.dt).c_str()));
+    }
+    // loop over the flattened reduce index
+    Scope L;
+    L.parent = &S0;
+    L.avail = S0.avail;
+    L.indent = 3;
+    std::string qdecomp;
+    line(qdecomp, 3, "int q_ = q0;");
+    for (size_t i = coop_ranges_.size(); i-- > 0;) {
+      int ord = coop_ranges_[i];
+      int64_t e = g_.ranges[(size_t)ord].extent;
+      std::string rv = strf("r%d", ord);
+      bool fastest = (i + 1 == coop_ranges_.size());
+      std::string nm = fastest && V > 1 ? rv + "_0" : rv;
+      if (i == 0) line(qdecomp, 3, strf("const int %s = q_;", nm.c_str()));
+      else line(qdecomp, 3, strf("const int %s = q_ %% %lld; q_ /= %lld;", nm.c_str(), (long long)e, (long long)e));
+      em_.bind_range(ord, nm);
+      if (!(fastest && V > 1)) L.avail |= (uint64_t)1 << ord;
+    }
+    std::vector<int> roots;
+    for (int id : top_reduces_) roots.push_back(g_.n(id).src[0]);
+    std::vector<int> pres;
+    std::string loop_body;
+    if (V > 1) {
+      pres = hoist_vector_loads(roots, QF, V, strf("r%d_0", QF), &L, true);
+      Scope U;
+      U.parent = &L;
+      U.avail = L.avail | ((uint64_t)1 << QF);
+      U.indent = 4;
+      em_.bind_range(QF, strf("r%d", QF));
+      for (int id : top_reduces_) {
+        const KNode &k = g_.n(id);
+        std::string v = em_.emit(k.src[0], &U);
+        std::string acc = strf("acc%d", id);
+        line(U.code, 4, strf("%s = %s;", acc.c_str(), Emitter::reduce_combine(reduce_op(k), k.dt, acc, v).c_str()));
+      }
+      loop_body = L.code;
+      line(loop_body, 3, "#pragma unroll");
+      line(loop_body, 3, strf("for (int u = 0; u < %d; u++) {", V));
+      line(loop_body, 4, strf("const int r%d = r%d_0 + u;", QF, QF));
+      loop_body += U.code;
+      line(loop_body, 3, "}");
+    } else {
+      for (int id : top_reduces_) {
+        const KNode &k = g_.n(id);
+        std::string v = em_.emit(k.src[0], &L);
+        std::string acc = strf("acc%d", id);
+        line(L.code, 3, strf("%s = %s;", acc.c_str(), Emitter::reduce_combine(reduce_op(k), k.dt, acc, v).c_str()));
+      }
+      loop_body = L.code;
+    }
+    for (int n : pres) em_.clear_preset(n);
+    // S0.code now holds everything hoisted out of the loop (row-invariant values)
+    std::string pre_loop = S0.code;
+    S0.code.clear();
+    std::string red;
+    int nred = (int)top_reduces_.size();
+    for (int id : top_reduces_) {
+      const KNode &k = g_.n(id);
+      line(red, 2, strf("acc%d = %s;", id, wave_reduce_call(reduce_op(k), k.dt, strf("acc%d", id)).c_str()));
+    }
+    if (G == 256) {
+      int ri = 0;
+      for (int id : top_reduces_) {
+        const KNode &k = g_.n(id);
+        line(red, 2, strf("if ((threadIdx.x & 63) == 0) red%d[threadIdx.x >> 6] = acc%d;", ri, id));
+        ri++;
+        (void)k;
+      }
+      line(red, 2, "__syncthreads();");
+      ri = 0;
+      for (int id : top_reduces_) {
+        const KNode &k = g_.n(id);
+        PolyOps op = reduce_op(k);
+        std::string e = strf("red%d[0]", ri);
+        for (int w = 1; w < 4; w++) e = Emitter::reduce_combine(op, k.dt, e, strf("red%d[%d]", ri, w));
+        line(red, 2, strf("acc%d = %s;", id, e.c_str()));
+        ri++;
+      }
+    }
+    for (int id : top_reduces_) em_.preset(id, strf("acc%d", id));
+    // tail: value + store by lane 0
+    std::string tail_stores;
+    for (int si : gr.stores) {
+      const StoreInfo &st = g_.stores[(size_t)si];
+      std::string v = em_.emit(st.value, &S0);
+      std::string idx = em_.emit(g_.n(st.index).src[1], &S0);
+      int p = g_.param_slot(st.param);
+      std::string cond = "lane == 0";
+      if (st.gate >= 0) cond += " && " + em_.emit(st.gate, &S0);
+      line(tail_stores, 2, strf("if (%s) data%d[%s] = %s;", cond.c_str(), p, idx.c_str(), v.c_str()));
+    }
+    std::string tail = S0.code + tail_stores;
+
+    if (G == 256) {
+      int ri = 0;
+      for (int id : top_reduces_) {
+        line(body, 1, strf("__shared__ %s red%d[4];", dt_cname(g_.n(id).dt), ri));
+        ri++;
+      }
+      line(body, 1, "{");
+    } else {
+      line(body, 1, strf("if (row < %lldll) {", (long long)rows));
+    }
+    body += decomp + accs + pre_loop;
+    line(body, 2, strf("for (int q0 = lane * %d; q0 < %lld; q0 += %d) {", V, (long long)coop_R_, G * V));
+    body += qdecomp + loop_body;
+    line(body, 2, "}");
+    body += red + tail;
+    line(body, 1, "}");
+    (void)nred;
+
+    double blocks = G == 256 ? rows : std::ceil(rows / rows_per_block);
+    if (blocks > 2147483647.0) { error_ = "grid too large"; return body; }
+    out->launch.grid[0] = (unsigned)std::max(1.0, blocks);
+    out->launch.block[0] = (unsigned)opt_.block;
+    out->klass = KernelClass::ROW_REDUCE;
+    out->strategy = strf("row-reduce G=%d vec%d R=%lld rows=%.0f", G, V, (long long)coop_R_, rows);
+    return body;
+  }
+
+  // Algorithmic bytes: distinct elements each access can touch, capped by the
+  // buffer size, summed over buffers.
+  void account(RenderedKernel *out) const {
+    std::vector<double> touched(g_.params.size(), 0.0);
+    auto distinct = [&](int idx_node) {
+      uint64_t d = g_.n(idx_node).deps;
+      double n = 1;
+      for (size_t r = 0; r < g_.ranges.size(); r++)
+        if (d & ((uint64_t)1 << r)) n *= (double)std::max<int64_t>(1, g_.ranges[r].extent);
+      return n;
+    };
+    for (const KNode &k : g_.nodes) {
+      if (k.op == POLY_OP_LOAD) {
+        const KNode &ix = g_.n(k.src[0]);
+        touched[(size_t)g_.param_slot(ix.src[0])] += distinct(ix.src[1]);
+      }
+    }
+    for (const StoreInfo &st : g_.stores) touched[(size_t)g_.param_slot(st.param)] += distinct(g_.n(st.index).src[1]);
+    double bytes = 0;
+    for (size_t i = 0; i < g_.params.size(); i++) {
+      double n = touched[i];
+      if (g_.params[i].numel > 0) n = std::min(n, (double)g_.params[i].numel * ((g_.params[i].read && g_.params[i].written) ? 2 : 1));
+      bytes += n * dt_size(g_.params[i].dt);
+    }
+    out->bytes = bytes;
+  }
+};
+
+}  // namespace
+
+bool render_kernel(const KernelGraph &g, const std::string &fn_name, const RenderOptions &opt,
+                   RenderedKernel *out, std::string *err) {
+  if (opt.allow_templates) {
+    if (try_render_matmul(g, fn_name, opt, out)) return true;
+    if (try_render_gather(g, fn_name, opt, out)) return true;
+  }
+  *out = RenderedKernel();
+  Generic gen(g, fn_name, opt);
+  return gen.run(out, err);
+}
+
+}  // namespace polyhip

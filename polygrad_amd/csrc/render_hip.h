@@ -1,0 +1,110 @@
+// render_hip: lowers one analysed kernel graph to gfx950 HIP C source plus a
+// launch description.  Replaces (does not port) the reference's CUDA lowering
+// (src/render_cuda.c:176-570, src/codegen.c:4149-4581): all non-reduce ranges
+// are flattened over the grid, accesses are vectorised to 128 bit when the
+// fastest index is unit-stride, row reductions run one wave or one workgroup
+// per row with DPP/ds_swizzle wave reductions, and matmul-shaped reductions are
+// handed to the MFMA template.
+#pragma once
+#include <string>
+#include <unordered_map>
+#include <vector>
+
+#include "kgraph.h"
+
+namespace polyhip {
+
+// How the kernel is launched.  Sizes may depend on DEFINE_VAR values when a
+// range bound is symbolic; then `dyn_*` describe how to recompute them.
+struct LaunchSpec {
+  unsigned grid[3] = {1, 1, 1};
+  unsigned block[3] = {256, 1, 1};
+  unsigned lds_bytes = 0;
+};
+
+enum class KernelClass { ELEMENTWISE, ROW_REDUCE, THREAD_REDUCE, MATMUL_MFMA, GATHER, COPY };
+
+struct RenderedKernel {
+  std::string source;      // complete HIP C translation unit
+  std::string entry;       // kernel symbol
+  LaunchSpec launch;
+  KernelClass klass = KernelClass::ELEMENTWISE;
+  std::string strategy;    // human-readable summary for dumps and profiles
+  int n_params = 0;        // buffer parameters (args[0..n_params-1])
+  int n_vars = 0;          // DEFINE_VAR ints appended after the buffers
+  // Algorithmic work of one launch, for roofline accounting.
+  double bytes = 0;        // distinct buffer elements touched * element size
+  double flops = 0;        // 2*M*N*K for matmul-shaped kernels, else 0
+  // Guarded fast paths: a small check kernel must succeed for the fast kernel
+  // to be valid; otherwise `fallback` runs (always the generic lowering).
+  struct Guard {
+    std::string source, entry;
+    LaunchSpec launch;
+    std::vector<int> arg_params;   // which buffer params the check reads
+  };
+  std::vector<Guard> guards;
+  std::string fallback_source, fallback_entry;
+  LaunchSpec fallback_launch;
+};
+
+struct RenderOptions {
+  bool allow_templates = true;   // MFMA matmul / gather fast paths
+  bool allow_vectorize = true;
+  bool allow_coop_reduce = true;
+  int block = 256;
+  // When set, the kernel takes one more argument `const int* poly_flag` after the
+  // vars and returns at once if *poly_flag != 0 (the slow twin of a guarded fast path).
+  bool exit_if_flag = false;
+};
+
+// Returns false and sets *err on unsupported graphs (never falls back to a
+// host path).
+bool render_kernel(const KernelGraph &g, const std::string &fn_name, const RenderOptions &opt,
+                   RenderedKernel *out, std::string *err);
+
+// ── expression emitter shared by the generic path and the templates ───────
+struct Scope {
+  uint64_t avail = 0;   // range ordinals bound in this scope (including parents)
+  std::string code;
+  std::unordered_map<int, std::string> names;       // node id -> C name
+  std::unordered_map<int, std::string> atom_names;  // atom id -> C name
+  Scope *parent = nullptr;
+  int indent = 1;
+};
+
+class Emitter {
+ public:
+  explicit Emitter(const KernelGraph &g) : g_(g) {}
+  // Binds a range ordinal to a C expression (a variable name).
+  void bind_range(int ord, const std::string &name) { range_name_[ord] = name; }
+  // Overrides the value of a node (vector-loaded values, reduce results, ...).
+  void preset(int node, const std::string &expr) { preset_[node] = expr; }
+  void clear_preset(int node) { preset_.erase(node); }
+  std::string emit(int node, Scope *s);
+  std::string emit_lin(const Lin &l, Scope *s);
+  std::string load_expr(int load_node, Scope *s);
+  // Serial reduction of REDUCE node `id` placed in scope `s`.
+  std::string emit_reduce_serial(int id, Scope *s);
+  static std::string float_literal(double v, DT dt);
+  static std::string reduce_identity(PolyOps op, DT dt);
+  static std::string reduce_combine(PolyOps op, DT dt, const std::string &acc, const std::string &v);
+  bool failed() const { return !error_.empty(); }
+  const std::string &error() const { return error_; }
+  bool uses_threefry = false;
+
+ private:
+  std::string emit_atom(int atom, Scope *s);
+  std::string emit_raw(int node, Scope *s);
+  Scope *place(uint64_t deps, Scope *s);
+  void stmt(Scope *s, const std::string &line);
+  const KernelGraph &g_;
+  std::unordered_map<int, std::string> range_name_;
+  std::unordered_map<int, std::string> preset_;
+  std::string error_;
+};
+
+// Prelude with the wave/workgroup reduction helpers and small utilities that
+// every generated kernel may use.
+const char *hip_prelude();
+
+}  // namespace polyhip

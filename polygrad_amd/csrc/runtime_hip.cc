@@ -1,0 +1,216 @@
+// runtime_hip: device runtime for the HIP backend -- device/stream set-up,
+// memory, copies, hiprtc compilation for gfx950 with an in-process and an
+// on-disk code-object cache, and kernel launches on one HIP stream.
+//
+// Takes the place of the reference's CUDA runtime (src/runtime_cuda.c:192-435)
+// with the same call surface (init / alloc / free / copy / memset / compile /
+// launch / sync / program_destroy) but none of its mechanism: it links
+// libamdhip64 and libhiprtc directly, never synchronises after a launch, and
+// shares one module between all runners whose source text is identical.
+#include "runtime_hip.h"
+
+#include <hip/hip_runtime.h>
+#include <hip/hiprtc.h>
+#include <sys/stat.h>
+#include <unistd.h>
+
+#include <cstdlib>
+#include <cstring>
+#include <fstream>
+#include <map>
+#include <memory>
+
+namespace polyhip {
+
+namespace {
+
+struct Module {
+  hipModule_t mod = nullptr;
+  std::vector<char> code;
+  ~Module() { if (mod) (void)hipModuleUnload(mod); }
+};
+
+struct Runtime {
+  bool tried = false;
+  bool ok = false;
+  int device = 0;
+  hipStream_t stream = nullptr;
+  std::map<uint64_t, std::weak_ptr<Module>> modules;   // keyed by source hash
+  std::map<uint64_t, std::vector<char>> code_cache;    // compiled, not yet loaded
+};
+
+Runtime &rt() {
+  static Runtime r;
+  return r;
+}
+
+bool check(hipError_t e, const char *what) {
+  if (e == hipSuccess) return true;
+  log_err("runtime_hip", "%s failed: %s", what, hipGetErrorString(e));
+  return false;
+}
+
+std::string cache_dir() {
+  const char *off = getenv("POLY_CACHE");
+  if (off && strcmp(off, "0") == 0) return "";
+  std::string base;
+  if (const char *d = getenv("POLY_HIP_CACHE_DIR")) base = d;
+  else if (const char *x = getenv("XDG_CACHE_HOME")) base = std::string(x) + "/polygrad_hip";
+  else if (const char *h = getenv("HOME")) base = std::string(h) + "/.cache/polygrad_hip";
+  else return "";
+  mkdir(base.substr(0, base.find_last_of('/')).c_str(), 0755);
+  mkdir(base.c_str(), 0755);
+  return base;
+}
+
+}  // namespace
+
+// hiprtc needs no device, so this also serves compile-only checks.
+bool compile_to_code_object(const std::string &source, std::vector<char> *code, std::string *log) {
+  uint64_t h = fnv1a(source.data(), source.size());
+  Runtime &r = rt();
+  auto it = r.code_cache.find(h);
+  if (it != r.code_cache.end()) { *code = it->second; return true; }
+  std::string dir = cache_dir();
+  std::string path = dir.empty() ? "" : strf("%s/%016llx.hsaco", dir.c_str(), (unsigned long long)h);
+  if (!path.empty()) {
+    std::ifstream f(path, std::ios::binary);
+    if (f) {
+      code->assign(std::istreambuf_iterator<char>(f), std::istreambuf_iterator<char>());
+      if (!code->empty()) { r.code_cache[h] = *code; return true; }
+    }
+  }
+  hiprtcProgram prog;
+  if (hiprtcCreateProgram(&prog, source.c_str(), "poly_kernel.hip", 0, nullptr, nullptr) != HIPRTC_SUCCESS) {
+    *log = "hiprtcCreateProgram failed";
+    return false;
+  }
+  // Packed FP32 instructions are kept out of generated code on purpose.
+  const char *opts[] = {"--offload-arch=gfx950", "-O3", "-std=c++17", "-Xclang", "-target-feature",
+                        "-Xclang", "-packed-fp32-ops", "-Wno-unused-value"};
+  hiprtcResult res = hiprtcCompileProgram(prog, (int)(sizeof(opts) / sizeof(opts[0])), opts);
+  size_t ls = 0;
+  hiprtcGetProgramLogSize(prog, &ls);
+  if (ls > 1) { log->resize(ls); hiprtcGetProgramLog(prog, &(*log)[0]); }
+  if (res != HIPRTC_SUCCESS) { hiprtcDestroyProgram(&prog); return false; }
+  size_t cs = 0;
+  hiprtcGetCodeSize(prog, &cs);
+  code->resize(cs);
+  hiprtcGetCode(prog, code->data());
+  hiprtcDestroyProgram(&prog);
+  r.code_cache[h] = *code;
+  if (!path.empty()) {
+    std::string tmp = path + strf(".%d.tmp", (int)getpid());
+    std::ofstream f(tmp, std::ios::binary);
+    if (f) {
+      f.write(code->data(), (std::streamsize)code->size());
+      f.close();
+      rename(tmp.c_str(), path.c_str());
+    }
+  }
+  return true;
+}
+
+int runtime_init() {
+  Runtime &r = rt();
+  if (r.tried) return r.ok ? 0 : -1;
+  r.tried = true;
+  int n = 0;
+  if (hipGetDeviceCount(&n) != hipSuccess || n < 1) {
+    log_err("runtime_hip", "no HIP device available");
+    return -1;
+  }
+  int dev = 0;
+  if (const char *d = getenv("POLY_HIP_DEVICE")) dev = atoi(d);
+  if (dev < 0 || dev >= n) dev = 0;
+  if (!check(hipSetDevice(dev), "hipSetDevice")) return -1;
+  r.device = dev;
+  if (!check(hipStreamCreateWithFlags(&r.stream, hipStreamNonBlocking), "hipStreamCreate")) return -1;
+  r.ok = true;
+  return 0;
+}
+
+void *runtime_stream() { return runtime_init() == 0 ? (void *)rt().stream : nullptr; }
+
+void *runtime_alloc(size_t nbytes) {
+  if (runtime_init() != 0) return nullptr;
+  void *p = nullptr;
+  if (nbytes == 0) nbytes = 4;
+  if (!check(hipMalloc(&p, nbytes), "hipMalloc")) return nullptr;
+  return p;
+}
+
+void runtime_free(void *p) {
+  if (!p || runtime_init() != 0) return;
+  // The stream may still be using the memory.
+  (void)hipStreamSynchronize(rt().stream);
+  (void)hipFree(p);
+}
+
+int runtime_copy(void *dst, const void *src, size_t n, int kind) {
+  if (runtime_init() != 0) return -1;
+  hipMemcpyKind k = kind == 0 ? hipMemcpyHostToDevice : kind == 1 ? hipMemcpyDeviceToHost : hipMemcpyDeviceToDevice;
+  if (n == 0) return 0;
+  if (!check(hipMemcpyAsync(dst, src, n, k, rt().stream), "hipMemcpyAsync")) return -1;
+  return check(hipStreamSynchronize(rt().stream), "hipStreamSynchronize") ? 0 : -1;
+}
+
+int runtime_memset(void *p, int value, size_t n) {
+  if (runtime_init() != 0) return -1;
+  if (n == 0) return 0;
+  return check(hipMemsetAsync(p, value, n, rt().stream), "hipMemsetAsync") ? 0 : -1;
+}
+
+int runtime_sync() {
+  if (runtime_init() != 0) return -1;
+  return check(hipStreamSynchronize(rt().stream), "hipStreamSynchronize") ? 0 : -1;
+}
+
+struct Program {
+  std::shared_ptr<Module> module;
+  hipFunction_t fn = nullptr;
+  std::string entry;
+};
+
+Program *program_create(const std::string &source, const std::string &entry) {
+  if (runtime_init() != 0) return nullptr;
+  if (getenv("POLY_DUMP_KERNELS"))
+    fprintf(stderr, "=== HIP KERNEL %s ===\n%s\n=== END ===\n", entry.c_str(), source.c_str());
+  Runtime &r = rt();
+  uint64_t h = fnv1a(source.data(), source.size());
+  std::shared_ptr<Module> m;
+  auto it = r.modules.find(h);
+  if (it != r.modules.end()) m = it->second.lock();
+  if (!m) {
+    std::vector<char> code;
+    std::string log;
+    if (!compile_to_code_object(source, &code, &log)) {
+      log_err("runtime_hip", "hiprtc failed for %s:\n%s", entry.c_str(), log.c_str());
+      fprintf(stderr, "=== FAILED HIP KERNEL %s ===\n%s\n=== END ===\n", entry.c_str(), source.c_str());
+      return nullptr;
+    }
+    m = std::make_shared<Module>();
+    m->code = std::move(code);
+    if (!check(hipModuleLoadData(&m->mod, m->code.data()), "hipModuleLoadData")) return nullptr;
+    r.modules[h] = m;
+  }
+  Program *p = new Program();
+  p->module = m;
+  p->entry = entry;
+  if (!check(hipModuleGetFunction(&p->fn, m->mod, entry.c_str()), "hipModuleGetFunction")) {
+    delete p;
+    return nullptr;
+  }
+  return p;
+}
+
+void program_destroy(Program *p) { delete p; }
+
+int program_launch(Program *p, void **kernel_args, const LaunchSpec &ls) {
+  if (!p || runtime_init() != 0) return -1;
+  hipError_t e = hipModuleLaunchKernel(p->fn, ls.grid[0], ls.grid[1], ls.grid[2], ls.block[0], ls.block[1],
+                                       ls.block[2], ls.lds_bytes, rt().stream, kernel_args, nullptr);
+  return check(e, "hipModuleLaunchKernel") ? 0 : -1;
+}
+
+}  // namespace polyhip

@@ -1,0 +1,44 @@
+// Internal C++ face of the device runtime (the C ABI wraps these).
+#pragma once
+#include <string>
+#include <vector>
+
+#include "common.h"
+#include "render_hip.h"
+
+namespace polyhip {
+
+struct Program;  // one kernel entry inside a loaded (shared) module
+
+int runtime_init();
+void *runtime_stream();
+void *runtime_alloc(size_t nbytes);
+void runtime_free(void *p);
+// kind: 0 host->device, 1 device->host, 2 device->device; returns once done
+int runtime_copy(void *dst, const void *src, size_t n, int kind);
+int runtime_memset(void *p, int value, size_t n);
+int runtime_sync();
+
+bool compile_to_code_object(const std::string &source, std::vector<char> *code, std::string *log);
+Program *program_create(const std::string &source, const std::string &entry);
+void program_destroy(Program *p);
+int program_launch(Program *p, void **kernel_args, const LaunchSpec &ls);
+
+// One lowered kernel: the program(s) plus how to call them.
+struct HipRunner {
+  RenderedKernel rk;
+  Program *main = nullptr;
+  std::vector<Program *> guards;
+  Program *fallback = nullptr;
+  void *flag = nullptr;            // device int written by the guards
+  std::string name;
+  std::vector<void *> ptr_store;   // argument storage reused by every launch
+  std::vector<int> var_store;
+  std::vector<void *> arg_ptrs;
+};
+
+HipRunner *runner_create(const PolyUOp *root, const char *fn_name, int flags);
+int runner_launch(HipRunner *r, void **args, int n_args);
+void runner_destroy(HipRunner *r);
+
+}  // namespace polyhip

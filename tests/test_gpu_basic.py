@@ -1,0 +1,106 @@
+"""GPU parity, first tier: one graph per kernel class, HIP backend (through the
+C ABI) against the reference CPU backend on the same seeded inputs.
+
+Tolerances are the ones the task states: bit-exact for integer/index/movement
+ops, rtol 1e-5 fp32 elementwise, rtol 1e-4 fp32 reductions and matmul, rtol 2e-2
+for bf16/fp16."""
+import numpy as np
+import pytest
+
+import refpoly as R
+from hipharness import assert_close, run_hip, run_ref
+
+pytestmark = [pytest.mark.gpu, pytest.mark.skipif(not R.available(), reason="reference library not built")]
+
+
+def rng(seed):
+    return np.random.default_rng(seed)
+
+
+def test_fused_chain_fp32():
+    c = R.Ctx()
+    g = rng(1)
+    shape = (256, 512)
+    a, b, d, o = (c.buffer(shape, name=n) for n in "abdo")
+    y = (a * b + d).exp2().clamp(-4, 4)
+    sink = c.sink((o, y))
+    arrays = {a: g.uniform(-1, 1, shape).astype(np.float32), b: g.uniform(-1, 1, shape).astype(np.float32),
+              d: g.uniform(-1, 1, shape).astype(np.float32), o: np.zeros(shape, np.float32)}
+    want = run_ref(c, sink, arrays)
+    got, info = run_hip(c, sink, arrays)
+    assert info[0]["klass"] == "elementwise"
+    assert_close(got[o], want[o], rtol=1e-5, what="chain")
+    c.close()
+
+
+@pytest.mark.parametrize("cols", [8, 100, 128, 1024, 4096, 5000])
+def test_row_reductions_fp32(cols):
+    c = R.Ctx()
+    g = rng(2)
+    shape = (96, cols)
+    x = c.buffer(shape, name="x")
+    s_out, m_out = c.buffer((96,), name="sum"), c.buffer((96,), name="max")
+    arrays = {x: g.uniform(-1, 1, shape).astype(np.float32), s_out: np.zeros(96, np.float32), m_out: np.zeros(96, np.float32)}
+    for out, val in ((s_out, x.sum()), (m_out, x.max())):
+        sink = c.sink((out, val))
+        sub = {x: arrays[x], out: arrays[out]}
+        want = run_ref(c, sink, sub)
+        got, _ = run_hip(c, sink, sub)
+        assert_close(got[out], want[out], rtol=1e-4, atol=1e-6, what=f"reduce cols={cols}")
+    c.close()
+
+
+def test_softmax_layernorm_fp32():
+    c = R.Ctx()
+    g = rng(3)
+    shape = (64, 768)
+    x = c.buffer(shape, name="x")
+    o = c.buffer(shape, name="o")
+    arrays = {x: g.normal(0, 1, shape).astype(np.float32), o: np.zeros(shape, np.float32)}
+    for name, val in (("softmax", x.softmax()), ("layernorm", x.layernorm(1e-5))):
+        sink = c.sink((o, val))
+        want = run_ref(c, sink, arrays)
+        got, info = run_hip(c, sink, arrays)
+        assert_close(got[o], want[o], rtol=1e-4, atol=1e-6, what=name)
+        assert any(k["klass"] == "row-reduce" for k in info)
+    c.close()
+
+
+def test_matmul_fp32_small():
+    c = R.Ctx()
+    g = rng(4)
+    A, B, O = c.buffer((64, 48), name="A"), c.buffer((48, 80), name="B"), c.buffer((64, 80), name="O")
+    sink = c.sink((O, A.dot(B)))
+    arrays = {A: g.normal(0, 1, (64, 48)).astype(np.float32), B: g.normal(0, 1, (48, 80)).astype(np.float32),
+              O: np.zeros((64, 80), np.float32)}
+    want = run_ref(c, sink, arrays)
+    got, _ = run_hip(c, sink, arrays)
+    assert_close(got[O], want[O], rtol=1e-4, atol=1e-5, what="matmul")
+    c.close()
+
+
+def test_movement_ops_bit_exact():
+    c = R.Ctx()
+    g = rng(5)
+    x = c.buffer((6, 10, 8), R.I32, name="x")
+    o = c.buffer((8, 5, 8), R.I32, name="o")
+    y = x.permute((2, 1, 0)).shrink(((0, 8), (2, 7), (1, 5))).pad(((0, 0), (0, 0), (2, 2))).flip((1,))
+    sink = c.sink((o, y))
+    arrays = {x: g.integers(-1000, 1000, (6, 10, 8)).astype(np.int32), o: np.zeros((8, 5, 8), np.int32)}
+    want = run_ref(c, sink, arrays)
+    got, _ = run_hip(c, sink, arrays)
+    assert np.array_equal(got[o], want[o])
+    c.close()
+
+
+def test_graph_replay_matches_eager():
+    c = R.Ctx()
+    g = rng(6)
+    shape = (32, 256)
+    x, o = c.buffer(shape, name="x"), c.buffer(shape, name="o")
+    sink = c.sink((o, x.softmax()))
+    arrays = {x: g.normal(0, 1, shape).astype(np.float32), o: np.zeros(shape, np.float32)}
+    eager, _ = run_hip(c, sink, arrays, graph=False)
+    replay, _ = run_hip(c, sink, arrays, graph=True, repeats=4)
+    assert np.array_equal(eager[o], replay[o])
+    c.close()
