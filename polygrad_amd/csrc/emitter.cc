@@ -341,7 +341,17 @@ std::string Emitter::emit_raw(int id, Scope *s) {
     case POLY_OP_RECIPROCAL: e = strf("(1/%s)", S(0).c_str()); break;
     case POLY_OP_ADD: e = strf("(%s+%s)", S(0).c_str(), S(1).c_str()); break;
     case POLY_OP_SUB: e = strf("(%s-%s)", S(0).c_str(), S(1).c_str()); break;
-    case POLY_OP_MUL: e = strf("(%s*%s)", S(0).c_str(), S(1).c_str()); break;
+    case POLY_OP_MUL: {
+      // a * (1/b) is a single division, as the reference's late rewrite makes it
+      // (src/codegen.c:1867-1883; the reciprocal must be the second factor)
+      const KNode &rb = g_.n(k.src[1]);
+      if (dt_is_float(k.dt) && rb.op == POLY_OP_RECIPROCAL && rb.src.size() == 1) {
+        e = strf("(%s/%s)", S(0).c_str(), emit(rb.src[0], t).c_str());
+        break;
+      }
+      e = strf("(%s*%s)", S(0).c_str(), S(1).c_str());
+      break;
+    }
     case POLY_OP_FDIV: e = strf("(%s/%s)", S(0).c_str(), S(1).c_str()); break;
     case POLY_OP_IDIV: e = strf("(%s/%s)", S(0).c_str(), S(1).c_str()); break;
     case POLY_OP_MOD: e = strf("(%s%%%s)", S(0).c_str(), S(1).c_str()); break;

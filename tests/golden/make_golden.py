@@ -1,0 +1,146 @@
+"""Generates the committed golden fixtures: for each small case, the scheduled
+plan (as a plan file) and the inputs plus the outputs computed by the REAL
+reference CPU backend (oracle/_ref/libpolygrad.so, built from /root/reference).
+
+Run from the repository root in the build container:
+    python tests/golden/make_golden.py
+Writes tests/golden/<case>.polyplan and tests/golden/<case>.npz
+(npz keys: in<slot> = initial contents of external slot, out<slot> = contents
+after the reference ran).  bf16 data is stored as uint16 bit patterns.
+"""
+import ctypes as C
+import os
+import sys
+
+import numpy as np
+
+HERE = os.path.dirname(os.path.abspath(__file__))
+ROOT = os.path.dirname(os.path.dirname(HERE))
+sys.path.insert(0, ROOT)
+sys.path.insert(0, os.path.join(ROOT, "tests"))
+
+import graphs  # noqa: E402
+import refpoly as R  # noqa: E402
+from hipharness import schedule_slots  # noqa: E402
+from polygrad_amd import save_schedule  # noqa: E402
+
+
+def emit(name, c, sink, arrays):
+    want = {t: np.array(a, copy=True) for t, a in arrays.items()}
+    c.realize_cpu(sink, want)
+    sched = c.schedule(sink)
+    slots, n = schedule_slots(c, sched)
+    names = [None] * n
+    data = {}
+    for i, tn in slots.items():
+        t, nm = tn
+        names[i] = nm
+        data[f"in{i}"] = np.ascontiguousarray(arrays[t]).reshape(-1)
+        data[f"out{i}"] = np.ascontiguousarray(want[t]).reshape(-1)
+    save_schedule(sched, names, os.path.join(HERE, name + ".polyplan"))
+    np.savez_compressed(os.path.join(HERE, name + ".npz"), **data)
+    c.L.poly_schedule_free(sched)
+    print(f"{name}: {n} slots, {sum(v.nbytes for v in data.values())} bytes of vectors")
+
+
+def main():
+    g = np.random.default_rng(1234)
+
+    # reference KAT: (2,3)@(3,4) = [[38,44,50,56],[83,98,113,128]]  (test/test_nn.c:417-439)
+    c = R.Ctx()
+    A, B, O = c.buffer((2, 3), name="A"), c.buffer((3, 4), name="B"), c.buffer((2, 4), name="O")
+    emit("kat_matmul_2x3x4", c, c.sink((O, A.dot(B))),
+         {A: np.arange(1, 7, dtype=np.float32), B: np.arange(1, 13, dtype=np.float32), O: np.zeros(8, np.float32)})
+    c.close()
+
+    # reference KAT: threefry2x32, key 1337, counters 0..19 (test/test_nn.c:1122-1197)
+    for dt, npdt, nm in ((R.U32, np.uint32, "u32"), (R.U64, np.uint64, "u64")):
+        c = R.Ctx()
+        ctr, key, out = c.buffer((20,), dt, name="counter"), c.buffer((20,), dt, name="key"), c.buffer((20,), dt, name="out")
+        thr = ctr._bin("THREEFRY", key)
+        emit(f"kat_threefry_{nm}", c, c.sink((out, thr)),
+             {ctr: np.arange(20, dtype=npdt), key: np.full(20, 1337, npdt), out: np.zeros(20, npdt)})
+        c.close()
+
+    # cross-entropy of uniform logits over 3 classes = log 3 (test/test_nn.c:518-624)
+    c = R.Ctx()
+    lg, tg, o = c.buffer((4, 3), name="logits"), c.buffer((4, 3), name="target"), c.buffer((1,), name="loss")
+    onehot = np.zeros((4, 3), np.float32)
+    onehot[np.arange(4), [0, 1, 2, 1]] = 1
+    emit("kat_xent_uniform", c, c.sink((o, lg.cross_entropy(tg))),
+         {lg: np.full((4, 3), 0.7, np.float32), tg: onehot, o: np.zeros(1, np.float32)})
+    c.close()
+
+    # fused chain + row ops (config 2 at a reduced shape)
+    c = R.Ctx()
+    (a, b, d), outs, sinks = graphs.fused_rowops(c, 24, 160)
+    base = {a: g.uniform(-1, 1, (24, 160)).astype(np.float32), b: g.uniform(-1, 1, (24, 160)).astype(np.float32),
+            d: g.uniform(-1, 1, (24, 160)).astype(np.float32)}
+    for k in ("sum", "max", "softmax", "layernorm"):
+        arr = dict(base)
+        arr[outs[k]] = np.zeros(int(np.prod(outs[k].shape)), np.float32)
+        emit(f"rowops_{k}", c, sinks[k], arr)
+    c.close()
+
+    # special values through exp2 / log2 / sqrt / reciprocal
+    c = R.Ctx()
+    x, o1, o2 = c.buffer((32,), name="x"), c.buffer((32,), name="exp2"), c.buffer((32,), name="log2")
+    xs = np.array([0, -0.0, 1, -1, 0.5, 10, -10, 127, 128, 129, -126, -149, -150, -151, 1e-40, 3.14159,
+                   np.inf, -np.inf, np.nan, 1e-4, 1e-5, 2.0**-127, 88.7, -88.7, 1e30, 1e-30, 7, 0.1, 0.9999999, 1.0000001,
+                   1024, 3], np.float32)
+    emit("special_exp2", c, c.sink((o1, x.exp2())), {x: xs, o1: np.zeros(32, np.float32)})
+    emit("special_log2", c, c.sink((o2, x.log2())), {x: xs, o2: np.zeros(32, np.float32)})
+    c.close()
+
+    # movement ops on integers: permute / shrink / pad / flip, bit exact
+    c = R.Ctx()
+    x = c.buffer((6, 10, 8), R.I32, name="x")
+    o = c.buffer((8, 5, 8), R.I32, name="o")
+    y = x.permute((2, 1, 0)).shrink(((0, 8), (2, 7), (1, 5))).pad(((0, 0), (0, 0), (2, 2))).flip((1,))
+    emit("movement_i32", c, c.sink((o, y)), {x: g.integers(-1000, 1000, 480).astype(np.int32), o: np.zeros(320, np.int32)})
+    c.close()
+
+    # integer ALU: div / mod / shifts / bit ops, bit exact
+    c = R.Ctx()
+    p, q, o = c.buffer((64,), R.I32, name="p"), c.buffer((64,), R.I32, name="q"), c.buffer((64,), R.I32, name="o")
+    y = (p.idiv(q) + p.mod(q)).bxor(p.shl(c.const(3, R.I32))).band(q.bor(c.const(255, R.I32))) + p.shr(c.const(2, R.I32)) * q
+    emit("int_alu", c, c.sink((o, y)),
+         {p: g.integers(-5000, 5000, 64).astype(np.int32), q: g.integers(1, 50, 64).astype(np.int32), o: np.zeros(64, np.int32)})
+    c.close()
+
+    # bf16: elementwise GELU and matmul with f32 accumulate
+    c = R.Ctx()
+    x, o = c.buffer((8, 32), R.BF16, name="x"), c.buffer((8, 32), R.BF16, name="o")
+    emit("bf16_gelu", c, c.sink((o, x.gelu())),
+         {x: R.f32_to_bf16_bits(g.normal(0, 1.5, 256)), o: np.zeros(256, np.uint16)})
+    c.close()
+    c = R.Ctx()
+    A, Bm, O, sink = graphs.matmul_bf16(c, 24, 40, 48)
+    emit("bf16_matmul", c, sink, {A: R.f32_to_bf16_bits(g.normal(0, 0.02, 24 * 48)), Bm: R.f32_to_bf16_bits(g.normal(0, 0.02, 48 * 40)),
+                                  O: np.zeros(24 * 40, np.float32)})
+    c.close()
+    c = R.Ctx()
+    A, Bm, O, sink = graphs.matmul_bf16(c, 16, 24, 32, transposed_b=True, batch=3)
+    emit("bf16_matmul_bt_batch", c, sink, {A: R.f32_to_bf16_bits(g.normal(0, 0.02, 3 * 16 * 32)), Bm: R.f32_to_bf16_bits(g.normal(0, 0.02, 24 * 32)),
+                                           O: np.zeros(3 * 16 * 24, np.float32)})
+    c.close()
+
+    # fp16 casts and arithmetic (test/test_f16.c)
+    c = R.Ctx()
+    x, o = c.buffer((64,), R.F32, name="x"), c.buffer((64,), R.F16, name="o")
+    xs = np.concatenate([g.normal(0, 100, 56).astype(np.float32),
+                         np.array([0, -0.0, 65504, 65520, 1e-8, 6e-8, 6.1e-5, np.inf], np.float32)])
+    emit("f16_cast_mul", c, c.sink((o, x.cast(R.F16) * x.cast(R.F16))), {x: xs, o: np.zeros(64, np.float16)})
+    c.close()
+
+    # tiny GPT-2, fp32 and bf16 (2 layers, d_model 32, vocab 97, T=16, B=2)
+    for wdt, nm in ((R.F32, "f32"), (R.BF16, "bf16")):
+        c = R.Ctx()
+        sink, bufs = graphs.gpt2_forward(c, graphs.GPT2_TINY, wdt)
+        arrays = graphs.gpt2_inputs(graphs.GPT2_TINY, bufs, seed=3, wdt=wdt)
+        emit(f"gpt2_tiny_{nm}", c, sink, arrays)
+        c.close()
+
+
+if __name__ == "__main__":
+    main()

@@ -1,0 +1,214 @@
+"""Tensor-level graphs of the benchmark configurations, built through the REAL
+reference frontend (tests/refpoly.py).  Test infrastructure only.
+
+gpt2_forward follows the topology of the reference's GPT-2 builder
+(src/modelzoo/models/gpt2.c:320-526: one-hot embedding, pre-LayerNorm blocks,
+Conv1D-style linears, additive causal mask, softmax, GELU, tied LM head, a
+realize barrier after every op) and adds the bf16 variant the benchmark names:
+bf16 buffers, CAST to f32 in front of every reduction (matmul, LayerNorm
+statistics, softmax max/sum, embedding sum) and CAST back to bf16 after it.
+"""
+import math
+
+import numpy as np
+
+import refpoly as R
+
+
+class GPT2Config:
+    def __init__(self, n_layer=12, n_head=12, d_model=768, vocab=50257, ctx=1024, batch=8, eps=1e-5):
+        self.n_layer, self.n_head, self.d_model, self.vocab, self.ctx, self.batch, self.eps = \
+            n_layer, n_head, d_model, vocab, ctx, batch, eps
+
+    def key(self):
+        return f"L{self.n_layer}_H{self.n_head}_D{self.d_model}_V{self.vocab}_T{self.ctx}_B{self.batch}"
+
+
+GPT2_SMALL = GPT2Config()
+GPT2_TINY = GPT2Config(n_layer=2, n_head=2, d_model=32, vocab=97, ctx=16, batch=2)
+
+
+def _embedding(c, table, n_rows, d, idx, idx_shape, arange, wdt):
+    """out[..., j] = sum_v where(idx[...] == arange[v], table[v, j], 0)  (src/modelzoo/models/gpt2.c:93-153)."""
+    nd = len(idx_shape)
+    idx_e = idx.reshape(idx_shape + (1,)).expand(idx_shape + (n_rows,))
+    ar_e = arange.reshape((1,) * nd + (n_rows,)).expand(idx_shape + (n_rows,))
+    mask = idx_e.eq(ar_e).reshape(idx_shape + (n_rows, 1)).expand(idx_shape + (n_rows, d))
+    tbl = table.reshape((1,) * nd + (n_rows, d)).expand(idx_shape + (n_rows, d))
+    if wdt != R.F32:
+        tbl = tbl.cast(R.F32)
+    sel = mask.where(tbl, c.const(0.0))
+    out = sel.reduce_axes("ADD", [nd]).reshape(idx_shape + (d,))
+    return out.cast(wdt) if wdt != R.F32 else out
+
+
+def _linear(x, w, b, wdt):
+    """x @ w + b with HF Conv1D weight layout (in, out); f32 accumulate."""
+    if wdt != R.F32:
+        y = x.cast(R.F32).dot(w.cast(R.F32)).cast(wdt)
+    else:
+        y = x.dot(w)
+    if b is not None:
+        y = y + b.reshape((1,) * (len(y.shape) - 1) + (b.shape[-1],)).expand(y.shape)
+    return y
+
+
+def _layernorm(x, w, b, eps, wdt):
+    d = x.shape[-1]
+    xf = x.cast(R.F32) if wdt != R.F32 else x
+    y = xf.layernorm(eps)
+    if wdt != R.F32:
+        y = y.cast(wdt)
+    bc = (1,) * (len(x.shape) - 1) + (d,)
+    return y * w.reshape(bc).expand(x.shape) + b.reshape(bc).expand(x.shape)
+
+
+def gpt2_forward(c, cfg, wdt=R.BF16):
+    """Returns (sink, bufs) where bufs maps names to buffer T's; logits go to bufs['output']."""
+    V, D, H, L, T, B = cfg.vocab, cfg.d_model, cfg.n_head, cfg.n_layer, cfg.ctx, cfg.batch
+    hd = D // H
+    bufs = {}
+
+    def P(name, shape, dt=None):
+        bufs[name] = c.buffer(shape, wdt if dt is None else dt, name=name)
+        return bufs[name]
+
+    wte = P("wte.weight", (V, D))
+    wpe = P("wpe.weight", (T, D))
+    layers = []
+    for i in range(L):
+        p = f"h.{i}."
+        layers.append(dict(
+            ln1_w=P(p + "ln_1.weight", (D,)), ln1_b=P(p + "ln_1.bias", (D,)),
+            attn_w=P(p + "attn.c_attn.weight", (D, 3 * D)), attn_b=P(p + "attn.c_attn.bias", (3 * D,)),
+            proj_w=P(p + "attn.c_proj.weight", (D, D)), proj_b=P(p + "attn.c_proj.bias", (D,)),
+            ln2_w=P(p + "ln_2.weight", (D,)), ln2_b=P(p + "ln_2.bias", (D,)),
+            fc_w=P(p + "mlp.c_fc.weight", (D, 4 * D)), fc_b=P(p + "mlp.c_fc.bias", (4 * D,)),
+            fc2_w=P(p + "mlp.c_proj.weight", (4 * D, D)), fc2_b=P(p + "mlp.c_proj.bias", (D,))))
+    lnf_w, lnf_b = P("ln_f.weight", (D,)), P("ln_f.bias", (D,))
+    # token ids, positions and the aranges are FLOAT buffers, as in the reference
+    x = P("x", (B, T), R.F32)
+    out = P("output", (B, T, V))
+    pos = P("positions", (1, T), R.F32)
+    arange = P("arange", (T,), R.F32)
+    varange = P("vocab_arange", (V,), R.F32)
+
+    tok = _embedding(c, wte, V, D, x, (B, T), varange, wdt).contiguous()
+    pe = _embedding(c, wpe, T, D, pos, (1, T), arange, wdt).contiguous()
+    h = (tok + pe.expand((B, T, D))).contiguous()
+
+    row = arange.reshape((T, 1)).expand((T, T))
+    col = arange.reshape((1, T)).expand((T, T))
+    mask = row.lt(col).where(c.const(-1e9, wdt), c.const(0.0, wdt)).reshape((1, 1, T, T)).contiguous()
+
+    scale = 1.0 / math.sqrt(hd)
+    for lp in layers:
+        ln1 = _layernorm(h, lp["ln1_w"], lp["ln1_b"], cfg.eps, wdt).contiguous()
+        qkv = _linear(ln1, lp["attn_w"], lp["attn_b"], wdt).contiguous()
+        q = qkv.shrink(((0, B), (0, T), (0, D))).contiguous()
+        k = qkv.shrink(((0, B), (0, T), (D, 2 * D))).contiguous()
+        v = qkv.shrink(((0, B), (0, T), (2 * D, 3 * D))).contiguous()
+        q = q.reshape((B, T, H, hd)).permute((0, 2, 1, 3))
+        k = k.reshape((B, T, H, hd)).permute((0, 2, 1, 3))
+        v = v.reshape((B, T, H, hd)).permute((0, 2, 1, 3))
+        kt = k.permute((0, 1, 3, 2))
+        if wdt != R.F32:
+            scores = q.cast(R.F32).dot(kt.cast(R.F32)).cast(wdt).contiguous()
+        else:
+            scores = q.dot(kt).contiguous()
+        scores = (scores * c.const(scale, wdt) + mask.expand((B, H, T, T))).contiguous()
+        if wdt != R.F32:
+            attn = scores.cast(R.F32).softmax(-1).cast(wdt).contiguous()
+            ctxv = attn.cast(R.F32).dot(v.cast(R.F32)).cast(wdt).contiguous()
+        else:
+            attn = scores.softmax(-1).contiguous()
+            ctxv = attn.dot(v).contiguous()
+        merged = ctxv.permute((0, 2, 1, 3)).reshape((B, T, D))
+        a_out = _linear(merged, lp["proj_w"], lp["proj_b"], wdt).contiguous()
+        h = (h + a_out).contiguous()
+        ln2 = _layernorm(h, lp["ln2_w"], lp["ln2_b"], cfg.eps, wdt).contiguous()
+        ff = _linear(ln2, lp["fc_w"], lp["fc_b"], wdt).contiguous()
+        ff = ff.gelu().contiguous()
+        ff = _linear(ff, lp["fc2_w"], lp["fc2_b"], wdt).contiguous()
+        h = (h + ff).contiguous()
+
+    h = _layernorm(h, lnf_w, lnf_b, cfg.eps, wdt).contiguous()
+    wte_t = wte.reshape((V, D)).permute((1, 0))
+    if wdt != R.F32:
+        logits = h.cast(R.F32).dot(wte_t.cast(R.F32)).cast(wdt)
+    else:
+        logits = h.dot(wte_t)
+    sink = c.sink((out, logits))
+    return sink, bufs
+
+
+def gpt2_inputs(cfg, bufs, seed=3, wdt=R.BF16):
+    """Random-init weights and inputs per the benchmark config: weights ~ N(0, 0.02),
+    LayerNorm weights 1, biases 0, token ids uniform in [0, vocab) stored as floats."""
+    g = np.random.default_rng(seed)
+    arrays = {}
+    for name, t in bufs.items():
+        n = int(np.prod(t.shape))
+        if name == "x":
+            a = g.integers(0, cfg.vocab, n).astype(np.float32)
+        elif name in ("positions", "arange"):
+            a = np.arange(cfg.ctx, dtype=np.float32)
+        elif name == "vocab_arange":
+            a = np.arange(cfg.vocab, dtype=np.float32)
+        elif name == "output":
+            a = np.zeros(n, np.float32)
+        elif name.endswith("ln_1.weight") or name.endswith("ln_2.weight") or name == "ln_f.weight":
+            a = np.ones(n, np.float32)
+        elif name.endswith(".bias"):
+            a = np.zeros(n, np.float32)
+        else:
+            a = g.normal(0.0, 0.02, n).astype(np.float32)
+        if t.dt == R.BF16:
+            a = R.f32_to_bf16_bits(a)
+        elif t.dt == R.F16:
+            a = a.astype(np.float16)
+        arrays[t] = a
+    return arrays
+
+
+def fused_rowops(c, rows, cols):
+    """Config 2: y = clamp(exp2(a*b + c), -4, 4); sum, max, softmax, LayerNorm over the last axis."""
+    a, b, d = (c.buffer((rows, cols), name=n) for n in ("a", "b", "c"))
+    y = (a * b + d).exp2().clamp(-4, 4)
+    outs = {"sum": c.buffer((rows,), name="sum"), "max": c.buffer((rows,), name="max"),
+            "softmax": c.buffer((rows, cols), name="softmax"), "layernorm": c.buffer((rows, cols), name="layernorm")}
+    sinks = {"sum": c.sink((outs["sum"], y.sum())), "max": c.sink((outs["max"], y.max())),
+             "softmax": c.sink((outs["softmax"], y.softmax())),
+             "layernorm": c.sink((outs["layernorm"], y.layernorm(1e-5)))}
+    return (a, b, d), outs, sinks
+
+
+def matmul_bf16(c, m, n, k, transposed_b=False, batch=None):
+    """Config 3: C = A@B, bf16 inputs, f32 accumulate and output."""
+    a_shape = (m, k) if batch is None else (batch, m, k)
+    A = c.buffer(a_shape, R.BF16, name="A")
+    if transposed_b:
+        Bm = c.buffer((n, k), R.BF16, name="B")
+        b = Bm.permute((1, 0))
+    else:
+        Bm = c.buffer((k, n), R.BF16, name="B")
+        b = Bm
+    O = c.buffer(a_shape[:-1] + (n,), R.F32, name="C")
+    sink = c.sink((O, A.cast(R.F32).dot(b.cast(R.F32))))
+    return A, Bm, O, sink
+
+
+def mlp_train_step(c, batch=4096, d_in=784, d_hid=512, d_out=10, lr=0.01):
+    """Config 1: 2-layer MLP forward + backward + one SGD step, built from the public
+    ops (the reference's own loss entrypoints fail for batch > 1)."""
+    X = c.buffer((batch, d_in), name="X")
+    W1 = c.buffer((d_hid, d_in), name="W1")
+    b1 = c.buffer((d_hid,), name="b1")
+    W2 = c.buffer((d_out, d_hid), name="W2")
+    b2 = c.buffer((d_out,), name="b2")
+    Y = c.buffer((batch, d_out), name="Y")  # one-hot labels
+    h = (X.dot(W1.permute((1, 0))) + b1.reshape((1, d_hid)).expand((batch, d_hid))).relu()
+    logits = h.dot(W2.permute((1, 0))) + b2.reshape((1, d_out)).expand((batch, d_out))
+    logp = logits.log_softmax(-1)
+    loss = (logp * Y).sum().sum(0) * c.const(-1.0 / batch)
+    return dict(X=X, W1=W1, b1=b1, W2=W2, b2=b2, Y=Y), logits, loss

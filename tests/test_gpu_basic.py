@@ -41,12 +41,16 @@ def test_row_reductions_fp32(cols):
     x = c.buffer(shape, name="x")
     s_out, m_out = c.buffer((96,), name="sum"), c.buffer((96,), name="max")
     arrays = {x: g.uniform(-1, 1, shape).astype(np.float32), s_out: np.zeros(96, np.float32), m_out: np.zeros(96, np.float32)}
+    # A sum with cancellation is only defined to within the rounding of its
+    # terms: the bound is rtol * sum(|x|) (the CPU's left-to-right order and the
+    # GPU's tree order are both within it), which for same-sign data is plain rtol.
+    atol = 1e-6 * float(np.abs(arrays[x]).sum(axis=1).max())
     for out, val in ((s_out, x.sum()), (m_out, x.max())):
         sink = c.sink((out, val))
         sub = {x: arrays[x], out: arrays[out]}
         want = run_ref(c, sink, sub)
         got, _ = run_hip(c, sink, sub)
-        assert_close(got[out], want[out], rtol=1e-4, atol=1e-6, what=f"reduce cols={cols}")
+        assert_close(got[out], want[out], rtol=1e-4, atol=atol, what=f"reduce cols={cols}")
     c.close()
 
 

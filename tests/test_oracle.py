@@ -1,0 +1,108 @@
+"""Pins the CPU oracle (oracle/oracle.c) -- CPU only, no GPU needed.
+
+1. Scalar pieces against closed forms and independent implementations.
+2. Every committed golden fixture (outputs of the REAL reference CPU backend,
+   tests/golden/make_golden.py) -- including the reference's own known-answer
+   vectors (matmul 2x3.3x4, threefry key 1337, uniform-logit cross-entropy).
+3. Where the reference library is built, random graphs against it, bit for bit.
+"""
+import math
+
+import numpy as np
+import pytest
+
+import fixtures as F
+
+# Fixtures the oracle must reproduce bit for bit (it restates the arithmetic exactly).
+BIT_EXACT = {"kat_matmul_2x3x4", "kat_threefry_u32", "kat_threefry_u64", "movement_i32", "int_alu",
+             "rowops_sum", "rowops_max", "rowops_softmax", "rowops_layernorm", "special_exp2", "special_log2",
+             "bf16_matmul", "bf16_matmul_bt_batch", "f16_cast_mul", "kat_xent_uniform", "gpt2_tiny_f32",
+             "bf16_gelu", "gpt2_tiny_bf16"}
+
+
+def test_bf16_conversion_is_round_to_nearest_even():
+    o = F.oracle()
+    # exactly representable, ties, NaN, inf (test/test_f16.c cast patterns)
+    cases = {1.0: 0x3F80, -2.0: 0xC000, 0.0: 0x0000, float("inf"): 0x7F80, 1.00390625: 0x3F80, 1.01171875: 0x3F82,
+             3.140625: 0x4049, 65280.0: 0x477F}
+    for x, bits in cases.items():
+        assert o.oracle_f32_to_bf16(x) == bits, x
+    assert o.oracle_f32_to_bf16(float("nan")) & 0x7FC0 == 0x7FC0
+    # brute force: every bf16 value round-trips; midpoints go to the even neighbour
+    for h in range(0, 0x7F80, 97):
+        f = o.oracle_bf16_to_f32(h)
+        assert o.oracle_f32_to_bf16(f) == h
+        up = o.oracle_bf16_to_f32(h + 1)
+        mid = np.float32((np.float64(f) + np.float64(up)) / 2)
+        assert o.oracle_f32_to_bf16(float(mid)) == (h if h % 2 == 0 else h + 1)
+
+
+def test_f16_conversion_matches_ieee_half():
+    o = F.oracle()
+    g = np.random.default_rng(0)
+    xs = np.concatenate([g.normal(0, 1000, 2000), g.normal(0, 1e-5, 2000), [0.0, -0.0, 65504, 65519.9, 65520, 1e-8, 5.96e-8, 2.98e-8, 6.1e-5]]).astype(np.float32)
+    for x in xs:
+        want = int(np.float32(x).astype(np.float16).view(np.uint16))
+        assert o.oracle_f32_to_f16(float(x)) == want, x
+    for h in range(0, 0x7C00, 53):
+        assert o.oracle_f16_to_f32(h) == float(np.uint16(h).view(np.float16))
+
+
+def test_exp2_log2_closed_forms_and_accuracy():
+    o = F.oracle()
+    for k in range(-126, 128):
+        assert o.oracle_exp2f(float(k)) == 2.0 ** k
+        assert o.oracle_log2f(2.0 ** k) == float(k)
+    assert o.oracle_exp2f(128.0) == math.inf and o.oracle_exp2f(-151.0) == 0.0
+    assert math.isnan(o.oracle_exp2f(math.nan)) and o.oracle_exp2f(-math.inf) == 0.0 and o.oracle_exp2f(math.inf) == math.inf
+    assert o.oracle_log2f(0.0) == -math.inf and math.isnan(o.oracle_log2f(-1.0)) and o.oracle_log2f(math.inf) == math.inf
+    assert o.oracle_log2f(-0.0) == -math.inf
+    g = np.random.default_rng(1)
+    for x in g.uniform(-120, 120, 3000).astype(np.float32):
+        assert abs(o.oracle_exp2f(float(x)) - 2.0 ** float(x)) <= 4e-7 * 2.0 ** float(x)
+    for x in np.exp(g.uniform(-80, 80, 3000)).astype(np.float32):
+        assert abs(o.oracle_log2f(float(x)) - math.log2(float(x))) <= 4e-7 * max(1.0, abs(math.log2(float(x))))
+    for x in g.uniform(-1000, 1000, 2000):
+        assert abs(o.oracle_exp2(float(x)) - 2.0 ** float(x)) <= 1e-15 * 2.0 ** float(x)
+    for x in np.exp(g.uniform(-300, 300, 2000)):
+        assert abs(o.oracle_log2(float(x)) - math.log2(float(x))) <= 2e-15 * max(1.0, abs(math.log2(float(x))))
+
+
+def test_threefry_known_answers():
+    # JAX threefry2x32, key 1337, counters 0..19 (reference test/test_nn.c:1126-1131, 1161-1169)
+    ref32 = [2732499619, 3322027265, 2482432314, 3871860445, 3571867126, 3019569655, 2459680734, 2731866067,
+             986922480, 1616040745, 4238711754, 3594775990, 3046419939, 3519108299, 586160567, 3928687287,
+             4074505382, 4210472430, 4094881238, 3306411770]
+    ref64 = [2091981003842036387, 7289724007706926337, 5665610599518103866, 1710967476831381213,
+             10223482319493553654, 17028600460329286135, 17124603982541209566, 3105577853879908307,
+             2086892522412654064, 3335679299718140713, 16051258882154404810, 6689751810128997814,
+             14143017499898457571, 15433975895207007435, 585627789352245687, 6751685475094430391,
+             13535415641566872742, 11824248585908041198, 12094218887010381270, 17901838715724224250]
+    o = F.oracle()
+    for i in range(20):
+        v = o.oracle_threefry(i, 1337)
+        assert v == ref64[i]
+        assert v & 0xFFFFFFFF == ref32[i]
+
+
+@pytest.mark.parametrize("name", F.case_names())
+def test_oracle_reproduces_reference_fixture(name):
+    fx = F.Fixture(name)
+    got = F.run_oracle_schedule(fx.plan.schedule, fx.n_slots, fx.inputs)
+    for slot in fx.external:
+        want = fx.expected[slot]
+        have = got[slot]
+        if name in BIT_EXACT:
+            assert have.tobytes() == want.tobytes(), f"{name}: slot {slot} ({fx.plan.names[slot]}) differs from the reference"
+        else:
+            np.testing.assert_allclose(F.as_float(have), F.as_float(want), rtol=1e-6, atol=1e-7)
+
+
+def test_kat_values_are_the_published_ones():
+    # the fixtures themselves hold the values the reference's tests assert
+    fx = F.Fixture("kat_matmul_2x3x4")
+    out = [i for i in fx.external if fx.plan.names[i] == "O"][0]
+    assert fx.expected[out].tolist() == [38, 44, 50, 56, 83, 98, 113, 128]
+    fx = F.Fixture("kat_xent_uniform")
+    out = [i for i in fx.external if fx.plan.names[i] == "loss"][0]
+    assert abs(float(fx.expected[out][0]) - math.log(3.0)) < 1e-6
