@@ -88,6 +88,12 @@ char *poly_hip_describe(PolyUOp *scheduled_root, int flags);
 /* Compiles source for gfx950 with hiprtc only (no device needed). 0 = ok. */
 int poly_hip_compile_check(const char *source);
 void poly_hip_free_string(char *s);
+/* Self-check used by the CPU tests: evaluates every integer index expression of
+ * the kernel both as written and in the simplified form the renderer emits, at
+ * `samples` points of the iteration space.  Returns the number of mismatches
+ * (0 = consistent), <0 on a malformed root.  No reference counterpart: the
+ * reference relies on its symbolic pass (src/sym.c) being right. */
+int poly_hip_check_index_simplification(PolyUOp *scheduled_root, int samples);
 
 /* ── Plan level (replaces src/exec_plan.c:801-1096 for this device) ─────── */
 

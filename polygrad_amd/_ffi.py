@@ -87,6 +87,7 @@ SYMBOLS = {
     "poly_hip_describe": (C.c_void_p, [C.c_void_p, C.c_int]),
     "poly_hip_compile_check": (C.c_int, [C.c_char_p]),
     "poly_hip_free_string": (None, [C.c_void_p]),
+    "poly_hip_check_index_simplification": (C.c_int, [C.c_void_p, C.c_int]),
     "poly_hip_compile_schedule": (C.c_void_p, [C.c_void_p, C.c_void_p]),
     "poly_hip_plan_run": (C.c_int, [C.c_void_p, C.POINTER(C.c_void_p), C.c_int, C.c_void_p, C.c_int]),
     "poly_hip_plan_free": (None, [C.c_void_p]),

@@ -238,4 +238,13 @@ int poly_hip_compile_check(const char *source) {
 
 void poly_hip_free_string(char *s) { free(s); }
 
+int poly_hip_check_index_simplification(PolyUOp *scheduled_root, int samples) {
+  KernelGraph g;
+  if (!scheduled_root || !g.build(scheduled_root)) return -1;
+  std::string bad;
+  int n = g.check_lins(samples > 0 ? samples : 4096, &bad);
+  if (n > 0) log_err("render_hip", "index simplification self-check: %d mismatches, first: %s", n, bad.c_str());
+  return n;
+}
+
 }  // extern "C"

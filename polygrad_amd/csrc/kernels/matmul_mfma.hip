@@ -1,0 +1,287 @@
+// matmul_mfma.hip -- hand-written CDNA4 (gfx950) matmul template.
+//
+// C[z][m][n] = epilogue( sum_k A(z,m,k) * B(z,k,n) ) with 16-bit float inputs
+// (bf16 or fp16) and fp32 accumulation on the 32x32x16 MFMA.  The renderer
+// (templates.cc) instantiates it by prepending a configuration block:
+//
+//   POLY_TIN            input element type (__bf16 or _Float16)
+//   POLY_MFMA(a,b,c)    the MFMA builtin for that type
+//   POLY_M/N/K/Z        problem sizes (rows, columns, depth, batch)
+//   POLY_BM/BN/BK       workgroup tile; 4 waves as POLY_WM x POLY_WN
+//   POLY_A_KC/B_KC      1: operand is contiguous along K in memory (16-byte loads
+//                       along K); 0: contiguous along M (resp. N): 16-byte loads
+//                       along that axis and a register transpose on the way to LDS
+//   POLY_A_PTR/B_PTR    the kernel parameters holding A and B
+//   poly_a_row(m), poly_b_row(n), poly_a_z(z), poly_b_z(z), poly_a_k(k), poly_b_k(k)
+//                       element offsets contributed by each coordinate
+//   POLY_SIGNATURE      the kernel's parameter list
+//   POLY_EPILOGUE(acc, m, n, z)   stores one finished element (generated from the
+//                       UOps around the REDUCE: casts, bias, activation, index)
+//
+// Data path: global --16B loads--> registers --(transpose if needed)--> LDS
+// [row][K] with padded rows, double buffered; each wave reads 16-byte A and B
+// fragments and issues (WM/32)*(WN/32) MFMAs per 16-deep K step.
+#ifdef POLY_TEMPLATE_STANDALONE
+#include <hip/hip_runtime.h>
+#define POLY_TIN __bf16
+#define POLY_MFMA(a, b, c) __builtin_amdgcn_mfma_f32_32x32x16_bf16(a, b, c, 0, 0, 0)
+#define POLY_M 4096
+#define POLY_N 4096
+#define POLY_K 4096
+#define POLY_Z 1
+#define POLY_BM 128
+#define POLY_BN 128
+#define POLY_BK 64
+#define POLY_WAVES_M 2
+#define POLY_WAVES_N 2
+#define POLY_A_KC 1
+#define POLY_B_KC 0
+#define POLY_A_PTR data1
+#define POLY_B_PTR data2
+__device__ __forceinline__ int poly_a_row(int m) { return m * POLY_K; }
+__device__ __forceinline__ int poly_b_row(int n) { return n; }
+__device__ __forceinline__ int poly_a_z(int z) { return 0; }
+__device__ __forceinline__ int poly_b_z(int z) { return 0; }
+__device__ __forceinline__ int poly_a_k(int k) { return k; }
+__device__ __forceinline__ int poly_b_k(int k) { return k * POLY_N; }
+#define POLY_SIGNATURE float *data0, const __bf16 *__restrict__ data1, const __bf16 *__restrict__ data2
+#define POLY_EPILOGUE(acc, m, n, z) data0[(m) * POLY_N + (n)] = (acc)
+#endif
+
+typedef POLY_TIN poly_in8 __attribute__((ext_vector_type(8)));
+typedef POLY_TIN poly_in4 __attribute__((ext_vector_type(4)));
+typedef float poly_acc16 __attribute__((ext_vector_type(16)));
+typedef unsigned int poly_u32x4 __attribute__((ext_vector_type(4)));
+typedef unsigned int poly_u32x2 __attribute__((ext_vector_type(2)));
+typedef poly_u32x4 poly_u32x4_u __attribute__((aligned(2)));
+
+#define POLY_WM (POLY_BM / POLY_WAVES_M)
+#define POLY_WN (POLY_BN / POLY_WAVES_N)
+#define POLY_TM (POLY_WM / 32)
+#define POLY_TN (POLY_WN / 32)
+#define POLY_NTHREADS (64 * POLY_WAVES_M * POLY_WAVES_N)
+// LDS row: BK elements + 8 elements (16 bytes) of padding keeps 16-byte fragment
+// reads of 8 consecutive rows on distinct banks.
+#define POLY_LDK (POLY_BK + 8)
+#define POLY_KT (POLY_K / POLY_BK)
+
+// Number of 16-byte global loads per thread for one operand tile.
+#define POLY_A_LOADS ((POLY_BM * POLY_BK / 8) / POLY_NTHREADS)
+#define POLY_B_LOADS ((POLY_BN * POLY_BK / 8) / POLY_NTHREADS)
+
+// ── K-contiguous operand: thread -> (row, 8-wide k chunk) ──────────────────
+// chunks per row = BK/8; consecutive threads walk along K first (full 128-byte
+// lines per row when BK = 64).
+template <int ROWS, int NLOADS>
+struct PolyKC {
+  static __device__ __forceinline__ void load(const POLY_TIN *__restrict__ base, const int *row_off, int kofs,
+                                              poly_u32x4 (&regs)[NLOADS]) {
+#pragma unroll
+    for (int i = 0; i < NLOADS; i++) {
+      const int c = threadIdx.x + i * POLY_NTHREADS;
+      const int kc = c % (POLY_BK / 8);
+      regs[i] = *(const poly_u32x4_u *)(base + row_off[i] + kofs + kc * 8);
+    }
+  }
+  static __device__ __forceinline__ void store(POLY_TIN *lds, const poly_u32x4 (&regs)[NLOADS]) {
+#pragma unroll
+    for (int i = 0; i < NLOADS; i++) {
+      const int c = threadIdx.x + i * POLY_NTHREADS;
+      const int row = c / (POLY_BK / 8), kc = c % (POLY_BK / 8);
+      *(poly_u32x4 *)(lds + row * POLY_LDK + kc * 8) = regs[i];
+    }
+  }
+};
+
+// ── operand contiguous along its row axis (M or N): thread -> (8-wide row chunk,
+// group of 4 k) ; 4 loads of 16 bytes give a 4(k) x 8(row) block that is
+// transposed in registers into 8 rows x 4 k and written as 8-byte LDS stores.
+// When the tile has fewer 4x8 blocks than the workgroup has threads, the upper
+// threads sit the staging out. ──
+template <int ROWS>
+struct PolyXC {
+  static constexpr int CHUNKS = ROWS / 8;                 // row chunks per tile
+  static constexpr int TOTAL = CHUNKS * (POLY_BK / 4);    // 4x8 blocks per tile
+  static constexpr int NBLK = (TOTAL + POLY_NTHREADS - 1) / POLY_NTHREADS;
+  static constexpr int NLOADS = NBLK * 4;
+  static __device__ __forceinline__ void load(const POLY_TIN *__restrict__ base, const int *chunk_off, const int *k_off,
+                                              poly_u32x4 (&regs)[NLOADS]) {
+#pragma unroll
+    for (int b = 0; b < NBLK; b++) {
+      if (TOTAL % POLY_NTHREADS == 0 || (int)threadIdx.x + b * POLY_NTHREADS < TOTAL) {
+#pragma unroll
+        for (int i = 0; i < 4; i++) regs[b * 4 + i] = *(const poly_u32x4_u *)(base + chunk_off[b] + k_off[b * 4 + i]);
+      }
+    }
+  }
+  static __device__ __forceinline__ void store(POLY_TIN *lds, const poly_u32x4 (&regs)[NLOADS]) {
+#pragma unroll
+    for (int b = 0; b < NBLK; b++) {
+      const int c = threadIdx.x + b * POLY_NTHREADS;
+      if (TOTAL % POLY_NTHREADS != 0 && c >= TOTAL) continue;
+      const int chunk = c % CHUNKS, kq = c / CHUNKS;
+#pragma unroll
+      for (int j = 0; j < 4; j++) {
+        // dword j of load i holds rows 2j (low half) and 2j+1 (high half) at k = kq*4+i
+        const unsigned int a0 = regs[b * 4 + 0][j], a1 = regs[b * 4 + 1][j], a2 = regs[b * 4 + 2][j], a3 = regs[b * 4 + 3][j];
+        poly_u32x2 lo, hi;
+        lo[0] = (a0 & 0xffffu) | (a1 << 16);
+        lo[1] = (a2 & 0xffffu) | (a3 << 16);
+        hi[0] = (a0 >> 16) | (a1 & 0xffff0000u);
+        hi[1] = (a2 >> 16) | (a3 & 0xffff0000u);
+        *(poly_u32x2 *)(lds + (chunk * 8 + 2 * j) * POLY_LDK + kq * 4) = lo;
+        *(poly_u32x2 *)(lds + (chunk * 8 + 2 * j + 1) * POLY_LDK + kq * 4) = hi;
+      }
+    }
+  }
+};
+
+extern "C" __global__ void __launch_bounds__(POLY_NTHREADS) poly_k(POLY_SIGNATURE) {
+  __shared__ __attribute__((aligned(16))) POLY_TIN lds_a[2][POLY_BM * POLY_LDK];
+  __shared__ __attribute__((aligned(16))) POLY_TIN lds_b[2][POLY_BN * POLY_LDK];
+
+  // Tile coordinates.  Consecutive workgroup ids go to different XCDs (8 of them,
+  // each with its own L2), so ids are regrouped: all ids congruent mod 8 form one
+  // contiguous run of tiles, and runs walk down M within a band of columns so the
+  // B panel stays resident in that XCD's L2.
+  constexpr int TILES_M = (POLY_M + POLY_BM - 1) / POLY_BM;
+  constexpr int TILES_N = (POLY_N + POLY_BN - 1) / POLY_BN;
+  constexpr int NT = TILES_M * TILES_N;
+  int bid = blockIdx.x;
+  {
+    constexpr int PER = NT / 8, REM = NT % 8;
+    const int xcd = bid & 7, idx = bid >> 3;
+    bid = (xcd < REM ? xcd * (PER + 1) : REM * (PER + 1) + (xcd - REM) * PER) + idx;
+  }
+  const int tile_m = bid % TILES_M, tile_n = bid / TILES_M;
+  const int z = blockIdx.y;
+  const int m0 = tile_m * POLY_BM, n0 = tile_n * POLY_BN;
+
+  const POLY_TIN *__restrict__ gA = POLY_A_PTR + poly_a_z(z);
+  const POLY_TIN *__restrict__ gB = POLY_B_PTR + poly_b_z(z);
+
+  // Per-thread global offsets of the rows (or row chunks) this thread stages.
+  // Rows past the edge are clamped to the last valid row: they are loaded and
+  // multiplied but never stored.
+#if POLY_A_KC
+  poly_u32x4 ra[POLY_A_LOADS];
+  int a_off[POLY_A_LOADS];
+#pragma unroll
+  for (int i = 0; i < POLY_A_LOADS; i++) {
+    int row = m0 + (threadIdx.x + i * POLY_NTHREADS) / (POLY_BK / 8);
+    a_off[i] = poly_a_row(row < POLY_M ? row : POLY_M - 1);
+  }
+  typedef PolyKC<POLY_BM, POLY_A_LOADS> StageA;
+#else
+  typedef PolyXC<POLY_BM> StageA;
+  poly_u32x4 ra[StageA::NLOADS];
+  int a_off[StageA::NBLK], a_kq[StageA::NBLK];
+#pragma unroll
+  for (int b = 0; b < StageA::NBLK; b++) {
+    const int c = (threadIdx.x + b * POLY_NTHREADS) % StageA::TOTAL;
+    int row = m0 + (c % (POLY_BM / 8)) * 8;
+    a_off[b] = poly_a_row(row < POLY_M ? row : POLY_M - 8);
+    a_kq[b] = (c / (POLY_BM / 8)) * 4;
+  }
+#endif
+#if POLY_B_KC
+  poly_u32x4 rb[POLY_B_LOADS];
+  int b_off[POLY_B_LOADS];
+#pragma unroll
+  for (int i = 0; i < POLY_B_LOADS; i++) {
+    int row = n0 + (threadIdx.x + i * POLY_NTHREADS) / (POLY_BK / 8);
+    b_off[i] = poly_b_row(row < POLY_N ? row : POLY_N - 1);
+  }
+  typedef PolyKC<POLY_BN, POLY_B_LOADS> StageB;
+#else
+  typedef PolyXC<POLY_BN> StageB;
+  poly_u32x4 rb[StageB::NLOADS];
+  int b_off[StageB::NBLK], b_kq[StageB::NBLK];
+#pragma unroll
+  for (int b = 0; b < StageB::NBLK; b++) {
+    const int c = (threadIdx.x + b * POLY_NTHREADS) % StageB::TOTAL;
+    int row = n0 + (c % (POLY_BN / 8)) * 8;
+    b_off[b] = poly_b_row(row < POLY_N ? row : POLY_N - 8);
+    b_kq[b] = (c / (POLY_BN / 8)) * 4;
+  }
+#endif
+
+  auto load_tiles = [&](int kt) {
+    const int k0 = kt * POLY_BK;
+#if POLY_A_KC
+    StageA::load(gA, a_off, poly_a_k(k0), ra);
+#else
+    int ak[StageA::NLOADS];
+#pragma unroll
+    for (int b = 0; b < StageA::NBLK; b++)
+#pragma unroll
+      for (int i = 0; i < 4; i++) ak[b * 4 + i] = poly_a_k(k0 + a_kq[b] + i);
+    StageA::load(gA, a_off, ak, ra);
+#endif
+#if POLY_B_KC
+    StageB::load(gB, b_off, poly_b_k(k0), rb);
+#else
+    int bk[StageB::NLOADS];
+#pragma unroll
+    for (int b = 0; b < StageB::NBLK; b++)
+#pragma unroll
+      for (int i = 0; i < 4; i++) bk[b * 4 + i] = poly_b_k(k0 + b_kq[b] + i);
+    StageB::load(gB, b_off, bk, rb);
+#endif
+  };
+
+  const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
+  const int wm = (wave % POLY_WAVES_M) * POLY_WM, wn = (wave / POLY_WAVES_M) * POLY_WN;
+  const int frag_row = lane & 31, frag_k = (lane >> 5) * 8;
+
+  poly_acc16 acc[POLY_TM][POLY_TN];
+#pragma unroll
+  for (int i = 0; i < POLY_TM; i++)
+#pragma unroll
+    for (int j = 0; j < POLY_TN; j++)
+#pragma unroll
+      for (int r = 0; r < 16; r++) acc[i][j][r] = 0.0f;
+
+  load_tiles(0);
+  StageA::store(lds_a[0], ra);
+  StageB::store(lds_b[0], rb);
+  __syncthreads();
+
+  for (int kt = 0; kt < POLY_KT; kt++) {
+    const int cur = kt & 1;
+    if (kt + 1 < POLY_KT) load_tiles(kt + 1);
+    const POLY_TIN *la = lds_a[cur] + (wm + frag_row) * POLY_LDK + frag_k;
+    const POLY_TIN *lb = lds_b[cur] + (wn + frag_row) * POLY_LDK + frag_k;
+#pragma unroll
+    for (int ks = 0; ks < POLY_BK / 16; ks++) {
+      poly_in8 fa[POLY_TM], fb[POLY_TN];
+#pragma unroll
+      for (int i = 0; i < POLY_TM; i++) fa[i] = *(const poly_in8 *)(la + i * 32 * POLY_LDK + ks * 16);
+#pragma unroll
+      for (int j = 0; j < POLY_TN; j++) fb[j] = *(const poly_in8 *)(lb + j * 32 * POLY_LDK + ks * 16);
+#pragma unroll
+      for (int i = 0; i < POLY_TM; i++)
+#pragma unroll
+        for (int j = 0; j < POLY_TN; j++) acc[i][j] = POLY_MFMA(fa[i], fb[j], acc[i][j]);
+    }
+    if (kt + 1 < POLY_KT) {
+      StageA::store(lds_a[cur ^ 1], ra);
+      StageB::store(lds_b[cur ^ 1], rb);
+    }
+    __syncthreads();
+  }
+
+  // Accumulator layout of the 32x32 MFMA: register r of lane l holds
+  // row 8*(r/4) + 4*(l/32) + r%4, column l%32 of the tile.
+#pragma unroll
+  for (int i = 0; i < POLY_TM; i++)
+#pragma unroll
+    for (int j = 0; j < POLY_TN; j++) {
+      const int n = n0 + wn + j * 32 + (lane & 31);
+#pragma unroll
+      for (int r = 0; r < 16; r++) {
+        const int m = m0 + wm + i * 32 + 8 * (r >> 2) + 4 * (lane >> 5) + (r & 3);
+        if (m < POLY_M && n < POLY_N) { POLY_EPILOGUE(acc[i][j][r], m, n, z); }
+      }
+    }
+}

@@ -2,6 +2,7 @@
 
 #include <algorithm>
 #include <climits>
+#include <cstdlib>
 #include <cstring>
 
 namespace polyhip {
@@ -64,9 +65,22 @@ Lin KernelGraph::lin_recombine(const Lin &a) const {
     if (m.kind != Atom::MOD) continue;
     for (size_t j = 0; j < a.terms.size(); j++) {
       const Atom &d = atoms[(size_t)a.terms[j].atom];
-      if (d.kind != Atom::DIV || d.c != m.c) continue;
+      if (d.kind != Atom::DIV) continue;
       if (a.terms[j].coef != a.terms[i].coef * m.c) continue;
-      if (lin_key(d.inner) != lin_key(m.inner)) continue;
+      if (d.c != m.c || lin_key(d.inner) != lin_key(m.inner)) {
+        // nested form: c*(Y/(p*c)) + (Y/p)%c == Y/p
+        if (m.inner.c0 != 0 || m.inner.terms.size() != 1 || m.inner.terms[0].coef != 1) continue;
+        const Atom &in = atoms[(size_t)m.inner.terms[0].atom];
+        if (in.kind != Atom::DIV || d.c != in.c * m.c || lin_key(d.inner) != lin_key(in.inner)) continue;
+        int64_t lo2, hi2;
+        lin_bounds(in.inner, &lo2, &hi2);
+        if (lo2 < 0) continue;
+        Lin rest2;
+        rest2.c0 = a.c0;
+        for (size_t t = 0; t < a.terms.size(); t++)
+          if (t != i && t != j) rest2.terms.push_back(a.terms[t]);
+        return lin_recombine(lin_add(rest2, lin_scale(m.inner, a.terms[i].coef)));
+      }
       int64_t lo, hi;
       lin_bounds(d.inner, &lo, &hi);
       if (lo < 0) continue;
@@ -162,19 +176,35 @@ Lin KernelGraph::lin_div(const Lin &a, int64_t c) {
     lin_bounds(R, &rlo, &rhi);
     if (rlo >= 0) {
       if (rhi < c) return Q;
-      // reduce R and c by their common factor: (g*R')/(g*c') == R'/c'
-      int64_t g = c;
-      for (const Term &t : R.terms) g = gcd64(g, t.coef);
+      // floor((g*X + S) / (g*c')) == floor(X / c') when 0 <= S < g: split R into
+      // the terms whose coefficients share a factor g with c and a small rest S.
+      // Candidates for g: gcd of c with the coefficients not smaller than each term's.
       int64_t cc = c;
-      if (g > 1) {
-        // floor((g*R' + r0)/ (g*c')) == floor(R'/c') when 0 <= r0 < g
+      for (size_t pick = 0; pick <= R.terms.size(); pick++) {
+        int64_t thresh = pick < R.terms.size() ? std::llabs(R.terms[pick].coef) : 0;
+        if (pick == R.terms.size() && !R.terms.empty()) break;
+        int64_t g = c;
+        for (const Term &t : R.terms) if (std::llabs(t.coef) >= thresh) g = gcd64(g, t.coef);
+        if (g <= 1) continue;
+        Lin X, S;
+        for (const Term &t : R.terms) {
+          if (t.coef % g == 0) X.terms.push_back({t.coef / g, t.atom});
+          else S.terms.push_back(t);
+        }
         int64_t r0 = R.c0 % g;
-        Lin Rp;
-        Rp.c0 = (R.c0 - r0) / g;
-        for (const Term &t : R.terms) Rp.terms.push_back({t.coef / g, t.atom});
-        R = Rp;
+        X.c0 = (R.c0 - r0) / g;
+        S.c0 = r0;
+        int64_t slo, shi;
+        lin_bounds(S, &slo, &shi);
+        if (slo < 0 || shi >= g) continue;
+        int64_t xlo, xhi;
+        lin_bounds(X, &xlo, &xhi);
+        if (xlo < 0) continue;
+        R = X;
         cc = c / g;
         if (cc == 1) return lin_add(Q, R);
+        if (xhi < cc) return Q;
+        break;
       }
       Atom d;
       d.kind = Atom::DIV; d.inner = R; d.c = cc;
@@ -514,6 +544,91 @@ bool KernelGraph::build(const PolyUOp *root) {
     lins.push_back(out);
   }
   return true;
+}
+
+
+// ── self-check of the index simplifier ────────────────────────────────────
+
+namespace {
+struct RawEval {
+  const KernelGraph &g;
+  const std::vector<int64_t> &rv;   // value per range ordinal
+  bool ok = true;
+  int64_t node(int id) {
+    const KNode &k = g.n(id);
+    auto S = [&](size_t i) { return node(k.src[i]); };
+    switch (k.op) {
+      case POLY_OP_CONST: return k.u->arg.i;
+      case POLY_OP_RANGE: return rv[(size_t)g.range_ord.at(id)];
+      case POLY_OP_ADD: return S(0) + S(1);
+      case POLY_OP_SUB: return S(0) - S(1);
+      case POLY_OP_MUL: return S(0) * S(1);
+      case POLY_OP_NEG: return -S(0);
+      case POLY_OP_IDIV: { int64_t b = S(1); if (b == 0) { ok = false; return 0; } return (int64_t)((int32_t)S(0) / (int32_t)b); }
+      case POLY_OP_MOD: { int64_t b = S(1); if (b == 0) { ok = false; return 0; } return (int64_t)((int32_t)S(0) % (int32_t)b); }
+      case POLY_OP_SHL: return S(0) << (S(1) & 31);
+      case POLY_OP_SHR: return S(0) >> (S(1) & 31);
+      case POLY_OP_CAST:
+        if (g.n(k.src[0]).dt == DT_I32 || g.n(k.src[0]).dt == DT_INDEX) return S(0);
+        ok = false; return 0;
+      default: ok = false; return 0;
+    }
+  }
+  int64_t atom(int a) {
+    const Atom &at = g.atoms[(size_t)a];
+    switch (at.kind) {
+      case Atom::RANGE: return rv[(size_t)g.range_ord.at(at.node)];
+      case Atom::DIV: return lin(at.inner) / at.c;
+      case Atom::MOD: return lin(at.inner) % at.c;
+      case Atom::OPAQUE: return node_raw_opaque(at.node);
+      default: ok = false; return 0;
+    }
+  }
+  int64_t node_raw_opaque(int id) { return node(id); }
+  int64_t lin(const Lin &l) {
+    int64_t v = l.c0;
+    for (const Term &t : l.terms) v += t.coef * atom(t.atom);
+    return v;
+  }
+};
+}  // namespace
+
+int KernelGraph::check_lins(int samples, std::string *first_bad) const {
+  std::vector<int64_t> ext;
+  double space = 1;
+  for (const RangeInfo &r : ranges) { ext.push_back(r.extent > 0 ? r.extent : 1); space *= (double)ext.back(); }
+  std::vector<int64_t> rv(ranges.size(), 0);
+  int bad = 0;
+  uint64_t rng = 0x9E3779B97F4A7C15ull;
+  bool exhaustive = space <= (double)samples;
+  int64_t total = exhaustive ? (int64_t)space : samples;
+  for (int64_t it = 0; it < total; it++) {
+    if (exhaustive) {
+      int64_t t = it;
+      for (size_t r = 0; r < ext.size(); r++) { rv[r] = t % ext[r]; t /= ext[r]; }
+    } else {
+      for (size_t r = 0; r < ext.size(); r++) {
+        rng ^= rng << 13; rng ^= rng >> 7; rng ^= rng << 17;
+        uint64_t pick = rng % 8;
+        rv[r] = pick == 0 ? 0 : pick == 1 ? ext[r] - 1 : (int64_t)((rng >> 8) % (uint64_t)ext[r]);
+      }
+    }
+    for (int i = 0; i < (int)nodes.size(); i++) {
+      const KNode &k = nodes[(size_t)i];
+      if (k.lin < 0 || k.op == POLY_OP_RANGE || k.op == POLY_OP_CONST) continue;
+      RawEval e{*this, rv};
+      int64_t raw = e.node(i);
+      if (!e.ok) continue;
+      int64_t viaLin = e.lin(lins[(size_t)k.lin]);
+      if (!e.ok) continue;
+      if (raw != viaLin) {
+        if (bad == 0 && first_bad)
+          *first_bad = strf("node %d (%s): raw %lld, simplified %lld", i, op_name(k.op), (long long)raw, (long long)viaLin);
+        bad++;
+      }
+    }
+  }
+  return bad;
 }
 
 }  // namespace polyhip

@@ -114,6 +114,10 @@ struct KernelGraph {
 
   const KNode &n(int id) const { return nodes[(size_t)id]; }
   int param_slot(int param_node) const;   // position in params[]
+  // Self-check of the canonical forms: evaluates every index-typed node both from
+  // its raw ops and from its Lin at `samples` range assignments (all of them when
+  // the iteration space is small).  Returns the number of mismatches.
+  int check_lins(int samples, std::string *first_bad) const;
 };
 
 const char *op_name(PolyOps op);

@@ -1,12 +1,310 @@
 // Hand-written kernel templates selected by pattern match on the scheduled
-// root: MFMA matmul and the guarded embedding gather.
+// root (where the structure is still explicit: one REDUCE over a product of
+// two loads is a matmul, a REDUCE over WHERE(idx == arange, table, 0) is an
+// embedding lookup).  Anything that does not match falls through to the
+// generic lowering in render_hip.cc; nothing here changes results beyond the
+// order of the fp32 accumulation.
+#include <algorithm>
+#include <cmath>
+#include <cstdlib>
+
 #include "render_hip.h"
 
 namespace polyhip {
 
-bool try_render_matmul(const KernelGraph &, const std::string &, const RenderOptions &, RenderedKernel *) {
+namespace {
+
+const char *const kMatmulTemplate =
+#include "matmul_mfma.hip.inc"
+    ;
+
+PolyOps reduce_op(const KNode &k) {
+  return k.u->arg.kind == POLY_ARG_OPS ? k.u->arg.ops : (PolyOps)k.u->arg.i;
+}
+
+// One operand of the product: LOAD(INDEX(PARAM, lin)) optionally under a CAST to f32.
+struct Operand {
+  int load = -1, param = -1, lin = -1;
+  DT dt = DT_VOID;
+};
+
+bool match_operand(const KernelGraph &g, int node, Operand *o) {
+  const KNode *k = &g.n(node);
+  if (k->op == POLY_OP_CAST && k->dt == DT_F32) { node = k->src[0]; k = &g.n(node); }
+  if (k->op != POLY_OP_LOAD || k->guard >= 0) return false;
+  const KNode &ix = g.n(k->src[0]);
+  if (ix.src.size() != 2) return false;  // gated
+  o->load = node;
+  o->param = g.param_slot(ix.src[0]);
+  o->lin = g.n(ix.src[1]).lin;
+  o->dt = k->dt;
+  return o->lin >= 0 && o->param >= 0;
+}
+
+struct KSplit { int64_t kb, s_hi, s_lo; };  // off(k) = (k / kb) * s_hi + (k % kb) * s_lo
+
+// Extracts the dependence of `l` on reduce range `kr` (extent K).
+bool k_dependence(const KernelGraph &g, const Lin &l, int kr, int64_t K, KSplit *ks) {
+  bool have_plain = false, have_div = false, have_mod = false;
+  int64_t s = 0, s_hi = 0, s_lo = 0, c_div = 0, c_mod = 0;
+  for (const Term &t : l.terms) {
+    const Atom &a = g.atoms[(size_t)t.atom];
+    if (!(g.atom_deps(t.atom) & ((uint64_t)1 << kr))) continue;
+    if (a.kind == Atom::RANGE) { have_plain = true; s = t.coef; continue; }
+    if (a.kind != Atom::DIV && a.kind != Atom::MOD) return false;
+    // inner must be exactly the range k
+    if (a.inner.c0 != 0 || a.inner.terms.size() != 1 || a.inner.terms[0].coef != 1) return false;
+    const Atom &in = g.atoms[(size_t)a.inner.terms[0].atom];
+    if (in.kind != Atom::RANGE || g.range_ord.at(in.node) != kr) return false;
+    if (a.kind == Atom::DIV) { if (have_div) return false; have_div = true; s_hi = t.coef; c_div = a.c; }
+    else { if (have_mod) return false; have_mod = true; s_lo = t.coef; c_mod = a.c; }
+  }
+  if (have_plain) {
+    if (have_div || have_mod) return false;
+    *ks = {K, 0, s};
+    return true;
+  }
+  if (have_div && have_mod && c_div == c_mod) { *ks = {c_div, s_hi, s_lo}; return true; }
+  if (have_div && !have_mod) { *ks = {c_div, s_hi, 0}; return true; }
+  if (have_mod && !have_div) { *ks = {c_mod, 0, s_lo}; return true; }
+  return false;  // no dependence on k at all
+}
+
+// One output coordinate: an END range, or the high / low part of a range that
+// the indices only use as r / c and r % c (a flattened M*N range).
+struct Dim { int ord; int64_t extent, ca, cb; int part = 0; int64_t c = 0; };
+
+// How a Lin uses global range `ord`: a plain coefficient, or coefficients on
+// DIV(r, c) / MOD(r, c).  Returns false for any other use.
+struct RangeUse { bool plain = false, split = false; int64_t coef = 0, c = 0, hi = 0, lo = 0; };
+bool range_use(const KernelGraph &g, const Lin &l, int ord, RangeUse *u) {
+  for (const Term &t : l.terms) {
+    const Atom &a = g.atoms[(size_t)t.atom];
+    if (!(g.atom_deps(t.atom) & ((uint64_t)1 << ord))) continue;
+    if (a.kind == Atom::RANGE) { u->plain = true; u->coef += t.coef; continue; }
+    if (a.kind != Atom::DIV && a.kind != Atom::MOD) return false;
+    if (a.inner.c0 != 0 || a.inner.terms.size() != 1 || a.inner.terms[0].coef != 1) return false;
+    const Atom &in = g.atoms[(size_t)a.inner.terms[0].atom];
+    if (in.kind != Atom::RANGE || g.range_ord.at(in.node) != ord) return false;
+    if (u->split && u->c != a.c) return false;
+    u->split = true; u->c = a.c;
+    if (a.kind == Atom::DIV) u->hi += t.coef; else u->lo += t.coef;
+  }
+  return !(u->plain && u->split);
+}
+
+std::string offset_fn(const char *name, const std::vector<Dim> &dims, bool use_a, int64_t c0) {
+  // dims are outermost first; the flattened coordinate has the last one fastest
+  std::string s = strf("__device__ __forceinline__ int %s(int x) {\n", name);
+  s += strf("  int off = %lld;\n", (long long)c0);
+  for (size_t i = dims.size(); i-- > 0;) {
+    int64_t c = use_a ? dims[i].ca : dims[i].cb;
+    if (i == 0) s += strf("  off += x * %lld;\n", (long long)c);
+    else s += strf("  off += (x %% %lld) * %lld; x /= %lld;\n", (long long)dims[i].extent, (long long)c, (long long)dims[i].extent);
+  }
+  s += "  return off;\n}\n";
+  return s;
+}
+
+// Merges adjacent dims whose strides nest exactly for both operands.
+void collapse(std::vector<Dim> &dims) {
+  for (size_t i = 0; i + 1 < dims.size();) {
+    Dim &o = dims[i], &in = dims[i + 1];
+    if (o.ca == in.ca * in.extent && o.cb == in.cb * in.extent) {
+      in.extent *= o.extent;
+      dims.erase(dims.begin() + (long)i);
+    } else i++;
+  }
+}
+
+static bool reject(int line) {
+  if (getenv("POLY_HIP_DEBUG")) fprintf(stderr, "polygrad: render_hip: matmul template rejected at templates.cc:%d\n", line);
   return false;
 }
+
+}  // namespace
+
+bool try_render_matmul(const KernelGraph &g, const std::string &fn, const RenderOptions &opt, RenderedKernel *out) {
+  (void)fn; (void)opt;
+  if (g.stores.size() != 1 || g.reduces.size() != 1 || !g.vars.empty()) return reject(__LINE__);
+  const StoreInfo &st = g.stores[0];
+  if (st.gate >= 0) return reject(__LINE__);
+  const int red = g.reduces[0];
+  const KNode &R = g.n(red);
+  if (reduce_op(R) != POLY_OP_ADD || R.dt != DT_F32 || R.src.size() != 2) return reject(__LINE__);
+  const int kr = g.range_ord.at(R.src[1]);
+  const int64_t K = g.ranges[(size_t)kr].extent;
+  if (K < 16) return reject(__LINE__);
+  const KNode &mul = g.n(R.src[0]);
+  if (mul.op != POLY_OP_MUL || mul.dt != DT_F32) return reject(__LINE__);
+  Operand A, B;
+  if (!match_operand(g, mul.src[0], &A) || !match_operand(g, mul.src[1], &B)) return reject(__LINE__);
+  if (A.dt != B.dt || (A.dt != DT_BF16 && A.dt != DT_F16)) return reject(__LINE__);
+  for (const ParamInfo &p : g.params) if (p.numel >= ((int64_t)1 << 31)) return reject(__LINE__);
+  const Lin &la = g.lins[(size_t)A.lin], &lb = g.lins[(size_t)B.lin];
+  KSplit ka, kb;
+  if (!k_dependence(g, la, kr, K, &ka) || !k_dependence(g, lb, kr, K, &kb)) return reject(__LINE__);
+
+  // classify the END ranges of the store
+  std::vector<Dim> md, nd, zd;
+  auto place_dim = [&](const Dim &d) {
+    if (d.ca != 0 && d.cb == 0) md.push_back(d);
+    else if (d.ca == 0 && d.cb != 0) nd.push_back(d);
+    else zd.push_back(d);
+  };
+  for (int r : st.ranges) {
+    const int64_t e = g.ranges[(size_t)r].extent;
+    if (e < 0) return reject(__LINE__);
+    RangeUse ua, ub;
+    if (!range_use(g, la, r, &ua) || !range_use(g, lb, r, &ub)) return reject(__LINE__);
+    if (ua.split || ub.split) {
+      if (ua.plain || ub.plain) return reject(__LINE__);
+      int64_t c = ua.split ? ua.c : ub.c;
+      if ((ua.split && ub.split && ua.c != ub.c) || c <= 0 || e % c != 0) return reject(__LINE__);
+      Dim hi{r, e / c, ua.hi, ub.hi, 1, c}, lo{r, c, ua.lo, ub.lo, 2, c};
+      place_dim(hi);
+      place_dim(lo);
+    } else {
+      place_dim(Dim{r, e, ua.coef, ub.coef, 0, 0});
+    }
+  }
+  if (md.empty() || nd.empty()) return reject(__LINE__);
+  // every other atom in the operand indices must be a plain range handled above
+  auto only_known = [&](const Lin &l) {
+    for (const Term &t : l.terms) {
+      const Atom &a = g.atoms[(size_t)t.atom];
+      uint64_t d = g.atom_deps(t.atom);
+      if (d & ((uint64_t)1 << kr)) continue;            // checked by k_dependence
+      (void)a;                                          // global ranges were vetted by range_use
+    }
+    return true;
+  };
+  if (!only_known(la) || !only_known(lb)) return reject(__LINE__);
+
+  // dims keep END order (outermost first); the innermost one is the fast coordinate
+  std::vector<Dim> md_full = md, nd_full = nd, zd_full = zd;
+  collapse(md); collapse(nd); collapse(zd);
+  int64_t M = 1, N = 1, Z = 1;
+  for (const Dim &d : md) M *= d.extent;
+  for (const Dim &d : nd) N *= d.extent;
+  for (const Dim &d : zd) Z *= d.extent;
+  if (M > 2147483647LL || N > 2147483647LL || Z > 65535) return reject(__LINE__);
+
+  const int BK = 64;
+  // operand layout: contiguous along K, or along its row axis
+  auto layout = [&](const KSplit &ks, const std::vector<Dim> &dims, bool is_a, int64_t rows, bool *kc) {
+    int64_t inner_c = is_a ? dims.back().ca : dims.back().cb;
+    if (ks.s_lo == 1 && K % BK == 0 && ks.kb % BK == 0) { *kc = true; return true; }
+    if (inner_c == 1 && dims.back().extent % 8 == 0 && rows % 8 == 0 && K % BK == 0) { *kc = false; return true; }
+    return reject(__LINE__);
+  };
+  bool a_kc, b_kc;
+  if (!layout(ka, md, true, M, &a_kc) || !layout(kb, nd, false, N, &b_kc)) return reject(__LINE__);
+
+  // tile shape: 4 waves; narrow outputs get a narrow tile
+  int BM = 128, BN = 128, WVM = 2, WVN = 2;
+  if (N <= 64) { BN = 64; BM = 256; WVM = 4; WVN = 1; }
+  else if (M <= 64) { BM = 64; BN = 256; WVM = 1; WVN = 4; }
+  const int64_t tiles = ((M + BM - 1) / BM) * ((N + BN - 1) / BN);
+  if (tiles > 2147483647LL / 2) return reject(__LINE__);
+
+  // ── epilogue: everything outside the REDUCE, per output element ──────────
+  Emitter em(g);
+  Scope S0;
+  S0.indent = 1;
+  for (int r : st.ranges) S0.avail |= (uint64_t)1 << r;
+  std::string decomp;
+  std::vector<std::pair<int, int64_t>> split_ranges;   // (ordinal, c) needing r = hi*c + lo
+  auto decompose = [&](const std::vector<Dim> &dims, const char *var) {
+    if (dims.empty()) return;
+    decomp += strf("  int t_%s = %s;\n", var, var);
+    for (size_t i = dims.size(); i-- > 0;) {
+      const Dim &d = dims[i];
+      std::string rv = d.part == 0 ? strf("r%d", d.ord) : strf("r%d_%s", d.ord, d.part == 1 ? "hi" : "lo");
+      if (i == 0) decomp += strf("  const int %s = t_%s;\n", rv.c_str(), var);
+      else decomp += strf("  const int %s = t_%s %% %lld; t_%s /= %lld;\n", rv.c_str(), var, (long long)d.extent, var, (long long)d.extent);
+      if (d.part == 0) em.bind_range(d.ord, rv);
+      else if (d.part == 1) split_ranges.push_back({d.ord, d.c});
+    }
+  };
+  decompose(md_full, "m");
+  decompose(nd_full, "n");
+  decompose(zd_full, "z");
+  for (auto &sr : split_ranges) {
+    decomp += strf("  const int r%d = r%d_hi * %lld + r%d_lo;\n", sr.first, sr.first, (long long)sr.second, sr.first);
+    em.bind_range(sr.first, strf("r%d", sr.first));
+  }
+  em.preset(red, "acc");
+  std::string val = em.emit(st.value, &S0);
+  std::string idx = em.emit(g.n(st.index).src[1], &S0);
+  if (em.failed()) return reject(__LINE__);
+  const int pout = g.param_slot(st.param);
+  std::string params_decl, params_call;
+  for (size_t i = 0; i < g.params.size(); i++) {
+    const ParamInfo &p = g.params[i];
+    if (i) { params_decl += ", "; params_call += ", "; }
+    if (p.written) params_decl += strf("%s* data%zu", dt_cname(p.dt), i);
+    else params_decl += strf("const %s* __restrict__ data%zu", dt_cname(p.dt), i);
+    params_call += strf("data%zu", i);
+  }
+  std::string epi = strf("__device__ __forceinline__ void poly_epilogue(float acc, int m, int n, int z, %s) {\n", params_decl.c_str());
+  epi += decomp + S0.code;
+  epi += strf("  data%d[%s] = %s;\n}\n", pout, idx.c_str(), val.c_str());
+
+  // ── configuration block ───────────────────────────────────────────────────
+  std::string cfg;
+  cfg += strf("#define POLY_TIN %s\n", dt_cname(A.dt));
+  cfg += strf("#define POLY_MFMA(a, b, c) __builtin_amdgcn_mfma_f32_32x32x16_%s(a, b, c, 0, 0, 0)\n", A.dt == DT_BF16 ? "bf16" : "f16");
+  cfg += strf("#define POLY_M %lld\n#define POLY_N %lld\n#define POLY_K %lld\n#define POLY_Z %lld\n", (long long)M, (long long)N, (long long)K, (long long)Z);
+  cfg += strf("#define POLY_BM %d\n#define POLY_BN %d\n#define POLY_BK %d\n#define POLY_WAVES_M %d\n#define POLY_WAVES_N %d\n", BM, BN, BK, WVM, WVN);
+  cfg += strf("#define POLY_A_KC %d\n#define POLY_B_KC %d\n", a_kc ? 1 : 0, b_kc ? 1 : 0);
+  cfg += strf("#define POLY_A_PTR data%d\n#define POLY_B_PTR data%d\n", A.param, B.param);
+  cfg += offset_fn("poly_a_row", md, true, 0);
+  cfg += offset_fn("poly_b_row", nd, false, 0);
+  if (zd.empty()) {
+    cfg += strf("__device__ __forceinline__ int poly_a_z(int) { return %lld; }\n", (long long)la.c0);
+    cfg += strf("__device__ __forceinline__ int poly_b_z(int) { return %lld; }\n", (long long)lb.c0);
+  } else {
+    cfg += offset_fn("poly_a_z", zd, true, la.c0);
+    cfg += offset_fn("poly_b_z", zd, false, lb.c0);
+  }
+  auto kfn = [&](const char *name, const KSplit &ks) {
+    if (ks.kb >= K) return strf("__device__ __forceinline__ int %s(int k) { return k * %lld; }\n", name, (long long)ks.s_lo);
+    return strf("__device__ __forceinline__ int %s(int k) { return (k / %lld) * %lld + (k %% %lld) * %lld; }\n", name,
+                (long long)ks.kb, (long long)ks.s_hi, (long long)ks.kb, (long long)ks.s_lo);
+  };
+  cfg += kfn("poly_a_k", ka);
+  cfg += kfn("poly_b_k", kb);
+  cfg += strf("#define POLY_SIGNATURE %s\n", params_decl.c_str());
+  cfg += epi;
+  cfg += strf("#define POLY_EPILOGUE(acc, m, n, z) poly_epilogue(acc, m, n, z, %s)\n", params_call.c_str());
+
+  *out = RenderedKernel();
+  out->source = std::string(hip_prelude()) + cfg + kMatmulTemplate;
+  out->entry = "poly_k";
+  out->launch.grid[0] = (unsigned)tiles;
+  out->launch.grid[1] = (unsigned)Z;
+  out->launch.block[0] = 256;
+  out->klass = KernelClass::MATMUL_MFMA;
+  out->strategy = strf("mfma 32x32x16 %s M=%lld N=%lld K=%lld Z=%lld tile %dx%dx%d A:%s B:%s", A.dt == DT_BF16 ? "bf16" : "f16",
+                       (long long)M, (long long)N, (long long)K, (long long)Z, BM, BN, BK, a_kc ? "k-major" : "m-major",
+                       b_kc ? "k-major" : "n-major");
+  out->n_params = (int)g.params.size();
+  out->n_vars = 0;
+  out->flops = 2.0 * (double)M * (double)N * (double)K * (double)Z;
+  // distinct elements: A, B once each (broadcast operands counted once), output once,
+  // plus whatever the epilogue reads per output row/column
+  double bytes = 0;
+  for (size_t i = 0; i < g.params.size(); i++) {
+    const ParamInfo &p = g.params[i];
+    double n = (double)std::max<int64_t>(p.numel, 0);
+    if ((int)i == pout) n = (double)M * N * Z;
+    bytes += n * dt_size(p.dt);
+  }
+  out->bytes = bytes;
+  return true;
+}
+
 bool try_render_gather(const KernelGraph &, const std::string &, const RenderOptions &, RenderedKernel *) {
   return false;
 }

@@ -1,0 +1,119 @@
+"""GPU parity of the MFMA matmul template against the reference CPU backend:
+bf16 / fp16 inputs, fp32 accumulate, every operand layout the template
+distinguishes (k-major and row-major operands, batches, broadcast batch,
+two-level K from merged heads, bias epilogue, ragged M and N)."""
+import numpy as np
+import pytest
+
+import graphs
+import refpoly as R
+from hipharness import assert_close, run_hip, run_ref
+
+pytestmark = [pytest.mark.gpu, pytest.mark.skipif(not R.available(), reason="reference library not built")]
+
+
+def bf16(g, shape, scale=0.02):
+    return R.f32_to_bf16_bits(g.normal(0, scale, int(np.prod(shape))).astype(np.float32))
+
+
+def check(c, sink, arrays, out, what, rtol=1e-3, expect_mfma=True):
+    want = run_ref(c, sink, arrays)
+    got, info = run_hip(c, sink, arrays)
+    if expect_mfma:
+        assert any(k["klass"] == "matmul-mfma" for k in info), [k["desc"] for k in info]
+    w, h = want[out], got[out]
+    if w.dtype == np.uint16:
+        w, h = R.bf16_bits_to_f32(w), R.bf16_bits_to_f32(h)
+    # accumulation order differs: tolerance relative to the magnitude of the sums
+    atol = rtol * float(np.abs(w).mean() + 1e-12)
+    assert_close(h, w, rtol=rtol, atol=atol, what=what)
+
+
+@pytest.mark.parametrize("m,n,k,tb", [(256, 512, 128, False), (256, 512, 128, True), (128, 192, 64, False),
+                                       (200, 328, 192, True), (136, 128, 64, False), (64, 1000, 64, True)])
+def test_matmul_bf16_layouts(m, n, k, tb):
+    c = R.Ctx()
+    g = np.random.default_rng(m * 7 + n)
+    A, Bm, O, sink = graphs.matmul_bf16(c, m, n, k, transposed_b=tb)
+    arrays = {A: bf16(g, (m, k)), Bm: bf16(g, (k, n)), O: np.zeros(m * n, np.float32)}
+    check(c, sink, arrays, O, f"matmul {m}x{n}x{k} tb={tb}")
+    c.close()
+
+
+def test_matmul_broadcast_batch():
+    c = R.Ctx()
+    g = np.random.default_rng(11)
+    A, Bm, O, sink = graphs.matmul_bf16(c, 128, 128, 64, batch=4)
+    arrays = {A: bf16(g, (4, 128, 64)), Bm: bf16(g, (64, 128)), O: np.zeros(4 * 128 * 128, np.float32)}
+    check(c, sink, arrays, O, "broadcast batch")
+    c.close()
+
+
+def test_matmul_fp16():
+    c = R.Ctx()
+    g = np.random.default_rng(12)
+    A = c.buffer((128, 64), R.F16, name="A")
+    B = c.buffer((64, 128), R.F16, name="B")
+    O = c.buffer((128, 128), R.F32, name="C")
+    sink = c.sink((O, A.cast(R.F32).dot(B.cast(R.F32))))
+    arrays = {A: g.normal(0, 0.5, (128, 64)).astype(np.float16), B: g.normal(0, 0.5, (64, 128)).astype(np.float16),
+              O: np.zeros((128, 128), np.float32)}
+    check(c, sink, arrays, O, "fp16 matmul")
+    c.close()
+
+
+def test_attention_shaped_matmuls_with_bias_and_merged_heads():
+    """The four matmul forms of one GPT-2 block at a reduced size: QK^T (both operands
+    k-major, two batch dims with non-nesting strides), attn@V (row-major B), merged
+    heads @ W + bias (A with a two-level K index), all with bf16 outputs."""
+    B, T, H, hd = 2, 128, 2, 64
+    D = H * hd
+    c = R.Ctx()
+    g = np.random.default_rng(13)
+    q, k, v = (c.buffer((B, T, D), R.BF16, name=n) for n in "qkv")
+    w = c.buffer((D, D), R.BF16, name="w")
+    bias = c.buffer((D,), R.BF16, name="bias")
+    scores_o = c.buffer((B, H, T, T), R.BF16, name="scores")
+    ctx_o = c.buffer((B, H, T, hd), R.BF16, name="ctx")
+    proj_o = c.buffer((B, T, D), R.BF16, name="proj")
+    qh = q.reshape((B, T, H, hd)).permute((0, 2, 1, 3))
+    kh = k.reshape((B, T, H, hd)).permute((0, 2, 1, 3))
+    vh = v.reshape((B, T, H, hd)).permute((0, 2, 1, 3))
+    scores = qh.cast(R.F32).dot(kh.permute((0, 1, 3, 2)).cast(R.F32)).cast(R.BF16)
+    arr = {q: bf16(g, (B, T, D), 1.0), k: bf16(g, (B, T, D), 1.0), v: bf16(g, (B, T, D), 1.0),
+           w: bf16(g, (D, D), 0.1), bias: bf16(g, (D,), 1.0)}
+    a1 = {q: arr[q], k: arr[k], scores_o: np.zeros(B * H * T * T, np.uint16)}
+    check(c, c.sink((scores_o, scores)), a1, scores_o, "QK^T", rtol=2e-2)
+    attn = c.buffer((B, H, T, T), R.BF16, name="attn")
+    ctxv = attn.cast(R.F32).dot(vh.cast(R.F32)).cast(R.BF16)
+    a2 = {attn: bf16(g, (B, H, T, T), 0.1), v: arr[v], ctx_o: np.zeros(B * H * T * hd, np.uint16)}
+    check(c, c.sink((ctx_o, ctxv)), a2, ctx_o, "attn@V", rtol=2e-2)
+    ctx_in = c.buffer((B, H, T, hd), R.BF16, name="ctx_in")
+    merged = ctx_in.permute((0, 2, 1, 3)).reshape((B, T, D))
+    proj = merged.cast(R.F32).dot(w.cast(R.F32)).cast(R.BF16) + bias.reshape((1, 1, D)).expand((B, T, D))
+    a3 = {ctx_in: bf16(g, (B, H, T, hd), 1.0), w: arr[w], bias: arr[bias], proj_o: np.zeros(B * T * D, np.uint16)}
+    check(c, c.sink((proj_o, proj)), a3, proj_o, "merged heads @ W + bias", rtol=2e-2)
+    c.close()
+
+
+def test_full_size_row_block_matches_cpu_bit_pattern_of_sums():
+    """At a benchmark shape (4096^3 is too slow on one CPU core) the CPU result of a
+    row block is the full result for those rows: compare 8 rows of a 1024x4096x4096
+    product computed on the GPU at full size with the CPU backend on the 8-row slice."""
+    m, n, k = 1024, 4096, 4096
+    g = np.random.default_rng(14)
+    a_bits, b_bits = bf16(g, (m, k)), bf16(g, (k, n))
+    c = R.Ctx()
+    A, Bm, O, sink = graphs.matmul_bf16(c, m, n, k)
+    got, info = run_hip(c, sink, {A: a_bits, Bm: b_bits, O: np.zeros(m * n, np.float32)})
+    assert info[0]["klass"] == "matmul-mfma"
+    c.close()
+    rows = [0, 1, 127, 128, 500, 777, 1022, 1023]
+    c = R.Ctx()
+    A8, B8, O8, sink8 = graphs.matmul_bf16(c, 8, n, k)
+    a8 = a_bits.reshape(m, k)[rows].reshape(-1)
+    want = run_ref(c, sink8, {A8: a8, B8: b_bits, O8: np.zeros(8 * n, np.float32)})
+    c.close()
+    h = got[O].reshape(m, n)[rows]
+    w = want[O8].reshape(8, n)
+    assert_close(h, w, rtol=1e-4, atol=1e-4 * float(np.abs(w).mean()), what="row block of 1024x4096x4096")
