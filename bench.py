@@ -1,0 +1,201 @@
+#!/usr/bin/env python3
+"""Benchmark of the HIP backend on one MI355X.
+
+Default workload: GPT-2 small forward, random-init, B=8, T=1024, bf16 weights and
+activations with fp32 reductions (BASELINE.json configs[3], the configuration the
+headline metric is quoted on).  One step = one pass of the compiled plan over one
+batch resident in HBM: poly_hip_plan_run() replaying the captured hipGraph.
+
+Prints ONE JSON line: whole-job tokens/s, the roofline figures of the dominant
+kernel (algorithmic flops or bytes / its average launch duration, measured with
+HIP events on the backend's stream), a per-class breakdown, and the reference CPU
+backend timed on a bounded sample of the same workload on this box's host cores.
+
+    python bench.py --gpus 1 --steps 20 --warmup 3
+    python bench.py --workload matmul_bf16_8192x8192x8192     (any plan in polygrad_amd/plans)
+"""
+import argparse
+import json
+import os
+import sys
+import time
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+sys.path.insert(0, ROOT)
+
+PEAK_HBM_GBS = 8000.0          # MI355X HBM3E
+PEAK_MFMA_TFLOPS = 2500.0      # MI355X dense bf16/fp16 MFMA
+GPT2_PLAN = "gpt2_small_bf16_b8_t1024"
+
+
+def log(*a):
+    print(*a, file=sys.stderr, flush=True)
+
+
+def kernel_key(desc):
+    # "hip0_k12 row-reduce: ..." -> drop the per-plan kernel name
+    return desc.split(" ", 1)[1] if " " in desc else desc
+
+
+def run_gpu(workload, steps, warmup):
+    import torch
+    from polygrad_amd import HipPlan
+    from polygrad_amd.inputs import gpt2_slot_tensors, random_slot_tensors
+
+    path = os.path.join(ROOT, "polygrad_amd", "plans", workload + ".polyplan")
+    t0 = time.perf_counter()
+    plan = HipPlan.from_file(path)
+    compile_s = time.perf_counter() - t0
+    if workload.startswith("gpt2"):
+        data, _ = gpt2_slot_tensors(plan)
+        tokens = [s for s in plan.slots if s.name == "x"][0].numel
+    else:
+        data = random_slot_tensors(plan, seed=2, scale=0.05 if "matmul" in workload else 1.0)
+        tokens = None
+    torch.cuda.synchronize()
+    for _ in range(max(warmup, 1)):
+        plan.run(data, sync=False)
+    plan.sync()
+    t0 = time.perf_counter()
+    for _ in range(steps):
+        plan.run(data, sync=False)
+    plan.sync()
+    elapsed = time.perf_counter() - t0
+    ms_per_step = elapsed / steps * 1e3
+
+    # per-kernel durations: HIP events around every launch on the backend stream
+    info = plan.kernel_info()
+    passes = 3
+    acc = [0.0] * len(info)
+    for _ in range(passes):
+        for i, ms in enumerate(plan.profile(data)):
+            acc[i] += ms
+    per_kernel_ms = [a / passes for a in acc]
+    groups = {}
+    for k, ms in zip(info, per_kernel_ms):
+        g = groups.setdefault(kernel_key(k["desc"]), dict(klass=k["klass"], launches=0, ms=0.0, bytes=k["bytes"], flops=k["flops"]))
+        g["launches"] += 1
+        g["ms"] += ms
+    dominant_key = max(groups, key=lambda k: groups[k]["ms"])
+    d = groups[dominant_key]
+    avg_ms = d["ms"] / d["launches"]
+    if d["flops"] > 0:
+        achieved = d["flops"] / (avg_ms * 1e-3) / 1e12
+        roofline = dict(bound="mfma", achieved=round(achieved, 2), peak=PEAK_MFMA_TFLOPS, unit="TFLOP/s",
+                        frac=round(achieved / PEAK_MFMA_TFLOPS, 4), traffic=None)
+    else:
+        achieved = d["bytes"] / (avg_ms * 1e-3) / 1e9
+        roofline = dict(bound="hbm", achieved=round(achieved, 1), peak=PEAK_HBM_GBS, unit="GB/s",
+                        frac=round(achieved / PEAK_HBM_GBS, 4), traffic=None)
+    roofline.update(kernel=dominant_key, launches_per_step=d["launches"], avg_launch_ms=round(avg_ms, 4),
+                    algorithmic_bytes=d["bytes"], algorithmic_flops=d["flops"])
+
+    classes = {}
+    for k, ms in zip(info, per_kernel_ms):
+        c = classes.setdefault(k["klass"], dict(launches=0, ms=0.0, bytes=0.0, flops=0.0))
+        c["launches"] += 1
+        c["ms"] += ms
+        c["bytes"] += k["bytes"]
+        c["flops"] += k["flops"]
+    for c in classes.values():
+        c["GBps"] = round(c["bytes"] / (c["ms"] * 1e-3) / 1e9, 1) if c["ms"] > 0 else 0.0
+        c["TFLOPs"] = round(c["flops"] / (c["ms"] * 1e-3) / 1e12, 1) if c["ms"] > 0 else 0.0
+        c["hbm_frac"] = round(c["GBps"] / PEAK_HBM_GBS, 4)
+        c["mfma_frac"] = round(c["TFLOPs"] / PEAK_MFMA_TFLOPS, 4)
+        c["ms"] = round(c["ms"], 4)
+        c["bytes"] = int(c["bytes"])
+        c["flops"] = int(c["flops"])
+    total_flops = sum(k["flops"] for k in info)
+    total_bytes = sum(k["bytes"] for k in info)
+    extra = dict(classes=classes, n_kernels=len(info), eager_sum_ms=round(sum(per_kernel_ms), 3),
+                 plan_flops=int(total_flops), plan_bytes=int(total_bytes),
+                 flop_time_ms=round(total_flops / (PEAK_MFMA_TFLOPS * 1e12) * 1e3, 3),
+                 byte_time_ms=round(total_bytes / (PEAK_HBM_GBS * 1e9) * 1e3, 3),
+                 workspace_MiB=round(plan.workspace_bytes() / 2**20, 1), compile_s=round(compile_s, 1))
+    top = sorted(groups.items(), key=lambda kv: -kv[1]["ms"])[:8]
+    for key, g in top:
+        log(f"  {g['ms']:8.3f} ms  x{g['launches']:3d}  {key[:150]}")
+    plan.close()
+    return ms_per_step, tokens, roofline, extra
+
+
+def cpu_baseline_reference(seconds_hint=20):
+    """Times the REAL reference CPU backend (oracle/_ref/libpolygrad.so, built from the
+    reference sources) on a bounded sample: GPT-2 small, 12 layers, bf16, one sequence
+    of 32 tokens, single core (the reference has no threads)."""
+    sys.path.insert(0, os.path.join(ROOT, "tests"))
+    import graphs
+    import refpoly as R
+    if not R.available():
+        return None
+    cfg = graphs.GPT2Config(batch=1, ctx=32)
+    c = R.Ctx()
+    sink, bufs = graphs.gpt2_forward(c, cfg, R.BF16)
+    arrays = graphs.gpt2_inputs(cfg, bufs, seed=3, wdt=R.BF16)
+    t0 = time.perf_counter()
+    c.realize_cpu(sink, arrays)          # first call: JIT (fork + clang per kernel), not timed as throughput
+    jit_s = time.perf_counter() - t0
+    t0 = time.perf_counter()
+    c.realize_cpu(sink, arrays)          # warm call
+    warm_s = time.perf_counter() - t0
+    c.close()
+    toks = cfg.batch * cfg.ctx
+    return dict(value=round(toks / warm_s, 3), unit="tokens/s", cores=1, kind="reference",
+                sample=f"GPT-2 small forward bf16, 12 layers, B=1, T=32 ({toks} tokens), warm poly_realize "
+                       f"{warm_s:.2f} s (first call incl. clang JIT {jit_s:.1f} s); 1 of {os.cpu_count()} cores",
+                warm_s=round(warm_s, 3))
+
+
+def cpu_baseline_port():
+    """Fallback when the reference library is not present: the CPU oracle on the tiny fixture."""
+    sys.path.insert(0, os.path.join(ROOT, "tests"))
+    import fixtures as F
+    fx = F.Fixture("gpt2_tiny_bf16")
+    t0 = time.perf_counter()
+    F.run_oracle_schedule(fx.plan.schedule, fx.n_slots, fx.inputs)
+    dt = time.perf_counter() - t0
+    return dict(value=round(32 / dt, 3), unit="tokens/s", cores=1, kind="port",
+                sample=f"CPU oracle on the tiny GPT-2 fixture (2 layers, d_model 32, vocab 97, 32 tokens) in {dt:.2f} s")
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=20)
+    ap.add_argument("--warmup", type=int, default=3)
+    ap.add_argument("--workload", default=GPT2_PLAN)
+    ap.add_argument("--no-cpu-baseline", action="store_true")
+    args = ap.parse_args()
+    if args.gpus != 1:
+        sys.exit("bench.py: this backend runs on one GPU; --gpus must be 1 (nothing here shards across devices)")
+    import torch
+    if not torch.cuda.is_available():
+        sys.exit("bench.py: no GPU available (there is no CPU path to benchmark)")
+
+    ms, tokens, roofline, extra = run_gpu(args.workload, args.steps, args.warmup)
+    cpu = None
+    if not args.no_cpu_baseline and args.workload.startswith("gpt2"):
+        try:
+            cpu = cpu_baseline_reference() or cpu_baseline_port()
+        except Exception as e:  # the baseline is reported, never required
+            log(f"cpu baseline failed: {e}")
+    if tokens is not None:
+        metric, value, unit = "GPT-2-small fwd tokens/s on 1 MI355X", tokens / (ms * 1e-3), "tokens/s"
+        workload = "GPT-2 small forward, random-init, B=8 T=1024, bf16 weights/activations, fp32 reductions (BASELINE.json configs[3])"
+    else:
+        metric, value, unit = "plan passes/s on 1 MI355X", 1e3 / ms, "passes/s"
+        workload = args.workload
+    line = {
+        "metric": metric, "value": round(value, 1), "unit": unit, "n_gpus": 1, "steps": args.steps,
+        "warmup": args.warmup, "ms_per_step": round(ms, 4), "higher_is_better": True, "scaling": "weak",
+        "vs_baseline": None, "dtype": "bf16", "data": "synthetic",
+        "config": {"workload": workload, "plan": args.workload, "global_batch": 8 if tokens else None,
+                   "seq_len": 1024 if tokens else None, "parallelism": "single GPU",
+                   "execution": "hipGraph replay of the compiled plan, inputs resident in HBM"},
+        "roofline": roofline, "cpu_baseline": cpu, "detail": extra,
+    }
+    print(json.dumps(line), flush=True)
+
+
+if __name__ == "__main__":
+    main()

@@ -311,7 +311,8 @@ std::string Emitter::emit_raw(int id, Scope *s) {
     return it->second;
   }
   if (k.op == POLY_OP_REDUCE) {
-    std::string acc = emit_reduce_serial(id, t);
+    auto cu = custom_.find(id);
+    std::string acc = cu != custom_.end() ? cu->second(t) : emit_reduce_serial(id, t);
     t->names[id] = acc;
     return acc;
   }

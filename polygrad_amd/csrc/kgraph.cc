@@ -200,11 +200,8 @@ Lin KernelGraph::lin_div(const Lin &a, int64_t c) {
         int64_t xlo, xhi;
         lin_bounds(X, &xlo, &xhi);
         if (xlo < 0) continue;
-        R = X;
-        cc = c / g;
-        if (cc == 1) return lin_add(Q, R);
-        if (xhi < cc) return Q;
-        break;
+        // X / c' may simplify further (e.g. a quotient of a quotient)
+        return lin_add(Q, lin_div(X, c / g));
       }
       Atom d;
       d.kind = Atom::DIV; d.inner = R; d.c = cc;
@@ -240,6 +237,26 @@ Lin KernelGraph::lin_mod(const Lin &a, int64_t c) {
           atoms[(size_t)R.terms[0].atom].c % c == 0) {
         const Atom at = atoms[(size_t)R.terms[0].atom];
         return lin_mod(at.inner, c);
+      }
+      // (g*X + S) % (g*c') == g*(X % c') + S when 0 <= S < g
+      for (size_t pick = 0; pick < R.terms.size(); pick++) {
+        int64_t thresh = std::llabs(R.terms[pick].coef);
+        int64_t g = c;
+        for (const Term &t : R.terms) if (std::llabs(t.coef) >= thresh) g = gcd64(g, t.coef);
+        if (g <= 1 || g == c) continue;
+        Lin X, S;
+        for (const Term &t : R.terms) {
+          if (t.coef % g == 0) X.terms.push_back({t.coef / g, t.atom});
+          else S.terms.push_back(t);
+        }
+        int64_t r0 = R.c0 % g;
+        X.c0 = (R.c0 - r0) / g;
+        S.c0 = r0;
+        int64_t slo, shi, xlo, xhi;
+        lin_bounds(S, &slo, &shi);
+        lin_bounds(X, &xlo, &xhi);
+        if (slo < 0 || shi >= g || xlo < 0) continue;
+        return lin_add(lin_scale(lin_mod(X, c / g), g), S);
       }
       Atom m;
       m.kind = Atom::MOD; m.inner = R; m.c = c;
@@ -542,6 +559,27 @@ bool KernelGraph::build(const PolyUOp *root) {
     }
     k.lin = (int)lins.size();
     lins.push_back(out);
+  }
+
+  // Tighten the range dependencies with the simplified forms: an index that
+  // mentions a range only in terms that cancelled no longer depends on it.
+  for (int i = 0; i < (int)nodes.size(); i++) {
+    KNode &k = nodes[(size_t)i];
+    if (k.op == POLY_OP_RANGE) continue;
+    if (k.lin >= 0) {
+      const Lin &l = lins[(size_t)k.lin];
+      bool self = l.c0 == 0 && l.terms.size() == 1 && atoms[(size_t)l.terms[0].atom].kind == Atom::OPAQUE &&
+                  atoms[(size_t)l.terms[0].atom].node == i;
+      if (!self) { k.deps = lin_deps(l); continue; }
+    }
+    uint64_t d = 0;
+    for (int s : k.src) d |= nodes[(size_t)s].deps;
+    if (k.op == POLY_OP_REDUCE || k.op == POLY_OP_END)
+      for (size_t s = 1; s < k.src.size(); s++) {
+        auto it = range_ord.find(k.src[s]);
+        if (it != range_ord.end()) d &= ~((uint64_t)1 << it->second);
+      }
+    k.deps = d;
   }
   return true;
 }

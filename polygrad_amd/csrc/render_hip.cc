@@ -46,9 +46,13 @@ class Generic {
 
   bool run(RenderedKernel *out, std::string *err) {
     if (!prepare(err)) return false;
+    for (auto &ov : opt_.reduce_override) {
+      auto fn = ov.second;
+      em_.custom_reduce(ov.first, [this, fn](Scope *s) { return fn(em_, s); });
+    }
     std::string body;
     bool coop = false;
-    if (!g_.reduces.empty() && opt_.allow_coop_reduce && groups_.size() == 1) coop = plan_coop();
+    if (n_loop_reduces() > 0 && opt_.allow_coop_reduce && groups_.size() == 1 && opt_.reduce_override.empty()) coop = plan_coop();
     if (coop) {
       body = render_coop(out);
     } else {
@@ -56,7 +60,8 @@ class Generic {
     }
     if (em_.failed()) { *err = em_.error(); return false; }
     if (!error_.empty()) { *err = error_; return false; }
-    std::string prologue = opt_.exit_if_flag ? "  if (*poly_flag != 0) return;\n" : "";
+    std::string prologue = opt_.exit_if_flag ? "  if (*poly_flag != 0) return;\n"
+                           : opt_.exit_unless_flag ? "  if (*poly_flag == 0) return;\n" : "";
     out->source = std::string(hip_prelude()) + signature() + " {\n" + prologue + body + "}\n";
     out->entry = fn_;
     out->n_params = (int)g_.params.size();
@@ -78,6 +83,13 @@ class Generic {
   int64_t coop_R_ = 0;
   std::vector<int> coop_ranges_;
 
+  // REDUCE nodes that still need a loop (not replaced by a caller-supplied value)
+  int n_loop_reduces() const {
+    int n = 0;
+    for (int r : g_.reduces) if (!opt_.reduce_override.count(r)) n++;
+    return n;
+  }
+
   std::string signature() const {
     std::string s = strf("extern \"C\" __global__ void __launch_bounds__(%d) %s(", opt_.block, fn_.c_str());
     bool first = true;
@@ -93,7 +105,7 @@ class Generic {
       first = false;
       s += strf("const int var%zu", i);
     }
-    if (opt_.exit_if_flag) s += std::string(first ? "" : ", ") + "const int* __restrict__ poly_flag";
+    if (opt_.exit_if_flag || opt_.exit_unless_flag) s += std::string(first ? "" : ", ") + "const int* __restrict__ poly_flag";
     return s + ")";
   }
 
@@ -236,7 +248,7 @@ class Generic {
     line(body, 1, "const long long gid = (long long)blockIdx.x * blockDim.x + threadIdx.x;");
     double max_threads = 1;
     bool dynamic = false;
-    bool any_reduce = !g_.reduces.empty();
+    bool any_reduce = n_loop_reduces() > 0;
     std::string strat;
     for (size_t gi = 0; gi < groups_.size(); gi++) {
       const Group &gr = groups_[gi];

@@ -6,6 +6,7 @@
 // per row with DPP/ds_swizzle wave reductions, and matmul-shaped reductions are
 // handed to the MFMA template.
 #pragma once
+#include <functional>
 #include <string>
 #include <unordered_map>
 #include <vector>
@@ -47,6 +48,8 @@ struct RenderedKernel {
   LaunchSpec fallback_launch;
 };
 
+struct Scope;
+class Emitter;
 struct RenderOptions {
   bool allow_templates = true;   // MFMA matmul / gather fast paths
   bool allow_vectorize = true;
@@ -55,6 +58,11 @@ struct RenderOptions {
   // When set, the kernel takes one more argument `const int* poly_flag` after the
   // vars and returns at once if *poly_flag != 0 (the slow twin of a guarded fast path).
   bool exit_if_flag = false;
+  // The fast twin: same extra argument, returns at once if *poly_flag == 0.
+  bool exit_unless_flag = false;
+  // REDUCE nodes whose value the caller computes without a loop (gather fast
+  // path); the kernel is then lowered as if it had no such reduction.
+  std::unordered_map<int, std::function<std::string(Emitter &, Scope *)>> reduce_override;
 };
 
 // Returns false and sets *err on unsupported graphs (never falls back to a
@@ -80,6 +88,11 @@ class Emitter {
   // Overrides the value of a node (vector-loaded values, reduce results, ...).
   void preset(int node, const std::string &expr) { preset_[node] = expr; }
   void clear_preset(int node) { preset_.erase(node); }
+  // Replaces the serial loop of a REDUCE node by caller-generated code; the
+  // callback receives the scope the value is placed in and returns its C name.
+  void custom_reduce(int node, std::function<std::string(Scope *)> fn) { custom_[node] = std::move(fn); }
+  bool has_custom(int node) const { return custom_.count(node) != 0; }
+  void stmt(Scope *s, const std::string &line);
   std::string emit(int node, Scope *s);
   std::string emit_lin(const Lin &l, Scope *s);
   std::string load_expr(int load_node, Scope *s);
@@ -96,10 +109,10 @@ class Emitter {
   std::string emit_atom(int atom, Scope *s);
   std::string emit_raw(int node, Scope *s);
   Scope *place(uint64_t deps, Scope *s);
-  void stmt(Scope *s, const std::string &line);
   const KernelGraph &g_;
   std::unordered_map<int, std::string> range_name_;
   std::unordered_map<int, std::string> preset_;
+  std::unordered_map<int, std::function<std::string(Scope *)>> custom_;
   std::string error_;
 };
 

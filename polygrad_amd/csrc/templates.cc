@@ -70,27 +70,64 @@ bool k_dependence(const KernelGraph &g, const Lin &l, int kr, int64_t K, KSplit 
   return false;  // no dependence on k at all
 }
 
-// One output coordinate: an END range, or the high / low part of a range that
-// the indices only use as r / c and r % c (a flattened M*N range).
-struct Dim { int ord; int64_t extent, ca, cb; int part = 0; int64_t c = 0; };
+// One output coordinate: a digit of an END range.  A range r that the indices use
+// only through r / a, r % b and (r / a) % b is a mixed-radix number; each digit
+// d = (r / cut) % extent becomes a coordinate of its own (a plain range is the
+// single digit with cut 1).
+struct Dim { int ord; int64_t extent, ca, cb; int64_t cut = 1; };
 
-// How a Lin uses global range `ord`: a plain coefficient, or coefficients on
-// DIV(r, c) / MOD(r, c).  Returns false for any other use.
-struct RangeUse { bool plain = false, split = false; int64_t coef = 0, c = 0, hi = 0, lo = 0; };
-bool range_use(const KernelGraph &g, const Lin &l, int ord, RangeUse *u) {
+struct DigitUse { int64_t coef, a, b; };  // coef * ((r / a) % b), b = 0: no modulus
+
+// Collects how `l` uses global range `ord`; false when some use is not of the
+// digit form above.
+bool digit_uses(const KernelGraph &g, const Lin &l, int ord, std::vector<DigitUse> *uses) {
+  auto is_range = [&](const Lin &in) {
+    if (in.c0 != 0 || in.terms.size() != 1 || in.terms[0].coef != 1) return false;
+    const Atom &a = g.atoms[(size_t)in.terms[0].atom];
+    return a.kind == Atom::RANGE && g.range_ord.at(a.node) == ord;
+  };
   for (const Term &t : l.terms) {
     const Atom &a = g.atoms[(size_t)t.atom];
     if (!(g.atom_deps(t.atom) & ((uint64_t)1 << ord))) continue;
-    if (a.kind == Atom::RANGE) { u->plain = true; u->coef += t.coef; continue; }
-    if (a.kind != Atom::DIV && a.kind != Atom::MOD) return false;
-    if (a.inner.c0 != 0 || a.inner.terms.size() != 1 || a.inner.terms[0].coef != 1) return false;
-    const Atom &in = g.atoms[(size_t)a.inner.terms[0].atom];
-    if (in.kind != Atom::RANGE || g.range_ord.at(in.node) != ord) return false;
-    if (u->split && u->c != a.c) return false;
-    u->split = true; u->c = a.c;
-    if (a.kind == Atom::DIV) u->hi += t.coef; else u->lo += t.coef;
+    if (a.kind == Atom::RANGE) { uses->push_back({t.coef, 1, 0}); continue; }
+    if (a.kind == Atom::DIV && is_range(a.inner)) { uses->push_back({t.coef, a.c, 0}); continue; }
+    if (a.kind == Atom::MOD && is_range(a.inner)) { uses->push_back({t.coef, 1, a.c}); continue; }
+    if (a.kind == Atom::MOD && a.inner.c0 == 0 && a.inner.terms.size() == 1 && a.inner.terms[0].coef == 1) {
+      const Atom &d = g.atoms[(size_t)a.inner.terms[0].atom];
+      if (d.kind == Atom::DIV && is_range(d.inner)) { uses->push_back({t.coef, d.c, a.c}); continue; }
+    }
+    return false;
   }
-  return !(u->plain && u->split);
+  return true;
+}
+
+// Splits range `ord` (extent E) into digits consistent with every use in la / lb
+// and returns them outermost first with their coefficients in both operands.
+bool factor_range(const KernelGraph &g, const Lin &la, const Lin &lb, int ord, int64_t E, std::vector<Dim> *out) {
+  std::vector<DigitUse> ua, ub;
+  if (!digit_uses(g, la, ord, &ua) || !digit_uses(g, lb, ord, &ub)) return false;
+  std::vector<int64_t> cuts{1, E};
+  for (const std::vector<DigitUse> *u : {&ua, &ub})
+    for (const DigitUse &d : *u) {
+      cuts.push_back(d.a);
+      if (d.b > 0) cuts.push_back(d.a * d.b);
+    }
+  std::sort(cuts.begin(), cuts.end());
+  cuts.erase(std::unique(cuts.begin(), cuts.end()), cuts.end());
+  while (!cuts.empty() && cuts.back() > E) cuts.pop_back();
+  for (size_t i = 0; i + 1 < cuts.size(); i++) if (cuts[i + 1] % cuts[i] != 0) return false;
+  if (cuts.back() != E) return false;
+  auto coef = [&](const std::vector<DigitUse> &u, int64_t cut) {
+    int64_t c = 0;
+    for (const DigitUse &d : u)
+      if (cut >= d.a && (d.b == 0 || cut < d.a * d.b)) c += d.coef * (cut / d.a);
+    return c;
+  };
+  for (size_t i = cuts.size() - 1; i-- > 0;) {
+    Dim d{ord, cuts[i + 1] / cuts[i], coef(ua, cuts[i]), coef(ub, cuts[i]), cuts[i]};
+    out->push_back(d);
+  }
+  return true;
 }
 
 std::string offset_fn(const char *name, const std::vector<Dim> &dims, bool use_a, int64_t c0) {
@@ -155,18 +192,9 @@ bool try_render_matmul(const KernelGraph &g, const std::string &fn, const Render
   for (int r : st.ranges) {
     const int64_t e = g.ranges[(size_t)r].extent;
     if (e < 0) return reject(__LINE__);
-    RangeUse ua, ub;
-    if (!range_use(g, la, r, &ua) || !range_use(g, lb, r, &ub)) return reject(__LINE__);
-    if (ua.split || ub.split) {
-      if (ua.plain || ub.plain) return reject(__LINE__);
-      int64_t c = ua.split ? ua.c : ub.c;
-      if ((ua.split && ub.split && ua.c != ub.c) || c <= 0 || e % c != 0) return reject(__LINE__);
-      Dim hi{r, e / c, ua.hi, ub.hi, 1, c}, lo{r, c, ua.lo, ub.lo, 2, c};
-      place_dim(hi);
-      place_dim(lo);
-    } else {
-      place_dim(Dim{r, e, ua.coef, ub.coef, 0, 0});
-    }
+    std::vector<Dim> digits;
+    if (!factor_range(g, la, lb, r, e, &digits)) return reject(__LINE__);
+    for (const Dim &d : digits) place_dim(d);
   }
   if (md.empty() || nd.empty()) return reject(__LINE__);
   // every other atom in the operand indices must be a plain range handled above
@@ -214,25 +242,27 @@ bool try_render_matmul(const KernelGraph &g, const std::string &fn, const Render
   S0.indent = 1;
   for (int r : st.ranges) S0.avail |= (uint64_t)1 << r;
   std::string decomp;
-  std::vector<std::pair<int, int64_t>> split_ranges;   // (ordinal, c) needing r = hi*c + lo
+  std::vector<std::pair<int, std::string>> range_sum;   // ordinal -> sum of digit * cut
   auto decompose = [&](const std::vector<Dim> &dims, const char *var) {
     if (dims.empty()) return;
     decomp += strf("  int t_%s = %s;\n", var, var);
     for (size_t i = dims.size(); i-- > 0;) {
       const Dim &d = dims[i];
-      std::string rv = d.part == 0 ? strf("r%d", d.ord) : strf("r%d_%s", d.ord, d.part == 1 ? "hi" : "lo");
-      if (i == 0) decomp += strf("  const int %s = t_%s;\n", rv.c_str(), var);
-      else decomp += strf("  const int %s = t_%s %% %lld; t_%s /= %lld;\n", rv.c_str(), var, (long long)d.extent, var, (long long)d.extent);
-      if (d.part == 0) em.bind_range(d.ord, rv);
-      else if (d.part == 1) split_ranges.push_back({d.ord, d.c});
+      std::string dv = strf("d%d_%lld", d.ord, (long long)d.cut);
+      if (i == 0) decomp += strf("  const int %s = t_%s;\n", dv.c_str(), var);
+      else decomp += strf("  const int %s = t_%s %% %lld; t_%s /= %lld;\n", dv.c_str(), var, (long long)d.extent, var, (long long)d.extent);
+      std::string term = d.cut == 1 ? dv : strf("%s * %lld", dv.c_str(), (long long)d.cut);
+      bool found = false;
+      for (auto &rs : range_sum) if (rs.first == d.ord) { rs.second += " + " + term; found = true; }
+      if (!found) range_sum.push_back({d.ord, term});
     }
   };
   decompose(md_full, "m");
   decompose(nd_full, "n");
   decompose(zd_full, "z");
-  for (auto &sr : split_ranges) {
-    decomp += strf("  const int r%d = r%d_hi * %lld + r%d_lo;\n", sr.first, sr.first, (long long)sr.second, sr.first);
-    em.bind_range(sr.first, strf("r%d", sr.first));
+  for (auto &rs : range_sum) {
+    decomp += strf("  const int r%d = %s;\n", rs.first, rs.second.c_str());
+    em.bind_range(rs.first, strf("r%d", rs.first));
   }
   em.preset(red, "acc");
   std::string val = em.emit(st.value, &S0);
@@ -305,8 +335,154 @@ bool try_render_matmul(const KernelGraph &g, const std::string &fn, const Render
   return true;
 }
 
-bool try_render_gather(const KernelGraph &, const std::string &, const RenderOptions &, RenderedKernel *) {
+// ── guarded embedding gather ──────────────────────────────────────────────
+//
+// The frontend expresses an embedding lookup as a masked sum over the whole
+// table (src/frontend.c:3494-3583, src/modelzoo/models/gpt2.c:93-153):
+//     out[..., j] = sum_v where(ids[...] == arange[v], table[v, j], 0)
+// When arange[v] == v for every v, at most one term is non-zero and the sum is
+// table[ids, j] (or 0 for an id that is not an integer in range).  The fast
+// kernel does that one load; a one-workgroup guard kernel checks the arange
+// buffer on every run, and the generic lowering runs instead when it fails.
+
+namespace {
+
+// cond is "a == b" in one of the forms the frontend produces.
+bool match_equal(const KernelGraph &g, int node, int *a, int *b) {
+  const KNode *k = &g.n(node);
+  if (k->op == POLY_OP_CAST && k->src.size() == 1) { node = k->src[0]; k = &g.n(node); }
+  if (k->op == POLY_OP_CMPEQ) { *a = k->src[0]; *b = k->src[1]; return true; }
+  if (k->op == POLY_OP_WHERE) {
+    const KNode &c = g.n(k->src[0]), &t = g.n(k->src[1]), &f = g.n(k->src[2]);
+    if (c.op != POLY_OP_CMPNE || t.op != POLY_OP_CONST || f.op != POLY_OP_CONST) return false;
+    auto cval = [](const KNode &n) { return n.u->arg.kind == POLY_ARG_FLOAT ? n.u->arg.f : (double)n.u->arg.i; };
+    if (cval(t) != 0.0 || cval(f) == 0.0) return false;
+    *a = c.src[0]; *b = c.src[1];
+    return true;
+  }
+  if (k->op == POLY_OP_NEG && k->dt == DT_BOOL && g.n(k->src[0]).op == POLY_OP_CMPNE) {
+    *a = g.n(k->src[0]).src[0]; *b = g.n(k->src[0]).src[1];
+    return true;
+  }
   return false;
+}
+
+bool is_zero_const(const KNode &n) {
+  if (n.op != POLY_OP_CONST) return false;
+  return n.u->arg.kind == POLY_ARG_FLOAT ? n.u->arg.f == 0.0 : n.u->arg.i == 0;
+}
+
+}  // namespace
+
+bool try_render_gather(const KernelGraph &g, const std::string &fn, const RenderOptions &opt, RenderedKernel *out) {
+  if (g.reduces.size() != 1 || !g.vars.empty() || opt.exit_if_flag || opt.exit_unless_flag) return reject(__LINE__);
+  const int red = g.reduces[0];
+  const KNode &R = g.n(red);
+  if (reduce_op(R) != POLY_OP_ADD || !dt_is_float(R.dt) || R.src.size() != 2) return reject(__LINE__);
+  const int vr = g.range_ord.at(R.src[1]);
+  const int64_t V = g.ranges[(size_t)vr].extent;
+  if (V < 64) return reject(__LINE__);
+  const KNode &W = g.n(R.src[0]);
+  if (W.op != POLY_OP_WHERE || !is_zero_const(g.n(W.src[2]))) return reject(__LINE__);
+  int ea, eb;
+  if (!match_equal(g, W.src[0], &ea, &eb)) return reject(__LINE__);
+  const uint64_t vbit = (uint64_t)1 << vr;
+  // one side of the comparison is arange[v], the other does not depend on v
+  int ids = -1, ar = -1;
+  if (!(g.n(ea).deps & vbit) && (g.n(eb).deps & vbit)) { ids = ea; ar = eb; }
+  else if (!(g.n(eb).deps & vbit) && (g.n(ea).deps & vbit)) { ids = eb; ar = ea; }
+  else return reject(__LINE__);
+  const KNode &AR = g.n(ar);
+  if (AR.op != POLY_OP_LOAD || AR.guard >= 0) return reject(__LINE__);
+  const KNode &arix = g.n(AR.src[0]);
+  if (arix.src.size() != 2) return reject(__LINE__);
+  const int ar_lin = g.n(arix.src[1]).lin;
+  if (ar_lin < 0) return reject(__LINE__);
+  {
+    const Lin &l = g.lins[(size_t)ar_lin];
+    if (l.c0 != 0 || l.terms.size() != 1 || l.terms[0].coef != 1) return reject(__LINE__);
+    const Atom &a = g.atoms[(size_t)l.terms[0].atom];
+    if (a.kind != Atom::RANGE || g.range_ord.at(a.node) != vr) return reject(__LINE__);
+  }
+  const int ar_param = g.param_slot(arix.src[0]);
+  if (g.params[(size_t)ar_param].written || g.params[(size_t)ar_param].numel < V) return reject(__LINE__);
+  const DT ids_dt = g.n(ids).dt;
+  if (ids_dt != AR.dt || !(dt_is_float(ids_dt) || dt_is_int(ids_dt))) return reject(__LINE__);
+  // the selected value: [CAST](LOAD(table[affine in v]))
+  int val = W.src[1];
+  if (g.n(val).dt != R.dt) return reject(__LINE__);
+  int tl = val;
+  if (g.n(tl).op == POLY_OP_CAST) tl = g.n(tl).src[0];
+  const KNode &TL = g.n(tl);
+  if (TL.op != POLY_OP_LOAD) return reject(__LINE__);
+  const KNode &tix = g.n(TL.src[0]);
+  if (tix.src.size() != 2) return reject(__LINE__);
+  const int t_lin = g.n(tix.src[1]).lin;
+  if (t_lin < 0) return reject(__LINE__);
+  bool aff;
+  const int64_t cv = g.lin_range_coef(g.lins[(size_t)t_lin], vr, &aff);
+  if (!aff || cv <= 0) return reject(__LINE__);
+  const int t_param = g.param_slot(tix.src[0]);
+  if (g.params[(size_t)t_param].written) return reject(__LINE__);
+  // nothing else under the REDUCE may depend on v
+  // (ids side was checked; the table index is affine in v; the comparison is consumed)
+
+  const DT rdt = R.dt, tdt = TL.dt;
+  RenderOptions fast = opt;
+  fast.allow_templates = false;
+  fast.exit_unless_flag = true;
+  fast.reduce_override[red] = [=, &g](Emitter &em, Scope *t) -> std::string {
+    std::string idv = em.emit(ids, t);
+    std::string gi = strf("gi%d", red), gh = strf("gh%d", red), acc = strf("acc%d", red);
+    em.stmt(t, strf("const int %s = (int)(%s);", gi.c_str(), idv.c_str()));
+    em.stmt(t, strf("const bool %s = ((%s)%s == %s) && %s >= 0 && %s < %lld;", gh.c_str(), dt_cname(ids_dt), gi.c_str(),
+                    idv.c_str(), gi.c_str(), gi.c_str(), (long long)V));
+    em.bind_range(vr, gi);
+    std::string addr = em.emit_lin(g.lins[(size_t)t_lin], t);
+    // 0 + x: the sum starts from +0, so a selected -0 comes out as +0
+    em.stmt(t, strf("const %s %s = %s ? (%s)0 + (%s)((%s)data%d[%s]) : (%s)0;", dt_cname(rdt), acc.c_str(), gh.c_str(),
+                    dt_cname(rdt), dt_cname(rdt), dt_cname(tdt), t_param, addr.c_str(), dt_cname(rdt)));
+    return acc;
+  };
+  std::string err;
+  RenderedKernel fk;
+  if (!render_kernel(g, fn, fast, &fk, &err)) return reject(__LINE__);
+  RenderOptions slow = opt;
+  slow.allow_templates = false;
+  slow.allow_coop_reduce = false;   // one thread per output: a small grid that exits at once when unused
+  slow.exit_if_flag = true;
+  RenderedKernel sk;
+  if (!render_kernel(g, fn, slow, &sk, &err)) return reject(__LINE__);
+
+  RenderedKernel::Guard gd;
+  gd.entry = "poly_guard";
+  gd.source = strf(R"HIP(
+extern "C" __global__ void __launch_bounds__(256) poly_guard(int* flag, const %s* __restrict__ ar) {
+  __shared__ int bad;
+  if (threadIdx.x == 0) bad = 0;
+  __syncthreads();
+  for (int i = threadIdx.x; i < %lld; i += 256)
+    if (ar[i] != (%s)i) bad = 1;
+  __syncthreads();
+  if (threadIdx.x == 0) *flag = bad ? 0 : 1;
+}
+)HIP", dt_cname(AR.dt), (long long)V, dt_cname(AR.dt));
+  gd.launch.grid[0] = 1;
+  gd.launch.block[0] = 256;
+  gd.arg_params.push_back(ar_param);
+
+  *out = fk;
+  out->klass = KernelClass::GATHER;
+  out->strategy = "guarded gather (arange check) + " + fk.strategy;
+  out->guards.push_back(gd);
+  out->fallback_source = sk.source;
+  out->fallback_entry = sk.entry;
+  out->fallback_launch = sk.launch;
+  // algorithmic bytes: ids + gathered rows + output (not the V-long masked sum)
+  double outn = 1;
+  for (int r : g.stores[0].ranges) outn *= (double)std::max<int64_t>(1, g.ranges[(size_t)r].extent);
+  out->bytes = outn * (dt_size(tdt) + dt_size(g.n(g.stores[0].param).dt)) + (double)V * dt_size(AR.dt);
+  return true;
 }
 
 }  // namespace polyhip

@@ -1,0 +1,70 @@
+"""Writes the serialized schedules (plan files) that bench.py and smoke() load on
+the GPU box, where the reference frontend is not part of the product path:
+
+    polygrad_amd/plans/gpt2_small_bf16_b8_t1024.polyplan   GPT-2 small forward, B=8, T=1024, bf16
+    polygrad_amd/plans/gpt2_small_bf16_b1_t1024.polyplan   the same graph for one sequence (parity slice)
+    polygrad_amd/plans/rowops_f32_8192.polyplan            config 2 (fused chain + row ops), 8192x8192 fp32
+    polygrad_amd/plans/matmul_bf16_<m>x<n>x<k>[_bt].polyplan   config 3 shapes
+
+The graphs are built with the REAL reference frontend and scheduler
+(oracle/_ref/libpolygrad.so through tests/refpoly.py); only the scheduled kernel
+graphs are stored, no reference code.  Run from the repository root:
+    python tests/golden/make_plans.py
+"""
+import os
+import sys
+
+import numpy as np
+
+HERE = os.path.dirname(os.path.abspath(__file__))
+ROOT = os.path.dirname(os.path.dirname(HERE))
+sys.path.insert(0, ROOT)
+sys.path.insert(0, os.path.join(ROOT, "tests"))
+
+import graphs  # noqa: E402
+import refpoly as R  # noqa: E402
+from hipharness import schedule_slots  # noqa: E402
+from polygrad_amd import save_schedule  # noqa: E402
+
+OUT = os.path.join(ROOT, "polygrad_amd", "plans")
+
+
+def save(c, sink, name):
+    sched = c.schedule(sink)
+    slots, n = schedule_slots(c, sched)
+    names = [None] * n
+    for i, tn in slots.items():
+        names[i] = tn[1]
+    path = os.path.join(OUT, name + ".polyplan")
+    save_schedule(sched, names, path)
+    c.L.poly_schedule_free(sched)
+    print(f"{name}: {os.path.getsize(path)} bytes")
+
+
+def main():
+    os.makedirs(OUT, exist_ok=True)
+    for batch in (8, 1):
+        c = R.Ctx()
+        cfg = graphs.GPT2Config(batch=batch)
+        sink, _ = graphs.gpt2_forward(c, cfg, R.BF16)
+        save(c, sink, f"gpt2_small_bf16_b{batch}_t1024")
+        c.close()
+    c = R.Ctx()
+    _, outs, sinks = graphs.fused_rowops(c, 8192, 8192)
+    for k, s in sinks.items():
+        save(c, s, f"rowops_f32_8192_{k}")
+    c.close()
+    for m, n, k, tb in ((4096, 4096, 4096, False), (8192, 8192, 8192, False), (16384, 3072, 768, False),
+                        (8192, 768, 3072, False), (4096, 4096, 4096, True)):
+        c = R.Ctx()
+        _, _, _, sink = graphs.matmul_bf16(c, m, n, k, transposed_b=tb)
+        save(c, sink, f"matmul_bf16_{m}x{n}x{k}" + ("_bt" if tb else ""))
+        c.close()
+    c = R.Ctx()
+    _, _, _, sink = graphs.matmul_bf16(c, 1024, 1024, 1024, batch=16)
+    save(c, sink, "matmul_bf16_b16_1024x1024x1024")
+    c.close()
+
+
+if __name__ == "__main__":
+    main()
