@@ -27,6 +27,28 @@ static bool render_root(const PolyUOp *root, const char *fn_name, int flags, Ren
     log_err("render_hip", "%s: %s", fn_name, err.c_str());
     return false;
   }
+  // Kernel symbols name what the kernel is (class, and a hash of its source), so
+  // identical kernels share one module and a profiler can tell the others apart.
+  static const char *const tag[] = {"ew", "rowred", "thrred", "mm", "gather", "copy"};
+  auto rename = [](std::string &src, const std::string &from, const std::string &to) {
+    for (size_t pos = 0; (pos = src.find(from, pos)) != std::string::npos; pos += to.size()) src.replace(pos, from.size(), to);
+  };
+  uint64_t h = fnv1a(rk->source.data(), rk->source.size());
+  std::string name = strf("poly_%s_%08x", tag[(int)rk->klass], (unsigned)(h ^ (h >> 32)));
+  if (rk->klass == KernelClass::MATMUL_MFMA) {
+    // strategy: "mfma 32x32x16 bf16 M=.. N=.. K=.. Z=.. tile .. A:k-major B:n-major"
+    long long M = 0, N = 0, K = 0, Z = 0;
+    const char *p = strstr(rk->strategy.c_str(), "M=");
+    if (p && sscanf(p, "M=%lld N=%lld K=%lld Z=%lld", &M, &N, &K, &Z) == 4)
+      name = strf("poly_mm_%lldx%lldx%lld_z%lld_%s%s_%08x", M, N, K, Z, strstr(p, "A:k-major") ? "k" : "m",
+                  strstr(p, "B:k-major") ? "k" : "n", (unsigned)(h ^ (h >> 32)));
+  }
+  rename(rk->source, " poly_k(", " " + name + "(");
+  rk->entry = name;
+  if (!rk->fallback_source.empty()) {
+    rename(rk->fallback_source, " poly_k(", " " + name + "_slow(");
+    rk->fallback_entry = name + "_slow";
+  }
   return true;
 }
 
