@@ -32,6 +32,8 @@
 #define POLY_BM 128
 #define POLY_BN 128
 #define POLY_BK 64
+#define POLY_GROUP_M 8
+#define POLY_PIPE 3
 #define POLY_WAVES_M 2
 #define POLY_WAVES_N 2
 #define POLY_A_KC 1
@@ -60,9 +62,13 @@ typedef poly_u32x4 poly_u32x4_u __attribute__((aligned(2)));
 #define POLY_TM (POLY_WM / 32)
 #define POLY_TN (POLY_WN / 32)
 #define POLY_NTHREADS (64 * POLY_WAVES_M * POLY_WAVES_N)
-// LDS row: BK elements + 8 elements (16 bytes) of padding keeps 16-byte fragment
-// reads of 8 consecutive rows on distinct banks.
-#define POLY_LDK (POLY_BK + 8)
+// LDS tile: [row][BK] with the 16-byte columns of a row XOR-swizzled by the row
+// number, so that the 16-byte fragment reads of 8 consecutive rows, the 16-byte
+// stores of one row and the 8-byte transposed stores of rows 8 apart all spread
+// over the banks without padding.
+#define POLY_LDK POLY_BK
+#define POLY_NCOL (POLY_BK / 8)
+__device__ __forceinline__ int poly_swz(int row) { return (row ^ (row >> 3)) & (POLY_NCOL - 1); }
 #define POLY_KT (POLY_K / POLY_BK)
 
 // Number of 16-byte global loads per thread for one operand tile.
@@ -88,7 +94,7 @@ struct PolyKC {
     for (int i = 0; i < NLOADS; i++) {
       const int c = threadIdx.x + i * POLY_NTHREADS;
       const int row = c / (POLY_BK / 8), kc = c % (POLY_BK / 8);
-      *(poly_u32x4 *)(lds + row * POLY_LDK + kc * 8) = regs[i];
+      *(poly_u32x4 *)(lds + row * POLY_LDK + ((kc ^ poly_swz(row)) * 8)) = regs[i];
     }
   }
 };
@@ -129,8 +135,9 @@ struct PolyXC {
         lo[1] = (a2 & 0xffffu) | (a3 << 16);
         hi[0] = (a0 >> 16) | (a1 & 0xffff0000u);
         hi[1] = (a2 >> 16) | (a3 & 0xffff0000u);
-        *(poly_u32x2 *)(lds + (chunk * 8 + 2 * j) * POLY_LDK + kq * 4) = lo;
-        *(poly_u32x2 *)(lds + (chunk * 8 + 2 * j + 1) * POLY_LDK + kq * 4) = hi;
+        const int r0 = chunk * 8 + 2 * j, r1 = r0 + 1;
+        *(poly_u32x2 *)(lds + r0 * POLY_LDK + (((kq >> 1) ^ poly_swz(r0)) * 8) + (kq & 1) * 4) = lo;
+        *(poly_u32x2 *)(lds + r1 * POLY_LDK + (((kq >> 1) ^ poly_swz(r1)) * 8) + (kq & 1) * 4) = hi;
       }
     }
   }
@@ -153,7 +160,18 @@ extern "C" __global__ void __launch_bounds__(POLY_NTHREADS) poly_k(POLY_SIGNATUR
     const int xcd = bid & 7, idx = bid >> 3;
     bid = (xcd < REM ? xcd * (PER + 1) : REM * (PER + 1) + (xcd - REM) * PER) + idx;
   }
-  const int tile_m = bid % TILES_M, tile_n = bid / TILES_M;
+  // Within a run, tiles are visited in groups of POLY_GROUP_M tile rows so that the
+  // workgroups resident on one XCD at a time share both A and B panels.
+  int tile_m, tile_n;
+  {
+    constexpr int GM = POLY_GROUP_M;
+    const int per_group = GM * TILES_N;
+    const int group = bid / per_group, first_m = group * GM;
+    const int gsz = (TILES_M - first_m) < GM ? (TILES_M - first_m) : GM;
+    const int in_group = bid - group * per_group;
+    tile_m = first_m + in_group % gsz;
+    tile_n = in_group / gsz;
+  }
   const int z = blockIdx.y;
   const int m0 = tile_m * POLY_BM, n0 = tile_n * POLY_BN;
 
@@ -164,7 +182,7 @@ extern "C" __global__ void __launch_bounds__(POLY_NTHREADS) poly_k(POLY_SIGNATUR
   // Rows past the edge are clamped to the last valid row: they are loaded and
   // multiplied but never stored.
 #if POLY_A_KC
-  poly_u32x4 ra[POLY_A_LOADS];
+  poly_u32x4 ra0[POLY_A_LOADS], ra1[POLY_A_LOADS];
   int a_off[POLY_A_LOADS];
 #pragma unroll
   for (int i = 0; i < POLY_A_LOADS; i++) {
@@ -174,7 +192,7 @@ extern "C" __global__ void __launch_bounds__(POLY_NTHREADS) poly_k(POLY_SIGNATUR
   typedef PolyKC<POLY_BM, POLY_A_LOADS> StageA;
 #else
   typedef PolyXC<POLY_BM> StageA;
-  poly_u32x4 ra[StageA::NLOADS];
+  poly_u32x4 ra0[StageA::NLOADS], ra1[StageA::NLOADS];
   int a_off[StageA::NBLK], a_kq[StageA::NBLK];
 #pragma unroll
   for (int b = 0; b < StageA::NBLK; b++) {
@@ -185,7 +203,7 @@ extern "C" __global__ void __launch_bounds__(POLY_NTHREADS) poly_k(POLY_SIGNATUR
   }
 #endif
 #if POLY_B_KC
-  poly_u32x4 rb[POLY_B_LOADS];
+  poly_u32x4 rb0[POLY_B_LOADS], rb1[POLY_B_LOADS];
   int b_off[POLY_B_LOADS];
 #pragma unroll
   for (int i = 0; i < POLY_B_LOADS; i++) {
@@ -195,7 +213,7 @@ extern "C" __global__ void __launch_bounds__(POLY_NTHREADS) poly_k(POLY_SIGNATUR
   typedef PolyKC<POLY_BN, POLY_B_LOADS> StageB;
 #else
   typedef PolyXC<POLY_BN> StageB;
-  poly_u32x4 rb[StageB::NLOADS];
+  poly_u32x4 rb0[StageB::NLOADS], rb1[StageB::NLOADS];
   int b_off[StageB::NBLK], b_kq[StageB::NBLK];
 #pragma unroll
   for (int b = 0; b < StageB::NBLK; b++) {
@@ -206,7 +224,7 @@ extern "C" __global__ void __launch_bounds__(POLY_NTHREADS) poly_k(POLY_SIGNATUR
   }
 #endif
 
-  auto load_tiles = [&](int kt) {
+  auto load_tiles = [&](int kt, auto &ra, auto &rb) {
     const int k0 = kt * POLY_BK;
 #if POLY_A_KC
     StageA::load(gA, a_off, poly_a_k(k0), ra);
@@ -232,7 +250,7 @@ extern "C" __global__ void __launch_bounds__(POLY_NTHREADS) poly_k(POLY_SIGNATUR
 
   const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
   const int wm = (wave % POLY_WAVES_M) * POLY_WM, wn = (wave / POLY_WAVES_M) * POLY_WN;
-  const int frag_row = lane & 31, frag_k = (lane >> 5) * 8;
+  const int frag_row = lane & 31;
 
   poly_acc16 acc[POLY_TM][POLY_TN];
 #pragma unroll
@@ -242,34 +260,91 @@ extern "C" __global__ void __launch_bounds__(POLY_NTHREADS) poly_k(POLY_SIGNATUR
 #pragma unroll
       for (int r = 0; r < 16; r++) acc[i][j][r] = 0.0f;
 
-  load_tiles(0);
-  StageA::store(lds_a[0], ra);
-  StageB::store(lds_b[0], rb);
-  __syncthreads();
+  // fragment addresses: row part and per-tile swizzle are loop invariant
+  int a_row_off[POLY_TM], a_swz[POLY_TM], b_row_off[POLY_TN], b_swz[POLY_TN];
+#pragma unroll
+  for (int i = 0; i < POLY_TM; i++) { const int r = wm + i * 32 + frag_row; a_row_off[i] = r * POLY_LDK; a_swz[i] = poly_swz(r); }
+#pragma unroll
+  for (int j = 0; j < POLY_TN; j++) { const int r = wn + j * 32 + frag_row; b_row_off[j] = r * POLY_LDK; b_swz[j] = poly_swz(r); }
+  const int frag_col = lane >> 5;   // which 8-wide half of a 16-deep K step
 
-  for (int kt = 0; kt < POLY_KT; kt++) {
-    const int cur = kt & 1;
-    if (kt + 1 < POLY_KT) load_tiles(kt + 1);
-    const POLY_TIN *la = lds_a[cur] + (wm + frag_row) * POLY_LDK + frag_k;
-    const POLY_TIN *lb = lds_b[cur] + (wn + frag_row) * POLY_LDK + frag_k;
+  // Fragments are double buffered in registers: the LDS reads of K step ks+1 are
+  // issued before the MFMAs of step ks, so their latency hides behind the math.
+  poly_in8 fa[2][POLY_TM], fb[2][POLY_TN];
+  auto read_frags = [&](int cur, int ks, int buf) {
 #pragma unroll
-    for (int ks = 0; ks < POLY_BK / 16; ks++) {
-      poly_in8 fa[POLY_TM], fb[POLY_TN];
+    for (int i = 0; i < POLY_TM; i++) fa[buf][i] = *(const poly_in8 *)(lds_a[cur] + a_row_off[i] + (((ks * 2 + frag_col) ^ a_swz[i]) * 8));
 #pragma unroll
-      for (int i = 0; i < POLY_TM; i++) fa[i] = *(const poly_in8 *)(la + i * 32 * POLY_LDK + ks * 16);
+    for (int j = 0; j < POLY_TN; j++) fb[buf][j] = *(const poly_in8 *)(lds_b[cur] + b_row_off[j] + (((ks * 2 + frag_col) ^ b_swz[j]) * 8));
+  };
+  auto compute = [&](int cur, int ks_begin, int ks_end) {
+    read_frags(cur, ks_begin, ks_begin & 1);
 #pragma unroll
-      for (int j = 0; j < POLY_TN; j++) fb[j] = *(const poly_in8 *)(lb + j * 32 * POLY_LDK + ks * 16);
+    for (int ks = ks_begin; ks < ks_end; ks++) {
+      if (ks + 1 < ks_end) read_frags(cur, ks + 1, (ks + 1) & 1);
 #pragma unroll
       for (int i = 0; i < POLY_TM; i++)
 #pragma unroll
-        for (int j = 0; j < POLY_TN; j++) acc[i][j] = POLY_MFMA(fa[i], fb[j], acc[i][j]);
+        for (int j = 0; j < POLY_TN; j++) acc[i][j] = POLY_MFMA(fa[ks & 1][i], fb[ks & 1][j], acc[i][j]);
     }
+  };
+
+  constexpr int KS = POLY_BK / 16, KS_HALF = KS / 2;
+#if POLY_PIPE == 3
+  // Software pipeline, three tiles deep: tile kt is multiplied out of one LDS
+  // buffer; tile kt+1 waits in one register set and is written to the other LDS
+  // buffer in the middle of the iteration; tile kt+2 is in flight into the second
+  // register set, and the loads of tile kt+3 are issued as soon as the first set
+  // is free.  Every global load has about two and a half iterations to land.
+  // Tile t always uses register set t & 1, hence the loop is unrolled by two.
+  load_tiles(0, ra0, rb0);
+  StageA::store(lds_a[0], ra0);
+  StageB::store(lds_b[0], rb0);
+  if (POLY_KT > 1) load_tiles(1, ra1, rb1);
+  if (POLY_KT > 2) load_tiles(2, ra0, rb0);
+  __syncthreads();
+
+  auto iteration = [&](int kt, auto &ra_next, auto &rb_next) {
+    const int cur = kt & 1;
+    compute(cur, 0, KS_HALF);
+    __builtin_amdgcn_sched_barrier(0);
     if (kt + 1 < POLY_KT) {
-      StageA::store(lds_a[cur ^ 1], ra);
-      StageB::store(lds_b[cur ^ 1], rb);
+      StageA::store(lds_a[cur ^ 1], ra_next);
+      StageB::store(lds_b[cur ^ 1], rb_next);
     }
+    if (kt + 3 < POLY_KT) load_tiles(kt + 3, ra_next, rb_next);
+    __builtin_amdgcn_sched_barrier(0);
+    compute(cur, KS_HALF, KS);
+    __syncthreads();
+  };
+  for (int kt = 0; kt < POLY_KT; kt += 2) {
+    iteration(kt, ra1, rb1);
+    if (kt + 1 < POLY_KT) iteration(kt + 1, ra0, rb0);
+  }
+#else
+  // Software pipeline, two tiles deep (for tiles whose accumulators leave no room
+  // for a second staging register set): the global loads of tile kt+1 are issued
+  // before the first half of tile kt is multiplied, and land in the other LDS
+  // buffer between the two halves.
+  load_tiles(0, ra0, rb0);
+  StageA::store(lds_a[0], ra0);
+  StageB::store(lds_b[0], rb0);
+  __syncthreads();
+  for (int kt = 0; kt < POLY_KT; kt++) {
+    const int cur = kt & 1;
+    if (kt + 1 < POLY_KT) load_tiles(kt + 1, ra0, rb0);
+    __builtin_amdgcn_sched_barrier(0);
+    compute(cur, 0, KS_HALF);
+    __builtin_amdgcn_sched_barrier(0);
+    if (kt + 1 < POLY_KT) {
+      StageA::store(lds_a[cur ^ 1], ra0);
+      StageB::store(lds_b[cur ^ 1], rb0);
+    }
+    __builtin_amdgcn_sched_barrier(0);
+    compute(cur, KS_HALF, KS);
     __syncthreads();
   }
+#endif
 
   // Accumulator layout of the 32x32 MFMA: register r of lane l holds
   // row 8*(r/4) + 4*(l/32) + r%4, column l%32 of the tile.

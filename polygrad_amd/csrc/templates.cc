@@ -218,7 +218,8 @@ bool try_render_matmul(const KernelGraph &g, const std::string &fn, const Render
   for (const Dim &d : zd) Z *= d.extent;
   if (M > 2147483647LL || N > 2147483647LL || Z > 65535) return reject(__LINE__);
 
-  const int BK = 64;
+  int BK = 64;
+  if (const char *e = getenv("POLY_HIP_MM_BK")) BK = atoi(e) == 32 ? 32 : 64;
   // operand layout: contiguous along K, or along its row axis
   auto layout = [&](const KSplit &ks, const std::vector<Dim> &dims, bool is_a, int64_t rows, bool *kc) {
     int64_t inner_c = is_a ? dims.back().ca : dims.back().cb;
@@ -230,9 +231,28 @@ bool try_render_matmul(const KernelGraph &g, const std::string &fn, const Render
   if (!layout(ka, md, true, M, &a_kc) || !layout(kb, nd, false, N, &b_kc)) return reject(__LINE__);
 
   // tile shape: 4 waves; narrow outputs get a narrow tile
+  // Candidates: (BM, BN, waves M x N, workgroups resident per CU, throughput of one CU
+  // relative to the 256x256 tile as measured on 8192^3).  Pick the smallest estimated
+  // time = rounds over the chip * time of one tile.
   int BM = 128, BN = 128, WVM = 2, WVN = 2;
   if (N <= 64) { BN = 64; BM = 256; WVM = 4; WVN = 1; }
   else if (M <= 64) { BM = 64; BN = 256; WVM = 1; WVN = 4; }
+  else {
+    struct Cand { int bm, bn, wm, wn, per_cu; double thr; };
+    static const Cand cands[] = {{256, 256, 4, 2, 1, 1.00}, {256, 128, 4, 2, 1, 0.84}, {128, 256, 2, 4, 1, 0.84}, {128, 128, 2, 2, 2, 0.80}};
+    double best = 0;
+    for (const Cand &c : cands) {
+      if (!a_kc && M % 8) continue;
+      double t = (double)((M + c.bm - 1) / c.bm) * (double)((N + c.bn - 1) / c.bn) * (double)Z;
+      double rounds = std::ceil(t / (256.0 * c.per_cu));
+      double est = rounds * (double)c.bm * c.bn / (c.thr / c.per_cu);
+      if (best == 0 || est < best) { best = est; BM = c.bm; BN = c.bn; WVM = c.wm; WVN = c.wn; }
+    }
+  }
+  if (const char *ov = getenv("POLY_HIP_MM_TILE")) {   // "BM,BN,WVM,WVN": tuning experiments
+    int a, b2, c2, d2;
+    if (sscanf(ov, "%d,%d,%d,%d", &a, &b2, &c2, &d2) == 4) { BM = a; BN = b2; WVM = c2; WVN = d2; }
+  }
   const int64_t tiles = ((M + BM - 1) / BM) * ((N + BN - 1) / BN);
   if (tiles > 2147483647LL / 2) return reject(__LINE__);
 
@@ -287,6 +307,12 @@ bool try_render_matmul(const KernelGraph &g, const std::string &fn, const Render
   cfg += strf("#define POLY_MFMA(a, b, c) __builtin_amdgcn_mfma_f32_32x32x16_%s(a, b, c, 0, 0, 0)\n", A.dt == DT_BF16 ? "bf16" : "f16");
   cfg += strf("#define POLY_M %lld\n#define POLY_N %lld\n#define POLY_K %lld\n#define POLY_Z %lld\n", (long long)M, (long long)N, (long long)K, (long long)Z);
   cfg += strf("#define POLY_BM %d\n#define POLY_BN %d\n#define POLY_BK %d\n#define POLY_WAVES_M %d\n#define POLY_WAVES_N %d\n", BM, BN, BK, WVM, WVN);
+  cfg += strf("#define POLY_GROUP_M %d\n", BM >= 256 ? 4 : 8);
+  // a 256x256 tile holds 128 accumulator registers per lane: no room for the second
+  // staging register set of the three-deep pipeline
+  int pipe = (BM * BN >= 256 * 256) ? 2 : 3;
+  if (const char *e = getenv("POLY_HIP_MM_PIPE")) pipe = atoi(e) == 2 ? 2 : 3;
+  cfg += strf("#define POLY_PIPE %d\n", pipe);
   cfg += strf("#define POLY_A_KC %d\n#define POLY_B_KC %d\n", a_kc ? 1 : 0, b_kc ? 1 : 0);
   cfg += strf("#define POLY_A_PTR data%d\n#define POLY_B_PTR data%d\n", A.param, B.param);
   cfg += offset_fn("poly_a_row", md, true, 0);
@@ -314,7 +340,7 @@ bool try_render_matmul(const KernelGraph &g, const std::string &fn, const Render
   out->entry = "poly_k";
   out->launch.grid[0] = (unsigned)tiles;
   out->launch.grid[1] = (unsigned)Z;
-  out->launch.block[0] = 256;
+  out->launch.block[0] = (unsigned)(64 * WVM * WVN);
   out->klass = KernelClass::MATMUL_MFMA;
   out->strategy = strf("mfma 32x32x16 %s M=%lld N=%lld K=%lld Z=%lld tile %dx%dx%d A:%s B:%s", A.dt == DT_BF16 ? "bf16" : "f16",
                        (long long)M, (long long)N, (long long)K, (long long)Z, BM, BN, BK, a_kc ? "k-major" : "m-major",
