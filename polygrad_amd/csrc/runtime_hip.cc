@@ -67,12 +67,19 @@ std::string cache_dir() {
 
 // hiprtc needs no device, so this also serves compile-only checks.
 bool compile_to_code_object(const std::string &source, std::vector<char> *code, std::string *log) {
+  // Compiler options; they are part of the cache key.  Contraction to FMA is off so
+  // that a*b+c rounds twice, as in the reference's CPU backend (x86-64 baseline, no FMA).
+  // Packed FP32 instructions are kept out of generated code on purpose.
+  static const char *opts[] = {"--offload-arch=gfx950", "-O3", "-std=c++17", "-ffp-contract=off", "-Xclang",
+                               "-target-feature", "-Xclang", "-packed-fp32-ops", "-Wno-unused-value"};
+  const int n_opts = (int)(sizeof(opts) / sizeof(opts[0]));
   uint64_t h = fnv1a(source.data(), source.size());
+  for (int i = 0; i < n_opts; i++) h = h * 1099511628211ULL ^ fnv1a(opts[i], strlen(opts[i]));
   Runtime &r = rt();
   auto it = r.code_cache.find(h);
   if (it != r.code_cache.end()) { *code = it->second; return true; }
   std::string dir = cache_dir();
-  std::string path = dir.empty() ? "" : strf("%s/%016llx.hsaco", dir.c_str(), (unsigned long long)h);
+  std::string path = dir.empty() ? "" : strf("%s/%016llx_%zu.hsaco", dir.c_str(), (unsigned long long)h, source.size());
   if (!path.empty()) {
     std::ifstream f(path, std::ios::binary);
     if (f) {
@@ -85,10 +92,7 @@ bool compile_to_code_object(const std::string &source, std::vector<char> *code, 
     *log = "hiprtcCreateProgram failed";
     return false;
   }
-  // Packed FP32 instructions are kept out of generated code on purpose.
-  const char *opts[] = {"--offload-arch=gfx950", "-O3", "-std=c++17", "-Xclang", "-target-feature",
-                        "-Xclang", "-packed-fp32-ops", "-Wno-unused-value"};
-  hiprtcResult res = hiprtcCompileProgram(prog, (int)(sizeof(opts) / sizeof(opts[0])), opts);
+  hiprtcResult res = hiprtcCompileProgram(prog, n_opts, opts);
   size_t ls = 0;
   hiprtcGetProgramLogSize(prog, &ls);
   if (ls > 1) { log->resize(ls); hiprtcGetProgramLog(prog, &(*log)[0]); }
@@ -137,6 +141,9 @@ void *runtime_alloc(size_t nbytes) {
   void *p = nullptr;
   if (nbytes == 0) nbytes = 4;
   if (!check(hipMalloc(&p, nbytes), "hipMalloc")) return nullptr;
+  // Fresh memory reads as zero, like the reference's host allocator (calloc,
+  // src/exec_plan.c:228-231); ordered on the stream every kernel runs on.
+  if (!check(hipMemsetAsync(p, 0, nbytes, rt().stream), "hipMemsetAsync")) { (void)hipFree(p); return nullptr; }
   return p;
 }
 
