@@ -53,6 +53,7 @@ class HipPlan:
         self.slots = [Slot(i, s.buf_slots[i], (names[i] if names and i < len(names) else "") or "")
                       for i in range(s.n_buf_slots)]
         self.n_kernels = self.lib.poly_hip_plan_n_kernels(self.handle)
+        self._ext_stream = None
 
     @classmethod
     def from_file(cls, path):
@@ -73,9 +74,20 @@ class HipPlan:
     def external_slots(self):
         return [s for s in self.slots if not s.is_intermediate]
 
+    def _order_after_torch(self):
+        """The backend launches on its own non-blocking stream: make that stream wait
+        for whatever torch has queued so far (fills, copies, random init of the tensors
+        handed in), without blocking the host."""
+        import torch
+        if self._ext_stream is None:
+            self._ext_stream = torch.cuda.ExternalStream(self.lib.poly_hip_stream())
+        self._ext_stream.wait_stream(torch.cuda.current_stream())
+
     def _ptr_array(self, slot_data):
         n = len(self.slots)
         arr = (C.c_void_p * n)()
+        if any(v is not None and not isinstance(v, int) for v in slot_data):
+            self._order_after_torch()
         for i in range(n):
             v = slot_data[i] if i < len(slot_data) else None
             if v is None:

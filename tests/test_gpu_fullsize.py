@@ -1,0 +1,210 @@
+"""Parity at the benchmark configurations' full sizes, where the CPU reference
+takes minutes to hours: the GPU result is checked through properties that do
+not depend on size (rows of a softmax sum to 1, LayerNorm rows have mean 0 and
+variance 1, independence of batch elements) and against float64 arithmetic of
+the same formula on sampled rows.  The plans are the schedules the reference's
+scheduler produced for these graphs (tests/golden/make_plans.py)."""
+import os
+
+import numpy as np
+import pytest
+
+import graphs
+import refpoly as R
+from hipharness import assert_close, run_hip, run_ref
+from polygrad_amd import HipPlan
+from polygrad_amd.inputs import gpt2_slot_tensors
+
+pytestmark = pytest.mark.gpu
+
+PLANS = os.path.join(os.path.dirname(os.path.abspath(__file__)), "..", "polygrad_amd", "plans")
+
+
+def load(name):
+    return HipPlan.from_file(os.path.join(PLANS, name + ".polyplan"))
+
+
+def slot(plan, name):
+    return [s for s in plan.slots if s.name == name][0]
+
+
+# ── config 2: y = clamp(exp2(a*b + c), -4, 4) on 8192 x 8192 fp32, then row ops ──────────
+
+N2 = 8192
+
+
+@pytest.fixture(scope="module")
+def rowops_inputs():
+    import torch
+    g = torch.Generator(device="cuda")
+    g.manual_seed(1)
+    a, b, c = (torch.rand(N2 * N2, generator=g, device="cuda", dtype=torch.float32) * 2 - 1 for _ in range(3))
+    y64 = torch.clamp(torch.exp2(a.double() * b.double() + c.double()), -4.0, 4.0).view(N2, N2)
+    return dict(a=a, b=b, c=c), y64
+
+
+def run_rowop(kind, inputs):
+    import torch
+    plan = load(f"rowops_f32_8192_{kind}")
+    data = [None] * len(plan.slots)
+    out = None
+    for s in plan.external_slots():
+        if s.name in inputs:
+            data[s.index] = inputs[s.name]
+        else:
+            assert s.name == kind
+            out = torch.full((s.numel,), float("nan"), device="cuda", dtype=torch.float32)
+            data[s.index] = out
+    plan.run(data)
+    plan.run(data)
+    info = plan.kernel_info()
+    plan.close()
+    return out, info
+
+
+def test_rowops_sum_and_max_full_size(rowops_inputs):
+    inputs, y64 = rowops_inputs
+    got, info = run_rowop("sum", inputs)
+    assert all(k["klass"] == "row-reduce" for k in info)
+    want = y64.sum(1)
+    # fp32 tree sum of 8192 positive terms of size <= 4: 1e-4 relative is ~100x the expected error
+    assert_close(got.cpu().numpy(), want.cpu().numpy(), rtol=1e-4, what="row sums 8192x8192")
+    got, info = run_rowop("max", inputs)
+    # max is order independent: only the elementwise chain's rounding (exp2 polynomial, fp32 a*b+c) remains
+    assert_close(got.cpu().numpy(), y64.max(1).values.cpu().numpy(), rtol=1e-5, what="row maxima 8192x8192")
+
+
+def test_rowops_softmax_full_size(rowops_inputs):
+    import torch
+    inputs, y64 = rowops_inputs
+    got, _ = run_rowop("softmax", inputs)
+    got = got.view(N2, N2)
+    sums = got.double().sum(1)
+    assert float((sums - 1).abs().max()) < 1e-5, "softmax rows must sum to 1"
+    assert float(got.min()) >= 0.0
+    want = torch.softmax(y64, dim=1)
+    err = ((got.double() - want).abs() / want).max()
+    assert float(err) < 1e-4, f"softmax relative error {float(err):.3e}"
+
+
+def test_rowops_layernorm_full_size(rowops_inputs):
+    import torch
+    inputs, y64 = rowops_inputs
+    got, _ = run_rowop("layernorm", inputs)
+    got = got.view(N2, N2).double()
+    assert float(got.mean(1).abs().max()) < 1e-5, "LayerNorm rows must have mean 0"
+    assert float((got.var(1, unbiased=False) - 1).abs().max()) < 1e-3, "LayerNorm rows must have variance 1"
+    mu = y64.mean(1, keepdim=True)
+    var = ((y64 - mu) ** 2).mean(1, keepdim=True)
+    want = (y64 - mu) / torch.sqrt(var + 1e-5)
+    # normalised values are O(1); fp32 statistics over 8192 elements leave ~1e-6
+    assert float((got - want).abs().max()) < 1e-4
+
+
+# ── config 3: bf16 matmul sweep at full size ─────────────────────────────────────────────
+
+SWEEP = [("matmul_bf16_4096x4096x4096", 4096, 4096, 4096, False, None),
+         ("matmul_bf16_8192x8192x8192", 8192, 8192, 8192, False, None),
+         ("matmul_bf16_16384x3072x768", 16384, 3072, 768, False, None),
+         ("matmul_bf16_8192x768x3072", 8192, 768, 3072, False, None),
+         ("matmul_bf16_4096x4096x4096_bt", 4096, 4096, 4096, True, None),
+         ("matmul_bf16_b16_1024x1024x1024", 1024, 1024, 1024, False, 16)]
+
+
+@pytest.mark.parametrize("name,m,n,k,tb,batch", SWEEP)
+def test_matmul_sweep_full_size_sampled_rows(name, m, n, k, tb, batch):
+    import torch
+    plan = load(name)
+    g = torch.Generator(device="cuda")
+    g.manual_seed(2)
+    data = [None] * len(plan.slots)
+    for s in plan.external_slots():
+        if s.name == "C":
+            data[s.index] = torch.full((s.numel,), float("nan"), device="cuda", dtype=torch.float32)
+        else:
+            data[s.index] = (torch.randn(s.numel, generator=g, device="cuda") * 0.02).to(torch.bfloat16)
+    plan.run(data)
+    info = plan.kernel_info()
+    plan.close()
+    assert len(info) == 1 and info[0]["klass"] == "matmul-mfma", info
+    A = data[slot(plan, "A").index]
+    B = data[slot(plan, "B").index]
+    Cm = data[slot(plan, "C").index]
+    assert bool(torch.isfinite(Cm).all())
+    nb = batch or 1
+    A = A.view(nb, m, k)
+    Cm = Cm.view(nb, m, n)
+    B64 = (B.view(n, k).t() if tb else B.view(k, n)).double()
+    rows = torch.tensor(sorted({0, 1, 31, 32, 127, 128, 255, 256, m // 2 - 1, m // 2, m - 257, m - 2, m - 1}), device="cuda")
+    for z in sorted({0, nb - 1}):
+        a64 = A[z][rows].double()
+        want = a64 @ B64
+        bound = a64.abs() @ B64.abs()          # sum of |terms|: scale of the rounding error of any summation order
+        err = (Cm[z][rows].double() - want).abs()
+        assert bool((err <= 1e-4 * bound + 1e-30).all()), f"{name}: max err/bound {float((err / bound).max()):.3e}"
+
+
+# ── config 4: GPT-2 small ────────────────────────────────────────────────────────────────
+
+def test_gpt2_small_batch_elements_are_independent():
+    """B=8 and B=1 plans (different grids and tile choices) give the same logits for
+    the same sequence: attention is per (batch, head), every other op per row."""
+    import torch
+    p8 = load("gpt2_small_bf16_b8_t1024")
+    d8, n8 = gpt2_slot_tensors(p8, seed=3)
+    p8.run(d8)
+    T, V = 1024, 50257
+    out8 = n8["output"].view(8, T, V)
+    assert bool(torch.isfinite(out8.float()).all()) and float(out8.float().abs().max()) > 0
+    p1 = load("gpt2_small_bf16_b1_t1024")
+    d1, n1 = gpt2_slot_tensors(p1, seed=3)
+    for s in p1.external_slots():            # same weights, sequence 5 of the batch
+        if s.name == "x":
+            d1[s.index].copy_(n8["x"].view(8, T)[5])
+        elif s.name != "output":
+            d1[s.index].copy_(n8[s.name])
+    p1.run(d1)
+    a = n1["output"].view(T, V).float()
+    b = out8[5].float()
+    p8.close()
+    p1.close()
+    diff = (a - b).abs()
+    assert float(diff.max()) <= 2e-2 * float(b.abs().max()), f"max diff {float(diff.max())}"
+    assert float((diff > 0).float().mean()) < 1e-3, "same arithmetic per element: batch size must not change the logits"
+
+
+def test_gpt2_small_full_width_short_context_matches_reference():
+    """GPT-2 small at its real width and depth (12 layers, d_model 768, vocab 50257) on one
+    32-token sequence: the reference CPU backend finishes it in seconds.
+
+    Twelve layers of bf16 rounding amplify the one-ulp differences that a different
+    summation order causes, so besides the element-wise bf16 tolerance (2e-2 of the value
+    plus 2e-2 of the tensor's scale) the GPU logits must be as close to the fp32 evaluation
+    of the same network (reference CPU backend, f32 graph, same bf16-valued weights) as the
+    reference's own bf16 logits are."""
+    if not R.available():
+        pytest.skip("reference library not built")
+    cfg = graphs.GPT2Config(batch=1, ctx=32)
+    c = R.Ctx()
+    sink, bufs = graphs.gpt2_forward(c, cfg, R.BF16)
+    arrays = graphs.gpt2_inputs(cfg, bufs, seed=3, wdt=R.BF16)
+    want = run_ref(c, sink, arrays)
+    got, info = run_hip(c, sink, arrays)
+    by_name = {n: arrays[t] for n, t in bufs.items()}
+    out = bufs["output"]
+    w = R.bf16_bits_to_f32(want[out]).astype(np.float64)
+    h = R.bf16_bits_to_f32(got[out]).astype(np.float64)
+    c.close()
+    assert np.isfinite(h).all() and np.abs(h).max() > 0
+    assert sum(k["klass"] == "matmul-mfma" for k in info) >= 12 * 4
+    assert_close(h, w, rtol=2e-2, atol=2e-2 * float(np.abs(w).max()), what="GPT-2 small logits, T=32")
+
+    c = R.Ctx()
+    sink32, bufs32 = graphs.gpt2_forward(c, cfg, R.F32)
+    arr32 = {t: (R.bf16_bits_to_f32(by_name[n]) if by_name[n].dtype == np.uint16 else by_name[n].astype(np.float32))
+             for n, t in bufs32.items()}
+    truth = run_ref(c, sink32, arr32)[bufs32["output"]].astype(np.float64)
+    c.close()
+    rms = lambda d: float(np.sqrt((d ** 2).mean()))
+    e_gpu, e_ref = rms(h - truth), rms(w - truth)
+    assert e_gpu <= 1.25 * e_ref, f"GPU rms error {e_gpu:.3e} vs reference rms error {e_ref:.3e} against the fp32 network"
