@@ -110,11 +110,20 @@ PolyHipPlan *poly_hip_compile_schedule(PolyCtx *ctx, const PolySchedule *schedul
 int poly_hip_plan_run(PolyHipPlan *plan, void **slot_data, int n_slots,
                       const PolyVarBinding *var_bindings, int n_var_bindings);
 void poly_hip_plan_free(PolyHipPlan *plan);
+/* Kernel groups of `schedule` that poly_hip_compile_schedule runs as ONE launch
+ * (attention: scores, scale/mask, row max, row sum, normalise, weighted sum of
+ * values -- src/modelzoo/models/gpt2.c:411-441 builds it as separate realized
+ * tensors).  Returns their number, <0 on a malformed schedule; needs no device.
+ * For 0 <= index < count, *n_items_out receives how many scheduled kernels the
+ * group replaces and *source_out its HIP source (free with poly_hip_free_string).
+ * No reference counterpart: the reference launches every scheduled kernel. */
+int poly_hip_fused_groups(const PolySchedule *schedule, int index, char **source_out, int *n_items_out);
 /* Introspection for benches and tests. */
 int poly_hip_plan_n_kernels(const PolyHipPlan *plan);
 /* Fills at most cap entries; per kernel (in execution order): class id
  * (0 elementwise, 1 row-reduce, 2 thread-reduce, 3 matmul-mfma, 4 gather,
- * 5 copy), algorithmic bytes, flops. Returns the number of kernels. */
+ * 5 copy, 6 attention-mfma), algorithmic bytes, flops.  A "kernel" here is one
+ * launch: a fused group counts once.  Returns the number of launches. */
 int poly_hip_plan_kernel_info(const PolyHipPlan *plan, int cap, int *klass, double *bytes,
                               double *flops);
 /* Times each kernel of one plan run with HIP events on the backend stream;

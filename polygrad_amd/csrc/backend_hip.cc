@@ -19,17 +19,10 @@ static RenderOptions options_from_flags(int flags) {
   return o;
 }
 
-static bool render_root(const PolyUOp *root, const char *fn_name, int flags, RenderedKernel *rk) {
-  KernelGraph g;
-  if (!g.build(root)) { log_err("render_hip", "%s: %s", fn_name, g.error.c_str()); return false; }
-  std::string err;
-  if (!render_kernel(g, "poly_k", options_from_flags(flags), rk, &err)) {
-    log_err("render_hip", "%s: %s", fn_name, err.c_str());
-    return false;
-  }
-  // Kernel symbols name what the kernel is (class, and a hash of its source), so
-  // identical kernels share one module and a profiler can tell the others apart.
-  static const char *const tag[] = {"ew", "rowred", "thrred", "mm", "gather", "copy"};
+// Kernel symbols name what the kernel is (class, and a hash of its source), so
+// identical kernels share one module and a profiler can tell the others apart.
+static void name_kernel(RenderedKernel *rk) {
+  static const char *const tag[] = {"ew", "rowred", "thrred", "mm", "gather", "copy", "attn"};
   auto rename = [](std::string &src, const std::string &from, const std::string &to) {
     for (size_t pos = 0; (pos = src.find(from, pos)) != std::string::npos; pos += to.size()) src.replace(pos, from.size(), to);
   };
@@ -49,14 +42,33 @@ static bool render_root(const PolyUOp *root, const char *fn_name, int flags, Ren
     rename(rk->fallback_source, " poly_k(", " " + name + "_slow(");
     rk->fallback_entry = name + "_slow";
   }
+}
+
+static bool render_root(const PolyUOp *root, const char *fn_name, int flags, RenderedKernel *rk) {
+  KernelGraph g;
+  if (!g.build(root)) { log_err("render_hip", "%s: %s", fn_name, g.error.c_str()); return false; }
+  std::string err;
+  if (!render_kernel(g, "poly_k", options_from_flags(flags), rk, &err)) {
+    log_err("render_hip", "%s: %s", fn_name, err.c_str());
+    return false;
+  }
+  name_kernel(rk);
   return true;
 }
 
 HipRunner *runner_create(const PolyUOp *root, const char *fn_name, int flags) {
   if (runtime_init() != 0) return nullptr;
+  RenderedKernel rk;
+  if (!render_root(root, fn_name ? fn_name : "kernel", flags, &rk)) return nullptr;
+  return runner_from_rendered(rk, fn_name, true);
+}
+
+HipRunner *runner_from_rendered(const RenderedKernel &rk, const char *fn_name, bool named) {
+  if (runtime_init() != 0) return nullptr;
   HipRunner *r = new HipRunner();
   r->name = fn_name ? fn_name : "kernel";
-  if (!render_root(root, r->name.c_str(), flags, &r->rk)) { delete r; return nullptr; }
+  r->rk = rk;
+  if (!named) name_kernel(&r->rk);
   r->main = program_create(r->rk.source, r->rk.entry);
   if (!r->main) { runner_destroy(r); return nullptr; }
   if (!r->rk.guards.empty()) {

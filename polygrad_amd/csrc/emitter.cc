@@ -336,7 +336,11 @@ std::string Emitter::emit_raw(int id, Scope *s) {
     case POLY_OP_NEG: e = k.dt == DT_BOOL ? strf("(!%s)", S(0).c_str()) : strf("(-%s)", S(0).c_str()); break;
     case POLY_OP_SQRT: e = k.dt == DT_F64 ? strf("__builtin_sqrt(%s)", S(0).c_str()) : strf("__builtin_sqrtf(%s)", S(0).c_str()); break;
     case POLY_OP_TRUNC: e = k.dt == DT_F64 ? strf("__builtin_trunc(%s)", S(0).c_str()) : strf("__builtin_truncf(%s)", S(0).c_str()); break;
-    case POLY_OP_EXP2: e = k.dt == DT_F64 ? strf("__builtin_exp2(%s)", S(0).c_str()) : strf("__builtin_exp2f(%s)", S(0).c_str()); break;
+    case POLY_OP_EXP2:
+      if (k.dt == DT_F64) e = strf("__builtin_exp2(%s)", S(0).c_str());
+      else if (k.dt == DT_F32 && raw_exp2) e = strf("__builtin_amdgcn_exp2f(%s)", S(0).c_str());
+      else e = strf("__builtin_exp2f(%s)", S(0).c_str());
+      break;
     case POLY_OP_LOG2: e = k.dt == DT_F64 ? strf("__builtin_log2(%s)", S(0).c_str()) : strf("__builtin_log2f(%s)", S(0).c_str()); break;
     case POLY_OP_SIN: e = k.dt == DT_F64 ? strf("__builtin_sin(%s)", S(0).c_str()) : strf("__builtin_sinf(%s)", S(0).c_str()); break;
     case POLY_OP_RECIPROCAL: e = strf("(1/%s)", S(0).c_str()); break;

@@ -1,0 +1,572 @@
+// Plan-level fusion: kernel groups of a schedule that one launch can execute
+// without materialising their intermediates.
+//
+// The only group recognised so far is attention as a scheduler cuts it
+// (reference builder: src/modelzoo/models/gpt2.c:411-441):
+//     S   : scores[z,m,n] = f(sum_k Q[z,m,k] K[z,n,k])           (matmul, 16-bit operands)
+//     E*  : pointwise kernels on the score tensor (scale, mask)   (0..4 of them)
+//     MAX : mx[z,m]  = max_n  cast(x[z,m,n])
+//     SUM : sum[z,m] = sum_n  exp2((cast(x[z,m,n]) - mx[z,m]) * c)
+//     P   : p[z,m,n] = g(x[z,m,n], mx[z,m], sum[z,m])             (pointwise)
+//     PV  : out[z,m,d] = h(sum_n p[z,m,n] V[z,n,d])               (matmul)
+// The match is structural: which buffer feeds which kernel, that every consumer
+// reads the score tensor at the index the producer wrote (pointwise), that the
+// reductions run over the key axis, and that nothing outside the group reads the
+// intermediates.  f, the E kernels, g and h are not interpreted; their code is
+// generated from their own graphs into the hooks of kernels/attention_mfma.hip.
+#include "fusion.h"
+
+#include <algorithm>
+#include <cstdlib>
+#include <map>
+#include <set>
+
+namespace polyhip {
+
+namespace {
+
+const char *const kAttentionTemplate =
+#include "attention_mfma.hip.inc"
+    ;
+
+bool fa_reject(int line) {
+  if (getenv("POLY_HIP_DEBUG")) fprintf(stderr, "polygrad: fusion: attention group rejected at fusion.cc:%d\n", line);
+  return false;
+}
+#define FA_REJECT() return fa_reject(__LINE__)
+
+PolyOps reduce_op(const KNode &k) { return k.u->arg.kind == POLY_ARG_OPS ? k.u->arg.ops : (PolyOps)k.u->arg.i; }
+
+// An index expression in the coordinates of the group's first kernel ("master"
+// ranges): constant + sum of coef * master range.
+struct Aff {
+  std::map<int, int64_t> c;
+  int64_t c0 = 0;
+  bool operator==(const Aff &o) const { return c0 == o.c0 && c == o.c; }
+};
+typedef std::map<int, int> RangeMap;   // range ordinal of a kernel -> master ordinal
+
+bool lin_to_aff(const KernelGraph &g, const Lin &l, const RangeMap &rm, Aff *out) {
+  out->c.clear();
+  out->c0 = l.c0;
+  for (const Term &t : l.terms) {
+    const Atom &a = g.atoms[(size_t)t.atom];
+    if (a.kind != Atom::RANGE) return false;
+    auto it = rm.find(g.range_ord.at(a.node));
+    if (it == rm.end()) return false;
+    out->c[it->second] += t.coef;
+  }
+  for (auto it = out->c.begin(); it != out->c.end();) it = it->second == 0 ? out->c.erase(it) : std::next(it);
+  return true;
+}
+
+// A consumer reads the producer's buffer at `l` (in its own ranges); the producer
+// wrote it at `prod` (master coordinates).  When both are affine with pairwise
+// distinct coefficients, equal coefficients identify the consumer's ranges with
+// master ranges.  Extends *rm; false when the two cannot describe the same element.
+bool derive_map(const KernelGraph &g, const Lin &l, const Aff &prod, const std::vector<int64_t> &master_extent, RangeMap *rm) {
+  if (l.c0 != prod.c0 || l.terms.size() != prod.c.size()) return false;
+  std::set<int64_t> seen;
+  for (auto &kv : prod.c) if (!seen.insert(kv.second).second) return false;
+  for (const Term &t : l.terms) {
+    const Atom &a = g.atoms[(size_t)t.atom];
+    if (a.kind != Atom::RANGE) return false;
+    const int ord = g.range_ord.at(a.node);
+    int master = -1;
+    for (auto &kv : prod.c) if (kv.second == t.coef) master = kv.first;
+    if (master < 0) return false;
+    if (g.ranges[(size_t)ord].extent != master_extent[(size_t)master]) return false;
+    auto it = rm->find(ord);
+    if (it != rm->end() && it->second != master) return false;
+    for (auto &kv : *rm) if (kv.second == master && kv.first != ord) return false;
+    (*rm)[ord] = master;
+  }
+  return true;
+}
+
+struct LoadRef { int node, lin; };
+
+// every LOAD of buffer parameter `param` (position in g.params); false when one is gated
+bool loads_of(const KernelGraph &g, int param, std::vector<LoadRef> *out) {
+  for (int id = 0; id < (int)g.nodes.size(); id++) {
+    const KNode &k = g.n(id);
+    if (k.op != POLY_OP_LOAD) continue;
+    const KNode &ix = g.n(k.src[0]);
+    if (g.param_slot(ix.src[0]) != param) continue;
+    if (ix.src.size() != 2 || k.guard >= 0) return false;
+    const int lin = g.n(ix.src[1]).lin;
+    if (lin < 0) return false;
+    out->push_back({id, lin});
+  }
+  return true;
+}
+
+struct Sched {
+  const PolySchedule *s;
+  const std::vector<KernelGraph> &graphs;
+  std::vector<int> step_of;                  // item -> position in exec_order
+  std::vector<std::vector<int>> readers, writers;   // per slot: items
+  int slot(int item, int param) const { return s->items[item].buf_slot_indices[param]; }
+  int param_of(int item, int sl) const {
+    const PolyExecItem &it = s->items[item];
+    for (int i = 0; i < it.n_buf_slots; i++) if (it.buf_slot_indices[i] == sl) return i;
+    return -1;
+  }
+};
+
+// One kernel of the group with its ranges expressed in master coordinates.
+struct Member {
+  int item = -1;
+  RangeMap rm;
+  std::map<int, std::string> preset;   // node -> C expression replacing it
+};
+
+std::string params_decl(const KernelGraph &g) {
+  std::string d;
+  for (size_t i = 0; i < g.params.size(); i++) {
+    const ParamInfo &p = g.params[i];
+    if (i) d += ", ";
+    if (p.written) d += strf("%s* data%zu", dt_cname(p.dt), i);
+    else d += strf("const %s* __restrict__ data%zu", dt_cname(p.dt), i);
+  }
+  return d;
+}
+
+}  // namespace
+
+// Tries to grow an attention group from the matmul at schedule item `s_item`.
+static bool match_attention(const Sched &sc, int s_item, const std::vector<char> &taken, FusedGroup *out) {
+  const PolySchedule *s = sc.s;
+  const KernelGraph &gS = sc.graphs[(size_t)s_item];
+  MatmulMatch mS;
+  if (!match_matmul(gS, &mS, nullptr)) return false;   // not a matmul: not a candidate, no diagnostics
+  if (mS.K != 64 || mS.M % 128 != 0 || mS.N % 64 != 0 || mS.Z > (1 << 20)) FA_REJECT();
+  if (mS.ka.kb < mS.K || mS.kb.kb < mS.K || mS.ka.s_lo != 1 || mS.kb.s_lo != 1) FA_REJECT();   // features contiguous
+  if (mS.nd_full.size() != 1 || mS.nd_full[0].cut != 1) FA_REJECT();                         // keys: one plain range
+  const int n_master = mS.nd_full[0].ord;
+  const StoreInfo &stS = gS.stores[0];
+  const DT tin = mS.A.dt;
+  if (gS.n(stS.value).dt != tin) FA_REJECT();
+  std::vector<int64_t> mext(gS.ranges.size());
+  for (size_t i = 0; i < gS.ranges.size(); i++) mext[i] = gS.ranges[i].extent;
+  RangeMap idS;
+  for (int r : stS.ranges) idS[r] = r;
+  const int lsi = gS.n(gS.n(stS.index).src[1]).lin;
+  Aff aS;
+  if (lsi < 0 || !lin_to_aff(gS, gS.lins[(size_t)lsi], idS, &aS)) FA_REJECT();
+  if (aS.c.size() != stS.ranges.size()) FA_REJECT();   // the store covers a dense [z, m, n] box
+
+  std::vector<Member> members;      // S, E*, MAX, SUM, P, PV in this order
+  std::set<int> internal;           // slots that stay inside the fused kernel
+  { Member m; m.item = s_item; m.rm = idS; members.push_back(m); }
+  int cur = sc.slot(s_item, gS.param_slot(stS.param));
+  const int64_t big_numel = s->buf_slots[cur].numel;
+
+  auto only_group_reads = [&](int sl, std::set<int> expect) {
+    if (!s->buf_slots[sl].is_intermediate) return false;
+    std::set<int> r(sc.readers[(size_t)sl].begin(), sc.readers[(size_t)sl].end());
+    return r == expect && sc.writers[(size_t)sl].size() == 1;
+  };
+  // pointwise consumer of `cur`: maps its ranges, presets its loads of cur, checks its store
+  auto pointwise = [&](int item, Member *m, const char *value_name) {
+    const KernelGraph &g = sc.graphs[(size_t)item];
+    if (!g.reduces.empty() || g.stores.size() != 1 || g.stores[0].gate >= 0 || !g.vars.empty()) return false;
+    std::vector<LoadRef> lds;
+    const int p = sc.param_of(item, cur);
+    if (p < 0 || !loads_of(g, p, &lds) || lds.empty()) return false;
+    m->item = item;
+    for (const LoadRef &l : lds) {
+      if (!derive_map(g, g.lins[(size_t)l.lin], aS, mext, &m->rm)) return false;
+      m->preset[l.node] = value_name;
+    }
+    for (int r : g.stores[0].ranges) if (!m->rm.count(r)) return false;
+    const int li = g.n(g.n(g.stores[0].index).src[1]).lin;
+    Aff a;
+    if (li < 0 || !lin_to_aff(g, g.lins[(size_t)li], m->rm, &a) || !(a == aS)) return false;
+    const int outp = g.param_slot(g.stores[0].param);
+    if (s->buf_slots[sc.slot(item, outp)].numel != big_numel) return false;
+    return true;
+  };
+
+  // ── the pointwise chain ────────────────────────────────────────────────
+  std::vector<int> tail;
+  for (int depth = 0;; depth++) {
+    std::vector<int> rd = sc.readers[(size_t)cur];
+    if (!s->buf_slots[cur].is_intermediate || sc.writers[(size_t)cur].size() != 1) FA_REJECT();
+    if (rd.size() == 3) { tail = rd; break; }
+    if (rd.size() != 1 || depth >= 4) FA_REJECT();
+    Member m;
+    if (taken[(size_t)rd[0]] || !pointwise(rd[0], &m, "x")) FA_REJECT();
+    const KernelGraph &g = sc.graphs[(size_t)rd[0]];
+    if (g.n(g.stores[0].value).dt != tin) FA_REJECT();
+    internal.insert(cur);
+    members.push_back(m);
+    cur = sc.slot(rd[0], g.param_slot(g.stores[0].param));
+  }
+  const size_t n_chain = members.size() - 1;
+  internal.insert(cur);
+
+  // ── MAX, SUM, P ────────────────────────────────────────────────────────
+  int i_max = -1, i_sum = -1, i_p = -1;
+  for (int it : tail) {
+    if (taken[(size_t)it]) FA_REJECT();
+    const KernelGraph &g = sc.graphs[(size_t)it];
+    if (g.reduces.empty()) { if (i_p >= 0) FA_REJECT(); i_p = it; continue; }
+    if (g.reduces.size() != 1) FA_REJECT();
+    const PolyOps op = reduce_op(g.n(g.reduces[0]));
+    if (op == POLY_OP_MAX) { if (i_max >= 0) FA_REJECT(); i_max = it; }
+    else if (op == POLY_OP_ADD) { if (i_sum >= 0) FA_REJECT(); i_sum = it; }
+    else FA_REJECT();
+  }
+  if (i_max < 0 || i_sum < 0 || i_p < 0) FA_REJECT();
+
+  // a row reduction over the key axis whose body reads `cur` at the producer's index
+  auto row_reduce = [&](int item, Member *m, int *body, Aff *store_aff) {
+    const KernelGraph &g = sc.graphs[(size_t)item];
+    if (g.stores.size() != 1 || g.stores[0].gate >= 0 || !g.vars.empty()) return false;
+    const int red = g.reduces[0];
+    const KNode &R = g.n(red);
+    if (R.src.size() != 2 || R.dt != DT_F32 || g.stores[0].value != red) return false;
+    std::vector<LoadRef> lds;
+    const int p = sc.param_of(item, cur);
+    if (p < 0 || !loads_of(g, p, &lds) || lds.size() != 1) return false;
+    m->item = item;
+    if (!derive_map(g, g.lins[(size_t)lds[0].lin], aS, mext, &m->rm)) return false;
+    m->preset[lds[0].node] = "x";
+    const int kr = g.range_ord.at(R.src[1]);
+    if (!m->rm.count(kr) || m->rm[kr] != n_master) return false;
+    for (int r : g.stores[0].ranges) if (!m->rm.count(r)) return false;
+    const int li = g.n(g.n(g.stores[0].index).src[1]).lin;
+    if (li < 0 || !lin_to_aff(g, g.lins[(size_t)li], m->rm, store_aff)) return false;
+    if (store_aff->c.count(n_master)) return false;
+    *body = R.src[0];
+    return true;
+  };
+  auto strip_cast = [](const KernelGraph &g, int node) {
+    const KNode &k = g.n(node);
+    return (k.op == POLY_OP_CAST && k.dt == DT_F32) ? k.src[0] : node;
+  };
+
+  Member mMax, mSum, mP;
+  int body_max = -1, body_sum = -1;
+  Aff aMax, aSum;
+  if (!row_reduce(i_max, &mMax, &body_max, &aMax)) FA_REJECT();
+  {
+    // the maximum is taken over the stored values themselves, so it is one of them
+    const KernelGraph &g = sc.graphs[(size_t)i_max];
+    if (!mMax.preset.count(strip_cast(g, body_max))) FA_REJECT();
+  }
+  const int sl_max = sc.slot(i_max, sc.graphs[(size_t)i_max].param_slot(sc.graphs[(size_t)i_max].stores[0].param));
+  if (!row_reduce(i_sum, &mSum, &body_sum, &aSum)) FA_REJECT();
+  const int sl_sum = sc.slot(i_sum, sc.graphs[(size_t)i_sum].param_slot(sc.graphs[(size_t)i_sum].stores[0].param));
+  // term = exp2((cast(x) - mx) * c), c > 0: this is what makes term(a, m2) = term(a, m1) * term(m1, m2)
+  // and term monotone in x.  Returns the SUB node's operands and c.
+  auto match_term = [&](const KernelGraph &g, int node, int *x_node, int *mx_node, double *c_out) {
+    const KNode &e = g.n(node);
+    if (e.op != POLY_OP_EXP2 || e.dt != DT_F32) return false;
+    const KNode &mul = g.n(e.src[0]);
+    if (mul.op != POLY_OP_MUL) return false;
+    int sub = -1;
+    for (int side = 0; side < 2; side++) {
+      const KNode &c = g.n(mul.src[(size_t)side]);
+      if (c.op == POLY_OP_CONST && c.u->arg.kind == POLY_ARG_FLOAT && c.u->arg.f > 0) { sub = mul.src[(size_t)(1 - side)]; *c_out = c.u->arg.f; }
+    }
+    if (sub < 0 || g.n(sub).op != POLY_OP_SUB) return false;
+    *x_node = strip_cast(g, g.n(sub).src[0]);
+    *mx_node = g.n(sub).src[1];
+    return true;
+  };
+  double c_sum = 0;
+  {
+    const KernelGraph &g = sc.graphs[(size_t)i_sum];
+    int xn, mn;
+    if (!match_term(g, body_sum, &xn, &mn, &c_sum) || !mSum.preset.count(xn)) FA_REJECT();
+    std::vector<LoadRef> lm;
+    const int pm = sc.param_of(i_sum, sl_max);
+    if (pm < 0 || !loads_of(g, pm, &lm) || lm.size() != 1 || lm[0].node != mn) FA_REJECT();
+    Aff a;
+    if (!lin_to_aff(g, g.lins[(size_t)lm[0].lin], mSum.rm, &a) || !(a == aMax)) FA_REJECT();
+    mSum.preset[lm[0].node] = "mx";
+  }
+  if (!pointwise(i_p, &mP, "x")) FA_REJECT();
+  {
+    const KernelGraph &g = sc.graphs[(size_t)i_p];
+    if (g.n(g.stores[0].value).dt != tin) FA_REJECT();
+    for (int which = 0; which < 2; which++) {
+      std::vector<LoadRef> l;
+      const int p = sc.param_of(i_p, which == 0 ? sl_max : sl_sum);
+      if (p < 0 || !loads_of(g, p, &l) || l.empty()) FA_REJECT();
+      for (const LoadRef &r : l) {
+        Aff a;
+        if (!lin_to_aff(g, g.lins[(size_t)r.lin], mP.rm, &a) || !(a == (which == 0 ? aMax : aSum))) FA_REJECT();
+        mP.preset[r.node] = which == 0 ? "mx" : "sum";
+      }
+    }
+  }
+  // When p = cast(term(x, mx) / sum) with the very term of the sum kernel, a key block whose
+  // terms are all exactly zero has probabilities that are all exactly zero (for a finite,
+  // non-zero sum), and pass 2 may skip it.
+  bool p_is_term_over_sum = false;
+  {
+    const KernelGraph &g = sc.graphs[(size_t)i_p];
+    int v = g.stores[0].value;
+    if (g.n(v).op == POLY_OP_CAST) v = g.n(v).src[0];
+    const KNode &q = g.n(v);
+    int num = -1, den = -1;
+    if (q.op == POLY_OP_FDIV) { num = q.src[0]; den = q.src[1]; }
+    else if (q.op == POLY_OP_MUL) {
+      for (int side = 0; side < 2; side++) {
+        const KNode &r = g.n(q.src[(size_t)side]);
+        if (r.op == POLY_OP_RECIPROCAL) { den = r.src[0]; num = q.src[(size_t)(1 - side)]; }
+      }
+    }
+    int xn, mn;
+    double c_p = 0;
+    if (num >= 0 && q.dt == DT_F32 && match_term(g, num, &xn, &mn, &c_p) && c_p == c_sum && mP.preset.count(xn) &&
+        mP.preset.count(mn) && mP.preset[mn] == "mx" && mP.preset.count(den) && mP.preset[den] == "sum" && mP.preset[xn] == "x")
+      p_is_term_over_sum = true;
+  }
+  const int sl_p = sc.slot(i_p, sc.graphs[(size_t)i_p].param_slot(sc.graphs[(size_t)i_p].stores[0].param));
+  if (!only_group_reads(cur, {i_max, i_sum, i_p}) || !only_group_reads(sl_max, {i_sum, i_p}) || !only_group_reads(sl_sum, {i_p})) FA_REJECT();
+  if (sc.readers[(size_t)sl_p].size() != 1 || !s->buf_slots[sl_p].is_intermediate || sc.writers[(size_t)sl_p].size() != 1) FA_REJECT();
+  internal.insert(sl_max); internal.insert(sl_sum); internal.insert(sl_p);
+
+  // ── PV ─────────────────────────────────────────────────────────────────
+  const int i_pv = sc.readers[(size_t)sl_p][0];
+  if (taken[(size_t)i_pv]) FA_REJECT();
+  const KernelGraph &gP = sc.graphs[(size_t)i_pv];
+  MatmulMatch mV;
+  if (!match_matmul(gP, &mV, nullptr)) FA_REJECT();
+  if (mV.A.dt != tin || sc.slot(i_pv, mV.A.param) != sl_p || sc.slot(i_pv, mV.B.param) == sl_p) FA_REJECT();
+  if (mV.M != mS.M || mV.Z != mS.Z || mV.K != mS.N || mV.N != 64) FA_REJECT();
+  if (mV.ka.kb < mV.K || mV.kb.kb < mV.K) FA_REJECT();
+  if (mV.nd.size() != 1 || mV.nd[0].cb != 1) FA_REJECT();      // V features contiguous
+  if (mV.nd_full.size() != 1 || mV.nd_full[0].cut != 1) FA_REJECT();   // features: one plain range
+  const int d_ord = mV.nd_full[0].ord;
+  // P is read where it was written: the A operand index identifies PV's ranges (z, m and
+  // its reduce range) with master ranges; PV's own numbering of z is never used
+  Member mPV;
+  mPV.item = i_pv;
+  if (!derive_map(gP, gP.lins[(size_t)mV.A.lin], aS, mext, &mPV.rm)) FA_REJECT();
+  if (!mPV.rm.count(mV.kr) || mPV.rm[mV.kr] != n_master) FA_REJECT();
+  Aff aV;   // index of V in master coordinates, without the feature term
+  {
+    RangeMap with_d = mPV.rm;
+    with_d[d_ord] = -1;   // placeholder coordinate for the feature range
+    if (!lin_to_aff(gP, gP.lins[(size_t)mV.B.lin], with_d, &aV)) FA_REJECT();
+    if (!aV.c.count(-1) || aV.c[-1] != 1) FA_REJECT();
+    aV.c.erase(-1);
+    for (const MmDim &d : mS.md_full) if (aV.c.count(d.ord)) FA_REJECT();   // V does not depend on the query
+  }
+  const StoreInfo &stP = gP.stores[0];
+  const int out_slot = sc.slot(i_pv, gP.param_slot(stP.param));
+
+  // ── schedule constraints: the group runs where PV ran ───────────────────
+  std::vector<Member> all = members;
+  all.push_back(mMax); all.push_back(mSum); all.push_back(mP);
+  all.push_back(mPV);
+  std::set<int> group_items;
+  for (const Member &m : all) group_items.insert(m.item);
+  if (group_items.size() != all.size()) FA_REJECT();
+  const int first_step = sc.step_of[(size_t)s_item], last_step = sc.step_of[(size_t)i_pv];
+  for (int it : group_items) if (sc.step_of[(size_t)it] < first_step || sc.step_of[(size_t)it] > last_step) FA_REJECT();
+    std::set<int> inputs;
+  std::map<int, int> first_read;   // input slot -> earliest original step of a member reading it
+  for (int it : group_items) {
+    const PolyExecItem &e = s->items[it];
+    for (int i = 0; i < e.n_buf_slots; i++) {
+      const int sl = e.buf_slot_indices[i];
+      if (internal.count(sl) || sl == out_slot) continue;
+      if (sc.graphs[(size_t)it].params[(size_t)i].written) FA_REJECT();
+      inputs.insert(sl);
+      const int st = sc.step_of[(size_t)it];
+      if (!first_read.count(sl) || st < first_read[sl]) first_read[sl] = st;
+    }
+  }
+  // a member that read an input at its own step now reads it at the group's step: the
+  // input must not change in between
+  for (int sl : inputs)
+    for (int w : sc.writers[(size_t)sl])
+      if (sc.step_of[(size_t)w] >= first_read[sl] && sc.step_of[(size_t)w] <= last_step) FA_REJECT();
+  for (int w : sc.writers[(size_t)out_slot]) if (w != i_pv && sc.step_of[(size_t)w] >= first_step && sc.step_of[(size_t)w] <= last_step) FA_REJECT();
+  for (int r : sc.readers[(size_t)out_slot]) if (sc.step_of[(size_t)r] >= first_step && sc.step_of[(size_t)r] <= last_step && r != i_pv) FA_REJECT();
+  if (internal.count(out_slot) || inputs.count(out_slot)) FA_REJECT();
+
+  // every load of an internal buffer must have been replaced by a value
+  for (const Member &m : all) {
+    const KernelGraph &g = sc.graphs[(size_t)m.item];
+    for (int id = 0; id < (int)g.nodes.size(); id++) {
+      if (g.n(id).op != POLY_OP_LOAD) continue;
+      const int p = g.param_slot(g.n(g.n(id).src[0]).src[0]);
+      if (!internal.count(sc.slot(m.item, p))) continue;
+      const bool is_pv_a = m.item == i_pv && id == mV.A.load;
+      if (!m.preset.count(id) && !is_pv_a) FA_REJECT();
+    }
+  }
+
+  // ── code generation ────────────────────────────────────────────────────
+  std::vector<int> arg_slots;
+  arg_slots.push_back(out_slot);
+  for (int sl : inputs) arg_slots.push_back(sl);
+  auto arg_of = [&](int sl) { return (int)(std::find(arg_slots.begin(), arg_slots.end(), sl) - arg_slots.begin()); };
+  auto call_args = [&](int item) {
+    const KernelGraph &g = sc.graphs[(size_t)item];
+    std::string c;
+    for (size_t i = 0; i < g.params.size(); i++) {
+      const int sl = sc.slot(item, (int)i);
+      if (i) c += ", ";
+      if (internal.count(sl)) c += strf("(%s%s*)0", g.params[i].written ? "" : "const ", dt_cname(g.params[i].dt));
+      else c += strf("fa%d", arg_of(sl));
+    }
+    return c;
+  };
+  std::string sig;
+  for (size_t j = 0; j < arg_slots.size(); j++) {
+    DT dt = DT_VOID;
+    for (int it : group_items) {
+      const int p = sc.param_of(it, arg_slots[j]);
+      if (p >= 0) dt = sc.graphs[(size_t)it].params[(size_t)p].dt;
+    }
+    if (j) sig += ", ";
+    sig += j == 0 ? strf("%s* fa%zu", dt_cname(dt), j) : strf("const %s* __restrict__ fa%zu", dt_cname(dt), j);
+  }
+
+  const std::string master_decomp = matmul_decompose(mS, nullptr);
+  const char *tn = dt_cname(tin);
+  std::string cfg;
+  bool failed = false;
+  // one device function per kernel of the group: value of `node` with the member's presets
+  // The softmax terms use the bare exp2 instruction: a term below 2^-126 of the row's
+  // largest (which is exactly 1, so the sum is at least 1) cannot change the fp32 sum, and
+  // the probability it would give is below the smallest normal 16-bit float.
+  auto value_fn = [&](const Member &m, const char *name, const char *ret, const char *lead_args, int node,
+                      const std::map<int, std::string> &extra_preset) {
+    const KernelGraph &g = sc.graphs[(size_t)m.item];
+    Emitter em(g);
+    em.raw_exp2 = (m.item == i_sum || m.item == i_p);
+    Scope S0;
+    S0.indent = 1;
+    for (auto &kv : m.rm) { em.bind_range(kv.first, strf("r%d", kv.second)); S0.avail |= (uint64_t)1 << kv.first; }
+    for (auto &kv : m.preset) em.preset(kv.first, kv.second);
+    for (auto &kv : extra_preset) em.preset(kv.first, kv.second);
+    std::string v = em.emit(node, &S0);
+    if (em.failed() || em.uses_threefry) failed = true;
+    cfg += strf("__device__ __forceinline__ %s %s(%s, int m, int n, int z, %s) {\n", ret, name, lead_args, params_decl(g).c_str());
+    cfg += master_decomp + S0.code;
+    cfg += strf("  return %s;\n}\n", v.c_str());
+  };
+  cfg += strf("#define POLY_TIN %s\n", tn);
+  cfg += strf("#define POLY_MFMA(a, b, c) __builtin_amdgcn_mfma_f32_32x32x16_%s(a, b, c, 0, 0, 0)\n", tin == DT_BF16 ? "bf16" : "f16");
+  cfg += strf("#define POLY_FA_M %lld\n#define POLY_FA_N %lld\n#define POLY_FA_Z %lld\n", (long long)mS.M, (long long)mS.N, (long long)mS.Z);
+  cfg += strf("#define POLY_Q_PTR fa%d\n#define POLY_K_PTR fa%d\n#define POLY_V_PTR fa%d\n", arg_of(sc.slot(s_item, mS.A.param)),
+              arg_of(sc.slot(s_item, mS.B.param)), arg_of(sc.slot(i_pv, mV.B.param)));
+  cfg += matmul_offset_fn("poly_fa_qz", mS.zd, true, mS.a_c0) + matmul_offset_fn("poly_fa_qm", mS.md, true, 0);
+  cfg += matmul_offset_fn("poly_fa_kz", mS.zd, false, mS.b_c0) + matmul_offset_fn("poly_fa_kn", mS.nd, false, 0);
+  cfg += "__device__ __forceinline__ int poly_q_off(int z, int m) { return poly_fa_qz(z) + poly_fa_qm(m); }\n";
+  cfg += "__device__ __forceinline__ int poly_k_off(int z, int n) { return poly_fa_kz(z) + poly_fa_kn(n); }\n";
+  {
+    std::string e = strf("%lld", (long long)aV.c0);
+    for (auto &kv : aV.c) e += strf(" + %lld * r%d", (long long)kv.second, kv.first);
+    cfg += "__device__ __forceinline__ int poly_v_off(int z, int n) {\n  const int m = 0;\n" + master_decomp + "  return " + e + ";\n}\n";
+  }
+  cfg += strf("#define POLY_SIGNATURE %s\n", sig.c_str());
+  cfg += strf("#define POLY_FA_SKIP_DEAD_BLOCKS %d\n", p_is_term_over_sum ? 1 : 0);
+
+  // score: epilogue of S, then the pointwise chain
+  {
+    const Member &m = all[0];
+    value_fn(m, "poly_fa_s", tn, "float acc", stS.value, {{mS.red, "acc"}});
+  }
+  std::string score = strf("poly_fa_s(acc, m, n, z, %s)", call_args(s_item).c_str());
+  for (size_t e = 1; e <= n_chain; e++) {
+    const Member &m = all[e];
+    const KernelGraph &g = sc.graphs[(size_t)m.item];
+    const std::string fn = strf("poly_fa_e%zu", e);
+    value_fn(m, fn.c_str(), tn, strf("%s x", tn).c_str(), g.stores[0].value, {});
+    score = strf("%s(%s, m, n, z, %s)", fn.c_str(), score.c_str(), call_args(m.item).c_str());
+  }
+  cfg += strf("#define POLY_FA_SCORE(acc, m, n, z) %s\n", score.c_str());
+  value_fn(mMax, "poly_fa_maxv", "float", strf("%s x", tn).c_str(), body_max, {});
+  cfg += strf("#define POLY_FA_MAXV(x, m, n, z) poly_fa_maxv(x, m, n, z, %s)\n", call_args(i_max).c_str());
+  value_fn(mSum, "poly_fa_term", "float", strf("%s x, float mx", tn).c_str(), body_sum, {});
+  cfg += strf("#define POLY_FA_TERM(x, mx, m, n, z) poly_fa_term(x, mx, m, n, z, %s)\n", call_args(i_sum).c_str());
+  value_fn(mP, "poly_fa_p", tn, strf("%s x, float mx, float sum", tn).c_str(), sc.graphs[(size_t)i_p].stores[0].value, {});
+  cfg += strf("#define POLY_FA_P(x, mx, sum, m, n, z) poly_fa_p(x, mx, sum, m, n, z, %s)\n", call_args(i_p).c_str());
+  {
+    // output: epilogue of PV; its z and m ranges in master coordinates, its feature range = d
+    Emitter em(gP);
+    Scope S0;
+    S0.indent = 1;
+    for (int r : stP.ranges) {
+      S0.avail |= (uint64_t)1 << r;
+      if (r == d_ord) em.bind_range(r, "d");
+      else if (mPV.rm.count(r)) em.bind_range(r, strf("r%d", mPV.rm[r]));
+      else failed = true;
+    }
+    std::string decomp = "  const int n = 0;\n" + master_decomp;
+    em.preset(mV.red, "acc");
+    std::string val = em.emit(stP.value, &S0);
+    std::string idx = em.emit(gP.n(stP.index).src[1], &S0);
+    if (em.failed() || em.uses_threefry) failed = true;
+    cfg += strf("__device__ __forceinline__ void poly_fa_out(float acc, int m, int d, int z, %s) {\n", params_decl(gP).c_str());
+    cfg += decomp + S0.code;
+    cfg += strf("  data%d[%s] = %s;\n}\n", gP.param_slot(stP.param), idx.c_str(), val.c_str());
+    cfg += strf("#define POLY_FA_OUT(acc, m, d, z) poly_fa_out(acc, m, d, z, %s)\n", call_args(i_pv).c_str());
+  }
+  if (failed) FA_REJECT();
+
+  out->items.clear();
+  for (const Member &m : all) out->items.push_back(m.item);
+  out->launch_item = i_pv;
+  out->internal_slots.assign(internal.begin(), internal.end());
+  out->arg_slots = arg_slots;
+  RenderedKernel &rk = out->rk;
+  rk = RenderedKernel();
+  rk.source = std::string(hip_prelude()) + cfg + kAttentionTemplate;
+  rk.entry = "poly_k";
+  rk.launch.grid[0] = (unsigned)((mS.M / 128) * mS.Z);
+  rk.launch.block[0] = 256;
+  rk.klass = KernelClass::ATTENTION;
+  rk.strategy = strf("fused attention (%zu kernels): mfma 32x32x16 %s Z=%lld M=%lld N=%lld D=64, two passes over keys", all.size(),
+                     tin == DT_BF16 ? "bf16" : "f16", (long long)mS.Z, (long long)mS.M, (long long)mS.N);
+  rk.n_params = (int)arg_slots.size();
+  rk.n_vars = 0;
+  rk.flops = 2.0 * (double)mS.Z * (double)mS.M * (double)mS.N * (double)(mS.K + mV.N);
+  double bytes = 0;
+  for (int sl : arg_slots) bytes += (double)s->buf_slots[sl].nbytes;
+  rk.bytes = bytes;
+  return true;
+}
+
+void find_fused_groups(const PolySchedule *s, const std::vector<KernelGraph> &graphs, std::vector<FusedGroup> *out) {
+  out->clear();
+  if (getenv("POLY_HIP_NO_FUSION")) return;
+  Sched sc{s, graphs, {}, {}, {}};
+  sc.step_of.assign((size_t)s->n_items, 0);
+  for (int st = 0; st < s->n_items; st++) sc.step_of[(size_t)s->exec_order[st]] = st;
+  sc.readers.assign((size_t)s->n_buf_slots, {});
+  sc.writers.assign((size_t)s->n_buf_slots, {});
+  for (int k = 0; k < s->n_items; k++) {
+    const PolyExecItem &it = s->items[k];
+    const KernelGraph &g = graphs[(size_t)k];
+    if ((int)g.params.size() != it.n_buf_slots) return;
+    for (int i = 0; i < it.n_buf_slots; i++) {
+      const int sl = it.buf_slot_indices[i];
+      if (sl < 0 || sl >= s->n_buf_slots) return;
+      if (g.params[(size_t)i].read) sc.readers[(size_t)sl].push_back(k);
+      if (g.params[(size_t)i].written) sc.writers[(size_t)sl].push_back(k);
+    }
+  }
+  for (auto &v : sc.readers) { std::sort(v.begin(), v.end()); v.erase(std::unique(v.begin(), v.end()), v.end()); }
+  std::vector<char> taken((size_t)s->n_items, 0);
+  for (int st = 0; st < s->n_items; st++) {
+    const int k = s->exec_order[st];
+    if (taken[(size_t)k] || graphs[(size_t)k].reduces.size() != 1) continue;
+    FusedGroup fg;
+    if (!match_attention(sc, k, taken, &fg)) continue;
+    for (int it : fg.items) taken[(size_t)it] = 1;
+    out->push_back(std::move(fg));
+  }
+}
+
+}  // namespace polyhip

@@ -1,0 +1,23 @@
+// Plan-level fusion of kernel groups (see fusion.cc).
+#pragma once
+#include <vector>
+
+#include "polygrad_abi.h"
+#include "templates.h"
+
+namespace polyhip {
+
+// A set of schedule items replaced by one launch.
+struct FusedGroup {
+  std::vector<int> items;           // schedule items the fused kernel stands for
+  int launch_item = -1;             // the fused kernel runs at this item's place in exec_order
+  std::vector<int> internal_slots;  // buffers that are never materialised
+  std::vector<int> arg_slots;       // slot of each kernel argument, in order
+  RenderedKernel rk;
+};
+
+// Finds the fusable groups of a schedule.  graphs[k] is the analysed kernel of item k.
+// Setting POLY_HIP_NO_FUSION in the environment disables the search.
+void find_fused_groups(const PolySchedule *s, const std::vector<KernelGraph> &graphs, std::vector<FusedGroup> *out);
+
+}  // namespace polyhip

@@ -1,0 +1,322 @@
+// Fused attention for gfx950: the kernel group
+//     S = Q K^T  ->  pointwise chain (scale, mask, ...)  ->  row max  ->  row sum of
+//     exp-terms  ->  normalise  ->  O = P V
+// that a scheduler emits as six or more kernels, executed as one launch that never
+// writes the [Z, M, N] score tensor to memory.  Only the STRUCTURE is fixed here; all
+// arithmetic on scores (epilogue of the first matmul, the pointwise chain, the term
+// that is summed, the normalisation, the epilogue of the second matmul) is generated
+// from the kernels' own graphs and arrives through the POLY_FA_* hooks, rounding steps
+// included, so every probability is computed by the same expression as in the unfused
+// kernels.
+//
+// Two passes over the keys.  Pass 1 computes each row's maximum and the sum of its terms
+// (running maximum with rescaling; the hooks guarantee term(x, m) = exp2((x - m) * c),
+// which makes the rescaling factor term(m_old, m_new)).  Pass 2 recomputes the scores
+// (bit-identical: same MFMA sequence), turns them into probabilities with the final
+// maximum and sum, and accumulates P V.
+//
+// Orientation: a wave owns 32 queries.  Scores are computed transposed,
+// S^T[key][query] = K Q^T, so a lane holds ONE query (lane % 32) and 16 keys per 32x32
+// tile in its accumulator registers: row statistics are in-register reductions plus one
+// exchange between lane l and l ^ 32, and the probabilities are already laid out as the
+// A operand of the second MFMA (8 keys per lane per 16-key step, in the key order
+// 8*(i/4) + 4*(lane/32) + i%4 that the V fragment reads mirror).
+//
+// Configuration (defined by the host before this text):
+//   POLY_TIN, POLY_MFMA(a, b, c)       16-bit input type and its 32x32x16 MFMA
+//   POLY_FA_M, POLY_FA_N, POLY_FA_Z    queries, keys, batch*heads; M % 128 == 0, N % 64 == 0
+//   POLY_Q_PTR, POLY_K_PTR, POLY_V_PTR operand pointers (names from POLY_SIGNATURE)
+//   poly_q_off(z, m), poly_k_off(z, n), poly_v_off(z, n)
+//                                      element offset of the 64 contiguous head features
+//   POLY_FA_SCORE(acc, m, n, z)        -> POLY_TIN  score as the last pointwise kernel stores it
+//   POLY_FA_MAXV(x, m, n, z)           -> float     what the max reduction compares
+//   POLY_FA_TERM(x, mx, m, n, z)       -> float     what the sum reduction adds
+//   POLY_FA_P(x, mx, sum, m, n, z)     -> POLY_TIN  the probability as stored
+//   POLY_FA_OUT(acc, m, d, z)          stores one output element
+//   POLY_FA_SKIP_DEAD_BLOCKS           1 when p = cast(term(x, mx) / sum): then a key block whose
+//                                      terms are all exactly 0 has probabilities exactly 0
+//   POLY_SIGNATURE
+//
+// Dead key blocks (every term of the block exactly zero for all 32 queries of a wave, as
+// under a causal mask) are detected from the values themselves, never assumed: term is
+// monotone in x, so term(block maximum, row maximum) == 0 bounds the whole block.  Pass 1
+// then skips the exponentials of that block (they would add exact zeros) and pass 2 skips
+// its scores and probabilities, multiplying V by exact zeros instead so that a non-finite
+// V still propagates as it does in the unfused kernels.  Blocks with a NaN score are
+// never treated as dead.
+#ifdef POLY_TEMPLATE_STANDALONE
+#include <hip/hip_runtime.h>
+#define POLY_TIN __bf16
+#define POLY_MFMA(a, b, c) __builtin_amdgcn_mfma_f32_32x32x16_bf16(a, b, c, 0, 0, 0)
+#define POLY_FA_M 1024
+#define POLY_FA_N 1024
+#define POLY_FA_Z 96
+#define POLY_Q_PTR data1
+#define POLY_K_PTR data2
+#define POLY_V_PTR data3
+__device__ __forceinline__ int poly_q_off(int z, int m) { return (z / 12) * 786432 + (z % 12) * 64 + m * 768; }
+__device__ __forceinline__ int poly_k_off(int z, int n) { return (z / 12) * 786432 + (z % 12) * 64 + n * 768; }
+__device__ __forceinline__ int poly_v_off(int z, int n) { return (z / 12) * 786432 + (z % 12) * 64 + n * 768; }
+#define POLY_SIGNATURE __bf16 *data0, const __bf16 *__restrict__ data1, const __bf16 *__restrict__ data2, const __bf16 *__restrict__ data3, const __bf16 *__restrict__ data4
+#define POLY_FA_SCORE(acc, m, n, z) ((__bf16)((float)(__bf16)((float)(__bf16)(acc) * 0.125f) + (float)data4[(m) * 1024 + (n)]))
+#define POLY_FA_MAXV(x, m, n, z) ((float)(x))
+#define POLY_FA_TERM(x, mx, m, n, z) __builtin_amdgcn_exp2f(((float)(x) - (mx)) * 0x1.715476p+0f)
+#define POLY_FA_P(x, mx, sum, m, n, z) ((__bf16)(__builtin_amdgcn_exp2f(((float)(x) - (mx)) * 0x1.715476p+0f) / (sum)))
+#define POLY_FA_OUT(acc, m, d, z) data0[((z) / 12) * 786432 + ((z) % 12) * 65536 + (m) * 64 + (d)] = (__bf16)(acc)
+#define POLY_FA_SKIP_DEAD_BLOCKS 1
+#endif
+
+typedef POLY_TIN fa_in8 __attribute__((ext_vector_type(8)));
+typedef float fa_acc16 __attribute__((ext_vector_type(16)));
+typedef unsigned int fa_u32x4 __attribute__((ext_vector_type(4)));
+typedef unsigned int fa_u32x2 __attribute__((ext_vector_type(2)));
+typedef fa_u32x4 fa_u32x4_u __attribute__((aligned(2)));
+
+#define FA_BM 128        // queries per workgroup: 4 waves x 32
+#define FA_BN 64         // keys per step
+#define FA_D 64          // head features
+#define FA_THREADS 256
+#define FA_NKB (POLY_FA_N / FA_BN)
+
+// LDS tiles are [row][64] 16-bit values; the eight 16-byte columns of a row are
+// XOR-swizzled by the row number so fragment reads and staging writes spread over banks.
+__device__ __forceinline__ int fa_swz(int row) { return (row ^ (row >> 3)) & 7; }
+
+__device__ __forceinline__ float fa_other_half(float v) {
+  // value held by lane ^ 32
+  const int lane = (int)(threadIdx.x & 63);
+  return __builtin_bit_cast(float, __builtin_amdgcn_ds_bpermute(((lane ^ 32) << 2), __builtin_bit_cast(int, v)));
+}
+
+// Three workgroups per CU (three waves per SIMD): the arithmetic on the scores is VALU work,
+// and it is the other resident waves that hide its latencies.
+extern "C" __global__ void __launch_bounds__(FA_THREADS) __attribute__((amdgpu_waves_per_eu(3, 3))) poly_k(POLY_SIGNATURE) {
+  __shared__ __attribute__((aligned(16))) POLY_TIN lds_k[2][FA_BN * FA_D];   // [key][feature]
+  __shared__ __attribute__((aligned(16))) POLY_TIN lds_v[2][FA_D * FA_BN];   // [feature][key]
+  __shared__ __attribute__((aligned(16))) POLY_TIN lds_q[FA_BM * FA_D];      // [query][feature]
+
+  // Workgroup -> (z, block of queries).  Consecutive ids go to different XCDs (id % 8), each
+  // with its own L2: an XCD keeps a fixed set of z, so the query blocks that share K and V
+  // meet in one L2.  Under a causal mask late query blocks have more live key tiles than
+  // early ones, so within an XCD the late blocks are handed out first.
+  constexpr int MB = POLY_FA_M / FA_BM;
+  int z, mb;
+  if (POLY_FA_Z % 8 == 0) {
+    constexpr int ZX = POLY_FA_Z / 8 > 0 ? POLY_FA_Z / 8 : 1;   // z per XCD
+    const int xcd = blockIdx.x & 7, j = blockIdx.x >> 3;
+    mb = MB - 1 - j / ZX;
+    z = xcd * ZX + j % ZX;
+  } else {
+    mb = MB - 1 - (int)blockIdx.x / POLY_FA_Z;
+    z = (int)blockIdx.x % POLY_FA_Z;
+  }
+  const int m0 = mb * FA_BM;
+  const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63, lq = lane & 31, half = lane >> 5;
+  const int mq = m0 + wave * 32 + lq;   // the query this lane owns in the score tiles
+
+  // Q block of the workgroup -> LDS once (128 queries x 8 chunks of 16 bytes, four per
+  // thread); it is the B operand of S^T = K Q^T: a lane reads Q[mq][16 s + 8 half .. + 7]
+#pragma unroll
+  for (int i = 0; i < 4; i++) {
+    const int c = threadIdx.x + i * FA_THREADS;
+    const int q = c >> 3, col = c & 7;
+    const fa_u32x4 v = *(const fa_u32x4_u *)(POLY_Q_PTR + poly_q_off(z, m0 + q) + col * 8);
+    *(fa_u32x4 *)(lds_q + q * FA_D + ((col ^ fa_swz(q)) * 8)) = v;
+  }
+  const POLY_TIN *q_row = lds_q + (wave * 32 + lq) * FA_D;
+  const int q_sw = fa_swz(wave * 32 + lq);
+
+  // staging of K: 64 keys x 8 chunks of 16 bytes = 512 chunks, two per thread
+  int k_key[2], k_col[2];
+#pragma unroll
+  for (int i = 0; i < 2; i++) {
+    const int c = threadIdx.x + i * FA_THREADS;
+    k_key[i] = c >> 3;
+    k_col[i] = c & 7;
+  }
+  auto load_k = [&](int kb, fa_u32x4 (&rk)[2]) {
+#pragma unroll
+    for (int i = 0; i < 2; i++)
+      rk[i] = *(const fa_u32x4_u *)(POLY_K_PTR + poly_k_off(z, kb * FA_BN + k_key[i]) + k_col[i] * 8);
+  };
+  auto store_k = [&](int buf, const fa_u32x4 (&rk)[2]) {
+#pragma unroll
+    for (int i = 0; i < 2; i++)
+      *(fa_u32x4 *)(lds_k[buf] + k_key[i] * FA_D + ((k_col[i] ^ fa_swz(k_key[i])) * 8)) = rk[i];
+  };
+  // staging of V: 4 keys x 8 features per thread (threads 0..127), transposed in
+  // registers into 8 feature rows x 4 keys and written as 8-byte pieces
+  const bool v_thread = threadIdx.x < 128;
+  const int v_chunk = threadIdx.x & 7, v_kq = (threadIdx.x >> 3) & 15;   // features 8*chunk.., keys 4*kq..
+  auto load_v = [&](int kb, fa_u32x4 (&rv)[4]) {
+    if (v_thread) {
+#pragma unroll
+      for (int i = 0; i < 4; i++)
+        rv[i] = *(const fa_u32x4_u *)(POLY_V_PTR + poly_v_off(z, kb * FA_BN + v_kq * 4 + i) + v_chunk * 8);
+    }
+  };
+  auto store_v = [&](int buf, const fa_u32x4 (&rv)[4]) {
+    if (v_thread) {
+#pragma unroll
+      for (int j = 0; j < 4; j++) {
+        // dword j of load i holds features 2j (low half) and 2j+1 (high half) of key 4*kq+i
+        const unsigned int a0 = rv[0][j], a1 = rv[1][j], a2 = rv[2][j], a3 = rv[3][j];
+        fa_u32x2 lo, hi;
+        lo[0] = (a0 & 0xffffu) | (a1 << 16);
+        lo[1] = (a2 & 0xffffu) | (a3 << 16);
+        hi[0] = (a0 >> 16) | (a1 & 0xffff0000u);
+        hi[1] = (a2 >> 16) | (a3 & 0xffff0000u);
+        const int r0 = v_chunk * 8 + 2 * j, r1 = r0 + 1;
+        *(fa_u32x2 *)(lds_v[buf] + r0 * FA_BN + (((v_kq >> 1) ^ fa_swz(r0)) * 8) + (v_kq & 1) * 4) = lo;
+        *(fa_u32x2 *)(lds_v[buf] + r1 * FA_BN + (((v_kq >> 1) ^ fa_swz(r1)) * 8) + (v_kq & 1) * 4) = hi;
+      }
+    }
+  };
+
+  // S^T tile of this wave: 32 keys (tile t of the staged block) x 32 queries
+  auto scores = [&](int buf, int t, fa_acc16 &st) {
+#pragma unroll
+    for (int r = 0; r < 16; r++) st[r] = 0.0f;
+    const int key = 32 * t + lq;
+    const POLY_TIN *row = lds_k[buf] + key * FA_D;
+    const int sw = fa_swz(key);
+#pragma unroll
+    for (int s = 0; s < FA_D / 16; s++) {
+      const fa_in8 kf = *(const fa_in8 *)(row + (((2 * s + half) ^ sw) * 8));
+      const fa_in8 qf = *(const fa_in8 *)(q_row + (((2 * s + half) ^ q_sw) * 8));
+      st = POLY_MFMA(kf, qf, st);
+    }
+  };
+  // key index of accumulator register r of tile t
+  auto key_of = [&](int kb, int t, int r) { return kb * FA_BN + 32 * t + 8 * (r >> 2) + 4 * half + (r & 3); };
+
+  // ── pass 1: row maximum and sum of terms, one 32-key tile at a time ─────────
+  float row_max = -__builtin_inff(), row_sum = 0.0f;
+  unsigned long long dead = 0;   // wave-uniform: 32-key tiles whose terms are all exactly zero
+  {
+    fa_u32x4 rk[2];
+    load_k(0, rk);
+    store_k(0, rk);
+    __syncthreads();
+    for (int kb = 0; kb < FA_NKB; kb++) {
+      const int cur = kb & 1;
+      if (kb + 1 < FA_NKB) load_k(kb + 1, rk);
+#pragma unroll
+      for (int t = 0; t < 2; t++) {
+        fa_acc16 st;
+        scores(cur, t, st);
+        POLY_TIN x[16];
+        float bm = -__builtin_inff(), nan_probe = 0.0f;
+#pragma unroll
+        for (int r = 0; r < 16; r++) {
+          const int n = key_of(kb, t, r);
+          x[r] = POLY_FA_SCORE(st[r], mq, n, z);
+          const float v = POLY_FA_MAXV(x[r], mq, n, z);
+          bm = (bm < v) ? v : bm;
+          nan_probe = nan_probe + v;      // NaN if any value is (or +inf meets -inf: then not skipped)
+        }
+        const float new_max = (row_max < bm) ? bm : row_max;
+        // upper bound of this lane's terms in this tile
+        const float bound = POLY_FA_TERM((POLY_TIN)bm, new_max, mq, 0, z);
+        const bool lane_dead = (bound == 0.0f) && (nan_probe == nan_probe);
+        if (__builtin_amdgcn_ballot_w64(!lane_dead) != 0) {
+          float acc = row_sum * POLY_FA_TERM((POLY_TIN)row_max, new_max, mq, 0, z);
+#pragma unroll
+          for (int r = 0; r < 16; r++) acc = acc + POLY_FA_TERM(x[r], new_max, mq, key_of(kb, t, r), z);
+          row_sum = acc;
+          row_max = new_max;
+        } else {
+          // every term is an exact zero and the maximum did not move: nothing to add
+          if (2 * kb + t < 64) dead |= 1ull << (2 * kb + t);
+        }
+      }
+      if (kb + 1 < FA_NKB) store_k(cur ^ 1, rk);
+      __syncthreads();
+    }
+    // the two lanes of a query (l, l ^ 32) each saw half of the keys
+    const float o_max = fa_other_half(row_max), o_sum = fa_other_half(row_sum);
+    const float f_max = (row_max < o_max) ? o_max : row_max;
+    const float mine = row_sum * POLY_FA_TERM((POLY_TIN)row_max, f_max, mq, 0, z);
+    const float theirs = o_sum * POLY_FA_TERM((POLY_TIN)o_max, f_max, mq, 0, z);
+    // same operand order on both lanes, so both hold the identical sum
+    row_sum = half == 0 ? mine + theirs : theirs + mine;
+    row_max = f_max;
+  }
+
+  // ── pass 2: probabilities and P V ───────────────────────────────────────────
+  fa_acc16 o[2];
+#pragma unroll
+  for (int dt = 0; dt < 2; dt++)
+#pragma unroll
+    for (int r = 0; r < 16; r++) o[dt][r] = 0.0f;
+  {
+    // zero / sum is an exact zero only for a finite, non-zero sum
+    const bool sums_ok = __builtin_amdgcn_ballot_w64(!(row_sum > 0.0f && row_sum < __builtin_inff())) == 0;
+    fa_u32x4 rk[2], rv[4];
+    load_k(0, rk);
+    load_v(0, rv);
+    store_k(0, rk);
+    store_v(0, rv);
+    __syncthreads();
+    for (int kb = 0; kb < FA_NKB; kb++) {
+      const int cur = kb & 1;
+      if (kb + 1 < FA_NKB) { load_k(kb + 1, rk); load_v(kb + 1, rv); }
+      // V fragment (B operand) for the 16 keys 32t + 16u .. of feature tile dt
+      auto v_frag = [&](int t, int u, int dt) {
+        const int col0 = 4 * t + 2 * u;   // 16-byte column of keys 32t+16u .. +7 in a V^T row
+        const int d = 32 * dt + lq;
+        const POLY_TIN *row = lds_v[cur] + d * FA_BN;
+        const int sw = fa_swz(d);
+        const fa_u32x2 lo = *(const fa_u32x2 *)(row + ((col0 ^ sw) * 8) + half * 4);
+        const fa_u32x2 hi = *(const fa_u32x2 *)(row + (((col0 + 1) ^ sw) * 8) + half * 4);
+        fa_u32x4 both;
+        both[0] = lo[0]; both[1] = lo[1]; both[2] = hi[0]; both[3] = hi[1];
+        return __builtin_bit_cast(fa_in8, both);
+      };
+#pragma unroll
+      for (int t = 0; t < 2; t++) {
+        const int tile = 2 * kb + t;
+        const bool skip = POLY_FA_SKIP_DEAD_BLOCKS && sums_ok && tile < 64 && ((dead >> tile) & 1ull);
+        if (skip) {
+          // probabilities are exact zeros; 0 * V keeps a non-finite V visible
+          fa_in8 zf;
+#pragma unroll
+          for (int i = 0; i < 8; i++) zf[i] = (POLY_TIN)0.0f;
+#pragma unroll
+          for (int u = 0; u < 2; u++)
+#pragma unroll
+            for (int dt = 0; dt < 2; dt++) o[dt] = POLY_MFMA(zf, v_frag(t, u, dt), o[dt]);
+        } else {
+          fa_acc16 st;
+          scores(cur, t, st);
+          POLY_TIN p[16];
+#pragma unroll
+          for (int r = 0; r < 16; r++) {
+            const int n = key_of(kb, t, r);
+            const POLY_TIN x = POLY_FA_SCORE(st[r], mq, n, z);
+            p[r] = POLY_FA_P(x, row_max, row_sum, mq, n, z);
+          }
+#pragma unroll
+          for (int u = 0; u < 2; u++) {
+            fa_in8 pf;
+#pragma unroll
+            for (int i = 0; i < 8; i++) pf[i] = p[8 * u + i];
+#pragma unroll
+            for (int dt = 0; dt < 2; dt++) o[dt] = POLY_MFMA(pf, v_frag(t, u, dt), o[dt]);
+          }
+        }
+      }
+      if (kb + 1 < FA_NKB) { store_k(cur ^ 1, rk); store_v(cur ^ 1, rv); }
+      __syncthreads();
+    }
+  }
+
+  // Output tile: register r of lane l holds query row 8*(r/4) + 4*(l/32) + r%4, feature l%32.
+#pragma unroll
+  for (int dt = 0; dt < 2; dt++)
+#pragma unroll
+    for (int r = 0; r < 16; r++) {
+      const int m = m0 + wave * 32 + 8 * (r >> 2) + 4 * half + (r & 3);
+      POLY_FA_OUT(o[dt][r], m, 32 * dt + lq, z);
+    }
+}

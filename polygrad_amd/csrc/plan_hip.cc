@@ -11,7 +11,9 @@
 //   * kernels are enqueued on one stream with no per-kernel synchronisation and
 //     no per-launch allocation (src/exec_plan.c:590-607 does both);
 //   * the launch sequence is captured into a hipGraph and replayed while the
-//     bound pointers and variable values repeat.
+//     bound pointers and variable values repeat;
+//   * kernel groups that fusion.cc recognises run as one launch and their
+//     intermediates get no memory at all.
 #include <hip/hip_runtime.h>
 
 #include <algorithm>
@@ -19,6 +21,7 @@
 #include <cstring>
 #include <memory>
 
+#include "fusion.h"
 #include "polygrad_hip.h"
 #include "runtime_hip.h"
 
@@ -43,16 +46,25 @@ extern "C" __global__ void __launch_bounds__(256) poly_fill0(unsigned int* p, lo
 
 }  // namespace
 
+// One launch of the plan: a scheduled kernel, or a fused group of them.
+struct Unit {
+  HipRunner *runner = nullptr;
+  int item = -1;                 // schedule item (also for a fused group: the item it runs in place of)
+  std::vector<int> slots;        // buffer slot per kernel argument
+  int n_vars = 0;                // DEFINE_VAR arguments (taken from `item`)
+  int n_items = 1;               // schedule items this launch stands for
+};
+
 struct PolyHipPlan {
   const PolySchedule *sched = nullptr;
-  std::vector<HipRunner *> runners;          // by item index
+  std::vector<Unit> units;                   // in execution order
   std::vector<void *> slot_ptr;              // device pointer per slot (intermediates fixed)
   std::vector<size_t> slot_off;
   std::vector<char> slot_needs_zero;
   void *arena = nullptr;
   size_t arena_bytes = 0;
-  std::vector<std::vector<void *>> kargs;    // per item: args array handed to runner_launch
-  std::vector<std::vector<int>> var_vals;    // per item: storage for var ints
+  std::vector<std::vector<void *>> kargs;    // per unit: args array handed to runner_launch
+  std::vector<std::vector<int>> var_vals;    // per unit: storage for var ints
   std::vector<PolyVarBinding> merged;
   Program *fill = nullptr;
   bool use_graph = true;
@@ -63,7 +75,7 @@ struct PolyHipPlan {
       if (g.exec) (void)hipGraphExecDestroy(g.exec);
       if (g.graph) (void)hipGraphDestroy(g.graph);
     }
-    for (HipRunner *r : runners) runner_destroy(r);
+    for (Unit &u : units) runner_destroy(u.runner);
     if (fill) program_destroy(fill);
     if (arena) runtime_free(arena);
   }
@@ -114,11 +126,10 @@ int enqueue_all(PolyHipPlan *plan) {
     ls.grid[0] = (unsigned)std::min<long long>((words + 255) / 256, 65536);
     if (program_launch(plan->fill, args, ls) != 0) return -1;
   }
-  for (int step = 0; step < s->n_items; step++) {
-    int k = s->exec_order[step];
-    std::vector<void *> &a = plan->kargs[(size_t)k];
-    if (runner_launch(plan->runners[(size_t)k], a.data(), (int)a.size()) != 0) {
-      log_err("plan_run", "kernel %d failed to launch", k);
+  for (size_t u = 0; u < plan->units.size(); u++) {
+    std::vector<void *> &a = plan->kargs[u];
+    if (runner_launch(plan->units[u].runner, a.data(), (int)a.size()) != 0) {
+      log_err("plan_run", "kernel %d failed to launch", plan->units[u].item);
       return -1;
     }
   }
@@ -137,39 +148,63 @@ PolyHipPlan *poly_hip_compile_schedule(PolyCtx *ctx, const PolySchedule *s) {
   plan->sched = s;
   static int plan_counter = 0;
   std::vector<KernelGraph> graphs((size_t)s->n_items);
-  plan->runners.assign((size_t)s->n_items, nullptr);
   for (int k = 0; k < s->n_items; k++) {
     const PolyExecItem &it = s->items[k];
     if (it.kind != POLY_EXEC_COMPUTE) {
       log_err("compile_schedule", "non-COMPUTE item %d not supported", k);
       return nullptr;
     }
-    std::string name = strf("hip%d_k%d", plan_counter, k);
     if (!graphs[(size_t)k].build(it.root)) {
       log_err("compile_schedule", "kernel %d: %s", k, graphs[(size_t)k].error.c_str());
       return nullptr;
     }
-    HipRunner *r = runner_create(it.root, name.c_str(), 0);
-    if (!r) {
+  }
+  // kernel groups that run as one launch
+  std::vector<FusedGroup> groups;
+  find_fused_groups(s, graphs, &groups);
+  std::vector<int> group_of((size_t)s->n_items, -1);
+  std::vector<char> internal((size_t)s->n_buf_slots, 0);
+  for (size_t gi = 0; gi < groups.size(); gi++) {
+    for (int it : groups[gi].items) group_of[(size_t)it] = (int)gi;
+    for (int sl : groups[gi].internal_slots) internal[(size_t)sl] = 1;
+  }
+  for (int step = 0; step < s->n_items; step++) {
+    const int k = s->exec_order[step];
+    const PolyExecItem &it = s->items[k];
+    std::string name = strf("hip%d_k%d", plan_counter, k);
+    Unit u;
+    u.item = k;
+    if (group_of[(size_t)k] >= 0) {
+      FusedGroup &fg = groups[(size_t)group_of[(size_t)k]];
+      if (fg.launch_item != k) continue;   // runs as part of the group, later
+      u.runner = runner_from_rendered(fg.rk, name.c_str(), false);
+      u.slots = fg.arg_slots;
+      u.n_items = (int)fg.items.size();
+    } else {
+      u.runner = runner_create(it.root, name.c_str(), 0);
+      if (u.runner && (u.runner->rk.n_params != it.n_buf_slots || u.runner->rk.n_vars != it.n_var_uops)) {
+        log_err("compile_schedule", "kernel %d: %d params / %d vars in the graph, %d / %d in the schedule", k,
+                u.runner->rk.n_params, u.runner->rk.n_vars, it.n_buf_slots, it.n_var_uops);
+        runner_destroy(u.runner);
+        return nullptr;
+      }
+      u.slots.assign(it.buf_slot_indices, it.buf_slot_indices + it.n_buf_slots);
+      u.n_vars = it.n_var_uops;
+    }
+    if (!u.runner) {
       log_err("compile_schedule", "backend 'hip' failed for kernel %d", k);
       return nullptr;
     }
-    plan->runners[(size_t)k] = r;
-    if (r->rk.n_params != it.n_buf_slots || r->rk.n_vars != it.n_var_uops) {
-      log_err("compile_schedule", "kernel %d: %d params / %d vars in the graph, %d / %d in the schedule", k,
-              r->rk.n_params, r->rk.n_vars, it.n_buf_slots, it.n_var_uops);
-      return nullptr;
-    }
+    plan->units.push_back(u);
   }
   plan_counter++;
 
   // ── lifetimes of intermediates in execution order ──────────────────────
   const int ns = s->n_buf_slots;
   std::vector<int> first((size_t)ns, -1), last((size_t)ns, -1);
-  for (int step = 0; step < s->n_items; step++) {
-    const PolyExecItem &it = s->items[s->exec_order[step]];
-    for (int i = 0; i < it.n_buf_slots; i++) {
-      int sl = it.buf_slot_indices[i];
+  const int n_units = (int)plan->units.size();
+  for (int step = 0; step < n_units; step++) {
+    for (int sl : plan->units[(size_t)step].slots) {
       if (sl < 0 || sl >= ns) { log_err("compile_schedule", "bad slot index %d", sl); return nullptr; }
       if (first[(size_t)sl] < 0) first[(size_t)sl] = step;
       last[(size_t)sl] = step;
@@ -179,7 +214,7 @@ PolyHipPlan *poly_hip_compile_schedule(PolyCtx *ctx, const PolySchedule *s) {
   struct Placed { size_t off, size; int first, last; };
   std::vector<Placed> placed;
   std::vector<int> order;
-  for (int i = 0; i < ns; i++) if (s->buf_slots[i].is_intermediate) order.push_back(i);
+  for (int i = 0; i < ns; i++) if (s->buf_slots[i].is_intermediate && !internal[(size_t)i]) order.push_back(i);
   const bool no_alias = getenv("POLY_HIP_NO_ALIAS") != nullptr;
   std::sort(order.begin(), order.end(), [&](int a, int b) {
     if (s->buf_slots[a].nbytes != s->buf_slots[b].nbytes) return s->buf_slots[a].nbytes > s->buf_slots[b].nbytes;
@@ -190,8 +225,8 @@ PolyHipPlan *poly_hip_compile_schedule(PolyCtx *ctx, const PolySchedule *s) {
   for (int sl : order) {
     size_t size = align_up((size_t)std::max<int64_t>(s->buf_slots[sl].nbytes, 4), 256);
     int f = first[(size_t)sl], l = last[(size_t)sl];
-    if (f < 0) { f = 0; l = s->n_items; }
-    if (no_alias) { f = 0; l = s->n_items; }
+    if (f < 0) { f = 0; l = n_units; }
+    if (no_alias) { f = 0; l = n_units; }
     // candidate offsets: 0 and the end of every conflicting block
     std::vector<Placed> conflicts;
     for (const Placed &p : placed)
@@ -222,11 +257,11 @@ PolyHipPlan *poly_hip_compile_schedule(PolyCtx *ctx, const PolySchedule *s) {
     plan->fill = program_create(kFillSrc, "poly_fill0");
     if (!plan->fill) return nullptr;
   }
-  plan->kargs.resize((size_t)s->n_items);
-  plan->var_vals.resize((size_t)s->n_items);
-  for (int k = 0; k < s->n_items; k++) {
-    plan->kargs[(size_t)k].assign((size_t)(s->items[k].n_buf_slots + s->items[k].n_var_uops), nullptr);
-    plan->var_vals[(size_t)k].assign((size_t)s->items[k].n_var_uops, 0);
+  plan->kargs.resize((size_t)n_units);
+  plan->var_vals.resize((size_t)n_units);
+  for (int u = 0; u < n_units; u++) {
+    plan->kargs[(size_t)u].assign(plan->units[(size_t)u].slots.size() + (size_t)plan->units[(size_t)u].n_vars, nullptr);
+    plan->var_vals[(size_t)u].assign((size_t)plan->units[(size_t)u].n_vars, 0);
   }
   return plan.release();
 }
@@ -249,24 +284,25 @@ static int bind_args(PolyHipPlan *plan, void **slot_data, int n_slots, const Pol
       if (m.var == vb[i].var) { m.value = vb[i].value; found = true; break; }
     if (!found) plan->merged.push_back(vb[i]);
   }
-  for (int k = 0; k < s->n_items; k++) {
-    const PolyExecItem &it = s->items[k];
-    std::vector<void *> &a = plan->kargs[(size_t)k];
-    for (int i = 0; i < it.n_buf_slots; i++) {
-      void *p = plan->slot_ptr[(size_t)it.buf_slot_indices[i]];
+  for (size_t u = 0; u < plan->units.size(); u++) {
+    const Unit &un = plan->units[u];
+    const PolyExecItem &it = s->items[un.item];
+    std::vector<void *> &a = plan->kargs[u];
+    for (size_t i = 0; i < un.slots.size(); i++) {
+      void *p = plan->slot_ptr[(size_t)un.slots[i]];
       if (!p) {
-        log_err("plan_run", "missing data for param %d (slot %d) in kernel %d", i, it.buf_slot_indices[i], k);
+        log_err("plan_run", "missing data for param %zu (slot %d) in kernel %d", i, un.slots[i], un.item);
         return -1;
       }
-      a[(size_t)i] = p;
+      a[i] = p;
     }
-    for (int v = 0; v < it.n_var_uops; v++) {
+    for (int v = 0; v < un.n_vars; v++) {
       bool found = false;
       for (const PolyVarBinding &m : plan->merged)
-        if (m.var == it.var_uops[v]) { plan->var_vals[(size_t)k][(size_t)v] = m.value; found = true; break; }
-      if (!found) { log_err("plan_run", "no binding for DEFINE_VAR in kernel %d", k); return -1; }
-      a[(size_t)(it.n_buf_slots + v)] = &plan->var_vals[(size_t)k][(size_t)v];
-      key = fnv1a(&plan->var_vals[(size_t)k][(size_t)v], sizeof(int), key);
+        if (m.var == it.var_uops[v]) { plan->var_vals[u][(size_t)v] = m.value; found = true; break; }
+      if (!found) { log_err("plan_run", "no binding for DEFINE_VAR in kernel %d", un.item); return -1; }
+      a[un.slots.size() + (size_t)v] = &plan->var_vals[u][(size_t)v];
+      key = fnv1a(&plan->var_vals[u][(size_t)v], sizeof(int), key);
     }
   }
   *key_out = key;
@@ -322,53 +358,70 @@ int poly_hip_plan_run(PolyHipPlan *plan, void **slot_data, int n_slots, const Po
   return 0;
 }
 
+int poly_hip_fused_groups(const PolySchedule *s, int index, char **source_out, int *n_items_out) {
+  if (!s) return -1;
+  std::vector<KernelGraph> graphs((size_t)s->n_items);
+  for (int k = 0; k < s->n_items; k++)
+    if (s->items[k].kind != POLY_EXEC_COMPUTE || !graphs[(size_t)k].build(s->items[k].root)) return -1;
+  std::vector<FusedGroup> groups;
+  find_fused_groups(s, graphs, &groups);
+  if (index >= 0 && index < (int)groups.size()) {
+    if (n_items_out) *n_items_out = (int)groups[(size_t)index].items.size();
+    if (source_out) {
+      const std::string &src = groups[(size_t)index].rk.source;
+      *source_out = (char *)malloc(src.size() + 1);
+      if (*source_out) memcpy(*source_out, src.c_str(), src.size() + 1);
+    }
+  }
+  return (int)groups.size();
+}
+
 void poly_hip_plan_free(PolyHipPlan *plan) {
   if (!plan) return;
   runtime_sync();
   delete plan;
 }
 
-int poly_hip_plan_n_kernels(const PolyHipPlan *plan) { return plan ? (int)plan->runners.size() : -1; }
+int poly_hip_plan_n_kernels(const PolyHipPlan *plan) { return plan ? (int)plan->units.size() : -1; }
 
 int poly_hip_plan_kernel_info(const PolyHipPlan *plan, int cap, int *klass, double *bytes, double *flops) {
   if (!plan) return -1;
-  const PolySchedule *s = plan->sched;
-  for (int step = 0; step < s->n_items && step < cap; step++) {
-    const HipRunner *r = plan->runners[(size_t)s->exec_order[step]];
+  const int n = (int)plan->units.size();
+  for (int step = 0; step < n && step < cap; step++) {
+    const HipRunner *r = plan->units[(size_t)step].runner;
     if (klass) klass[step] = (int)r->rk.klass;
     if (bytes) bytes[step] = r->rk.bytes;
     if (flops) flops[step] = r->rk.flops;
   }
-  return s->n_items;
+  return n;
 }
 
 int poly_hip_plan_profile(PolyHipPlan *plan, void **slot_data, int n_slots, float *ms_out, int cap) {
   if (!plan) return -1;
   uint64_t key;
   if (bind_args(plan, slot_data, n_slots, nullptr, 0, &key) != 0) return -1;
-  const PolySchedule *s = plan->sched;
+  const int n = (int)plan->units.size();
   hipStream_t stream = (hipStream_t)runtime_stream();
-  std::vector<hipEvent_t> ev((size_t)s->n_items + 1);
+  std::vector<hipEvent_t> ev((size_t)n + 1);
   for (hipEvent_t &e : ev) if (hipEventCreate(&e) != hipSuccess) return -1;
   int rc = 0;
   (void)hipEventRecord(ev[0], stream);
-  for (int step = 0; step < s->n_items && rc == 0; step++) {
-    int k = s->exec_order[step];
-    std::vector<void *> &a = plan->kargs[(size_t)k];
-    rc = runner_launch(plan->runners[(size_t)k], a.data(), (int)a.size());
+  for (int step = 0; step < n && rc == 0; step++) {
+    std::vector<void *> &a = plan->kargs[(size_t)step];
+    rc = runner_launch(plan->units[(size_t)step].runner, a.data(), (int)a.size());
     (void)hipEventRecord(ev[(size_t)step + 1], stream);
   }
   (void)hipStreamSynchronize(stream);
-  for (int step = 0; step < s->n_items && step < cap && rc == 0; step++)
+  for (int step = 0; step < n && step < cap && rc == 0; step++)
     (void)hipEventElapsedTime(&ms_out[step], ev[(size_t)step], ev[(size_t)step + 1]);
   for (hipEvent_t &e : ev) (void)hipEventDestroy(e);
-  return rc == 0 ? s->n_items : -1;
+  return rc == 0 ? n : -1;
 }
 
 char *poly_hip_plan_kernel_desc(const PolyHipPlan *plan, int step) {
-  if (!plan || step < 0 || step >= plan->sched->n_items) return nullptr;
-  const HipRunner *r = plan->runners[(size_t)plan->sched->exec_order[step]];
-  static const char *const kn[] = {"elementwise", "row-reduce", "thread-reduce", "matmul-mfma", "gather", "copy"};
+  if (!plan || step < 0 || step >= (int)plan->units.size()) return nullptr;
+  const HipRunner *r = plan->units[(size_t)step].runner;
+  static const char *const kn[] = {"elementwise", "row-reduce", "thread-reduce", "matmul-mfma", "gather", "copy", "attention-mfma"};
   std::string d = strf("%s %s: %s grid=%u,%u,%u bytes=%.0f flops=%.0f", r->name.c_str(), kn[(int)r->rk.klass],
                        r->rk.strategy.c_str(), r->rk.launch.grid[0], r->rk.launch.grid[1], r->rk.launch.grid[2],
                        r->rk.bytes, r->rk.flops);

@@ -13,17 +13,13 @@
 //                 (short reductions, or reductions this file cannot split).
 // Matmul-shaped and gather-shaped kernels are tried first in templates.cc.
 #include "render_hip.h"
+#include "templates.h"
 
 #include <algorithm>
 #include <cmath>
 #include <set>
 
 namespace polyhip {
-
-bool try_render_matmul(const KernelGraph &g, const std::string &fn, const RenderOptions &opt,
-                       RenderedKernel *out);
-bool try_render_gather(const KernelGraph &g, const std::string &fn, const RenderOptions &opt,
-                       RenderedKernel *out);
 
 namespace {
 

@@ -23,7 +23,7 @@ struct LaunchSpec {
   unsigned lds_bytes = 0;
 };
 
-enum class KernelClass { ELEMENTWISE, ROW_REDUCE, THREAD_REDUCE, MATMUL_MFMA, GATHER, COPY };
+enum class KernelClass { ELEMENTWISE, ROW_REDUCE, THREAD_REDUCE, MATMUL_MFMA, GATHER, COPY, ATTENTION };
 
 struct RenderedKernel {
   std::string source;      // complete HIP C translation unit
@@ -104,6 +104,9 @@ class Emitter {
   bool failed() const { return !error_.empty(); }
   const std::string &error() const { return error_; }
   bool uses_threefry = false;
+  // f32 EXP2 as the bare hardware instruction: results below 2^-126 come out as 0 instead
+  // of denormals (the library form wraps the instruction in a range-scaling sequence).
+  bool raw_exp2 = false;
 
  private:
   std::string emit_atom(int atom, Scope *s);

@@ -38,6 +38,9 @@ struct HipRunner {
 };
 
 HipRunner *runner_create(const PolyUOp *root, const char *fn_name, int flags);
+// From a kernel rendered elsewhere (fused groups); `named` false: the entry is still the
+// placeholder poly_k and gets its descriptive symbol here.
+HipRunner *runner_from_rendered(const RenderedKernel &rk, const char *fn_name, bool named);
 int runner_launch(HipRunner *r, void **args, int n_args);
 void runner_destroy(HipRunner *r);
 

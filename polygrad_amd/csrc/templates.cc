@@ -8,7 +8,7 @@
 #include <cmath>
 #include <cstdlib>
 
-#include "render_hip.h"
+#include "templates.h"
 
 namespace polyhip {
 
@@ -22,11 +22,8 @@ PolyOps reduce_op(const KNode &k) {
   return k.u->arg.kind == POLY_ARG_OPS ? k.u->arg.ops : (PolyOps)k.u->arg.i;
 }
 
-// One operand of the product: LOAD(INDEX(PARAM, lin)) optionally under a CAST to f32.
-struct Operand {
-  int load = -1, param = -1, lin = -1;
-  DT dt = DT_VOID;
-};
+typedef MmOperand Operand;
+typedef MmDim Dim;
 
 bool match_operand(const KernelGraph &g, int node, Operand *o) {
   const KNode *k = &g.n(node);
@@ -40,8 +37,6 @@ bool match_operand(const KernelGraph &g, int node, Operand *o) {
   o->dt = k->dt;
   return o->lin >= 0 && o->param >= 0;
 }
-
-struct KSplit { int64_t kb, s_hi, s_lo; };  // off(k) = (k / kb) * s_hi + (k % kb) * s_lo
 
 // Extracts the dependence of `l` on reduce range `kr` (extent K).
 bool k_dependence(const KernelGraph &g, const Lin &l, int kr, int64_t K, KSplit *ks) {
@@ -69,12 +64,6 @@ bool k_dependence(const KernelGraph &g, const Lin &l, int kr, int64_t K, KSplit 
   if (have_mod && !have_div) { *ks = {c_mod, 0, s_lo}; return true; }
   return false;  // no dependence on k at all
 }
-
-// One output coordinate: a digit of an END range.  A range r that the indices use
-// only through r / a, r % b and (r / a) % b is a mixed-radix number; each digit
-// d = (r / cut) % extent becomes a coordinate of its own (a plain range is the
-// single digit with cut 1).
-struct Dim { int ord; int64_t extent, ca, cb; int64_t cut = 1; };
 
 struct DigitUse { int64_t coef, a, b; };  // coef * ((r / a) % b), b = 0: no modulus
 
@@ -161,26 +150,26 @@ static bool reject(int line) {
 
 }  // namespace
 
-bool try_render_matmul(const KernelGraph &g, const std::string &fn, const RenderOptions &opt, RenderedKernel *out) {
-  (void)fn; (void)opt;
-  if (g.stores.size() != 1 || g.reduces.size() != 1 || !g.vars.empty()) return reject(__LINE__);
+bool match_matmul(const KernelGraph &g, MatmulMatch *mm, int *reject_line) {
+#define MM_REJECT() do { if (reject_line) *reject_line = __LINE__; return false; } while (0)
+  if (g.stores.size() != 1 || g.reduces.size() != 1 || !g.vars.empty()) MM_REJECT();
   const StoreInfo &st = g.stores[0];
-  if (st.gate >= 0) return reject(__LINE__);
+  if (st.gate >= 0) MM_REJECT();
   const int red = g.reduces[0];
   const KNode &R = g.n(red);
-  if (reduce_op(R) != POLY_OP_ADD || R.dt != DT_F32 || R.src.size() != 2) return reject(__LINE__);
+  if (reduce_op(R) != POLY_OP_ADD || R.dt != DT_F32 || R.src.size() != 2) MM_REJECT();
   const int kr = g.range_ord.at(R.src[1]);
   const int64_t K = g.ranges[(size_t)kr].extent;
-  if (K < 16) return reject(__LINE__);
+  if (K < 16) MM_REJECT();
   const KNode &mul = g.n(R.src[0]);
-  if (mul.op != POLY_OP_MUL || mul.dt != DT_F32) return reject(__LINE__);
+  if (mul.op != POLY_OP_MUL || mul.dt != DT_F32) MM_REJECT();
   Operand A, B;
-  if (!match_operand(g, mul.src[0], &A) || !match_operand(g, mul.src[1], &B)) return reject(__LINE__);
-  if (A.dt != B.dt || (A.dt != DT_BF16 && A.dt != DT_F16)) return reject(__LINE__);
-  for (const ParamInfo &p : g.params) if (p.numel >= ((int64_t)1 << 31)) return reject(__LINE__);
+  if (!match_operand(g, mul.src[0], &A) || !match_operand(g, mul.src[1], &B)) MM_REJECT();
+  if (A.dt != B.dt || (A.dt != DT_BF16 && A.dt != DT_F16)) MM_REJECT();
+  for (const ParamInfo &p : g.params) if (p.numel >= ((int64_t)1 << 31)) MM_REJECT();
   const Lin &la = g.lins[(size_t)A.lin], &lb = g.lins[(size_t)B.lin];
   KSplit ka, kb;
-  if (!k_dependence(g, la, kr, K, &ka) || !k_dependence(g, lb, kr, K, &kb)) return reject(__LINE__);
+  if (!k_dependence(g, la, kr, K, &ka) || !k_dependence(g, lb, kr, K, &kb)) MM_REJECT();
 
   // classify the END ranges of the store
   std::vector<Dim> md, nd, zd;
@@ -191,33 +180,102 @@ bool try_render_matmul(const KernelGraph &g, const std::string &fn, const Render
   };
   for (int r : st.ranges) {
     const int64_t e = g.ranges[(size_t)r].extent;
-    if (e < 0) return reject(__LINE__);
+    if (e < 0) MM_REJECT();
     std::vector<Dim> digits;
-    if (!factor_range(g, la, lb, r, e, &digits)) return reject(__LINE__);
+    if (!factor_range(g, la, lb, r, e, &digits)) MM_REJECT();
     for (const Dim &d : digits) place_dim(d);
   }
-  if (md.empty() || nd.empty()) return reject(__LINE__);
-  // every other atom in the operand indices must be a plain range handled above
-  auto only_known = [&](const Lin &l) {
-    for (const Term &t : l.terms) {
-      const Atom &a = g.atoms[(size_t)t.atom];
-      uint64_t d = g.atom_deps(t.atom);
-      if (d & ((uint64_t)1 << kr)) continue;            // checked by k_dependence
-      (void)a;                                          // global ranges were vetted by range_use
-    }
-    return true;
-  };
-  if (!only_known(la) || !only_known(lb)) return reject(__LINE__);
+  if (md.empty() || nd.empty()) MM_REJECT();
+#undef MM_REJECT
 
   // dims keep END order (outermost first); the innermost one is the fast coordinate
-  std::vector<Dim> md_full = md, nd_full = nd, zd_full = zd;
+  mm->md_full = md; mm->nd_full = nd; mm->zd_full = zd;
   collapse(md); collapse(nd); collapse(zd);
-  int64_t M = 1, N = 1, Z = 1;
-  for (const Dim &d : md) M *= d.extent;
-  for (const Dim &d : nd) N *= d.extent;
-  for (const Dim &d : zd) Z *= d.extent;
-  if (M > 2147483647LL || N > 2147483647LL || Z > 65535) return reject(__LINE__);
+  mm->md = md; mm->nd = nd; mm->zd = zd;
+  mm->M = mm->N = mm->Z = 1;
+  for (const Dim &d : md) mm->M *= d.extent;
+  for (const Dim &d : nd) mm->N *= d.extent;
+  for (const Dim &d : zd) mm->Z *= d.extent;
+  mm->red = red; mm->kr = kr; mm->K = K;
+  mm->A = A; mm->B = B; mm->ka = ka; mm->kb = kb;
+  mm->a_c0 = la.c0; mm->b_c0 = lb.c0;
+  return true;
+}
 
+std::string matmul_decompose(const MatmulMatch &mm, Emitter *em) {
+  std::string decomp;
+  std::vector<std::pair<int, std::string>> range_sum;   // ordinal -> sum of digit * cut
+  auto decompose = [&](const std::vector<Dim> &dims, const char *var) {
+    if (dims.empty()) return;
+    decomp += strf("  int t_%s = %s;\n", var, var);
+    for (size_t i = dims.size(); i-- > 0;) {
+      const Dim &d = dims[i];
+      std::string dv = strf("d%d_%lld", d.ord, (long long)d.cut);
+      if (i == 0) decomp += strf("  const int %s = t_%s;\n", dv.c_str(), var);
+      else decomp += strf("  const int %s = t_%s %% %lld; t_%s /= %lld;\n", dv.c_str(), var, (long long)d.extent, var, (long long)d.extent);
+      std::string term = d.cut == 1 ? dv : strf("%s * %lld", dv.c_str(), (long long)d.cut);
+      bool found = false;
+      for (auto &rs : range_sum) if (rs.first == d.ord) { rs.second += " + " + term; found = true; }
+      if (!found) range_sum.push_back({d.ord, term});
+    }
+  };
+  decompose(mm.md_full, "m");
+  decompose(mm.nd_full, "n");
+  decompose(mm.zd_full, "z");
+  for (auto &rs : range_sum) {
+    decomp += strf("  const int r%d = %s;\n", rs.first, rs.second.c_str());
+    if (em) em->bind_range(rs.first, strf("r%d", rs.first));
+  }
+  return decomp;
+}
+
+std::string matmul_offset_fn(const char *name, const std::vector<MmDim> &dims, bool use_a, int64_t c0) {
+  return offset_fn(name, dims, use_a, c0);
+}
+
+std::string matmul_k_fn(const char *name, const KSplit &ks, int64_t K) {
+  if (ks.kb >= K) return strf("__device__ __forceinline__ int %s(int k) { return k * %lld; }\n", name, (long long)ks.s_lo);
+  return strf("__device__ __forceinline__ int %s(int k) { return (k / %lld) * %lld + (k %% %lld) * %lld; }\n", name,
+              (long long)ks.kb, (long long)ks.s_hi, (long long)ks.kb, (long long)ks.s_lo);
+}
+
+int64_t matmul_eval_offset(const std::vector<MmDim> &dims, bool use_a, int64_t x) {
+  int64_t off = 0;
+  for (size_t i = dims.size(); i-- > 0;) {
+    const int64_t c = use_a ? dims[i].ca : dims[i].cb;
+    if (i == 0) off += x * c;
+    else { off += (x % dims[i].extent) * c; x /= dims[i].extent; }
+  }
+  return off;
+}
+
+int64_t matmul_range_value(const MatmulMatch &mm, int ord, int64_t m, int64_t n, int64_t z) {
+  int64_t v = 0;
+  auto walk = [&](const std::vector<MmDim> &dims, int64_t x) {
+    for (size_t i = dims.size(); i-- > 0;) {
+      int64_t digit = i == 0 ? x : x % dims[i].extent;
+      if (i != 0) x /= dims[i].extent;
+      if (dims[i].ord == ord) v += digit * dims[i].cut;
+    }
+  };
+  walk(mm.md_full, m);
+  walk(mm.nd_full, n);
+  walk(mm.zd_full, z);
+  return v;
+}
+
+bool try_render_matmul(const KernelGraph &g, const std::string &fn, const RenderOptions &opt, RenderedKernel *out) {
+  (void)fn; (void)opt;
+  MatmulMatch mm;
+  int line = 0;
+  if (!match_matmul(g, &mm, &line)) return reject(line);
+  const StoreInfo &st = g.stores[0];
+  const int red = mm.red;
+  const int64_t K = mm.K, M = mm.M, N = mm.N, Z = mm.Z;
+  const Operand &A = mm.A, &B = mm.B;
+  const KSplit &ka = mm.ka, &kb = mm.kb;
+  const std::vector<Dim> &md = mm.md, &nd = mm.nd, &zd = mm.zd;
+  if (M > 2147483647LL || N > 2147483647LL || Z > 65535) return reject(__LINE__);
   int BK = 64;
   if (const char *e = getenv("POLY_HIP_MM_BK")) BK = atoi(e) == 32 ? 32 : 64;
   // operand layout: contiguous along K, or along its row axis
@@ -261,29 +319,7 @@ bool try_render_matmul(const KernelGraph &g, const std::string &fn, const Render
   Scope S0;
   S0.indent = 1;
   for (int r : st.ranges) S0.avail |= (uint64_t)1 << r;
-  std::string decomp;
-  std::vector<std::pair<int, std::string>> range_sum;   // ordinal -> sum of digit * cut
-  auto decompose = [&](const std::vector<Dim> &dims, const char *var) {
-    if (dims.empty()) return;
-    decomp += strf("  int t_%s = %s;\n", var, var);
-    for (size_t i = dims.size(); i-- > 0;) {
-      const Dim &d = dims[i];
-      std::string dv = strf("d%d_%lld", d.ord, (long long)d.cut);
-      if (i == 0) decomp += strf("  const int %s = t_%s;\n", dv.c_str(), var);
-      else decomp += strf("  const int %s = t_%s %% %lld; t_%s /= %lld;\n", dv.c_str(), var, (long long)d.extent, var, (long long)d.extent);
-      std::string term = d.cut == 1 ? dv : strf("%s * %lld", dv.c_str(), (long long)d.cut);
-      bool found = false;
-      for (auto &rs : range_sum) if (rs.first == d.ord) { rs.second += " + " + term; found = true; }
-      if (!found) range_sum.push_back({d.ord, term});
-    }
-  };
-  decompose(md_full, "m");
-  decompose(nd_full, "n");
-  decompose(zd_full, "z");
-  for (auto &rs : range_sum) {
-    decomp += strf("  const int r%d = %s;\n", rs.first, rs.second.c_str());
-    em.bind_range(rs.first, strf("r%d", rs.first));
-  }
+  std::string decomp = matmul_decompose(mm, &em);
   em.preset(red, "acc");
   std::string val = em.emit(st.value, &S0);
   std::string idx = em.emit(g.n(st.index).src[1], &S0);
@@ -318,19 +354,14 @@ bool try_render_matmul(const KernelGraph &g, const std::string &fn, const Render
   cfg += offset_fn("poly_a_row", md, true, 0);
   cfg += offset_fn("poly_b_row", nd, false, 0);
   if (zd.empty()) {
-    cfg += strf("__device__ __forceinline__ int poly_a_z(int) { return %lld; }\n", (long long)la.c0);
-    cfg += strf("__device__ __forceinline__ int poly_b_z(int) { return %lld; }\n", (long long)lb.c0);
+    cfg += strf("__device__ __forceinline__ int poly_a_z(int) { return %lld; }\n", (long long)mm.a_c0);
+    cfg += strf("__device__ __forceinline__ int poly_b_z(int) { return %lld; }\n", (long long)mm.b_c0);
   } else {
-    cfg += offset_fn("poly_a_z", zd, true, la.c0);
-    cfg += offset_fn("poly_b_z", zd, false, lb.c0);
+    cfg += offset_fn("poly_a_z", zd, true, mm.a_c0);
+    cfg += offset_fn("poly_b_z", zd, false, mm.b_c0);
   }
-  auto kfn = [&](const char *name, const KSplit &ks) {
-    if (ks.kb >= K) return strf("__device__ __forceinline__ int %s(int k) { return k * %lld; }\n", name, (long long)ks.s_lo);
-    return strf("__device__ __forceinline__ int %s(int k) { return (k / %lld) * %lld + (k %% %lld) * %lld; }\n", name,
-                (long long)ks.kb, (long long)ks.s_hi, (long long)ks.kb, (long long)ks.s_lo);
-  };
-  cfg += kfn("poly_a_k", ka);
-  cfg += kfn("poly_b_k", kb);
+  cfg += matmul_k_fn("poly_a_k", ka, K);
+  cfg += matmul_k_fn("poly_b_k", kb, K);
   cfg += strf("#define POLY_SIGNATURE %s\n", params_decl.c_str());
   cfg += epi;
   cfg += strf("#define POLY_EPILOGUE(acc, m, n, z) poly_epilogue(acc, m, n, z, %s)\n", params_call.c_str());

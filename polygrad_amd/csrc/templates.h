@@ -1,0 +1,54 @@
+// Pattern matches shared by the single-kernel templates (templates.cc) and the
+// plan-level fusion of kernel groups (fusion.cc).
+#pragma once
+#include <string>
+#include <vector>
+
+#include "render_hip.h"
+
+namespace polyhip {
+
+// One operand of a matmul product: LOAD(INDEX(PARAM, lin)) optionally under a CAST to f32.
+struct MmOperand {
+  int load = -1, param = -1, lin = -1;   // param: position in KernelGraph::params
+  DT dt = DT_VOID;
+};
+
+// off(k) = (k / kb) * s_hi + (k % kb) * s_lo ; kb >= K means a plain stride s_lo
+struct KSplit { int64_t kb, s_hi, s_lo; };
+
+// One output coordinate: a digit of an END range.  A range r that the indices use
+// only through r / a, r % b and (r / a) % b is a mixed-radix number; each digit
+// d = (r / cut) % extent becomes a coordinate of its own (a plain range is the
+// single digit with cut 1).  ca / cb: coefficient in the A / B operand index.
+struct MmDim { int ord; int64_t extent, ca, cb; int64_t cut = 1; };
+
+// Structure of a kernel of the form STORE(f(REDUCE(ADD, cast(A[..]) * cast(B[..]), k))).
+struct MatmulMatch {
+  int red = -1, kr = -1;        // REDUCE node, ordinal of the reduce range
+  int64_t K = 0, M = 1, N = 1, Z = 1;
+  MmOperand A, B;
+  KSplit ka{0, 0, 0}, kb{0, 0, 0};
+  // digits of the END ranges, outermost first: those only A depends on (M), only B (N),
+  // both or neither (Z); *_full keep every digit, the others merge digits that nest
+  std::vector<MmDim> md, nd, zd, md_full, nd_full, zd_full;
+  int64_t a_c0 = 0, b_c0 = 0;   // constant parts of the operand indices
+};
+
+bool match_matmul(const KernelGraph &g, MatmulMatch *mm, int *reject_line);
+
+// C text that splits the flattened coordinates `m`, `n`, `z` (ints in scope) into the
+// kernel's END ranges, declared as `const int r<ord>`; binds them in `em` when given.
+std::string matmul_decompose(const MatmulMatch &mm, Emitter *em);
+// "__device__ int name(int x)": offset contribution of a flattened coordinate.
+std::string matmul_offset_fn(const char *name, const std::vector<MmDim> &dims, bool use_a, int64_t c0);
+std::string matmul_k_fn(const char *name, const KSplit &ks, int64_t K);
+// Host-side evaluation of the same maps (used to cross-check fused groups).
+int64_t matmul_eval_offset(const std::vector<MmDim> &dims, bool use_a, int64_t x);
+// value of END range `ord` at flattened coordinates (m, n, z)
+int64_t matmul_range_value(const MatmulMatch &mm, int ord, int64_t m, int64_t n, int64_t z);
+
+bool try_render_matmul(const KernelGraph &g, const std::string &fn, const RenderOptions &opt, RenderedKernel *out);
+bool try_render_gather(const KernelGraph &g, const std::string &fn, const RenderOptions &opt, RenderedKernel *out);
+
+}  // namespace polyhip

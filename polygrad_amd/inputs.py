@@ -45,7 +45,8 @@ def gpt2_slot_tensors(plan, vocab=50257, seed=3, device="cuda"):
 
 
 def random_slot_tensors(plan, seed=0, device="cuda", scale=1.0, outputs=()):
-    """Uniform(-scale, scale) floats (or small ints) for every external slot."""
+    """Uniform(-scale, scale) floats (or small ints) for every external slot; slots named
+    like the reference's index helpers (arange, positions, vocab_arange) hold 0..n-1."""
     g = torch.Generator(device=device)
     g.manual_seed(seed)
     data = [None] * len(plan.slots)
@@ -55,6 +56,8 @@ def random_slot_tensors(plan, seed=0, device="cuda", scale=1.0, outputs=()):
         dt = torch_dtype(s.dtype)
         if s.name in outputs:
             t = torch.zeros(s.numel, dtype=dt, device=device)
+        elif s.name in ("positions", "arange", "vocab_arange"):
+            t = torch.arange(s.numel, device=device).to(dt)
         elif dt.is_floating_point:
             t = ((torch.rand(s.numel, generator=g, device=device, dtype=torch.float32) * 2 - 1) * scale).to(dt)
         else:

@@ -12,7 +12,7 @@ from . import _ffi
 
 DT_NAMES = ["void", "bool", "int8", "uint8", "int16", "uint16", "int32", "uint32", "int64", "uint64",
             "float16", "bfloat16", "float32", "float64", "index"]
-KERNEL_CLASSES = ["elementwise", "row-reduce", "thread-reduce", "matmul-mfma", "gather", "copy"]
+KERNEL_CLASSES = ["elementwise", "row-reduce", "thread-reduce", "matmul-mfma", "gather", "copy", "attention-mfma"]
 
 
 def _dt_code(d):

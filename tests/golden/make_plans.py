@@ -5,6 +5,7 @@ the GPU box, where the reference frontend is not part of the product path:
     polygrad_amd/plans/gpt2_small_bf16_b1_t1024.polyplan   the same graph for one sequence (parity slice)
     polygrad_amd/plans/rowops_f32_8192.polyplan            config 2 (fused chain + row ops), 8192x8192 fp32
     polygrad_amd/plans/matmul_bf16_<m>x<n>x<k>[_bt].polyplan   config 3 shapes
+    polygrad_amd/plans/attention_bf16_b8_h12_t1024_d64.polyplan   the attention block of config 4 alone
 
 The graphs are built with the REAL reference frontend and scheduler
 (oracle/_ref/libpolygrad.so through tests/refpoly.py); only the scheduled kernel
@@ -60,6 +61,10 @@ def main():
         _, _, _, sink = graphs.matmul_bf16(c, m, n, k, transposed_b=tb)
         save(c, sink, f"matmul_bf16_{m}x{n}x{k}" + ("_bt" if tb else ""))
         c.close()
+    c = R.Ctx()
+    _, sink = graphs.attention_bf16(c, batch=8, heads=12, ctx=1024, hd=64)
+    save(c, sink, "attention_bf16_b8_h12_t1024_d64")
+    c.close()
     c = R.Ctx()
     _, _, _, sink = graphs.matmul_bf16(c, 1024, 1024, 1024, batch=16)
     save(c, sink, "matmul_bf16_b16_1024x1024x1024")

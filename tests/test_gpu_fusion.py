@@ -1,0 +1,58 @@
+"""Plan-level fusion on the GPU: the attention kernel group (scores, scale + mask,
+row max, row sum, normalise, weighted sum of values) run as one launch must give
+what the separately launched kernels give, and what the reference CPU backend gives."""
+import os
+
+import numpy as np
+import pytest
+
+import graphs
+import refpoly as R
+from hipharness import assert_close, run_hip, run_ref
+
+pytestmark = pytest.mark.gpu
+
+
+def small_gpt2(seed, qk_gain):
+    """Two layers, two heads of 64 features, 256 positions: the smallest shape the fused
+    kernel takes (128-query blocks, 64-key steps).  The q/k/v projection weights are
+    scaled up so that the softmax is far from uniform."""
+    cfg = graphs.GPT2Config(n_layer=2, n_head=2, d_model=128, vocab=211, ctx=256, batch=2)
+    c = R.Ctx()
+    sink, bufs = graphs.gpt2_forward(c, cfg, R.BF16)
+    arrays = graphs.gpt2_inputs(cfg, bufs, seed=seed, wdt=R.BF16)
+    for name, t in bufs.items():
+        if name.endswith("attn.c_attn.weight"):
+            w = R.bf16_bits_to_f32(arrays[t]) * qk_gain
+            arrays[t] = R.f32_to_bf16_bits(w.astype(np.float32))
+    return c, cfg, sink, bufs, arrays
+
+
+def logits(arrays_out, bufs):
+    return R.bf16_bits_to_f32(arrays_out[bufs["output"]]).astype(np.float64)
+
+
+@pytest.mark.parametrize("qk_gain", [1.0, 12.0])
+def test_fused_attention_matches_unfused_and_reference(qk_gain):
+    c, cfg, sink, bufs, arrays = small_gpt2(seed=11, qk_gain=qk_gain)
+    want = logits(run_ref(c, sink, arrays), bufs)
+    got, info = run_hip(c, sink, arrays)
+    assert sum(k["klass"] == "attention-mfma" for k in info) == cfg.n_layer, [k["klass"] for k in info]
+    os.environ["POLY_HIP_NO_FUSION"] = "1"
+    try:
+        plain, info_plain = run_hip(c, sink, arrays)
+    finally:
+        del os.environ["POLY_HIP_NO_FUSION"]
+    c.close()
+    assert not any(k["klass"] == "attention-mfma" for k in info_plain)
+    assert len(info_plain) == len(info) + 5 * cfg.n_layer      # six kernels became one, per layer
+    h, p = logits(got, bufs), logits(plain, bufs)
+    scale = float(np.abs(want).max())
+    assert np.isfinite(h).all()
+    # same expressions per element; only the order of the fp32 sums differs
+    assert_close(h, p, rtol=2e-2, atol=2e-2 * scale, what="fused vs separately launched kernels")
+    assert float(np.mean(h != p)) < 0.05, "bf16 logits should rarely differ at all"
+    assert_close(h, want, rtol=2e-2, atol=2e-2 * scale, what="fused vs reference CPU backend")
+    e_fused = float(np.sqrt(np.mean((h - want) ** 2)))
+    e_plain = float(np.sqrt(np.mean((p - want) ** 2)))
+    assert e_fused <= 1.5 * e_plain + 1e-6 * scale, (e_fused, e_plain)
