@@ -132,7 +132,195 @@ std::string params_decl(const KernelGraph &g) {
   return d;
 }
 
+// `item` as a pointwise consumer of buffer `cur` (written at `prod` in master coordinates):
+// maps its ranges, replaces its loads of `cur` by `value_name`, and checks that it stores
+// its own result at the very same index into a buffer of the same size.
+bool pointwise_member(const Sched &sc, int item, int cur, const Aff &prod, const std::vector<int64_t> &mext,
+                      const char *value_name, Member *m) {
+  const PolySchedule *s = sc.s;
+  const KernelGraph &g = sc.graphs[(size_t)item];
+  if (!g.reduces.empty() || g.stores.size() != 1 || g.stores[0].gate >= 0 || !g.vars.empty()) return false;
+  std::vector<LoadRef> lds;
+  const int p = sc.param_of(item, cur);
+  if (p < 0 || !loads_of(g, p, &lds) || lds.empty()) return false;
+  m->item = item;
+  for (const LoadRef &l : lds) {
+    if (!derive_map(g, g.lins[(size_t)l.lin], prod, mext, &m->rm)) return false;
+    m->preset[l.node] = value_name;
+  }
+  for (int r : g.stores[0].ranges) if (!m->rm.count(r)) return false;
+  const int li = g.n(g.n(g.stores[0].index).src[1]).lin;
+  Aff a;
+  if (li < 0 || !lin_to_aff(g, g.lins[(size_t)li], m->rm, &a) || !(a == prod)) return false;
+  const int outp = g.param_slot(g.stores[0].param);
+  if (outp == p || s->buf_slots[sc.slot(item, outp)].numel != s->buf_slots[cur].numel) return false;
+  return true;
+}
+
+// Emits "__device__ ret name(lead_args, int m, int n, int z, <params of the member's kernel>)"
+// returning the value of `node`, with the member's ranges bound to the master ranges
+// r<ord> that `master_decomp` declares, and its presets applied.  When store_param >= 0
+// the function instead stores the value at the kernel's own store index and returns void.
+bool emit_member_fn(const Sched &sc, const Member &m, const std::string &master_decomp, const char *name, const char *ret,
+                    const std::string &lead_args, int node, const std::map<int, std::string> &extra_preset, bool raw_exp2,
+                    bool as_store, std::string *code) {
+  const KernelGraph &g = sc.graphs[(size_t)m.item];
+  Emitter em(g);
+  em.raw_exp2 = raw_exp2;
+  Scope S0;
+  S0.indent = 1;
+  for (auto &kv : m.rm) { em.bind_range(kv.first, strf("r%d", kv.second)); S0.avail |= (uint64_t)1 << kv.first; }
+  for (auto &kv : m.preset) em.preset(kv.first, kv.second);
+  for (auto &kv : extra_preset) em.preset(kv.first, kv.second);
+  std::string v = em.emit(node, &S0);
+  std::string idx;
+  if (as_store) idx = em.emit(g.n(g.stores[0].index).src[1], &S0);
+  if (em.failed() || em.uses_threefry) return false;
+  *code += strf("__device__ __forceinline__ %s %s(%s, int m, int n, int z, %s) {\n", as_store ? "void" : ret, name, lead_args.c_str(),
+                params_decl(g).c_str());
+  *code += master_decomp + S0.code;
+  if (as_store) *code += strf("  data%d[%s] = %s;\n}\n", g.param_slot(g.stores[0].param), idx.c_str(), v.c_str());
+  else *code += strf("  return %s;\n}\n", v.c_str());
+  return true;
+}
+
+// Checks that running the group's kernels at the place of its last one changes nothing:
+// all members lie between the first and the last in execution order, nobody else writes
+// an input after the member that read it, and nobody else touches the output in between.
+bool group_is_schedulable(const Sched &sc, const std::vector<int> &items, int first_item, int last_item,
+                          const std::set<int> &internal, int out_slot, std::set<int> *inputs) {
+  const PolySchedule *s = sc.s;
+  const int first_step = sc.step_of[(size_t)first_item], last_step = sc.step_of[(size_t)last_item];
+  std::set<int> uniq(items.begin(), items.end());
+  if (uniq.size() != items.size()) return false;
+  for (int it : items) if (sc.step_of[(size_t)it] < first_step || sc.step_of[(size_t)it] > last_step) return false;
+  std::map<int, int> first_read;   // input slot -> earliest original step of a member reading it
+  for (int it : items) {
+    const PolyExecItem &e = s->items[it];
+    for (int i = 0; i < e.n_buf_slots; i++) {
+      const int sl = e.buf_slot_indices[i];
+      if (internal.count(sl) || sl == out_slot) continue;
+      if (sc.graphs[(size_t)it].params[(size_t)i].written) return false;
+      inputs->insert(sl);
+      const int st = sc.step_of[(size_t)it];
+      if (!first_read.count(sl) || st < first_read[sl]) first_read[sl] = st;
+    }
+  }
+  for (int sl : *inputs)
+    for (int w : sc.writers[(size_t)sl])
+      if (sc.step_of[(size_t)w] >= first_read[sl] && sc.step_of[(size_t)w] <= last_step) return false;
+  for (int w : sc.writers[(size_t)out_slot]) if (w != last_item && sc.step_of[(size_t)w] >= first_step && sc.step_of[(size_t)w] <= last_step) return false;
+  for (int r : sc.readers[(size_t)out_slot]) if (r != last_item && sc.step_of[(size_t)r] >= first_step && sc.step_of[(size_t)r] <= last_step) return false;
+  if (internal.count(out_slot) || inputs->count(out_slot)) return false;
+  return true;
+}
+
+// Every LOAD of an internal buffer in a member must have been replaced by a value
+// (`exempt`: a load the template performs itself).
+bool internal_loads_replaced(const Sched &sc, const Member &m, const std::set<int> &internal, int exempt) {
+  const KernelGraph &g = sc.graphs[(size_t)m.item];
+  for (int id = 0; id < (int)g.nodes.size(); id++) {
+    if (g.n(id).op != POLY_OP_LOAD) continue;
+    const int p = g.param_slot(g.n(g.n(id).src[0]).src[0]);
+    if (!internal.count(sc.slot(m.item, p))) continue;
+    if (!m.preset.count(id) && id != exempt) return false;
+  }
+  return true;
+}
+
 }  // namespace
+
+// A matmul whose result only feeds a chain of pointwise kernels (bias/activation/residual
+// realised as kernels of their own): the chain becomes the matmul's epilogue.
+static bool match_matmul_tail(const Sched &sc, int s_item, const std::vector<char> &taken, FusedGroup *out) {
+  const PolySchedule *s = sc.s;
+  const KernelGraph &gS = sc.graphs[(size_t)s_item];
+  MatmulMatch mS;
+  if (!match_matmul(gS, &mS, nullptr)) return false;
+  const StoreInfo &stS = gS.stores[0];
+  std::vector<int64_t> mext(gS.ranges.size());
+  for (size_t i = 0; i < gS.ranges.size(); i++) mext[i] = gS.ranges[i].extent;
+  RangeMap idS;
+  for (int r : stS.ranges) idS[r] = r;
+  const int lsi = gS.n(gS.n(stS.index).src[1]).lin;
+  Aff aS;
+  if (lsi < 0 || !lin_to_aff(gS, gS.lins[(size_t)lsi], idS, &aS) || aS.c.size() != stS.ranges.size()) return false;
+
+  std::vector<Member> members;
+  { Member m; m.item = s_item; m.rm = idS; members.push_back(m); }
+  std::set<int> internal;
+  int cur = sc.slot(s_item, gS.param_slot(stS.param));
+  while (members.size() < 4) {
+    if (!s->buf_slots[cur].is_intermediate || sc.writers[(size_t)cur].size() != 1 || sc.readers[(size_t)cur].size() != 1) break;
+    const int r = sc.readers[(size_t)cur][0];
+    Member m;
+    if (taken[(size_t)r] || !pointwise_member(sc, r, cur, aS, mext, "x", &m)) break;
+    internal.insert(cur);
+    members.push_back(m);
+    const KernelGraph &g = sc.graphs[(size_t)r];
+    cur = sc.slot(r, g.param_slot(g.stores[0].param));
+  }
+  if (members.size() < 2) return false;
+  const int out_slot = cur, last_item = members.back().item;
+  std::vector<int> items;
+  for (const Member &m : members) items.push_back(m.item);
+  std::set<int> inputs;
+  if (!group_is_schedulable(sc, items, s_item, last_item, internal, out_slot, &inputs)) FA_REJECT();
+  for (const Member &m : members) if (!internal_loads_replaced(sc, m, internal, -1)) FA_REJECT();
+
+  std::vector<int> arg_slots;
+  arg_slots.push_back(out_slot);
+  for (int sl : inputs) arg_slots.push_back(sl);
+  auto arg_of = [&](int sl) { return (int)(std::find(arg_slots.begin(), arg_slots.end(), sl) - arg_slots.begin()); };
+  auto call_args = [&](int item) {
+    const KernelGraph &g = sc.graphs[(size_t)item];
+    std::string c;
+    for (size_t i = 0; i < g.params.size(); i++) {
+      const int sl = sc.slot(item, (int)i);
+      if (i) c += ", ";
+      if (internal.count(sl)) c += strf("(%s%s*)0", g.params[i].written ? "" : "const ", dt_cname(g.params[i].dt));
+      else c += strf("fa%d", arg_of(sl));
+    }
+    return c;
+  };
+  MatmulEpilogue ep;
+  for (size_t j = 0; j < arg_slots.size(); j++) {
+    DT dt = DT_VOID;
+    for (int it : items) {
+      const int p = sc.param_of(it, arg_slots[j]);
+      if (p >= 0) dt = sc.graphs[(size_t)it].params[(size_t)p].dt;
+    }
+    if (j) ep.signature += ", ";
+    ep.signature += j == 0 ? strf("%s* fa%zu", dt_cname(dt), j) : strf("const %s* __restrict__ fa%zu", dt_cname(dt), j);
+    ep.bytes += (double)s->buf_slots[arg_slots[j]].nbytes;
+  }
+  const std::string master_decomp = matmul_decompose(mS, nullptr);
+  if (!emit_member_fn(sc, members[0], master_decomp, "poly_ep_s", dt_cname(gS.n(stS.value).dt), "float acc", stS.value,
+                      {{mS.red, "acc"}}, false, false, &ep.code)) FA_REJECT();
+  std::string call = strf("poly_ep_s(acc, m, n, z, %s)", call_args(s_item).c_str());
+  DT prev_dt = gS.n(stS.value).dt;
+  for (size_t e = 1; e < members.size(); e++) {
+    const Member &m = members[e];
+    const KernelGraph &g = sc.graphs[(size_t)m.item];
+    const bool last = e + 1 == members.size();
+    const std::string fn = strf("poly_ep_e%zu", e);
+    if (!emit_member_fn(sc, m, master_decomp, fn.c_str(), dt_cname(g.n(g.stores[0].value).dt), strf("%s x", dt_cname(prev_dt)),
+                        g.stores[0].value, {}, false, last, &ep.code)) FA_REJECT();
+    call = strf("%s(%s, m, n, z, %s)", fn.c_str(), call.c_str(), call_args(m.item).c_str());
+    prev_dt = g.n(g.stores[0].value).dt;
+  }
+  ep.call = call;
+  ep.a_ptr = strf("fa%d", arg_of(sc.slot(s_item, mS.A.param)));
+  ep.b_ptr = strf("fa%d", arg_of(sc.slot(s_item, mS.B.param)));
+  ep.n_params = (int)arg_slots.size();
+  if (!render_matmul(mS, ep, &out->rk)) return false;
+  out->rk.strategy += strf(" + %zu pointwise kernel%s in the epilogue", members.size() - 1, members.size() > 2 ? "s" : "");
+  out->items = items;
+  out->launch_item = last_item;
+  out->internal_slots.assign(internal.begin(), internal.end());
+  out->arg_slots = arg_slots;
+  return true;
+}
 
 // Tries to grow an attention group from the matmul at schedule item `s_item`.
 static bool match_attention(const Sched &sc, int s_item, const std::vector<char> &taken, FusedGroup *out) {
@@ -563,7 +751,7 @@ void find_fused_groups(const PolySchedule *s, const std::vector<KernelGraph> &gr
     const int k = s->exec_order[st];
     if (taken[(size_t)k] || graphs[(size_t)k].reduces.size() != 1) continue;
     FusedGroup fg;
-    if (!match_attention(sc, k, taken, &fg)) continue;
+    if (!match_attention(sc, k, taken, &fg) && !match_matmul_tail(sc, k, taken, &fg)) continue;
     for (int it : fg.items) taken[(size_t)it] = 1;
     out->push_back(std::move(fg));
   }

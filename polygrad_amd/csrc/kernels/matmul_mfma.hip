@@ -56,6 +56,7 @@ typedef float poly_acc16 __attribute__((ext_vector_type(16)));
 typedef unsigned int poly_u32x4 __attribute__((ext_vector_type(4)));
 typedef unsigned int poly_u32x2 __attribute__((ext_vector_type(2)));
 typedef poly_u32x4 poly_u32x4_u __attribute__((aligned(2)));
+typedef float poly_f32x4 __attribute__((ext_vector_type(4)));
 
 #define POLY_WM (POLY_BM / POLY_WAVES_M)
 #define POLY_WN (POLY_BN / POLY_WAVES_N)
@@ -70,6 +71,9 @@ typedef poly_u32x4 poly_u32x4_u __attribute__((aligned(2)));
 #define POLY_NCOL (POLY_BK / 8)
 __device__ __forceinline__ int poly_swz(int row) { return (row ^ (row >> 3)) & (POLY_NCOL - 1); }
 #define POLY_KT (POLY_K / POLY_BK)
+// row pitch (floats) of the 32x32 output staging tile: 16-byte aligned rows, and rows 4
+// apart (the two halves of a wave) land on different banks
+#define POLY_STAGE_LD 36
 
 // Number of 16-byte global loads per thread for one operand tile.
 #define POLY_A_LOADS ((POLY_BM * POLY_BK / 8) / POLY_NTHREADS)
@@ -144,8 +148,10 @@ struct PolyXC {
 };
 
 extern "C" __global__ void __launch_bounds__(POLY_NTHREADS) poly_k(POLY_SIGNATURE) {
-  __shared__ __attribute__((aligned(16))) POLY_TIN lds_a[2][POLY_BM * POLY_LDK];
-  __shared__ __attribute__((aligned(16))) POLY_TIN lds_b[2][POLY_BN * POLY_LDK];
+  // one allocation: the operand tiles during the K loop, the per-wave output staging after it
+  __shared__ __attribute__((aligned(16))) POLY_TIN lds_raw[2 * (POLY_BM + POLY_BN) * POLY_LDK];
+  auto lds_a = [&](int buf) { return lds_raw + buf * (POLY_BM * POLY_LDK); };
+  auto lds_b = [&](int buf) { return lds_raw + 2 * POLY_BM * POLY_LDK + buf * (POLY_BN * POLY_LDK); };
 
   // Tile coordinates.  Consecutive workgroup ids go to different XCDs (8 of them,
   // each with its own L2), so ids are regrouped: all ids congruent mod 8 form one
@@ -273,9 +279,9 @@ extern "C" __global__ void __launch_bounds__(POLY_NTHREADS) poly_k(POLY_SIGNATUR
   poly_in8 fa[2][POLY_TM], fb[2][POLY_TN];
   auto read_frags = [&](int cur, int ks, int buf) {
 #pragma unroll
-    for (int i = 0; i < POLY_TM; i++) fa[buf][i] = *(const poly_in8 *)(lds_a[cur] + a_row_off[i] + (((ks * 2 + frag_col) ^ a_swz[i]) * 8));
+    for (int i = 0; i < POLY_TM; i++) fa[buf][i] = *(const poly_in8 *)(lds_a(cur) + a_row_off[i] + (((ks * 2 + frag_col) ^ a_swz[i]) * 8));
 #pragma unroll
-    for (int j = 0; j < POLY_TN; j++) fb[buf][j] = *(const poly_in8 *)(lds_b[cur] + b_row_off[j] + (((ks * 2 + frag_col) ^ b_swz[j]) * 8));
+    for (int j = 0; j < POLY_TN; j++) fb[buf][j] = *(const poly_in8 *)(lds_b(cur) + b_row_off[j] + (((ks * 2 + frag_col) ^ b_swz[j]) * 8));
   };
   auto compute = [&](int cur, int ks_begin, int ks_end) {
     read_frags(cur, ks_begin, ks_begin & 1);
@@ -298,8 +304,8 @@ extern "C" __global__ void __launch_bounds__(POLY_NTHREADS) poly_k(POLY_SIGNATUR
   // is free.  Every global load has about two and a half iterations to land.
   // Tile t always uses register set t & 1, hence the loop is unrolled by two.
   load_tiles(0, ra0, rb0);
-  StageA::store(lds_a[0], ra0);
-  StageB::store(lds_b[0], rb0);
+  StageA::store(lds_a(0), ra0);
+  StageB::store(lds_b(0), rb0);
   if (POLY_KT > 1) load_tiles(1, ra1, rb1);
   if (POLY_KT > 2) load_tiles(2, ra0, rb0);
   __syncthreads();
@@ -309,8 +315,8 @@ extern "C" __global__ void __launch_bounds__(POLY_NTHREADS) poly_k(POLY_SIGNATUR
     compute(cur, 0, KS_HALF);
     __builtin_amdgcn_sched_barrier(0);
     if (kt + 1 < POLY_KT) {
-      StageA::store(lds_a[cur ^ 1], ra_next);
-      StageB::store(lds_b[cur ^ 1], rb_next);
+      StageA::store(lds_a(cur ^ 1), ra_next);
+      StageB::store(lds_b(cur ^ 1), rb_next);
     }
     if (kt + 3 < POLY_KT) load_tiles(kt + 3, ra_next, rb_next);
     __builtin_amdgcn_sched_barrier(0);
@@ -327,8 +333,8 @@ extern "C" __global__ void __launch_bounds__(POLY_NTHREADS) poly_k(POLY_SIGNATUR
   // before the first half of tile kt is multiplied, and land in the other LDS
   // buffer between the two halves.
   load_tiles(0, ra0, rb0);
-  StageA::store(lds_a[0], ra0);
-  StageB::store(lds_b[0], rb0);
+  StageA::store(lds_a(0), ra0);
+  StageB::store(lds_b(0), rb0);
   __syncthreads();
   for (int kt = 0; kt < POLY_KT; kt++) {
     const int cur = kt & 1;
@@ -337,8 +343,8 @@ extern "C" __global__ void __launch_bounds__(POLY_NTHREADS) poly_k(POLY_SIGNATUR
     compute(cur, 0, KS_HALF);
     __builtin_amdgcn_sched_barrier(0);
     if (kt + 1 < POLY_KT) {
-      StageA::store(lds_a[cur ^ 1], ra0);
-      StageB::store(lds_b[cur ^ 1], rb0);
+      StageA::store(lds_a(cur ^ 1), ra0);
+      StageB::store(lds_b(cur ^ 1), rb0);
     }
     __builtin_amdgcn_sched_barrier(0);
     compute(cur, KS_HALF, KS);
@@ -347,7 +353,14 @@ extern "C" __global__ void __launch_bounds__(POLY_NTHREADS) poly_k(POLY_SIGNATUR
 #endif
 
   // Accumulator layout of the 32x32 MFMA: register r of lane l holds
-  // row 8*(r/4) + 4*(l/32) + r%4, column l%32 of the tile.
+  // row 8*(r/4) + 4*(l/32) + r%4, column l%32 of the tile: a lane owns one column, so
+  // its stores would be single elements.  Each 32x32 tile therefore goes through a
+  // per-wave LDS staging area and comes back with 8 consecutive columns of one row per
+  // lane, so that whatever the epilogue loads and stores along n is 16 bytes wide (for
+  // 16-bit data) and a wave writes full 64-byte row segments.
+#if POLY_N % 8 != 0
+  // Rows of the output do not start on 16-byte boundaries: store straight from the
+  // accumulator layout, where the 32 lanes of a half-wave write 32 consecutive columns.
 #pragma unroll
   for (int i = 0; i < POLY_TM; i++)
 #pragma unroll
@@ -359,4 +372,37 @@ extern "C" __global__ void __launch_bounds__(POLY_NTHREADS) poly_k(POLY_SIGNATUR
         if (m < POLY_M && n < POLY_N) { POLY_EPILOGUE(acc[i][j][r], m, n, z); }
       }
     }
+#else
+  static_assert(POLY_NTHREADS / 64 * 32 * POLY_STAGE_LD * 4 <= (int)sizeof(lds_raw), "staging area exceeds the operand tiles");
+  __syncthreads();   // every wave is done reading the operand tiles
+  float *const stage = (float *)lds_raw + wave * (32 * POLY_STAGE_LD);
+#pragma unroll
+  for (int i = 0; i < POLY_TM; i++)
+#pragma unroll
+    for (int j = 0; j < POLY_TN; j++) {
+#pragma unroll
+      for (int r = 0; r < 16; r++)
+        stage[(8 * (r >> 2) + 4 * (lane >> 5) + (r & 3)) * POLY_STAGE_LD + (lane & 31)] = acc[i][j][r];
+      // LDS operations of one wave complete in order; the fences only keep the compiler
+      // from moving the reads above the writes (and the next tile's writes above the reads)
+      __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+      __builtin_amdgcn_wave_barrier();
+      __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+#pragma unroll
+      for (int h = 0; h < 2; h++) {
+        const int row = (lane >> 2) + 16 * h, c0 = (lane & 3) * 8;
+        const poly_f32x4 lo = *(const poly_f32x4 *)(stage + row * POLY_STAGE_LD + c0);
+        const poly_f32x4 hi = *(const poly_f32x4 *)(stage + row * POLY_STAGE_LD + c0 + 4);
+        const float v[8] = {lo[0], lo[1], lo[2], lo[3], hi[0], hi[1], hi[2], hi[3]};
+        const int m = m0 + wm + i * 32 + row, n = n0 + wn + j * 32 + c0;
+        if (m < POLY_M && n < POLY_N) {
+#pragma unroll
+          for (int e = 0; e < 8; e++) { POLY_EPILOGUE(v[e], m, n + e, z); }
+        }
+      }
+      __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+      __builtin_amdgcn_wave_barrier();
+      __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+    }
+#endif
 }

@@ -269,8 +269,46 @@ bool try_render_matmul(const KernelGraph &g, const std::string &fn, const Render
   MatmulMatch mm;
   int line = 0;
   if (!match_matmul(g, &mm, &line)) return reject(line);
+  // epilogue: everything outside the REDUCE, per output element
   const StoreInfo &st = g.stores[0];
-  const int red = mm.red;
+  Emitter em(g);
+  Scope S0;
+  S0.indent = 1;
+  for (int r : st.ranges) S0.avail |= (uint64_t)1 << r;
+  std::string decomp = matmul_decompose(mm, &em);
+  em.preset(mm.red, "acc");
+  std::string val = em.emit(st.value, &S0);
+  std::string idx = em.emit(g.n(st.index).src[1], &S0);
+  if (em.failed()) return reject(__LINE__);
+  const int pout = g.param_slot(st.param);
+  MatmulEpilogue ep;
+  std::string params_call;
+  for (size_t i = 0; i < g.params.size(); i++) {
+    const ParamInfo &p = g.params[i];
+    if (i) { ep.signature += ", "; params_call += ", "; }
+    if (p.written) ep.signature += strf("%s* data%zu", dt_cname(p.dt), i);
+    else ep.signature += strf("const %s* __restrict__ data%zu", dt_cname(p.dt), i);
+    params_call += strf("data%zu", i);
+  }
+  ep.code = strf("__device__ __forceinline__ void poly_epilogue(float acc, int m, int n, int z, %s) {\n", ep.signature.c_str());
+  ep.code += decomp + S0.code;
+  ep.code += strf("  data%d[%s] = %s;\n}\n", pout, idx.c_str(), val.c_str());
+  ep.call = strf("poly_epilogue(acc, m, n, z, %s)", params_call.c_str());
+  ep.a_ptr = strf("data%d", mm.A.param);
+  ep.b_ptr = strf("data%d", mm.B.param);
+  ep.n_params = (int)g.params.size();
+  // distinct elements: A, B once each (broadcast operands counted once), output once,
+  // plus whatever the epilogue reads per output row/column
+  for (size_t i = 0; i < g.params.size(); i++) {
+    const ParamInfo &p = g.params[i];
+    double n = (double)std::max<int64_t>(p.numel, 0);
+    if ((int)i == pout) n = (double)mm.M * mm.N * mm.Z;
+    ep.bytes += n * dt_size(p.dt);
+  }
+  return render_matmul(mm, ep, out);
+}
+
+bool render_matmul(const MatmulMatch &mm, const MatmulEpilogue &ep, RenderedKernel *out) {
   const int64_t K = mm.K, M = mm.M, N = mm.N, Z = mm.Z;
   const Operand &A = mm.A, &B = mm.B;
   const KSplit &ka = mm.ka, &kb = mm.kb;
@@ -314,29 +352,6 @@ bool try_render_matmul(const KernelGraph &g, const std::string &fn, const Render
   const int64_t tiles = ((M + BM - 1) / BM) * ((N + BN - 1) / BN);
   if (tiles > 2147483647LL / 2) return reject(__LINE__);
 
-  // ── epilogue: everything outside the REDUCE, per output element ──────────
-  Emitter em(g);
-  Scope S0;
-  S0.indent = 1;
-  for (int r : st.ranges) S0.avail |= (uint64_t)1 << r;
-  std::string decomp = matmul_decompose(mm, &em);
-  em.preset(red, "acc");
-  std::string val = em.emit(st.value, &S0);
-  std::string idx = em.emit(g.n(st.index).src[1], &S0);
-  if (em.failed()) return reject(__LINE__);
-  const int pout = g.param_slot(st.param);
-  std::string params_decl, params_call;
-  for (size_t i = 0; i < g.params.size(); i++) {
-    const ParamInfo &p = g.params[i];
-    if (i) { params_decl += ", "; params_call += ", "; }
-    if (p.written) params_decl += strf("%s* data%zu", dt_cname(p.dt), i);
-    else params_decl += strf("const %s* __restrict__ data%zu", dt_cname(p.dt), i);
-    params_call += strf("data%zu", i);
-  }
-  std::string epi = strf("__device__ __forceinline__ void poly_epilogue(float acc, int m, int n, int z, %s) {\n", params_decl.c_str());
-  epi += decomp + S0.code;
-  epi += strf("  data%d[%s] = %s;\n}\n", pout, idx.c_str(), val.c_str());
-
   // ── configuration block ───────────────────────────────────────────────────
   std::string cfg;
   cfg += strf("#define POLY_TIN %s\n", dt_cname(A.dt));
@@ -350,7 +365,7 @@ bool try_render_matmul(const KernelGraph &g, const std::string &fn, const Render
   if (const char *e = getenv("POLY_HIP_MM_PIPE")) pipe = atoi(e) == 2 ? 2 : 3;
   cfg += strf("#define POLY_PIPE %d\n", pipe);
   cfg += strf("#define POLY_A_KC %d\n#define POLY_B_KC %d\n", a_kc ? 1 : 0, b_kc ? 1 : 0);
-  cfg += strf("#define POLY_A_PTR data%d\n#define POLY_B_PTR data%d\n", A.param, B.param);
+  cfg += strf("#define POLY_A_PTR %s\n#define POLY_B_PTR %s\n", ep.a_ptr.c_str(), ep.b_ptr.c_str());
   cfg += offset_fn("poly_a_row", md, true, 0);
   cfg += offset_fn("poly_b_row", nd, false, 0);
   if (zd.empty()) {
@@ -362,9 +377,11 @@ bool try_render_matmul(const KernelGraph &g, const std::string &fn, const Render
   }
   cfg += matmul_k_fn("poly_a_k", ka, K);
   cfg += matmul_k_fn("poly_b_k", kb, K);
-  cfg += strf("#define POLY_SIGNATURE %s\n", params_decl.c_str());
-  cfg += epi;
-  cfg += strf("#define POLY_EPILOGUE(acc, m, n, z) poly_epilogue(acc, m, n, z, %s)\n", params_call.c_str());
+  cfg += strf("#define POLY_SIGNATURE %s\n", ep.signature.c_str());
+  cfg += ep.code;
+  if (getenv("POLY_HIP_MM_NOEPI")) cfg += strf("#define POLY_EPILOGUE(acc, m, n, z) do { if (((m) | (n)) == -1) { %s; } } while (0)\n", ep.call.c_str());
+  else
+  cfg += strf("#define POLY_EPILOGUE(acc, m, n, z) %s\n", ep.call.c_str());
 
   *out = RenderedKernel();
   out->source = std::string(hip_prelude()) + cfg + kMatmulTemplate;
@@ -376,19 +393,10 @@ bool try_render_matmul(const KernelGraph &g, const std::string &fn, const Render
   out->strategy = strf("mfma 32x32x16 %s M=%lld N=%lld K=%lld Z=%lld tile %dx%dx%d A:%s B:%s", A.dt == DT_BF16 ? "bf16" : "f16",
                        (long long)M, (long long)N, (long long)K, (long long)Z, BM, BN, BK, a_kc ? "k-major" : "m-major",
                        b_kc ? "k-major" : "n-major");
-  out->n_params = (int)g.params.size();
+  out->n_params = ep.n_params;
   out->n_vars = 0;
   out->flops = 2.0 * (double)M * (double)N * (double)K * (double)Z;
-  // distinct elements: A, B once each (broadcast operands counted once), output once,
-  // plus whatever the epilogue reads per output row/column
-  double bytes = 0;
-  for (size_t i = 0; i < g.params.size(); i++) {
-    const ParamInfo &p = g.params[i];
-    double n = (double)std::max<int64_t>(p.numel, 0);
-    if ((int)i == pout) n = (double)M * N * Z;
-    bytes += n * dt_size(p.dt);
-  }
-  out->bytes = bytes;
+  out->bytes = ep.bytes;
   return true;
 }
 
@@ -513,19 +521,25 @@ bool try_render_gather(const KernelGraph &g, const std::string &fn, const Render
 
   RenderedKernel::Guard gd;
   gd.entry = "poly_guard";
+  // one workgroup of 1024 threads, four consecutive elements per thread and step
   gd.source = strf(R"HIP(
-extern "C" __global__ void __launch_bounds__(256) poly_guard(int* flag, const %s* __restrict__ ar) {
+extern "C" __global__ void __launch_bounds__(1024) poly_guard(int* flag, const %s* __restrict__ ar) {
   __shared__ int bad;
   if (threadIdx.x == 0) bad = 0;
   __syncthreads();
-  for (int i = threadIdx.x; i < %lld; i += 256)
-    if (ar[i] != (%s)i) bad = 1;
+  int mine = 0;
+  for (long long i = (long long)threadIdx.x * 4; i < %lldll; i += 4096) {
+#pragma unroll
+    for (int j = 0; j < 4; j++)
+      if (i + j < %lldll && ar[i + j] != (%s)(i + j)) mine = 1;
+  }
+  if (mine) bad = 1;
   __syncthreads();
   if (threadIdx.x == 0) *flag = bad ? 0 : 1;
 }
-)HIP", dt_cname(AR.dt), (long long)V, dt_cname(AR.dt));
+)HIP", dt_cname(AR.dt), (long long)V, (long long)V, dt_cname(AR.dt));
   gd.launch.grid[0] = 1;
-  gd.launch.block[0] = 256;
+  gd.launch.block[0] = 1024;
   gd.arg_params.push_back(ar_param);
 
   *out = fk;

@@ -48,6 +48,17 @@ int64_t matmul_eval_offset(const std::vector<MmDim> &dims, bool use_a, int64_t x
 // value of END range `ord` at flattened coordinates (m, n, z)
 int64_t matmul_range_value(const MatmulMatch &mm, int ord, int64_t m, int64_t n, int64_t z);
 
+// What the MFMA template does with each accumulator: the kernel's signature, which of
+// its pointers are the operands, device functions, and the statement (in terms of acc, m,
+// n, z) that finishes one output element.
+struct MatmulEpilogue {
+  std::string signature, a_ptr, b_ptr, code, call;
+  int n_params = 0;
+  double bytes = 0;    // algorithmic bytes of the whole kernel
+};
+// Chooses layouts and tile shape and instantiates kernels/matmul_mfma.hip.
+bool render_matmul(const MatmulMatch &mm, const MatmulEpilogue &ep, RenderedKernel *out);
+
 bool try_render_matmul(const KernelGraph &g, const std::string &fn, const RenderOptions &opt, RenderedKernel *out);
 bool try_render_gather(const KernelGraph &g, const std::string &fn, const RenderOptions &opt, RenderedKernel *out);
 

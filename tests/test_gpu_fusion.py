@@ -1,6 +1,7 @@
 """Plan-level fusion on the GPU: the attention kernel group (scores, scale + mask,
-row max, row sum, normalise, weighted sum of values) run as one launch must give
-what the separately launched kernels give, and what the reference CPU backend gives."""
+row max, row sum, normalise, weighted sum of values) run as one launch, and pointwise
+kernels run as the epilogue of the matmul that feeds them, must give what the separately
+launched kernels give, and what the reference CPU backend gives."""
 import os
 
 import numpy as np
@@ -45,7 +46,10 @@ def test_fused_attention_matches_unfused_and_reference(qk_gain):
         del os.environ["POLY_HIP_NO_FUSION"]
     c.close()
     assert not any(k["klass"] == "attention-mfma" for k in info_plain)
-    assert len(info_plain) == len(info) + 5 * cfg.n_layer      # six kernels became one, per layer
+    # per layer: six attention kernels became one, and three pointwise kernels (attention
+    # residual, GELU, MLP residual) moved into the epilogue of the matmul in front of them
+    assert len(info_plain) == len(info) + (5 + 3) * cfg.n_layer
+    assert sum("in the epilogue" in k["desc"] for k in info) == 3 * cfg.n_layer
     h, p = logits(got, bufs), logits(plain, bufs)
     scale = float(np.abs(want).max())
     assert np.isfinite(h).all()

@@ -140,22 +140,34 @@ int main(void) {
     assert outs[0] == outs[1]
 
 
-def test_attention_groups_of_the_gpt2_plan_fuse_and_compile(hiplib):
-    """Needs no device: the plan compiler recognises one attention group per layer in the
-    benchmark schedule, each replacing six scheduled kernels, and its source compiles."""
+def test_kernel_groups_of_the_gpt2_plan_fuse_and_compile(hiplib):
+    """Needs no device: in the benchmark schedule the plan compiler recognises, per layer,
+    one attention group (six scheduled kernels) and three matmuls followed by a pointwise
+    kernel (residual add, GELU, residual add); the generated sources compile."""
     from polygrad_amd import PlanFile
     pf = PlanFile(os.path.join(ROOT, "polygrad_amd", "plans", "gpt2_small_bf16_b8_t1024.polyplan"))
-    src, n = C.c_void_p(), C.c_int()
-    count = hiplib.poly_hip_fused_groups(pf.schedule, 0, C.byref(src), C.byref(n))
-    assert count == 12 and n.value == 6
-    text = _ffi.take_string(src.value)
-    assert "poly_fa_term" in text and "__builtin_amdgcn_mfma_f32_32x32x16_bf16" in text
-    assert hiplib.poly_hip_compile_check(text.encode()) == 0
+    count = hiplib.poly_hip_fused_groups(pf.schedule, -1, None, None)
+    assert count == 48
+    seen = {}
+    for i in range(count):
+        src, n = C.c_void_p(), C.c_int()
+        hiplib.poly_hip_fused_groups(pf.schedule, i, C.byref(src), C.byref(n))
+        text = _ffi.take_string(src.value)
+        kind = "attention" if "POLY_FA_M" in text else "tail"
+        assert n.value == (6 if kind == "attention" else 2)
+        seen.setdefault(kind, []).append(text)
+    assert len(seen["attention"]) == 12 and len(seen["tail"]) == 36
+    att = seen["attention"][0]
+    assert "poly_fa_term" in att and "__builtin_amdgcn_mfma_f32_32x32x16_bf16" in att
+    assert hiplib.poly_hip_compile_check(att.encode()) == 0
+    for text in seen["tail"][:3]:      # one layer: attention residual, GELU, MLP residual
+        assert "poly_ep_e1" in text
+        assert hiplib.poly_hip_compile_check(text.encode()) == 0
     os.environ["POLY_HIP_NO_FUSION"] = "1"
     try:
         assert hiplib.poly_hip_fused_groups(pf.schedule, -1, None, None) == 0
     finally:
         del os.environ["POLY_HIP_NO_FUSION"]
-    # a plan without attention has nothing to fuse
+    # a plan without matmuls has nothing to fuse
     pf2 = PlanFile(os.path.join(ROOT, "polygrad_amd", "plans", "rowops_f32_8192_softmax.polyplan"))
     assert hiplib.poly_hip_fused_groups(pf2.schedule, -1, None, None) == 0
