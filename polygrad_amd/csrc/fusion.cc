@@ -17,6 +17,7 @@
 #include "fusion.h"
 
 #include <algorithm>
+#include <cmath>
 #include <cstdlib>
 #include <map>
 #include <set>
@@ -319,6 +320,357 @@ static bool match_matmul_tail(const Sched &sc, int s_item, const std::vector<cha
   out->launch_item = last_item;
   out->internal_slots.assign(internal.begin(), internal.end());
   out->arg_slots = arg_slots;
+  return true;
+}
+
+// ── row chains ──────────────────────────────────────────────────────────────
+//
+// LayerNorm and softmax reach the backend as three kernels (reference frontend:
+// src/frontend.c:3585-3625 and :1131-1159): a row reduction, a second row reduction that
+// reads the first one's result, and a pointwise kernel that reads both.  All three walk
+// the same rows, so one wave (or one workgroup for long rows) can run the three of them
+// back to back for its row: the statistics stay in registers and the row is read from
+// HBM once (the second and third reads hit cache).  Each phase is generated from its
+// own kernel's graph; only the row structure is matched.
+
+struct RowPhase {
+  Member m;
+  bool is_map = false;
+  int red = -1, own_red_ord = -1;   // REDUCE node and its range ordinal (reduce phases)
+};
+
+// Maps the ranges of `item` onto master ranges through the buffers it shares with the
+// phases before it: results of earlier phases (read at the row they were stored at) and
+// inputs that an earlier phase read as well.
+static bool map_phase(const Sched &sc, int item, const std::vector<int64_t> &mext,
+                      const std::vector<std::pair<int, Aff>> &ref_loads,       // (slot, index) of earlier loads
+                      const std::vector<std::pair<int, Aff>> &results,         // (slot, store index) of earlier results
+                      const std::vector<std::string> &result_names, Member *m) {
+  const KernelGraph &g = sc.graphs[(size_t)item];
+  m->item = item;
+  for (int id = 0; id < (int)g.nodes.size(); id++) {
+    const KNode &k = g.n(id);
+    if (k.op != POLY_OP_LOAD) continue;
+    const KNode &ix = g.n(k.src[0]);
+    const int sl = sc.slot(item, g.param_slot(ix.src[0]));
+    const int lin = g.n(ix.src[1]).lin;
+    bool is_result = false;
+    for (size_t r = 0; r < results.size(); r++) {
+      if (results[r].first != sl) continue;
+      is_result = true;
+      if (ix.src.size() != 2 || k.guard >= 0 || lin < 0) return false;
+      if (!derive_map(g, g.lins[(size_t)lin], results[r].second, mext, &m->rm)) return false;
+      m->preset[id] = result_names[r];
+    }
+    if (is_result || lin < 0) continue;
+    for (const auto &ref : ref_loads) {
+      if (ref.first != sl) continue;
+      RangeMap trial = m->rm;
+      if (derive_map(g, g.lins[(size_t)lin], ref.second, mext, &trial)) { m->rm = trial; break; }
+    }
+  }
+  return true;
+}
+
+static void collect_ref_loads(const Sched &sc, const Member &m, std::vector<std::pair<int, Aff>> *out) {
+  const KernelGraph &g = sc.graphs[(size_t)m.item];
+  for (int id = 0; id < (int)g.nodes.size(); id++) {
+    const KNode &k = g.n(id);
+    if (k.op != POLY_OP_LOAD || m.preset.count(id)) continue;
+    const KNode &ix = g.n(k.src[0]);
+    const int lin = g.n(ix.src[1]).lin;
+    Aff a;
+    if (lin < 0 || !lin_to_aff(g, g.lins[(size_t)lin], m.rm, &a)) continue;
+    out->push_back({sc.slot(m.item, g.param_slot(ix.src[0])), a});
+  }
+}
+
+static bool match_row_chain(const Sched &sc, int a_item, const std::vector<char> &taken, FusedGroup *out) {
+  const PolySchedule *s = sc.s;
+  const KernelGraph &gA = sc.graphs[(size_t)a_item];
+  auto reduce_shape = [&](const KernelGraph &g, int *red, int *ord) {
+    if (g.reduces.size() != 1 || g.stores.size() != 1 || g.stores[0].gate >= 0 || !g.vars.empty()) return false;
+    const KNode &R = g.n(g.reduces[0]);
+    if (R.src.size() != 2 || (dt_size(R.dt) != 4 && dt_size(R.dt) != 8)) return false;
+    const PolyOps op = reduce_op(R);
+    if (op != POLY_OP_ADD && op != POLY_OP_MAX && op != POLY_OP_MUL) return false;
+    // the REDUCE must not sit inside another loop of its own kernel
+    *red = g.reduces[0];
+    *ord = g.range_ord.at(R.src[1]);
+    for (int r : g.stores[0].ranges) if (g.ranges[(size_t)r].extent < 0 || r == *ord) return false;
+    return g.ranges[(size_t)*ord].extent >= 128;
+  };
+  RowPhase A;
+  if (!reduce_shape(gA, &A.red, &A.own_red_ord)) return false;
+  const int64_t R = gA.ranges[(size_t)A.own_red_ord].extent;
+  const int red_master = A.own_red_ord;
+  std::vector<int64_t> mext(gA.ranges.size());
+  for (size_t i = 0; i < gA.ranges.size(); i++) mext[i] = gA.ranges[i].extent;
+  A.m.item = a_item;
+  for (int r : gA.stores[0].ranges) A.m.rm[r] = r;
+  A.m.rm[A.own_red_ord] = A.own_red_ord;
+  double rows = 1;
+  for (int r : gA.stores[0].ranges) rows *= (double)gA.ranges[(size_t)r].extent;
+  if (rows < 1 || rows > 2147483647.0) return false;
+
+  auto store_aff = [&](const Member &m, Aff *a) {
+    const KernelGraph &g = sc.graphs[(size_t)m.item];
+    const int li = g.n(g.n(g.stores[0].index).src[1]).lin;
+    return li >= 0 && lin_to_aff(g, g.lins[(size_t)li], m.rm, a) && !a->c.count(red_master);
+  };
+  auto out_slot_of = [&](int item) {
+    const KernelGraph &g = sc.graphs[(size_t)item];
+    return sc.slot(item, g.param_slot(g.stores[0].param));
+  };
+  std::vector<RowPhase> phases{A};
+  std::vector<std::pair<int, Aff>> results, ref_loads;
+  std::vector<std::string> names;
+  std::set<int> internal;
+  {
+    Aff a;
+    if (!store_aff(A.m, &a)) return false;
+    results.push_back({out_slot_of(a_item), a});
+    names.push_back("s1");
+  }
+  collect_ref_loads(sc, A.m, &ref_loads);
+  // grow: the readers of the latest result decide what comes next
+  for (;;) {
+    const int cur = results.back().first;
+    if (!s->buf_slots[cur].is_intermediate || sc.writers[(size_t)cur].size() != 1) return false;
+    internal.insert(cur);
+    int next_reduce = -1, next_map = -1;
+    for (int r : sc.readers[(size_t)cur]) {
+      if (taken[(size_t)r]) return false;
+      const KernelGraph &g = sc.graphs[(size_t)r];
+      if (g.reduces.empty()) { if (next_map >= 0 && next_map != r) return false; next_map = r; }
+      else { if (next_reduce >= 0) return false; next_reduce = r; }
+    }
+    if (next_map < 0) return false;                    // every chain ends in a pointwise kernel
+    if (next_reduce >= 0 && phases.size() < 3) {
+      RowPhase B;
+      const KernelGraph &g = sc.graphs[(size_t)next_reduce];
+      if (!reduce_shape(g, &B.red, &B.own_red_ord)) return false;
+      if (!map_phase(sc, next_reduce, mext, ref_loads, results, names, &B.m)) FA_REJECT();
+      if (!B.m.rm.count(B.own_red_ord) || B.m.rm[B.own_red_ord] != red_master) FA_REJECT();
+      for (int r : g.stores[0].ranges) if (!B.m.rm.count(r)) FA_REJECT();
+      Aff a;
+      if (!store_aff(B.m, &a)) FA_REJECT();
+      phases.push_back(B);
+      results.push_back({out_slot_of(next_reduce), a});
+      names.push_back(strf("s%zu", results.size()));
+      collect_ref_loads(sc, B.m, &ref_loads);
+      continue;
+    }
+    if (next_reduce >= 0) return false;
+    RowPhase C;
+    C.is_map = true;
+    const KernelGraph &g = sc.graphs[(size_t)next_map];
+    if (!g.reduces.empty() || g.stores.size() != 1 || g.stores[0].gate >= 0 || !g.vars.empty()) return false;
+    if (!map_phase(sc, next_map, mext, ref_loads, results, names, &C.m)) FA_REJECT();
+    std::set<int> covered;
+    for (int r : g.stores[0].ranges) {
+      if (!C.m.rm.count(r)) FA_REJECT();
+      covered.insert(C.m.rm[r]);
+    }
+    if (covered.size() != gA.stores[0].ranges.size() + 1 || !covered.count(red_master)) FA_REJECT();
+    phases.push_back(C);
+    break;
+  }
+  // every result is read inside the group only
+  std::vector<int> items;
+  for (const RowPhase &p : phases) items.push_back(p.m.item);
+  for (const auto &res : results)
+    for (int r : sc.readers[(size_t)res.first])
+      if (std::find(items.begin(), items.end(), r) == items.end()) FA_REJECT();
+  const int last_item = items.back();
+  const int out_slot = out_slot_of(last_item);
+  std::set<int> inputs;
+  if (!group_is_schedulable(sc, items, a_item, last_item, internal, out_slot, &inputs)) FA_REJECT();
+  for (const RowPhase &p : phases) if (!internal_loads_replaced(sc, p.m, internal, -1)) FA_REJECT();
+
+  // ── code generation ────────────────────────────────────────────────────
+  const int G = (R >= 4096 || (rows < 2048 && R >= 1024)) ? 256 : 64;
+  std::vector<int> arg_slots;
+  arg_slots.push_back(out_slot);
+  for (int sl : inputs) arg_slots.push_back(sl);
+  auto arg_of = [&](int sl) { return (int)(std::find(arg_slots.begin(), arg_slots.end(), sl) - arg_slots.begin()); };
+  auto call_args = [&](int item) {
+    const KernelGraph &g = sc.graphs[(size_t)item];
+    std::string c;
+    for (size_t i = 0; i < g.params.size(); i++) {
+      const int sl = sc.slot(item, (int)i);
+      if (i) c += ", ";
+      if (internal.count(sl)) c += strf("(%s%s*)0", g.params[i].written ? "" : "const ", dt_cname(g.params[i].dt));
+      else c += strf("fa%d", arg_of(sl));
+    }
+    return c;
+  };
+  std::string sig;
+  double bytes = 0;
+  for (size_t j = 0; j < arg_slots.size(); j++) {
+    DT dt = DT_VOID;
+    for (int it : items) {
+      const int p = sc.param_of(it, arg_slots[j]);
+      if (p >= 0) dt = sc.graphs[(size_t)it].params[(size_t)p].dt;
+    }
+    if (j) sig += ", ";
+    sig += j == 0 ? strf("%s* fa%zu", dt_cname(dt), j) : strf("const %s* __restrict__ fa%zu", dt_cname(dt), j);
+    bytes += (double)s->buf_slots[arg_slots[j]].nbytes;
+  }
+  // master row decomposition: fastest row range = smallest stride in the first result
+  std::string row_decomp;
+  {
+    std::vector<std::pair<int64_t, int>> keyed;
+    for (int r : gA.stores[0].ranges) {
+      auto it = results[0].second.c.find(r);
+      keyed.push_back({it == results[0].second.c.end() ? ((int64_t)1 << 50) : std::abs(it->second), r});
+    }
+    std::sort(keyed.begin(), keyed.end());
+    row_decomp += "  long long t_ = row;\n";
+    for (size_t i = 0; i < keyed.size(); i++) {
+      const int ord = keyed[i].second;
+      const int64_t e = gA.ranges[(size_t)ord].extent;
+      if (i + 1 == keyed.size()) row_decomp += strf("  const int r%d = (int)t_;\n", ord);
+      else row_decomp += strf("  const int r%d = (int)(t_ %% %lld); t_ /= %lld;\n", ord, (long long)e, (long long)e);
+    }
+  }
+  std::string code, calls, strat;
+  std::string lead;   // results so far, as parameters
+  std::string lead_call;
+  for (size_t pi = 0; pi < phases.size(); pi++) {
+    const RowPhase &ph = phases[pi];
+    const KernelGraph &g = sc.graphs[(size_t)ph.m.item];
+    Emitter em(g);
+    Scope S0;                        // row-invariant values
+    S0.indent = 1;
+    int own_f = -1;                  // this kernel's range that walks along the row
+    for (auto &kv : ph.m.rm) {
+      if (kv.second == red_master) { own_f = kv.first; continue; }
+      em.bind_range(kv.first, strf("r%d", kv.second));
+      S0.avail |= (uint64_t)1 << kv.first;
+    }
+    if (own_f < 0) FA_REJECT();
+    for (auto &kv : ph.m.preset) em.preset(kv.first, kv.second);
+    const std::vector<int> roots{ph.is_map ? g.stores[0].value : g.n(ph.red).src[0]};
+    // vector width along the row
+    int V = 1;
+    {
+      int maxsz = 1;
+      std::vector<char> mark(g.nodes.size(), 0);
+      mark_reachable(g, roots[0], mark);
+      for (int i = 0; i < (int)g.nodes.size(); i++)
+        if (mark[(size_t)i] && g.n(i).op == POLY_OP_LOAD && !ph.m.preset.count(i) && (g.n(i).deps & ((uint64_t)1 << own_f)))
+          maxsz = std::max(maxsz, dt_size(g.n(i).dt));
+      if (ph.is_map) maxsz = std::max(maxsz, dt_size(g.n(g.stores[0].param).dt));
+      V = std::max(1, 16 / maxsz);
+      while (V > 1 && (R % V != 0 || R < (int64_t)G * V)) V /= 2;
+      if (ph.is_map) {
+        const int li = g.n(g.n(g.stores[0].index).src[1]).lin;
+        while (V > 1 && (li < 0 || !lin_vec_ok(g, g.lins[(size_t)li], own_f, V) ||
+                         dt_size(g.n(g.stores[0].value).dt) != dt_size(g.n(g.stores[0].param).dt))) V /= 2;
+      }
+    }
+    const std::string fv = strf("f%d", own_f);           // C name of the position along the row
+    Scope L;                          // loop body, one vector per step
+    L.parent = &S0;
+    L.avail = S0.avail;
+    L.indent = 2;
+    std::vector<int> pres;
+    if (V > 1) pres = hoist_vector_loads(g, em, roots, own_f, V, fv + "_0", &L);
+    Scope U;                          // one element
+    U.parent = &L;
+    U.avail = L.avail | ((uint64_t)1 << own_f);
+    U.indent = 3;
+    em.bind_range(own_f, fv);
+    std::string fn = strf("poly_row_p%zu", pi);
+    std::string ret = "void", result_expr, tail;
+    std::string loop;
+    if (!ph.is_map) {
+      const KNode &Rn = g.n(ph.red);
+      const PolyOps op = reduce_op(Rn);
+      std::string v = em.emit(Rn.src[0], &U);
+      U.code += strf("      acc = %s;\n", Emitter::reduce_combine(op, Rn.dt, "acc", v).c_str());
+      loop += strf("  %s acc = %s;\n", dt_cname(Rn.dt), Emitter::reduce_identity(op, Rn.dt).c_str());
+      loop += S0.code;
+      S0.code.clear();
+      loop += strf("  for (int %s_0 = lane * %d; %s_0 < %lld; %s_0 += %d) {\n", fv.c_str(), V, fv.c_str(), (long long)R, fv.c_str(), G * V);
+      loop += L.code;
+      loop += strf("#pragma unroll\n    for (int u = 0; u < %d; u++) {\n      const int %s = %s_0 + u;\n", V, fv.c_str(), fv.c_str());
+      loop += U.code + "    }\n  }\n";
+      loop += strf("  acc = %s;\n", wave_reduce_call(op, Rn.dt, "acc").c_str());
+      if (G == 256) {
+        loop += strf("  __shared__ %s red[4];\n  __syncthreads();\n  if ((threadIdx.x & 63) == 0) red[threadIdx.x >> 6] = acc;\n  __syncthreads();\n",
+                     dt_cname(Rn.dt));
+        std::string e = "red[0]";
+        for (int w = 1; w < 4; w++) e = Emitter::reduce_combine(op, Rn.dt, e, strf("red[%d]", w));
+        loop += strf("  acc = %s;\n", e.c_str());
+      }
+      for (int n : pres) em.clear_preset(n);
+      em.preset(ph.red, "acc");
+      result_expr = em.emit(g.stores[0].value, &S0);
+      tail = S0.code + strf("  return %s;\n", result_expr.c_str());
+      ret = dt_cname(g.n(g.stores[0].value).dt);
+    } else {
+      const StoreInfo &st = g.stores[0];
+      const int li = g.n(g.n(st.index).src[1]).lin;
+      const int p = g.param_slot(st.param);
+      std::string v = em.emit(st.value, &U);
+      const char *odt = dt_cname(g.n(st.param).dt);
+      if (V > 1) {
+        U.code += strf("      out.v[u] = %s;\n", v.c_str());
+      } else {
+        std::string idx = em.emit(g.n(st.index).src[1], &U);
+        U.code += strf("      data%d[%s] = %s;\n", p, idx.c_str(), v.c_str());
+      }
+      std::string addr;
+      if (V > 1) { em.bind_range(own_f, fv + "_0"); addr = em.emit_lin(g.lins[(size_t)li], &L); em.bind_range(own_f, fv); }
+      loop += S0.code;
+      S0.code.clear();
+      loop += strf("  for (int %s_0 = lane * %d; %s_0 < %lld; %s_0 += %d) {\n", fv.c_str(), V, fv.c_str(), (long long)R, fv.c_str(), G * V);
+      loop += L.code;
+      if (V > 1) loop += strf("    poly_vec<%s,%d> out;\n", odt, V);
+      loop += strf("#pragma unroll\n    for (int u = 0; u < %d; u++) {\n      const int %s = %s_0 + u;\n", V, fv.c_str(), fv.c_str());
+      loop += U.code + "    }\n";
+      if (V > 1) loop += strf("    poly_vstore<%s,%d>(data%d + %s, out);\n", odt, V, p, addr.c_str());
+      loop += "  }\n";
+    }
+    if (em.failed() || em.uses_threefry) FA_REJECT();
+    code += strf("__device__ __forceinline__ %s %s(const long long row, const int lane%s, %s) {\n", ret.c_str(), fn.c_str(), lead.c_str(),
+                 params_decl(g).c_str());
+    code += row_decomp + loop + tail + "}\n";
+    if (!ph.is_map) {
+      calls += strf("    const %s %s = %s(row, lane%s, %s);\n", ret.c_str(), names[pi].c_str(), fn.c_str(), lead_call.c_str(),
+                    call_args(ph.m.item).c_str());
+      lead += strf(", const %s %s", ret.c_str(), names[pi].c_str());
+      lead_call += ", " + names[pi];
+    } else {
+      calls += strf("    %s(row, lane%s, %s);\n", fn.c_str(), lead_call.c_str(), call_args(ph.m.item).c_str());
+    }
+    strat += strf("%s%s vec%d", pi ? ", " : "", ph.is_map ? "map" : "reduce", V);
+  }
+  std::string body = strf("extern \"C\" __global__ void __launch_bounds__(256) poly_k(%s) {\n", sig.c_str());
+  if (G == 64) {
+    body += "  const int lane = threadIdx.x & 63;\n  const long long row = (long long)blockIdx.x * 4 + (threadIdx.x >> 6);\n";
+    body += strf("  if (row < %lldll) {\n", (long long)rows);
+  } else {
+    body += "  const int lane = threadIdx.x;\n  const long long row = blockIdx.x;\n  {\n";
+  }
+  body += calls + "  }\n}\n";
+
+  out->items = items;
+  out->launch_item = last_item;
+  out->internal_slots.assign(internal.begin(), internal.end());
+  out->arg_slots = arg_slots;
+  RenderedKernel &rk = out->rk;
+  rk = RenderedKernel();
+  rk.source = std::string(hip_prelude()) + code + body;
+  rk.entry = "poly_k";
+  rk.launch.grid[0] = (unsigned)(G == 256 ? rows : std::ceil(rows / 4));
+  rk.launch.block[0] = 256;
+  rk.klass = KernelClass::ROW_REDUCE;
+  rk.strategy = strf("row chain of %zu kernels (%s) G=%d R=%lld rows=%.0f", phases.size(), strat.c_str(), G, (long long)R, rows);
+  rk.n_params = (int)arg_slots.size();
+  rk.bytes = bytes;
   return true;
 }
 
@@ -751,7 +1103,7 @@ void find_fused_groups(const PolySchedule *s, const std::vector<KernelGraph> &gr
     const int k = s->exec_order[st];
     if (taken[(size_t)k] || graphs[(size_t)k].reduces.size() != 1) continue;
     FusedGroup fg;
-    if (!match_attention(sc, k, taken, &fg) && !match_matmul_tail(sc, k, taken, &fg)) continue;
+    if (!match_attention(sc, k, taken, &fg) && !match_matmul_tail(sc, k, taken, &fg) && !match_row_chain(sc, k, taken, &fg)) continue;
     for (int it : fg.items) taken[(size_t)it] = 1;
     out->push_back(std::move(fg));
   }

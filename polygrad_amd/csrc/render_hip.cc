@@ -21,6 +21,83 @@
 
 namespace polyhip {
 
+bool lin_vec_ok(const KernelGraph &g_, const Lin &l, int F, int V) {
+  if (l.c0 % V) return false;
+  bool seenF = false;
+  for (const Term &t : l.terms) {
+    const Atom &a = g_.atoms[(size_t)t.atom];
+    if (a.kind == Atom::RANGE && g_.range_ord.at(a.node) == F) {
+      if (t.coef != 1) return false;
+      seenF = true;
+    } else {
+      if (g_.atom_deps(t.atom) & ((uint64_t)1 << F)) return false;
+      if (t.coef % V) return false;
+    }
+  }
+  return seenF;
+}
+
+void mark_reachable(const KernelGraph &g_, int root, std::vector<char> &mark) {
+  std::vector<int> st{root};
+  while (!st.empty()) {
+    int n = st.back(); st.pop_back();
+    if (mark[(size_t)n]) continue;
+    mark[(size_t)n] = 1;
+    for (int s : g_.n(n).src) st.push_back(s);
+  }
+}
+
+std::vector<int> hoist_vector_loads(const KernelGraph &g_, Emitter &em_, const std::vector<int> &roots, int F, int V,
+                                    const std::string &f0, Scope *outer) {
+  std::vector<char> mark(g_.nodes.size(), 0);
+  for (int r : roots) mark_reachable(g_, r, mark);
+  std::vector<int> done;
+  for (int i = 0; i < (int)g_.nodes.size(); i++) {
+    if (!mark[(size_t)i]) continue;
+    const KNode &k = g_.n(i);
+    if (k.op != POLY_OP_LOAD) continue;
+    if (em_.is_preset(i)) continue;
+    if (!(k.deps & ((uint64_t)1 << F))) continue;
+    // loads that also depend on ranges not bound in `outer` (nested serial
+    // reduces) stay scalar
+    if (k.deps & ~(outer->avail | ((uint64_t)1 << F))) continue;
+    const KNode &ix = g_.n(k.src[0]);
+    int li = g_.n(ix.src[1]).lin;
+    if (li < 0 || !lin_vec_ok(g_, g_.lins[(size_t)li], F, V)) continue;
+    if (ix.src.size() >= 3 && (g_.n(ix.src[2]).deps & ((uint64_t)1 << F))) continue;
+    if (k.guard >= 0 && (g_.n(k.guard).deps & ((uint64_t)1 << F))) continue;
+    if (dt_size(k.dt) * V > 16) continue;
+    int p = g_.param_slot(ix.src[0]);
+    em_.bind_range(F, f0);
+    std::string addr = em_.emit_lin(g_.lins[(size_t)li], outer);
+    std::string name = strf("ld%d", i);
+    std::string ld = strf("poly_vload<%s,%d>(data%d + %s)", dt_cname(k.dt), V, p, addr.c_str());
+    std::string gate;
+    if (ix.src.size() >= 3) gate = em_.emit(ix.src[2], outer);
+    if (k.guard >= 0) {
+      std::string g2 = em_.emit(k.guard, outer);
+      if (k.guard_neg) g2 = "(!" + g2 + ")";
+      gate = gate.empty() ? g2 : "(" + gate + "&&" + g2 + ")";
+    }
+    if (!gate.empty()) ld = strf("(%s ? %s : poly_vec<%s,%d>{})", gate.c_str(), ld.c_str(), dt_cname(k.dt), V);
+    outer->code.append((size_t)outer->indent * 2, ' ');
+    outer->code += strf("const poly_vec<%s,%d> %s = %s;\n", dt_cname(k.dt), V, name.c_str(), ld.c_str());
+    em_.preset(i, name + ".v[u]");
+    done.push_back(i);
+  }
+  return done;
+}
+
+std::string wave_reduce_call(PolyOps op, DT dt, const std::string &v) {
+  if (dt == DT_F32) {
+    const char *fn = op == POLY_OP_ADD ? "poly_wave_add_f32" : op == POLY_OP_MUL ? "poly_wave_mul_f32" : "poly_wave_max_f32";
+    return strf("%s(%s)", fn, v.c_str());
+  }
+  const char *ct = dt_cname(dt);
+  std::string comb = Emitter::reduce_combine(op, dt, "a_", "b_");
+  return strf("poly_wave_reduce_any<%s>(%s, [](%s a_, %s b_) { return (%s)%s; })", ct, v.c_str(), ct, ct, ct, comb.c_str());
+}
+
 namespace {
 
 struct Group {
@@ -155,81 +232,12 @@ class Generic {
     return order;
   }
 
-  // Can `lin` be accessed as a V-wide vector along range `F`?  Needs unit stride
-  // in F and every other contribution a multiple of V (keeps the natural
-  // alignment of the vector type).
-  bool vec_ok(const Lin &l, int F, int V) const {
-    if (l.c0 % V) return false;
-    bool seenF = false;
-    for (const Term &t : l.terms) {
-      const Atom &a = g_.atoms[(size_t)t.atom];
-      if (a.kind == Atom::RANGE && g_.range_ord.at(a.node) == F) {
-        if (t.coef != 1) return false;
-        seenF = true;
-      } else {
-        if (g_.atom_deps(t.atom) & ((uint64_t)1 << F)) return false;
-        if (t.coef % V) return false;
-        if (a.kind == Atom::VAR || a.kind == Atom::OPAQUE) {
-          // symbolic values: only fine when the coefficient already carries V
-        }
-      }
-    }
-    return seenF;
-  }
+  bool vec_ok(const Lin &l, int F, int V) const { return lin_vec_ok(g_, l, F, V); }
 
-  bool node_under(int root, std::vector<char> &mark) const {
-    // marks every node reachable from root
-    std::vector<int> st{root};
-    while (!st.empty()) {
-      int n = st.back(); st.pop_back();
-      if (mark[(size_t)n]) continue;
-      mark[(size_t)n] = 1;
-      for (int s : g_.n(n).src) st.push_back(s);
-    }
-    return true;
-  }
-
-  // Emits vector loads (hoisted out of the unrolled loop) for every LOAD under
-  // `roots` that is unit-stride along F; returns the preset nodes.
+  bool node_under(int root, std::vector<char> &mark) const { mark_reachable(g_, root, mark); return true; }
   std::vector<int> hoist_vector_loads(const std::vector<int> &roots, int F, int V, const std::string &f0,
-                                      Scope *outer, bool skip_inside_reduce) {
-    std::vector<char> mark(g_.nodes.size(), 0);
-    for (int r : roots) node_under(r, mark);
-    std::vector<int> done;
-    for (int i = 0; i < (int)g_.nodes.size(); i++) {
-      if (!mark[(size_t)i]) continue;
-      const KNode &k = g_.n(i);
-      if (k.op != POLY_OP_LOAD) continue;
-      if (!(k.deps & ((uint64_t)1 << F))) continue;
-      // loads that also depend on ranges not bound in `outer` (nested serial
-      // reduces) stay scalar
-      if (k.deps & ~(outer->avail | ((uint64_t)1 << F))) continue;
-      (void)skip_inside_reduce;
-      const KNode &ix = g_.n(k.src[0]);
-      int li = g_.n(ix.src[1]).lin;
-      if (li < 0 || !vec_ok(g_.lins[(size_t)li], F, V)) continue;
-      if (ix.src.size() >= 3 && (g_.n(ix.src[2]).deps & ((uint64_t)1 << F))) continue;
-      if (k.guard >= 0 && (g_.n(k.guard).deps & ((uint64_t)1 << F))) continue;
-      if (dt_size(k.dt) * V > 16) continue;
-      int p = g_.param_slot(ix.src[0]);
-      em_.bind_range(F, f0);
-      std::string addr = em_.emit_lin(g_.lins[(size_t)li], outer);
-      std::string name = strf("ld%d", i);
-      std::string ld = strf("poly_vload<%s,%d>(data%d + %s)", dt_cname(k.dt), V, p, addr.c_str());
-      std::string gate;
-      if (ix.src.size() >= 3) gate = em_.emit(ix.src[2], outer);
-      if (k.guard >= 0) {
-        std::string g2 = em_.emit(k.guard, outer);
-        if (k.guard_neg) g2 = "(!" + g2 + ")";
-        gate = gate.empty() ? g2 : "(" + gate + "&&" + g2 + ")";
-      }
-      if (!gate.empty()) ld = strf("(%s ? %s : poly_vec<%s,%d>{})", gate.c_str(), ld.c_str(), dt_cname(k.dt), V);
-      outer->code.append((size_t)outer->indent * 2, ' ');
-      outer->code += strf("const poly_vec<%s,%d> %s = %s;\n", dt_cname(k.dt), V, name.c_str(), ld.c_str());
-      em_.preset(i, name + ".v[u]");
-      done.push_back(i);
-    }
-    return done;
+                                      Scope *outer, bool) {
+    return polyhip::hoist_vector_loads(g_, em_, roots, F, V, f0, outer);
   }
 
   static void line(std::string &code, int indent, const std::string &s) {
@@ -403,15 +411,7 @@ class Generic {
     return true;
   }
 
-  std::string wave_reduce_call(PolyOps op, DT dt, const std::string &v) const {
-    if (dt == DT_F32) {
-      const char *fn = op == POLY_OP_ADD ? "poly_wave_add_f32" : op == POLY_OP_MUL ? "poly_wave_mul_f32" : "poly_wave_max_f32";
-      return strf("%s(%s)", fn, v.c_str());
-    }
-    const char *ct = dt_cname(dt);
-    std::string comb = Emitter::reduce_combine(op, dt, "a_", "b_");
-    return strf("poly_wave_reduce_any<%s>(%s, [](%s a_, %s b_) { return (%s)%s; })", ct, v.c_str(), ct, ct, ct, comb.c_str());
-  }
+  std::string wave_reduce_call(PolyOps op, DT dt, const std::string &v) const { return polyhip::wave_reduce_call(op, dt, v); }
 
   std::string render_coop(RenderedKernel *out) {
     const Group &gr = groups_[0];

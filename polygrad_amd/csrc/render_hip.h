@@ -88,6 +88,7 @@ class Emitter {
   // Overrides the value of a node (vector-loaded values, reduce results, ...).
   void preset(int node, const std::string &expr) { preset_[node] = expr; }
   void clear_preset(int node) { preset_.erase(node); }
+  bool is_preset(int node) const { return preset_.count(node) != 0; }
   // Replaces the serial loop of a REDUCE node by caller-generated code; the
   // callback receives the scope the value is placed in and returns its C name.
   void custom_reduce(int node, std::function<std::string(Scope *)> fn) { custom_[node] = std::move(fn); }
@@ -118,6 +119,19 @@ class Emitter {
   std::unordered_map<int, std::function<std::string(Scope *)>> custom_;
   std::string error_;
 };
+
+// Pieces of the generic lowering that fused kernels reuse.
+// Can `l` be accessed as a V-wide vector along range ordinal F (unit stride in F, every
+// other contribution a multiple of V)?
+bool lin_vec_ok(const KernelGraph &g, const Lin &l, int F, int V);
+void mark_reachable(const KernelGraph &g, int root, std::vector<char> &mark);
+// Emits V-wide vector loads into `outer` for every LOAD under `roots` that is unit-stride
+// along F (starting at the C expression f0) and presets those nodes to "<name>.v[u]";
+// returns the preset nodes.
+std::vector<int> hoist_vector_loads(const KernelGraph &g, Emitter &em, const std::vector<int> &roots, int F, int V,
+                                    const std::string &f0, Scope *outer);
+// C expression reducing `v` over the 64 lanes of a wave.
+std::string wave_reduce_call(PolyOps op, DT dt, const std::string &v);
 
 // Prelude with the wave/workgroup reduction helpers and small utilities that
 // every generated kernel may use.

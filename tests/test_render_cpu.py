@@ -142,21 +142,23 @@ int main(void) {
 
 def test_kernel_groups_of_the_gpt2_plan_fuse_and_compile(hiplib):
     """Needs no device: in the benchmark schedule the plan compiler recognises, per layer,
-    one attention group (six scheduled kernels) and three matmuls followed by a pointwise
-    kernel (residual add, GELU, residual add); the generated sources compile."""
+    one attention group (six scheduled kernels), three matmuls followed by a pointwise
+    kernel (residual add, GELU, residual add) and two LayerNorms of three kernels each
+    (plus the final LayerNorm); the generated sources compile."""
     from polygrad_amd import PlanFile
     pf = PlanFile(os.path.join(ROOT, "polygrad_amd", "plans", "gpt2_small_bf16_b8_t1024.polyplan"))
     count = hiplib.poly_hip_fused_groups(pf.schedule, -1, None, None)
-    assert count == 48
+    assert count == 12 + 36 + 25
     seen = {}
     for i in range(count):
         src, n = C.c_void_p(), C.c_int()
         hiplib.poly_hip_fused_groups(pf.schedule, i, C.byref(src), C.byref(n))
         text = _ffi.take_string(src.value)
-        kind = "attention" if "POLY_FA_M" in text else "tail"
-        assert n.value == (6 if kind == "attention" else 2)
+        kind = "attention" if "POLY_FA_M" in text else "rows" if "poly_row_p0" in text else "tail"
+        assert n.value == {"attention": 6, "tail": 2, "rows": 3}[kind]
         seen.setdefault(kind, []).append(text)
-    assert len(seen["attention"]) == 12 and len(seen["tail"]) == 36
+    assert len(seen["attention"]) == 12 and len(seen["tail"]) == 36 and len(seen["rows"]) == 25
+    assert hiplib.poly_hip_compile_check(seen["rows"][0].encode()) == 0
     att = seen["attention"][0]
     assert "poly_fa_term" in att and "__builtin_amdgcn_mfma_f32_32x32x16_bf16" in att
     assert hiplib.poly_hip_compile_check(att.encode()) == 0
@@ -168,6 +170,10 @@ def test_kernel_groups_of_the_gpt2_plan_fuse_and_compile(hiplib):
         assert hiplib.poly_hip_fused_groups(pf.schedule, -1, None, None) == 0
     finally:
         del os.environ["POLY_HIP_NO_FUSION"]
-    # a plan without matmuls has nothing to fuse
-    pf2 = PlanFile(os.path.join(ROOT, "polygrad_amd", "plans", "rowops_f32_8192_softmax.polyplan"))
-    assert hiplib.poly_hip_fused_groups(pf2.schedule, -1, None, None) == 0
+    # softmax and LayerNorm on their own: one row chain each; a single reduction: nothing
+    for name, want in (("softmax", 1), ("layernorm", 1), ("sum", 0)):
+        pf2 = PlanFile(os.path.join(ROOT, "polygrad_amd", "plans", f"rowops_f32_8192_{name}.polyplan"))
+        src = C.c_void_p()
+        assert hiplib.poly_hip_fused_groups(pf2.schedule, 0, C.byref(src), None) == want
+        if want:
+            assert hiplib.poly_hip_compile_check(_ffi.take_string(src.value).encode()) == 0
