@@ -674,6 +674,53 @@ static bool match_row_chain(const Sched &sc, int a_item, const std::vector<char>
   return true;
 }
 
+// A kernel that only moves data: out[store index] = in[load index], both affine in the
+// kernel's ranges, the store covering its buffer densely (row-major in some order of the
+// ranges).  Then element p of the output is element src(p) of the input, with
+// src(p) = c0 + sum_i ((p / stride_i) % extent_i) * coef_i.
+struct CopyMap {
+  int item = -1, src_slot = -1;
+  int64_t c0 = 0;
+  struct Digit { int64_t stride, extent, coef; };
+  std::vector<Digit> digits;   // by decreasing stride
+};
+
+static bool match_copy(const Sched &sc, int item, CopyMap *cm) {
+  const KernelGraph &g = sc.graphs[(size_t)item];
+  if (!g.reduces.empty() || g.stores.size() != 1 || g.stores[0].gate >= 0 || !g.vars.empty()) return false;
+  const StoreInfo &st = g.stores[0];
+  const KNode &v = g.n(st.value);
+  if (v.op != POLY_OP_LOAD || v.guard >= 0 || v.dt != g.n(st.param).dt) return false;
+  const KNode &ix = g.n(v.src[0]);
+  if (ix.src.size() != 2) return false;
+  const int ll = g.n(ix.src[1]).lin, ls = g.n(g.n(st.index).src[1]).lin;
+  if (ll < 0 || ls < 0) return false;
+  RangeMap id;
+  for (int r : st.ranges) id[r] = r;
+  Aff as, al;
+  if (!lin_to_aff(g, g.lins[(size_t)ls], id, &as) || !lin_to_aff(g, g.lins[(size_t)ll], id, &al)) return false;
+  if (as.c0 != 0 || as.c.size() != st.ranges.size()) return false;
+  std::vector<CopyMap::Digit> d;
+  for (auto &kv : as.c) {
+    if (kv.second <= 0) return false;
+    auto it = al.c.find(kv.first);
+    d.push_back({kv.second, g.ranges[(size_t)kv.first].extent, it == al.c.end() ? 0 : it->second});
+  }
+  std::sort(d.begin(), d.end(), [](const CopyMap::Digit &a, const CopyMap::Digit &b) { return a.stride > b.stride; });
+  int64_t expect = 1;
+  for (size_t i = d.size(); i-- > 0;) {
+    if (d[i].extent <= 0 || d[i].stride != expect) return false;
+    expect *= d[i].extent;
+  }
+  const int out_slot = sc.slot(item, g.param_slot(st.param));
+  if (expect != sc.s->buf_slots[out_slot].numel) return false;
+  cm->item = item;
+  cm->src_slot = sc.slot(item, g.param_slot(ix.src[0]));
+  cm->c0 = al.c0;
+  cm->digits = d;
+  return cm->src_slot != out_slot;
+}
+
 // Tries to grow an attention group from the matmul at schedule item `s_item`.
 static bool match_attention(const Sched &sc, int s_item, const std::vector<char> &taken, FusedGroup *out) {
   const PolySchedule *s = sc.s;
@@ -908,8 +955,42 @@ static bool match_attention(const Sched &sc, int s_item, const std::vector<char>
   std::set<int> group_items;
   for (const Member &m : all) group_items.insert(m.item);
   if (group_items.size() != all.size()) FA_REJECT();
-  const int first_step = sc.step_of[(size_t)s_item], last_step = sc.step_of[(size_t)i_pv];
+  const int last_step = sc.step_of[(size_t)i_pv];
+  int first_step = sc.step_of[(size_t)s_item];
   for (int it : group_items) if (sc.step_of[(size_t)it] < first_step || sc.step_of[(size_t)it] > last_step) FA_REJECT();
+  // Operands that are plain copies of a slice of another buffer (the q / k / v split of a
+  // fused projection) are read from that buffer directly: the copy kernel joins the group
+  // and its output is never materialised.  Needs the 64 features of a row to stay
+  // contiguous and 64-aligned through the copy.
+  const int op_slot[3] = {sc.slot(s_item, mS.A.param), sc.slot(s_item, mS.B.param), sc.slot(i_pv, mV.B.param)};
+  const int op_reader[3] = {s_item, s_item, i_pv};
+  CopyMap folded[3];
+  std::vector<int> copy_items;
+  auto multiple_of_64 = [&](const std::vector<MmDim> &dims, bool use_a) {
+    for (const MmDim &d : dims) if ((use_a ? d.ca : d.cb) % 64) return false;
+    return true;
+  };
+  bool op_aligned[3] = {mS.a_c0 % 64 == 0 && multiple_of_64(mS.zd, true) && multiple_of_64(mS.md, true),
+                        mS.b_c0 % 64 == 0 && multiple_of_64(mS.zd, false) && multiple_of_64(mS.nd, false), aV.c0 % 64 == 0};
+  for (auto &kv : aV.c) if (kv.second % 64) op_aligned[2] = false;
+  for (int o = 0; o < 3; o++) {
+    const int sl = op_slot[o];
+    if (getenv("POLY_HIP_NO_COPY_FOLD") || !op_aligned[o] || !s->buf_slots[sl].is_intermediate || internal.count(sl)) continue;
+    if (sc.writers[(size_t)sl].size() != 1 || sc.readers[(size_t)sl].size() != 1 || sc.readers[(size_t)sl][0] != op_reader[o]) continue;
+    if ((o == 0 && sl == op_slot[1]) || (o == 1 && sl == op_slot[0])) continue;   // Q and K from one buffer: keep it simple
+    const int w = sc.writers[(size_t)sl][0];
+    CopyMap cm;
+    if (taken[(size_t)w] || group_items.count(w) || sc.step_of[(size_t)w] > sc.step_of[(size_t)op_reader[o]] || !match_copy(sc, w, &cm)) continue;
+    if (cm.digits.empty() || cm.digits.back().extent % 64 || cm.digits.back().coef != 1 || cm.c0 % 8) continue;
+    bool ok = true;
+    for (size_t i = 0; i + 1 < cm.digits.size(); i++) if (cm.digits[i].coef % 8) ok = false;
+    if (!ok || internal.count(cm.src_slot)) continue;
+    folded[o] = cm;
+    copy_items.push_back(w);
+    group_items.insert(w);
+    internal.insert(sl);
+    first_step = std::min(first_step, sc.step_of[(size_t)w]);
+  }
     std::set<int> inputs;
   std::map<int, int> first_read;   // input slot -> earliest original step of a member reading it
   for (int it : group_items) {
@@ -939,8 +1020,10 @@ static bool match_attention(const Sched &sc, int s_item, const std::vector<char>
       if (g.n(id).op != POLY_OP_LOAD) continue;
       const int p = g.param_slot(g.n(g.n(id).src[0]).src[0]);
       if (!internal.count(sc.slot(m.item, p))) continue;
-      const bool is_pv_a = m.item == i_pv && id == mV.A.load;
-      if (!m.preset.count(id) && !is_pv_a) FA_REJECT();
+      // loads the template performs itself: P, and operands folded into their source
+      const bool by_template = (m.item == i_pv && (id == mV.A.load || id == mV.B.load)) ||
+                               (m.item == s_item && (id == mS.A.load || id == mS.B.load));
+      if (!m.preset.count(id) && !by_template) FA_REJECT();
     }
   }
 
@@ -998,16 +1081,62 @@ static bool match_attention(const Sched &sc, int s_item, const std::vector<char>
   cfg += strf("#define POLY_TIN %s\n", tn);
   cfg += strf("#define POLY_MFMA(a, b, c) __builtin_amdgcn_mfma_f32_32x32x16_%s(a, b, c, 0, 0, 0)\n", tin == DT_BF16 ? "bf16" : "f16");
   cfg += strf("#define POLY_FA_M %lld\n#define POLY_FA_N %lld\n#define POLY_FA_Z %lld\n", (long long)mS.M, (long long)mS.N, (long long)mS.Z);
-  cfg += strf("#define POLY_Q_PTR fa%d\n#define POLY_K_PTR fa%d\n#define POLY_V_PTR fa%d\n", arg_of(sc.slot(s_item, mS.A.param)),
-              arg_of(sc.slot(s_item, mS.B.param)), arg_of(sc.slot(i_pv, mV.B.param)));
+  auto operand_arg = [&](int o) { return arg_of(folded[o].item >= 0 ? folded[o].src_slot : op_slot[o]); };
+  cfg += strf("#define POLY_Q_PTR fa%d\n#define POLY_K_PTR fa%d\n#define POLY_V_PTR fa%d\n", operand_arg(0), operand_arg(1), operand_arg(2));
+  // position in the operand's own buffer -> position in the buffer it was copied from
+  const char *src_name[3] = {"poly_fa_qsrc", "poly_fa_ksrc", "poly_fa_vsrc"};
+  for (int o = 0; o < 3; o++) {
+    std::string f = strf("__device__ __forceinline__ int %s(int p) {\n", src_name[o]);
+    if (folded[o].item < 0) f += "  return p;\n}\n";
+    else {
+      f += strf("  int off = %lld;\n", (long long)folded[o].c0);
+      for (const CopyMap::Digit &d : folded[o].digits)
+        f += strf("  off += ((p / %lld) %% %lld) * %lld;\n", (long long)d.stride, (long long)d.extent, (long long)d.coef);
+      f += "  return off;\n}\n";
+    }
+    cfg += f;
+  }
   cfg += matmul_offset_fn("poly_fa_qz", mS.zd, true, mS.a_c0) + matmul_offset_fn("poly_fa_qm", mS.md, true, 0);
   cfg += matmul_offset_fn("poly_fa_kz", mS.zd, false, mS.b_c0) + matmul_offset_fn("poly_fa_kn", mS.nd, false, 0);
-  cfg += "__device__ __forceinline__ int poly_q_off(int z, int m) { return poly_fa_qz(z) + poly_fa_qm(m); }\n";
-  cfg += "__device__ __forceinline__ int poly_k_off(int z, int n) { return poly_fa_kz(z) + poly_fa_kn(n); }\n";
-  {
-    std::string e = strf("%lld", (long long)aV.c0);
-    for (auto &kv : aV.c) e += strf(" + %lld * r%d", (long long)kv.second, kv.first);
-    cfg += "__device__ __forceinline__ int poly_v_off(int z, int n) {\n  const int m = 0;\n" + master_decomp + "  return " + e + ";\n}\n";
+  // Row offsets as the kernel sees them: source position of row x (query or key) of batch z.
+  // When that is affine in x for every z -- the usual case -- the z part is evaluated once
+  // and the row part is a multiplication; otherwise the general digit form is kept.
+  auto eval_src = [&](int o, int64_t p) {
+    if (folded[o].item < 0) return p;
+    int64_t off = folded[o].c0;
+    for (const CopyMap::Digit &d : folded[o].digits) off += ((p / d.stride) % d.extent) * d.coef;
+    return off;
+  };
+  auto raw_off = [&](int o, int64_t z, int64_t x) {
+    if (o == 0) return mS.a_c0 + matmul_eval_offset(mS.zd, true, z) + matmul_eval_offset(mS.md, true, x);
+    if (o == 1) return mS.b_c0 + matmul_eval_offset(mS.zd, false, z) + matmul_eval_offset(mS.nd, false, x);
+    int64_t v = aV.c0;
+    for (auto &kv : aV.c) v += kv.second * matmul_range_value(mS, kv.first, 0, x, z);
+    return v;
+  };
+  std::string v_expr = strf("%lld", (long long)aV.c0);
+  for (auto &kv : aV.c) v_expr += strf(" + %lld * r%d", (long long)kv.second, kv.first);
+  const char *off_name[3] = {"poly_q_off", "poly_k_off", "poly_v_off"};
+  const std::string general[3] = {
+      "__device__ __forceinline__ int poly_fa_q0(int z, int m) { return poly_fa_qz(z) + poly_fa_qm(m); }\n",
+      "__device__ __forceinline__ int poly_fa_k0(int z, int n) { return poly_fa_kz(z) + poly_fa_kn(n); }\n",
+      "__device__ __forceinline__ int poly_fa_v0(int z, int n) {\n  const int m = 0;\n" + master_decomp + "  return " + v_expr + ";\n}\n"};
+  const char *raw_name[3] = {"poly_fa_q0", "poly_fa_k0", "poly_fa_v0"};
+  for (int o = 0; o < 3; o++) {
+    cfg += general[o];
+    const int64_t X = o == 0 ? mS.M : mS.N;
+    bool affine = mS.Z * X <= (int64_t)1 << 24;
+    const int64_t step = eval_src(o, raw_off(o, 0, 1)) - eval_src(o, raw_off(o, 0, 0));
+    for (int64_t z = 0; z < mS.Z && affine; z++) {
+      const int64_t base = eval_src(o, raw_off(o, z, 0));
+      for (int64_t x = 0; x < X; x++)
+        if (eval_src(o, raw_off(o, z, x)) != base + x * step) { affine = false; break; }
+    }
+    if (affine)
+      cfg += strf("__device__ __forceinline__ int %s(int z, int x) { return %s(%s(z, 0)) + x * %lld; }\n", off_name[o], src_name[o],
+                  raw_name[o], (long long)step);
+    else
+      cfg += strf("__device__ __forceinline__ int %s(int z, int x) { return %s(%s(z, x)); }\n", off_name[o], src_name[o], raw_name[o]);
   }
   cfg += strf("#define POLY_SIGNATURE %s\n", sig.c_str());
   cfg += strf("#define POLY_FA_SKIP_DEAD_BLOCKS %d\n", p_is_term_over_sum ? 1 : 0);
@@ -1056,6 +1185,7 @@ static bool match_attention(const Sched &sc, int s_item, const std::vector<char>
   if (failed) FA_REJECT();
 
   out->items.clear();
+  for (int w : copy_items) out->items.push_back(w);
   for (const Member &m : all) out->items.push_back(m.item);
   out->launch_item = i_pv;
   out->internal_slots.assign(internal.begin(), internal.end());
@@ -1067,7 +1197,7 @@ static bool match_attention(const Sched &sc, int s_item, const std::vector<char>
   rk.launch.grid[0] = (unsigned)((mS.M / 128) * mS.Z);
   rk.launch.block[0] = 256;
   rk.klass = KernelClass::ATTENTION;
-  rk.strategy = strf("fused attention (%zu kernels): mfma 32x32x16 %s Z=%lld M=%lld N=%lld D=64, two passes over keys", all.size(),
+  rk.strategy = strf("fused attention (%zu kernels): mfma 32x32x16 %s Z=%lld M=%lld N=%lld D=64, two passes over keys", all.size() + copy_items.size(),
                      tin == DT_BF16 ? "bf16" : "f16", (long long)mS.Z, (long long)mS.M, (long long)mS.N);
   rk.n_params = (int)arg_slots.size();
   rk.n_vars = 0;

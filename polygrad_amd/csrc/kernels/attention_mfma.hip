@@ -212,7 +212,7 @@ extern "C" __global__ void __launch_bounds__(FA_THREADS) __attribute__((amdgpu_w
           const int n = key_of(kb, t, r);
           x[r] = POLY_FA_SCORE(st[r], mq, n, z);
           const float v = POLY_FA_MAXV(x[r], mq, n, z);
-          bm = (bm < v) ? v : bm;
+          bm = __builtin_fmaxf(bm, v);   // like (bm < v) ? v : bm, a NaN v is ignored
           nan_probe = nan_probe + v;      // NaN if any value is (or +inf meets -inf: then not skipped)
         }
         const float new_max = (row_max < bm) ? bm : row_max;

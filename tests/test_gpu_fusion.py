@@ -46,11 +46,12 @@ def test_fused_attention_matches_unfused_and_reference(qk_gain):
         del os.environ["POLY_HIP_NO_FUSION"]
     c.close()
     assert not any(k["klass"] == "attention-mfma" for k in info_plain)
-    # per layer: six attention kernels became one, three pointwise kernels (attention
+    # per layer: six attention kernels and the three copies that split q, k and v out of
+    # the fused projection became one, three pointwise kernels (attention
     # residual, GELU, MLP residual) moved into the epilogue of the matmul in front of them,
     # and each LayerNorm (two per layer and the final one) runs its three kernels as one
     n_ln = 2 * cfg.n_layer + 1
-    assert len(info_plain) == len(info) + (5 + 3) * cfg.n_layer + 2 * n_ln
+    assert len(info_plain) == len(info) + (8 + 3) * cfg.n_layer + 2 * n_ln
     assert sum("in the epilogue" in k["desc"] for k in info) == 3 * cfg.n_layer
     assert sum("row chain of 3 kernels" in k["desc"] for k in info) == n_ln
     h, p = logits(got, bufs), logits(plain, bufs)

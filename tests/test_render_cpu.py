@@ -142,7 +142,7 @@ int main(void) {
 
 def test_kernel_groups_of_the_gpt2_plan_fuse_and_compile(hiplib):
     """Needs no device: in the benchmark schedule the plan compiler recognises, per layer,
-    one attention group (six scheduled kernels), three matmuls followed by a pointwise
+    one attention group (six scheduled kernels plus the three q/k/v copies), three matmuls followed by a pointwise
     kernel (residual add, GELU, residual add) and two LayerNorms of three kernels each
     (plus the final LayerNorm); the generated sources compile."""
     from polygrad_amd import PlanFile
@@ -155,7 +155,7 @@ def test_kernel_groups_of_the_gpt2_plan_fuse_and_compile(hiplib):
         hiplib.poly_hip_fused_groups(pf.schedule, i, C.byref(src), C.byref(n))
         text = _ffi.take_string(src.value)
         kind = "attention" if "POLY_FA_M" in text else "rows" if "poly_row_p0" in text else "tail"
-        assert n.value == {"attention": 6, "tail": 2, "rows": 3}[kind]
+        assert n.value == {"attention": 9, "tail": 2, "rows": 3}[kind]
         seen.setdefault(kind, []).append(text)
     assert len(seen["attention"]) == 12 and len(seen["tail"]) == 36 and len(seen["rows"]) == 25
     assert hiplib.poly_hip_compile_check(seen["rows"][0].encode()) == 0
