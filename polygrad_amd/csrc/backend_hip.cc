@@ -82,7 +82,12 @@ HipRunner *runner_from_rendered(const RenderedKernel &rk, const char *fn_name, b
     r->fallback = program_create(r->rk.fallback_source, r->rk.fallback_entry);
     if (!r->fallback) { runner_destroy(r); return nullptr; }
   }
-  size_t n = (size_t)r->rk.n_params + (size_t)r->rk.n_vars + 1;
+  for (const RenderedKernel::Table &t : r->rk.tables) {
+    std::shared_ptr<void> tab = runtime_table(t.source, t.entry, t.bytes, t.launch);
+    if (!tab) { runner_destroy(r); return nullptr; }
+    r->tables.push_back(tab);
+  }
+  size_t n = (size_t)r->rk.n_params + (size_t)r->rk.n_vars + r->rk.tables.size() + 1;
   r->ptr_store.resize(n);
   r->var_store.resize(n);
   r->arg_ptrs.resize(n);
@@ -115,11 +120,16 @@ int runner_launch(HipRunner *r, void **args, int n_args) {
     r->var_store[(size_t)v] = *(const int *)args[np + v];
     r->arg_ptrs[(size_t)(np + v)] = &r->var_store[(size_t)v];
   }
+  const int nt = (int)r->tables.size();
+  for (int t = 0; t < nt; t++) {
+    r->ptr_store[(size_t)(np + nv + t)] = r->tables[(size_t)t].get();
+    r->arg_ptrs[(size_t)(np + nv + t)] = &r->ptr_store[(size_t)(np + nv + t)];
+  }
   if (r->guards.empty()) return program_launch(r->main, r->arg_ptrs.data(), r->rk.launch);
   // The guard writes *flag (1 = fast path valid, 0 = not); the fast kernel and
   // its generic twin both launch and exactly one of them does the work.
-  r->ptr_store[(size_t)(np + nv)] = r->flag;
-  r->arg_ptrs[(size_t)(np + nv)] = &r->ptr_store[(size_t)(np + nv)];
+  r->ptr_store[(size_t)(np + nv + nt)] = r->flag;
+  r->arg_ptrs[(size_t)(np + nv + nt)] = &r->ptr_store[(size_t)(np + nv + nt)];
   for (size_t gi = 0; gi < r->guards.size(); gi++) {
     const RenderedKernel::Guard &gd = r->rk.guards[gi];
     std::vector<void *> gargs;

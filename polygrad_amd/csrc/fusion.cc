@@ -231,6 +231,57 @@ bool internal_loads_replaced(const Sched &sc, const Member &m, const std::set<in
 
 }  // namespace
 
+// Does the value of `node` depend on nothing but the member's preset nodes (no other
+// load, no range, no variable)?  Counts the arithmetic nodes on the way.
+static bool only_depends_on_presets(const KernelGraph &g, const Member &m, int node, int *n_alu) {
+  std::vector<int> st{node};
+  std::set<int> seen;
+  while (!st.empty()) {
+    const int id = st.back(); st.pop_back();
+    if (!seen.insert(id).second || m.preset.count(id)) continue;
+    const KNode &k = g.n(id);
+    if (k.op == POLY_OP_LOAD || k.op == POLY_OP_RANGE || k.op == POLY_OP_DEFINE_VAR || k.op == POLY_OP_REDUCE ||
+        k.op == POLY_OP_SPECIAL || k.op == POLY_OP_INDEX || k.op == POLY_OP_PARAM || k.op == POLY_OP_BIND) return false;
+    if (k.op != POLY_OP_CONST) (*n_alu)++;
+    for (int sidx : k.src) st.push_back(sidx);
+  }
+  return true;
+}
+
+// A pointwise kernel whose result is a function of ONE 16-bit value has only 65536
+// possible results: a table filled once by the kernel's own expression replaces the
+// arithmetic (bit-identical by construction, and a gather instead of dozens of VALU
+// instructions per element when the expression rounds to 16 bits after every step).
+static bool make_unary_table(const Sched &sc, const Member &m, RenderedKernel::Table *t, std::string *out_type) {
+  const KernelGraph &g = sc.graphs[(size_t)m.item];
+  const StoreInfo &st = g.stores[0];
+  if (m.preset.size() != 1) return false;
+  const KNode &in = g.n(m.preset.begin()->first);
+  if (in.dt != DT_BF16 && in.dt != DT_F16) return false;
+  const DT odt = g.n(st.value).dt;
+  if (dt_size(odt) > 4 || odt == DT_BOOL) return false;
+  int n_alu = 0;
+  if (!only_depends_on_presets(g, m, st.value, &n_alu) || n_alu < 8) return false;
+  Emitter em(g);
+  Scope S0;
+  S0.indent = 1;
+  em.preset(m.preset.begin()->first, "x");
+  std::string v = em.emit(st.value, &S0);
+  if (em.failed() || em.uses_threefry) return false;
+  t->source = std::string(hip_prelude()) +
+              strf("extern \"C\" __global__ void __launch_bounds__(256) poly_lut_fill(%s* out) {\n"
+                   "  const unsigned int i = blockIdx.x * 256u + threadIdx.x;\n"
+                   "  const %s x = __builtin_bit_cast(%s, (unsigned short)i);\n",
+                   dt_cname(odt), dt_cname(in.dt), dt_cname(in.dt)) +
+              S0.code + strf("  out[i] = %s;\n}\n", v.c_str());
+  t->entry = "poly_lut_fill";
+  t->bytes = (size_t)65536 * (size_t)dt_size(odt);
+  t->launch.grid[0] = 256;
+  t->launch.block[0] = 256;
+  *out_type = dt_cname(odt);
+  return true;
+}
+
 // A matmul whose result only feeds a chain of pointwise kernels (bias/activation/residual
 // realised as kernels of their own): the chain becomes the matmul's epilogue.
 static bool match_matmul_tail(const Sched &sc, int s_item, const std::vector<char> &taken, FusedGroup *out) {
@@ -300,22 +351,81 @@ static bool match_matmul_tail(const Sched &sc, int s_item, const std::vector<cha
                       {{mS.red, "acc"}}, false, false, &ep.code)) FA_REJECT();
   std::string call = strf("poly_ep_s(acc, m, n, z, %s)", call_args(s_item).c_str());
   DT prev_dt = gS.n(stS.value).dt;
+  std::vector<RenderedKernel::Table> tables;
+  std::map<size_t, int> table_of;     // member -> table index
+  std::map<size_t, std::string> lead_of, lut_arg_of;
   for (size_t e = 1; e < members.size(); e++) {
     const Member &m = members[e];
     const KernelGraph &g = sc.graphs[(size_t)m.item];
     const bool last = e + 1 == members.size();
     const std::string fn = strf("poly_ep_e%zu", e);
-    if (!emit_member_fn(sc, m, master_decomp, fn.c_str(), dt_cname(g.n(g.stores[0].value).dt), strf("%s x", dt_cname(prev_dt)),
-                        g.stores[0].value, {}, false, last, &ep.code)) FA_REJECT();
-    call = strf("%s(%s, m, n, z, %s)", fn.c_str(), call.c_str(), call_args(m.item).c_str());
+    std::string lead = strf("%s x", dt_cname(prev_dt));
+    std::map<int, std::string> extra;
+    RenderedKernel::Table tab;
+    std::string tab_type;
+    if (!getenv("POLY_HIP_NO_LUT") && make_unary_table(sc, m, &tab, &tab_type)) {
+      table_of[e] = (int)tables.size();
+      lead += strf(", const %s* __restrict__ poly_lut", tab_type.c_str());
+      lut_arg_of[e] = strf(", poly_lut%zu", tables.size());
+      extra[g.stores[0].value] = "poly_lut[__builtin_bit_cast(unsigned short, x)]";
+      ep.signature += strf(", const %s* __restrict__ poly_lut%zu", tab_type.c_str(), tables.size());
+      tables.push_back(tab);
+    }
+    lead_of[e] = lead;
+    if (!emit_member_fn(sc, m, master_decomp, fn.c_str(), dt_cname(g.n(g.stores[0].value).dt), lead, g.stores[0].value, extra, false, last,
+                        &ep.code)) FA_REJECT();
+    call = strf("%s(%s%s, m, n, z, %s)", fn.c_str(), call.c_str(), lut_arg_of.count(e) ? lut_arg_of[e].c_str() : "", call_args(m.item).c_str());
     prev_dt = g.n(g.stores[0].value).dt;
   }
   ep.call = call;
+  {
+    // value and address of the last kernel's store, separately, when rows are contiguous
+    const Member &m = members.back();
+    const KernelGraph &g = sc.graphs[(size_t)m.item];
+    const StoreInfo &st = g.stores[0];
+    const int li = g.n(g.n(st.index).src[1]).lin;
+    Aff a;
+    const MmDim &inner = mS.nd_full.back();
+    const bool contiguous = li >= 0 && lin_to_aff(g, g.lins[(size_t)li], m.rm, &a) && inner.cut == 1 && a.c.count(inner.ord) &&
+                            a.c[inner.ord] == 1 && (mS.nd_full.size() == 1 || inner.extent % 8 == 0) &&
+                            g.n(st.value).dt == g.n(st.param).dt;
+    if (contiguous) {
+      // `call` is f_last(f_prev(...)): the same chain with the value form of the last link
+      const std::string fn = strf("poly_ep_e%zuv", members.size() - 1);
+      const size_t open = call.find('(');
+      std::string vcall = fn + call.substr(open);
+      std::string code2;
+      DT before = members.size() >= 3 ? sc.graphs[(size_t)members[members.size() - 2].item].n(sc.graphs[(size_t)members[members.size() - 2].item].stores[0].value).dt
+                                      : gS.n(stS.value).dt;
+      (void)before;
+      const size_t le = members.size() - 1;
+      std::map<int, std::string> extra;
+      if (table_of.count(le)) extra[st.value] = "poly_lut[__builtin_bit_cast(unsigned short, x)]";
+      bool ok = emit_member_fn(sc, m, master_decomp, fn.c_str(), dt_cname(g.n(st.value).dt), lead_of[le], st.value, extra, false, false, &code2);
+      // address: the store index in master coordinates
+      Emitter ea(g);
+      Scope Sa;
+      Sa.indent = 1;
+      for (auto &kv : m.rm) { ea.bind_range(kv.first, strf("r%d", kv.second)); Sa.avail |= (uint64_t)1 << kv.first; }
+      std::string idx = ea.emit(g.n(st.index).src[1], &Sa);
+      if (ok && !ea.failed()) {
+        ep.out_type = dt_cname(g.n(st.param).dt);
+        code2 += strf("__device__ __forceinline__ %s* poly_ep_ptr(int m, int n, int z, %s) {\n", ep.out_type.c_str(), params_decl(g).c_str());
+        code2 += master_decomp + Sa.code + strf("  return data%d + %s;\n}\n", g.param_slot(st.param), idx.c_str());
+        ep.code += code2;
+        ep.value_call = vcall;
+        ep.ptr_call = strf("poly_ep_ptr(m, n, z, %s)", call_args(m.item).c_str());
+        ep.contiguous_n = true;
+      }
+    }
+  }
   ep.a_ptr = strf("fa%d", arg_of(sc.slot(s_item, mS.A.param)));
   ep.b_ptr = strf("fa%d", arg_of(sc.slot(s_item, mS.B.param)));
   ep.n_params = (int)arg_slots.size();
   if (!render_matmul(mS, ep, &out->rk)) return false;
+  out->rk.tables = tables;
   out->rk.strategy += strf(" + %zu pointwise kernel%s in the epilogue", members.size() - 1, members.size() > 2 ? "s" : "");
+  if (!tables.empty()) out->rk.strategy += strf(" (%zu as a 16-bit lookup table)", tables.size());
   out->items = items;
   out->launch_item = last_item;
   out->internal_slots.assign(internal.begin(), internal.end());

@@ -17,6 +17,10 @@
 //   POLY_SIGNATURE      the kernel's parameter list
 //   POLY_EPILOGUE(acc, m, n, z)   stores one finished element (generated from the
 //                       UOps around the REDUCE: casts, bias, activation, index)
+//   POLY_EP_CONTIG      1 when consecutive n of a row are consecutive in memory; then
+//                       POLY_EP_TYPE, POLY_EP_VALUE(acc, m, n, z) and POLY_EP_PTR(m, n, z)
+//                       give the element type, value and address separately and the
+//                       template writes 8 values of a row with one store
 //
 // Data path: global --16B loads--> registers --(transpose if needed)--> LDS
 // [row][K] with padded rows, double buffered; each wave reads 16-byte A and B
@@ -48,6 +52,10 @@ __device__ __forceinline__ int poly_a_k(int k) { return k; }
 __device__ __forceinline__ int poly_b_k(int k) { return k * POLY_N; }
 #define POLY_SIGNATURE float *data0, const __bf16 *__restrict__ data1, const __bf16 *__restrict__ data2
 #define POLY_EPILOGUE(acc, m, n, z) data0[(m) * POLY_N + (n)] = (acc)
+#define POLY_EP_CONTIG 1
+#define POLY_EP_TYPE float
+#define POLY_EP_VALUE(acc, m, n, z) (acc)
+#define POLY_EP_PTR(m, n, z) (data0 + (m) * POLY_N + (n))
 #endif
 
 typedef POLY_TIN poly_in8 __attribute__((ext_vector_type(8)));
@@ -358,9 +366,9 @@ extern "C" __global__ void __launch_bounds__(POLY_NTHREADS) poly_k(POLY_SIGNATUR
   // per-wave LDS staging area and comes back with 8 consecutive columns of one row per
   // lane, so that whatever the epilogue loads and stores along n is 16 bytes wide (for
   // 16-bit data) and a wave writes full 64-byte row segments.
-#if POLY_N % 8 != 0
-  // Rows of the output do not start on 16-byte boundaries: store straight from the
-  // accumulator layout, where the 32 lanes of a half-wave write 32 consecutive columns.
+#if !POLY_EP_CONTIG && POLY_N % 8 != 0
+  // Neither rows of 8 nor contiguous: store straight from the accumulator layout, where
+  // the 32 lanes of a half-wave write 32 consecutive columns.
 #pragma unroll
   for (int i = 0; i < POLY_TM; i++)
 #pragma unroll
@@ -395,10 +403,34 @@ extern "C" __global__ void __launch_bounds__(POLY_NTHREADS) poly_k(POLY_SIGNATUR
         const poly_f32x4 hi = *(const poly_f32x4 *)(stage + row * POLY_STAGE_LD + c0 + 4);
         const float v[8] = {lo[0], lo[1], lo[2], lo[3], hi[0], hi[1], hi[2], hi[3]};
         const int m = m0 + wm + i * 32 + row, n = n0 + wn + j * 32 + c0;
+#if POLY_EP_CONTIG
+        if (m < POLY_M && n < POLY_N) {
+          // 8 finished values of one row; a full group goes out as one store (rows need
+          // not start on 16-byte boundaries: global stores take any alignment)
+          typedef POLY_EP_TYPE poly_out8 __attribute__((ext_vector_type(8)));
+          typedef poly_out8 poly_out8_u __attribute__((aligned(sizeof(POLY_EP_TYPE))));
+          poly_out8 o;
+#pragma unroll
+          for (int e = 0; e < 8; e++) {
+            // (keep n + e plain when every group is full: whatever the epilogue loads
+            // along n must stay visibly consecutive to be fetched as one vector)
+            const int ne = (POLY_N % 8 == 0 || n + e < POLY_N) ? n + e : n;
+            o[e] = POLY_EP_VALUE(v[e], m, ne, z);
+          }
+          if (POLY_N % 8 == 0 || n + 7 < POLY_N) {
+            *(poly_out8_u *)POLY_EP_PTR(m, n, z) = o;
+          } else {
+#pragma unroll
+            for (int e = 0; e < 8; e++)
+              if (n + e < POLY_N) *POLY_EP_PTR(m, n + e, z) = o[e];
+          }
+        }
+#else
         if (m < POLY_M && n < POLY_N) {
 #pragma unroll
           for (int e = 0; e < 8; e++) { POLY_EPILOGUE(v[e], m, n + e, z); }
         }
+#endif
       }
       __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
       __builtin_amdgcn_wave_barrier();

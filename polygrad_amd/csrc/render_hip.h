@@ -44,6 +44,15 @@ struct RenderedKernel {
     std::vector<int> arg_params;   // which buffer params the check reads
   };
   std::vector<Guard> guards;
+  // Lookup tables the kernel reads: `source` holds a kernel `entry(T* out)` that fills
+  // `bytes` bytes once, when the runner is created; the table pointers follow the
+  // buffer and variable arguments of every launch (before the guard flag).
+  struct Table {
+    std::string source, entry;
+    size_t bytes = 0;
+    LaunchSpec launch;
+  };
+  std::vector<Table> tables;
   std::string fallback_source, fallback_entry;
   LaunchSpec fallback_launch;
 };

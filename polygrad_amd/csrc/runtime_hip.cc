@@ -16,6 +16,7 @@
 
 #include <cstdlib>
 #include <cstring>
+#include <unordered_map>
 #include <fstream>
 #include <map>
 #include <memory>
@@ -212,6 +213,27 @@ Program *program_create(const std::string &source, const std::string &entry) {
 }
 
 void program_destroy(Program *p) { delete p; }
+
+std::shared_ptr<void> runtime_table(const std::string &source, const std::string &entry, size_t bytes, const LaunchSpec &ls) {
+  if (runtime_init() != 0) return nullptr;
+  static std::unordered_map<uint64_t, std::weak_ptr<void>> cache;
+  const uint64_t h = fnv1a(source.data(), source.size()) ^ (uint64_t)bytes;
+  auto it = cache.find(h);
+  if (it != cache.end()) if (std::shared_ptr<void> live = it->second.lock()) return live;
+  void *buf = runtime_alloc(bytes);
+  if (!buf) return nullptr;
+  std::shared_ptr<void> owner(buf, [](void *p) { runtime_free(p); });
+  Program *prog = program_create(source, entry);
+  if (!prog) return nullptr;
+  void *arg = buf;
+  void *args[1] = {&arg};
+  int rc = program_launch(prog, args, ls);
+  if (rc == 0) rc = runtime_sync();
+  program_destroy(prog);
+  if (rc != 0) return nullptr;
+  cache[h] = owner;
+  return owner;
+}
 
 int program_launch(Program *p, void **kernel_args, const LaunchSpec &ls) {
   if (!p || runtime_init() != 0) return -1;

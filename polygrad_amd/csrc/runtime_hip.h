@@ -1,5 +1,6 @@
 // Internal C++ face of the device runtime (the C ABI wraps these).
 #pragma once
+#include <memory>
 #include <string>
 #include <vector>
 
@@ -18,6 +19,9 @@ void runtime_free(void *p);
 int runtime_copy(void *dst, const void *src, size_t n, int kind);
 int runtime_memset(void *p, int value, size_t n);
 int runtime_sync();
+// A device buffer of `bytes` bytes filled once by running kernel `entry(T* out)` of
+// `source` with the given launch; identical sources share one buffer.
+std::shared_ptr<void> runtime_table(const std::string &source, const std::string &entry, size_t bytes, const LaunchSpec &ls);
 
 bool compile_to_code_object(const std::string &source, std::vector<char> *code, std::string *log);
 Program *program_create(const std::string &source, const std::string &entry);
@@ -31,6 +35,7 @@ struct HipRunner {
   std::vector<Program *> guards;
   Program *fallback = nullptr;
   void *flag = nullptr;            // device int written by the guards
+  std::vector<std::shared_ptr<void>> tables;   // filled lookup tables (shared between identical kernels)
   std::string name;
   std::vector<void *> ptr_store;   // argument storage reused by every launch
   std::vector<int> var_store;

@@ -264,6 +264,22 @@ int64_t matmul_range_value(const MatmulMatch &mm, int ord, int64_t m, int64_t n,
   return v;
 }
 
+bool matmul_store_contiguous(const KernelGraph &g, const MatmulMatch &mm, const Lin &l) {
+  if (mm.nd_full.empty()) return false;
+  const MmDim &inner = mm.nd_full.back();
+  if (inner.cut != 1) return false;
+  if (mm.nd_full.size() > 1 && inner.extent % 8 != 0) return false;
+  bool aff;
+  const int64_t c = g.lin_range_coef(l, inner.ord, &aff);
+  if (!aff || c != 1) return false;
+  // a range split into several digits contributes through / and % atoms: not affine
+  for (const Term &t : l.terms) {
+    const Atom &a = g.atoms[(size_t)t.atom];
+    if (a.kind != Atom::RANGE && (g.atom_deps(t.atom) & ((uint64_t)1 << inner.ord))) return false;
+  }
+  return true;
+}
+
 bool try_render_matmul(const KernelGraph &g, const std::string &fn, const RenderOptions &opt, RenderedKernel *out) {
   (void)fn; (void)opt;
   MatmulMatch mm;
@@ -294,6 +310,32 @@ bool try_render_matmul(const KernelGraph &g, const std::string &fn, const Render
   ep.code += decomp + S0.code;
   ep.code += strf("  data%d[%s] = %s;\n}\n", pout, idx.c_str(), val.c_str());
   ep.call = strf("poly_epilogue(acc, m, n, z, %s)", params_call.c_str());
+  {
+    const int li = g.n(g.n(st.index).src[1]).lin;
+    const DT odt = g.n(st.param).dt;
+    if (li >= 0 && g.n(st.value).dt == odt && matmul_store_contiguous(g, mm, g.lins[(size_t)li])) {
+      // the same code once more, split into the value and the address of an element
+      Emitter ev(g), ea(g);
+      Scope Sv, Sa;
+      Sv.indent = Sa.indent = 1;
+      Sv.avail = Sa.avail = S0.avail;
+      matmul_decompose(mm, &ev);
+      matmul_decompose(mm, &ea);
+      ev.preset(mm.red, "acc");
+      std::string v2 = ev.emit(st.value, &Sv);
+      std::string i2 = ea.emit(g.n(st.index).src[1], &Sa);
+      if (!ev.failed() && !ea.failed()) {
+        ep.out_type = dt_cname(odt);
+        ep.code += strf("__device__ __forceinline__ %s poly_ep_value(float acc, int m, int n, int z, %s) {\n", ep.out_type.c_str(), ep.signature.c_str());
+        ep.code += decomp + Sv.code + strf("  return %s;\n}\n", v2.c_str());
+        ep.code += strf("__device__ __forceinline__ %s* poly_ep_ptr(int m, int n, int z, %s) {\n", ep.out_type.c_str(), ep.signature.c_str());
+        ep.code += decomp + Sa.code + strf("  return data%d + %s;\n}\n", pout, i2.c_str());
+        ep.value_call = strf("poly_ep_value(acc, m, n, z, %s)", params_call.c_str());
+        ep.ptr_call = strf("poly_ep_ptr(m, n, z, %s)", params_call.c_str());
+        ep.contiguous_n = true;
+      }
+    }
+  }
   ep.a_ptr = strf("data%d", mm.A.param);
   ep.b_ptr = strf("data%d", mm.B.param);
   ep.n_params = (int)g.params.size();
@@ -382,6 +424,13 @@ bool render_matmul(const MatmulMatch &mm, const MatmulEpilogue &ep, RenderedKern
   if (getenv("POLY_HIP_MM_NOEPI")) cfg += strf("#define POLY_EPILOGUE(acc, m, n, z) do { if (((m) | (n)) == -1) { %s; } } while (0)\n", ep.call.c_str());
   else
   cfg += strf("#define POLY_EPILOGUE(acc, m, n, z) %s\n", ep.call.c_str());
+  const bool split = ep.contiguous_n && !getenv("POLY_HIP_MM_NOEPI") && (ep.out_type == "__bf16" || ep.out_type == "_Float16" || ep.out_type == "float");
+  cfg += strf("#define POLY_EP_CONTIG %d\n", split ? 1 : 0);
+  if (split) {
+    cfg += strf("#define POLY_EP_TYPE %s\n", ep.out_type.c_str());
+    cfg += strf("#define POLY_EP_VALUE(acc, m, n, z) %s\n", ep.value_call.c_str());
+    cfg += strf("#define POLY_EP_PTR(m, n, z) %s\n", ep.ptr_call.c_str());
+  }
 
   *out = RenderedKernel();
   out->source = std::string(hip_prelude()) + cfg + kMatmulTemplate;

@@ -52,10 +52,21 @@ int64_t matmul_range_value(const MatmulMatch &mm, int ord, int64_t m, int64_t n,
 // its pointers are the operands, device functions, and the statement (in terms of acc, m,
 // n, z) that finishes one output element.
 struct MatmulEpilogue {
-  std::string signature, a_ptr, b_ptr, code, call;
+  std::string signature, a_ptr, b_ptr, code;
+  std::string call;        // statement storing one element: uses acc, m, n, z
+  // Optional split of `call` into value and address, for outputs that are contiguous
+  // along n: the template then stores 8 values of a row with one 16-byte store.
+  std::string value_call;  // expression of type out_type: uses acc, m, n, z
+  std::string ptr_call;    // expression of type out_type*: uses m, n, z
+  std::string out_type;
+  bool contiguous_n = false;
   int n_params = 0;
   double bytes = 0;    // algorithmic bytes of the whole kernel
 };
+// Is element (m, n + 1) of the kernel's output stored right after (m, n), for every n
+// that is not the last of an aligned group of 8?  (store index affine with coefficient 1
+// on the innermost digit of n, digits not crossed inside a group)
+bool matmul_store_contiguous(const KernelGraph &g, const MatmulMatch &mm, const Lin &store_lin);
 // Chooses layouts and tile shape and instantiates kernels/matmul_mfma.hip.
 bool render_matmul(const MatmulMatch &mm, const MatmulEpilogue &ep, RenderedKernel *out);
 

@@ -64,3 +64,30 @@ def test_fused_attention_matches_unfused_and_reference(qk_gain):
     e_fused = float(np.sqrt(np.mean((h - want) ** 2)))
     e_plain = float(np.sqrt(np.mean((p - want) ** 2)))
     assert e_fused <= 1.5 * e_plain + 1e-6 * scale, (e_fused, e_plain)
+
+
+def test_lookup_table_epilogue_is_bit_identical_to_the_arithmetic():
+    """A pointwise kernel of one 16-bit input fused behind a matmul is evaluated through a
+    65536-entry table filled by its own expression: results must not change by a bit."""
+    m, n, k = 512, 768, 256
+    g = np.random.default_rng(21)
+    c = R.Ctx()
+    A = c.buffer((m, k), R.BF16, name="A")
+    W = c.buffer((k, n), R.BF16, name="W")
+    O = c.buffer((m, n), R.BF16, name="O")
+    y = A.cast(R.F32).dot(W.cast(R.F32)).cast(R.BF16).contiguous()
+    sink = c.sink((O, y.gelu()))
+    arrays = {A: R.f32_to_bf16_bits(g.normal(0, 1.0, m * k).astype(np.float32)),
+              W: R.f32_to_bf16_bits(g.normal(0, 0.2, k * n).astype(np.float32)), O: np.zeros(m * n, np.uint16)}
+    with_table, info = run_hip(c, sink, arrays)
+    assert any("lookup table" in kk["desc"] for kk in info), [kk["desc"] for kk in info]
+    os.environ["POLY_HIP_NO_LUT"] = "1"
+    try:
+        plain, info2 = run_hip(c, sink, arrays)
+    finally:
+        del os.environ["POLY_HIP_NO_LUT"]
+    assert not any("lookup table" in kk["desc"] for kk in info2) and len(info2) == len(info)
+    assert with_table[O].tobytes() == plain[O].tobytes()
+    want = run_ref(c, sink, arrays)
+    c.close()
+    assert_close(R.bf16_bits_to_f32(with_table[O]), R.bf16_bits_to_f32(want[O]), rtol=2e-2, atol=2e-2, what="matmul + GELU vs reference")
