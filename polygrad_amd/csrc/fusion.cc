@@ -120,7 +120,16 @@ struct Member {
   int item = -1;
   RangeMap rm;
   std::map<int, std::string> preset;   // node -> C expression replacing it
+  // ranges bound to an expression of master ranges instead of to one of them (a kernel
+  // that walks the buffer with ONE flattened range: the expression is the flat position)
+  std::map<int, std::string> range_expr;
 };
+
+std::string aff_expr(const Aff &a) {
+  std::string e = strf("%lld", (long long)a.c0);
+  for (auto &kv : a.c) e += strf(" + %lld * r%d", (long long)kv.second, kv.first);
+  return "(" + e + ")";
+}
 
 std::string params_decl(const KernelGraph &g) {
   std::string d;
@@ -145,15 +154,36 @@ bool pointwise_member(const Sched &sc, int item, int cur, const Aff &prod, const
   const int p = sc.param_of(item, cur);
   if (p < 0 || !loads_of(g, p, &lds) || lds.empty()) return false;
   m->item = item;
+  const int li = g.n(g.n(g.stores[0].index).src[1]).lin;
+  if (li < 0) return false;
+  const int outp = g.param_slot(g.stores[0].param);
+  // a kernel over one flattened range p that reads and writes element p
+  auto is_flat = [&](const Lin &l, int ord) {
+    if (l.c0 != 0 || l.terms.size() != 1 || l.terms[0].coef != 1) return false;
+    const Atom &a = g.atoms[(size_t)l.terms[0].atom];
+    return a.kind == Atom::RANGE && g.range_ord.at(a.node) == ord;
+  };
+  if (g.stores[0].ranges.size() == 1 && prod.c0 == 0) {
+    const int ord = g.stores[0].ranges[0];
+    bool flat = g.ranges[(size_t)ord].extent == s->buf_slots[cur].numel && is_flat(g.lins[(size_t)li], ord);
+    for (const LoadRef &l : lds) flat = flat && is_flat(g.lins[(size_t)l.lin], ord);
+    // the producer must cover [0, numel) densely for the flat position to be its index
+    int64_t span = 1;
+    for (auto &kv : prod.c) span += (mext[(size_t)kv.first] - 1) * kv.second;
+    if (flat && span == s->buf_slots[cur].numel && prod.c.size() > 1) {
+      for (const LoadRef &l : lds) m->preset[l.node] = value_name;
+      m->range_expr[ord] = aff_expr(prod);
+      if (outp == p || s->buf_slots[sc.slot(item, outp)].numel != s->buf_slots[cur].numel) return false;
+      return true;
+    }
+  }
   for (const LoadRef &l : lds) {
     if (!derive_map(g, g.lins[(size_t)l.lin], prod, mext, &m->rm)) return false;
     m->preset[l.node] = value_name;
   }
   for (int r : g.stores[0].ranges) if (!m->rm.count(r)) return false;
-  const int li = g.n(g.n(g.stores[0].index).src[1]).lin;
   Aff a;
-  if (li < 0 || !lin_to_aff(g, g.lins[(size_t)li], m->rm, &a) || !(a == prod)) return false;
-  const int outp = g.param_slot(g.stores[0].param);
+  if (!lin_to_aff(g, g.lins[(size_t)li], m->rm, &a) || !(a == prod)) return false;
   if (outp == p || s->buf_slots[sc.slot(item, outp)].numel != s->buf_slots[cur].numel) return false;
   return true;
 }
@@ -171,6 +201,12 @@ bool emit_member_fn(const Sched &sc, const Member &m, const std::string &master_
   Scope S0;
   S0.indent = 1;
   for (auto &kv : m.rm) { em.bind_range(kv.first, strf("r%d", kv.second)); S0.avail |= (uint64_t)1 << kv.first; }
+  std::string flat_decl;
+  for (auto &kv : m.range_expr) {
+    flat_decl += strf("  const int p%d = %s;\n", kv.first, kv.second.c_str());
+    em.bind_range(kv.first, strf("p%d", kv.first));
+    S0.avail |= (uint64_t)1 << kv.first;
+  }
   for (auto &kv : m.preset) em.preset(kv.first, kv.second);
   for (auto &kv : extra_preset) em.preset(kv.first, kv.second);
   std::string v = em.emit(node, &S0);
@@ -179,7 +215,7 @@ bool emit_member_fn(const Sched &sc, const Member &m, const std::string &master_
   if (em.failed() || em.uses_threefry) return false;
   *code += strf("__device__ __forceinline__ %s %s(%s, int m, int n, int z, %s) {\n", as_store ? "void" : ret, name, lead_args.c_str(),
                 params_decl(g).c_str());
-  *code += master_decomp + S0.code;
+  *code += master_decomp + flat_decl + S0.code;
   if (as_store) *code += strf("  data%d[%s] = %s;\n}\n", g.param_slot(g.stores[0].param), idx.c_str(), v.c_str());
   else *code += strf("  return %s;\n}\n", v.c_str());
   return true;
@@ -386,7 +422,9 @@ static bool match_matmul_tail(const Sched &sc, int s_item, const std::vector<cha
     const int li = g.n(g.n(st.index).src[1]).lin;
     Aff a;
     const MmDim &inner = mS.nd_full.back();
-    const bool contiguous = li >= 0 && lin_to_aff(g, g.lins[(size_t)li], m.rm, &a) && inner.cut == 1 && a.c.count(inner.ord) &&
+    bool have_aff = li >= 0 && lin_to_aff(g, g.lins[(size_t)li], m.rm, &a);
+    if (!have_aff && !m.range_expr.empty()) { a = aS; have_aff = true; }   // flat kernel: it stores where the matmul would have
+    const bool contiguous = have_aff && inner.cut == 1 && a.c.count(inner.ord) &&
                             a.c[inner.ord] == 1 && (mS.nd_full.size() == 1 || inner.extent % 8 == 0) &&
                             g.n(st.value).dt == g.n(st.param).dt;
     if (contiguous) {
@@ -407,11 +445,17 @@ static bool match_matmul_tail(const Sched &sc, int s_item, const std::vector<cha
       Scope Sa;
       Sa.indent = 1;
       for (auto &kv : m.rm) { ea.bind_range(kv.first, strf("r%d", kv.second)); Sa.avail |= (uint64_t)1 << kv.first; }
+      std::string flat_decl;
+      for (auto &kv : m.range_expr) {
+        flat_decl += strf("  const int p%d = %s;\n", kv.first, kv.second.c_str());
+        ea.bind_range(kv.first, strf("p%d", kv.first));
+        Sa.avail |= (uint64_t)1 << kv.first;
+      }
       std::string idx = ea.emit(g.n(st.index).src[1], &Sa);
       if (ok && !ea.failed()) {
         ep.out_type = dt_cname(g.n(st.param).dt);
         code2 += strf("__device__ __forceinline__ %s* poly_ep_ptr(int m, int n, int z, %s) {\n", ep.out_type.c_str(), params_decl(g).c_str());
-        code2 += master_decomp + Sa.code + strf("  return data%d + %s;\n}\n", g.param_slot(st.param), idx.c_str());
+        code2 += master_decomp + flat_decl + Sa.code + strf("  return data%d + %s;\n}\n", g.param_slot(st.param), idx.c_str());
         ep.code += code2;
         ep.value_call = vcall;
         ep.ptr_call = strf("poly_ep_ptr(m, n, z, %s)", call_args(m.item).c_str());
