@@ -37,6 +37,7 @@
 #define POLY_BN 128
 #define POLY_BK 64
 #define POLY_GROUP_M 8
+#define POLY_GROUP_ALONG_N 0
 #define POLY_PIPE 3
 #define POLY_WAVES_M 2
 #define POLY_WAVES_N 2
@@ -174,17 +175,28 @@ extern "C" __global__ void __launch_bounds__(POLY_NTHREADS) poly_k(POLY_SIGNATUR
     const int xcd = bid & 7, idx = bid >> 3;
     bid = (xcd < REM ? xcd * (PER + 1) : REM * (PER + 1) + (xcd - REM) * PER) + idx;
   }
-  // Within a run, tiles are visited in groups of POLY_GROUP_M tile rows so that the
-  // workgroups resident on one XCD at a time share both A and B panels.
+  // Within a run, tiles are visited in bands of POLY_GROUP_M tile rows (walking along N
+  // inside a band) so that the workgroups resident on one XCD at a time share both A and
+  // B panels.  When B is the larger operand the roles swap (POLY_GROUP_ALONG_N): bands of
+  // tile columns, so that an XCD streams its slice of B once instead of all of B.
   int tile_m, tile_n;
   {
     constexpr int GM = POLY_GROUP_M;
+#if POLY_GROUP_ALONG_N
+    const int per_group = GM * TILES_M;
+    const int group = bid / per_group, first_n = group * GM;
+    const int gsz = (TILES_N - first_n) < GM ? (TILES_N - first_n) : GM;
+    const int in_group = bid - group * per_group;
+    tile_n = first_n + in_group % gsz;
+    tile_m = in_group / gsz;
+#else
     const int per_group = GM * TILES_N;
     const int group = bid / per_group, first_m = group * GM;
     const int gsz = (TILES_M - first_m) < GM ? (TILES_M - first_m) : GM;
     const int in_group = bid - group * per_group;
     tile_m = first_m + in_group % gsz;
     tile_n = in_group / gsz;
+#endif
   }
   const int z = blockIdx.y;
   const int m0 = tile_m * POLY_BM, n0 = tile_n * POLY_BN;

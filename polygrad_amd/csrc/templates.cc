@@ -401,6 +401,8 @@ bool render_matmul(const MatmulMatch &mm, const MatmulEpilogue &ep, RenderedKern
   cfg += strf("#define POLY_M %lld\n#define POLY_N %lld\n#define POLY_K %lld\n#define POLY_Z %lld\n", (long long)M, (long long)N, (long long)K, (long long)Z);
   cfg += strf("#define POLY_BM %d\n#define POLY_BN %d\n#define POLY_BK %d\n#define POLY_WAVES_M %d\n#define POLY_WAVES_N %d\n", BM, BN, BK, WVM, WVN);
   cfg += strf("#define POLY_GROUP_M %d\n", BM >= 256 ? 4 : 8);
+  // each XCD (own L2) works on a contiguous run of tiles: let it re-read the smaller operand
+  cfg += strf("#define POLY_GROUP_ALONG_N %d\n", (N > 2 * M && !getenv("POLY_HIP_MM_GROUP_M")) ? 1 : 0);
   // a 256x256 tile holds 128 accumulator registers per lane: no room for the second
   // staging register set of the three-deep pipeline
   int pipe = (BM * BN >= 256 * 256) ? 2 : 3;
