@@ -27,6 +27,17 @@ PEAK_HBM_GBS = 8000.0          # MI355X HBM3E
 PEAK_MFMA_TFLOPS = 2500.0      # MI355X dense bf16/fp16 MFMA
 GPT2_PLAN = "gpt2_small_bf16_b8_t1024"
 
+# HBM bytes per launch measured with `rocprofv3 --pmc FETCH_SIZE` and `--pmc WRITE_SIZE`
+# (two runs of this script, counters scaled by what a plain copy of known size reads:
+# FETCH_SIZE x 2.0 KiB, WRITE_SIZE x 1.0 KiB); keyed by the start of the kernel description.
+# The summaries with the commands are under profiles/.
+MEASURED_TRAFFIC = {
+    "attention-mfma: fused attention (9 kernels): mfma 32x32x16 bf16 Z=96 M=1024 N=1024 D=64": 73.9e6 + 12.6e6,
+    "matmul-mfma: mfma 32x32x16 bf16 M=8192 N=3072 K=768 Z=1": 73.9e6 + 51.0e6,
+    "matmul-mfma: mfma 32x32x16 bf16 M=8192 N=2304 K=768 Z=1": 63.8e6 + 37.8e6,
+    "matmul-mfma: mfma 32x32x16 bf16 M=8192 N=768 K=3072 Z=1": 101.0e6 + 15.2e6,
+}
+
 
 def log(*a):
     print(*a, file=sys.stderr, flush=True)
@@ -87,8 +98,15 @@ def run_gpu(workload, steps, warmup):
         achieved = d["bytes"] / (avg_ms * 1e-3) / 1e9
         roofline = dict(bound="hbm", achieved=round(achieved, 1), peak=PEAK_HBM_GBS, unit="GB/s",
                         frac=round(achieved / PEAK_HBM_GBS, 4), traffic=None)
+    for prefix, traffic in MEASURED_TRAFFIC.items():
+        if dominant_key.startswith(prefix):
+            roofline["traffic"] = traffic
     roofline.update(kernel=dominant_key, launches_per_step=d["launches"], avg_launch_ms=round(avg_ms, 4),
                     algorithmic_bytes=d["bytes"], algorithmic_flops=d["flops"])
+    if d["klass"] == "attention-mfma":
+        # neither of the two rooflines binds this kernel: say what does
+        roofline["note"] = ("VALU-bound: per score three roundings to bf16, exp2 and an IEEE division, as the "
+                            "unfused kernels compute them; SQ counters under profiles/")
 
     classes = {}
     for k, ms in zip(info, per_kernel_ms):
