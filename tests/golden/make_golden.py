@@ -3,7 +3,7 @@ plan (as a plan file) and the inputs plus the outputs computed by the REAL
 reference CPU backend (oracle/_ref/libpolygrad.so, built from /root/reference).
 
 Run from the repository root in the build container:
-    python tests/golden/make_golden.py
+    python tests/golden/make_golden.py [case ...]
 Writes tests/golden/<case>.polyplan and tests/golden/<case>.npz
 (npz keys: in<slot> = initial contents of external slot, out<slot> = contents
 after the reference ran).  bf16 data is stored as uint16 bit patterns.
@@ -25,7 +25,12 @@ from hipharness import schedule_slots  # noqa: E402
 from polygrad_amd import save_schedule  # noqa: E402
 
 
+ONLY = set(sys.argv[1:])     # optional: regenerate only the named cases
+
+
 def emit(name, c, sink, arrays):
+    if ONLY and name not in ONLY:
+        return
     want = {t: np.array(a, copy=True) for t, a in arrays.items()}
     c.realize_cpu(sink, want)
     sched = c.schedule(sink)
@@ -140,6 +145,56 @@ def main():
         arrays = graphs.gpt2_inputs(graphs.GPT2_TINY, bufs, seed=3, wdt=wdt)
         emit(f"gpt2_tiny_{nm}", c, sink, arrays)
         c.close()
+
+    # benchmark configuration 1 in small: MLP forward, cross-entropy, gradients, SGD step
+    # with in-place parameter updates (22 kernels; src/instance.c:1152-1224 builds the same
+    # p - lr * g ASSIGNs)
+    c = R.Ctx()
+    bufs, sink = graphs.mlp_train_step(c, batch=32, d_in=48, d_hid=40, d_out=10, lr=0.05)
+    arrays = {}
+    for name, t in bufs.items():
+        n = int(np.prod(t.shape))
+        if name == "X":
+            a = g.normal(0, 1, n)
+        elif name.startswith("W"):
+            lim = (6.0 / t.shape[1]) ** 0.5
+            a = g.uniform(-lim, lim, n)
+        elif name == "Y":
+            a = np.eye(10)[g.integers(0, 10, 32)].reshape(-1)
+        else:
+            a = np.zeros(n)
+        arrays[t] = a.astype(np.float32)
+    emit("mlp_train_b32", c, sink, arrays)
+    c.close()
+
+    # the kernel groups the plan compiler fuses, at the smallest shapes it takes them:
+    # attention (128-query blocks, 64 features per head), matmul + GELU, LayerNorm rows
+    c = R.Ctx()
+    bufs, sink = graphs.attention_bf16(c, batch=1, heads=2, ctx=256, hd=64)
+    arrays = {bufs[n]: R.f32_to_bf16_bits(g.normal(0, 1.0, 256 * 128).astype(np.float32)) for n in ("q", "k", "v")}
+    arrays[bufs["arange"]] = np.arange(256, dtype=np.float32)
+    arrays[bufs["out"]] = np.zeros(256 * 128, np.uint16)
+    emit("attention_bf16_t256", c, sink, arrays)
+    c.close()
+    c = R.Ctx()
+    A = c.buffer((128, 64), R.BF16, name="A")
+    W = c.buffer((64, 256), R.BF16, name="W")
+    bias = c.buffer((256,), R.BF16, name="bias")
+    O = c.buffer((128, 256), R.BF16, name="O")
+    y = (A.cast(R.F32).dot(W.cast(R.F32)).cast(R.BF16) + bias.reshape((1, 256)).expand((128, 256))).contiguous()
+    emit("bf16_matmul_gelu", c, c.sink((O, y.gelu())),
+         {A: R.f32_to_bf16_bits(g.normal(0, 1.0, 128 * 64).astype(np.float32)), W: R.f32_to_bf16_bits(g.normal(0, 0.3, 64 * 256).astype(np.float32)),
+          bias: R.f32_to_bf16_bits(g.normal(0, 0.1, 256).astype(np.float32)), O: np.zeros(128 * 256, np.uint16)})
+    c.close()
+    c = R.Ctx()
+    x = c.buffer((24, 256), R.BF16, name="x")
+    w = c.buffer((256,), R.BF16, name="w")
+    b = c.buffer((256,), R.BF16, name="b")
+    o = c.buffer((24, 256), R.BF16, name="o")
+    emit("bf16_layernorm_rows", c, c.sink((o, graphs._layernorm(x, w, b, 1e-5, R.BF16).contiguous())),
+         {x: R.f32_to_bf16_bits(g.normal(0.3, 2.0, 24 * 256).astype(np.float32)), w: R.f32_to_bf16_bits(g.normal(1, 0.1, 256).astype(np.float32)),
+          b: R.f32_to_bf16_bits(g.normal(0, 0.1, 256).astype(np.float32)), o: np.zeros(24 * 256, np.uint16)})
+    c.close()
 
 
 if __name__ == "__main__":

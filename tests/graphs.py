@@ -223,16 +223,34 @@ def attention_bf16(c, batch=8, heads=12, ctx=1024, hd=64):
 
 
 def mlp_train_step(c, batch=4096, d_in=784, d_hid=512, d_out=10, lr=0.01):
-    """Config 1: 2-layer MLP forward + backward + one SGD step, built from the public
-    ops (the reference's own loss entrypoints fail for batch > 1)."""
+    """Config 1: 2-layer MLP (weights stored (out, in) as the reference's model_mlp.c does),
+    softmax cross-entropy against one-hot labels, reverse-mode gradients from the
+    reference's poly_grad, one SGD step.  Returns (bufs, sink): the sink stores logits and
+    loss and updates the four parameters in place (ASSIGN)."""
     X = c.buffer((batch, d_in), name="X")
     W1 = c.buffer((d_hid, d_in), name="W1")
     b1 = c.buffer((d_hid,), name="b1")
     W2 = c.buffer((d_out, d_hid), name="W2")
     b2 = c.buffer((d_out,), name="b2")
     Y = c.buffer((batch, d_out), name="Y")  # one-hot labels
+    logits_out = c.buffer((batch, d_out), name="logits")
+    loss_out = c.buffer((1,), name="loss")
     h = (X.dot(W1.permute((1, 0))) + b1.reshape((1, d_hid)).expand((batch, d_hid))).relu()
     logits = h.dot(W2.permute((1, 0))) + b2.reshape((1, d_out)).expand((batch, d_out))
     logp = logits.log_softmax(-1)
     loss = (logp * Y).sum().sum(0) * c.const(-1.0 / batch)
-    return dict(X=X, W1=W1, b1=b1, W2=W2, b2=b2, Y=Y), logits, loss
+    pairs = []
+    for p in (W1, b1, W2, b2):
+        n = int(np.prod(p.shape))
+        g = T_grad(c, loss, p, n)
+        pairs.append((p, p.reshape((n,)) - g * c.const(lr)))
+    bufs = dict(X=X, W1=W1, b1=b1, W2=W2, b2=b2, Y=Y, logits=logits_out, loss=loss_out)
+    return bufs, c.sink_mixed([(logits_out, logits), (loss_out, loss.reshape((1,)))], pairs)
+
+
+def T_grad(c, loss, param, numel):
+    """d loss / d param as a flat tensor (reference poly_grad, src/autograd.c:773)."""
+    u = c.L.poly_grad(c.ctx, loss.u, param.buf)
+    if not u:
+        raise RuntimeError("poly_grad failed")
+    return R.T(c, u, (numel,), param.dt)

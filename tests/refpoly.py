@@ -165,6 +165,18 @@ class Ctx:
         arr = (C.c_void_p * len(srcs))(*srcs)
         return self.L.poly_sink_n(self.ctx, arr, len(srcs))
 
+    def sink_mixed(self, stores, assigns):
+        """One SINK holding plain stores (out buffer, value) and in-place updates (target, value)."""
+        srcs = []
+        for out, val in stores:
+            flat = val.reshape((int(np.prod(val.shape)) if val.shape else 1,))
+            srcs.append(self.L.poly_store_val(self.ctx, out.buf, flat.u))
+        for tgt, val in assigns:
+            flat = val.reshape((int(np.prod(val.shape)),))
+            srcs.append(self.L.poly_assign(self.ctx, tgt.buf, flat.u))
+        arr = (C.c_void_p * len(srcs))(*srcs)
+        return self.L.poly_sink_n(self.ctx, arr, len(srcs))
+
     # ── running the reference ──────────────────────────────────────────────
     def realize_cpu(self, sink, arrays):
         """Runs the reference CPU backend (fork+clang JIT). arrays: {buffer T: ndarray}."""

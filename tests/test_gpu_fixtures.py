@@ -19,7 +19,13 @@ TOL = {
     "special_exp2": (1e-5, 1e-38), "special_log2": (1e-5, 1e-6),
     "bf16_gelu": (2e-2, 1e-3), "bf16_matmul": (2e-2, 1e-6), "bf16_matmul_bt_batch": (2e-2, 1e-6),
     "f16_cast_mul": (2e-2, 0), "gpt2_tiny_f32": (1e-4, 1e-5), "gpt2_tiny_bf16": (2e-2, 2e-3),
+    "mlp_train_b32": (1e-4, 1e-5), "attention_bf16_t256": (2e-2, 2e-3), "bf16_matmul_gelu": (2e-2, 2e-3),
+    "bf16_layernorm_rows": (2e-2, 2e-3),
 }
+# plans that update their inputs in place: a second run would start from other parameters
+STATEFUL = {"mlp_train_b32"}
+# fixtures whose plan must come out as one of the fused kernel groups
+FUSED = {"attention_bf16_t256": "attention-mfma", "bf16_matmul_gelu": "lookup table", "bf16_layernorm_rows": "row chain of 3"}
 
 
 def run_fixture_on_gpu(fx, env_flags=None):
@@ -30,7 +36,8 @@ def run_fixture_on_gpu(fx, env_flags=None):
         dev[i] = to_device(fx.inputs[i])
     torch.cuda.synchronize()
     plan.run(dev)
-    plan.run(dev)  # second run replays the captured graph
+    if fx.name not in STATEFUL:
+        plan.run(dev)  # second run replays the captured graph
     out = {i: from_device(dev[i], fx.inputs[i].dtype) for i in fx.external}
     info = plan.kernel_info()
     plan.close()
@@ -40,7 +47,9 @@ def run_fixture_on_gpu(fx, env_flags=None):
 @pytest.mark.parametrize("name", F.case_names())
 def test_fixture_on_gpu(name):
     fx = F.Fixture(name)
-    got, _ = run_fixture_on_gpu(fx)
+    got, info = run_fixture_on_gpu(fx)
+    if name in FUSED:
+        assert any(FUSED[name] in k["desc"] for k in info), [k["desc"] for k in info]
     for slot in fx.external:
         want = fx.expected[slot]
         if name in BIT_EXACT:
