@@ -23,6 +23,10 @@ class PolyScheduleBufSlot(C.Structure):
                 ("buf_uop", C.c_void_p), ("is_intermediate", C.c_bool), ("external_buf_idx", C.c_int)]
 
 
+class PolyVarBinding(C.Structure):
+    _fields_ = [("var", C.c_void_p), ("value", C.c_int32)]
+
+
 class PolyExecItem(C.Structure):
     _fields_ = [("kind", C.c_int), ("root", C.c_void_p), ("buf_slot_indices", C.POINTER(C.c_int)),
                 ("n_buf_slots", C.c_int), ("fixedvars", C.c_void_p), ("n_fixedvars", C.c_int),
@@ -89,7 +93,7 @@ SYMBOLS = {
     "poly_hip_free_string": (None, [C.c_void_p]),
     "poly_hip_check_index_simplification": (C.c_int, [C.c_void_p, C.c_int]),
     "poly_hip_compile_schedule": (C.c_void_p, [C.c_void_p, C.c_void_p]),
-    "poly_hip_plan_run": (C.c_int, [C.c_void_p, C.POINTER(C.c_void_p), C.c_int, C.c_void_p, C.c_int]),
+    "poly_hip_plan_run": (C.c_int, [C.c_void_p, C.POINTER(C.c_void_p), C.c_int, C.POINTER(PolyVarBinding), C.c_int]),
     "poly_hip_plan_free": (None, [C.c_void_p]),
     "poly_hip_fused_groups": (C.c_int, [C.c_void_p, C.c_int, C.POINTER(C.c_void_p), C.POINTER(C.c_int)]),
     "poly_hip_plan_n_kernels": (C.c_int, [C.c_void_p]),

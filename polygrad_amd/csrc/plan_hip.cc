@@ -51,7 +51,8 @@ struct Unit {
   HipRunner *runner = nullptr;
   int item = -1;                 // schedule item (also for a fused group: the item it runs in place of)
   std::vector<int> slots;        // buffer slot per kernel argument
-  int n_vars = 0;                // DEFINE_VAR arguments (taken from `item`)
+  int n_vars = 0;                // DEFINE_VAR arguments of the kernel
+  std::vector<const PolyUOp *> var_uops;   // which variable each of them is
   int n_items = 1;               // schedule items this launch stands for
 };
 
@@ -182,14 +183,17 @@ PolyHipPlan *poly_hip_compile_schedule(PolyCtx *ctx, const PolySchedule *s) {
       u.n_items = (int)fg.items.size();
     } else {
       u.runner = runner_create(it.root, name.c_str(), 0);
-      if (u.runner && (u.runner->rk.n_params != it.n_buf_slots || u.runner->rk.n_vars != it.n_var_uops)) {
+      // (a kernel may use fewer variables than the schedule lists for it: a buffer sized by
+      // a variable that the kernel itself walks over its full allocation)
+      if (u.runner && (u.runner->rk.n_params != it.n_buf_slots || u.runner->rk.n_vars > it.n_var_uops)) {
         log_err("compile_schedule", "kernel %d: %d params / %d vars in the graph, %d / %d in the schedule", k,
                 u.runner->rk.n_params, u.runner->rk.n_vars, it.n_buf_slots, it.n_var_uops);
         runner_destroy(u.runner);
         return nullptr;
       }
       u.slots.assign(it.buf_slot_indices, it.buf_slot_indices + it.n_buf_slots);
-      u.n_vars = it.n_var_uops;
+      u.n_vars = u.runner ? u.runner->rk.n_vars : 0;
+      if (u.runner) for (const void *v : u.runner->rk.var_uops) u.var_uops.push_back((const PolyUOp *)v);
     }
     if (!u.runner) {
       log_err("compile_schedule", "backend 'hip' failed for kernel %d", k);
@@ -296,10 +300,11 @@ static int bind_args(PolyHipPlan *plan, void **slot_data, int n_slots, const Pol
       }
       a[i] = p;
     }
+    (void)it;
     for (int v = 0; v < un.n_vars; v++) {
       bool found = false;
       for (const PolyVarBinding &m : plan->merged)
-        if (m.var == it.var_uops[v]) { plan->var_vals[u][(size_t)v] = m.value; found = true; break; }
+        if (m.var == un.var_uops[(size_t)v]) { plan->var_vals[u][(size_t)v] = m.value; found = true; break; }
       if (!found) { log_err("plan_run", "no binding for DEFINE_VAR in kernel %d", un.item); return -1; }
       a[un.slots.size() + (size_t)v] = &plan->var_vals[u][(size_t)v];
       key = fnv1a(&plan->var_vals[u][(size_t)v], sizeof(int), key);

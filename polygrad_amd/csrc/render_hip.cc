@@ -139,6 +139,7 @@ class Generic {
     out->entry = fn_;
     out->n_params = (int)g_.params.size();
     out->n_vars = (int)g_.vars.size();
+    for (const VarInfo &v : g_.vars) out->var_uops.push_back(g_.n(v.node).u);
     account(out);
     return true;
   }
@@ -290,7 +291,16 @@ class Generic {
         int ord = order[oi];
         Ext e = extent(ord, &S0);
         std::string rv = strf("r%d", ord);
-        if (e.n < 0) dynamic = true;
+        int64_t e_hi = e.n;
+        if (e.n < 0) {
+          // symbolic extent (a DEFINE_VAR or an expression of some): the grid is sized
+          // for its upper bound and the kernel compares against the run-time value
+          const int bl = g_.n(g_.ranges[(size_t)ord].bound_node).lin;
+          int64_t lo = 0, hi = -1;
+          if (bl >= 0) g_.lin_bounds(g_.lins[(size_t)bl], &lo, &hi);
+          if (hi <= 0) dynamic = true;
+          e_hi = hi;
+        }
         if (oi == 0 && V > 1) {
           int64_t nv = e.n / V;
           line(decomp, 2, strf("const int %s_0 = (int)(t_ %% %lld) * %d; t_ /= %lld;", rv.c_str(), (long long)nv, V, (long long)nv));
@@ -302,7 +312,7 @@ class Generic {
           else
             line(decomp, 2, strf("const int %s = (int)(t_ %% %s); t_ /= %s;", rv.c_str(), e.expr.c_str(), e.expr.c_str()));
           nthreads += "*(long long)" + e.expr;
-          nthreads_n *= e.n < 0 ? 1.0 : (double)e.n;
+          nthreads_n *= (double)std::max<int64_t>(e_hi, 1);
           em_.bind_range(ord, rv);
         }
       }
@@ -369,7 +379,7 @@ class Generic {
       body += decomp + sect;
       line(body, 1, "}");
     }
-    if (dynamic) { error_ = "symbolic range bounds are not supported by the flat lowering yet"; return body; }
+    if (dynamic) { error_ = "a symbolic range bound has no known upper limit"; return body; }
     double blocks = std::ceil(max_threads / opt_.block);
     if (blocks > 2147483647.0) { error_ = "grid too large"; return body; }
     out->launch.grid[0] = (unsigned)std::max(1.0, blocks);

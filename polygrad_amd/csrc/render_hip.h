@@ -33,6 +33,7 @@ struct RenderedKernel {
   std::string strategy;    // human-readable summary for dumps and profiles
   int n_params = 0;        // buffer parameters (args[0..n_params-1])
   int n_vars = 0;          // DEFINE_VAR ints appended after the buffers
+  std::vector<const void *> var_uops;   // the DEFINE_VAR UOps, in the order of those ints
   // Algorithmic work of one launch, for roofline accounting.
   double bytes = 0;        // distinct buffer elements touched * element size
   double flops = 0;        // 2*M*N*K for matmul-shaped kernels, else 0

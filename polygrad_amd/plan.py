@@ -103,11 +103,16 @@ class HipPlan:
                 arr[i] = v.data_ptr()
         return arr
 
-    def run(self, slot_data, sync=True):
+    def run(self, slot_data, sync=True, var_bindings=None):
         """Enqueues one pass of the plan.  slot_data[i]: tensor / device pointer for
-        every external slot i (None for intermediates)."""
+        every external slot i (None for intermediates).  var_bindings: [(DEFINE_VAR UOp
+        pointer, int value)] overriding the schedule's defaults."""
         arr = self._ptr_array(slot_data)
-        rc = self.lib.poly_hip_plan_run(self.handle, arr, len(self.slots), None, 0)
+        vb, nvb = None, 0
+        if var_bindings:
+            nvb = len(var_bindings)
+            vb = (_ffi.PolyVarBinding * nvb)(*[_ffi.PolyVarBinding(v, val) for v, val in var_bindings])
+        rc = self.lib.poly_hip_plan_run(self.handle, arr, len(self.slots), vb, nvb)
         if rc != 0:
             raise RuntimeError("poly_hip_plan_run failed (see stderr)")
         if sync:

@@ -96,6 +96,7 @@ def lib():
         "poly_compiled_plan_free": (None, [P]),
         "poly_grad": (P, [P, P, P]),
         "poly_define_var": (P, [P, C.c_char_p, C.c_int64, C.c_int64]), "poly_bind_var": (P, [P, P, C.c_int64]),
+        "poly_buffer_var": (P, [P, PolyDType, P, I64P, C.c_int]),
         "poly_op_name": (C.c_char_p, [C.c_int]),
     }
     for name, (res, args) in sig.items():
@@ -139,6 +140,21 @@ class Ctx:
         t = T(self, u, (n,), dt, buf=u)
         self.buffers.append((t, name or f"buf{len(self.buffers)}"))
         return t.reshape(shape) if shape != (n,) else t
+
+    def define_var(self, name, lo, hi):
+        """A DEFINE_VAR UOp (symbolic size in [lo, hi])."""
+        self._keep = getattr(self, "_keep", [])
+        b = name.encode()
+        self._keep.append(b)
+        return self.L.poly_define_var(self.ctx, b, lo, hi)
+
+    def buffer_var(self, var, max_val, inner=(), dt=F32, name=None):
+        """A buffer whose leading dimension is the variable `var` (allocated for max_val),
+        as poly_buffer_var builds it (src/frontend.c:163-179)."""
+        u = self.L.poly_buffer_var(self.ctx, dtype_struct(dt), var, _i64(inner) if inner else None, len(inner))
+        t = T(self, u, (max_val,) + tuple(inner), dt, buf=u)
+        self.buffers.append((t, name or f"buf{len(self.buffers)}"))
+        return t
 
     def const(self, v, dt=F32):
         if dt in (F32,):
