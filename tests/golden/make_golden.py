@@ -146,6 +146,16 @@ def main():
         emit(f"gpt2_tiny_{nm}", c, sink, arrays)
         c.close()
 
+    # sin over the ranges its decomposition distinguishes (src/codegen.c:2338-2660: small
+    # arguments, Cody-Waite reduction, Payne-Hanek for huge ones) and its special values
+    c = R.Ctx()
+    x, o = c.buffer((64,), name="x"), c.buffer((64,), name="o")
+    xs = np.concatenate([np.array([0, -0.0, 1e-8, -1e-8, 0.5, -0.5, 1, 2, 3, np.pi, -np.pi, np.pi / 2, 3 * np.pi / 2, 2 * np.pi, 10, 100, 1e3,
+                                   1e4, 1e5, 3e5, 1e6, 1e8, 1e12, 1e20, 1e30, 3e38, np.inf, -np.inf, np.nan, 7.7, -123.456, 0.1], np.float32),
+                         g.uniform(-30, 30, 32).astype(np.float32)])
+    emit("special_sin", c, c.sink((o, x.sin())), {x: xs, o: np.zeros(64, np.float32)})
+    c.close()
+
     # benchmark configuration 1 in small: MLP forward, cross-entropy, gradients, SGD step
     # with in-place parameter updates (22 kernels; src/instance.c:1152-1224 builds the same
     # p - lr * g ASSIGNs)

@@ -16,7 +16,7 @@ BIT_EXACT = {"kat_threefry_u32", "kat_threefry_u64", "movement_i32", "int_alu"}
 TOL = {
     "kat_matmul_2x3x4": (1e-4, 0), "kat_xent_uniform": (1e-4, 1e-6),
     "rowops_sum": (1e-4, 1e-5), "rowops_max": (1e-5, 0), "rowops_softmax": (1e-4, 1e-7), "rowops_layernorm": (1e-4, 1e-5),
-    "special_exp2": (1e-5, 1e-38), "special_log2": (1e-5, 1e-6),
+    "special_exp2": (1e-5, 1e-38), "special_log2": (1e-5, 1e-6), "special_sin": (1e-5, 1e-6),
     "bf16_gelu": (2e-2, 1e-3), "bf16_matmul": (2e-2, 1e-6), "bf16_matmul_bt_batch": (2e-2, 1e-6),
     "f16_cast_mul": (2e-2, 0), "gpt2_tiny_f32": (1e-4, 1e-5), "gpt2_tiny_bf16": (2e-2, 2e-3),
     "mlp_train_b32": (1e-4, 1e-5), "attention_bf16_t256": (2e-2, 2e-3), "bf16_matmul_gelu": (2e-2, 2e-3),
