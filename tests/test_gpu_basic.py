@@ -108,3 +108,24 @@ def test_graph_replay_matches_eager():
     replay, _ = run_hip(c, sink, arrays, graph=True, repeats=4)
     assert np.array_equal(eager[o], replay[o])
     c.close()
+
+
+@pytest.mark.parametrize("seed", range(6))
+def test_random_graphs_match_reference(seed):
+    """Random elementwise / movement / reduction graphs (the generator the oracle is pinned
+    with) on the GPU against the reference CPU backend."""
+    from test_oracle import _random_graph
+    g = np.random.default_rng(1000 + seed)
+    c = R.Ctx()
+    x, y = c.buffer((6, 8), name="x"), c.buffer((6, 8), name="y")
+    val, shape = _random_graph(c, R, g, x, y)
+    o = c.buffer(shape, name="o")
+    sink = c.sink((o, val))
+    bx, by, bo = [t for t, _ in c.buffers]
+    arrays = {bx: g.normal(0, 2, 48).astype(np.float32), by: g.normal(0, 2, 48).astype(np.float32),
+              bo: np.zeros(int(np.prod(shape)), np.float32)}
+    want = run_ref(c, sink, arrays)
+    got, _ = run_hip(c, sink, arrays)
+    c.close()
+    scale = float(np.nanmax(np.abs(want[bo][np.isfinite(want[bo])]))) if np.isfinite(want[bo]).any() else 1.0
+    assert_close(got[bo], want[bo], rtol=1e-4, atol=1e-5 * max(scale, 1.0), what=f"random graph {seed}")

@@ -105,3 +105,62 @@ def test_kat_values_are_the_published_ones():
     fx = F.Fixture("kat_xent_uniform")
     out = [i for i in fx.external if fx.plan.names[i] == "loss"][0]
     assert abs(float(fx.expected[out][0]) - math.log(3.0)) < 1e-6
+
+
+def _random_graph(c, R, g, x, y):
+    """A random expression over two (6, 8) fp32 tensors: elementwise ops the frontend
+    offers, dtype round trips, movement ops and a final optional reduction."""
+    vals = [x, y]
+    for _ in range(int(g.integers(4, 10))):
+        a = vals[int(g.integers(0, len(vals)))]
+        b = vals[int(g.integers(0, len(vals)))]
+        k = int(g.integers(0, 13))
+        if k == 0: v = a + b
+        elif k == 1: v = a * b
+        elif k == 2: v = a - b
+        elif k == 3: v = a / (b * b + c.const(0.5))
+        elif k == 4: v = a.maximum(b)
+        elif k == 5: v = (a * c.const(0.25)).exp2()
+        elif k == 6: v = (a * a + c.const(1e-3)).log2()
+        elif k == 7: v = (a * a).sqrt()
+        elif k == 8: v = a.lt(b).where(a, b * c.const(-1.5))
+        elif k == 9: v = a.cast(R.BF16).cast(R.F32)
+        elif k == 10: v = a.cast(R.F16).cast(R.F32)
+        elif k == 11: v = (a * c.const(7.0)).cast(R.I32).cast(R.F32)
+        else: v = a.permute((1, 0)).flip((0,)).permute((1, 0))
+        vals.append(v)
+    out = vals[-1]
+    mode = int(g.integers(0, 4))
+    if mode == 0: return out.sum(-1), (6,)
+    if mode == 1: return out.max(-1), (6,)
+    if mode == 2: return out.softmax(-1), (6, 8)
+    return out, (6, 8)
+
+
+@pytest.mark.parametrize("seed", range(8))
+def test_oracle_matches_live_reference_on_random_graphs(seed):
+    """Where the real reference library is built (the build container), random graphs go
+    through its CPU backend and through the oracle: results must agree bit for bit."""
+    import refpoly as R
+    from hipharness import schedule_slots
+    if not R.available():
+        pytest.skip("reference library not built here")
+    g = np.random.default_rng(1000 + seed)
+    c = R.Ctx()
+    x, y = c.buffer((6, 8), name="x"), c.buffer((6, 8), name="y")
+    val, shape = _random_graph(c, R, g, x, y)
+    o = c.buffer(shape, name="o")
+    sink = c.sink((o, val))
+    bx, by, bo = [t for t, _ in c.buffers]
+    arrays = {bx: g.normal(0, 2, 48).astype(np.float32), by: g.normal(0, 2, 48).astype(np.float32),
+              bo: np.zeros(int(np.prod(shape)), np.float32)}
+    want = {t: a.copy() for t, a in arrays.items()}
+    c.realize_cpu(sink, want)
+    sched = c.schedule(sink)
+    slots, n = schedule_slots(c, sched)
+    got = F.run_oracle_schedule(sched, n, {i: arrays[t] for i, (t, _) in slots.items()})
+    out_slot = [i for i, (t, _) in slots.items() if t is bo][0]
+    c.L.poly_schedule_free(sched)
+    c.close()
+    assert got[out_slot].tobytes() == want[bo].tobytes(), \
+        f"seed {seed}: max abs diff {np.nanmax(np.abs(got[out_slot] - want[bo]))}"
