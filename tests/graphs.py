@@ -183,8 +183,17 @@ def fused_rowops(c, rows, cols):
     return (a, b, d), outs, sinks
 
 
-def matmul_bf16(c, m, n, k, transposed_b=False, batch=None):
-    """Config 3: C = A@B, bf16 inputs, f32 accumulate and output."""
+def matmul_bf16(c, m, n, k, transposed_b=False, batch=None, transposed_a=False):
+    """Config 3: C = A@B, bf16 inputs, f32 accumulate and output.  transposed_a / transposed_b:
+    the operand is stored (k, m) / (n, k) and permuted in the graph (the forms the backward
+    pass of a linear layer produces: dX = dY W^T, dW = X^T dY)."""
+    if transposed_a:
+        assert batch is None
+        At = c.buffer((k, m), R.BF16, name="A")
+        Bm = c.buffer((n, k), R.BF16, name="B") if transposed_b else c.buffer((k, n), R.BF16, name="B")
+        b = Bm.permute((1, 0)) if transposed_b else Bm
+        O = c.buffer((m, n), R.F32, name="C")
+        return At, Bm, O, c.sink((O, At.permute((1, 0)).cast(R.F32).dot(b.cast(R.F32))))
     a_shape = (m, k) if batch is None else (batch, m, k)
     A = c.buffer(a_shape, R.BF16, name="A")
     if transposed_b:

@@ -144,6 +144,39 @@ def test_matmul_sweep_full_size_sampled_rows(name, m, n, k, tb, batch):
         assert bool((err <= 1e-4 * bound + 1e-30).all()), f"{name}: max err/bound {float((err / bound).max()):.3e}"
 
 
+# ── config 5: the matmul shapes of a GPT-2 medium train step (B=4, T=1024: 4096 rows) ──
+
+C5_SHAPES = [  # (m, n, k, transposed_a, transposed_b): forward, dX = dY W^T, dW = X^T dY
+    (4096, 3072, 1024, False, False), (4096, 1024, 1024, False, False), (4096, 4096, 1024, False, False),
+    (4096, 1024, 4096, False, False), (4096, 1024, 3072, False, True), (4096, 1024, 4096, False, True),
+    (1024, 3072, 4096, True, False), (4096, 1024, 4096, True, False), (4096, 50257, 1024, False, True),
+]
+
+
+@pytest.mark.parametrize("m,n,k,ta,tb", C5_SHAPES)
+def test_gpt2_medium_train_matmul_shapes(m, n, k, ta, tb):
+    import torch
+    c = R.Ctx()
+    A, Bm, O, sink = graphs.matmul_bf16(c, m, n, k, transposed_a=ta, transposed_b=tb)
+    g = np.random.default_rng(m + 3 * n + 7 * k)
+    a_bits = R.f32_to_bf16_bits(g.normal(0, 0.05, m * k).astype(np.float32))
+    b_bits = R.f32_to_bf16_bits(g.normal(0, 0.05, k * n).astype(np.float32))
+    got, info = run_hip(c, sink, {A: a_bits, Bm: b_bits, O: np.full(m * n, np.nan, np.float32)})
+    c.close()
+    assert len(info) == 1 and info[0]["klass"] == "matmul-mfma", info
+    C = torch.from_numpy(got[O]).view(m, n)
+    assert bool(torch.isfinite(C).all())
+    a = torch.from_numpy(R.bf16_bits_to_f32(a_bits)).double()
+    b = torch.from_numpy(R.bf16_bits_to_f32(b_bits)).double()
+    a = a.view(k, m).t() if ta else a.view(m, k)
+    b = b.view(n, k).t() if tb else b.view(k, n)
+    rows = sorted({0, 1, 127, 128, 255, 256, m // 2, m - 129, m - 1})
+    want = a[rows] @ b
+    bound = a[rows].abs() @ b.abs()
+    err = (C[rows].double() - want).abs()
+    assert bool((err <= 1e-4 * bound + 1e-30).all()), f"max err/bound {float((err / bound).max()):.3e}"
+
+
 # ── config 4: GPT-2 small ────────────────────────────────────────────────────────────────
 
 def test_gpt2_small_batch_elements_are_independent():
