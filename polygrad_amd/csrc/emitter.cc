@@ -16,6 +16,8 @@ namespace polyhip {
 
 const char *hip_prelude() {
   return R"HIP(
+extern "C" __device__ float __ocml_sin_f32(float);
+extern "C" __device__ double __ocml_sin_f64(double);
 typedef float  poly_f32x4 __attribute__((ext_vector_type(4)));
 typedef float  poly_f32x2 __attribute__((ext_vector_type(2)));
 typedef __bf16 poly_bf16x8 __attribute__((ext_vector_type(8)));
@@ -342,7 +344,9 @@ std::string Emitter::emit_raw(int id, Scope *s) {
       else e = strf("__builtin_exp2f(%s)", S(0).c_str());
       break;
     case POLY_OP_LOG2: e = k.dt == DT_F64 ? strf("__builtin_log2(%s)", S(0).c_str()) : strf("__builtin_log2f(%s)", S(0).c_str()); break;
-    case POLY_OP_SIN: e = k.dt == DT_F64 ? strf("__builtin_sin(%s)", S(0).c_str()) : strf("__builtin_sinf(%s)", S(0).c_str()); break;
+    // the device library's sin (argument reduction for any magnitude); the builtin would
+    // become the hardware approximation, which loses accuracy beyond a few periods
+    case POLY_OP_SIN: e = k.dt == DT_F64 ? strf("__ocml_sin_f64(%s)", S(0).c_str()) : strf("__ocml_sin_f32(%s)", S(0).c_str()); break;
     case POLY_OP_RECIPROCAL: e = strf("(1/%s)", S(0).c_str()); break;
     case POLY_OP_ADD: e = strf("(%s+%s)", S(0).c_str(), S(1).c_str()); break;
     case POLY_OP_SUB: e = strf("(%s-%s)", S(0).c_str(), S(1).c_str()); break;

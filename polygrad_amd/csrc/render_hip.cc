@@ -413,6 +413,38 @@ class Generic {
     double rows = 1;
     for (int r : groups_[0].ranges) rows *= (double)g_.ranges[(size_t)r].extent;
     if (R < 128) return false;
+    // Lanes that walk along the reduce range only pay off when some operand is contiguous
+    // along it.  When every load is strided there (X^T W forms: the reduce axis is the
+    // outer axis of both operands) but contiguous along an output range, one thread per
+    // output with a serial loop is the coalesced mapping: neighbouring lanes read
+    // neighbouring addresses at every step.
+    {
+      const int QF = rr.back();
+      bool unit_along_reduce = false, unit_along_output = false;
+      std::vector<char> mark(g_.nodes.size(), 0);
+      for (int id : top_reduces_) mark_reachable(g_, g_.n(id).src[0], mark);
+      for (int i = 0; i < (int)g_.nodes.size(); i++) {
+        if (!mark[(size_t)i] || g_.n(i).op != POLY_OP_LOAD) continue;
+        const int li = g_.n(g_.n(g_.n(i).src[0]).src[1]).lin;
+        if (li < 0) { unit_along_reduce = true; continue; }   // unknown: keep the default
+        bool aff;
+        if (g_.lin_range_coef(g_.lins[(size_t)li], QF, &aff) == 1 && aff) unit_along_reduce = true;
+        // unit stride along an output range, or along the fastest digit (r % c) of a
+        // flattened one
+        for (const Term &t : g_.lins[(size_t)li].terms) {
+          if (t.coef != 1) continue;
+          const Atom &a = g_.atoms[(size_t)t.atom];
+          const Atom *base = &a;
+          if (a.kind == Atom::MOD && a.inner.c0 == 0 && a.inner.terms.size() == 1 && a.inner.terms[0].coef == 1)
+            base = &g_.atoms[(size_t)a.inner.terms[0].atom];
+          else if (a.kind != Atom::RANGE) continue;
+          if (base->kind != Atom::RANGE) continue;
+          const int ord = g_.range_ord.at(base->node);
+          for (int r : groups_[0].ranges) if (r == ord) unit_along_output = true;
+        }
+      }
+      if (!unit_along_reduce && unit_along_output && rows >= 65536) return false;
+    }
     // Long rows, or too few rows to fill the chip with one wave each: a whole
     // workgroup per row.
     if (R >= 4096 || (rows < 2048 && R >= 1024)) coop_G_ = 256; else coop_G_ = 64;

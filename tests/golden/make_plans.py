@@ -6,6 +6,8 @@ the GPU box, where the reference frontend is not part of the product path:
     polygrad_amd/plans/rowops_f32_8192.polyplan            config 2 (fused chain + row ops), 8192x8192 fp32
     polygrad_amd/plans/matmul_bf16_<m>x<n>x<k>[_bt].polyplan   config 3 shapes
     polygrad_amd/plans/attention_bf16_b8_h12_t1024_d64.polyplan   the attention block of config 4 alone
+    polygrad_amd/plans/mlp_train_f32_b4096.polyplan        config 1: MLP forward + backward + SGD step
+    polygrad_amd/plans/adamw_f32_355m.polyplan             config 5: AdamW update of 355 M fp32 parameters
 
 The graphs are built with the REAL reference frontend and scheduler
 (oracle/_ref/libpolygrad.so through tests/refpoly.py); only the scheduled kernel
@@ -61,6 +63,14 @@ def main():
         _, _, _, sink = graphs.matmul_bf16(c, m, n, k, transposed_b=tb)
         save(c, sink, f"matmul_bf16_{m}x{n}x{k}" + ("_bt" if tb else ""))
         c.close()
+    c = R.Ctx()
+    _, sink = graphs.mlp_train_step(c, batch=4096)
+    save(c, sink, "mlp_train_f32_b4096")
+    c.close()
+    c = R.Ctx()
+    _, sink = graphs.adamw_step(c, 354_823_168)      # GPT-2 medium parameter count
+    save(c, sink, "adamw_f32_355m")
+    c.close()
     c = R.Ctx()
     _, sink = graphs.attention_bf16(c, batch=8, heads=12, ctx=1024, hd=64)
     save(c, sink, "attention_bf16_b8_h12_t1024_d64")

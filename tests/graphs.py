@@ -263,3 +263,20 @@ def T_grad(c, loss, param, numel):
     if not u:
         raise RuntimeError("poly_grad failed")
     return R.T(c, u, (numel,), param.dt)
+
+
+def adamw_step(c, numel, lr=3e-4, beta1=0.9, beta2=0.999, eps=1e-8, weight_decay=0.1):
+    """One AdamW update of a flat parameter, built the way the reference's training graph
+    builds it (src/instance.c:1162-1224): decoupled decay, moments, bias corrections read
+    from one-element buffers and expanded, three in-place ASSIGNs (param, m, v)."""
+    p, g, m, v = (c.buffer((numel,), name=n) for n in ("p", "g", "m", "v"))
+    bc1, bc2 = c.buffer((1,), name="bc1"), c.buffer((1,), name="bc2")
+    p_cur = p * c.const(1.0 - lr * weight_decay)
+    m_new = c.const(beta1) * m + c.const(1.0 - beta1) * g
+    v_new = c.const(beta2) * v + c.const(1.0 - beta2) * (g * g)
+    m_hat = m_new * bc1.expand((numel,))
+    v_hat = v_new * bc2.expand((numel,))
+    denom = v_hat.sqrt() + c.const(eps)
+    p_new = p_cur - c.const(lr) * (m_hat * denom.un("RECIPROCAL"))
+    bufs = dict(p=p, g=g, m=m, v=v, bc1=bc1, bc2=bc2)
+    return bufs, c.sink_assign((p, p_new), (m, m_new), (v, v_new))
