@@ -1309,6 +1309,10 @@ static bool match_attention(const Sched &sc, int s_item, const std::vector<char>
     score = strf("%s(%s, m, n, z, %s)", fn.c_str(), score.c_str(), call_args(m.item).c_str());
   }
   cfg += strf("#define POLY_FA_SCORE(acc, m, n, z) %s\n", score.c_str());
+  // Single-pass form when the group is a plain softmax: p = cast(term / sum) with
+  // term = exp2((x - max) * c) and the maximum taken over the scores themselves.
+  const bool online = p_is_term_over_sum && !getenv("POLY_HIP_EXACT_ATTENTION");
+  cfg += strf("#define POLY_FA_ONLINE %d\n#define POLY_FA_C %s\n", online ? 1 : 0, Emitter::float_literal(c_sum, DT_F32).c_str());
   value_fn(mMax, "poly_fa_maxv", "float", strf("%s x", tn).c_str(), body_max, {});
   cfg += strf("#define POLY_FA_MAXV(x, m, n, z) poly_fa_maxv(x, m, n, z, %s)\n", call_args(i_max).c_str());
   value_fn(mSum, "poly_fa_term", "float", strf("%s x, float mx", tn).c_str(), body_sum, {});
@@ -1351,8 +1355,9 @@ static bool match_attention(const Sched &sc, int s_item, const std::vector<char>
   rk.launch.grid[0] = (unsigned)((mS.M / 128) * mS.Z);
   rk.launch.block[0] = 256;
   rk.klass = KernelClass::ATTENTION;
-  rk.strategy = strf("fused attention (%zu kernels): mfma 32x32x16 %s Z=%lld M=%lld N=%lld D=64, two passes over keys", all.size() + copy_items.size(),
-                     tin == DT_BF16 ? "bf16" : "f16", (long long)mS.Z, (long long)mS.M, (long long)mS.N);
+  rk.strategy = strf("fused attention (%zu kernels): mfma 32x32x16 %s Z=%lld M=%lld N=%lld D=64, %s", all.size() + copy_items.size(),
+                     tin == DT_BF16 ? "bf16" : "f16", (long long)mS.Z, (long long)mS.M, (long long)mS.N,
+                     cfg.find("#define POLY_FA_ONLINE 1") != std::string::npos ? "one pass, online softmax" : "two passes over keys, exact roundings");
   rk.n_params = (int)arg_slots.size();
   rk.n_vars = 0;
   rk.flops = 2.0 * (double)mS.Z * (double)mS.M * (double)mS.N * (double)(mS.K + mV.N);

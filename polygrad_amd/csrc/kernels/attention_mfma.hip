@@ -9,7 +9,11 @@
 // included, so every probability is computed by the same expression as in the unfused
 // kernels.
 //
-// Two passes over the keys.  Pass 1 computes each row's maximum and the sum of its terms
+// Two forms.  The exact form (below, POLY_FA_ONLINE 0) reproduces every rounding step of
+// the unfused kernels; the online form (POLY_FA_ONLINE 1, further down) is the usual
+// single-pass streaming softmax.
+//
+// Exact form: two passes over the keys.  Pass 1 computes each row's maximum and the sum of its terms
 // (running maximum with rescaling; the hooks guarantee term(x, m) = exp2((x - m) * c),
 // which makes the rescaling factor term(m_old, m_new)).  Pass 2 recomputes the scores
 // (bit-identical: same MFMA sequence), turns them into probabilities with the final
@@ -36,6 +40,21 @@
 //   POLY_FA_SKIP_DEAD_BLOCKS           1 when p = cast(term(x, mx) / sum): then a key block whose
 //                                      terms are all exactly 0 has probabilities exactly 0
 //   POLY_SIGNATURE
+//   POLY_FA_ONLINE                     1: single pass (needs p = cast(term / sum),
+//                                      term(x, mx) = exp2((x - mx) * POLY_FA_C) and the
+//                                      maximum taken over the scores themselves)
+//
+// Online form: one pass.  Per 32-key tile a wave computes the scores x exactly as the
+// pointwise chain stores them (POLY_FA_SCORE, roundings included), the new running
+// maximum m of each query, t = exp2((x - m) * c) in fp32, rescales the running sum and
+// the output accumulators by exp2((m_old - m) * c) when a maximum moved, and accumulates
+// O^T += V^T cast(t)^T; the division by the sum happens once at the end.  Against the
+// unfused kernels the 16-bit rounding of the probabilities moves from t / sum to t (the
+// output differs from theirs by about one 16-bit rounding), and a key tile whose scores
+// are all -inf is skipped outright, so a non-finite V under zero probability does not
+// propagate.
+// The output is transposed relative to the exact form: a lane holds ONE query in both
+// MFMAs, so maximum, sum and rescaling factor are per-lane scalars.
 //
 // Dead key blocks (every term of the block exactly zero for all 32 queries of a wave, as
 // under a causal mask) are detected from the values themselves, never assumed: term is
@@ -64,6 +83,11 @@ __device__ __forceinline__ int poly_v_off(int z, int n) { return (z / 12) * 7864
 #define POLY_FA_P(x, mx, sum, m, n, z) ((__bf16)(__builtin_amdgcn_exp2f(((float)(x) - (mx)) * 0x1.715476p+0f) / (sum)))
 #define POLY_FA_OUT(acc, m, d, z) data0[((z) / 12) * 786432 + ((z) % 12) * 65536 + (m) * 64 + (d)] = (__bf16)(acc)
 #define POLY_FA_SKIP_DEAD_BLOCKS 1
+#define POLY_FA_ONLINE 1
+#define POLY_FA_C 0x1.715476p+0f
+#endif
+#ifndef POLY_FA_ONLINE
+#define POLY_FA_ONLINE 0
 #endif
 
 typedef POLY_TIN fa_in8 __attribute__((ext_vector_type(8)));
@@ -190,6 +214,99 @@ extern "C" __global__ void __launch_bounds__(FA_THREADS) __attribute__((amdgpu_w
   // key index of accumulator register r of tile t
   auto key_of = [&](int kb, int t, int r) { return kb * FA_BN + 32 * t + 8 * (r >> 2) + 4 * half + (r & 3); };
 
+#if POLY_FA_ONLINE
+  // ── online form: one pass over the keys ─────────────────────────────────────
+  fa_acc16 o[2];
+#pragma unroll
+  for (int dt = 0; dt < 2; dt++)
+#pragma unroll
+    for (int r = 0; r < 16; r++) o[dt][r] = 0.0f;
+  float m_run = -__builtin_inff(), l_run = 0.0f;   // identical maximum on both lanes of a query; sum of this lane's keys
+  {
+    const float c = POLY_FA_C;
+    fa_u32x4 rk[2], rv[4];
+    load_k(0, rk);
+    load_v(0, rv);
+    store_k(0, rk);
+    store_v(0, rv);
+    __syncthreads();
+    for (int kb = 0; kb < FA_NKB; kb++) {
+      const int cur = kb & 1;
+      if (kb + 1 < FA_NKB) { load_k(kb + 1, rk); load_v(kb + 1, rv); }
+      // V^T fragment (A operand): feature row 32 dt + lq, the 8 keys of this lane's half
+      // of the 16 keys 32t + 16u .., in the key order of the score registers
+      auto v_frag = [&](int t, int u, int dt) {
+        const int col0 = 4 * t + 2 * u;
+        const int d = 32 * dt + lq;
+        const POLY_TIN *row = lds_v[cur] + d * FA_BN;
+        const int sw = fa_swz(d);
+        const fa_u32x2 lo = *(const fa_u32x2 *)(row + ((col0 ^ sw) * 8) + half * 4);
+        const fa_u32x2 hi = *(const fa_u32x2 *)(row + (((col0 + 1) ^ sw) * 8) + half * 4);
+        fa_u32x4 both;
+        both[0] = lo[0]; both[1] = lo[1]; both[2] = hi[0]; both[3] = hi[1];
+        return __builtin_bit_cast(fa_in8, both);
+      };
+#pragma unroll
+      for (int t = 0; t < 2; t++) {
+        fa_acc16 st;
+        scores(cur, t, st);
+        float x[16];
+        float bm = -__builtin_inff(), nan_probe = 0.0f;
+#pragma unroll
+        for (int r = 0; r < 16; r++) {
+          const int n = key_of(kb, t, r);
+          x[r] = POLY_FA_MAXV(POLY_FA_SCORE(st[r], mq, n, z), mq, n, z);
+          bm = __builtin_fmaxf(bm, x[r]);     // ignores a NaN ...
+          nan_probe = nan_probe + x[r];        // ... which this catches (as does +inf meeting -inf)
+        }
+        bm = __builtin_fmaxf(bm, fa_other_half(bm));
+        // every score of the tile is -inf for all 32 queries: all its terms are exact zeros
+        const bool lane_live = (bm != -__builtin_inff()) || (nan_probe != nan_probe);
+        if (__builtin_amdgcn_ballot_w64(lane_live) == 0) continue;
+        const float m_new = __builtin_fmaxf(m_run, bm);
+        // a query whose keys were all -inf so far: subtract 0 instead (its terms come out 0,
+        // not NaN; if the row stays empty the final 0 / 0 is the NaN the unfused kernels give)
+        const float m_use = (m_new == -__builtin_inff()) ? 0.0f : m_new;
+        const float mc = m_use * c;
+        const float alpha = __builtin_amdgcn_exp2f((m_run - m_use) * c);
+        float sum = 0.0f;
+        POLY_TIN p[16];
+#pragma unroll
+        for (int r = 0; r < 16; r++) {
+          const float tt = __builtin_amdgcn_exp2f(__builtin_fmaf(x[r], c, -mc));
+          sum = sum + tt;
+          p[r] = (POLY_TIN)tt;
+        }
+        l_run = l_run * alpha + sum;
+        m_run = m_new;
+        if (__builtin_amdgcn_ballot_w64(alpha != 1.0f) != 0) {
+#pragma unroll
+          for (int dt = 0; dt < 2; dt++)
+#pragma unroll
+            for (int r = 0; r < 16; r++) o[dt][r] = o[dt][r] * alpha;
+        }
+#pragma unroll
+        for (int u = 0; u < 2; u++) {
+          fa_in8 pf;
+#pragma unroll
+          for (int i = 0; i < 8; i++) pf[i] = p[8 * u + i];
+#pragma unroll
+          for (int dt = 0; dt < 2; dt++) o[dt] = POLY_MFMA(v_frag(t, u, dt), pf, o[dt]);
+        }
+      }
+      if (kb + 1 < FA_NKB) { store_k(cur ^ 1, rk); store_v(cur ^ 1, rv); }
+      __syncthreads();
+    }
+  }
+  // the two lanes of a query each summed half of the keys (a + b == b + a bit for bit)
+  const float l_tot = l_run + fa_other_half(l_run);
+  // O^T tile: register r of lane l holds feature 8*(r/4) + 4*(l/32) + r%4 of query l%32
+#pragma unroll
+  for (int dt = 0; dt < 2; dt++)
+#pragma unroll
+    for (int r = 0; r < 16; r++)
+      POLY_FA_OUT(o[dt][r] / l_tot, mq, 32 * dt + 8 * (r >> 2) + 4 * half + (r & 3), z);
+#else
   // ── pass 1: row maximum and sum of terms, one 32-key tile at a time ─────────
   float row_max = -__builtin_inff(), row_sum = 0.0f;
   unsigned long long dead = 0;   // wave-uniform: 32-key tiles whose terms are all exactly zero
@@ -319,4 +436,5 @@ extern "C" __global__ void __launch_bounds__(FA_THREADS) __attribute__((amdgpu_w
       const int m = m0 + wave * 32 + 8 * (r >> 2) + 4 * half + (r & 3);
       POLY_FA_OUT(o[dt][r], m, 32 * dt + lq, z);
     }
+#endif
 }

@@ -79,7 +79,9 @@ typedef float poly_f32x4 __attribute__((ext_vector_type(4)));
 #define POLY_LDK POLY_BK
 #define POLY_NCOL (POLY_BK / 8)
 __device__ __forceinline__ int poly_swz(int row) { return (row ^ (row >> 3)) & (POLY_NCOL - 1); }
+#ifndef POLY_KT
 #define POLY_KT (POLY_K / POLY_BK)
+#endif
 // row pitch (floats) of the 32x32 output staging tile: 16-byte aligned rows, and rows 4
 // apart (the two halves of a wave) land on different banks
 #define POLY_STAGE_LD 36
@@ -93,22 +95,28 @@ __device__ __forceinline__ int poly_swz(int row) { return (row ^ (row >> 3)) & (
 // lines per row when BK = 64).
 template <int ROWS, int NLOADS>
 struct PolyKC {
+  // staging work is cut into UNITS pieces (one 16-byte load and store each) so that the
+  // K loop can spread it between its MFMAs
+  static constexpr int UNITS = NLOADS;
+  static __device__ __forceinline__ void load_unit(const POLY_TIN *__restrict__ base, const int *row_off, int kofs,
+                                                   poly_u32x4 (&regs)[NLOADS], int i) {
+    const int c = threadIdx.x + i * POLY_NTHREADS;
+    const int kc = c % (POLY_BK / 8);
+    regs[i] = *(const poly_u32x4_u *)(base + row_off[i] + kofs + kc * 8);
+  }
+  static __device__ __forceinline__ void store_unit(POLY_TIN *lds, const poly_u32x4 (&regs)[NLOADS], int i) {
+    const int c = threadIdx.x + i * POLY_NTHREADS;
+    const int row = c / (POLY_BK / 8), kc = c % (POLY_BK / 8);
+    *(poly_u32x4 *)(lds + row * POLY_LDK + ((kc ^ poly_swz(row)) * 8)) = regs[i];
+  }
   static __device__ __forceinline__ void load(const POLY_TIN *__restrict__ base, const int *row_off, int kofs,
                                               poly_u32x4 (&regs)[NLOADS]) {
 #pragma unroll
-    for (int i = 0; i < NLOADS; i++) {
-      const int c = threadIdx.x + i * POLY_NTHREADS;
-      const int kc = c % (POLY_BK / 8);
-      regs[i] = *(const poly_u32x4_u *)(base + row_off[i] + kofs + kc * 8);
-    }
+    for (int i = 0; i < NLOADS; i++) load_unit(base, row_off, kofs, regs, i);
   }
   static __device__ __forceinline__ void store(POLY_TIN *lds, const poly_u32x4 (&regs)[NLOADS]) {
 #pragma unroll
-    for (int i = 0; i < NLOADS; i++) {
-      const int c = threadIdx.x + i * POLY_NTHREADS;
-      const int row = c / (POLY_BK / 8), kc = c % (POLY_BK / 8);
-      *(poly_u32x4 *)(lds + row * POLY_LDK + ((kc ^ poly_swz(row)) * 8)) = regs[i];
-    }
+    for (int i = 0; i < NLOADS; i++) store_unit(lds, regs, i);
   }
 };
 
@@ -123,36 +131,43 @@ struct PolyXC {
   static constexpr int TOTAL = CHUNKS * (POLY_BK / 4);    // 4x8 blocks per tile
   static constexpr int NBLK = (TOTAL + POLY_NTHREADS - 1) / POLY_NTHREADS;
   static constexpr int NLOADS = NBLK * 4;
+  // staging units for spreading the work over the K loop: unit u writes row pair u % 4 of
+  // block u / 4; the four loads of a block can be reissued once its last unit is stored
+  static constexpr int UNITS = NBLK * 4;
+  static __device__ __forceinline__ bool active(int b) {
+    return TOTAL % POLY_NTHREADS == 0 || (int)threadIdx.x + b * POLY_NTHREADS < TOTAL;
+  }
+  static __device__ __forceinline__ void load_block(const POLY_TIN *__restrict__ base, const int *chunk_off, const int *k_off,
+                                                    poly_u32x4 (&regs)[NLOADS], int b) {
+    if (active(b)) {
+#pragma unroll
+      for (int i = 0; i < 4; i++) regs[b * 4 + i] = *(const poly_u32x4_u *)(base + chunk_off[b] + k_off[b * 4 + i]);
+    }
+  }
+  static __device__ __forceinline__ void store_unit(POLY_TIN *lds, const poly_u32x4 (&regs)[NLOADS], int u) {
+    const int b = u >> 2, j = u & 3;
+    if (!active(b)) return;
+    const int c = threadIdx.x + b * POLY_NTHREADS;
+    const int chunk = c % CHUNKS, kq = c / CHUNKS;
+    // dword j of load i holds rows 2j (low half) and 2j+1 (high half) at k = kq*4+i
+    const unsigned int a0 = regs[b * 4 + 0][j], a1 = regs[b * 4 + 1][j], a2 = regs[b * 4 + 2][j], a3 = regs[b * 4 + 3][j];
+    poly_u32x2 lo, hi;
+    lo[0] = (a0 & 0xffffu) | (a1 << 16);
+    lo[1] = (a2 & 0xffffu) | (a3 << 16);
+    hi[0] = (a0 >> 16) | (a1 & 0xffff0000u);
+    hi[1] = (a2 >> 16) | (a3 & 0xffff0000u);
+    const int r0 = chunk * 8 + 2 * j, r1 = r0 + 1;
+    *(poly_u32x2 *)(lds + r0 * POLY_LDK + (((kq >> 1) ^ poly_swz(r0)) * 8) + (kq & 1) * 4) = lo;
+    *(poly_u32x2 *)(lds + r1 * POLY_LDK + (((kq >> 1) ^ poly_swz(r1)) * 8) + (kq & 1) * 4) = hi;
+  }
   static __device__ __forceinline__ void load(const POLY_TIN *__restrict__ base, const int *chunk_off, const int *k_off,
                                               poly_u32x4 (&regs)[NLOADS]) {
 #pragma unroll
-    for (int b = 0; b < NBLK; b++) {
-      if (TOTAL % POLY_NTHREADS == 0 || (int)threadIdx.x + b * POLY_NTHREADS < TOTAL) {
-#pragma unroll
-        for (int i = 0; i < 4; i++) regs[b * 4 + i] = *(const poly_u32x4_u *)(base + chunk_off[b] + k_off[b * 4 + i]);
-      }
-    }
+    for (int b = 0; b < NBLK; b++) load_block(base, chunk_off, k_off, regs, b);
   }
   static __device__ __forceinline__ void store(POLY_TIN *lds, const poly_u32x4 (&regs)[NLOADS]) {
 #pragma unroll
-    for (int b = 0; b < NBLK; b++) {
-      const int c = threadIdx.x + b * POLY_NTHREADS;
-      if (TOTAL % POLY_NTHREADS != 0 && c >= TOTAL) continue;
-      const int chunk = c % CHUNKS, kq = c / CHUNKS;
-#pragma unroll
-      for (int j = 0; j < 4; j++) {
-        // dword j of load i holds rows 2j (low half) and 2j+1 (high half) at k = kq*4+i
-        const unsigned int a0 = regs[b * 4 + 0][j], a1 = regs[b * 4 + 1][j], a2 = regs[b * 4 + 2][j], a3 = regs[b * 4 + 3][j];
-        poly_u32x2 lo, hi;
-        lo[0] = (a0 & 0xffffu) | (a1 << 16);
-        lo[1] = (a2 & 0xffffu) | (a3 << 16);
-        hi[0] = (a0 >> 16) | (a1 & 0xffff0000u);
-        hi[1] = (a2 >> 16) | (a3 & 0xffff0000u);
-        const int r0 = chunk * 8 + 2 * j, r1 = r0 + 1;
-        *(poly_u32x2 *)(lds + r0 * POLY_LDK + (((kq >> 1) ^ poly_swz(r0)) * 8) + (kq & 1) * 4) = lo;
-        *(poly_u32x2 *)(lds + r1 * POLY_LDK + (((kq >> 1) ^ poly_swz(r1)) * 8) + (kq & 1) * 4) = hi;
-      }
-    }
+    for (int u = 0; u < UNITS; u++) store_unit(lds, regs, u);
   }
 };
 
@@ -274,6 +289,44 @@ extern "C" __global__ void __launch_bounds__(POLY_NTHREADS) poly_k(POLY_SIGNATUR
 #endif
   };
 
+  // One piece of the staging work, for spreading it between the MFMAs of the K loop:
+  // the units of both operands that fall into part `part` of `nparts` write their share
+  // of the tile held in (ra, rb) to LDS buffer `buf` (if st) and then refill those
+  // registers from tile kt_load (if ld).
+  auto stage_part = [&](int part, int nparts, bool st, int buf, bool ld, int kt_load, auto &ra, auto &rb) {
+    const int k0 = kt_load * POLY_BK;
+#pragma unroll
+    for (int u = 0; u < StageA::UNITS; u++) {
+      if (u * nparts / StageA::UNITS != part) continue;
+      if (st) StageA::store_unit(lds_a(buf), ra, u);
+#if POLY_A_KC
+      if (ld) StageA::load_unit(gA, a_off, poly_a_k(k0), ra, u);
+#else
+      if (ld && (u & 3) == 3) {
+        int ak[StageA::NLOADS];
+#pragma unroll
+        for (int i = 0; i < 4; i++) ak[(u >> 2) * 4 + i] = poly_a_k(k0 + a_kq[u >> 2] + i);
+        StageA::load_block(gA, a_off, ak, ra, u >> 2);
+      }
+#endif
+    }
+#pragma unroll
+    for (int u = 0; u < StageB::UNITS; u++) {
+      if (u * nparts / StageB::UNITS != part) continue;
+      if (st) StageB::store_unit(lds_b(buf), rb, u);
+#if POLY_B_KC
+      if (ld) StageB::load_unit(gB, b_off, poly_b_k(k0), rb, u);
+#else
+      if (ld && (u & 3) == 3) {
+        int bk[StageB::NLOADS];
+#pragma unroll
+        for (int i = 0; i < 4; i++) bk[(u >> 2) * 4 + i] = poly_b_k(k0 + b_kq[u >> 2] + i);
+        StageB::load_block(gB, b_off, bk, rb, u >> 2);
+      }
+#endif
+    }
+  };
+
   const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
   const int wm = (wave % POLY_WAVES_M) * POLY_WM, wn = (wave / POLY_WAVES_M) * POLY_WN;
   const int frag_row = lane & 31;
@@ -294,35 +347,68 @@ extern "C" __global__ void __launch_bounds__(POLY_NTHREADS) poly_k(POLY_SIGNATUR
   for (int j = 0; j < POLY_TN; j++) { const int r = wn + j * 32 + frag_row; b_row_off[j] = r * POLY_LDK; b_swz[j] = poly_swz(r); }
   const int frag_col = lane >> 5;   // which 8-wide half of a 16-deep K step
 
-  // Fragments are double buffered in registers: the LDS reads of K step ks+1 are
-  // issued before the MFMAs of step ks, so their latency hides behind the math.
-  poly_in8 fa[2][POLY_TM], fb[2][POLY_TN];
+  // Fragment registers.  Small wave tiles keep two sets (the reads of K step ks+1 are
+  // issued before the MFMAs of step ks).  Wave tiles of 8 or more MFMAs per step keep one
+  // set and refill it on the fly: MFMAs run row by row, so the A fragment of row i is
+  // dead after its last column and the B fragment of column j after the last row; each is
+  // reread for the next step right there, at least three MFMAs before its next use.
+#ifndef POLY_FRAG_ROLL
+#define POLY_FRAG_ROLL (POLY_TM * POLY_TN >= 8)
+#endif
+  poly_in8 fa[POLY_FRAG_ROLL ? 1 : 2][POLY_TM], fb[POLY_FRAG_ROLL ? 1 : 2][POLY_TN];
+  auto read_a = [&](int cur, int ks, int buf, int i) {
+    fa[buf][i] = *(const poly_in8 *)(lds_a(cur) + a_row_off[i] + (((ks * 2 + frag_col) ^ a_swz[i]) * 8));
+  };
+  auto read_b = [&](int cur, int ks, int buf, int j) {
+    fb[buf][j] = *(const poly_in8 *)(lds_b(cur) + b_row_off[j] + (((ks * 2 + frag_col) ^ b_swz[j]) * 8));
+  };
   auto read_frags = [&](int cur, int ks, int buf) {
 #pragma unroll
-    for (int i = 0; i < POLY_TM; i++) fa[buf][i] = *(const poly_in8 *)(lds_a(cur) + a_row_off[i] + (((ks * 2 + frag_col) ^ a_swz[i]) * 8));
+    for (int i = 0; i < POLY_TM; i++) read_a(cur, ks, buf, i);
 #pragma unroll
-    for (int j = 0; j < POLY_TN; j++) fb[buf][j] = *(const poly_in8 *)(lds_b(cur) + b_row_off[j] + (((ks * 2 + frag_col) ^ b_swz[j]) * 8));
+    for (int j = 0; j < POLY_TN; j++) read_b(cur, ks, buf, j);
   };
-  auto compute = [&](int cur, int ks_begin, int ks_end) {
-    read_frags(cur, ks_begin, ks_begin & 1);
+
+  // The K loop keeps the matrix pipe and the LDS pipe busy at the same time.  A K tile is
+  // KS steps of MT MFMAs: KS * MT slots.  Each slot issues one MFMA, then the fragment
+  // refills that became possible, then its share of the staging work (LDS stores of the
+  // next tile, global loads of a later one), so that the stores drain while the MFMAs
+  // execute instead of in a phase of their own.  The order is pinned slot by slot.
+  constexpr int KS = POLY_BK / 16, MT = POLY_TM * POLY_TN;
+  auto k_tile = [&](int cur, auto &&stage_slot) {
+    read_frags(cur, 0, 0);
 #pragma unroll
-    for (int ks = ks_begin; ks < ks_end; ks++) {
-      if (ks + 1 < ks_end) read_frags(cur, ks + 1, (ks + 1) & 1);
+    for (int ks = 0; ks < KS; ks++) {
+      constexpr int R = POLY_FRAG_ROLL;
+      if (!R && ks + 1 < KS) read_frags(cur, ks + 1, (ks + 1) & 1);
+      __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
       for (int i = 0; i < POLY_TM; i++)
 #pragma unroll
-        for (int j = 0; j < POLY_TN; j++) acc[i][j] = POLY_MFMA(fa[ks & 1][i], fb[ks & 1][j], acc[i][j]);
+        for (int j = 0; j < POLY_TN; j++) {
+          const int buf = R ? 0 : (ks & 1);
+          acc[i][j] = POLY_MFMA(fa[buf][i], fb[buf][j], acc[i][j]);
+          if (R && ks + 1 < KS) {
+            if (j == POLY_TN - 1) read_a(cur, ks + 1, 0, i);
+            if (i == POLY_TM - 1) read_b(cur, ks + 1, 0, j);
+          }
+          stage_slot(ks * MT + i * POLY_TN + j);
+          // (small wave tiles: pinned per K step only, the compiler places the staging
+          // work among the step's few MFMAs)
+          if (R) __builtin_amdgcn_sched_barrier(0);
+        }
+      if (!R) __builtin_amdgcn_sched_barrier(0);
     }
+    __syncthreads();
   };
 
-  constexpr int KS = POLY_BK / 16, KS_HALF = KS / 2;
 #if POLY_PIPE == 3
-  // Software pipeline, three tiles deep: tile kt is multiplied out of one LDS
-  // buffer; tile kt+1 waits in one register set and is written to the other LDS
-  // buffer in the middle of the iteration; tile kt+2 is in flight into the second
-  // register set, and the loads of tile kt+3 are issued as soon as the first set
-  // is free.  Every global load has about two and a half iterations to land.
-  // Tile t always uses register set t & 1, hence the loop is unrolled by two.
+  // Three tiles deep: tile kt is multiplied out of one LDS buffer; tile kt+1 waits in
+  // one register set and moves to the other LDS buffer during the iteration; tile kt+2
+  // is in flight into the second register set; each register of the first set is
+  // refilled from tile kt+3 as soon as it is stored.  Every global load has about two
+  // iterations to land.  Tile t always uses register set t & 1, hence the loop is
+  // unrolled by two.
   load_tiles(0, ra0, rb0);
   StageA::store(lds_a(0), ra0);
   StageB::store(lds_b(0), rb0);
@@ -330,46 +416,40 @@ extern "C" __global__ void __launch_bounds__(POLY_NTHREADS) poly_k(POLY_SIGNATUR
   if (POLY_KT > 2) load_tiles(2, ra0, rb0);
   __syncthreads();
 
-  auto iteration = [&](int kt, auto &ra_next, auto &rb_next) {
+  auto iteration = [&](int kt, auto &ra_next, auto &rb_next, bool st, bool ld) {
     const int cur = kt & 1;
-    compute(cur, 0, KS_HALF);
-    __builtin_amdgcn_sched_barrier(0);
-    if (kt + 1 < POLY_KT) {
-      StageA::store(lds_a(cur ^ 1), ra_next);
-      StageB::store(lds_b(cur ^ 1), rb_next);
-    }
-    if (kt + 3 < POLY_KT) load_tiles(kt + 3, ra_next, rb_next);
-    __builtin_amdgcn_sched_barrier(0);
-    compute(cur, KS_HALF, KS);
-    __syncthreads();
+    k_tile(cur, [&](int slot) { stage_part(slot, KS * MT, st, cur ^ 1, ld, kt + 3, ra_next, rb_next); });
   };
-  for (int kt = 0; kt < POLY_KT; kt += 2) {
-    iteration(kt, ra1, rb1);
-    if (kt + 1 < POLY_KT) iteration(kt + 1, ra0, rb0);
+  // steady state (every iteration stores and loads: no branches in the loop body), then
+  // the last iterations with their conditions known at compile time
+  constexpr int STEADY = POLY_KT >= 3 ? ((POLY_KT - 3) & ~1) : 0;
+  for (int kt = 0; kt < STEADY; kt += 2) {
+    iteration(kt, ra1, rb1, true, true);
+    iteration(kt + 1, ra0, rb0, true, true);
+  }
+#pragma unroll
+  for (int kt = STEADY; kt < POLY_KT; kt++) {
+    if (kt & 1) iteration(kt, ra0, rb0, kt + 1 < POLY_KT, kt + 3 < POLY_KT);
+    else iteration(kt, ra1, rb1, kt + 1 < POLY_KT, kt + 3 < POLY_KT);
   }
 #else
-  // Software pipeline, two tiles deep (for tiles whose accumulators leave no room
-  // for a second staging register set): the global loads of tile kt+1 are issued
-  // before the first half of tile kt is multiplied, and land in the other LDS
-  // buffer between the two halves.
+  // Two tiles deep (for tiles whose accumulators leave no room for a second staging
+  // register set): the global loads of tile kt+1 are issued at the top of iteration kt
+  // and move to the other LDS buffer during the second half of its slots.
   load_tiles(0, ra0, rb0);
   StageA::store(lds_a(0), ra0);
   StageB::store(lds_b(0), rb0);
   __syncthreads();
-  for (int kt = 0; kt < POLY_KT; kt++) {
+  auto iteration = [&](int kt, bool st) {
     const int cur = kt & 1;
-    if (kt + 1 < POLY_KT) load_tiles(kt + 1, ra0, rb0);
-    __builtin_amdgcn_sched_barrier(0);
-    compute(cur, 0, KS_HALF);
-    __builtin_amdgcn_sched_barrier(0);
-    if (kt + 1 < POLY_KT) {
-      StageA::store(lds_a(cur ^ 1), ra0);
-      StageB::store(lds_b(cur ^ 1), rb0);
-    }
-    __builtin_amdgcn_sched_barrier(0);
-    compute(cur, KS_HALF, KS);
-    __syncthreads();
-  }
+    if (st) load_tiles(kt + 1, ra0, rb0);
+    constexpr int FIRST = (KS / 2) * MT, NSLOTS = KS * MT - FIRST;
+    k_tile(cur, [&](int slot) {
+      if (slot >= FIRST) stage_part(slot - FIRST, NSLOTS, st, cur ^ 1, false, 0, ra0, rb0);
+    });
+  };
+  for (int kt = 0; kt + 1 < POLY_KT; kt++) iteration(kt, true);
+  iteration(POLY_KT - 1, false);
 #endif
 
   // Accumulator layout of the 32x32 MFMA: register r of lane l holds

@@ -19,7 +19,10 @@ TOL = {
     "special_exp2": (1e-5, 1e-38), "special_log2": (1e-5, 1e-6), "special_sin": (1e-5, 1e-6),
     "bf16_gelu": (2e-2, 1e-3), "bf16_matmul": (2e-2, 1e-6), "bf16_matmul_bt_batch": (2e-2, 1e-6),
     "f16_cast_mul": (2e-2, 0), "gpt2_tiny_f32": (1e-4, 1e-5), "gpt2_tiny_bf16": (2e-2, 2e-3),
-    "mlp_train_b32": (1e-4, 1e-5), "attention_bf16_t256": (2e-2, 2e-3), "bf16_matmul_gelu": (2e-2, 2e-3),
+    # attention: the default single-pass kernel rounds exp-terms where the reference rounds
+    # probabilities; for the first queries (a handful of keys, outputs up to 1) that is two
+    # 16-bit steps of the output scale.  The exact two-pass form is held to 2e-3 below.
+    "mlp_train_b32": (1e-4, 1e-5), "attention_bf16_t256": (2e-2, 8e-3), "bf16_matmul_gelu": (2e-2, 2e-3),
     "bf16_layernorm_rows": (2e-2, 2e-3),
 }
 # plans that update their inputs in place: a second run would start from other parameters
@@ -57,6 +60,16 @@ def test_fixture_on_gpu(name):
         else:
             rtol, atol = TOL[name]
             assert_close(F.as_float(got[slot]), F.as_float(want), rtol=rtol, atol=atol, what=f"{name} slot {slot} ({fx.plan.names[slot]})")
+
+
+def test_attention_fixture_exact_form(monkeypatch):
+    """The two-pass attention kernel keeps every rounding of the unfused kernels."""
+    monkeypatch.setenv("POLY_HIP_EXACT_ATTENTION", "1")
+    fx = F.Fixture("attention_bf16_t256")
+    got, info = run_fixture_on_gpu(fx)
+    assert any("two passes" in k["desc"] for k in info), [k["desc"] for k in info]
+    for slot in fx.external:
+        assert_close(F.as_float(got[slot]), F.as_float(fx.expected[slot]), rtol=2e-2, atol=2e-3, what=f"exact attention slot {slot}")
 
 
 def test_oracle_agrees_with_gpu_on_fixture_inputs():

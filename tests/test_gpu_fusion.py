@@ -33,18 +33,27 @@ def logits(arrays_out, bufs):
     return R.bf16_bits_to_f32(arrays_out[bufs["output"]]).astype(np.float64)
 
 
+@pytest.mark.parametrize("form", ["online", "exact"])
 @pytest.mark.parametrize("qk_gain", [1.0, 12.0])
-def test_fused_attention_matches_unfused_and_reference(qk_gain):
+def test_fused_attention_matches_unfused_and_reference(qk_gain, form):
+    """form "online": the default single-pass fp32 softmax; "exact": the two-pass form that
+    keeps every 16-bit rounding of the unfused kernels (POLY_HIP_EXACT_ATTENTION=1)."""
     c, cfg, sink, bufs, arrays = small_gpt2(seed=11, qk_gain=qk_gain)
     want = logits(run_ref(c, sink, arrays), bufs)
-    got, info = run_hip(c, sink, arrays)
+    if form == "exact":
+        os.environ["POLY_HIP_EXACT_ATTENTION"] = "1"
+    try:
+        got, info = run_hip(c, sink, arrays)
+    finally:
+        os.environ.pop("POLY_HIP_EXACT_ATTENTION", None)
     assert sum(k["klass"] == "attention-mfma" for k in info) == cfg.n_layer, [k["klass"] for k in info]
+    marker = "one pass" if form == "online" else "two passes"
+    assert sum(marker in k["desc"] for k in info) == cfg.n_layer, [k["desc"] for k in info if k["klass"] == "attention-mfma"]
     os.environ["POLY_HIP_NO_FUSION"] = "1"
     try:
         plain, info_plain = run_hip(c, sink, arrays)
     finally:
         del os.environ["POLY_HIP_NO_FUSION"]
-    c.close()
     assert not any(k["klass"] == "attention-mfma" for k in info_plain)
     # per layer: six attention kernels and the three copies that split q, k and v out of
     # the fused projection became one, three pointwise kernels (attention
@@ -57,13 +66,31 @@ def test_fused_attention_matches_unfused_and_reference(qk_gain):
     h, p = logits(got, bufs), logits(plain, bufs)
     scale = float(np.abs(want).max())
     assert np.isfinite(h).all()
-    # same expressions per element; only the order of the fp32 sums differs
-    assert_close(h, p, rtol=2e-2, atol=2e-2 * scale, what="fused vs separately launched kernels")
-    assert float(np.mean(h != p)) < 0.05, "bf16 logits should rarely differ at all"
-    assert_close(h, want, rtol=2e-2, atol=2e-2 * scale, what="fused vs reference CPU backend")
-    e_fused = float(np.sqrt(np.mean((h - want) ** 2)))
-    e_plain = float(np.sqrt(np.mean((p - want) ** 2)))
-    assert e_fused <= 1.5 * e_plain + 1e-6 * scale, (e_fused, e_plain)
+    # With the projections scaled up the scores reach +-50 and one 16-bit rounding of an
+    # activation moves a probability by tens of percent: the network amplifies the
+    # rounding that the online form places differently, so that form gets three times the
+    # absolute tolerance there and is judged against the fp32 network below.
+    loose = 3.0 if (form == "online" and qk_gain > 1.0) else 1.0
+    assert_close(h, p, rtol=2e-2, atol=2e-2 * scale * loose, what="fused vs separately launched kernels")
+    assert_close(h, want, rtol=2e-2, atol=2e-2 * scale * loose, what="fused vs reference CPU backend")
+    rms = lambda d: float(np.sqrt(np.mean(d ** 2)))
+    if form == "exact":
+        # same expressions per element; only the order of the fp32 sums differs
+        assert float(np.mean(h != p)) < 0.05, "bf16 logits should rarely differ at all"
+        assert rms(h - want) <= 1.5 * rms(p - want) + 1e-6 * scale
+    else:
+        # fewer roundings than the reference: judged against the same network in fp32
+        sink32, bufs32 = graphs.gpt2_forward(c, cfg, R.F32)
+        arr32 = {}
+        for name, t in bufs32.items():
+            a = arrays[bufs[name]]
+            arr32[t] = R.bf16_bits_to_f32(a) if a.dtype == np.uint16 else a.astype(np.float32)
+        truth = run_ref(c, sink32, arr32)[bufs32["output"]].astype(np.float64)
+        e_gpu, e_ref = rms(h - truth), rms(want - truth)
+        print(f"qk_gain {qk_gain}: rms error against the fp32 network: GPU {e_gpu:.3e}, reference {e_ref:.3e}; "
+              f"max |GPU - reference| {np.abs(h - want).max():.3e} at scale {scale:.3e}")
+        assert e_gpu <= 1.1 * e_ref, f"GPU rms error {e_gpu:.3e} vs reference rms error {e_ref:.3e} against the fp32 network"
+    c.close()
 
 
 def test_lookup_table_epilogue_is_bit_identical_to_the_arithmetic():
