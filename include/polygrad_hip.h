@@ -115,7 +115,9 @@ void poly_hip_plan_free(PolyHipPlan *plan);
  * values -- src/modelzoo/models/gpt2.c:411-441 builds it as separate realized
  * tensors).  Returns their number, <0 on a malformed schedule; needs no device.
  * For 0 <= index < count, *n_items_out receives how many scheduled kernels the
- * group replaces and *source_out its HIP source (free with poly_hip_free_string).
+ * group replaces and *source_out its HIP source (free with poly_hip_free_string);
+ * kernels that fill the group's tables follow the main kernel, each after a line
+ * starting with "// ---- ".
  * No reference counterpart: the reference launches every scheduled kernel. */
 int poly_hip_fused_groups(const PolySchedule *schedule, int index, char **source_out, int *n_items_out);
 /* Introspection for benches and tests. */

@@ -386,6 +386,15 @@ std::string Emitter::emit_raw(int id, Scope *s) {
       return "0";
   }
   if (failed()) return "0";
+  if (pow2_mul16_exact && k.op == POLY_OP_MUL && (k.dt == DT_BF16 || k.dt == DT_F16)) {
+    for (int side = 0; side < 2; side++) {
+      const KNode &c = g_.n(k.src[(size_t)side]);
+      if (c.op != POLY_OP_CONST || c.u->arg.kind != POLY_ARG_FLOAT || g_.n(k.src[(size_t)(1 - side)]).dt != k.dt) continue;
+      int ex = 0;
+      const double v = c.u->arg.f;
+      if (std::isfinite(v) && v != 0 && std::fabs(std::frexp(v, &ex)) == 0.5 && ex > -100 && ex < 100) ct = "float";
+    }
+  }
   std::string name = strf("v%d", id);
   stmt(t, strf("const %s %s = %s;", ct, name.c_str(), e.c_str()));
   t->names[id] = name;

@@ -1216,11 +1216,13 @@ static bool match_attention(const Sched &sc, int s_item, const std::vector<char>
   // The softmax terms use the bare exp2 instruction: a term below 2^-126 of the row's
   // largest (which is exactly 1, so the sum is at least 1) cannot change the fp32 sum, and
   // the probability it would give is below the smallest normal 16-bit float.
+  const bool online = p_is_term_over_sum && !getenv("POLY_HIP_EXACT_ATTENTION");
   auto value_fn = [&](const Member &m, const char *name, const char *ret, const char *lead_args, int node,
                       const std::map<int, std::string> &extra_preset) {
     const KernelGraph &g = sc.graphs[(size_t)m.item];
     Emitter em(g);
     em.raw_exp2 = (m.item == i_sum || m.item == i_p);
+    em.pow2_mul16_exact = online;
     Scope S0;
     S0.indent = 1;
     for (auto &kv : m.rm) { em.bind_range(kv.first, strf("r%d", kv.second)); S0.avail |= (uint64_t)1 << kv.first; }
@@ -1311,7 +1313,6 @@ static bool match_attention(const Sched &sc, int s_item, const std::vector<char>
   cfg += strf("#define POLY_FA_SCORE(acc, m, n, z) %s\n", score.c_str());
   // Single-pass form when the group is a plain softmax: p = cast(term / sum) with
   // term = exp2((x - max) * c) and the maximum taken over the scores themselves.
-  const bool online = p_is_term_over_sum && !getenv("POLY_HIP_EXACT_ATTENTION");
   cfg += strf("#define POLY_FA_ONLINE %d\n#define POLY_FA_C %s\n", online ? 1 : 0, Emitter::float_literal(c_sum, DT_F32).c_str());
   value_fn(mMax, "poly_fa_maxv", "float", strf("%s x", tn).c_str(), body_max, {});
   cfg += strf("#define POLY_FA_MAXV(x, m, n, z) poly_fa_maxv(x, m, n, z, %s)\n", call_args(i_max).c_str());

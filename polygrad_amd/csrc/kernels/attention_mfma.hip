@@ -50,9 +50,9 @@
 // the output accumulators by exp2((m_old - m) * c) when a maximum moved, and accumulates
 // O^T += V^T cast(t)^T; the division by the sum happens once at the end.  Against the
 // unfused kernels the 16-bit rounding of the probabilities moves from t / sum to t (the
-// output differs from theirs by about one 16-bit rounding), and a key tile whose scores
-// are all -inf is skipped outright, so a non-finite V under zero probability does not
-// propagate.
+// output differs from theirs by about one 16-bit rounding), and a key tile whose terms are
+// all exact zeros against the running maxima (as under a causal mask) is skipped after
+// its scores, so a non-finite V under zero probability does not propagate.
 // The output is transposed relative to the exact form: a lane holds ONE query in both
 // MFMAs, so maximum, sum and rescaling factor are per-lane scalars.
 //
@@ -260,9 +260,12 @@ extern "C" __global__ void __launch_bounds__(FA_THREADS) __attribute__((amdgpu_w
           nan_probe = nan_probe + x[r];        // ... which this catches (as does +inf meeting -inf)
         }
         bm = __builtin_fmaxf(bm, fa_other_half(bm));
-        // every score of the tile is -inf for all 32 queries: all its terms are exact zeros
-        const bool lane_live = (bm != -__builtin_inff()) || (nan_probe != nan_probe);
-        if (__builtin_amdgcn_ballot_w64(lane_live) == 0) continue;
+        // Against the running maximum the largest term of this tile is exactly zero (the
+        // exponential underflows, or the scores are -inf) for all 32 queries: the maxima
+        // do not move and every term is an exact zero.  (A query with no finite score yet
+        // has m_run = -inf and counts as live.)
+        const bool lane_dead = (__builtin_amdgcn_exp2f((bm - m_run) * c) == 0.0f) && (nan_probe == nan_probe);
+        if (__builtin_amdgcn_ballot_w64(!lane_dead) == 0) continue;
         const float m_new = __builtin_fmaxf(m_run, bm);
         // a query whose keys were all -inf so far: subtract 0 instead (its terms come out 0,
         // not NaN; if the row stays empty the final 0 / 0 is the NaN the unfused kernels give)

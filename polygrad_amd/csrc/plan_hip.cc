@@ -373,7 +373,9 @@ int poly_hip_fused_groups(const PolySchedule *s, int index, char **source_out, i
   if (index >= 0 && index < (int)groups.size()) {
     if (n_items_out) *n_items_out = (int)groups[(size_t)index].items.size();
     if (source_out) {
-      const std::string &src = groups[(size_t)index].rk.source;
+      // the main kernel, then the kernels that fill its tables, as separate translation units
+      std::string src = groups[(size_t)index].rk.source;
+      for (const RenderedKernel::Table &t : groups[(size_t)index].rk.tables) src += "\n// ---- table " + t.entry + "\n" + t.source;
       *source_out = (char *)malloc(src.size() + 1);
       if (*source_out) memcpy(*source_out, src.c_str(), src.size() + 1);
     }

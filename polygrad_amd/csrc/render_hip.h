@@ -118,6 +118,10 @@ class Emitter {
   // f32 EXP2 as the bare hardware instruction: results below 2^-126 come out as 0 instead
   // of denormals (the library form wraps the instruction in a range-scaling sequence).
   bool raw_exp2 = false;
+  // A 16-bit float value times a power-of-two constant is kept in fp32 instead of being
+  // rounded back to 16 bits: the product is exactly representable unless it drops below
+  // the smallest normal number, so the only values that change are products under 2^-126.
+  bool pow2_mul16_exact = false;
 
  private:
   std::string emit_atom(int atom, Scope *s);
