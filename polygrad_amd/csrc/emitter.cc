@@ -325,6 +325,28 @@ std::string Emitter::emit_raw(int id, Scope *s) {
     case POLY_OP_LOAD: e = load_expr(id, t); break;
     case POLY_OP_CAST: {
       DT sdt = g_.n(k.src[0]).dt;
+      const KNode &q = g_.n(k.src[0]);
+      if (recip_div16 && (k.dt == DT_BF16 || k.dt == DT_F16) && sdt == DT_F32 && !is_preset(k.src[0])) {
+        int num = -1, den = -1;
+        if (q.op == POLY_OP_FDIV) { num = q.src[0]; den = q.src[1]; }
+        else if (q.op == POLY_OP_MUL && g_.n(q.src[1]).op == POLY_OP_RECIPROCAL && !is_preset(q.src[1])) { num = q.src[0]; den = g_.n(q.src[1]).src[0]; }
+        if (num >= 0 && (g_.n(den).deps & ~g_.n(num).deps) == 0 && g_.n(den).deps != g_.n(num).deps) {
+          // the divisor varies in fewer loops than the dividend: one reciprocal per value of it
+          Scope *td = place(g_.n(den).deps, t);
+          const int key = -2 - den;
+          auto f = td->names.find(key);
+          std::string rc;
+          if (f != td->names.end()) rc = f->second;
+          else {
+            rc = strf("rcp%d", den);
+            const std::string dv = emit(den, td);
+            stmt(td, strf("const float %s = 1.0f / %s;", rc.c_str(), dv.c_str()));
+            td->names[key] = rc;
+          }
+          e = strf("(%s)(%s * %s)", ct, emit(num, t).c_str(), rc.c_str());
+          break;
+        }
+      }
       if (k.dt == DT_BOOL && sdt != DT_BOOL) e = strf("(%s!=0)", S(0).c_str());
       else e = strf("(%s)(%s)", ct, S(0).c_str());
       break;

@@ -691,10 +691,17 @@ static bool match_row_chain(const Sched &sc, int a_item, const std::vector<char>
   std::string code, calls, strat;
   std::string lead;   // results so far, as parameters
   std::string lead_call;
+  // Short rows handled by one wave stay in registers between the phases: a vector load
+  // that an earlier phase made from the same buffer at the same index is kept instead of
+  // being repeated (the row is then read from memory once, not once per phase).
+  struct RowCache { std::string key, type; int nit; };
+  std::vector<RowCache> cache;
+  int n_cached_uses = 0;
   for (size_t pi = 0; pi < phases.size(); pi++) {
     const RowPhase &ph = phases[pi];
     const KernelGraph &g = sc.graphs[(size_t)ph.m.item];
     Emitter em(g);
+    em.recip_div16 = true;
     Scope S0;                        // row-invariant values
     S0.indent = 1;
     int own_f = -1;                  // this kernel's range that walks along the row
@@ -730,7 +737,27 @@ static bool match_row_chain(const Sched &sc, int a_item, const std::vector<char>
     L.avail = S0.avail;
     L.indent = 2;
     std::vector<int> pres;
-    if (V > 1) pres = hoist_vector_loads(g, em, roots, own_f, V, fv + "_0", &L);
+    const int nit = (int)((R + (int64_t)G * V - 1) / ((int64_t)G * V));
+    const bool unrolled = G == 64 && nit <= 4;   // iterations as an unrolled loop over `it`
+    const std::function<std::string(int, const std::string &)> keep = [&](int node, const std::string &ld) -> std::string {
+      const KNode &ix = g.n(g.n(node).src[0]);
+      Aff a;
+      if (!lin_to_aff(g, g.lins[(size_t)g.n(ix.src[1]).lin], ph.m.rm, &a)) return ld;
+      std::string key = strf("%d:%d:%d:%lld", sc.slot(ph.m.item, g.param_slot(ix.src[0])), V, (int)g.n(node).dt, (long long)a.c0);
+      for (auto &kv : a.c) key += strf(",%d*%lld", kv.first, (long long)kv.second);
+      for (size_t ci = 0; ci < cache.size(); ci++)
+        if (cache[ci].key == key && cache[ci].nit == nit) { n_cached_uses++; return strf("c%zu[it]", ci); }
+      if (pi + 1 == phases.size()) return ld;   // nobody comes after the last phase
+      cache.push_back({key, strf("poly_vec<%s,%d>", dt_cname(g.n(node).dt), V), nit});
+      return strf("(c%zu[it] = %s)", cache.size() - 1, ld.c_str());
+    };
+    if (V > 1) pres = hoist_vector_loads(g, em, roots, own_f, V, fv + "_0", &L, unrolled ? &keep : nullptr);
+    // the row loop: positions fv_0 = lane * V, + G * V, ...
+    const std::string loop_open = unrolled
+        ? strf("#pragma unroll\n  for (int it = 0; it < %d; it++) {\n  const int %s_0 = lane * %d + it * %d;\n  if (%s_0 < %lld) {\n", nit, fv.c_str(), V, G * V,
+               fv.c_str(), (long long)R)
+        : strf("  for (int %s_0 = lane * %d; %s_0 < %lld; %s_0 += %d) {\n", fv.c_str(), V, fv.c_str(), (long long)R, fv.c_str(), G * V);
+    const std::string loop_close = unrolled ? "  }\n  }\n" : "  }\n";
     Scope U;                          // one element
     U.parent = &L;
     U.avail = L.avail | ((uint64_t)1 << own_f);
@@ -747,10 +774,10 @@ static bool match_row_chain(const Sched &sc, int a_item, const std::vector<char>
       loop += strf("  %s acc = %s;\n", dt_cname(Rn.dt), Emitter::reduce_identity(op, Rn.dt).c_str());
       loop += S0.code;
       S0.code.clear();
-      loop += strf("  for (int %s_0 = lane * %d; %s_0 < %lld; %s_0 += %d) {\n", fv.c_str(), V, fv.c_str(), (long long)R, fv.c_str(), G * V);
+      loop += loop_open;
       loop += L.code;
       loop += strf("#pragma unroll\n    for (int u = 0; u < %d; u++) {\n      const int %s = %s_0 + u;\n", V, fv.c_str(), fv.c_str());
-      loop += U.code + "    }\n  }\n";
+      loop += U.code + "    }\n" + loop_close;
       loop += strf("  acc = %s;\n", wave_reduce_call(op, Rn.dt, "acc").c_str());
       if (G == 256) {
         loop += strf("  __shared__ %s red[4];\n  __syncthreads();\n  if ((threadIdx.x & 63) == 0) red[threadIdx.x >> 6] = acc;\n  __syncthreads();\n",
@@ -780,25 +807,30 @@ static bool match_row_chain(const Sched &sc, int a_item, const std::vector<char>
       if (V > 1) { em.bind_range(own_f, fv + "_0"); addr = em.emit_lin(g.lins[(size_t)li], &L); em.bind_range(own_f, fv); }
       loop += S0.code;
       S0.code.clear();
-      loop += strf("  for (int %s_0 = lane * %d; %s_0 < %lld; %s_0 += %d) {\n", fv.c_str(), V, fv.c_str(), (long long)R, fv.c_str(), G * V);
+      loop += loop_open;
       loop += L.code;
       if (V > 1) loop += strf("    poly_vec<%s,%d> out;\n", odt, V);
       loop += strf("#pragma unroll\n    for (int u = 0; u < %d; u++) {\n      const int %s = %s_0 + u;\n", V, fv.c_str(), fv.c_str());
       loop += U.code + "    }\n";
       if (V > 1) loop += strf("    poly_vstore<%s,%d>(data%d + %s, out);\n", odt, V, p, addr.c_str());
-      loop += "  }\n";
+      loop += loop_close;
     }
     if (em.failed() || em.uses_threefry) FA_REJECT();
-    code += strf("__device__ __forceinline__ %s %s(const long long row, const int lane%s, %s) {\n", ret.c_str(), fn.c_str(), lead.c_str(),
-                 params_decl(g).c_str());
+    std::string cache_params, cache_args;
+    for (size_t ci = 0; ci < cache.size(); ci++) {
+      cache_params += strf(", %s (&c%zu)[%d]", cache[ci].type.c_str(), ci, cache[ci].nit);
+      cache_args += strf(", c%zu", ci);
+    }
+    code += strf("__device__ __forceinline__ %s %s(const long long row, const int lane%s%s, %s) {\n", ret.c_str(), fn.c_str(), lead.c_str(),
+                 cache_params.c_str(), params_decl(g).c_str());
     code += row_decomp + loop + tail + "}\n";
     if (!ph.is_map) {
-      calls += strf("    const %s %s = %s(row, lane%s, %s);\n", ret.c_str(), names[pi].c_str(), fn.c_str(), lead_call.c_str(),
-                    call_args(ph.m.item).c_str());
+      calls += strf("    const %s %s = %s(row, lane%s%s, %s);\n", ret.c_str(), names[pi].c_str(), fn.c_str(), lead_call.c_str(),
+                    cache_args.c_str(), call_args(ph.m.item).c_str());
       lead += strf(", const %s %s", ret.c_str(), names[pi].c_str());
       lead_call += ", " + names[pi];
     } else {
-      calls += strf("    %s(row, lane%s, %s);\n", fn.c_str(), lead_call.c_str(), call_args(ph.m.item).c_str());
+      calls += strf("    %s(row, lane%s%s, %s);\n", fn.c_str(), lead_call.c_str(), cache_args.c_str(), call_args(ph.m.item).c_str());
     }
     strat += strf("%s%s vec%d", pi ? ", " : "", ph.is_map ? "map" : "reduce", V);
   }
@@ -809,6 +841,7 @@ static bool match_row_chain(const Sched &sc, int a_item, const std::vector<char>
   } else {
     body += "  const int lane = threadIdx.x;\n  const long long row = blockIdx.x;\n  {\n";
   }
+  for (size_t ci = 0; ci < cache.size(); ci++) body += strf("    %s c%zu[%d];\n", cache[ci].type.c_str(), ci, cache[ci].nit);
   body += calls + "  }\n}\n";
 
   out->items = items;
@@ -823,6 +856,7 @@ static bool match_row_chain(const Sched &sc, int a_item, const std::vector<char>
   rk.launch.block[0] = 256;
   rk.klass = KernelClass::ROW_REDUCE;
   rk.strategy = strf("row chain of %zu kernels (%s) G=%d R=%lld rows=%.0f", phases.size(), strat.c_str(), G, (long long)R, rows);
+  if (n_cached_uses) rk.strategy += strf(", %d row loads kept in registers", n_cached_uses);
   rk.n_params = (int)arg_slots.size();
   rk.bytes = bytes;
   return true;

@@ -48,7 +48,8 @@ void mark_reachable(const KernelGraph &g_, int root, std::vector<char> &mark) {
 }
 
 std::vector<int> hoist_vector_loads(const KernelGraph &g_, Emitter &em_, const std::vector<int> &roots, int F, int V,
-                                    const std::string &f0, Scope *outer) {
+                                    const std::string &f0, Scope *outer,
+                                    const std::function<std::string(int, const std::string &)> *wrap) {
   std::vector<char> mark(g_.nodes.size(), 0);
   for (int r : roots) mark_reachable(g_, r, mark);
   std::vector<int> done;
@@ -80,6 +81,7 @@ std::vector<int> hoist_vector_loads(const KernelGraph &g_, Emitter &em_, const s
       gate = gate.empty() ? g2 : "(" + gate + "&&" + g2 + ")";
     }
     if (!gate.empty()) ld = strf("(%s ? %s : poly_vec<%s,%d>{})", gate.c_str(), ld.c_str(), dt_cname(k.dt), V);
+    else if (wrap) ld = (*wrap)(i, ld);
     outer->code.append((size_t)outer->indent * 2, ' ');
     outer->code += strf("const poly_vec<%s,%d> %s = %s;\n", dt_cname(k.dt), V, name.c_str(), ld.c_str());
     em_.preset(i, name + ".v[u]");

@@ -122,6 +122,10 @@ class Emitter {
   // rounded back to 16 bits: the product is exactly representable unless it drops below
   // the smallest normal number, so the only values that change are products under 2^-126.
   bool pow2_mul16_exact = false;
+  // cast16(a / b) becomes cast16(a * (1 / b)) with the reciprocal placed where b is
+  // computed (outside the loops b does not depend on): the fp32 quotient may differ in its
+  // last bit, which the 16-bit rounding hides except at rounding ties.
+  bool recip_div16 = false;
 
  private:
   std::string emit_atom(int atom, Scope *s);
@@ -142,8 +146,11 @@ void mark_reachable(const KernelGraph &g, int root, std::vector<char> &mark);
 // Emits V-wide vector loads into `outer` for every LOAD under `roots` that is unit-stride
 // along F (starting at the C expression f0) and presets those nodes to "<name>.v[u]";
 // returns the preset nodes.
+// `wrap`, when given, may replace the load expression of an ungated LOAD node (e.g. by a
+// value kept from an earlier pass over the same addresses).
 std::vector<int> hoist_vector_loads(const KernelGraph &g, Emitter &em, const std::vector<int> &roots, int F, int V,
-                                    const std::string &f0, Scope *outer);
+                                    const std::string &f0, Scope *outer,
+                                    const std::function<std::string(int, const std::string &)> *wrap = nullptr);
 // C expression reducing `v` over the 64 lanes of a wave.
 std::string wave_reduce_call(PolyOps op, DT dt, const std::string &v);
 
