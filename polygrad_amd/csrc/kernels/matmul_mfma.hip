@@ -79,9 +79,7 @@ typedef float poly_f32x4 __attribute__((ext_vector_type(4)));
 #define POLY_LDK POLY_BK
 #define POLY_NCOL (POLY_BK / 8)
 __device__ __forceinline__ int poly_swz(int row) { return (row ^ (row >> 3)) & (POLY_NCOL - 1); }
-#ifndef POLY_KT
 #define POLY_KT (POLY_K / POLY_BK)
-#endif
 // row pitch (floats) of the 32x32 output staging tile: 16-byte aligned rows, and rows 4
 // apart (the two halves of a wave) land on different banks
 #define POLY_STAGE_LD 36

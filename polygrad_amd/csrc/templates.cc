@@ -423,9 +423,6 @@ bool render_matmul(const MatmulMatch &mm, const MatmulEpilogue &ep, RenderedKern
   cfg += matmul_k_fn("poly_b_k", kb, K);
   cfg += strf("#define POLY_SIGNATURE %s\n", ep.signature.c_str());
   cfg += ep.code;
-  if (const char *e = getenv("POLY_HIP_MM_ABLATE")) { int a = atoi(e); if (a & 1) cfg += "#define POLY_ABLATE_LOAD 1\n"; if (a & 2) cfg += "#define POLY_ABLATE_STORE 1\n"; if (a & 4) cfg += "#define POLY_ABLATE_FRAG 1\n"; }
-  if (const char *e = getenv("POLY_HIP_MM_VAR")) cfg += strf("#define POLY_VAR %d\n", atoi(e));
-  if (const char *e = getenv("POLY_HIP_MM_KT")) cfg += strf("#define POLY_KT %d\n", atoi(e));   // timing experiments only: wrong results
   if (getenv("POLY_HIP_MM_NOEPI")) cfg += strf("#define POLY_EPILOGUE(acc, m, n, z) do { if (((m) | (n)) == -1) { %s; } } while (0)\n", ep.call.c_str());
   else
   cfg += strf("#define POLY_EPILOGUE(acc, m, n, z) %s\n", ep.call.c_str());
