@@ -336,15 +336,22 @@ extern "C" __global__ void __launch_bounds__(FA_THREADS) __attribute__((amdgpu_w
           nan_probe = nan_probe + v;      // NaN if any value is (or +inf meets -inf: then not skipped)
         }
         const float new_max = (row_max < bm) ? bm : row_max;
+        // nothing but -inf so far for this lane's half of the keys: its sum stays 0 and its
+        // maximum -inf (terms against a maximum of -inf would be NaN; if the other half of
+        // the row has a finite score these keys get probability 0, otherwise the row is
+        // NaN as in the unfused kernels, which the merge below produces)
+        const bool empty = (new_max == -__builtin_inff()) && (nan_probe == nan_probe);
         // upper bound of this lane's terms in this tile
         const float bound = POLY_FA_TERM((POLY_TIN)bm, new_max, mq, 0, z);
-        const bool lane_dead = (bound == 0.0f) && (nan_probe == nan_probe);
+        const bool lane_dead = empty || ((bound == 0.0f) && (nan_probe == nan_probe));
         if (__builtin_amdgcn_ballot_w64(!lane_dead) != 0) {
           float acc = row_sum * POLY_FA_TERM((POLY_TIN)row_max, new_max, mq, 0, z);
 #pragma unroll
           for (int r = 0; r < 16; r++) acc = acc + POLY_FA_TERM(x[r], new_max, mq, key_of(kb, t, r), z);
-          row_sum = acc;
-          row_max = new_max;
+          if (!empty) {
+            row_sum = acc;
+            row_max = new_max;
+          }
         } else {
           // every term is an exact zero and the maximum did not move: nothing to add
           if (2 * kb + t < 64) dead |= 1ull << (2 * kb + t);

@@ -207,19 +207,25 @@ def matmul_bf16(c, m, n, k, transposed_b=False, batch=None, transposed_a=False):
     return A, Bm, O, sink
 
 
-def attention_bf16(c, batch=8, heads=12, ctx=1024, hd=64):
+def attention_bf16(c, batch=8, heads=12, ctx=1024, hd=64, mask_buffer=False):
     """The attention block of gpt2_forward on its own: q, k, v as [B, T, H*hd] bf16 buffers
     (heads interleaved along the feature axis, as the qkv projection leaves them), additive
-    causal mask built from an arange buffer, softmax in fp32, heads merged back into
-    [B, T, H*hd] by a separate copy kernel (in gpt2_forward the projection matmul reads
-    the per-head layout instead)."""
+    causal mask built from an arange buffer (or, with mask_buffer, any additive [T, T] bf16
+    mask handed in as a buffer), softmax in fp32, heads merged back into [B, T, H*hd] by a
+    separate copy kernel (in gpt2_forward the projection matmul reads the per-head layout
+    instead)."""
     D = heads * hd
     q, k, v = (c.buffer((batch, ctx, D), R.BF16, name=n) for n in ("q", "k", "v"))
-    arange = c.buffer((ctx,), R.F32, name="arange")
     out = c.buffer((batch, ctx, D), R.BF16, name="out")
-    row = arange.reshape((ctx, 1)).expand((ctx, ctx))
-    col = arange.reshape((1, ctx)).expand((ctx, ctx))
-    mask = row.lt(col).where(c.const(-1e9, R.BF16), c.const(0.0, R.BF16)).reshape((1, 1, ctx, ctx)).contiguous()
+    bufs = dict(q=q, k=k, v=v, out=out)
+    if mask_buffer:
+        bufs["mask"] = c.buffer((ctx, ctx), R.BF16, name="mask")
+        mask = bufs["mask"].reshape((1, 1, ctx, ctx))
+    else:
+        bufs["arange"] = arange = c.buffer((ctx,), R.F32, name="arange")
+        row = arange.reshape((ctx, 1)).expand((ctx, ctx))
+        col = arange.reshape((1, ctx)).expand((ctx, ctx))
+        mask = row.lt(col).where(c.const(-1e9, R.BF16), c.const(0.0, R.BF16)).reshape((1, 1, ctx, ctx)).contiguous()
     qh = q.reshape((batch, ctx, heads, hd)).permute((0, 2, 1, 3))
     kh = k.reshape((batch, ctx, heads, hd)).permute((0, 2, 1, 3))
     vh = v.reshape((batch, ctx, heads, hd)).permute((0, 2, 1, 3))
@@ -228,7 +234,7 @@ def attention_bf16(c, batch=8, heads=12, ctx=1024, hd=64):
     attn = scores.cast(R.F32).softmax(-1).cast(R.BF16).contiguous()
     ctxv = attn.cast(R.F32).dot(vh.cast(R.F32)).cast(R.BF16).contiguous()
     merged = ctxv.permute((0, 2, 1, 3)).reshape((batch, ctx, D))
-    return dict(q=q, k=k, v=v, arange=arange, out=out), c.sink((out, merged))
+    return bufs, c.sink((out, merged))
 
 
 def mlp_train_step(c, batch=4096, d_in=784, d_hid=512, d_out=10, lr=0.01):

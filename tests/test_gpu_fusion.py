@@ -93,6 +93,40 @@ def test_fused_attention_matches_unfused_and_reference(qk_gain, form):
     c.close()
 
 
+@pytest.mark.parametrize("form", ["online", "exact"])
+def test_attention_with_infinite_mask_entries(form):
+    """An additive mask handed in as a buffer, with -inf entries: causal; the first 64 keys
+    hidden from the last 128 queries (their first key tiles are fully masked, so the running
+    maximum starts at -inf); a band of keys hidden from everybody; one query with no key at
+    all, whose output row is NaN in the reference."""
+    ctx, heads, hd, batch = 256, 2, 64, 1
+    c = R.Ctx()
+    bufs, sink = graphs.attention_bf16(c, batch=batch, heads=heads, ctx=ctx, hd=hd, mask_buffer=True)
+    g = np.random.default_rng(5)
+    ninf = np.float32(-np.inf)
+    mask = np.where(np.arange(ctx)[:, None] < np.arange(ctx)[None, :], ninf, np.float32(0.0)).astype(np.float32)
+    mask[128:, :64] = ninf
+    mask[:, 96:128] = ninf
+    mask[5, :] = ninf
+    mask[200:, 200:] += g.normal(0, 1, (56, 56)).astype(np.float32)   # finite biases as well
+    arrays = {bufs["mask"]: R.f32_to_bf16_bits(mask), bufs["out"]: np.zeros(batch * ctx * heads * hd, np.uint16)}
+    for n in ("q", "k", "v"):
+        arrays[bufs[n]] = R.f32_to_bf16_bits(g.uniform(-1, 1, batch * ctx * heads * hd).astype(np.float32) * (3.0 if n != "v" else 1.0))
+    want = R.bf16_bits_to_f32(run_ref(c, sink, arrays)[bufs["out"]]).reshape(ctx, heads * hd)
+    if form == "exact":
+        os.environ["POLY_HIP_EXACT_ATTENTION"] = "1"
+    try:
+        got, info = run_hip(c, sink, arrays)
+    finally:
+        os.environ.pop("POLY_HIP_EXACT_ATTENTION", None)
+    c.close()
+    assert any(k["klass"] == "attention-mfma" and ("one pass" if form == "online" else "two passes") in k["desc"] for k in info), [k["desc"] for k in info]
+    have = R.bf16_bits_to_f32(got[bufs["out"]]).reshape(ctx, heads * hd)
+    assert np.isnan(want[5]).all() and np.isnan(have[5]).all()
+    assert np.isfinite(np.delete(want, 5, axis=0)).all() and np.isfinite(np.delete(have, 5, axis=0)).all()
+    assert_close(have, want, rtol=2e-2, atol=8e-3 if form == "online" else 2e-3, what=f"{form} attention with -inf mask entries")
+
+
 def test_lookup_table_epilogue_is_bit_identical_to_the_arithmetic():
     """A pointwise kernel of one 16-bit input fused behind a matmul is evaluated through a
     65536-entry table filled by its own expression: results must not change by a bit."""
