@@ -207,7 +207,7 @@ def matmul_bf16(c, m, n, k, transposed_b=False, batch=None, transposed_a=False):
     return A, Bm, O, sink
 
 
-def attention_bf16(c, batch=8, heads=12, ctx=1024, hd=64, mask_buffer=False):
+def attention_bf16(c, batch=8, heads=12, ctx=1024, hd=64, mask_buffer=False, dt=None):
     """The attention block of gpt2_forward on its own: q, k, v as [B, T, H*hd] bf16 buffers
     (heads interleaved along the feature axis, as the qkv projection leaves them), additive
     causal mask built from an arange buffer (or, with mask_buffer, any additive [T, T] bf16
@@ -215,24 +215,25 @@ def attention_bf16(c, batch=8, heads=12, ctx=1024, hd=64, mask_buffer=False):
     separate copy kernel (in gpt2_forward the projection matmul reads the per-head layout
     instead)."""
     D = heads * hd
-    q, k, v = (c.buffer((batch, ctx, D), R.BF16, name=n) for n in ("q", "k", "v"))
-    out = c.buffer((batch, ctx, D), R.BF16, name="out")
+    dt = R.BF16 if dt is None else dt   # the 16-bit type of q, k, v, scores and output
+    q, k, v = (c.buffer((batch, ctx, D), dt, name=n) for n in ("q", "k", "v"))
+    out = c.buffer((batch, ctx, D), dt, name="out")
     bufs = dict(q=q, k=k, v=v, out=out)
     if mask_buffer:
-        bufs["mask"] = c.buffer((ctx, ctx), R.BF16, name="mask")
+        bufs["mask"] = c.buffer((ctx, ctx), dt, name="mask")
         mask = bufs["mask"].reshape((1, 1, ctx, ctx))
     else:
         bufs["arange"] = arange = c.buffer((ctx,), R.F32, name="arange")
         row = arange.reshape((ctx, 1)).expand((ctx, ctx))
         col = arange.reshape((1, ctx)).expand((ctx, ctx))
-        mask = row.lt(col).where(c.const(-1e9, R.BF16), c.const(0.0, R.BF16)).reshape((1, 1, ctx, ctx)).contiguous()
+        mask = row.lt(col).where(c.const(-1e9, dt), c.const(0.0, dt)).reshape((1, 1, ctx, ctx)).contiguous()
     qh = q.reshape((batch, ctx, heads, hd)).permute((0, 2, 1, 3))
     kh = k.reshape((batch, ctx, heads, hd)).permute((0, 2, 1, 3))
     vh = v.reshape((batch, ctx, heads, hd)).permute((0, 2, 1, 3))
-    scores = qh.cast(R.F32).dot(kh.permute((0, 1, 3, 2)).cast(R.F32)).cast(R.BF16).contiguous()
-    scores = (scores * c.const(1.0 / math.sqrt(hd), R.BF16) + mask.expand((batch, heads, ctx, ctx))).contiguous()
-    attn = scores.cast(R.F32).softmax(-1).cast(R.BF16).contiguous()
-    ctxv = attn.cast(R.F32).dot(vh.cast(R.F32)).cast(R.BF16).contiguous()
+    scores = qh.cast(R.F32).dot(kh.permute((0, 1, 3, 2)).cast(R.F32)).cast(dt).contiguous()
+    scores = (scores * c.const(1.0 / math.sqrt(hd), dt) + mask.expand((batch, heads, ctx, ctx))).contiguous()
+    attn = scores.cast(R.F32).softmax(-1).cast(dt).contiguous()
+    ctxv = attn.cast(R.F32).dot(vh.cast(R.F32)).cast(dt).contiguous()
     merged = ctxv.permute((0, 2, 1, 3)).reshape((batch, ctx, D))
     return bufs, c.sink((out, merged))
 

@@ -127,6 +127,32 @@ def test_attention_with_infinite_mask_entries(form):
     assert_close(have, want, rtol=2e-2, atol=8e-3 if form == "online" else 2e-3, what=f"{form} attention with -inf mask entries")
 
 
+@pytest.mark.parametrize("form", ["online", "exact"])
+def test_attention_fp16(form):
+    """The same kernel group in fp16.  The reference's mask constant -1e9 is -inf in fp16,
+    so every masked score is -inf."""
+    ctx, heads, hd, batch = 256, 2, 64, 2
+    c = R.Ctx()
+    bufs, sink = graphs.attention_bf16(c, batch=batch, heads=heads, ctx=ctx, hd=hd, dt=R.F16)
+    g = np.random.default_rng(9)
+    n = batch * ctx * heads * hd
+    arrays = {bufs["arange"]: np.arange(ctx, dtype=np.float32), bufs["out"]: np.zeros(n, np.float16)}
+    for name in ("q", "k", "v"):
+        arrays[bufs[name]] = (g.uniform(-1, 1, n) * (2.0 if name != "v" else 1.0)).astype(np.float16)
+    want = run_ref(c, sink, arrays)[bufs["out"]].astype(np.float32)
+    if form == "exact":
+        os.environ["POLY_HIP_EXACT_ATTENTION"] = "1"
+    try:
+        got, info = run_hip(c, sink, arrays)
+    finally:
+        os.environ.pop("POLY_HIP_EXACT_ATTENTION", None)
+    c.close()
+    assert any(k["klass"] == "attention-mfma" and "f16" in k["desc"] and ("one pass" if form == "online" else "two passes") in k["desc"]
+               for k in info), [k["desc"] for k in info]
+    assert np.isfinite(want).all()
+    assert_close(got[bufs["out"]].astype(np.float32), want, rtol=2e-2, atol=2e-3, what=f"{form} attention in fp16")
+
+
 def test_lookup_table_epilogue_is_bit_identical_to_the_arithmetic():
     """A pointwise kernel of one 16-bit input fused behind a matmul is evaluated through a
     65536-entry table filled by its own expression: results must not change by a bit."""
