@@ -490,8 +490,88 @@ static bool match_matmul_tail(const Sched &sc, int s_item, const std::vector<cha
 struct RowPhase {
   Member m;
   bool is_map = false;
+  bool keeps_row = false;           // a map whose output row only later phases read: kept in registers
   int red = -1, own_red_ord = -1;   // REDUCE node and its range ordinal (reduce phases)
 };
+
+// Value of `l` -- an index expression of a kernel that walks a buffer with ONE flattened
+// range `flat_ord` -- in master coordinates, given that the flat position is `pos` there
+// (mixed radix: non-negative coefficients).  DIV and MOD by c are exact digit operations
+// when every coefficient is either a multiple of c or belongs to a part that stays below c.
+static bool flat_lin_to_aff(const KernelGraph &g, const Lin &l, int flat_ord, const Aff &pos, const std::vector<int64_t> &mext, Aff *out) {
+  out->c.clear();
+  out->c0 = l.c0;
+  for (const Term &t : l.terms) {
+    const Atom &a = g.atoms[(size_t)t.atom];
+    Aff v;
+    if (a.kind == Atom::RANGE) {
+      if (g.range_ord.at(a.node) != flat_ord) return false;
+      v = pos;
+    } else if (a.kind == Atom::DIV || a.kind == Atom::MOD) {
+      Aff in;
+      if (a.c <= 0 || !flat_lin_to_aff(g, a.inner, flat_ord, pos, mext, &in) || in.c0 < 0) return false;
+      int64_t low_max = in.c0 % a.c;
+      for (auto &kv : in.c) {
+        if (kv.second < 0) return false;
+        if (kv.second % a.c != 0) low_max += kv.second * (mext[(size_t)kv.first] - 1);
+      }
+      if (low_max >= a.c) return false;
+      v.c0 = a.kind == Atom::DIV ? in.c0 / a.c : in.c0 % a.c;
+      for (auto &kv : in.c) {
+        if (kv.second % a.c == 0) { if (a.kind == Atom::DIV) v.c[kv.first] = kv.second / a.c; }
+        else if (a.kind == Atom::MOD) v.c[kv.first] = kv.second;
+      }
+    } else {
+      return false;
+    }
+    out->c0 += t.coef * v.c0;
+    for (auto &kv : v.c) out->c[kv.first] += t.coef * kv.second;
+  }
+  for (auto it = out->c.begin(); it != out->c.end();) it = it->second == 0 ? out->c.erase(it) : std::next(it);
+  return true;
+}
+
+// A pointwise kernel with one flattened range over a buffer of rows x R elements, as the
+// last phase of a row chain: its flat position is where the row result `row_at` was stored.
+static bool map_phase_flat(const Sched &sc, int item, const std::vector<int64_t> &mext, int red_master,
+                           const std::vector<std::pair<int, Aff>> &results, const std::vector<char> &row_result,
+                           const std::vector<std::string> &result_names, Member *m) {
+  const KernelGraph &g = sc.graphs[(size_t)item];
+  if (g.stores.size() != 1 || g.stores[0].ranges.size() != 1) return false;
+  const int ord = g.stores[0].ranges[0];
+  // the position: the store index of the latest whole-row result, which must be dense
+  const Aff *pos = nullptr;
+  for (size_t r = results.size(); r-- > 0;) if (row_result[r]) { pos = &results[r].second; break; }
+  if (!pos || pos->c0 != 0 || !pos->c.count(red_master) || pos->c.at(red_master) != 1) return false;
+  int64_t span = 1;
+  for (auto &kv : pos->c) { if (kv.second <= 0) return false; span += (mext[(size_t)kv.first] - 1) * kv.second; }
+  int64_t numel = 1;
+  for (auto &kv : pos->c) numel *= mext[(size_t)kv.first];
+  if (span != numel || g.ranges[(size_t)ord].extent != numel) return false;
+  m->item = item;
+  for (int id = 0; id < (int)g.nodes.size(); id++) {
+    const KNode &k = g.n(id);
+    if (k.op != POLY_OP_LOAD) continue;
+    const KNode &ix = g.n(k.src[0]);
+    const int sl = sc.slot(item, g.param_slot(ix.src[0]));
+    const int lin = g.n(ix.src[1]).lin;
+    for (size_t r = 0; r < results.size(); r++) {
+      if (results[r].first != sl) continue;
+      Aff a;
+      if (ix.src.size() != 2 || k.guard >= 0 || lin < 0) return false;
+      if (!flat_lin_to_aff(g, g.lins[(size_t)lin], ord, *pos, mext, &a) || !(a == results[r].second)) return false;
+      m->preset[id] = result_names[r];
+    }
+  }
+  // it must store element p at index p
+  const int li = g.n(g.n(g.stores[0].index).src[1]).lin;
+  Aff st;
+  if (li < 0 || !flat_lin_to_aff(g, g.lins[(size_t)li], ord, *pos, mext, &st) || !(st == *pos)) return false;
+  Aff base = *pos;
+  base.c.erase(red_master);
+  m->range_expr[ord] = aff_expr(base);   // position of the row's first element
+  return true;
+}
 
 // Maps the ranges of `item` onto master ranges through the buffers it shares with the
 // phases before it: results of earlier phases (read at the row they were stored at) and
@@ -539,7 +619,7 @@ static void collect_ref_loads(const Sched &sc, const Member &m, std::vector<std:
   }
 }
 
-static bool match_row_chain(const Sched &sc, int a_item, const std::vector<char> &taken, FusedGroup *out) {
+static bool match_row_chain_impl(const Sched &sc, int a_item, const std::vector<char> &taken, FusedGroup *out, bool allow_rows) {
   const PolySchedule *s = sc.s;
   const KernelGraph &gA = sc.graphs[(size_t)a_item];
   auto reduce_shape = [&](const KernelGraph &g, int *red, int *ord) {
@@ -567,10 +647,10 @@ static bool match_row_chain(const Sched &sc, int a_item, const std::vector<char>
   for (int r : gA.stores[0].ranges) rows *= (double)gA.ranges[(size_t)r].extent;
   if (rows < 1 || rows > 2147483647.0) return false;
 
-  auto store_aff = [&](const Member &m, Aff *a) {
+  auto store_aff = [&](const Member &m, Aff *a, bool whole_row = false) {
     const KernelGraph &g = sc.graphs[(size_t)m.item];
     const int li = g.n(g.n(g.stores[0].index).src[1]).lin;
-    return li >= 0 && lin_to_aff(g, g.lins[(size_t)li], m.rm, a) && !a->c.count(red_master);
+    return li >= 0 && lin_to_aff(g, g.lins[(size_t)li], m.rm, a) && (a->c.count(red_master) != 0) == whole_row;
   };
   auto out_slot_of = [&](int item) {
     const KernelGraph &g = sc.graphs[(size_t)item];
@@ -588,6 +668,8 @@ static bool match_row_chain(const Sched &sc, int a_item, const std::vector<char>
   }
   collect_ref_loads(sc, A.m, &ref_loads);
   // grow: the readers of the latest result decide what comes next
+  std::vector<char> row_result{0};   // per result: a whole row (kept in registers) instead of one value per row
+  int n_reduces = 1;
   for (;;) {
     const int cur = results.back().first;
     if (!s->buf_slots[cur].is_intermediate || sc.writers[(size_t)cur].size() != 1) return false;
@@ -600,7 +682,7 @@ static bool match_row_chain(const Sched &sc, int a_item, const std::vector<char>
       else { if (next_reduce >= 0) return false; next_reduce = r; }
     }
     if (next_map < 0) return false;                    // every chain ends in a pointwise kernel
-    if (next_reduce >= 0 && phases.size() < 3) {
+    if (next_reduce >= 0 && n_reduces < 3) {
       RowPhase B;
       const KernelGraph &g = sc.graphs[(size_t)next_reduce];
       if (!reduce_shape(g, &B.red, &B.own_red_ord)) return false;
@@ -610,7 +692,9 @@ static bool match_row_chain(const Sched &sc, int a_item, const std::vector<char>
       Aff a;
       if (!store_aff(B.m, &a)) FA_REJECT();
       phases.push_back(B);
+      n_reduces++;
       results.push_back({out_slot_of(next_reduce), a});
+      row_result.push_back(0);
       names.push_back(strf("s%zu", results.size()));
       collect_ref_loads(sc, B.m, &ref_loads);
       continue;
@@ -620,13 +704,43 @@ static bool match_row_chain(const Sched &sc, int a_item, const std::vector<char>
     C.is_map = true;
     const KernelGraph &g = sc.graphs[(size_t)next_map];
     if (!g.reduces.empty() || g.stores.size() != 1 || g.stores[0].gate >= 0 || !g.vars.empty()) return false;
-    if (!map_phase(sc, next_map, mext, ref_loads, results, names, &C.m)) FA_REJECT();
-    std::set<int> covered;
-    for (int r : g.stores[0].ranges) {
-      if (!C.m.rm.count(r)) FA_REJECT();
-      covered.insert(C.m.rm[r]);
+    if (!map_phase(sc, next_map, mext, ref_loads, results, names, &C.m)) {
+      // one flattened range instead of (rows, position in the row)
+      C.m = Member();
+      if (!map_phase_flat(sc, next_map, mext, red_master, results, row_result, names, &C.m)) FA_REJECT();
+    } else {
+      std::set<int> covered;
+      for (int r : g.stores[0].ranges) {
+        if (!C.m.rm.count(r)) FA_REJECT();
+        covered.insert(C.m.rm[r]);
+      }
+      if (covered.size() != gA.stores[0].ranges.size() + 1 || !covered.count(red_master)) FA_REJECT();
     }
-    if (covered.size() != gA.stores[0].ranges.size() + 1 || !covered.count(red_master)) FA_REJECT();
+    // A map whose output is an intermediate that one more row reduction (and the map after
+    // it) reads -- softmax as max, exp, sum, divide; LayerNorm as mean, centre, variance,
+    // scale -- keeps its row in registers and the chain goes on.
+    const int c_out = out_slot_of(next_map);
+    Aff ca;
+    bool row_goes_on = allow_rows && C.m.range_expr.empty() && n_reduces < 3 && !row_result.back() && s->buf_slots[c_out].is_intermediate &&
+                       sc.writers[(size_t)c_out].size() == 1 && store_aff(C.m, &ca, true);
+    if (row_goes_on) {
+      int rr = 0, rm = 0;
+      for (int r : sc.readers[(size_t)c_out]) {
+        if (taken[(size_t)r]) row_goes_on = false;
+        else if (sc.graphs[(size_t)r].reduces.empty()) rm++;
+        else rr++;
+      }
+      if (rr != 1 || rm > 1) row_goes_on = false;
+    }
+    if (row_goes_on) {
+      C.keeps_row = true;
+      phases.push_back(C);
+      results.push_back({c_out, ca});
+      row_result.push_back(1);
+      names.push_back(strf("t%zu[it].v[u]", results.size()));
+      collect_ref_loads(sc, C.m, &ref_loads);
+      continue;
+    }
     phases.push_back(C);
     break;
   }
@@ -697,6 +811,8 @@ static bool match_row_chain(const Sched &sc, int a_item, const std::vector<char>
   struct RowCache { std::string key, type; int nit; };
   std::vector<RowCache> cache;
   int n_cached_uses = 0;
+  int row_V = 0, row_nit = 0;       // vector width and step count of the rows kept between phases
+  std::string row_decls;             // their declarations in the kernel body
   for (size_t pi = 0; pi < phases.size(); pi++) {
     const RowPhase &ph = phases[pi];
     const KernelGraph &g = sc.graphs[(size_t)ph.m.item];
@@ -710,6 +826,8 @@ static bool match_row_chain(const Sched &sc, int a_item, const std::vector<char>
       em.bind_range(kv.first, strf("r%d", kv.second));
       S0.avail |= (uint64_t)1 << kv.first;
     }
+    std::string flat_base;           // flat phase: position of the row's first element
+    for (auto &kv : ph.m.range_expr) { own_f = kv.first; flat_base = kv.second; }
     if (own_f < 0) FA_REJECT();
     for (auto &kv : ph.m.preset) em.preset(kv.first, kv.second);
     const std::vector<int> roots{ph.is_map ? g.stores[0].value : g.n(ph.red).src[0]};
@@ -724,7 +842,11 @@ static bool match_row_chain(const Sched &sc, int a_item, const std::vector<char>
           maxsz = std::max(maxsz, dt_size(g.n(i).dt));
       if (ph.is_map) maxsz = std::max(maxsz, dt_size(g.n(g.stores[0].param).dt));
       V = std::max(1, 16 / maxsz);
+      bool reads_row = false;
+      for (auto &kv : ph.m.preset) if (kv.second.find("[it]") != std::string::npos) reads_row = true;
+      if (reads_row) V = row_V;   // positions must line up with the phase that made the row
       while (V > 1 && (R % V != 0 || R < (int64_t)G * V)) V /= 2;
+      if (reads_row && V != row_V) FA_REJECT();
       if (ph.is_map) {
         const int li = g.n(g.n(g.stores[0].index).src[1]).lin;
         while (V > 1 && (li < 0 || !lin_vec_ok(g, g.lins[(size_t)li], own_f, V) ||
@@ -738,7 +860,19 @@ static bool match_row_chain(const Sched &sc, int a_item, const std::vector<char>
     L.indent = 2;
     std::vector<int> pres;
     const int nit = (int)((R + (int64_t)G * V - 1) / ((int64_t)G * V));
-    const bool unrolled = G == 64 && nit <= 4;   // iterations as an unrolled loop over `it`
+    // iterations as an unrolled loop over `it` (what is kept between phases is indexed by it)
+    const bool unrolled = (G == 64 && nit <= 4) || (G == 256 && nit <= 8);
+    {
+      bool reads_row = false;
+      for (auto &kv : ph.m.preset) if (kv.second.find("[it]") != std::string::npos) reads_row = true;
+      if ((reads_row || ph.keeps_row) && (!unrolled || V <= 1)) FA_REJECT();
+      if (reads_row && nit != row_nit) FA_REJECT();
+      if (ph.keeps_row) {
+        if (row_V && (row_V != V || row_nit != nit)) FA_REJECT();
+        row_V = V;
+        row_nit = nit;
+      }
+    }
     const std::function<std::string(int, const std::string &)> keep = [&](int node, const std::string &ld) -> std::string {
       const KNode &ix = g.n(g.n(node).src[0]);
       Aff a;
@@ -753,10 +887,13 @@ static bool match_row_chain(const Sched &sc, int a_item, const std::vector<char>
     };
     if (V > 1) pres = hoist_vector_loads(g, em, roots, own_f, V, fv + "_0", &L, unrolled ? &keep : nullptr);
     // the row loop: positions fv_0 = lane * V, + G * V, ...
+    // q: position in the row; the phase's own variable starts there (or, for a flat phase,
+    // at the row's first element plus q)
+    const std::string start = flat_base.empty() ? "q_0" : flat_base + " + q_0";
     const std::string loop_open = unrolled
-        ? strf("#pragma unroll\n  for (int it = 0; it < %d; it++) {\n  const int %s_0 = lane * %d + it * %d;\n  if (%s_0 < %lld) {\n", nit, fv.c_str(), V, G * V,
-               fv.c_str(), (long long)R)
-        : strf("  for (int %s_0 = lane * %d; %s_0 < %lld; %s_0 += %d) {\n", fv.c_str(), V, fv.c_str(), (long long)R, fv.c_str(), G * V);
+        ? strf("#pragma unroll\n  for (int it = 0; it < %d; it++) {\n  const int q_0 = lane * %d + it * %d;\n  if (q_0 < %lld) {\n  const int %s_0 = %s;\n", nit, V, G * V,
+               (long long)R, fv.c_str(), start.c_str())
+        : strf("  for (int q_0 = lane * %d; q_0 < %lld; q_0 += %d) {\n  const int %s_0 = %s;\n", V, (long long)R, G * V, fv.c_str(), start.c_str());
     const std::string loop_close = unrolled ? "  }\n  }\n" : "  }\n";
     Scope U;                          // one element
     U.parent = &L;
@@ -797,7 +934,9 @@ static bool match_row_chain(const Sched &sc, int a_item, const std::vector<char>
       const int p = g.param_slot(st.param);
       std::string v = em.emit(st.value, &U);
       const char *odt = dt_cname(g.n(st.param).dt);
-      if (V > 1) {
+      if (ph.keeps_row) {
+        U.code += strf("      %s = %s;\n", names[pi].c_str(), v.c_str());
+      } else if (V > 1) {
         U.code += strf("      out.v[u] = %s;\n", v.c_str());
       } else {
         std::string idx = em.emit(g.n(st.index).src[1], &U);
@@ -809,10 +948,10 @@ static bool match_row_chain(const Sched &sc, int a_item, const std::vector<char>
       S0.code.clear();
       loop += loop_open;
       loop += L.code;
-      if (V > 1) loop += strf("    poly_vec<%s,%d> out;\n", odt, V);
+      if (V > 1 && !ph.keeps_row) loop += strf("    poly_vec<%s,%d> out;\n", odt, V);
       loop += strf("#pragma unroll\n    for (int u = 0; u < %d; u++) {\n      const int %s = %s_0 + u;\n", V, fv.c_str(), fv.c_str());
       loop += U.code + "    }\n";
-      if (V > 1) loop += strf("    poly_vstore<%s,%d>(data%d + %s, out);\n", odt, V, p, addr.c_str());
+      if (V > 1 && !ph.keeps_row) loop += strf("    poly_vstore<%s,%d>(data%d + %s, out);\n", odt, V, p, addr.c_str());
       loop += loop_close;
     }
     if (em.failed() || em.uses_threefry) FA_REJECT();
@@ -824,7 +963,20 @@ static bool match_row_chain(const Sched &sc, int a_item, const std::vector<char>
     code += strf("__device__ __forceinline__ %s %s(const long long row, const int lane%s%s, %s) {\n", ret.c_str(), fn.c_str(), lead.c_str(),
                  cache_params.c_str(), params_decl(g).c_str());
     code += row_decomp + loop + tail + "}\n";
-    if (!ph.is_map) {
+    if (ph.keeps_row) {
+      // the row it makes: an array the later phases receive by reference
+      const std::string base = names[pi].substr(0, names[pi].find('['));
+      const std::string type = strf("poly_vec<%s,%d>", dt_cname(g.n(g.stores[0].value).dt), V);
+      row_decls += strf("    %s %s[%d];\n", type.c_str(), base.c_str(), nit);
+      const std::string param = strf(", %s (&%s)[%d]", type.c_str(), base.c_str(), nit);
+      // this phase's own signature needs it too: it was built above without it
+      const size_t sig_at = code.rfind(strf("%s(const long long row, const int lane%s", fn.c_str(), lead.c_str()));
+      if (sig_at == std::string::npos) FA_REJECT();
+      code.insert(sig_at + strf("%s(const long long row, const int lane%s", fn.c_str(), lead.c_str()).size(), param);
+      calls += strf("    %s(row, lane%s, %s%s, %s);\n", fn.c_str(), lead_call.c_str(), base.c_str(), cache_args.c_str(), call_args(ph.m.item).c_str());
+      lead += param;
+      lead_call += ", " + base;
+    } else if (!ph.is_map) {
       calls += strf("    const %s %s = %s(row, lane%s%s, %s);\n", ret.c_str(), names[pi].c_str(), fn.c_str(), lead_call.c_str(),
                     cache_args.c_str(), call_args(ph.m.item).c_str());
       lead += strf(", const %s %s", ret.c_str(), names[pi].c_str());
@@ -842,6 +994,7 @@ static bool match_row_chain(const Sched &sc, int a_item, const std::vector<char>
     body += "  const int lane = threadIdx.x;\n  const long long row = blockIdx.x;\n  {\n";
   }
   for (size_t ci = 0; ci < cache.size(); ci++) body += strf("    %s c%zu[%d];\n", cache[ci].type.c_str(), ci, cache[ci].nit);
+  body += row_decls;
   body += calls + "  }\n}\n";
 
   out->items = items;
@@ -857,9 +1010,15 @@ static bool match_row_chain(const Sched &sc, int a_item, const std::vector<char>
   rk.klass = KernelClass::ROW_REDUCE;
   rk.strategy = strf("row chain of %zu kernels (%s) G=%d R=%lld rows=%.0f", phases.size(), strat.c_str(), G, (long long)R, rows);
   if (n_cached_uses) rk.strategy += strf(", %d row loads kept in registers", n_cached_uses);
+  if (row_V) rk.strategy += ", intermediate rows kept in registers";
   rk.n_params = (int)arg_slots.size();
   rk.bytes = bytes;
   return true;
+}
+
+static bool match_row_chain(const Sched &sc, int a_item, const std::vector<char> &taken, FusedGroup *out) {
+  // first with maps in the middle of the chain (their rows kept in registers), then the plain form
+  return match_row_chain_impl(sc, a_item, taken, out, true) || match_row_chain_impl(sc, a_item, taken, out, false);
 }
 
 // A kernel that only moves data: out[store index] = in[load index], both affine in the
