@@ -208,7 +208,7 @@ def main():
     line = {
         "metric": metric, "value": round(value, 1), "unit": unit, "n_gpus": 1, "steps": args.steps,
         "warmup": args.warmup, "ms_per_step": round(ms, 4), "higher_is_better": True, "scaling": "weak",
-        "vs_baseline": None, "dtype": "bf16", "data": "synthetic",
+        "vs_baseline": None, "dtype": "f32" if "_f32" in args.workload else "bf16", "data": "synthetic",
         "config": {"workload": workload, "plan": args.workload, "global_batch": 8 if tokens else None,
                    "seq_len": 1024 if tokens else None, "parallelism": "single GPU",
                    "execution": "hipGraph replay of the compiled plan, inputs resident in HBM"},
