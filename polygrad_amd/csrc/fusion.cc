@@ -1080,6 +1080,7 @@ static bool match_attention(const Sched &sc, int s_item, const std::vector<char>
   const int n_master = mS.nd_full[0].ord;
   const StoreInfo &stS = gS.stores[0];
   const DT tin = mS.A.dt;
+  if (tin != DT_BF16 && tin != DT_F16) FA_REJECT();
   if (gS.n(stS.value).dt != tin) FA_REJECT();
   std::vector<int64_t> mext(gS.ranges.size());
   for (size_t i = 0; i < gS.ranges.size(); i++) mext[i] = gS.ranges[i].extent;

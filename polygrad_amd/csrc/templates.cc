@@ -17,6 +17,9 @@ namespace {
 const char *const kMatmulTemplate =
 #include "matmul_mfma.hip.inc"
     ;
+const char *const kMatmulF32Template =
+#include "matmul_f32_mfma.hip.inc"
+    ;
 
 PolyOps reduce_op(const KNode &k) {
   return k.u->arg.kind == POLY_ARG_OPS ? k.u->arg.ops : (PolyOps)k.u->arg.i;
@@ -165,7 +168,7 @@ bool match_matmul(const KernelGraph &g, MatmulMatch *mm, int *reject_line) {
   if (mul.op != POLY_OP_MUL || mul.dt != DT_F32) MM_REJECT();
   Operand A, B;
   if (!match_operand(g, mul.src[0], &A) || !match_operand(g, mul.src[1], &B)) MM_REJECT();
-  if (A.dt != B.dt || (A.dt != DT_BF16 && A.dt != DT_F16)) MM_REJECT();
+  if (A.dt != B.dt || (A.dt != DT_BF16 && A.dt != DT_F16 && A.dt != DT_F32)) MM_REJECT();
   for (const ParamInfo &p : g.params) if (p.numel >= ((int64_t)1 << 31)) MM_REJECT();
   const Lin &la = g.lins[(size_t)A.lin], &lb = g.lins[(size_t)B.lin];
   KSplit ka, kb;
@@ -350,12 +353,75 @@ bool try_render_matmul(const KernelGraph &g, const std::string &fn, const Render
   return render_matmul(mm, ep, out);
 }
 
+// fp32 operands: kernels/matmul_f32_mfma.hip (v_mfma_f32_32x32x2_f32, exact fp32 products).
+static bool render_matmul_f32(const MatmulMatch &mm, const MatmulEpilogue &ep, RenderedKernel *out) {
+  const int64_t K = mm.K, M = mm.M, N = mm.N, Z = mm.Z;
+  if (getenv("POLY_HIP_NO_F32_MFMA")) return reject(__LINE__);
+  // operand layout: 16-byte pieces along K, or along the operand's row axis
+  auto layout = [&](const KSplit &ks, const std::vector<Dim> &dims, bool is_a, int64_t rows, bool *kc) {
+    const int64_t inner_c = is_a ? dims.back().ca : dims.back().cb;
+    if (K % 16 != 0) return reject(__LINE__);
+    if (ks.s_lo == 1 && ks.kb % 16 == 0) { *kc = true; return true; }
+    if (inner_c == 1 && dims.back().extent % 4 == 0 && rows % 4 == 0) { *kc = false; return true; }
+    return reject(__LINE__);
+  };
+  bool a_kc, b_kc;
+  if (!layout(mm.ka, mm.md, true, M, &a_kc) || !layout(mm.kb, mm.nd, false, N, &b_kc)) return reject(__LINE__);
+  // 4 waves; narrow outputs get a narrow tile
+  int BM = 128, BN = 128, WVM = 2, WVN = 2;
+  if (N <= 32) { BN = 32; BM = 256; WVM = 4; WVN = 1; }
+  else if (N <= 64) { BN = 64; BM = 128; WVM = 4; WVN = 1; }
+  else if (M <= 32) { BM = 32; BN = 256; WVM = 1; WVN = 4; }
+  else if (M <= 64) { BM = 64; BN = 128; WVM = 1; WVN = 4; }
+  else if (((M + 127) / 128) * ((N + 127) / 128) * Z < 256) {
+    BM = 64; BN = 64; WVM = 2; WVN = 2;
+    // still fewer workgroups than CUs: two-wave workgroups on 32x64 tiles
+    if (((M + 63) / 64) * ((N + 63) / 64) * Z < 192) { BM = 32; BN = 64; WVM = 1; WVN = 2; }
+  }
+  const int64_t tiles = ((M + BM - 1) / BM) * ((N + BN - 1) / BN);
+  if (tiles > 2147483647LL / 2) return reject(__LINE__);
+  std::string cfg;
+  cfg += strf("#define POLY_M %lld\n#define POLY_N %lld\n#define POLY_K %lld\n#define POLY_Z %lld\n", (long long)M, (long long)N, (long long)K, (long long)Z);
+  cfg += strf("#define POLY_BM %d\n#define POLY_BN %d\n#define POLY_WAVES_M %d\n#define POLY_WAVES_N %d\n#define POLY_GROUP_M 8\n", BM, BN, WVM, WVN);
+  cfg += strf("#define POLY_A_KC %d\n#define POLY_B_KC %d\n", a_kc ? 1 : 0, b_kc ? 1 : 0);
+  cfg += strf("#define POLY_A_PTR %s\n#define POLY_B_PTR %s\n", ep.a_ptr.c_str(), ep.b_ptr.c_str());
+  cfg += offset_fn("poly_a_row", mm.md, true, 0);
+  cfg += offset_fn("poly_b_row", mm.nd, false, 0);
+  if (mm.zd.empty()) {
+    cfg += strf("__device__ __forceinline__ int poly_a_z(int) { return %lld; }\n", (long long)mm.a_c0);
+    cfg += strf("__device__ __forceinline__ int poly_b_z(int) { return %lld; }\n", (long long)mm.b_c0);
+  } else {
+    cfg += offset_fn("poly_a_z", mm.zd, true, mm.a_c0);
+    cfg += offset_fn("poly_b_z", mm.zd, false, mm.b_c0);
+  }
+  cfg += matmul_k_fn("poly_a_k", mm.ka, K);
+  cfg += matmul_k_fn("poly_b_k", mm.kb, K);
+  cfg += strf("#define POLY_SIGNATURE %s\n", ep.signature.c_str());
+  cfg += ep.code;
+  cfg += strf("#define POLY_EPILOGUE(acc, m, n, z) %s\n", ep.call.c_str());
+  *out = RenderedKernel();
+  out->source = std::string(hip_prelude()) + cfg + kMatmulF32Template;
+  out->entry = "poly_k";
+  out->launch.grid[0] = (unsigned)tiles;
+  out->launch.grid[1] = (unsigned)Z;
+  out->launch.block[0] = (unsigned)(64 * WVM * WVN);
+  out->klass = KernelClass::MATMUL_MFMA;
+  out->strategy = strf("mfma 32x32x2 f32 M=%lld N=%lld K=%lld Z=%lld tile %dx%dx16 A:%s B:%s", (long long)M, (long long)N, (long long)K,
+                       (long long)Z, BM, BN, a_kc ? "k-major" : "m-major", b_kc ? "k-major" : "n-major");
+  out->n_params = ep.n_params;
+  out->n_vars = 0;
+  out->flops = 2.0 * (double)M * (double)N * (double)K * (double)Z;
+  out->bytes = ep.bytes;
+  return true;
+}
+
 bool render_matmul(const MatmulMatch &mm, const MatmulEpilogue &ep, RenderedKernel *out) {
   const int64_t K = mm.K, M = mm.M, N = mm.N, Z = mm.Z;
   const Operand &A = mm.A, &B = mm.B;
   const KSplit &ka = mm.ka, &kb = mm.kb;
   const std::vector<Dim> &md = mm.md, &nd = mm.nd, &zd = mm.zd;
   if (M > 2147483647LL || N > 2147483647LL || Z > 65535) return reject(__LINE__);
+  if (A.dt == DT_F32) return render_matmul_f32(mm, ep, out);
   int BK = 64;
   if (const char *e = getenv("POLY_HIP_MM_BK")) BK = atoi(e) == 32 ? 32 : 64;
   // operand layout: contiguous along K, or along its row axis

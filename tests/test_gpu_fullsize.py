@@ -177,6 +177,48 @@ def test_gpt2_medium_train_matmul_shapes(m, n, k, ta, tb):
     assert bool((err <= 1e-4 * bound + 1e-30).all()), f"max err/bound {float((err / bound).max()):.3e}"
 
 
+# fp32 operands: the 32x32x2 MFMA template.  (m, n, k, A stored (k, m), B stored (n, k), batch)
+F32_SHAPES = [
+    (4096, 512, 784, False, True, None),    # config 1 forward: X W1^T
+    (512, 784, 4096, True, False, None),    # config 1 backward: dW1 = dH^T X (both operands row-major in k)
+    (1000, 200, 64, False, False, None),    # ragged tiles in both directions, B row-major
+    (96, 1000, 256, False, True, None),     # ragged, narrow M
+    (256, 48, 128, False, True, None),      # narrow N
+    (40, 36, 32, True, True, None),         # one small tile, A stored (k, m)
+    (128, 256, 512, False, False, 5),       # batch of A against one B
+]
+
+
+@pytest.mark.parametrize("m,n,k,ta,tb,batch", F32_SHAPES)
+def test_f32_matmul_template(m, n, k, ta, tb, batch):
+    import torch
+    c = R.Ctx()
+    g = np.random.default_rng(m + 3 * n + 7 * k)
+    nb = batch or 1
+    A = c.buffer((k, m) if ta else ((m, k) if batch is None else (batch, m, k)), name="A")
+    Bm = c.buffer((n, k) if tb else (k, n), name="B")
+    O = c.buffer((m, n) if batch is None else (batch, m, n), name="C")
+    a = A.permute((1, 0)) if ta else A
+    b = Bm.permute((1, 0)) if tb else Bm
+    sink = c.sink((O, a.dot(b)))
+    av = g.normal(0, 1, nb * m * k).astype(np.float32)
+    bv = g.normal(0, 1, k * n).astype(np.float32)
+    got, info = run_hip(c, sink, {A: av, Bm: bv, O: np.full(nb * m * n, np.nan, np.float32)})
+    c.close()
+    assert len(info) == 1 and info[0]["klass"] == "matmul-mfma" and "f32" in info[0]["desc"], info
+    C = torch.from_numpy(got[O]).view(nb, m, n).double()
+    assert bool(torch.isfinite(C).all())
+    at = torch.from_numpy(av).double()
+    at = at.view(k, m).t().unsqueeze(0) if ta else at.view(nb, m, k)
+    bt = torch.from_numpy(bv).double()
+    bt = bt.view(n, k).t() if tb else bt.view(k, n)
+    want = at @ bt
+    bound = at.abs() @ bt.abs()
+    err = (C - want).abs()
+    # exact fp32 products, fp32 accumulation in another order than the reference's
+    assert bool((err <= 1e-4 * bound / max(1.0, k ** 0.5) + 1e-30).all()), f"max err/bound {float((err / bound).max()):.3e}"
+
+
 # ── config 4: GPT-2 small ────────────────────────────────────────────────────────────────
 
 def test_gpt2_small_batch_elements_are_independent():
