@@ -170,10 +170,45 @@ def test_kernel_groups_of_the_gpt2_plan_fuse_and_compile(hiplib):
         assert hiplib.poly_hip_fused_groups(pf.schedule, -1, None, None) == 0
     finally:
         del os.environ["POLY_HIP_NO_FUSION"]
-    # softmax and LayerNorm on their own: one row chain each; a single reduction: nothing
+    # softmax and LayerNorm on their own (scheduled as reduce, pointwise, reduce, pointwise over
+    # rows of 8192): one row chain of all four kernels each, the inputs and the row in between
+    # kept in registers; a single reduction: nothing
     for name, want in (("softmax", 1), ("layernorm", 1), ("sum", 0)):
         pf2 = PlanFile(os.path.join(ROOT, "polygrad_amd", "plans", f"rowops_f32_8192_{name}.polyplan"))
-        src = C.c_void_p()
-        assert hiplib.poly_hip_fused_groups(pf2.schedule, 0, C.byref(src), None) == want
+        src, n = C.c_void_p(), C.c_int()
+        assert hiplib.poly_hip_fused_groups(pf2.schedule, 0, C.byref(src), C.byref(n)) == want
         if want:
-            assert hiplib.poly_hip_compile_check(_ffi.take_string(src.value).encode()) == 0
+            text = _ffi.take_string(src.value)
+            assert n.value == 4 and "poly_row_p3" in text and "c0[it] = poly_vload" in text and "t2[it].v[u] =" in text
+            assert hiplib.poly_hip_compile_check(text.encode()) == 0
+
+
+def test_attention_forms_and_fp32_matmul_render(hiplib):
+    """The attention group renders in its single-pass form by default and in the two-pass
+    form on request; fp32 matmuls of the MLP train step take the fp32 MFMA template."""
+    from polygrad_amd import PlanFile
+    pf = PlanFile(os.path.join(ROOT, "polygrad_amd", "plans", "attention_bf16_b8_h12_t1024_d64.polyplan"))
+    def attention_source():
+        for i in range(hiplib.poly_hip_fused_groups(pf.schedule, -1, None, None)):
+            src = C.c_void_p()
+            hiplib.poly_hip_fused_groups(pf.schedule, i, C.byref(src), None)
+            text = _ffi.take_string(src.value)
+            if "POLY_FA_M" in text:
+                return text
+        raise AssertionError("no attention group")
+    assert "#define POLY_FA_ONLINE 1" in attention_source()
+    os.environ["POLY_HIP_EXACT_ATTENTION"] = "1"
+    try:
+        exact = attention_source()
+    finally:
+        del os.environ["POLY_HIP_EXACT_ATTENTION"]
+    assert "#define POLY_FA_ONLINE 0" in exact and hiplib.poly_hip_compile_check(exact.encode()) == 0
+    mlp = PlanFile(os.path.join(ROOT, "polygrad_amd", "plans", "mlp_train_f32_b4096.polyplan"))
+    s = C.cast(mlp.schedule, C.POINTER(_ffi.PolySchedule)).contents
+    descs = [_ffi.take_string(hiplib.poly_hip_describe(s.items[k].root, 0)) for k in range(s.n_items)]
+    f32 = [d for d in descs if "mfma 32x32x2 f32" in d]
+    assert len(f32) == 2 and any("M=4096 N=512 K=784" in d for d in f32) and any("M=512 N=784 K=4096" in d for d in f32), descs
+    for k in range(s.n_items):
+        if "mfma 32x32x2 f32" in descs[k]:
+            src = _ffi.take_string(hiplib.poly_hip_render(s.items[k].root, b"k", 0, None))
+            assert "__builtin_amdgcn_mfma_f32_32x32x2f32" in src and hiplib.poly_hip_compile_check(src.encode()) == 0
