@@ -1505,6 +1505,87 @@ static bool match_attention(const Sched &sc, int s_item, const std::vector<char>
     score = strf("%s(%s, m, n, z, %s)", fn.c_str(), score.c_str(), call_args(m.item).c_str());
   }
   cfg += strf("#define POLY_FA_SCORE(acc, m, n, z) %s\n", score.c_str());
+  // An additive mask: the stored score is cast(f(acc) + mask[...]) with f made of casts
+  // and products with positive constants, and the mask a bf16 buffer read at consecutive
+  // positions for consecutive keys.  The kernel then loads the mask entries of a tile
+  // itself (POLY_FA_MASK_PTR), gets the chain with the entry as an argument
+  // (POLY_FA_SCORE_MASK) and the value of f alone (POLY_FA_SCORE_NOMASK), and treats tiles
+  // whose entries are all one value specially: all zero, the score is f(acc) itself
+  // (f(acc) is a 16-bit value, adding zero and rounding again change nothing); all one
+  // other value, the score is a non-decreasing function of acc alone, so the score of the
+  // tile's largest product bounds them all.
+  if (online && tin == DT_BF16 && !getenv("POLY_HIP_NO_MASK_PATHS") && mS.nd_full.size() == 1) {
+    const Member &lm = all[n_chain];
+    const KernelGraph &g = sc.graphs[(size_t)lm.item];
+    auto strip = [&](int v) { while (g.n(v).op == POLY_OP_CAST && dt_is_float(g.n(v).dt) && dt_is_float(g.n(g.n(v).src[0]).dt)) v = g.n(v).src[0]; return v; };
+    const int top = strip(n_chain ? g.stores[0].value : stS.value);
+    int mask_ld = -1, other = -1;
+    if (g.n(top).op == POLY_OP_ADD && g.n(top).dt == tin)
+      for (int side = 0; side < 2; side++) {
+        const int cand = g.n(top).src[(size_t)side];
+        if (g.n(cand).op != POLY_OP_LOAD || g.n(cand).dt != tin || lm.preset.count(cand) || g.n(cand).guard >= 0) continue;
+        const KNode &ix = g.n(g.n(cand).src[0]);
+        Aff a;
+        if (ix.src.size() != 2 || g.n(ix.src[1]).lin < 0 || !lin_to_aff(g, g.lins[(size_t)g.n(ix.src[1]).lin], lm.rm, &a)) continue;
+        auto it = a.c.find(mS.nd_full[0].ord);
+        if (it == a.c.end() || it->second != 1) continue;
+        mask_ld = cand;
+        other = g.n(top).src[(size_t)(1 - side)];
+      }
+    // f: from acc (or the chain input x) through casts and products with positive constants
+    std::function<bool(int)> plain = [&](int id) -> bool {
+      const KNode &k = g.n(id);
+      if (n_chain == 0 && id == mS.red) return true;
+      auto pr = lm.preset.find(id);
+      if (pr != lm.preset.end()) return pr->second == "x";
+      if (!dt_is_float(k.dt)) return false;
+      if (k.op == POLY_OP_CAST) return dt_is_float(g.n(k.src[0]).dt) && plain(k.src[0]);
+      if (k.op == POLY_OP_MUL)
+        for (int side = 0; side < 2; side++) {
+          const KNode &c = g.n(k.src[(size_t)side]);
+          if (c.op == POLY_OP_CONST && c.u->arg.kind == POLY_ARG_FLOAT && c.u->arg.f > 0) return plain(k.src[(size_t)(1 - side)]);
+        }
+      return false;
+    };
+    bool ok = mask_ld >= 0 && g.n(other).dt == tin && plain(other);
+    // the members in front of the last one must be monotone in acc as well: only the S epilogue
+    // (a cast) is accepted there
+    if (ok && n_chain > 1) ok = false;
+    if (ok && n_chain == 1) {
+      const KernelGraph &g0 = sc.graphs[(size_t)all[0].item];
+      int v = stS.value;
+      while (g0.n(v).op == POLY_OP_CAST && dt_is_float(g0.n(v).dt)) v = g0.n(v).src[0];
+      ok = v == mS.red;
+    }
+    if (ok) {
+      const size_t before = cfg.size();
+      const bool failed_before = failed;
+      // address of the mask entry
+      {
+        Emitter em(g);
+        Scope S0;
+        S0.indent = 1;
+        for (auto &kv : lm.rm) { em.bind_range(kv.first, strf("r%d", kv.second)); S0.avail |= (uint64_t)1 << kv.first; }
+        const KNode &ix = g.n(g.n(mask_ld).src[0]);
+        const std::string idx = em.emit(ix.src[1], &S0);
+        if (em.failed()) failed = true;
+        cfg += strf("__device__ __forceinline__ const %s* poly_fa_mask_ptr(int m, int n, int z, %s) {\n", tn, params_decl(g).c_str());
+        cfg += master_decomp + S0.code + strf("  return data%d + %s;\n}\n", g.param_slot(ix.src[0]), idx.c_str());
+        cfg += strf("#define POLY_FA_MASK_PTR(m, n, z) poly_fa_mask_ptr(m, n, z, %s)\n", call_args(lm.item).c_str());
+      }
+      const std::string head = n_chain ? strf("poly_fa_s(acc, m, n, z, %s)", call_args(s_item).c_str()) : std::string("acc");
+      const char *lead = n_chain ? "%s x, %s mk" : "float acc, %s mk";
+      std::map<int, std::string> pre_mask{{mask_ld, "mk"}};
+      if (!n_chain) pre_mask[mS.red] = "acc";
+      value_fn(lm, "poly_fa_score_mask", tn, n_chain ? strf(lead, tn, tn).c_str() : strf(lead, tn).c_str(), n_chain ? g.stores[0].value : stS.value, pre_mask);
+      cfg += strf("#define POLY_FA_SCORE_MASK(acc, mk, m, n, z) poly_fa_score_mask(%s, mk, m, n, z, %s)\n", head.c_str(), call_args(lm.item).c_str());
+      std::map<int, std::string> pre_acc;
+      if (!n_chain) pre_acc[mS.red] = "acc";
+      value_fn(lm, "poly_fa_score_nomask", "float", n_chain ? strf("%s x", tn).c_str() : "float acc", other, pre_acc);
+      cfg += strf("#define POLY_FA_SCORE_NOMASK(acc, m, n, z) poly_fa_score_nomask(%s, m, n, z, %s)\n", head.c_str(), call_args(lm.item).c_str());
+      if (failed && !failed_before) { failed = false; cfg.resize(before); }
+    }
+  }
   // Single-pass form when the group is a plain softmax: p = cast(term / sum) with
   // term = exp2((x - max) * c) and the maximum taken over the scores themselves.
   cfg += strf("#define POLY_FA_ONLINE %d\n#define POLY_FA_C %s\n", online ? 1 : 0, Emitter::float_literal(c_sum, DT_F32).c_str());

@@ -40,6 +40,11 @@
 //   POLY_FA_SKIP_DEAD_BLOCKS           1 when p = cast(term(x, mx) / sum): then a key block whose
 //                                      terms are all exactly 0 has probabilities exactly 0
 //   POLY_SIGNATURE
+//   POLY_FA_MASK_PTR(m, n, z), POLY_FA_SCORE_MASK(acc, mk, m, n, z), POLY_FA_SCORE_NOMASK(acc, m, n, z)
+//                                      (optional, online form, bf16) the score is
+//                                      cast(f(acc) + mask) with f non-decreasing: address of
+//                                      the mask entry (consecutive for consecutive n), the
+//                                      score given the entry, and f(acc) as a float
 //   POLY_FA_ONLINE                     1: single pass (needs p = cast(term / sum),
 //                                      term(x, mx) = exp2((x - mx) * POLY_FA_C) and the
 //                                      maximum taken over the scores themselves)
@@ -95,6 +100,7 @@ typedef float fa_acc16 __attribute__((ext_vector_type(16)));
 typedef unsigned int fa_u32x4 __attribute__((ext_vector_type(4)));
 typedef unsigned int fa_u32x2 __attribute__((ext_vector_type(2)));
 typedef fa_u32x4 fa_u32x4_u __attribute__((aligned(2)));
+typedef fa_u32x2 fa_u32x2_u __attribute__((aligned(2)));
 
 #define FA_BM 128        // queries per workgroup: 4 waves x 32
 #define FA_BN 64         // keys per step
@@ -248,14 +254,63 @@ extern "C" __global__ void __launch_bounds__(FA_THREADS) __attribute__((amdgpu_w
       };
 #pragma unroll
       for (int t = 0; t < 2; t++) {
+#ifdef POLY_FA_MASK_PTR
+        // mask entries of this lane's 16 keys: four runs of 4 consecutive keys, 8 bytes each
+        // (issued ahead of the MFMAs)
+        fa_u32x2 mraw[4];
+#pragma unroll
+        for (int gq = 0; gq < 4; gq++) mraw[gq] = *(const fa_u32x2_u *)POLY_FA_MASK_PTR(mq, key_of(kb, t, 4 * gq), z);
+#endif
         fa_acc16 st;
         scores(cur, t, st);
         float x[16];
-        float bm = -__builtin_inff(), nan_probe = 0.0f;
+#ifdef POLY_FA_MASK_PTR
+        // Do all 32 x 32 entries hold one value?  (compared as bit patterns)
+        const unsigned s0 = (unsigned)__builtin_amdgcn_readfirstlane((int)((mraw[0][0] & 0xffffu) * 0x10001u));
+        unsigned diff = 0;
+#pragma unroll
+        for (int gq = 0; gq < 4; gq++) diff |= (mraw[gq][0] ^ s0) | (mraw[gq][1] ^ s0);
+        const bool uniform = __builtin_amdgcn_ballot_w64(diff != 0) == 0;
+        const float cmask = __builtin_bit_cast(float, s0 << 16);
+        auto mask_of = [&](int r) {   // entry of register r as the 16-bit type
+          const unsigned d = mraw[r >> 2][(r >> 1) & 1];
+          return __builtin_bit_cast(POLY_TIN, (unsigned short)((r & 1) ? (d >> 16) : (d & 0xffffu)));
+        };
+        if (uniform && cmask == 0.0f) {
+          // nothing is added: the score is f(acc), already a 16-bit value
+#pragma unroll
+          for (int r = 0; r < 16; r++) x[r] = POLY_FA_SCORE_NOMASK(st[r], mq, key_of(kb, t, r), z);
+        } else {
+          if (uniform) {
+            // One value c is added everywhere: the score of the largest product bounds this
+            // lane's scores.  If even its term is an exact zero against the running maximum
+            // for all 32 queries, the tile adds nothing and moves no maximum.  (A NaN product
+            // goes unseen here: the key it belongs to is masked out for every query of the
+            // tile, and would have made the unfused kernels' rows NaN.)
+            float amax = st[0];
+#pragma unroll
+            for (int r = 1; r < 16; r++) amax = __builtin_fmaxf(amax, st[r]);
+            const int n0 = key_of(kb, t, 0);
+            const float bound = POLY_FA_MAXV(POLY_FA_SCORE_MASK(amax, mask_of(0), mq, n0, z), mq, n0, z);
+            const bool early_dead = __builtin_amdgcn_exp2f((bound - m_run) * c) == 0.0f;
+            if (__builtin_amdgcn_ballot_w64(!early_dead) == 0) continue;
+          }
+#pragma unroll
+          for (int r = 0; r < 16; r++) {
+            const int n = key_of(kb, t, r);
+            x[r] = POLY_FA_MAXV(POLY_FA_SCORE_MASK(st[r], mask_of(r), mq, n, z), mq, n, z);
+          }
+        }
+#else
 #pragma unroll
         for (int r = 0; r < 16; r++) {
           const int n = key_of(kb, t, r);
           x[r] = POLY_FA_MAXV(POLY_FA_SCORE(st[r], mq, n, z), mq, n, z);
+        }
+#endif
+        float bm = -__builtin_inff(), nan_probe = 0.0f;
+#pragma unroll
+        for (int r = 0; r < 16; r++) {
           bm = __builtin_fmaxf(bm, x[r]);     // ignores a NaN ...
           nan_probe = nan_probe + x[r];        // ... which this catches (as does +inf meeting -inf)
         }
