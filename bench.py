@@ -107,8 +107,9 @@ def run_gpu(workload, steps, warmup):
                     algorithmic_bytes=d["bytes"], algorithmic_flops=d["flops"])
     if d["klass"] == "attention-mfma":
         # neither of the two rooflines binds this kernel: say what does
-        roofline["note"] = ("VALU-bound: per score two roundings to bf16 (as the unfused kernels store it), the "
-                            "mask, running maximum, exp2 and the sum; SQ counters under profiles/")
+        roofline["note"] = ("bound by neither roofline: per score two roundings to bf16 (as the unfused kernels store "
+                            "it), the mask, running maximum, exp2 and the sum on the VALU, in a dependent chain between "
+                            "the two MFMAs of a tile at 3 waves per SIMD; SQ counters under profiles/")
 
     classes = {}
     for k, ms in zip(info, per_kernel_ms):
