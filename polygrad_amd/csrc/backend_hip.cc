@@ -94,6 +94,25 @@ HipRunner *runner_from_rendered(const RenderedKernel &rk, const char *fn_name, b
   return r;
 }
 
+int runner_use_variant(HipRunner *r, int idx) {
+  if (!r || idx < 0 || idx >= (int)r->rk.variants.size()) return -1;
+  const RenderedKernel::Variant &v = r->rk.variants[(size_t)idx];
+  RenderedKernel named;
+  named.klass = r->rk.klass;
+  named.source = v.source;
+  named.strategy = v.strategy;
+  name_kernel(&named);
+  Program *p = program_create(named.source, named.entry);
+  if (!p) return -1;
+  program_destroy(r->main);
+  r->main = p;
+  r->rk.source = named.source;
+  r->rk.entry = named.entry;
+  r->rk.strategy = v.strategy;
+  r->rk.launch = v.launch;
+  return 0;
+}
+
 void runner_destroy(HipRunner *r) {
   if (!r) return;
   if (r->main) program_destroy(r->main);
@@ -246,6 +265,7 @@ char *poly_hip_render(PolyUOp *scheduled_root, const char *fn_name, int flags, i
   std::string all = rk.source;
   for (const RenderedKernel::Guard &g : rk.guards) all += "\n// ---- guard ----\n" + g.source;
   if (!rk.fallback_source.empty()) all += "\n// ---- fallback ----\n" + rk.fallback_source;
+  for (size_t i = 1; i < rk.variants.size(); i++) all += "\n// ---- variant " + rk.variants[i].label + "\n" + rk.variants[i].source;
   return dup_string(all);
 }
 

@@ -468,8 +468,10 @@ static bool match_matmul_tail(const Sched &sc, int s_item, const std::vector<cha
   ep.n_params = (int)arg_slots.size();
   if (!render_matmul(mS, ep, &out->rk)) return false;
   out->rk.tables = tables;
-  out->rk.strategy += strf(" + %zu pointwise kernel%s in the epilogue", members.size() - 1, members.size() > 2 ? "s" : "");
-  if (!tables.empty()) out->rk.strategy += strf(" (%zu as a 16-bit lookup table)", tables.size());
+  std::string tail = strf(" + %zu pointwise kernel%s in the epilogue", members.size() - 1, members.size() > 2 ? "s" : "");
+  if (!tables.empty()) tail += strf(" (%zu as a 16-bit lookup table)", tables.size());
+  out->rk.strategy += tail;
+  for (RenderedKernel::Variant &v : out->rk.variants) v.strategy += tail;
   out->items = items;
   out->launch_item = last_item;
   out->internal_slots.assign(internal.begin(), internal.end());

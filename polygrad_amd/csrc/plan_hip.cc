@@ -15,10 +15,13 @@
 //   * kernel groups that fusion.cc recognises run as one launch and their
 //     intermediates get no memory at all.
 #include <hip/hip_runtime.h>
+#include <unistd.h>
 
 #include <algorithm>
+#include <cstdio>
 #include <cstdlib>
 #include <cstring>
+#include <map>
 #include <memory>
 
 #include "fusion.h"
@@ -54,6 +57,7 @@ struct Unit {
   int n_vars = 0;                // DEFINE_VAR arguments of the kernel
   std::vector<const PolyUOp *> var_uops;   // which variable each of them is
   int n_items = 1;               // schedule items this launch stands for
+  bool repeatable = false;       // writes no buffer it also reads: running it twice changes nothing
 };
 
 struct PolyHipPlan {
@@ -69,6 +73,7 @@ struct PolyHipPlan {
   std::vector<PolyVarBinding> merged;
   Program *fill = nullptr;
   bool use_graph = true;
+  bool tuned = false;            // candidates of the tunable kernels have been timed (or there are none)
   std::vector<GraphEntry> graphs;
   uint64_t tick = 0;
   ~PolyHipPlan() {
@@ -199,6 +204,26 @@ PolyHipPlan *poly_hip_compile_schedule(PolyCtx *ctx, const PolySchedule *s) {
       log_err("compile_schedule", "backend 'hip' failed for kernel %d", k);
       return nullptr;
     }
+    // which buffers the launch writes and which it reads (buffers internal to a group are
+    // neither); tuning may only repeat a launch whose two sets are disjoint
+    {
+      std::vector<int> members;
+      if (group_of[(size_t)k] >= 0) members = groups[(size_t)group_of[(size_t)k]].items;
+      else members.push_back(k);
+      std::vector<char> wr((size_t)s->n_buf_slots, 0), rd((size_t)s->n_buf_slots, 0);
+      for (int m : members) {
+        const PolyExecItem &mi = s->items[m];
+        const KernelGraph &g = graphs[(size_t)m];
+        for (size_t p = 0; p < g.params.size() && (int)p < mi.n_buf_slots; p++) {
+          const int sl = mi.buf_slot_indices[p];
+          if (sl < 0 || sl >= s->n_buf_slots || internal[(size_t)sl]) continue;
+          if (g.params[p].written) wr[(size_t)sl] = 1;
+          if (g.params[p].read) rd[(size_t)sl] = 1;
+        }
+      }
+      u.repeatable = true;
+      for (int sl = 0; sl < s->n_buf_slots; sl++) if (wr[(size_t)sl] && rd[(size_t)sl]) u.repeatable = false;
+    }
     plan->units.push_back(u);
   }
   plan_counter++;
@@ -314,10 +339,95 @@ static int bind_args(PolyHipPlan *plan, void **slot_data, int n_slots, const Pol
   return 0;
 }
 
+// ── on-device tuning ──────────────────────────────────────────────────────
+//
+// The reference searches kernel configurations by timing candidates on the machine
+// and keeps the winners on disk (src/codegen.c:1012-1105 times one candidate, :1108-1195
+// is the cache, :1207-1330 the search; enabled by POLY_BEAM, src/render_c.c:839).  Here the
+// candidates are the tile shapes and pipeline depths of the matmul template: with
+// POLY_BEAM > 0 every matmul launch of a plan carries them, and the first run of the plan
+// -- the first moment all its buffers exist -- times each one on the launch's own
+// arguments and keeps the fastest.  Decisions are remembered per process and in the
+// cache directory, keyed by the text of all candidates.
+
+static float time_runner(HipRunner *r, std::vector<void *> &args, hipEvent_t e0, hipEvent_t e1) {
+  hipStream_t stream = (hipStream_t)runtime_stream();
+  if (runner_launch(r, args.data(), (int)args.size()) != 0) return -1.0f;     // warm-up, loads the code
+  if (hipStreamSynchronize(stream) != hipSuccess) return -1.0f;
+  float best = -1.0f;
+  const int reps = 3;
+  for (int round = 0; round < 3; round++) {
+    (void)hipEventRecord(e0, stream);
+    for (int i = 0; i < reps; i++) if (runner_launch(r, args.data(), (int)args.size()) != 0) return -1.0f;
+    (void)hipEventRecord(e1, stream);
+    if (hipStreamSynchronize(stream) != hipSuccess) return -1.0f;
+    float ms = 0;
+    if (hipEventElapsedTime(&ms, e0, e1) != hipSuccess) return -1.0f;
+    ms /= reps;
+    if (best < 0 || ms < best) best = ms;
+  }
+  return best;
+}
+
+static void tune_plan(PolyHipPlan *plan) {
+  plan->tuned = true;
+  static std::map<uint64_t, std::string> decided;   // per process: identical kernels are timed once
+  const std::string dir = runtime_cache_dir();
+  hipEvent_t e0 = nullptr, e1 = nullptr;
+  for (size_t ui = 0; ui < plan->units.size(); ui++) {
+    Unit &u = plan->units[ui];
+    HipRunner *r = u.runner;
+    const std::vector<RenderedKernel::Variant> &vs = r->rk.variants;
+    if (vs.size() < 2 || !u.repeatable || !r->guards.empty()) continue;
+    uint64_t key = 1469598103934665603ull;
+    for (const RenderedKernel::Variant &v : vs) key = fnv1a(v.source.data(), v.source.size(), key);
+    std::string choice;
+    auto it = decided.find(key);
+    if (it != decided.end()) choice = it->second;
+    const std::string path = dir.empty() ? "" : strf("%s/%016llx.tune", dir.c_str(), (unsigned long long)key);
+    if (choice.empty() && !path.empty()) {
+      if (FILE *f = fopen(path.c_str(), "r")) {
+        char buf[64] = {0};
+        if (fscanf(f, "%63s", buf) == 1) choice = buf;
+        fclose(f);
+      }
+    }
+    int pick = -1;
+    for (size_t i = 0; i < vs.size(); i++) if (vs[i].label == choice) pick = (int)i;
+    if (pick < 0) {
+      if (!e0 && (hipEventCreate(&e0) != hipSuccess || hipEventCreate(&e1) != hipSuccess)) break;
+      float best = -1.0f;
+      std::string report;
+      for (size_t i = 0; i < vs.size(); i++) {
+        if (runner_use_variant(r, (int)i) != 0) continue;    // a candidate that does not compile is no candidate
+        const float ms = time_runner(r, plan->kargs[ui], e0, e1);
+        report += strf(" %s=%.4f", vs[i].label.c_str(), ms);
+        if (ms > 0 && (best < 0 || ms < best)) { best = ms; pick = (int)i; }
+      }
+      if (pick < 0) pick = 0;
+      if (getenv("POLY_HIP_DEBUG"))
+        fprintf(stderr, "polygrad: tune: %s -> %s (ms:%s)\n", vs[0].strategy.c_str(), vs[(size_t)pick].label.c_str(), report.c_str());
+      if (!path.empty()) {
+        const std::string tmp = path + strf(".%d.tmp", (int)getpid());
+        if (FILE *f = fopen(tmp.c_str(), "w")) {
+          fprintf(f, "%s\n", vs[(size_t)pick].label.c_str());
+          fclose(f);
+          rename(tmp.c_str(), path.c_str());
+        }
+      }
+    }
+    decided[key] = vs[(size_t)pick].label;
+    if (runner_use_variant(r, pick) != 0) (void)runner_use_variant(r, 0);
+  }
+  if (e0) (void)hipEventDestroy(e0);
+  if (e1) (void)hipEventDestroy(e1);
+}
+
 int poly_hip_plan_run(PolyHipPlan *plan, void **slot_data, int n_slots, const PolyVarBinding *vb, int nvb) {
   if (!plan || !plan->sched) return -1;
   uint64_t key = 0;
   if (bind_args(plan, slot_data, n_slots, vb, nvb, &key) != 0) return -1;
+  if (!plan->tuned) tune_plan(plan);
   hipStream_t stream = (hipStream_t)runtime_stream();
   if (!plan->use_graph || getenv("POLY_HIP_NO_GRAPH")) return enqueue_all(plan);
   plan->tick++;
@@ -376,6 +486,8 @@ int poly_hip_fused_groups(const PolySchedule *s, int index, char **source_out, i
       // the main kernel, then the kernels that fill its tables, as separate translation units
       std::string src = groups[(size_t)index].rk.source;
       for (const RenderedKernel::Table &t : groups[(size_t)index].rk.tables) src += "\n// ---- table " + t.entry + "\n" + t.source;
+      const std::vector<RenderedKernel::Variant> &vs = groups[(size_t)index].rk.variants;
+      for (size_t i = 1; i < vs.size(); i++) src += "\n// ---- variant " + vs[i].label + "\n" + vs[i].source;
       *source_out = (char *)malloc(src.size() + 1);
       if (*source_out) memcpy(*source_out, src.c_str(), src.size() + 1);
     }
@@ -407,6 +519,7 @@ int poly_hip_plan_profile(PolyHipPlan *plan, void **slot_data, int n_slots, floa
   if (!plan) return -1;
   uint64_t key;
   if (bind_args(plan, slot_data, n_slots, nullptr, 0, &key) != 0) return -1;
+  if (!plan->tuned) tune_plan(plan);
   const int n = (int)plan->units.size();
   hipStream_t stream = (hipStream_t)runtime_stream();
   std::vector<hipEvent_t> ev((size_t)n + 1);

@@ -56,6 +56,14 @@ struct RenderedKernel {
   std::vector<Table> tables;
   std::string fallback_source, fallback_entry;
   LaunchSpec fallback_launch;
+  // The same kernel in other configurations (tile shapes): candidates for timing on the
+  // device.  Empty unless tuning is enabled; otherwise variants[0] is `source` itself.
+  // Every variant takes the same arguments and writes the same values.
+  struct Variant {
+    std::string label, source, strategy;
+    LaunchSpec launch;
+  };
+  std::vector<Variant> variants;
 };
 
 struct Scope;

@@ -66,6 +66,8 @@ std::string cache_dir() {
 
 }  // namespace
 
+std::string runtime_cache_dir() { return cache_dir(); }
+
 // hiprtc needs no device, so this also serves compile-only checks.
 bool compile_to_code_object(const std::string &source, std::vector<char> *code, std::string *log) {
   // Compiler options; they are part of the cache key.  Contraction to FMA is off so

@@ -23,6 +23,8 @@ int runtime_sync();
 // `source` with the given launch; identical sources share one buffer.
 std::shared_ptr<void> runtime_table(const std::string &source, const std::string &entry, size_t bytes, const LaunchSpec &ls);
 
+// Directory of the on-disk caches (code objects, tuning decisions); empty when disabled.
+std::string runtime_cache_dir();
 bool compile_to_code_object(const std::string &source, std::vector<char> *code, std::string *log);
 Program *program_create(const std::string &source, const std::string &entry);
 void program_destroy(Program *p);
@@ -47,6 +49,9 @@ HipRunner *runner_create(const PolyUOp *root, const char *fn_name, int flags);
 // placeholder poly_k and gets its descriptive symbol here.
 HipRunner *runner_from_rendered(const RenderedKernel &rk, const char *fn_name, bool named);
 int runner_launch(HipRunner *r, void **args, int n_args);
+// Switches the runner to rk.variants[idx] (compiles it if needed); the runner is unchanged
+// when that fails.
+int runner_use_variant(HipRunner *r, int idx);
 void runner_destroy(HipRunner *r);
 
 }  // namespace polyhip

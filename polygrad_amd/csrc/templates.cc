@@ -415,9 +415,14 @@ static bool render_matmul_f32(const MatmulMatch &mm, const MatmulEpilogue &ep, R
   return true;
 }
 
+bool matmul_tuning_enabled() {
+  const char *e = getenv("POLY_BEAM");
+  return e && atoi(e) > 0;
+}
+
 bool render_matmul(const MatmulMatch &mm, const MatmulEpilogue &ep, RenderedKernel *out) {
   const int64_t K = mm.K, M = mm.M, N = mm.N, Z = mm.Z;
-  const Operand &A = mm.A, &B = mm.B;
+  const Operand &A = mm.A;
   const KSplit &ka = mm.ka, &kb = mm.kb;
   const std::vector<Dim> &md = mm.md, &nd = mm.nd, &zd = mm.zd;
   if (M > 2147483647LL || N > 2147483647LL || Z > 65535) return reject(__LINE__);
@@ -443,7 +448,8 @@ bool render_matmul(const MatmulMatch &mm, const MatmulEpilogue &ep, RenderedKern
   else if (M <= 64) { BM = 64; BN = 256; WVM = 1; WVN = 4; }
   else {
     struct Cand { int bm, bn, wm, wn, per_cu; double thr; };
-    static const Cand cands[] = {{256, 256, 4, 2, 1, 1.00}, {256, 128, 4, 2, 1, 0.84}, {128, 256, 2, 4, 1, 0.84}, {128, 128, 2, 2, 2, 0.80}};
+    // (128x256 before 256x128: equal by the estimate, 1-4 % faster when timed on the device)
+    static const Cand cands[] = {{256, 256, 4, 2, 1, 1.00}, {128, 256, 2, 4, 1, 0.84}, {256, 128, 4, 2, 1, 0.84}, {128, 128, 2, 2, 2, 0.80}};
     double best = 0;
     for (const Cand &c : cands) {
       if (!a_kc && M % 8) continue;
@@ -457,63 +463,81 @@ bool render_matmul(const MatmulMatch &mm, const MatmulEpilogue &ep, RenderedKern
     int a, b2, c2, d2;
     if (sscanf(ov, "%d,%d,%d,%d", &a, &b2, &c2, &d2) == 4) { BM = a; BN = b2; WVM = c2; WVN = d2; }
   }
-  const int64_t tiles = ((M + BM - 1) / BM) * ((N + BN - 1) / BN);
-  if (tiles > 2147483647LL / 2) return reject(__LINE__);
-
-  // ── configuration block ───────────────────────────────────────────────────
-  std::string cfg;
-  cfg += strf("#define POLY_TIN %s\n", dt_cname(A.dt));
-  cfg += strf("#define POLY_MFMA(a, b, c) __builtin_amdgcn_mfma_f32_32x32x16_%s(a, b, c, 0, 0, 0)\n", A.dt == DT_BF16 ? "bf16" : "f16");
-  cfg += strf("#define POLY_M %lld\n#define POLY_N %lld\n#define POLY_K %lld\n#define POLY_Z %lld\n", (long long)M, (long long)N, (long long)K, (long long)Z);
-  cfg += strf("#define POLY_BM %d\n#define POLY_BN %d\n#define POLY_BK %d\n#define POLY_WAVES_M %d\n#define POLY_WAVES_N %d\n", BM, BN, BK, WVM, WVN);
-  cfg += strf("#define POLY_GROUP_M %d\n", BM >= 256 ? 4 : 8);
-  // each XCD (own L2) works on a contiguous run of tiles: let it re-read the smaller operand
-  cfg += strf("#define POLY_GROUP_ALONG_N %d\n", (N > 2 * M && !getenv("POLY_HIP_MM_GROUP_M")) ? 1 : 0);
   // a 256x256 tile holds 128 accumulator registers per lane: no room for the second
   // staging register set of the three-deep pipeline
   int pipe = (BM * BN >= 256 * 256) ? 2 : 3;
   if (const char *e = getenv("POLY_HIP_MM_PIPE")) pipe = atoi(e) == 2 ? 2 : 3;
-  cfg += strf("#define POLY_PIPE %d\n", pipe);
-  cfg += strf("#define POLY_A_KC %d\n#define POLY_B_KC %d\n", a_kc ? 1 : 0, b_kc ? 1 : 0);
-  cfg += strf("#define POLY_A_PTR %s\n#define POLY_B_PTR %s\n", ep.a_ptr.c_str(), ep.b_ptr.c_str());
-  cfg += offset_fn("poly_a_row", md, true, 0);
-  cfg += offset_fn("poly_b_row", nd, false, 0);
-  if (zd.empty()) {
-    cfg += strf("__device__ __forceinline__ int poly_a_z(int) { return %lld; }\n", (long long)mm.a_c0);
-    cfg += strf("__device__ __forceinline__ int poly_b_z(int) { return %lld; }\n", (long long)mm.b_c0);
-  } else {
-    cfg += offset_fn("poly_a_z", zd, true, mm.a_c0);
-    cfg += offset_fn("poly_b_z", zd, false, mm.b_c0);
-  }
-  cfg += matmul_k_fn("poly_a_k", ka, K);
-  cfg += matmul_k_fn("poly_b_k", kb, K);
-  cfg += strf("#define POLY_SIGNATURE %s\n", ep.signature.c_str());
-  cfg += ep.code;
-  if (getenv("POLY_HIP_MM_NOEPI")) cfg += strf("#define POLY_EPILOGUE(acc, m, n, z) do { if (((m) | (n)) == -1) { %s; } } while (0)\n", ep.call.c_str());
-  else
-  cfg += strf("#define POLY_EPILOGUE(acc, m, n, z) %s\n", ep.call.c_str());
-  const bool split = ep.contiguous_n && !getenv("POLY_HIP_MM_NOEPI") && (ep.out_type == "__bf16" || ep.out_type == "_Float16" || ep.out_type == "float");
-  cfg += strf("#define POLY_EP_CONTIG %d\n", split ? 1 : 0);
-  if (split) {
-    cfg += strf("#define POLY_EP_TYPE %s\n", ep.out_type.c_str());
-    cfg += strf("#define POLY_EP_VALUE(acc, m, n, z) %s\n", ep.value_call.c_str());
-    cfg += strf("#define POLY_EP_PTR(m, n, z) %s\n", ep.ptr_call.c_str());
-  }
 
-  *out = RenderedKernel();
-  out->source = std::string(hip_prelude()) + cfg + kMatmulTemplate;
-  out->entry = "poly_k";
-  out->launch.grid[0] = (unsigned)tiles;
-  out->launch.grid[1] = (unsigned)Z;
-  out->launch.block[0] = (unsigned)(64 * WVM * WVN);
-  out->klass = KernelClass::MATMUL_MFMA;
-  out->strategy = strf("mfma 32x32x16 %s M=%lld N=%lld K=%lld Z=%lld tile %dx%dx%d A:%s B:%s", A.dt == DT_BF16 ? "bf16" : "f16",
-                       (long long)M, (long long)N, (long long)K, (long long)Z, BM, BN, BK, a_kc ? "k-major" : "m-major",
-                       b_kc ? "k-major" : "n-major");
-  out->n_params = ep.n_params;
-  out->n_vars = 0;
-  out->flops = 2.0 * (double)M * (double)N * (double)K * (double)Z;
-  out->bytes = ep.bytes;
+  auto emit = [&](int bm, int bn, int wvm, int wvn, int pp, RenderedKernel *rk) {
+    const int64_t tiles = ((M + bm - 1) / bm) * ((N + bn - 1) / bn);
+    if (tiles > 2147483647LL / 2) return reject(__LINE__);
+    // ── configuration block ─────────────────────────────────────────────────
+    std::string cfg;
+    cfg += strf("#define POLY_TIN %s\n", dt_cname(A.dt));
+    cfg += strf("#define POLY_MFMA(a, b, c) __builtin_amdgcn_mfma_f32_32x32x16_%s(a, b, c, 0, 0, 0)\n", A.dt == DT_BF16 ? "bf16" : "f16");
+    cfg += strf("#define POLY_M %lld\n#define POLY_N %lld\n#define POLY_K %lld\n#define POLY_Z %lld\n", (long long)M, (long long)N, (long long)K, (long long)Z);
+    cfg += strf("#define POLY_BM %d\n#define POLY_BN %d\n#define POLY_BK %d\n#define POLY_WAVES_M %d\n#define POLY_WAVES_N %d\n", bm, bn, BK, wvm, wvn);
+    cfg += strf("#define POLY_GROUP_M %d\n", bm >= 256 ? 4 : 8);
+    // each XCD (own L2) works on a contiguous run of tiles: let it re-read the smaller operand
+    cfg += strf("#define POLY_GROUP_ALONG_N %d\n", (N > 2 * M && !getenv("POLY_HIP_MM_GROUP_M")) ? 1 : 0);
+    cfg += strf("#define POLY_PIPE %d\n", pp);
+    cfg += strf("#define POLY_A_KC %d\n#define POLY_B_KC %d\n", a_kc ? 1 : 0, b_kc ? 1 : 0);
+    cfg += strf("#define POLY_A_PTR %s\n#define POLY_B_PTR %s\n", ep.a_ptr.c_str(), ep.b_ptr.c_str());
+    cfg += offset_fn("poly_a_row", md, true, 0);
+    cfg += offset_fn("poly_b_row", nd, false, 0);
+    if (zd.empty()) {
+      cfg += strf("__device__ __forceinline__ int poly_a_z(int) { return %lld; }\n", (long long)mm.a_c0);
+      cfg += strf("__device__ __forceinline__ int poly_b_z(int) { return %lld; }\n", (long long)mm.b_c0);
+    } else {
+      cfg += offset_fn("poly_a_z", zd, true, mm.a_c0);
+      cfg += offset_fn("poly_b_z", zd, false, mm.b_c0);
+    }
+    cfg += matmul_k_fn("poly_a_k", ka, K);
+    cfg += matmul_k_fn("poly_b_k", kb, K);
+    cfg += strf("#define POLY_SIGNATURE %s\n", ep.signature.c_str());
+    cfg += ep.code;
+    if (getenv("POLY_HIP_MM_NOEPI")) cfg += strf("#define POLY_EPILOGUE(acc, m, n, z) do { if (((m) | (n)) == -1) { %s; } } while (0)\n", ep.call.c_str());
+    else
+    cfg += strf("#define POLY_EPILOGUE(acc, m, n, z) %s\n", ep.call.c_str());
+    const bool split = ep.contiguous_n && !getenv("POLY_HIP_MM_NOEPI") && (ep.out_type == "__bf16" || ep.out_type == "_Float16" || ep.out_type == "float");
+    cfg += strf("#define POLY_EP_CONTIG %d\n", split ? 1 : 0);
+    if (split) {
+      cfg += strf("#define POLY_EP_TYPE %s\n", ep.out_type.c_str());
+      cfg += strf("#define POLY_EP_VALUE(acc, m, n, z) %s\n", ep.value_call.c_str());
+      cfg += strf("#define POLY_EP_PTR(m, n, z) %s\n", ep.ptr_call.c_str());
+    }
+
+    *rk = RenderedKernel();
+    rk->source = std::string(hip_prelude()) + cfg + kMatmulTemplate;
+    rk->entry = "poly_k";
+    rk->launch.grid[0] = (unsigned)tiles;
+    rk->launch.grid[1] = (unsigned)Z;
+    rk->launch.block[0] = (unsigned)(64 * wvm * wvn);
+    rk->klass = KernelClass::MATMUL_MFMA;
+    rk->strategy = strf("mfma 32x32x16 %s M=%lld N=%lld K=%lld Z=%lld tile %dx%dx%d A:%s B:%s", A.dt == DT_BF16 ? "bf16" : "f16",
+                        (long long)M, (long long)N, (long long)K, (long long)Z, bm, bn, BK, a_kc ? "k-major" : "m-major",
+                        b_kc ? "k-major" : "n-major");
+    rk->n_params = ep.n_params;
+    rk->n_vars = 0;
+    rk->flops = 2.0 * (double)M * (double)N * (double)K * (double)Z;
+    rk->bytes = ep.bytes;
+    return true;
+  };
+  if (!emit(BM, BN, WVM, WVN, pipe, out)) return false;
+  // Candidates for on-device tuning: the same kernel in the other tile shapes and
+  // pipeline depths; the plan times them on its first run when POLY_BEAM is set.
+  if (matmul_tuning_enabled() && M > 64 && N > 64 && !(!a_kc && M % 8)) {
+    struct Shape { int bm, bn, wm, wn, pp; };
+    static const Shape shapes[] = {{256, 256, 4, 2, 2}, {256, 128, 4, 2, 3}, {256, 128, 4, 2, 2}, {128, 256, 2, 4, 3},
+                                   {128, 256, 2, 4, 2}, {128, 128, 2, 2, 3}, {128, 128, 2, 2, 2}};
+    out->variants.push_back({strf("%dx%dw%dx%dp%d", BM, BN, WVM, WVN, pipe), out->source, out->strategy, out->launch});
+    for (const Shape &c : shapes) {
+      if (c.bm == BM && c.bn == BN && c.wm == WVM && c.wn == WVN && c.pp == pipe) continue;
+      RenderedKernel v;
+      if (emit(c.bm, c.bn, c.wm, c.wn, c.pp, &v))
+        out->variants.push_back({strf("%dx%dw%dx%dp%d", c.bm, c.bn, c.wm, c.wn, c.pp), v.source, v.strategy, v.launch});
+    }
+  }
   return true;
 }
 

@@ -67,7 +67,10 @@ struct MatmulEpilogue {
 // that is not the last of an aligned group of 8?  (store index affine with coefficient 1
 // on the innermost digit of n, digits not crossed inside a group)
 bool matmul_store_contiguous(const KernelGraph &g, const MatmulMatch &mm, const Lin &store_lin);
-// Chooses layouts and tile shape and instantiates kernels/matmul_mfma.hip.
+// Chooses layouts and tile shape and instantiates kernels/matmul_mfma.hip.  With tuning
+// enabled (POLY_BEAM > 0 in the environment, the switch of the reference's own search,
+// src/render_c.c:839) the other tile shapes come along as RenderedKernel::variants.
+bool matmul_tuning_enabled();
 bool render_matmul(const MatmulMatch &mm, const MatmulEpilogue &ep, RenderedKernel *out);
 
 bool try_render_matmul(const KernelGraph &g, const std::string &fn, const RenderOptions &opt, RenderedKernel *out);

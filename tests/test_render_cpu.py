@@ -212,3 +212,25 @@ def test_attention_forms_and_fp32_matmul_render(hiplib):
         if "mfma 32x32x2 f32" in descs[k]:
             src = _ffi.take_string(hiplib.poly_hip_render(s.items[k].root, b"k", 0, None))
             assert "__builtin_amdgcn_mfma_f32_32x32x2f32" in src and hiplib.poly_hip_compile_check(src.encode()) == 0
+
+
+def test_tuning_candidates_render_and_compile(hiplib):
+    """With POLY_BEAM set (the switch of the reference's own search, src/render_c.c:839) a
+    16-bit matmul comes with its other tile shapes as candidates, and every one compiles;
+    without it there are none."""
+    from polygrad_amd import PlanFile
+    pf = PlanFile(os.path.join(ROOT, "polygrad_amd", "plans", "matmul_bf16_8192x768x3072.polyplan"))
+    s = C.cast(pf.schedule, C.POINTER(_ffi.PolySchedule)).contents
+    plain = _ffi.take_string(hiplib.poly_hip_render(s.items[0].root, b"k", 0, None))
+    assert "// ---- variant" not in plain
+    os.environ["POLY_BEAM"] = "2"
+    try:
+        tuned = _ffi.take_string(hiplib.poly_hip_render(s.items[0].root, b"k", 0, None))
+    finally:
+        del os.environ["POLY_BEAM"]
+    labels = re.findall(r"// ---- variant (\S+)", tuned)
+    assert len(labels) == 6 and len(set(labels)) == 6, labels
+    assert tuned.startswith(plain)          # the default choice stays the kernel itself
+    shapes = set(re.findall(r"#define POLY_BM (\d+)\n#define POLY_BN (\d+)", tuned))
+    assert shapes == {("256", "256"), ("256", "128"), ("128", "256"), ("128", "128")}, shapes
+    assert hiplib.poly_hip_compile_check(tuned.encode()) == 0
