@@ -109,9 +109,10 @@ PolyHipPlan *poly_hip_compile_schedule(PolyCtx *ctx, const PolySchedule *schedul
  * intermediates).  Returns after enqueueing; poly_hip_sync() waits.
  * With POLY_BEAM > 0 in the environment at compile and run time (the switch of
  * the reference's kernel search, src/render_c.c:839; its timing loop and disk
- * cache are src/codegen.c:1012-1195), the first run times every matmul launch
- * in each tile shape of the template on the launch's own buffers, keeps the
- * fastest and records the decision in the cache directory. */
+ * cache are src/codegen.c:1012-1195), the first run goes through the launches
+ * in order and times every matmul in each tile shape of the template, on its
+ * own buffers once they hold their real values; it keeps the fastest and
+ * records the decision in the cache directory. */
 int poly_hip_plan_run(PolyHipPlan *plan, void **slot_data, int n_slots,
                       const PolyVarBinding *var_bindings, int n_var_bindings);
 void poly_hip_plan_free(PolyHipPlan *plan);
