@@ -56,7 +56,7 @@ def random_slot_tensors(plan, seed=0, device="cuda", scale=1.0, outputs=()):
         dt = torch_dtype(s.dtype)
         if s.name in outputs:
             t = torch.zeros(s.numel, dtype=dt, device=device)
-        elif s.name in ("positions", "arange", "vocab_arange"):
+        elif s.name in ("positions", "arange", "vocab_arange") or s.name.startswith("__arange_"):
             t = torch.arange(s.numel, device=device).to(dt)
         elif dt.is_floating_point:
             t = ((torch.rand(s.numel, generator=g, device=device, dtype=torch.float32) * 2 - 1) * scale).to(dt)

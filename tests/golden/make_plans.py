@@ -26,7 +26,7 @@ sys.path.insert(0, os.path.join(ROOT, "tests"))
 
 import graphs  # noqa: E402
 import refpoly as R  # noqa: E402
-from hipharness import schedule_slots  # noqa: E402
+from hipharness import constant_name, constant_slots, schedule_slots  # noqa: E402
 from polygrad_amd import save_schedule  # noqa: E402
 
 OUT = os.path.join(ROOT, "polygrad_amd", "plans")
@@ -36,8 +36,9 @@ def save(c, sink, name):
     sched = c.schedule(sink)
     slots, n = schedule_slots(c, sched)
     names = [None] * n
+    consts = constant_slots(c, sched)
     for i, tn in slots.items():
-        names[i] = tn[1]
+        names[i] = tn[1] if tn is not None else constant_name(consts[i])
     path = os.path.join(OUT, name + ".polyplan")
     save_schedule(sched, names, path)
     c.L.poly_schedule_free(sched)

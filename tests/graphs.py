@@ -287,3 +287,97 @@ def adamw_step(c, numel, lr=3e-4, beta1=0.9, beta2=0.999, eps=1e-8, weight_decay
     p_new = p_cur - c.const(lr) * (m_hat * denom.un("RECIPROCAL"))
     bufs = dict(p=p, g=g, m=m, v=v, bc1=bc1, bc2=bc2)
     return bufs, c.sink_assign((p, p_new), (m, m_new), (v, v_new))
+
+
+BLOCK_PARAMS = ("ln1_w", "ln1_b", "attn_w", "attn_b", "proj_w", "proj_b", "ln2_w", "ln2_b", "fc_w", "fc_b", "fc2_w", "fc2_b",
+                "lnf_w", "lnf_b", "head_w")
+
+
+def gpt2_block_train_step(c, batch=4, ctx=1024, d_model=1024, heads=16, vocab=50257, lr=3e-4, beta1=0.9, beta2=0.999,
+                          eps=1e-8, weight_decay=0.1, ln_eps=1e-5):
+    """One transformer block of config 5 (GPT-2 medium shapes) with the final LayerNorm,
+    the vocabulary projection and next-token cross-entropy, reverse-mode gradients from the
+    reference's poly_grad (src/autograd.c:773) and an AdamW update of every parameter
+    (src/instance.c:1162-1224).  Mixed precision: fp32 master parameters and optimizer
+    state, bf16 copies of the weights and bf16 activations for the matmuls, fp32
+    reductions.  The block's input activations stand in for the layers below it.
+    Returns (bufs, sink): the sink stores the loss and updates p, m, v of all 15 parameters."""
+    B, T, D, H, V = batch, ctx, d_model, heads, vocab
+    hd = D // H
+    shapes = dict(ln1_w=(D,), ln1_b=(D,), attn_w=(D, 3 * D), attn_b=(3 * D,), proj_w=(D, D), proj_b=(D,), ln2_w=(D,),
+                  ln2_b=(D,), fc_w=(D, 4 * D), fc_b=(4 * D,), fc2_w=(4 * D, D), fc2_b=(D,), lnf_w=(D,), lnf_b=(D,),
+                  head_w=(D, V))
+    bufs = {}
+    P = {}
+    for name in BLOCK_PARAMS:
+        P[name] = bufs[name] = c.buffer(shapes[name], R.F32, name=name)
+        bufs[name + ".m"] = c.buffer(shapes[name], R.F32, name=name + ".m")
+        bufs[name + ".v"] = c.buffer(shapes[name], R.F32, name=name + ".v")
+    h0 = bufs["h0"] = c.buffer((B, T, D), R.BF16, name="h0")
+    target = bufs["target"] = c.buffer((B * T,), R.F32, name="target")     # class ids as floats (sparse cross-entropy)
+    arange = bufs["arange"] = c.buffer((T,), R.F32, name="arange")
+    bc1, bc2 = c.buffer((1,), name="bc1"), c.buffer((1,), name="bc2")
+    bufs["bc1"], bufs["bc2"] = bc1, bc2
+    loss_out = bufs["loss"] = c.buffer((1,), R.F32, name="loss")
+    W = {k: v.cast(R.BF16).contiguous() for k, v in P.items()}             # bf16 working copies, one cast kernel each
+
+    row = arange.reshape((T, 1)).expand((T, T))
+    col = arange.reshape((1, T)).expand((T, T))
+    mask = row.lt(col).where(c.const(-1e9, R.BF16), c.const(0.0, R.BF16)).reshape((1, 1, T, T)).contiguous()
+    wdt = R.BF16
+    ln1 = _layernorm(h0, W["ln1_w"], W["ln1_b"], ln_eps, wdt).contiguous()
+    qkv = _linear(ln1, W["attn_w"], W["attn_b"], wdt).contiguous()
+    q = qkv.shrink(((0, B), (0, T), (0, D))).contiguous().reshape((B, T, H, hd)).permute((0, 2, 1, 3))
+    k = qkv.shrink(((0, B), (0, T), (D, 2 * D))).contiguous().reshape((B, T, H, hd)).permute((0, 2, 1, 3))
+    v = qkv.shrink(((0, B), (0, T), (2 * D, 3 * D))).contiguous().reshape((B, T, H, hd)).permute((0, 2, 1, 3))
+    scores = q.cast(R.F32).dot(k.permute((0, 1, 3, 2)).cast(R.F32)).cast(wdt).contiguous()
+    scores = (scores * c.const(1.0 / math.sqrt(hd), wdt) + mask.expand((B, H, T, T))).contiguous()
+    attn = scores.cast(R.F32).softmax(-1).cast(wdt).contiguous()
+    ctxv = attn.cast(R.F32).dot(v.cast(R.F32)).cast(wdt).contiguous()
+    merged = ctxv.permute((0, 2, 1, 3)).reshape((B, T, D))
+    h1 = (h0 + _linear(merged, W["proj_w"], W["proj_b"], wdt).contiguous()).contiguous()
+    ln2 = _layernorm(h1, W["ln2_w"], W["ln2_b"], ln_eps, wdt).contiguous()
+    ff = _linear(ln2, W["fc_w"], W["fc_b"], wdt).contiguous().gelu().contiguous()
+    h2 = (h1 + _linear(ff, W["fc2_w"], W["fc2_b"], wdt).contiguous()).contiguous()
+    lnf = _layernorm(h2, W["lnf_w"], W["lnf_b"], ln_eps, wdt).contiguous()
+    logits = lnf.reshape((B * T, D)).cast(R.F32).dot(W["head_w"].cast(R.F32)).contiguous()   # fp32 logits
+    loss = logits.cross_entropy(target)
+    assigns = []
+    for name in BLOCK_PARAMS:
+        p, m, vv = P[name], bufs[name + ".m"], bufs[name + ".v"]
+        n = int(np.prod(p.shape))
+        g = T_grad(c, loss, p, n)
+        pf, mf, vf = p.reshape((n,)), m.reshape((n,)), vv.reshape((n,))
+        m_new = c.const(beta1) * mf + c.const(1.0 - beta1) * g
+        v_new = c.const(beta2) * vf + c.const(1.0 - beta2) * (g * g)
+        denom = (v_new * bc2.expand((n,))).sqrt() + c.const(eps)
+        p_new = pf * c.const(1.0 - lr * weight_decay) - c.const(lr) * ((m_new * bc1.expand((n,))) * denom.un("RECIPROCAL"))
+        assigns += [(p, p_new), (m, m_new), (vv, v_new)]
+    return bufs, c.sink_mixed([(loss_out, loss.reshape((1,)))], assigns)
+
+
+def gpt2_block_train_inputs(bufs, batch, ctx, vocab, seed=4):
+    """Seeded inputs for gpt2_block_train_step: weights ~ N(0, 0.02), LayerNorm weights 1,
+    biases 0, optimizer state 0, activations ~ N(0, 1) as bf16, uniform random targets."""
+    g = np.random.default_rng(seed)
+    arrays = {}
+    for name, t in bufs.items():
+        n = int(np.prod(t.shape))
+        if name == "h0":
+            a = R.f32_to_bf16_bits(g.normal(0.0, 1.0, n).astype(np.float32))
+        elif name == "target":
+            a = g.integers(0, vocab, n).astype(np.float32)
+        elif name == "arange":
+            a = np.arange(ctx, dtype=np.float32)
+        elif name == "bc1":
+            a = np.array([1.0 / (1.0 - 0.9)], np.float32)
+        elif name == "bc2":
+            a = np.array([1.0 / (1.0 - 0.999)], np.float32)
+        elif name.endswith(".m") or name.endswith(".v") or name == "loss" or name.endswith("_b"):
+            a = np.zeros(n, np.float32)
+        elif name in ("ln1_w", "ln2_w", "lnf_w"):
+            a = np.ones(n, np.float32)
+        else:
+            a = g.normal(0.0, 0.02, n).astype(np.float32)
+        arrays[t] = a
+    return arrays

@@ -51,6 +51,33 @@ def schedule_slots(c, sched):
     return out, s.n_buf_slots
 
 
+def constant_slots(c, sched):
+    """External slots that are not caller buffers but constants the reference frontend
+    created itself (poly_arange inside poly_cross_entropy, src/frontend.c:1213, registered
+    at :253): slot index -> float32 array, read through poly_const_buffer_data
+    (src/frontend.h:156), which is how poly_realize fills them (src/frontend.c:2232)."""
+    s = C.cast(sched, C.POINTER(_ffi.PolySchedule)).contents
+    known = {t.buf for t, _ in c.buffers}
+    out = {}
+    for i in range(s.n_buf_slots):
+        sl = s.buf_slots[i]
+        if sl.is_intermediate or sl.buf_uop in known:
+            continue
+        p = c.L.poly_const_buffer_data(c.ctx, sl.buf_uop)
+        if p:
+            assert sl.nbytes == 4 * sl.numel, "registry constants are float32"
+            out[i] = np.ctypeslib.as_array(C.cast(p, C.POINTER(C.c_float)), shape=(int(sl.numel),)).copy()
+    return out
+
+
+def constant_name(a):
+    """Plan files carry no data: a registry constant is stored by a name that says how to
+    rebuild it (only aranges occur)."""
+    if np.array_equal(a, np.arange(a.size, dtype=np.float32)):
+        return f"__arange_{a.size}"
+    raise RuntimeError("registry constant that is not an arange")
+
+
 def run_hip(c, sink, arrays, graph=True, repeats=1):
     """Runs `sink` on the GPU through the plan-level C ABI.  arrays: {buffer T: ndarray}
     (inputs and outputs).  Returns {buffer T: ndarray} with device contents after the run."""
@@ -61,10 +88,16 @@ def run_hip(c, sink, arrays, graph=True, repeats=1):
     for i, tn in slots.items():
         if tn is not None:
             names[i] = tn[1]
+    consts = constant_slots(c, sched)
+    for i, a in consts.items():
+        names[i] = constant_name(a)
     plan = HipPlan(sched, ctx=c.ctx, names=names)
     dev = [None] * n
     owner = {}
     for i, tn in slots.items():
+        if tn is None and i in consts:
+            dev[i] = to_device(consts[i])
+            continue
         if tn is None:
             raise RuntimeError(f"external slot {i} has no known buffer")
         t = tn[0]

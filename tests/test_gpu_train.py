@@ -77,3 +77,42 @@ def test_adamw_update_matches_reference():
         assert not np.array_equal(want[t], arrays[t]), f"{name} did not change"
         assert_close(got[t], want[t], rtol=1e-5, atol=1e-9, what=f"AdamW {name}")
     assert got[bufs["g"]].tobytes() == arrays[bufs["g"]].tobytes()
+
+
+def test_gpt2_block_train_step_matches_reference():
+    """Benchmark configuration 5 at a reduced size: one transformer block, final LayerNorm,
+    vocabulary projection, next-token cross-entropy (sparse targets), reverse-mode
+    gradients from the reference's poly_grad and AdamW on all 15 parameters -- about 150
+    scheduled kernels with the backward forms of matmul, softmax, LayerNorm and GELU,
+    bf16 activations with fp32 master parameters.  The first moments after one step from
+    zero state are 0.1 x gradient, so they carry the gradient comparison."""
+    B, T, D, H, V = 1, 32, 64, 2, 97
+    lr = 3e-4
+    c = R.Ctx()
+    bufs, sink = graphs.gpt2_block_train_step(c, B, T, D, H, V, lr=lr)
+    arrays = graphs.gpt2_block_train_inputs(bufs, B, T, V)
+    want = run_ref(c, sink, arrays)
+    got, info = run_hip(c, sink, arrays)
+    c.close()
+    assert len(info) >= 100
+    assert_close(got[bufs["loss"]], want[bufs["loss"]], rtol=1e-4, what="loss")
+    assert abs(float(want[bufs["loss"]][0]) - np.log(V)) < 0.05       # random init: loss is ln(vocab)
+    for name in graphs.BLOCK_PARAMS:
+        m_ref, m_got = want[bufs[name + ".m"]], got[bufs[name + ".m"]]
+        scale = float(np.abs(m_ref).max())
+        assert scale > 0, f"no gradient reached {name}"
+        # gradients pass through bf16 activations: 2e-2 of the tensor's scale per element,
+        # and far less on average (different accumulation orders, same roundings)
+        assert_close(m_got, m_ref, rtol=2e-2, atol=2e-2 * scale, what=f"first moment of {name}")
+        assert float(np.abs(m_got - m_ref).mean()) <= 2e-3 * scale, name
+        v_ref, v_got = want[bufs[name + ".v"]], got[bufs[name + ".v"]]
+        assert_close(v_got, v_ref, rtol=4e-2, atol=4e-2 * float(np.abs(v_ref).max()), what=f"second moment of {name}")
+        # the first AdamW step moves every element by about lr * sign(g): where the
+        # gradients agree in sign the parameters agree closely, and nowhere by more than 2 lr
+        p0, p_ref, p_got = arrays[bufs[name]], want[bufs[name]], got[bufs[name]]
+        assert np.abs(p_ref - p0).max() > 0.5 * lr * 0.9
+        assert np.abs(p_got - p_ref).max() <= 2.2 * lr
+        same = np.sign(m_ref) == np.sign(m_got)
+        big = np.abs(m_ref) > 0.05 * scale
+        assert same[big].all(), name
+        assert_close(p_got[big], p_ref[big], rtol=0, atol=0.2 * lr, what=f"updated {name} where the gradient is not small")
