@@ -53,13 +53,16 @@ def kernel_key(desc):
 def run_gpu(workload, steps, warmup):
     import torch
     from polygrad_amd import HipPlan
-    from polygrad_amd.inputs import gpt2_slot_tensors, random_slot_tensors
+    from polygrad_amd.inputs import block_train_slot_tensors, gpt2_slot_tensors, random_slot_tensors
 
     path = os.path.join(ROOT, "polygrad_amd", "plans", workload + ".polyplan")
     t0 = time.perf_counter()
     plan = HipPlan.from_file(path)
     compile_s = time.perf_counter() - t0
-    if workload.startswith("gpt2"):
+    if workload.startswith("gpt2_medium_block_train"):
+        data, _ = block_train_slot_tensors(plan)
+        tokens = None
+    elif workload.startswith("gpt2"):
         data, _ = gpt2_slot_tensors(plan)
         tokens = [s for s in plan.slots if s.name == "x"][0].numel
     else:
@@ -195,7 +198,7 @@ def main():
 
     ms, tokens, roofline, extra = run_gpu(args.workload, args.steps, args.warmup)
     cpu = None
-    if not args.no_cpu_baseline and args.workload.startswith("gpt2"):
+    if not args.no_cpu_baseline and args.workload == GPT2_PLAN:
         try:
             cpu = cpu_baseline_reference() or cpu_baseline_port()
         except Exception as e:  # the baseline is reported, never required

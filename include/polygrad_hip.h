@@ -126,6 +126,12 @@ void poly_hip_plan_free(PolyHipPlan *plan);
  * starting with "// ---- ".
  * No reference counterpart: the reference launches every scheduled kernel. */
 int poly_hip_fused_groups(const PolySchedule *schedule, int index, char **source_out, int *n_items_out);
+/* How group `index` is launched, for checking its indexing away from the GPU: the
+ * buffer slot of each kernel argument in order (at most cap entries written to
+ * slots_out; tables and flags the kernel takes after them are not listed) and
+ * launch_out[0..3] = grid x, y, z and workgroup size.  Returns the number of buffer
+ * arguments, <0 on error.  No reference counterpart. */
+int poly_hip_fused_group_launch(const PolySchedule *schedule, int index, int *slots_out, int cap, int *launch_out);
 /* Introspection for benches and tests. */
 int poly_hip_plan_n_kernels(const PolyHipPlan *plan);
 /* Fills at most cap entries; per kernel (in execution order): class id

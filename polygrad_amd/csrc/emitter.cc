@@ -185,8 +185,20 @@ std::string Emitter::emit_atom(int atom, Scope *s) {
       if (f != t->atom_names.end()) return f->second;
       std::string inner = emit_lin(a.inner, t);
       std::string name = strf("q%d", atom);
-      stmt(t, strf("const int %s = (%s)%s%lld;", name.c_str(), inner.c_str(),
-                   a.kind == Atom::DIV ? "/" : "%", (long long)a.c));
+      int64_t lo = 0, hi = 0;
+      g_.lin_bounds(a.inner, &lo, &hi);
+      if (a.kind == Atom::MOD && lo < 0) {
+        // The dividend can be negative only where the value is not used (positions a pad
+        // or shrink masks out: `where(valid, x[...], 0)` still evaluates the index).  The
+        // reference's CPU code takes a power-of-two modulus as a bit mask there
+        // (src/codegen.c:1675-1748), which keeps such an index inside the buffer; C's %
+        // would make it negative.  Floor modulus does the same for every divisor.
+        if ((a.c & (a.c - 1)) == 0) stmt(t, strf("const int %s = (%s)&%lld;", name.c_str(), inner.c_str(), (long long)(a.c - 1)));
+        else stmt(t, strf("const int %s = (((%s)%%%lld)+%lld)%%%lld;", name.c_str(), inner.c_str(), (long long)a.c, (long long)a.c, (long long)a.c));
+      } else {
+        stmt(t, strf("const int %s = (%s)%s%lld;", name.c_str(), inner.c_str(),
+                     a.kind == Atom::DIV ? "/" : "%", (long long)a.c));
+      }
       t->atom_names[atom] = name;
       return name;
     }

@@ -11,6 +11,16 @@
 //                       written to LDS as four single floats)
 //   POLY_A_PTR/B_PTR, poly_a_row(m), poly_b_row(n), poly_a_z(z), poly_b_z(z), poly_a_k(k), poly_b_k(k)
 //   POLY_SIGNATURE, POLY_EPILOGUE(acc, m, n, z)
+//   POLY_GEN            1: the operands are expressions, not arrays.  Then instead of the
+//                       pointer/offset items above:
+//                         POLY_A_NLOADS, POLY_A_LOAD(m, k, z, raw)  fetches what element
+//                           A(z,m,k) is computed from into `unsigned int raw[POLY_A_NLOADS]`
+//                         POLY_A_MATH(m, k, z, raw)  the element as a float
+//                       (same for B with n), K may be any size (elements past K are 0), and
+//                       POLY_A_KC/B_KC only choose which way consecutive threads walk.
+//                       Fetches run ahead in the register ring like the plain loads; the
+//                       arithmetic happens on the way to LDS.
+//   POLY_PF_DEPTH       K tiles the global loads run ahead (default 4)
 //
 // Data path: global --16B loads, four K tiles ahead--> registers --> LDS [row][16 k]
 // (rows padded to 20 floats: 16-byte fragment reads of 16 consecutive rows then fall on
@@ -54,7 +64,13 @@ typedef float pf_acc16 __attribute__((ext_vector_type(16)));
 #define PF_TM (PF_WM / 32)
 #define PF_TN (PF_WN / 32)
 #define PF_NTHREADS (64 * POLY_WAVES_M * POLY_WAVES_N)
-#define PF_KT (POLY_K / PF_BK)
+#ifndef POLY_GEN
+#define POLY_GEN 0
+#endif
+#ifndef POLY_PF_DEPTH
+#define POLY_PF_DEPTH 4
+#endif
+#define PF_KT ((POLY_K + PF_BK - 1) / PF_BK)
 
 // Staging of one operand tile (ROWS x 16 floats): 16-byte pieces, ROWS * 4 of them.
 template <int ROWS, bool KC>
@@ -86,6 +102,11 @@ struct PfStage {
   }
 };
 
+#if POLY_GEN
+#define PF_A_NRAW POLY_A_NLOADS
+#define PF_B_NRAW POLY_B_NLOADS
+#endif
+
 extern "C" __global__ void __launch_bounds__(PF_NTHREADS) poly_k(POLY_SIGNATURE) {
   __shared__ __attribute__((aligned(16))) float lds_a[2][POLY_BM * PF_LDK];
   __shared__ __attribute__((aligned(16))) float lds_b[2][POLY_BN * PF_LDK];
@@ -113,14 +134,79 @@ extern "C" __global__ void __launch_bounds__(PF_NTHREADS) poly_k(POLY_SIGNATURE)
   }
   const int z = blockIdx.y;
   const int m0 = tile_m * POLY_BM, n0 = tile_n * POLY_BN;
-  const float *__restrict__ gA = POLY_A_PTR + poly_a_z(z);
-  const float *__restrict__ gB = POLY_B_PTR + poly_b_z(z);
-
   typedef PfStage<POLY_BM, POLY_A_KC != 0> StageA;
   typedef PfStage<POLY_BN, POLY_B_KC != 0> StageB;
   // Global loads run PF_DEPTH K tiles ahead of the math, in a ring of register sets (tile t
   // in set t % PF_DEPTH): with one small workgroup per CU nothing else hides their latency.
-  constexpr int PF_DEPTH = 4;
+  constexpr int PF_DEPTH = POLY_PF_DEPTH;
+#if POLY_GEN
+  // element e of piece i: (row + e, k) for row-walking pieces, (row, k + e) for k-walking
+  // ones; rows past the edge are clamped (computed, never stored), k past the end gives 0
+  unsigned int ra[PF_DEPTH][StageA::NL][4][PF_A_NRAW], rb[PF_DEPTH][StageB::NL][4][PF_B_NRAW];
+  auto a_coord = [&](int kt, int i, int e, int *m, int *k) {
+    const int row = m0 + StageA::row_of(i) + (POLY_A_KC ? 0 : e);
+    *m = row < POLY_M ? row : POLY_M - 1;
+    *k = kt * PF_BK + StageA::k_of(i) + (POLY_A_KC ? e : 0);
+  };
+  auto b_coord = [&](int kt, int i, int e, int *n, int *k) {
+    const int row = n0 + StageB::row_of(i) + (POLY_B_KC ? 0 : e);
+    *n = row < POLY_N ? row : POLY_N - 1;
+    *k = kt * PF_BK + StageB::k_of(i) + (POLY_B_KC ? e : 0);
+  };
+  auto load_tiles = [&](int kt, int set) {
+#pragma unroll
+    for (int i = 0; i < StageA::NL; i++)
+      if (StageA::active(i)) {
+#pragma unroll
+        for (int e = 0; e < 4; e++) {
+          int m, k;
+          a_coord(kt, i, e, &m, &k);
+#pragma unroll
+          for (int j = 0; j < PF_A_NRAW; j++) ra[set][i][e][j] = 0u;
+          if (POLY_K % PF_BK == 0 || k < POLY_K) { POLY_A_LOAD(m, k, z, ra[set][i][e]); }
+        }
+      }
+#pragma unroll
+    for (int i = 0; i < StageB::NL; i++)
+      if (StageB::active(i)) {
+#pragma unroll
+        for (int e = 0; e < 4; e++) {
+          int n, k;
+          b_coord(kt, i, e, &n, &k);
+#pragma unroll
+          for (int j = 0; j < PF_B_NRAW; j++) rb[set][i][e][j] = 0u;
+          if (POLY_K % PF_BK == 0 || k < POLY_K) { POLY_B_LOAD(n, k, z, rb[set][i][e]); }
+        }
+      }
+  };
+  auto store_tiles = [&](int kt, int set, int buf) {
+    pf_f32x4 va[StageA::NL], vb[StageB::NL];
+#pragma unroll
+    for (int i = 0; i < StageA::NL; i++)
+      if (StageA::active(i)) {
+#pragma unroll
+        for (int e = 0; e < 4; e++) {
+          int m, k;
+          a_coord(kt, i, e, &m, &k);
+          va[i][e] = (POLY_K % PF_BK == 0 || k < POLY_K) ? POLY_A_MATH(m, k, z, ra[set][i][e]) : 0.0f;
+        }
+      }
+#pragma unroll
+    for (int i = 0; i < StageB::NL; i++)
+      if (StageB::active(i)) {
+#pragma unroll
+        for (int e = 0; e < 4; e++) {
+          int n, k;
+          b_coord(kt, i, e, &n, &k);
+          vb[i][e] = (POLY_K % PF_BK == 0 || k < POLY_K) ? POLY_B_MATH(n, k, z, rb[set][i][e]) : 0.0f;
+        }
+      }
+    StageA::store(lds_a[buf], va);
+    StageB::store(lds_b[buf], vb);
+  };
+#else
+  const float *__restrict__ gA = POLY_A_PTR + poly_a_z(z);
+  const float *__restrict__ gB = POLY_B_PTR + poly_b_z(z);
   pf_f32x4 ra[PF_DEPTH][StageA::NL], rb[PF_DEPTH][StageB::NL];
   // Per-thread global offsets of the rows this thread stages.  Rows past the edge are
   // clamped to the last valid row (or row group): loaded and multiplied, never stored.
@@ -144,6 +230,12 @@ extern "C" __global__ void __launch_bounds__(PF_NTHREADS) poly_k(POLY_SIGNATURE)
     for (int i = 0; i < StageB::NL; i++)
       if (StageB::active(i)) rb[set][i] = *(const pf_f32x4_u *)(gB + b_off[i] + poly_b_k(k0 + StageB::k_of(i)));
   };
+  auto store_tiles = [&](int kt, int set, int buf) {
+    (void)kt;
+    StageA::store(lds_a[buf], ra[set]);
+    StageB::store(lds_b[buf], rb[set]);
+  };
+#endif
 
   const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63, half = lane >> 5;
   const int wm = (wave % POLY_WAVES_M) * PF_WM, wn = (wave / POLY_WAVES_M) * PF_WN;
@@ -158,8 +250,7 @@ extern "C" __global__ void __launch_bounds__(PF_NTHREADS) poly_k(POLY_SIGNATURE)
 #pragma unroll
   for (int d = 0; d < PF_DEPTH; d++)
     if (d < PF_KT) load_tiles(d, d);
-  StageA::store(lds_a[0], ra[0]);
-  StageB::store(lds_b[0], rb[0]);
+  store_tiles(0, 0, 0);
   if (PF_DEPTH < PF_KT) load_tiles(PF_DEPTH, 0);
   __syncthreads();
   for (int kt0 = 0; kt0 < PF_KT; kt0 += PF_DEPTH) {
@@ -186,8 +277,7 @@ extern "C" __global__ void __launch_bounds__(PF_NTHREADS) poly_k(POLY_SIGNATURE)
       if (kt + 1 < PF_KT) {
         // tile kt + 1 waits in the next set of the ring; once it is in LDS the set takes tile kt + 1 + PF_DEPTH
         const int nset = (d + 1) % PF_DEPTH;
-        StageA::store(lds_a[cur ^ 1], ra[nset]);
-        StageB::store(lds_b[cur ^ 1], rb[nset]);
+        store_tiles(kt + 1, nset, cur ^ 1);
         if (kt + 1 + PF_DEPTH < PF_KT) load_tiles(kt + 1 + PF_DEPTH, nset);
       }
       __syncthreads();

@@ -519,6 +519,23 @@ int poly_hip_fused_groups(const PolySchedule *s, int index, char **source_out, i
   return (int)groups.size();
 }
 
+int poly_hip_fused_group_launch(const PolySchedule *s, int index, int *slots_out, int cap, int *launch_out) {
+  if (!s) return -1;
+  std::vector<KernelGraph> graphs((size_t)s->n_items);
+  for (int k = 0; k < s->n_items; k++)
+    if (s->items[k].kind != POLY_EXEC_COMPUTE || !graphs[(size_t)k].build(s->items[k].root)) return -1;
+  std::vector<FusedGroup> groups;
+  find_fused_groups(s, graphs, &groups);
+  if (index < 0 || index >= (int)groups.size()) return -1;
+  const FusedGroup &fg = groups[(size_t)index];
+  for (size_t i = 0; i < fg.arg_slots.size() && (int)i < cap; i++) if (slots_out) slots_out[i] = fg.arg_slots[i];
+  if (launch_out) {
+    for (int i = 0; i < 3; i++) launch_out[i] = (int)fg.rk.launch.grid[i];
+    launch_out[3] = (int)fg.rk.launch.block[0];
+  }
+  return (int)fg.arg_slots.size();
+}
+
 void poly_hip_plan_free(PolyHipPlan *plan) {
   if (!plan) return;
   runtime_sync();

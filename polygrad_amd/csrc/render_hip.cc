@@ -660,6 +660,7 @@ bool render_kernel(const KernelGraph &g, const std::string &fn_name, const Rende
   if (opt.allow_templates) {
     if (try_render_matmul(g, fn_name, opt, out)) return true;
     if (try_render_gather(g, fn_name, opt, out)) return true;
+    if (try_render_matmul_generic(g, fn_name, opt, out)) return true;
   }
   *out = RenderedKernel();
   Generic gen(g, fn_name, opt);

@@ -283,12 +283,10 @@ bool matmul_store_contiguous(const KernelGraph &g, const MatmulMatch &mm, const 
   return true;
 }
 
-bool try_render_matmul(const KernelGraph &g, const std::string &fn, const RenderOptions &opt, RenderedKernel *out) {
-  (void)fn; (void)opt;
-  MatmulMatch mm;
-  int line = 0;
-  if (!match_matmul(g, &mm, &line)) return reject(line);
-  // epilogue: everything outside the REDUCE, per output element
+// The kernel's epilogue from its own graph: everything outside the REDUCE, per output
+// element (signature, device functions, the statement that stores one element, and the
+// value/address split when rows are contiguous along n).
+static bool epilogue_from_graph(const KernelGraph &g, const MatmulMatch &mm, MatmulEpilogue *epo) {
   const StoreInfo &st = g.stores[0];
   Emitter em(g);
   Scope S0;
@@ -300,7 +298,7 @@ bool try_render_matmul(const KernelGraph &g, const std::string &fn, const Render
   std::string idx = em.emit(g.n(st.index).src[1], &S0);
   if (em.failed()) return reject(__LINE__);
   const int pout = g.param_slot(st.param);
-  MatmulEpilogue ep;
+  MatmulEpilogue &ep = *epo;
   std::string params_call;
   for (size_t i = 0; i < g.params.size(); i++) {
     const ParamInfo &p = g.params[i];
@@ -339,8 +337,6 @@ bool try_render_matmul(const KernelGraph &g, const std::string &fn, const Render
       }
     }
   }
-  ep.a_ptr = strf("data%d", mm.A.param);
-  ep.b_ptr = strf("data%d", mm.B.param);
   ep.n_params = (int)g.params.size();
   // distinct elements: A, B once each (broadcast operands counted once), output once,
   // plus whatever the epilogue reads per output row/column
@@ -350,7 +346,34 @@ bool try_render_matmul(const KernelGraph &g, const std::string &fn, const Render
     if ((int)i == pout) n = (double)mm.M * mm.N * mm.Z;
     ep.bytes += n * dt_size(p.dt);
   }
+  return true;
+}
+
+bool try_render_matmul(const KernelGraph &g, const std::string &fn, const RenderOptions &opt, RenderedKernel *out) {
+  (void)fn; (void)opt;
+  MatmulMatch mm;
+  int line = 0;
+  if (!match_matmul(g, &mm, &line)) return reject(line);
+  MatmulEpilogue ep;
+  if (!epilogue_from_graph(g, mm, &ep)) return false;
+  ep.a_ptr = strf("data%d", mm.A.param);
+  ep.b_ptr = strf("data%d", mm.B.param);
   return render_matmul(mm, ep, out);
+}
+
+// Tile of the fp32 template: 4 waves; narrow outputs get a narrow tile.
+static void f32_tile(int64_t M, int64_t N, int64_t Z, int *bm, int *bn, int *wvm, int *wvn) {
+  int BM = 128, BN = 128, WVM = 2, WVN = 2;
+  if (N <= 32) { BN = 32; BM = 256; WVM = 4; WVN = 1; }
+  else if (N <= 64) { BN = 64; BM = 128; WVM = 4; WVN = 1; }
+  else if (M <= 32) { BM = 32; BN = 256; WVM = 1; WVN = 4; }
+  else if (M <= 64) { BM = 64; BN = 128; WVM = 1; WVN = 4; }
+  else if (((M + 127) / 128) * ((N + 127) / 128) * Z < 256) {
+    BM = 64; BN = 64; WVM = 2; WVN = 2;
+    // still fewer workgroups than CUs: two-wave workgroups on 32x64 tiles
+    if (((M + 63) / 64) * ((N + 63) / 64) * Z < 192) { BM = 32; BN = 64; WVM = 1; WVN = 2; }
+  }
+  *bm = BM; *bn = BN; *wvm = WVM; *wvn = WVN;
 }
 
 // fp32 operands: kernels/matmul_f32_mfma.hip (v_mfma_f32_32x32x2_f32, exact fp32 products).
@@ -367,17 +390,8 @@ static bool render_matmul_f32(const MatmulMatch &mm, const MatmulEpilogue &ep, R
   };
   bool a_kc, b_kc;
   if (!layout(mm.ka, mm.md, true, M, &a_kc) || !layout(mm.kb, mm.nd, false, N, &b_kc)) return reject(__LINE__);
-  // 4 waves; narrow outputs get a narrow tile
-  int BM = 128, BN = 128, WVM = 2, WVN = 2;
-  if (N <= 32) { BN = 32; BM = 256; WVM = 4; WVN = 1; }
-  else if (N <= 64) { BN = 64; BM = 128; WVM = 4; WVN = 1; }
-  else if (M <= 32) { BM = 32; BN = 256; WVM = 1; WVN = 4; }
-  else if (M <= 64) { BM = 64; BN = 128; WVM = 1; WVN = 4; }
-  else if (((M + 127) / 128) * ((N + 127) / 128) * Z < 256) {
-    BM = 64; BN = 64; WVM = 2; WVN = 2;
-    // still fewer workgroups than CUs: two-wave workgroups on 32x64 tiles
-    if (((M + 63) / 64) * ((N + 63) / 64) * Z < 192) { BM = 32; BN = 64; WVM = 1; WVN = 2; }
-  }
+  int BM, BN, WVM, WVN;
+  f32_tile(M, N, Z, &BM, &BN, &WVM, &WVN);
   const int64_t tiles = ((M + BM - 1) / BM) * ((N + BN - 1) / BN);
   if (tiles > 2147483647LL / 2) return reject(__LINE__);
   std::string cfg;
@@ -538,6 +552,279 @@ bool render_matmul(const MatmulMatch &mm, const MatmulEpilogue &ep, RenderedKern
         out->variants.push_back({strf("%dx%dw%dx%dp%d", c.bm, c.bn, c.wm, c.wn, c.pp), v.source, v.strategy, v.launch});
     }
   }
+  return true;
+}
+
+// ── matmul-shaped reductions whose operands are expressions ─────────────────
+//
+// Reverse-mode graphs multiply whatever the scheduler fused into the reduction: an fp32
+// gradient with a bf16 activation, a LayerNorm or softmax derivative evaluated in place,
+// sums over two ranges (batch and position), extents like 50257.  Any kernel of the form
+//     STORE(f(REDUCE(ADD, a * b, k...)))      a, b fp32-valued
+// in which some END range feeds only `a` and another only `b` is a matrix product
+// C[z][m][n] = sum_k A(z,m,k) B(z,k,n) of two computed operands.  The fp32 MFMA template
+// runs it with the operands evaluated on the way into LDS: the loads of an element are
+// issued K tiles ahead (phase 1, raw bits kept in registers), the arithmetic on them runs
+// when the tile is stored to LDS (phase 2).  Products are exact fp32, accumulation fp32.
+bool try_render_matmul_generic(const KernelGraph &g, const std::string &fn, const RenderOptions &opt, RenderedKernel *out) {
+  (void)fn; (void)opt;
+  if (getenv("POLY_HIP_NO_F32_MFMA") || getenv("POLY_HIP_NO_GENERIC_MM")) return reject(__LINE__);
+  if (g.stores.size() != 1 || g.reduces.size() != 1 || !g.vars.empty()) return reject(__LINE__);
+  const StoreInfo &st = g.stores[0];
+  if (st.gate >= 0) return reject(__LINE__);
+  const int red = g.reduces[0];
+  const KNode &R = g.n(red);
+  if (reduce_op(R) != POLY_OP_ADD || R.dt != DT_F32 || R.src.size() < 2) return reject(__LINE__);
+  const KNode &mul = g.n(R.src[0]);
+  if (mul.op != POLY_OP_MUL || mul.dt != DT_F32) return reject(__LINE__);
+  const int opnd[2] = {mul.src[0], mul.src[1]};
+  std::vector<int> kr;
+  int64_t K = 1;
+  uint64_t kmask = 0;
+  for (size_t i = 1; i < R.src.size(); i++) {
+    const int o = g.range_ord.at(R.src[i]);
+    const int64_t e = g.ranges[(size_t)o].extent;
+    if (e <= 0) return reject(__LINE__);
+    kr.push_back(o);
+    K *= e;
+    kmask |= (uint64_t)1 << o;
+  }
+  const uint64_t dep[2] = {g.n(opnd[0]).deps, g.n(opnd[1]).deps};
+  if (!(dep[0] & kmask) || !(dep[1] & kmask)) return reject(__LINE__);
+  // How each operand uses the END ranges.  A flat output range may carry the row of one
+  // operand in its upper digits and the column of the other in its lower ones (r / c and
+  // r % c in the load indices); such a range is cut into digits as in match_matmul.  That
+  // needs every use of the range inside the operand to be a load index: `direct` marks
+  // ranges an operand also reaches outside INDEX nodes (then the operand owns all of it).
+  std::vector<const Lin *> lins[2];
+  uint64_t direct[2] = {0, 0};
+  for (int side = 0; side < 2; side++) {
+    std::vector<int> stack{opnd[side]};
+    std::vector<char> seen(g.nodes.size(), 0);
+    while (!stack.empty()) {
+      const int id = stack.back();
+      stack.pop_back();
+      if (seen[(size_t)id]) continue;
+      seen[(size_t)id] = 1;
+      const KNode &k = g.n(id);
+      if (k.op == POLY_OP_RANGE) { direct[side] |= (uint64_t)1 << g.range_ord.at(id); continue; }
+      if (k.op == POLY_OP_INDEX) {
+        for (size_t i = 1; i < k.src.size(); i++) {
+          const int li = g.n(k.src[i]).lin;
+          if (li >= 0) lins[side].push_back(&g.lins[(size_t)li]);
+          else direct[side] |= g.n(k.src[i]).deps;      // an index or gate that is no canonical expression
+        }
+        continue;
+      }
+      for (int c : k.src) stack.push_back(c);
+    }
+  }
+  MatmulMatch mm;
+  for (int r : st.ranges) {
+    const int64_t e = g.ranges[(size_t)r].extent;
+    if (e <= 0) return reject(__LINE__);
+    const uint64_t bit = (uint64_t)1 << r;
+    std::vector<DigitUse> uses[2];
+    bool digits_ok = !((direct[0] | direct[1]) & bit);
+    for (int side = 0; side < 2 && digits_ok; side++)
+      for (const Lin *l : lins[side]) if (!digit_uses(g, *l, r, &uses[side])) { digits_ok = false; break; }
+    std::vector<int64_t> cuts{1, e};
+    if (digits_ok) {
+      for (int side = 0; side < 2; side++)
+        for (const DigitUse &d : uses[side]) {
+          cuts.push_back(d.a);
+          if (d.b > 0) cuts.push_back(d.a * d.b);
+        }
+      std::sort(cuts.begin(), cuts.end());
+      cuts.erase(std::unique(cuts.begin(), cuts.end()), cuts.end());
+      while (!cuts.empty() && cuts.back() > e) cuts.pop_back();
+      for (size_t i = 0; i + 1 < cuts.size(); i++) if (cuts[i + 1] % cuts[i] != 0) digits_ok = false;
+      if (cuts.empty() || cuts.back() != e) digits_ok = false;
+    }
+    if (!digits_ok) {
+      const bool in_a = (dep[0] & bit) != 0, in_b = (dep[1] & bit) != 0;
+      Dim d{r, e, 0, 0, 1};
+      if (in_a && !in_b) mm.md_full.push_back(d);
+      else if (in_b && !in_a) mm.nd_full.push_back(d);
+      else mm.zd_full.push_back(d);
+      continue;
+    }
+    auto used = [&](const std::vector<DigitUse> &u, int64_t cut) {
+      for (const DigitUse &d : u)
+        if (cut >= d.a && (d.b == 0 || cut < d.a * d.b) && d.coef != 0) return true;
+      return false;
+    };
+    for (size_t i = cuts.size() - 1; i-- > 0;) {
+      Dim d{r, cuts[i + 1] / cuts[i], 0, 0, cuts[i]};
+      const bool in_a = used(uses[0], cuts[i]), in_b = used(uses[1], cuts[i]);
+      if (in_a && !in_b) mm.md_full.push_back(d);
+      else if (in_b && !in_a) mm.nd_full.push_back(d);
+      else mm.zd_full.push_back(d);
+    }
+  }
+  if (mm.md_full.empty() || mm.nd_full.empty()) return reject(__LINE__);
+  mm.M = mm.N = mm.Z = 1;
+  for (const Dim &d : mm.md_full) mm.M *= d.extent;
+  for (const Dim &d : mm.nd_full) mm.N *= d.extent;
+  for (const Dim &d : mm.zd_full) mm.Z *= d.extent;
+  mm.md = mm.md_full; mm.nd = mm.nd_full; mm.zd = mm.zd_full;
+  mm.red = red; mm.K = K;
+  const int64_t M = mm.M, N = mm.N, Z = mm.Z;
+  // worth a tile pipeline: enough rows, columns and depth
+  if (M < 32 || N < 32 || K < 32 || Z > 65535 || M > 2147483647LL || N > 2147483647LL || K > 2147483647LL) return reject(__LINE__);
+  if ((double)M * (double)N * (double)K * (double)Z < 1048576.0) return reject(__LINE__);
+  for (const ParamInfo &p : g.params) if (p.numel >= ((int64_t)1 << 31)) return reject(__LINE__);
+
+  MatmulEpilogue ep;
+  if (!epilogue_from_graph(g, mm, &ep)) return reject(__LINE__);
+  std::string params_call;
+  for (size_t i = 0; i < g.params.size(); i++) params_call += strf("%sdata%zu", i ? ", " : "", i);
+
+  // C text that splits flattened coordinate `var` into digits (last one fastest); the
+  // value of a range is the sum of its digits times their cuts over the coordinates a
+  // function has (an operand never looks at the digits it does not get: they count as 0)
+  struct Bound { std::string code; std::map<int, std::string> range_sum; };
+  auto split_digits = [&](const std::vector<Dim> &dims, const char *var, Bound *b) {
+    if (dims.empty()) return;
+    b->code += strf("  int t_%s = %s;\n", var, var);
+    for (size_t i = dims.size(); i-- > 0;) {
+      const Dim &d = dims[i];
+      const std::string dv = strf("d%d_%lld", d.ord, (long long)d.cut);
+      if (i == 0) b->code += strf("  const int %s = t_%s;\n", dv.c_str(), var);
+      else b->code += strf("  const int %s = t_%s %% %lld; t_%s /= %lld;\n", dv.c_str(), var, (long long)d.extent, var, (long long)d.extent);
+      const std::string term = d.cut == 1 ? dv : strf("%s * %lld", dv.c_str(), (long long)d.cut);
+      std::string &sum = b->range_sum[d.ord];
+      sum = sum.empty() ? term : sum + " + " + term;
+    }
+  };
+  std::vector<Dim> k_dims;
+  for (int o : kr) k_dims.push_back(Dim{o, g.ranges[(size_t)o].extent, 0, 0, 1});
+  auto bind_all = [&](const std::vector<Dim> &rows, const char *rowvar, Emitter &em, Scope &S) {
+    Bound b;
+    split_digits(rows, rowvar, &b);
+    split_digits(k_dims, "k", &b);
+    split_digits(mm.zd_full, "z", &b);
+    for (auto &rs : b.range_sum) {
+      b.code += strf("  const int r%d = %s;\n", rs.first, rs.second.c_str());
+      em.bind_range(rs.first, strf("r%d", rs.first));
+      S.avail |= (uint64_t)1 << rs.first;
+    }
+    return b.code;
+  };
+  int n_loads[2] = {0, 0};
+  bool walk_k[2] = {true, true};
+  std::string code;
+  for (int side = 0; side < 2; side++) {
+    const char *nm = side == 0 ? "a" : "b";
+    const char *rowvar = side == 0 ? "m" : "n";
+    const std::vector<Dim> &row_dims = side == 0 ? mm.md_full : mm.nd_full;
+    // the loads under this operand, in topological order
+    std::vector<char> mark(g.nodes.size(), 0);
+    mark_reachable(g, opnd[side], mark);
+    std::vector<int> loads;
+    for (size_t id = 0; id < g.nodes.size(); id++)
+      if (mark[id] && g.n((int)id).op == POLY_OP_LOAD) {
+        const int sz = dt_size(g.n((int)id).dt);
+        if (sz != 1 && sz != 2 && sz != 4) return reject(__LINE__);
+        loads.push_back((int)id);
+      }
+    if (loads.size() > 6) return reject(__LINE__);
+    n_loads[side] = (int)loads.size();
+    // which way memory runs: along k when the first load has unit stride in the innermost
+    // reduce range, along the rows when it has unit stride in the innermost row range
+    if (!loads.empty()) {
+      const int li = g.n(g.n(g.n(loads[0]).src[0]).src[1]).lin;
+      if (li >= 0) {
+        const Lin &l = g.lins[(size_t)li];
+        bool aff_k;
+        const int64_t ck = g.lin_range_coef(l, kr.back(), &aff_k);
+        // stride of the innermost row digit
+        const Dim &rd = row_dims.back();
+        std::vector<DigitUse> u;
+        int64_t cr = 0;
+        if (digit_uses(g, l, rd.ord, &u))
+          for (const DigitUse &d : u)
+            if (rd.cut >= d.a && (d.b == 0 || rd.cut < d.a * d.b)) cr += d.coef * (rd.cut / d.a);
+        if (!(aff_k && (ck == 1 || ck == -1)) && (cr == 1 || cr == -1)) walk_k[side] = false;
+      }
+    }
+    const int nraw = std::max(1, n_loads[side]);
+    auto raw_of = [&](int j, DT dt) {
+      const int sz = dt_size(dt);
+      if (dt == DT_BOOL) return strf("(raw[%d] != 0u)", j);
+      if (sz == 4) return strf("__builtin_bit_cast(%s, raw[%d])", dt_cname(dt), j);
+      if (sz == 2) return strf("__builtin_bit_cast(%s, (unsigned short)raw[%d])", dt_cname(dt), j);
+      return strf("__builtin_bit_cast(%s, (unsigned char)raw[%d])", dt_cname(dt), j);
+    };
+    auto to_raw = [&](const std::string &v, DT dt) {
+      const int sz = dt_size(dt);
+      if (dt == DT_BOOL) return strf("((%s) ? 1u : 0u)", v.c_str());
+      if (sz == 4) return strf("__builtin_bit_cast(unsigned int, (%s)(%s))", dt_cname(dt), v.c_str());
+      if (sz == 2) return strf("(unsigned int)__builtin_bit_cast(unsigned short, (%s)(%s))", dt_cname(dt), v.c_str());
+      return strf("(unsigned int)__builtin_bit_cast(unsigned char, (%s)(%s))", dt_cname(dt), v.c_str());
+    };
+    // phase 1: the loads
+    {
+      Emitter em(g);
+      Scope S;
+      S.indent = 1;
+      std::string head = bind_all(row_dims, rowvar, em, S);
+      std::string body;
+      for (size_t j = 0; j < loads.size(); j++) {
+        const std::string v = em.emit(loads[j], &S);
+        body += strf("  raw[%zu] = %s;\n", j, to_raw(v, g.n(loads[j]).dt).c_str());
+      }
+      if (em.failed()) return reject(__LINE__);
+      code += strf("__device__ __forceinline__ void poly_%s_load(int %s, int k, int z, unsigned int (&raw)[%d], %s) {\n", nm, rowvar, nraw,
+                   ep.signature.c_str());
+      code += head + S.code + body + "}\n";
+    }
+    // phase 2: the arithmetic
+    {
+      Emitter em(g);
+      Scope S;
+      S.indent = 1;
+      std::string head = bind_all(row_dims, rowvar, em, S);
+      for (size_t j = 0; j < loads.size(); j++) em.preset(loads[j], raw_of((int)j, g.n(loads[j]).dt));
+      const std::string v = em.emit(opnd[side], &S);
+      if (em.failed()) return reject(__LINE__);
+      code += strf("__device__ __forceinline__ float poly_%s_math(int %s, int k, int z, const unsigned int (&raw)[%d], %s) {\n", nm, rowvar, nraw,
+                   ep.signature.c_str());
+      code += head + S.code + strf("  return %s;\n}\n", v.c_str());
+    }
+  }
+
+  int BM, BN, WVM, WVN;
+  f32_tile(M, N, Z, &BM, &BN, &WVM, &WVN);
+  const int64_t tiles = ((M + BM - 1) / BM) * ((N + BN - 1) / BN);
+  if (tiles > 2147483647LL / 2) return reject(__LINE__);
+  const int depth = n_loads[0] + n_loads[1] <= 2 ? 4 : n_loads[0] + n_loads[1] <= 4 ? 2 : 1;
+  std::string cfg;
+  cfg += strf("#define POLY_M %lld\n#define POLY_N %lld\n#define POLY_K %lld\n#define POLY_Z %lld\n", (long long)M, (long long)N, (long long)K, (long long)Z);
+  cfg += strf("#define POLY_BM %d\n#define POLY_BN %d\n#define POLY_WAVES_M %d\n#define POLY_WAVES_N %d\n#define POLY_GROUP_M 8\n", BM, BN, WVM, WVN);
+  cfg += strf("#define POLY_GEN 1\n#define POLY_PF_DEPTH %d\n#define POLY_A_KC %d\n#define POLY_B_KC %d\n", depth, walk_k[0] ? 1 : 0, walk_k[1] ? 1 : 0);
+  cfg += strf("#define POLY_A_NLOADS %d\n#define POLY_B_NLOADS %d\n", std::max(1, n_loads[0]), std::max(1, n_loads[1]));
+  cfg += strf("#define POLY_SIGNATURE %s\n", ep.signature.c_str());
+  cfg += ep.code + code;
+  cfg += strf("#define POLY_A_LOAD(m, k, z, raw) poly_a_load(m, k, z, raw, %s)\n#define POLY_A_MATH(m, k, z, raw) poly_a_math(m, k, z, raw, %s)\n",
+              params_call.c_str(), params_call.c_str());
+  cfg += strf("#define POLY_B_LOAD(n, k, z, raw) poly_b_load(n, k, z, raw, %s)\n#define POLY_B_MATH(n, k, z, raw) poly_b_math(n, k, z, raw, %s)\n",
+              params_call.c_str(), params_call.c_str());
+  cfg += strf("#define POLY_EPILOGUE(acc, m, n, z) %s\n", ep.call.c_str());
+  *out = RenderedKernel();
+  out->source = std::string(hip_prelude()) + cfg + kMatmulF32Template;
+  out->entry = "poly_k";
+  out->launch.grid[0] = (unsigned)tiles;
+  out->launch.grid[1] = (unsigned)Z;
+  out->launch.block[0] = (unsigned)(64 * WVM * WVN);
+  out->klass = KernelClass::MATMUL_MFMA;
+  out->strategy = strf("mfma 32x32x2 f32, operands as expressions (%d + %d loads per element pair, %d tiles ahead) M=%lld N=%lld K=%lld Z=%lld tile %dx%dx16 A:%s B:%s",
+                       n_loads[0], n_loads[1], depth, (long long)M, (long long)N, (long long)K, (long long)Z, BM, BN,
+                       walk_k[0] ? "k-major" : "m-major", walk_k[1] ? "k-major" : "n-major");
+  out->n_params = ep.n_params;
+  out->n_vars = 0;
+  out->flops = 2.0 * (double)M * (double)N * (double)K * (double)Z;
+  out->bytes = ep.bytes;
   return true;
 }
 

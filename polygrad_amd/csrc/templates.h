@@ -74,6 +74,9 @@ bool matmul_tuning_enabled();
 bool render_matmul(const MatmulMatch &mm, const MatmulEpilogue &ep, RenderedKernel *out);
 
 bool try_render_matmul(const KernelGraph &g, const std::string &fn, const RenderOptions &opt, RenderedKernel *out);
+// Matmul-shaped reductions of computed operands (mixed dtypes, derivatives fused into an
+// operand, several reduce ranges, ragged extents) on the fp32 MFMA template.
+bool try_render_matmul_generic(const KernelGraph &g, const std::string &fn, const RenderOptions &opt, RenderedKernel *out);
 bool try_render_gather(const KernelGraph &g, const std::string &fn, const RenderOptions &opt, RenderedKernel *out);
 
 }  // namespace polyhip

@@ -64,3 +64,38 @@ def random_slot_tensors(plan, seed=0, device="cuda", scale=1.0, outputs=()):
             t = torch.randint(0, 100, (s.numel,), generator=g, device=device).to(dt)
         data[s.index] = t
     return data
+
+
+def block_train_slot_tensors(plan, vocab=50257, seed=4, device="cuda"):
+    """Inputs of the one-block training plan (benchmark configuration 5): fp32 master
+    weights ~ N(0, 0.02), LayerNorm weights 1, biases and optimizer state 0, bf16
+    activations ~ N(0, 1), uniform random targets stored as floats, bias corrections of
+    the first AdamW step.  Returns (list indexed by slot, dict by name)."""
+    g = torch.Generator(device=device)
+    g.manual_seed(seed)
+    data = [None] * len(plan.slots)
+    by_name = {}
+    for s in plan.slots:
+        if s.is_intermediate:
+            continue
+        dt = torch_dtype(s.dtype)
+        n, name = s.numel, s.name
+        if name == "h0":
+            t = torch.randn(n, generator=g, device=device, dtype=torch.float32).to(dt)
+        elif name == "target":
+            t = torch.randint(0, vocab, (n,), generator=g, device=device).to(dt)
+        elif name == "arange" or name.startswith("__arange_"):
+            t = torch.arange(n, device=device).to(dt)
+        elif name == "bc1":
+            t = torch.full((n,), 1.0 / (1.0 - 0.9), dtype=dt, device=device)
+        elif name == "bc2":
+            t = torch.full((n,), 1.0 / (1.0 - 0.999), dtype=dt, device=device)
+        elif name.endswith(".m") or name.endswith(".v") or name == "loss" or name.endswith("_b"):
+            t = torch.zeros(n, dtype=dt, device=device)
+        elif name in ("ln1_w", "ln2_w", "lnf_w"):
+            t = torch.ones(n, dtype=dt, device=device)
+        else:
+            t = (torch.randn(n, generator=g, device=device, dtype=torch.float32) * 0.02).to(dt)
+        data[s.index] = t
+        by_name[name] = t
+    return data, by_name

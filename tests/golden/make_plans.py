@@ -8,6 +8,7 @@ the GPU box, where the reference frontend is not part of the product path:
     polygrad_amd/plans/attention_bf16_b8_h12_t1024_d64.polyplan   the attention block of config 4 alone
     polygrad_amd/plans/mlp_train_f32_b4096.polyplan        config 1: MLP forward + backward + SGD step
     polygrad_amd/plans/adamw_f32_355m.polyplan             config 5: AdamW update of 355 M fp32 parameters
+    polygrad_amd/plans/gpt2_medium_block_train_b4_t1024.polyplan   config 5: one block + head, backward, AdamW
 
 The graphs are built with the REAL reference frontend and scheduler
 (oracle/_ref/libpolygrad.so through tests/refpoly.py); only the scheduled kernel
@@ -79,6 +80,10 @@ def main():
     c = R.Ctx()
     _, _, _, sink = graphs.matmul_bf16(c, 1024, 1024, 1024, batch=16)
     save(c, sink, "matmul_bf16_b16_1024x1024x1024")
+    c.close()
+    c = R.Ctx()
+    _, sink = graphs.gpt2_block_train_step(c, batch=4, ctx=1024, d_model=1024, heads=16, vocab=50257)
+    save(c, sink, "gpt2_medium_block_train_b4_t1024")
     c.close()
 
 

@@ -294,7 +294,7 @@ BLOCK_PARAMS = ("ln1_w", "ln1_b", "attn_w", "attn_b", "proj_w", "proj_b", "ln2_w
 
 
 def gpt2_block_train_step(c, batch=4, ctx=1024, d_model=1024, heads=16, vocab=50257, lr=3e-4, beta1=0.9, beta2=0.999,
-                          eps=1e-8, weight_decay=0.1, ln_eps=1e-5):
+                          eps=1e-8, weight_decay=0.1, ln_eps=1e-5, head_vd=True):
     """One transformer block of config 5 (GPT-2 medium shapes) with the final LayerNorm,
     the vocabulary projection and next-token cross-entropy, reverse-mode gradients from the
     reference's poly_grad (src/autograd.c:773) and an AdamW update of every parameter
@@ -306,7 +306,7 @@ def gpt2_block_train_step(c, batch=4, ctx=1024, d_model=1024, heads=16, vocab=50
     hd = D // H
     shapes = dict(ln1_w=(D,), ln1_b=(D,), attn_w=(D, 3 * D), attn_b=(3 * D,), proj_w=(D, D), proj_b=(D,), ln2_w=(D,),
                   ln2_b=(D,), fc_w=(D, 4 * D), fc_b=(4 * D,), fc2_w=(4 * D, D), fc2_b=(D,), lnf_w=(D,), lnf_b=(D,),
-                  head_w=(D, V))
+                  head_w=(V, D) if head_vd else (D, V))      # (V, D): tied-embedding layout, as GPT-2 stores it
     bufs = {}
     P = {}
     for name in BLOCK_PARAMS:
@@ -340,7 +340,8 @@ def gpt2_block_train_step(c, batch=4, ctx=1024, d_model=1024, heads=16, vocab=50
     ff = _linear(ln2, W["fc_w"], W["fc_b"], wdt).contiguous().gelu().contiguous()
     h2 = (h1 + _linear(ff, W["fc2_w"], W["fc2_b"], wdt).contiguous()).contiguous()
     lnf = _layernorm(h2, W["lnf_w"], W["lnf_b"], ln_eps, wdt).contiguous()
-    logits = lnf.reshape((B * T, D)).cast(R.F32).dot(W["head_w"].cast(R.F32)).contiguous()   # fp32 logits
+    hw = W["head_w"].permute((1, 0)) if head_vd else W["head_w"]
+    logits = lnf.reshape((B * T, D)).cast(R.F32).dot(hw.cast(R.F32)).contiguous()   # fp32 logits
     loss = logits.cross_entropy(target)
     assigns = []
     for name in BLOCK_PARAMS:

@@ -117,3 +117,41 @@ def test_full_size_row_block_matches_cpu_bit_pattern_of_sums():
     h = got[O].reshape(m, n)[rows]
     w = want[O8].reshape(8, n)
     assert_close(h, w, rtol=1e-4, atol=1e-4 * float(np.abs(w).mean()), what="row block of 1024x4096x4096")
+
+
+def test_matmul_of_computed_operands():
+    """Matmul-shaped reductions that the plain templates do not take -- an fp32 operand
+    against a bf16 one, arithmetic fused into an operand, a ragged depth, two reduce
+    ranges, a flat output range shared by both operands -- run on the fp32 MFMA template
+    with the operands evaluated on the way into LDS.  Products are exact fp32, so the
+    tolerance is the fp32 reduction one."""
+    g = np.random.default_rng(21)
+    # (a) fp32 x bf16, K = 301 (not a multiple of the 16-deep K tile), relu fused into A
+    c = R.Ctx()
+    M, N, K = 96, 160, 301
+    A = c.buffer((M, K), R.F32, name="A")
+    Bm = c.buffer((K, N), R.BF16, name="B")
+    O = c.buffer((M, N), R.F32, name="C")
+    sink = c.sink((O, (A.relu() * c.const(0.5)).dot(Bm.cast(R.F32))))
+    arrays = {A: g.normal(0, 1, (M, K)).astype(np.float32), Bm: bf16(g, (K, N), 1.0), O: np.zeros((M, N), np.float32)}
+    want = run_ref(c, sink, arrays)
+    got, info = run_hip(c, sink, arrays)
+    c.close()
+    assert any("operands as expressions" in k["desc"] for k in info), [k["desc"] for k in info]
+    assert_close(got[O], want[O], rtol=1e-4, atol=1e-4 * float(np.abs(want[O]).mean()), what="fp32 x bf16, ragged K")
+    # (b) weight-gradient form: dW[i, j] = sum over (b, t) of X[b, t, i] * dY[b, t, j], flat output
+    c = R.Ctx()
+    Bt, T, I, J = 3, 100, 64, 96
+    X = c.buffer((Bt, T, I), R.BF16, name="X")
+    dY = c.buffer((Bt, T, J), R.F32, name="dY")
+    O = c.buffer((I * J,), R.F32, name="dW")
+    xe = X.cast(R.F32).reshape((Bt, T, I, 1)).expand((Bt, T, I, J))
+    ye = dY.reshape((Bt, T, 1, J)).expand((Bt, T, I, J))
+    dw = (xe * ye).reduce_axes("ADD", [0, 1]).reshape((I * J,))
+    sink = c.sink((O, dw))
+    arrays = {X: bf16(g, (Bt, T, I), 1.0), dY: g.normal(0, 1, (Bt, T, J)).astype(np.float32), O: np.zeros(I * J, np.float32)}
+    want = run_ref(c, sink, arrays)
+    got, info = run_hip(c, sink, arrays)
+    c.close()
+    assert any("operands as expressions" in k["desc"] for k in info), [k["desc"] for k in info]
+    assert_close(got[O], want[O], rtol=1e-4, atol=1e-4 * float(np.abs(want[O]).mean()), what="weight gradient over two ranges")

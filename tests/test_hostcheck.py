@@ -1,0 +1,51 @@
+"""Indexing of the generated kernels, checked without a GPU: every kernel of every
+golden fixture and of the reduced training step runs on the host under
+AddressSanitizer (tests/hostcheck.py), so an out-of-bounds load or store -- which on the
+device may go unnoticed or fault the card -- fails here with the offending line."""
+import ctypes as C
+import os
+
+import pytest
+
+import fixtures as F
+import hostcheck
+import refpoly as R
+from polygrad_amd import _ffi
+
+pytestmark = pytest.mark.skipif(not os.path.exists(hostcheck.CLANG), reason="no host clang with AddressSanitizer")
+
+
+def test_checker_sees_an_overrun(hiplib):
+    fx = F.Fixture("bf16_matmul")
+    jobs = list(hostcheck._jobs(hiplib, fx.plan.schedule, 1 << 21, None, False))
+    what, main, grid, block, sizes = jobs[0]
+    hostcheck.check_kernel(main, hostcheck._entry_name(main), grid, block, sizes)
+    with pytest.raises(AssertionError, match="out-of-bounds"):
+        hostcheck.check_kernel(main, hostcheck._entry_name(main), grid, block, [sizes[0] // 2] + list(sizes[1:]))
+
+
+def test_fixture_kernels_stay_in_bounds(hiplib):
+    total = 0
+    for name in F.case_names():
+        fx = F.Fixture(name)            # owns the schedule's memory
+        total += hostcheck.check_schedule(hiplib, fx.plan.schedule)
+    assert total > 100
+
+
+@pytest.mark.skipif(not R.available(), reason="reference library not built")
+@pytest.mark.parametrize("B,T,D,H,V", [(1, 32, 64, 2, 97), (2, 64, 128, 4, 301)])
+def test_training_step_kernels_stay_in_bounds(B, T, D, H, V, hiplib):
+    """The backward kernels of the one-block training step: among them the derivative of a
+    pad, `where(valid, reduce(...), 0)`, whose index arithmetic goes negative on the masked
+    positions (a modulus emitted as C's % read in front of its buffer there), and, at the
+    larger size, the matmul-shaped reductions with computed operands and ragged extents."""
+    import graphs
+    c = R.Ctx()
+    _, sink = graphs.gpt2_block_train_step(c, B, T, D, H, V)
+    sched = c.schedule(sink)
+    try:
+        n = hostcheck.check_schedule(hiplib, sched)
+    finally:
+        c.L.poly_schedule_free(sched)
+        c.close()
+    assert n > 60
