@@ -42,6 +42,10 @@ static void name_kernel(RenderedKernel *rk) {
     rename(rk->fallback_source, " poly_k(", " " + name + "_slow(");
     rk->fallback_entry = name + "_slow";
   }
+  if (!rk->pre_source.empty()) {
+    rename(rk->pre_source, " poly_k(", " " + name + "_terms(");
+    rk->pre_entry = name + "_terms";
+  }
 }
 
 static bool render_root(const PolyUOp *root, const char *fn_name, int flags, RenderedKernel *rk) {
@@ -82,12 +86,18 @@ HipRunner *runner_from_rendered(const RenderedKernel &rk, const char *fn_name, b
     r->fallback = program_create(r->rk.fallback_source, r->rk.fallback_entry);
     if (!r->fallback) { runner_destroy(r); return nullptr; }
   }
+  if (!r->rk.pre_source.empty()) {
+    if (!r->rk.guards.empty()) { log_err("lower", "%s: a two-stage kernel cannot also be guarded", r->name.c_str()); runner_destroy(r); return nullptr; }
+    r->pre = program_create(r->rk.pre_source, r->rk.pre_entry);
+    r->scratch = runtime_alloc(r->rk.scratch_bytes);
+    if (!r->pre || !r->scratch) { runner_destroy(r); return nullptr; }
+  }
   for (const RenderedKernel::Table &t : r->rk.tables) {
     std::shared_ptr<void> tab = runtime_table(t.source, t.entry, t.bytes, t.launch);
     if (!tab) { runner_destroy(r); return nullptr; }
     r->tables.push_back(tab);
   }
-  size_t n = (size_t)r->rk.n_params + (size_t)r->rk.n_vars + r->rk.tables.size() + 1;
+  size_t n = (size_t)r->rk.n_params + (size_t)r->rk.n_vars + r->rk.tables.size() + 2;
   r->ptr_store.resize(n);
   r->var_store.resize(n);
   r->arg_ptrs.resize(n);
@@ -118,6 +128,8 @@ void runner_destroy(HipRunner *r) {
   if (r->main) program_destroy(r->main);
   for (Program *p : r->guards) program_destroy(p);
   if (r->fallback) program_destroy(r->fallback);
+  if (r->pre) program_destroy(r->pre);
+  if (r->scratch) runtime_free(r->scratch);
   if (r->flag) runtime_free(r->flag);
   delete r;
 }
@@ -143,6 +155,12 @@ int runner_launch(HipRunner *r, void **args, int n_args) {
   for (int t = 0; t < nt; t++) {
     r->ptr_store[(size_t)(np + nv + t)] = r->tables[(size_t)t].get();
     r->arg_ptrs[(size_t)(np + nv + t)] = &r->ptr_store[(size_t)(np + nv + t)];
+  }
+  if (r->pre) {
+    r->ptr_store[(size_t)(np + nv + nt)] = r->scratch;
+    r->arg_ptrs[(size_t)(np + nv + nt)] = &r->ptr_store[(size_t)(np + nv + nt)];
+    if (program_launch(r->pre, r->arg_ptrs.data(), r->rk.pre_launch) != 0) return -1;
+    return program_launch(r->main, r->arg_ptrs.data(), r->rk.launch);
   }
   if (r->guards.empty()) return program_launch(r->main, r->arg_ptrs.data(), r->rk.launch);
   // The guard writes *flag (1 = fast path valid, 0 = not); the fast kernel and
@@ -265,6 +283,8 @@ char *poly_hip_render(PolyUOp *scheduled_root, const char *fn_name, int flags, i
   std::string all = rk.source;
   for (const RenderedKernel::Guard &g : rk.guards) all += "\n// ---- guard ----\n" + g.source;
   if (!rk.fallback_source.empty()) all += "\n// ---- fallback ----\n" + rk.fallback_source;
+  if (!rk.pre_source.empty())
+    all += strf("\n// ---- terms ---- grid=%u block=%u\n", rk.pre_launch.grid[0], rk.pre_launch.block[0]) + rk.pre_source;
   for (size_t i = 1; i < rk.variants.size(); i++) all += "\n// ---- variant " + rk.variants[i].label + "\n" + rk.variants[i].source;
   return dup_string(all);
 }

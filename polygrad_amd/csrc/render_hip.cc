@@ -181,6 +181,7 @@ class Generic {
       first = false;
       s += strf("const int var%zu", i);
     }
+    if (opt_.scratch_param) { s += std::string(first ? "" : ", ") + "float* poly_scratch"; first = false; }
     if (opt_.exit_if_flag || opt_.exit_unless_flag) s += std::string(first ? "" : ", ") + "const int* __restrict__ poly_flag";
     return s + ")";
   }
@@ -204,6 +205,16 @@ class Generic {
       if (in) for (int s : k.src) inside[(size_t)s] = 1;
     }
     for (int r : g_.reduces) if (!inside[(size_t)r]) top_reduces_.push_back(r);
+    if (opt_.promote_reduce >= 0) {
+      // the reductions directly inside the promoted one take its place
+      const int T = opt_.promote_reduce;
+      std::vector<char> in_t(g_.nodes.size(), 0), deeper(g_.nodes.size(), 0);
+      mark_reachable(g_, g_.n(T).src[0], in_t);
+      for (int r : g_.reduces) if (r != T && in_t[(size_t)r]) mark_reachable(g_, g_.n(r).src[0], deeper);
+      top_reduces_.clear();
+      for (int r : g_.reduces) if (r != T && in_t[(size_t)r] && !deeper[(size_t)r]) top_reduces_.push_back(r);
+      if (top_reduces_.empty() || groups_.size() != 1) { *err = "nothing to promote"; return false; }
+    }
     return true;
   }
 
@@ -215,6 +226,16 @@ class Generic {
 
   // Orders a group's ranges fastest-first using the first store's index strides.
   std::vector<int> fastest_first(const Group &gr) const {
+    if (opt_.promote_reduce >= 0) {
+      RenderOptions plain = opt_;
+      plain.promote_reduce = -1;
+      std::vector<int> order;
+      const KNode &T = g_.n(opt_.promote_reduce);
+      for (size_t i = T.src.size(); i-- > 1;) order.push_back(g_.range_ord.at(T.src[i]));
+      Generic base(g_, fn_, plain);
+      for (int r : base.fastest_first(gr)) order.push_back(r);
+      return order;
+    }
     const StoreInfo &st = g_.stores[(size_t)gr.stores[0]];
     int li = g_.n(g_.n(st.index).src[1]).lin;
     std::vector<std::pair<int64_t, int>> keyed;
@@ -445,7 +466,7 @@ class Generic {
           for (int r : groups_[0].ranges) if (r == ord) unit_along_output = true;
         }
       }
-      if (!unit_along_reduce && unit_along_output && rows >= 65536) return false;
+      if (!unit_along_reduce && unit_along_output && rows >= 65536 && opt_.promote_reduce < 0) return false;
     }
     // Long rows, or too few rows to fill the chip with one wave each: a whole
     // workgroup per row.
@@ -467,6 +488,10 @@ class Generic {
     Scope S0;
     S0.indent = 2;
     for (int r : gr.ranges) S0.avail |= (uint64_t)1 << r;
+    if (opt_.promote_reduce >= 0) {
+      const KNode &T = g_.n(opt_.promote_reduce);
+      for (size_t i = 1; i < T.src.size(); i++) S0.avail |= (uint64_t)1 << g_.range_ord.at(T.src[i]);
+    }
     if (G == 64) {
       line(body, 1, "const int lane = threadIdx.x & 63;");
       line(body, 1, strf("const long long row = (long long)blockIdx.x * %d + (threadIdx.x >> 6);", rows_per_block));
@@ -587,6 +612,10 @@ class Generic {
     for (int id : top_reduces_) em_.preset(id, strf("acc%d", id));
     // tail: value + store by lane 0
     std::string tail_stores;
+    if (opt_.promote_reduce >= 0) {
+      const std::string term = em_.emit(g_.n(opt_.promote_reduce).src[0], &S0);
+      line(tail_stores, 2, strf("if (lane == 0) poly_scratch[row] = %s;", term.c_str()));
+    } else
     for (int si : gr.stores) {
       const StoreInfo &st = g_.stores[(size_t)si];
       std::string v = em_.emit(st.value, &S0);
@@ -655,6 +684,81 @@ class Generic {
 
 }  // namespace
 
+// A reduction to few outputs whose terms are reductions themselves (a loss: the sum over
+// tokens of a sum over the vocabulary) would run on one workgroup per output, each thread
+// walking a whole inner row on its own.  It is cut in two kernels instead: the first
+// gives every (output, outer index) pair a workgroup that reduces the inner ranges
+// cooperatively and leaves the term in scratch memory; the second is the original kernel
+// with the outer REDUCE replaced by a sum over those terms, in index order.
+static bool try_split_reduce(const KernelGraph &g, const std::string &fn_name, const RenderOptions &opt, RenderedKernel *out) {
+  if (!opt.allow_coop_reduce || !opt.reduce_override.empty() || opt.exit_if_flag || opt.exit_unless_flag ||
+      opt.promote_reduce >= 0 || getenv("POLY_HIP_NO_SPLIT_REDUCE"))
+    return false;
+  if (g.stores.empty() || g.reduces.size() < 2) return false;
+  for (const StoreInfo &st : g.stores) if (st.ranges != g.stores[0].ranges) return false;
+  // exactly one REDUCE that is not nested in another: the one to promote
+  std::vector<char> inside(g.nodes.size(), 0);
+  for (int r : g.reduces) mark_reachable(g, g.n(r).src[0], inside);
+  int T = -1;
+  for (int r : g.reduces) if (!inside[(size_t)r]) { if (T >= 0) return false; T = r; }
+  if (T < 0) return false;
+  const KNode &tk = g.n(T);
+  const PolyOps top = tk.u->arg.kind == POLY_ARG_OPS ? tk.u->arg.ops : (PolyOps)tk.u->arg.i;
+  if (tk.dt != DT_F32 || (top != POLY_OP_ADD && top != POLY_OP_MAX && top != POLY_OP_MUL)) return false;
+  double rows = 1, rt = 1, inner = 0;
+  for (int r : g.stores[0].ranges) { if (g.ranges[(size_t)r].extent <= 0) return false; rows *= (double)g.ranges[(size_t)r].extent; }
+  for (size_t i = 1; i < tk.src.size(); i++) {
+    const int64_t e = g.ranges[(size_t)g.range_ord.at(tk.src[i])].extent;
+    if (e <= 0) return false;
+    rt *= (double)e;
+  }
+  for (int r : g.reduces) {
+    if (r == T) continue;
+    double n = 1;
+    for (size_t i = 1; i < g.n(r).src.size(); i++) {
+      const int64_t e = g.ranges[(size_t)g.range_ord.at(g.n(r).src[i])].extent;
+      if (e <= 0) return false;
+      n *= (double)e;
+    }
+    inner = std::max(inner, n);
+  }
+  // few outputs, many terms, long inner rows
+  if (rows > 64 || rt < 64 || inner < 256 || rows * rt > 16777216.0) return false;
+
+  RenderOptions o1 = opt;
+  o1.promote_reduce = T;
+  o1.scratch_param = true;
+  RenderedKernel pre;
+  std::string err;
+  {
+    Generic gen(g, fn_name, o1);
+    if (!gen.run(&pre, &err) || pre.klass != KernelClass::ROW_REDUCE) return false;
+  }
+  RenderOptions o2 = opt;
+  o2.scratch_param = true;
+  o2.allow_vectorize = false;       // thread id == flat output index, which is what the terms are filed under
+  const long long RT = (long long)rt;
+  o2.reduce_override[T] = [T, RT, top](Emitter &em, Scope *s) {
+    (void)em;
+    const std::string acc = strf("acc%d", T);
+    std::string pad((size_t)s->indent * 2, ' ');
+    s->code += pad + strf("float %s = %s;\n", acc.c_str(), Emitter::reduce_identity(top, DT_F32).c_str());
+    s->code += pad + strf("for (int q_ = 0; q_ < %lld; q_++) %s = %s;\n", RT, acc.c_str(),
+                          Emitter::reduce_combine(top, DT_F32, acc, strf("poly_scratch[gid * %lldll + q_]", RT)).c_str());
+    return acc;
+  };
+  Generic gen2(g, fn_name, o2);
+  if (!gen2.run(out, &err) || out->klass == KernelClass::ROW_REDUCE) return false;
+  out->pre_source = pre.source;
+  out->pre_entry = pre.entry;
+  out->pre_launch = pre.launch;
+  out->scratch_bytes = (size_t)(rows * rt) * sizeof(float);
+  out->klass = KernelClass::ROW_REDUCE;
+  out->strategy = "two stages: " + pre.strategy + " into scratch, then " + out->strategy;
+  out->bytes = pre.bytes;
+  return true;
+}
+
 bool render_kernel(const KernelGraph &g, const std::string &fn_name, const RenderOptions &opt,
                    RenderedKernel *out, std::string *err) {
   if (opt.allow_templates) {
@@ -662,6 +766,8 @@ bool render_kernel(const KernelGraph &g, const std::string &fn_name, const Rende
     if (try_render_gather(g, fn_name, opt, out)) return true;
     if (try_render_matmul_generic(g, fn_name, opt, out)) return true;
   }
+  *out = RenderedKernel();
+  if (try_split_reduce(g, fn_name, opt, out)) return true;
   *out = RenderedKernel();
   Generic gen(g, fn_name, opt);
   return gen.run(out, err);

@@ -64,6 +64,12 @@ struct RenderedKernel {
     LaunchSpec launch;
   };
   std::vector<Variant> variants;
+  // Two-stage reductions: `pre_source` runs first, with the same arguments plus one more
+  // pointer to `scratch_bytes` bytes of device memory that the runner owns; the main
+  // kernel takes that pointer too (after the variables and tables).
+  std::string pre_source, pre_entry;
+  LaunchSpec pre_launch;
+  size_t scratch_bytes = 0;
 };
 
 struct Scope;
@@ -81,6 +87,12 @@ struct RenderOptions {
   // REDUCE nodes whose value the caller computes without a loop (gather fast
   // path); the kernel is then lowered as if it had no such reduction.
   std::unordered_map<int, std::function<std::string(Emitter &, Scope *)>> reduce_override;
+  // First stage of a two-stage reduction: the ranges of REDUCE node `promote_reduce` count
+  // as output ranges (fastest), the reductions nested in its operand are the ones that run,
+  // and what would be one term of that REDUCE goes to poly_scratch[row].
+  int promote_reduce = -1;
+  // The kernel takes `float* poly_scratch` as its last pointer argument.
+  bool scratch_param = false;
 };
 
 // Returns false and sets *err on unsupported graphs (never falls back to a

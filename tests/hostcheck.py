@@ -141,6 +141,10 @@ def _jobs(lib, schedule, max_threads, only, groups):
         seen.add((main, sizes))
         grid = (launch[0], launch[1], launch[2])
         yield f"step {step}", main, grid, launch[3], sizes
+        for unit in text.split("\n// ---- ")[1:]:
+            m = re.match(r"terms ---- grid=(\d+) block=(\d+)\n", unit)
+            if m:       # first stage of a two-stage reduction: same arguments plus the scratch, its own launch
+                yield f"step {step} (terms)", unit[m.end():], (int(m.group(1)), 1, 1), int(m.group(2)), sizes
     if not groups or only is not None:
         return
     for gi in range(lib.poly_hip_fused_groups(schedule, -1, None, None)):
