@@ -284,7 +284,7 @@ char *poly_hip_render(PolyUOp *scheduled_root, const char *fn_name, int flags, i
   for (const RenderedKernel::Guard &g : rk.guards) all += "\n// ---- guard ----\n" + g.source;
   if (!rk.fallback_source.empty()) all += "\n// ---- fallback ----\n" + rk.fallback_source;
   if (!rk.pre_source.empty())
-    all += strf("\n// ---- terms ---- grid=%u block=%u\n", rk.pre_launch.grid[0], rk.pre_launch.block[0]) + rk.pre_source;
+    all += strf("\n// ---- terms ---- grid=%u block=%u scratch=%zu\n", rk.pre_launch.grid[0], rk.pre_launch.block[0], rk.scratch_bytes) + rk.pre_source;
   for (size_t i = 1; i < rk.variants.size(); i++) all += "\n// ---- variant " + rk.variants[i].label + "\n" + rk.variants[i].source;
   return dup_string(all);
 }

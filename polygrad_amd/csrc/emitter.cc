@@ -257,6 +257,9 @@ std::string Emitter::emit_reduce_serial(int id, Scope *t) {
     std::string rv = strf("r%d", ord);
     std::string bound = r.extent >= 0 ? strf("%lld", (long long)r.extent) : emit(r.bound_node, t);
     opens.append((size_t)inner.indent * 2, ' ');
+    if (id == slice_node_ && ord == slice_ord_)
+      opens += strf("for (int %s = %s; %s < %s; %s += %d) {\n", rv.c_str(), slice_first_.c_str(), rv.c_str(), bound.c_str(), rv.c_str(), slice_step_);
+    else
     opens += strf("for (int %s = 0; %s < %s; %s++) {\n", rv.c_str(), rv.c_str(), bound.c_str(), rv.c_str());
     bind_range(ord, rv);
     inner.avail |= (uint64_t)1 << ord;

@@ -330,7 +330,7 @@ class Generic {
           nthreads += strf("*%lldll", (long long)nv);
           nthreads_n *= (double)nv;
         } else {
-          if (oi + 1 == order.size())
+          if (oi + 1 == order.size() && opt_.slice_reduce < 0)
             line(decomp, 2, strf("const int %s = (int)t_;", rv.c_str()));
           else
             line(decomp, 2, strf("const int %s = (int)(t_ %% %s); t_ /= %s;", rv.c_str(), e.expr.c_str(), e.expr.c_str()));
@@ -339,8 +339,25 @@ class Generic {
           em_.bind_range(ord, rv);
         }
       }
-      max_threads = std::max(max_threads, nthreads_n);
       std::string sect;
+      if (opt_.slice_reduce >= 0) {
+        // first stage of a sliced reduction: the digit left in t_ is the part number
+        line(decomp, 2, "const int part_ = (int)t_;");
+        const std::string n_out = nthreads;
+        nthreads += strf("*%dll", opt_.slice_parts);
+        nthreads_n *= (double)opt_.slice_parts;
+        em_.slice_reduce(opt_.slice_reduce, opt_.slice_range, "part_", opt_.slice_parts);
+        const std::string v = em_.emit(opt_.slice_reduce, &S0);
+        line(S0.code, 2, strf("poly_scratch[(gid %% (%s)) * %dll + part_] = %s;", n_out.c_str(), opt_.slice_parts, v.c_str()));
+        sect = S0.code;
+        strat += strf("partial sums, %d per output; ", opt_.slice_parts);
+        max_threads = std::max(max_threads, nthreads_n);
+        line(body, 1, strf("if (gid < %s) {", nthreads.c_str()));
+        body += decomp + sect;
+        line(body, 1, "}");
+        continue;
+      }
+      max_threads = std::max(max_threads, nthreads_n);
       if (V > 1) {
         std::string f0 = strf("r%d_0", F);
         std::vector<int> roots;
@@ -466,7 +483,7 @@ class Generic {
           for (int r : groups_[0].ranges) if (r == ord) unit_along_output = true;
         }
       }
-      if (!unit_along_reduce && unit_along_output && rows >= 65536 && opt_.promote_reduce < 0) return false;
+      if (!unit_along_reduce && unit_along_output && (rows >= 65536 || opt_.coop_needs_unit_stride) && opt_.promote_reduce < 0) return false;
     }
     // Long rows, or too few rows to fill the chip with one wave each: a whole
     // workgroup per row.
@@ -684,6 +701,9 @@ class Generic {
 
 }  // namespace
 
+static bool split_in_two(const KernelGraph &g, const std::string &fn_name, const RenderOptions &opt, int T, PolyOps top,
+                         double rows, double per_output, int slice_range, int parts, RenderedKernel *out);
+
 // A reduction to few outputs whose terms are reductions themselves (a loss: the sum over
 // tokens of a sum over the vocabulary) would run on one workgroup per output, each thread
 // walking a whole inner row on its own.  It is cut in two kernels instead: the first
@@ -724,15 +744,68 @@ static bool try_split_reduce(const KernelGraph &g, const std::string &fn_name, c
   }
   // few outputs, many terms, long inner rows
   if (rows > 64 || rt < 64 || inner < 256 || rows * rt > 16777216.0) return false;
+  return split_in_two(g, fn_name, opt, T, top, rows, rt, -1, 0, out);
+}
+
+// The other shape: one REDUCE over many terms for a modest number of outputs, where lanes
+// along the outputs are the coalesced mapping (column sums: bias and LayerNorm-parameter
+// gradients) and one thread per output leaves most of the chip idle.  Each output gets
+// `parts` threads that walk the longest reduce range in steps of `parts`; the second
+// kernel adds the partial results in part order.
+static bool try_slice_reduce(const KernelGraph &g, const std::string &fn_name, const RenderOptions &opt, RenderedKernel *out) {
+  if (!opt.reduce_override.empty() || opt.exit_if_flag || opt.exit_unless_flag || opt.promote_reduce >= 0 ||
+      opt.slice_reduce >= 0 || getenv("POLY_HIP_NO_SPLIT_REDUCE"))
+    return false;
+  if (g.stores.empty() || g.reduces.size() != 1 || !g.vars.empty()) return false;
+  for (const StoreInfo &st : g.stores) if (st.ranges != g.stores[0].ranges) return false;
+  const int T = g.reduces[0];
+  const KNode &tk = g.n(T);
+  const PolyOps top = tk.u->arg.kind == POLY_ARG_OPS ? tk.u->arg.ops : (PolyOps)tk.u->arg.i;
+  if (tk.dt != DT_F32 || (top != POLY_OP_ADD && top != POLY_OP_MAX && top != POLY_OP_MUL)) return false;
+  double rows = 1, rt = 1;
+  for (int r : g.stores[0].ranges) { if (g.ranges[(size_t)r].extent <= 0) return false; rows *= (double)g.ranges[(size_t)r].extent; }
+  int longest = -1;
+  for (size_t i = 1; i < tk.src.size(); i++) {
+    const int ord = g.range_ord.at(tk.src[i]);
+    const int64_t e = g.ranges[(size_t)ord].extent;
+    if (e <= 0) return false;
+    rt *= (double)e;
+    if (longest < 0 || e > g.ranges[(size_t)longest].extent) longest = ord;
+  }
+  if (rows > 16384 || rt < 1024) return false;
+  // only where the plain lowering is one thread per output
+  {
+    RenderedKernel plain;
+    std::string err;
+    RenderOptions strict = opt;
+    strict.coop_needs_unit_stride = true;
+    Generic gen(g, fn_name, strict);
+    if (!gen.run(&plain, &err) || plain.klass != KernelClass::THREAD_REDUCE) return false;
+  }
+  int parts = 1;
+  while (parts < 128 && rows * parts < 65536.0 && (int64_t)parts * 8 <= g.ranges[(size_t)longest].extent) parts *= 2;
+  if (parts < 4) return false;
+  return split_in_two(g, fn_name, opt, T, top, rows, (double)parts, longest, parts, out);
+}
+
+// Renders the two kernels of a split reduction of REDUCE node T: the first stage leaves
+// `per_output` terms per output in scratch memory (promoted ranges when slice_range < 0,
+// else `parts` strided slices of that range), the second is the kernel itself with T
+// replaced by the combination of those terms in index order.
+static bool split_in_two(const KernelGraph &g, const std::string &fn_name, const RenderOptions &opt, int T, PolyOps top,
+                         double rows, double per_output, int slice_range, int parts, RenderedKernel *out) {
+  const double rt = per_output;
 
   RenderOptions o1 = opt;
-  o1.promote_reduce = T;
   o1.scratch_param = true;
+  if (slice_range >= 0) { o1.slice_reduce = T; o1.slice_range = slice_range; o1.slice_parts = parts; o1.allow_coop_reduce = false; }
+  else o1.promote_reduce = T;
   RenderedKernel pre;
   std::string err;
   {
     Generic gen(g, fn_name, o1);
-    if (!gen.run(&pre, &err) || pre.klass != KernelClass::ROW_REDUCE) return false;
+    if (!gen.run(&pre, &err)) return false;
+    if (slice_range < 0 && pre.klass != KernelClass::ROW_REDUCE) return false;
   }
   RenderOptions o2 = opt;
   o2.scratch_param = true;
@@ -768,6 +841,8 @@ bool render_kernel(const KernelGraph &g, const std::string &fn_name, const Rende
   }
   *out = RenderedKernel();
   if (try_split_reduce(g, fn_name, opt, out)) return true;
+  *out = RenderedKernel();
+  if (try_slice_reduce(g, fn_name, opt, out)) return true;
   *out = RenderedKernel();
   Generic gen(g, fn_name, opt);
   return gen.run(out, err);

@@ -93,6 +93,13 @@ struct RenderOptions {
   int promote_reduce = -1;
   // The kernel takes `float* poly_scratch` as its last pointer argument.
   bool scratch_param = false;
+  // Another first stage: one thread per (output, part); REDUCE node `slice_reduce` walks
+  // range ordinal `slice_range` from its part number in steps of `slice_parts`, and the
+  // partial result goes to poly_scratch[output * slice_parts + part].
+  int slice_reduce = -1, slice_range = -1, slice_parts = 0;
+  // Lanes along the reduce range only when some load is contiguous along it, however few
+  // rows there are (otherwise: only from 65536 rows up).
+  bool coop_needs_unit_stride = false;
 };
 
 // Returns false and sets *err on unsupported graphs (never falls back to a
@@ -122,6 +129,8 @@ class Emitter {
   // Replaces the serial loop of a REDUCE node by caller-generated code; the
   // callback receives the scope the value is placed in and returns its C name.
   void custom_reduce(int node, std::function<std::string(Scope *)> fn) { custom_[node] = std::move(fn); }
+  // The serial loop of REDUCE `node` takes range `ord` from `first` in steps of `step`.
+  void slice_reduce(int node, int ord, const std::string &first, int step) { slice_node_ = node; slice_ord_ = ord; slice_first_ = first; slice_step_ = step; }
   bool has_custom(int node) const { return custom_.count(node) != 0; }
   void stmt(Scope *s, const std::string &line);
   std::string emit(int node, Scope *s);
@@ -155,6 +164,8 @@ class Emitter {
   std::unordered_map<int, std::string> range_name_;
   std::unordered_map<int, std::string> preset_;
   std::unordered_map<int, std::function<std::string(Scope *)>> custom_;
+  int slice_node_ = -1, slice_ord_ = -1, slice_step_ = 1;
+  std::string slice_first_;
   std::string error_;
 };
 

@@ -92,19 +92,29 @@ def _arg_types(source, entry):
     return [p.rsplit(" ", 1)[0].replace("__restrict__", "").strip() for p in params]
 
 
+def _arg_names(source, entry):
+    head = source[source.index(" " + entry + "(") + len(entry) + 2:]
+    text = head[:head.index(")")].strip()
+    if text == "POLY_SIGNATURE":
+        text = [ln for ln in source.splitlines() if ln.startswith("#define POLY_SIGNATURE ")][0][len("#define POLY_SIGNATURE "):]
+    return [p.strip().rsplit(" ", 1)[-1].lstrip("*") for p in text.split(",")]
+
+
 def _entry_name(source):
     line = [ln for ln in source.splitlines() if ln.startswith('extern "C" __global__')][-1]
     return [m for m in re.findall(r"(\w+)\s*\(", line) if m.startswith("poly_")][-1]
 
 
-def check_kernel(source, entry, grid, block, buf_sizes, block_stride=1, timeout=600):
+def check_kernel(source, entry, grid, block, buf_sizes, block_stride=1, timeout=600, scratch_bytes=0):
     """Compiles `source` for the host and runs kernel `entry` over its whole launch (or
     every `block_stride`-th workgroup along x) with exact-size buffers.  Raises with the
     sanitizer's report on an out-of-bounds access."""
     types = _arg_types(source, entry)
     assert len(types) >= len(buf_sizes), (entry, types, buf_sizes)
     # what follows the buffers: DEFINE_VAR ints (passed as 0) and lookup tables (65536 entries of at most 4 bytes)
-    buf_sizes = list(buf_sizes) + [65536 * 4 for t in types[len(buf_sizes):] if "*" in t]
+    names = _arg_names(source, entry)
+    buf_sizes = list(buf_sizes) + [scratch_bytes if names[i] == "poly_scratch" else 65536 * 4
+                                   for i, t in enumerate(types) if i >= len(buf_sizes) and "*" in t]
     args = ", ".join(f"({t})bufs[{i}]" if "*" in t else "0" for i, t in enumerate(types))
     tail = (DRIVER_TAIL.replace("GX", str(grid[0])).replace("GY", str(grid[1])).replace("GZ", str(grid[2]))
             .replace("BX", str(block)).replace("NBUF", str(len(buf_sizes))).replace("STRIDE", str(block_stride))
@@ -140,11 +150,13 @@ def _jobs(lib, schedule, max_threads, only, groups):
             continue
         seen.add((main, sizes))
         grid = (launch[0], launch[1], launch[2])
-        yield f"step {step}", main, grid, launch[3], sizes
+        scratch = 0
         for unit in text.split("\n// ---- ")[1:]:
-            m = re.match(r"terms ---- grid=(\d+) block=(\d+)\n", unit)
+            m = re.match(r"terms ---- grid=(\d+) block=(\d+) scratch=(\d+)\n", unit)
             if m:       # first stage of a two-stage reduction: same arguments plus the scratch, its own launch
-                yield f"step {step} (terms)", unit[m.end():], (int(m.group(1)), 1, 1), int(m.group(2)), sizes
+                scratch = int(m.group(3))
+                yield f"step {step} (terms)", unit[m.end():], (int(m.group(1)), 1, 1), int(m.group(2)), sizes, scratch
+        yield f"step {step}", main, grid, launch[3], sizes, scratch
     if not groups or only is not None:
         return
     for gi in range(lib.poly_hip_fused_groups(schedule, -1, None, None)):
@@ -159,7 +171,7 @@ def _jobs(lib, schedule, max_threads, only, groups):
         if (main, sizes) in seen:
             continue
         seen.add((main, sizes))
-        yield f"group {gi}", main, (launch[0], launch[1], launch[2]), launch[3], sizes
+        yield f"group {gi}", main, (launch[0], launch[1], launch[2]), launch[3], sizes, 0
 
 
 def check_schedule(lib, schedule, max_threads=1 << 21, only=None, groups=True, workers=6):
@@ -170,10 +182,10 @@ def check_schedule(lib, schedule, max_threads=1 << 21, only=None, groups=True, w
     from concurrent.futures import ThreadPoolExecutor
 
     def one(job):
-        what, main, grid, block, sizes = job
+        what, main, grid, block, sizes, scratch = job
         threads = grid[0] * grid[1] * grid[2] * block
         try:
-            check_kernel(main, _entry_name(main), grid, block, sizes, block_stride=max(1, threads // max_threads))
+            check_kernel(main, _entry_name(main), grid, block, sizes, block_stride=max(1, threads // max_threads), scratch_bytes=scratch)
         except Exception as e:
             raise AssertionError(f"{what}: {e}") from e
         return 1

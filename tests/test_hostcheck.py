@@ -18,7 +18,7 @@ pytestmark = pytest.mark.skipif(not os.path.exists(hostcheck.CLANG), reason="no 
 def test_checker_sees_an_overrun(hiplib):
     fx = F.Fixture("bf16_matmul")
     jobs = list(hostcheck._jobs(hiplib, fx.plan.schedule, 1 << 21, None, False))
-    what, main, grid, block, sizes = jobs[0]
+    what, main, grid, block, sizes, _ = jobs[0]
     hostcheck.check_kernel(main, hostcheck._entry_name(main), grid, block, sizes)
     with pytest.raises(AssertionError, match="out-of-bounds"):
         hostcheck.check_kernel(main, hostcheck._entry_name(main), grid, block, [sizes[0] // 2] + list(sizes[1:]))
@@ -49,3 +49,14 @@ def test_training_step_kernels_stay_in_bounds(B, T, D, H, V, hiplib):
         c.L.poly_schedule_free(sched)
         c.close()
     assert n > 60
+
+
+@pytest.mark.parametrize("name", ["mlp_train_f32_b4096", "gpt2_small_bf16_b1_t1024", "attention_bf16_b8_h12_t1024_d64",
+                                  "matmul_bf16_b16_1024x1024x1024", "rowops_f32_8192_softmax"])
+def test_benchmark_plan_kernels_stay_in_bounds(name, hiplib):
+    """The benchmark plans at their real shapes (large launches sampled by workgroup):
+    MFMA templates, the fused attention kernel, matmul epilogues, row chains, the two-stage
+    reductions of the MLP step."""
+    from polygrad_amd import PlanFile
+    pf = PlanFile(os.path.join(os.path.dirname(os.path.abspath(__file__)), "..", "polygrad_amd", "plans", name + ".polyplan"))
+    assert hostcheck.check_schedule(hiplib, pf.schedule) >= 1
