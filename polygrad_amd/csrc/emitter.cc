@@ -272,6 +272,14 @@ std::string Emitter::emit_reduce_serial(int id, Scope *t) {
     closes.append((size_t)(t->indent + (int)i - 1) * 2, ' ');
     closes += "}\n";
   }
+  if (k.guard >= 0) {
+    // only the taken branch of the WHERE above needs the sum
+    std::string g = emit(k.guard, t);
+    if (k.guard_neg) g = "(!" + g + ")";
+    std::string pad((size_t)t->indent * 2, ' ');
+    opens = pad + "if (" + g + ") {\n" + opens;
+    closes += pad + "}\n";
+  }
   t->code += opens + inner.code + closes;
   return acc;
 }

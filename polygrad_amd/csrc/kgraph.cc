@@ -361,6 +361,9 @@ bool KernelGraph::build(const PolyUOp *root) {
       if (nodes[(size_t)n].op == POLY_OP_CAST && nodes[(size_t)n].n_uses == 1) n = nodes[(size_t)n].src[0];
       KNode &ld = nodes[(size_t)n];
       if (ld.op == POLY_OP_LOAD && ld.n_uses == 1 && ld.guard < 0) { ld.guard = w.src[0]; ld.guard_neg = (b == 2); }
+      // a reduction that only this branch uses need not run where the branch is not taken
+      // (the derivative of a concatenation: each output position takes one of several sums)
+      if (ld.op == POLY_OP_REDUCE && ld.n_uses == 1 && ld.guard < 0) { ld.guard = w.src[0]; ld.guard_neg = (b == 2); }
     }
   }
 

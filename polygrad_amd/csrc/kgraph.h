@@ -47,6 +47,8 @@ struct KNode {
   // LOADs whose only consumer is one branch of WHERE(cond, ., .) are predicated
   // on that condition, as the reference folds them into gated loads
   // (cond ? *p : 0); their index may be out of bounds when cond is false.
+  // A REDUCE in that position carries the condition too: its serial loop is skipped
+  // where the branch is not taken.
   int guard = -1;
   bool guard_neg = false;
 };
