@@ -42,9 +42,10 @@ static void name_kernel(RenderedKernel *rk) {
     rename(rk->fallback_source, " poly_k(", " " + name + "_slow(");
     rk->fallback_entry = name + "_slow";
   }
-  if (!rk->pre_source.empty()) {
-    rename(rk->pre_source, " poly_k(", " " + name + "_terms(");
-    rk->pre_entry = name + "_terms";
+  for (size_t i = 0; i < rk->pres.size(); i++) {
+    const std::string pn = name + (i == 0 ? "_pre" : strf("_pre%zu", i + 1));
+    rename(rk->pres[i].source, " poly_k(", " " + pn + "(");
+    rk->pres[i].entry = pn;
   }
 }
 
@@ -86,11 +87,15 @@ HipRunner *runner_from_rendered(const RenderedKernel &rk, const char *fn_name, b
     r->fallback = program_create(r->rk.fallback_source, r->rk.fallback_entry);
     if (!r->fallback) { runner_destroy(r); return nullptr; }
   }
-  if (!r->rk.pre_source.empty()) {
+  if (!r->rk.pres.empty()) {
     if (!r->rk.guards.empty()) { log_err("lower", "%s: a two-stage kernel cannot also be guarded", r->name.c_str()); runner_destroy(r); return nullptr; }
-    r->pre = program_create(r->rk.pre_source, r->rk.pre_entry);
+    for (const RenderedKernel::Pre &pk : r->rk.pres) {
+      Program *p = program_create(pk.source, pk.entry);
+      if (!p) { runner_destroy(r); return nullptr; }
+      r->pres.push_back(p);
+    }
     r->scratch = runtime_alloc(r->rk.scratch_bytes);
-    if (!r->pre || !r->scratch) { runner_destroy(r); return nullptr; }
+    if (!r->scratch) { runner_destroy(r); return nullptr; }
   }
   for (const RenderedKernel::Table &t : r->rk.tables) {
     std::shared_ptr<void> tab = runtime_table(t.source, t.entry, t.bytes, t.launch);
@@ -128,7 +133,7 @@ void runner_destroy(HipRunner *r) {
   if (r->main) program_destroy(r->main);
   for (Program *p : r->guards) program_destroy(p);
   if (r->fallback) program_destroy(r->fallback);
-  if (r->pre) program_destroy(r->pre);
+  for (Program *p : r->pres) program_destroy(p);
   if (r->scratch) runtime_free(r->scratch);
   if (r->flag) runtime_free(r->flag);
   delete r;
@@ -156,10 +161,11 @@ int runner_launch(HipRunner *r, void **args, int n_args) {
     r->ptr_store[(size_t)(np + nv + t)] = r->tables[(size_t)t].get();
     r->arg_ptrs[(size_t)(np + nv + t)] = &r->ptr_store[(size_t)(np + nv + t)];
   }
-  if (r->pre) {
+  if (!r->pres.empty()) {
     r->ptr_store[(size_t)(np + nv + nt)] = r->scratch;
     r->arg_ptrs[(size_t)(np + nv + nt)] = &r->ptr_store[(size_t)(np + nv + nt)];
-    if (program_launch(r->pre, r->arg_ptrs.data(), r->rk.pre_launch) != 0) return -1;
+    for (size_t i = 0; i < r->pres.size(); i++)
+      if (program_launch(r->pres[i], r->arg_ptrs.data(), r->rk.pres[i].launch) != 0) return -1;
     return program_launch(r->main, r->arg_ptrs.data(), r->rk.launch);
   }
   if (r->guards.empty()) return program_launch(r->main, r->arg_ptrs.data(), r->rk.launch);
@@ -283,8 +289,8 @@ char *poly_hip_render(PolyUOp *scheduled_root, const char *fn_name, int flags, i
   std::string all = rk.source;
   for (const RenderedKernel::Guard &g : rk.guards) all += "\n// ---- guard ----\n" + g.source;
   if (!rk.fallback_source.empty()) all += "\n// ---- fallback ----\n" + rk.fallback_source;
-  if (!rk.pre_source.empty())
-    all += strf("\n// ---- terms ---- grid=%u block=%u scratch=%zu\n", rk.pre_launch.grid[0], rk.pre_launch.block[0], rk.scratch_bytes) + rk.pre_source;
+  for (const RenderedKernel::Pre &pk : rk.pres)
+    all += strf("\n// ---- first stage ---- grid=%u,%u block=%u scratch=%zu\n", pk.launch.grid[0], pk.launch.grid[1], pk.launch.block[0], rk.scratch_bytes) + pk.source;
   for (size_t i = 1; i < rk.variants.size(); i++) all += "\n// ---- variant " + rk.variants[i].label + "\n" + rk.variants[i].source;
   return dup_string(all);
 }

@@ -822,9 +822,7 @@ static bool split_in_two(const KernelGraph &g, const std::string &fn_name, const
   };
   Generic gen2(g, fn_name, o2);
   if (!gen2.run(out, &err) || out->klass == KernelClass::ROW_REDUCE) return false;
-  out->pre_source = pre.source;
-  out->pre_entry = pre.entry;
-  out->pre_launch = pre.launch;
+  out->pres.push_back({pre.source, pre.entry, pre.launch});
   out->scratch_bytes = (size_t)(rows * rt) * sizeof(float);
   out->klass = KernelClass::ROW_REDUCE;
   out->strategy = "two stages: " + pre.strategy + " into scratch, then " + out->strategy;

@@ -64,11 +64,15 @@ struct RenderedKernel {
     LaunchSpec launch;
   };
   std::vector<Variant> variants;
-  // Two-stage reductions: `pre_source` runs first, with the same arguments plus one more
+  // Kernels in two stages (reductions through partial results, matmuls whose operands are
+  // prepared first): `pres` run first, in order, with the same arguments plus one more
   // pointer to `scratch_bytes` bytes of device memory that the runner owns; the main
   // kernel takes that pointer too (after the variables and tables).
-  std::string pre_source, pre_entry;
-  LaunchSpec pre_launch;
+  struct Pre {
+    std::string source, entry;
+    LaunchSpec launch;
+  };
+  std::vector<Pre> pres;
   size_t scratch_bytes = 0;
 };
 

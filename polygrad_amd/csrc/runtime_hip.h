@@ -36,8 +36,8 @@ struct HipRunner {
   Program *main = nullptr;
   std::vector<Program *> guards;
   Program *fallback = nullptr;
-  Program *pre = nullptr;          // first stage of a two-stage reduction
-  void *scratch = nullptr;         // its terms, read by the main kernel
+  std::vector<Program *> pres;     // first stage(s) of a two-stage kernel
+  void *scratch = nullptr;         // what they leave for the main kernel
   void *flag = nullptr;            // device int written by the guards
   std::vector<std::shared_ptr<void>> tables;   // filled lookup tables (shared between identical kernels)
   std::string name;

@@ -20,6 +20,9 @@ const char *const kMatmulTemplate =
 const char *const kMatmulF32Template =
 #include "matmul_f32_mfma.hip.inc"
     ;
+const char *const kOperandSplitTemplate =
+#include "operand_split.hip.inc"
+    ;
 
 PolyOps reduce_op(const KNode &k) {
   return k.u->arg.kind == POLY_ARG_OPS ? k.u->arg.ops : (PolyOps)k.u->arg.i;
@@ -791,6 +794,74 @@ bool try_render_matmul_generic(const KernelGraph &g, const std::string &fn, cons
       code += strf("__device__ __forceinline__ float poly_%s_math(int %s, int k, int z, const unsigned int (&raw)[%d], %s) {\n", nm, rowvar, nraw,
                    ep.signature.c_str());
       code += head + S.code + strf("  return %s;\n}\n", v.c_str());
+    }
+  }
+
+  // ── on the bf16 MFMA when the products allow it ───────────────────────────────
+  // An operand that is a bf16 value cast to fp32 is exact in bf16; an fp32-valued one is the
+  // sum of three bf16 pieces (kernels/operand_split.hip).  With at least one exact side,
+  // a first stage writes both operands as k-contiguous bf16 planes into scratch memory and
+  // the 16-bit template multiplies them (K' = planes x K rounded up to its K tile).
+  {
+    auto exact16 = [&](int node) {
+      const KNode &k = g.n(node);
+      return k.op == POLY_OP_CAST && k.dt == DT_F32 && g.n(k.src[0]).dt == DT_BF16;
+    };
+    const int parts[2] = {exact16(opnd[0]) ? 1 : 3, exact16(opnd[1]) ? 1 : 3};
+    const int P = std::max(parts[0], parts[1]);
+    const int64_t KP = (K + 63) / 64 * 64;
+    const double elems_a = (double)Z * (double)M * parts[0] * (double)KP, elems_b = (double)Z * (double)N * parts[1] * (double)KP;
+    const bool fits = elems_a < 2147483647.0 && elems_b < 2147483647.0;
+    // worth the extra pass over the operands only for deep or large products
+    const bool large = (double)M * (double)N * (double)K * (double)Z >= 1073741824.0;
+    if (!getenv("POLY_HIP_NO_BF16_SPLIT") && parts[0] + parts[1] <= 4 && fits && large) {
+      const size_t off_b = ((size_t)elems_a * 2 + 255) / 256 * 256;       // bytes
+      const size_t scratch_bytes = off_b + (size_t)elems_b * 2;
+      RenderedKernel::Pre pre[2];
+      for (int side = 0; side < 2; side++) {
+        const char *nm = side == 0 ? "a" : "b";
+        const int64_t rows = side == 0 ? M : N;
+        std::string c2;
+        c2 += strf("#define POLY_SP_ROWS %lld\n#define POLY_SP_K %lld\n#define POLY_SP_KP %lld\n#define POLY_SP_Z %lld\n", (long long)rows, (long long)K,
+                   (long long)KP, (long long)Z);
+        c2 += strf("#define POLY_SP_PARTS %d\n#define POLY_SP_WALK_K %d\n#define POLY_SP_NRAW %d\n", parts[side], walk_k[side] ? 1 : 0, std::max(1, n_loads[side]));
+        c2 += strf("#define POLY_SIGNATURE %s, __bf16* poly_scratch\n", ep.signature.c_str());
+        c2 += code;
+        c2 += strf("#define POLY_SP_LOAD(row, k, z, raw) poly_%s_load(row, k, z, raw, %s)\n#define POLY_SP_MATH(row, k, z, raw) poly_%s_math(row, k, z, raw, %s)\n",
+                   nm, params_call.c_str(), nm, params_call.c_str());
+        c2 += strf("#define POLY_SP_OUT ((__bf16*)((char*)poly_scratch + %zuull))\n", side == 0 ? (size_t)0 : off_b);
+        pre[side].source = std::string(hip_prelude()) + c2 + kOperandSplitTemplate;
+        pre[side].entry = "poly_k";
+        pre[side].launch.grid[0] = (unsigned)((KP / 64) * ((rows + 63) / 64));
+        pre[side].launch.grid[1] = (unsigned)Z;
+        pre[side].launch.block[0] = 256;
+      }
+      // the product of the planes, as the 16-bit template sees it
+      MatmulMatch m2;
+      m2.red = red; m2.K = P * KP; m2.M = M; m2.N = N; m2.Z = Z;
+      m2.A.dt = m2.B.dt = DT_BF16;
+      m2.ka = parts[0] == P ? KSplit{P * KP, 0, 1} : KSplit{KP, 0, 1};
+      m2.kb = parts[1] == P ? KSplit{P * KP, 0, 1} : KSplit{KP, 0, 1};
+      m2.md.push_back(Dim{-1, M, parts[0] * KP, 0, 1});
+      m2.nd.push_back(Dim{-1, N, 0, parts[1] * KP, 1});
+      if (Z > 1) m2.zd.push_back(Dim{-1, Z, M * parts[0] * KP, N * parts[1] * KP, 1});
+      m2.md_full = mm.md_full; m2.nd_full = mm.nd_full; m2.zd_full = mm.zd_full;
+      MatmulEpilogue ep2 = ep;
+      ep2.signature += ", __bf16* poly_scratch";
+      ep2.a_ptr = "((const __bf16*)poly_scratch)";
+      ep2.b_ptr = strf("((const __bf16*)((const char*)poly_scratch + %zuull))", off_b);
+      RenderedKernel main;
+      if (render_matmul(m2, ep2, &main)) {
+        *out = main;
+        out->pres.push_back(pre[0]);
+        out->pres.push_back(pre[1]);
+        out->scratch_bytes = scratch_bytes;
+        out->flops = 2.0 * (double)M * (double)N * (double)K * (double)Z;
+        out->strategy = strf("operands as expressions, written as bf16 planes first (%d + %d planes of K=%lld, %.0f MB): ", parts[0], parts[1],
+                             (long long)KP, (double)scratch_bytes / 1e6) + out->strategy;
+        for (RenderedKernel::Variant &v : out->variants) v.strategy = out->strategy;
+        return true;
+      }
     }
   }
 

@@ -152,10 +152,10 @@ def _jobs(lib, schedule, max_threads, only, groups):
         grid = (launch[0], launch[1], launch[2])
         scratch = 0
         for unit in text.split("\n// ---- ")[1:]:
-            m = re.match(r"terms ---- grid=(\d+) block=(\d+) scratch=(\d+)\n", unit)
-            if m:       # first stage of a two-stage reduction: same arguments plus the scratch, its own launch
-                scratch = int(m.group(3))
-                yield f"step {step} (terms)", unit[m.end():], (int(m.group(1)), 1, 1), int(m.group(2)), sizes, scratch
+            m = re.match(r"first stage ---- grid=(\d+),(\d+) block=(\d+) scratch=(\d+)\n", unit)
+            if m:       # first stage of a two-stage kernel: same arguments plus the scratch, its own launch
+                scratch = int(m.group(4))
+                yield f"step {step} (first stage)", unit[m.end():], (int(m.group(1)), int(m.group(2)), 1), int(m.group(3)), sizes, scratch
         yield f"step {step}", main, grid, launch[3], sizes, scratch
     if not groups or only is not None:
         return

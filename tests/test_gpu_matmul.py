@@ -155,3 +155,45 @@ def test_matmul_of_computed_operands():
     c.close()
     assert any("operands as expressions" in k["desc"] for k in info), [k["desc"] for k in info]
     assert_close(got[O], want[O], rtol=1e-4, atol=1e-4 * float(np.abs(want[O]).mean()), what="weight gradient over two ranges")
+
+
+def _planes_case(c, g):
+    """fp32 x bf16 with a ragged depth, large enough (2^30 multiply-adds) for the operands
+    to be written as bf16 planes and multiplied on the bf16 MFMA."""
+    M, N, K = 512, 512, 4100
+    A = c.buffer((M, K), R.F32, name="A")
+    Bm = c.buffer((K, N), R.BF16, name="B")
+    O = c.buffer((M, N), R.F32, name="C")
+    sink = c.sink((O, (A * c.const(1.5)).dot(Bm.cast(R.F32))))
+    a = g.normal(0, 1, (M, K)).astype(np.float32)
+    a[0, :8] = [1e-30, -3e30, 1.0 + 2.0 ** -20, 65504.0, 2.0 ** -126, 0.0, -0.0, 1e10]      # pieces at the edges of the exponent range
+    arrays = {A: a, Bm: bf16(g, (K, N), 1.0), O: np.zeros((M, N), np.float32)}
+    return sink, arrays, O
+
+
+def test_matmul_of_fp32_operand_as_three_bf16_planes():
+    """An fp32 operand is the sum of three bf16 pieces and a bf16 x bf16 product is exact
+    in fp32, so the product runs on the bf16 MFMA over three K-long planes written by a
+    first-stage kernel.  Held to the fp32 reduction tolerance against the reference, and
+    compared with the fp32 MFMA path of the same kernel (POLY_HIP_NO_BF16_SPLIT)."""
+    import os
+    g = np.random.default_rng(22)
+    c = R.Ctx()
+    sink, arrays, O = _planes_case(c, g)
+    want = run_ref(c, sink, arrays)
+    got, info = run_hip(c, sink, arrays)
+    assert any("bf16 planes" in k["desc"] for k in info), [k["desc"] for k in info]
+    os.environ["POLY_HIP_NO_BF16_SPLIT"] = "1"
+    try:
+        got32, info32 = run_hip(c, sink, arrays)
+    finally:
+        del os.environ["POLY_HIP_NO_BF16_SPLIT"]
+    c.close()
+    assert any("mfma 32x32x2 f32, operands as expressions" in k["desc"] for k in info32), [k["desc"] for k in info32]
+    w = want[O].astype(np.float64)
+    # scale of the rounding error of any summation order: sum of |terms| ~ K * E|a| * E|b|
+    bound = 1e-4 * float(np.abs(w).mean()) * 8
+    assert_close(got[O], want[O], rtol=1e-4, atol=bound, what="three bf16 planes vs reference")
+    assert_close(got32[O], want[O], rtol=1e-4, atol=bound, what="fp32 MFMA vs reference")
+    # the two device paths agree far more closely than either needs to
+    assert float(np.abs(got[O].astype(np.float64) - got32[O]).max()) <= 2e-5 * float(np.abs(w).max())
