@@ -241,6 +241,32 @@ std::string Emitter::load_expr(int id, Scope *s) {
   return e;
 }
 
+// Is the part of `root` that changes with range `ord` small enough to unroll: a few loads
+// whose indices need no division or modulus per iteration?
+bool Emitter::light_body(int root, int ord) const {
+  std::vector<char> mark(g_.nodes.size(), 0);
+  mark_reachable(g_, root, mark);
+  const uint64_t bit = (uint64_t)1 << ord;
+  int loads = 0, divmods = 0, ops = 0;
+  for (size_t id = 0; id < g_.nodes.size(); id++) {
+    if (!mark[id] || !(g_.n((int)id).deps & bit)) continue;
+    const KNode &n = g_.n((int)id);
+    if (n.op == POLY_OP_REDUCE) return false;
+    if (n.op == POLY_OP_LOAD) {
+      loads++;
+      const int li = g_.n(g_.n(n.src[0]).src[1]).lin;
+      if (li < 0) return false;
+      for (const Term &t : g_.lins[(size_t)li].terms) {
+        const Atom &a = g_.atoms[(size_t)t.atom];
+        if ((a.kind == Atom::DIV || a.kind == Atom::MOD) && (g_.atom_deps(t.atom) & bit)) divmods++;
+      }
+    } else if (n.lin < 0 && n.op != POLY_OP_INDEX && n.op != POLY_OP_RANGE) {
+      ops++;
+    }
+  }
+  return loads <= 4 && divmods == 0 && ops <= 16;
+}
+
 std::string Emitter::emit_reduce_serial(int id, Scope *t) {
   const KNode &k = g_.n(id);
   PolyOps rop = k.u->arg.kind == POLY_ARG_OPS ? k.u->arg.ops : (PolyOps)k.u->arg.i;
@@ -256,6 +282,11 @@ std::string Emitter::emit_reduce_serial(int id, Scope *t) {
     const RangeInfo &r = g_.ranges[(size_t)ord];
     std::string rv = strf("r%d", ord);
     std::string bound = r.extent >= 0 ? strf("%lld", (long long)r.extent) : emit(r.bound_node, t);
+    // the innermost loop: several iterations' loads in flight (same order of additions)
+    if (i + 1 == k.src.size() && (r.extent < 0 || r.extent >= 64) && light_body(k.src[0], ord)) {
+      opens.append((size_t)inner.indent * 2, ' ');
+      opens += "#pragma unroll 8\n";
+    }
     opens.append((size_t)inner.indent * 2, ' ');
     if (id == slice_node_ && ord == slice_ord_)
       opens += strf("for (int %s = %s; %s < %s; %s += %d) {\n", rv.c_str(), slice_first_.c_str(), rv.c_str(), bound.c_str(), rv.c_str(), slice_step_);

@@ -162,6 +162,7 @@ class Emitter {
 
  private:
   std::string emit_atom(int atom, Scope *s);
+  bool light_body(int root, int ord) const;
   std::string emit_raw(int node, Scope *s);
   Scope *place(uint64_t deps, Scope *s);
   const KernelGraph &g_;
