@@ -21,6 +21,10 @@
 //                       Fetches run ahead in the register ring like the plain loads; the
 //                       arithmetic happens on the way to LDS.
 //   POLY_PF_DEPTH       K tiles the global loads run ahead (default 4)
+//   POLY_KSPLIT         S > 1: the K tiles are dealt to S workgroups per output tile
+//                       (blockIdx.y = z * S + s; S divides the number of K tiles) and the
+//                       accumulators go to poly_scratch[s][z][m][n] (fp32) for a second
+//                       kernel to add up and finish; for deep products with few tiles
 //
 // Data path: global --16B loads, four K tiles ahead--> registers --> LDS [row][16 k]
 // (rows padded to 20 floats: 16-byte fragment reads of 16 consecutive rows then fall on
@@ -70,7 +74,10 @@ typedef float pf_acc16 __attribute__((ext_vector_type(16)));
 #ifndef POLY_PF_DEPTH
 #define POLY_PF_DEPTH 4
 #endif
-#define PF_KT ((POLY_K + PF_BK - 1) / PF_BK)
+#ifndef POLY_KSPLIT
+#define POLY_KSPLIT 1
+#endif
+#define PF_KT (((POLY_K + PF_BK - 1) / PF_BK) / POLY_KSPLIT)
 
 // Staging of one operand tile (ROWS x 16 floats): 16-byte pieces, ROWS * 4 of them.
 template <int ROWS, bool KC>
@@ -132,7 +139,8 @@ extern "C" __global__ void __launch_bounds__(PF_NTHREADS) poly_k(POLY_SIGNATURE)
     tile_m = first_m + in_group % gsz;
     tile_n = in_group / gsz;
   }
-  const int z = blockIdx.y;
+  const int z = blockIdx.y / POLY_KSPLIT;
+  const int kt_base = (blockIdx.y % POLY_KSPLIT) * PF_KT;      // first K tile of this workgroup's share
   const int m0 = tile_m * POLY_BM, n0 = tile_n * POLY_BN;
   typedef PfStage<POLY_BM, POLY_A_KC != 0> StageA;
   typedef PfStage<POLY_BN, POLY_B_KC != 0> StageB;
@@ -146,12 +154,12 @@ extern "C" __global__ void __launch_bounds__(PF_NTHREADS) poly_k(POLY_SIGNATURE)
   auto a_coord = [&](int kt, int i, int e, int *m, int *k) {
     const int row = m0 + StageA::row_of(i) + (POLY_A_KC ? 0 : e);
     *m = row < POLY_M ? row : POLY_M - 1;
-    *k = kt * PF_BK + StageA::k_of(i) + (POLY_A_KC ? e : 0);
+    *k = (kt_base + kt) * PF_BK + StageA::k_of(i) + (POLY_A_KC ? e : 0);
   };
   auto b_coord = [&](int kt, int i, int e, int *n, int *k) {
     const int row = n0 + StageB::row_of(i) + (POLY_B_KC ? 0 : e);
     *n = row < POLY_N ? row : POLY_N - 1;
-    *k = kt * PF_BK + StageB::k_of(i) + (POLY_B_KC ? e : 0);
+    *k = (kt_base + kt) * PF_BK + StageB::k_of(i) + (POLY_B_KC ? e : 0);
   };
   auto load_tiles = [&](int kt, int set) {
 #pragma unroll
@@ -222,7 +230,7 @@ extern "C" __global__ void __launch_bounds__(PF_NTHREADS) poly_k(POLY_SIGNATURE)
     b_off[i] = poly_b_row(POLY_B_KC ? (row < POLY_N ? row : POLY_N - 1) : (row + 3 < POLY_N ? row : POLY_N - 4));
   }
   auto load_tiles = [&](int kt, int set) {
-    const int k0 = kt * PF_BK;
+    const int k0 = (kt_base + kt) * PF_BK;
 #pragma unroll
     for (int i = 0; i < StageA::NL; i++)
       if (StageA::active(i)) ra[set][i] = *(const pf_f32x4_u *)(gA + a_off[i] + poly_a_k(k0 + StageA::k_of(i)));
@@ -295,7 +303,12 @@ extern "C" __global__ void __launch_bounds__(PF_NTHREADS) poly_k(POLY_SIGNATURE)
 #pragma unroll
       for (int r = 0; r < 16; r++) {
         const int m = m0 + wm + i * 32 + 8 * (r >> 2) + 4 * half + (r & 3);
+#if POLY_KSPLIT > 1
+        if (m < POLY_M && n < POLY_N)
+          poly_scratch[(((size_t)(blockIdx.y % POLY_KSPLIT) * POLY_Z + z) * POLY_M + m) * POLY_N + n] = acc[i][j][r];
+#else
         if (m < POLY_M && n < POLY_N) { POLY_EPILOGUE(acc[i][j][r], m, n, z); }
+#endif
       }
     }
 }

@@ -364,6 +364,33 @@ bool try_render_matmul(const KernelGraph &g, const std::string &fn, const Render
   return render_matmul(mm, ep, out);
 }
 
+// Second stage of a split-K product: adds the S partial accumulators of an output element
+// in split order and finishes the element with the kernel's epilogue.
+static const char *const kSplitKCombine = R"HIP(
+extern "C" __global__ void __launch_bounds__(256) poly_k(POLY_SIGNATURE) {
+  const long long gid = (long long)blockIdx.x * 256 + threadIdx.x;
+  if (gid >= (long long)POLY_Z * POLY_M * POLY_N) return;
+  const int n = (int)(gid % POLY_N), m = (int)((gid / POLY_N) % POLY_M), z = (int)(gid / ((long long)POLY_N * POLY_M));
+  float acc = poly_scratch[gid];
+#pragma unroll
+  for (int s = 1; s < POLY_KSPLIT; s++) acc += poly_scratch[(size_t)s * POLY_Z * POLY_M * POLY_N + gid];
+  POLY_EPILOGUE(acc, m, n, z);
+}
+)HIP";
+
+// How many workgroups should share the K tiles of one output tile: enough to give every CU
+// work when the product has few tiles and a deep K; 1 = no split.  S divides `k_tiles`.
+static int ksplit_for(int64_t tiles, int64_t k_tiles, int64_t min_tiles_per_split) {
+  if (getenv("POLY_HIP_NO_SPLIT_K") || tiles >= 128) return 1;
+  int best = 1;
+  for (int s = 2; s <= 16; s++) {
+    if (k_tiles % s != 0 || k_tiles / s < min_tiles_per_split) continue;
+    if (tiles * s > 640) break;
+    best = s;
+  }
+  return best;
+}
+
 // Tile of the fp32 template: 4 waves; narrow outputs get a narrow tile.
 static void f32_tile(int64_t M, int64_t N, int64_t Z, int *bm, int *bn, int *wvm, int *wvn) {
   int BM = 128, BN = 128, WVM = 2, WVN = 2;
@@ -395,6 +422,14 @@ static bool render_matmul_f32(const MatmulMatch &mm, const MatmulEpilogue &ep, R
   if (!layout(mm.ka, mm.md, true, M, &a_kc) || !layout(mm.kb, mm.nd, false, N, &b_kc)) return reject(__LINE__);
   int BM, BN, WVM, WVN;
   f32_tile(M, N, Z, &BM, &BN, &WVM, &WVN);
+  // deep product on few tiles: larger tiles, K dealt to several workgroups each
+  int S = 1;
+  if (M > 64 && N > 64 && K >= 2048) {
+    const int64_t t128 = ((M + 127) / 128) * ((N + 127) / 128) * Z, t64 = ((M + 63) / 64) * ((N + 63) / 64) * Z;
+    const int s128 = ksplit_for(t128, K / 16, 32), s64 = ksplit_for(t64, K / 16, 32);
+    if (s128 > 1 && t128 * s128 >= 128) { BM = BN = 128; WVM = WVN = 2; S = s128; }
+    else if (s64 > 1) { BM = BN = 64; WVM = WVN = 2; S = s64; }
+  }
   const int64_t tiles = ((M + BM - 1) / BM) * ((N + BN - 1) / BN);
   if (tiles > 2147483647LL / 2) return reject(__LINE__);
   std::string cfg;
@@ -413,14 +448,15 @@ static bool render_matmul_f32(const MatmulMatch &mm, const MatmulEpilogue &ep, R
   }
   cfg += matmul_k_fn("poly_a_k", mm.ka, K);
   cfg += matmul_k_fn("poly_b_k", mm.kb, K);
-  cfg += strf("#define POLY_SIGNATURE %s\n", ep.signature.c_str());
+  cfg += strf("#define POLY_SIGNATURE %s%s\n", ep.signature.c_str(), S > 1 ? ", float* poly_scratch" : "");
+  cfg += strf("#define POLY_KSPLIT %d\n", S);
   cfg += ep.code;
   cfg += strf("#define POLY_EPILOGUE(acc, m, n, z) %s\n", ep.call.c_str());
   *out = RenderedKernel();
   out->source = std::string(hip_prelude()) + cfg + kMatmulF32Template;
   out->entry = "poly_k";
   out->launch.grid[0] = (unsigned)tiles;
-  out->launch.grid[1] = (unsigned)Z;
+  out->launch.grid[1] = (unsigned)(Z * S);
   out->launch.block[0] = (unsigned)(64 * WVM * WVN);
   out->klass = KernelClass::MATMUL_MFMA;
   out->strategy = strf("mfma 32x32x2 f32 M=%lld N=%lld K=%lld Z=%lld tile %dx%dx16 A:%s B:%s", (long long)M, (long long)N, (long long)K,
@@ -429,6 +465,17 @@ static bool render_matmul_f32(const MatmulMatch &mm, const MatmulEpilogue &ep, R
   out->n_vars = 0;
   out->flops = 2.0 * (double)M * (double)N * (double)K * (double)Z;
   out->bytes = ep.bytes;
+  if (S > 1) {
+    // the template becomes the first stage; the kernel proper adds the partial results up
+    RenderedKernel::Pre pre{out->source, out->entry, out->launch};
+    out->pres.push_back(pre);
+    out->scratch_bytes = (size_t)S * (size_t)Z * (size_t)M * (size_t)N * sizeof(float);
+    out->source = std::string(hip_prelude()) + cfg + kSplitKCombine;
+    out->launch = LaunchSpec();
+    out->launch.grid[0] = (unsigned)(((double)Z * M * N + 255) / 256);
+    out->launch.block[0] = 256;
+    out->strategy += strf(", K dealt to %d workgroups per tile, partial results added by a second kernel", S);
+  }
   return true;
 }
 
