@@ -128,13 +128,20 @@ int runner_use_variant(HipRunner *r, int idx) {
   return 0;
 }
 
+void runner_share_scratch(HipRunner *r, void *pool) {
+  if (!r || !pool || r->rk.scratch_bytes == 0) return;
+  if (r->scratch && r->owns_scratch) runtime_free(r->scratch);
+  r->scratch = pool;
+  r->owns_scratch = false;
+}
+
 void runner_destroy(HipRunner *r) {
   if (!r) return;
   if (r->main) program_destroy(r->main);
   for (Program *p : r->guards) program_destroy(p);
   if (r->fallback) program_destroy(r->fallback);
   for (Program *p : r->pres) program_destroy(p);
-  if (r->scratch) runtime_free(r->scratch);
+  if (r->scratch && r->owns_scratch) runtime_free(r->scratch);
   if (r->flag) runtime_free(r->flag);
   delete r;
 }

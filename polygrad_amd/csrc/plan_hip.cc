@@ -68,6 +68,8 @@ struct PolyHipPlan {
   std::vector<char> slot_needs_zero;
   void *arena = nullptr;
   size_t arena_bytes = 0;
+  void *scratch_pool = nullptr;              // shared by the two-stage kernels of the plan (they run one after the other)
+  size_t scratch_bytes = 0;
   std::vector<std::vector<void *>> kargs;    // per unit: args array handed to runner_launch
   std::vector<std::vector<int>> var_vals;    // per unit: storage for var ints
   std::vector<PolyVarBinding> merged;
@@ -84,6 +86,7 @@ struct PolyHipPlan {
     for (Unit &u : units) runner_destroy(u.runner);
     if (fill) program_destroy(fill);
     if (arena) runtime_free(arena);
+    if (scratch_pool) runtime_free(scratch_pool);
   }
 };
 
@@ -285,6 +288,17 @@ PolyHipPlan *poly_hip_compile_schedule(PolyCtx *ctx, const PolySchedule *s) {
   if (any_zero) {
     plan->fill = program_create(kFillSrc, "poly_fill0");
     if (!plan->fill) return nullptr;
+  }
+  // one scratch pool for all two-stage kernels: the largest need
+  {
+    int users = 0;
+    for (const Unit &u : plan->units)
+      if (u.runner->rk.scratch_bytes > 0) { users++; plan->scratch_bytes = std::max(plan->scratch_bytes, u.runner->rk.scratch_bytes); }
+    if (users > 1) {
+      plan->scratch_pool = runtime_alloc(plan->scratch_bytes);
+      if (!plan->scratch_pool) return nullptr;
+      for (Unit &u : plan->units) runner_share_scratch(u.runner, plan->scratch_pool);
+    }
   }
   plan->kargs.resize((size_t)n_units);
   plan->var_vals.resize((size_t)n_units);
@@ -602,6 +616,6 @@ void *poly_hip_plan_slot_ptr(const PolyHipPlan *plan, int slot) {
 }
 
 void poly_hip_plan_set_graph(PolyHipPlan *plan, int enabled) { if (plan) plan->use_graph = enabled != 0; }
-size_t poly_hip_plan_workspace_bytes(const PolyHipPlan *plan) { return plan ? plan->arena_bytes : 0; }
+size_t poly_hip_plan_workspace_bytes(const PolyHipPlan *plan) { return plan ? plan->arena_bytes + plan->scratch_bytes : 0; }
 
 }  // extern "C"

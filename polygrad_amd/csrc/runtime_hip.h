@@ -38,6 +38,7 @@ struct HipRunner {
   Program *fallback = nullptr;
   std::vector<Program *> pres;     // first stage(s) of a two-stage kernel
   void *scratch = nullptr;         // what they leave for the main kernel
+  bool owns_scratch = true;        // false: the memory belongs to a pool shared with other runners
   void *flag = nullptr;            // device int written by the guards
   std::vector<std::shared_ptr<void>> tables;   // filled lookup tables (shared between identical kernels)
   std::string name;
@@ -50,6 +51,9 @@ HipRunner *runner_create(const PolyUOp *root, const char *fn_name, int flags);
 // From a kernel rendered elsewhere (fused groups); `named` false: the entry is still the
 // placeholder poly_k and gets its descriptive symbol here.
 HipRunner *runner_from_rendered(const RenderedKernel &rk, const char *fn_name, bool named);
+// Replaces the runner's own scratch memory by `pool` (at least rk.scratch_bytes large, owned
+// by the caller, who runs the runners sharing it one after the other on the stream).
+void runner_share_scratch(HipRunner *r, void *pool);
 int runner_launch(HipRunner *r, void **args, int n_args);
 // Switches the runner to rk.variants[idx] (compiles it if needed); the runner is unchanged
 // when that fails.
