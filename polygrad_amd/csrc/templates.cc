@@ -91,6 +91,11 @@ bool digit_uses(const KernelGraph &g, const Lin &l, int ord, std::vector<DigitUs
       const Atom &d = g.atoms[(size_t)a.inner.terms[0].atom];
       if (d.kind == Atom::DIV && is_range(d.inner)) { uses->push_back({t.coef, d.c, a.c}); continue; }
     }
+    // (r / c1) / c2 = r / (c1 c2) for a non-negative r
+    if (a.kind == Atom::DIV && a.inner.c0 == 0 && a.inner.terms.size() == 1 && a.inner.terms[0].coef == 1) {
+      const Atom &d = g.atoms[(size_t)a.inner.terms[0].atom];
+      if (d.kind == Atom::DIV && is_range(d.inner)) { uses->push_back({t.coef, d.c * a.c, 0}); continue; }
+    }
     return false;
   }
   return true;
