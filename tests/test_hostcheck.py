@@ -60,3 +60,20 @@ def test_benchmark_plan_kernels_stay_in_bounds(name, hiplib):
     from polygrad_amd import PlanFile
     pf = PlanFile(os.path.join(os.path.dirname(os.path.abspath(__file__)), "..", "polygrad_amd", "plans", name + ".polyplan"))
     assert hostcheck.check_schedule(hiplib, pf.schedule) >= 1
+
+
+@pytest.mark.skipif(not R.available(), reason="reference library not built")
+def test_bf16_plane_kernels_stay_in_bounds(hiplib):
+    """The three kernels of a matmul whose fp32 operand is cut into bf16 planes (two
+    first-stage kernels writing the planes, the 16-bit MFMA template reading them), with a
+    depth that is not a multiple of the K tile."""
+    import numpy as np
+    import test_gpu_matmul as T
+    c = R.Ctx()
+    sink, _, _ = T._planes_case(c, np.random.default_rng(0))
+    sched = c.schedule(sink)
+    try:
+        assert hostcheck.check_schedule(hiplib, sched) == 3
+    finally:
+        c.L.poly_schedule_free(sched)
+        c.close()
