@@ -863,7 +863,8 @@ bool try_render_matmul_generic(const KernelGraph &g, const std::string &fn, cons
     const int P = std::max(parts[0], parts[1]);
     const int64_t KP = (K + 63) / 64 * 64;
     const double elems_a = (double)Z * (double)M * parts[0] * (double)KP, elems_b = (double)Z * (double)N * parts[1] * (double)KP;
-    const bool fits = elems_a < 2147483647.0 && elems_b < 2147483647.0;
+    // (int offsets inside the template; and the planes should stay a small part of the card's memory)
+    const bool fits = elems_a < 2147483647.0 && elems_b < 2147483647.0 && (elems_a + elems_b) * 2.0 <= 8.0 * 1073741824.0;
     // worth the extra pass over the operands only for deep or large products
     const bool large = (double)M * (double)N * (double)K * (double)Z >= 1073741824.0;
     if (!getenv("POLY_HIP_NO_BF16_SPLIT") && parts[0] + parts[1] <= 4 && fits && large) {
