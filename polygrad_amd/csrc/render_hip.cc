@@ -130,6 +130,8 @@ class Generic {
     if (n_loop_reduces() > 0 && opt_.allow_coop_reduce && groups_.size() == 1 && opt_.reduce_override.empty()) coop = plan_coop();
     if (coop) {
       body = render_coop(out);
+    } else if (plan_ordered()) {
+      body = render_ordered(out);
     } else {
       body = render_flat(out);
     }
@@ -668,6 +670,140 @@ class Generic {
     out->launch.block[0] = (unsigned)opt_.block;
     out->klass = KernelClass::ROW_REDUCE;
     out->strategy = strf("row-reduce G=%d vec%d R=%lld rows=%.0f", G, V, (long long)coop_R_, rows);
+    return body;
+  }
+
+  // ── ordered reduction with cooperative loads ─────────────────────────────
+  //
+  // A long reduction for a few thousand outputs that must keep its order (a sum that
+  // accumulates in bf16: every partial sum is rounded, so the order is part of the result)
+  // and whose loads are contiguous along the outputs.  One thread per output leaves the
+  // chip idle and waits a full memory latency every few terms.  Here a workgroup owns 64
+  // outputs: all four waves compute terms (wave w the terms w*8 .. w*8+7 of each block of
+  // 32) into LDS, then the first wave adds the 32 terms of its outputs in order.
+  bool plan_ordered() const {
+    if (!opt_.allow_coop_reduce || opt_.promote_reduce >= 0 || opt_.slice_reduce >= 0 || !opt_.reduce_override.empty() ||
+        opt_.exit_if_flag || opt_.exit_unless_flag || getenv("POLY_HIP_NO_ORDERED_REDUCE"))
+      return false;
+    if (groups_.size() != 1 || g_.reduces.size() != 1 || top_reduces_.size() != 1 || !g_.vars.empty()) return false;
+    const KNode &T = g_.n(top_reduces_[0]);
+    const int sz = dt_size(T.dt);
+    if (sz != 2 && sz != 4) return false;
+    int64_t K = 1;
+    for (size_t i = 1; i < T.src.size(); i++) {
+      const int64_t e = g_.ranges[(size_t)g_.range_ord.at(T.src[i])].extent;
+      if (e <= 0) return false;
+      K *= e;
+    }
+    double outs = 1;
+    for (int r : groups_[0].ranges) {
+      if (g_.ranges[(size_t)r].extent <= 0) return false;
+      outs *= (double)g_.ranges[(size_t)r].extent;
+    }
+    if (K < 512 || K % 32 != 0 || outs < 64 || outs > 16384) return false;
+    // the loads must run along the outputs, not along the reduce range
+    const std::vector<int> order = fastest_first(groups_[0]);
+    const int F = order[0], QF = g_.range_ord.at(T.src.back());
+    std::vector<char> mark(g_.nodes.size(), 0);
+    mark_reachable(g_, T.src[0], mark);
+    bool along_out = false;
+    for (int i = 0; i < (int)g_.nodes.size(); i++) {
+      if (!mark[(size_t)i] || g_.n(i).op != POLY_OP_LOAD) continue;
+      const int li = g_.n(g_.n(g_.n(i).src[0]).src[1]).lin;
+      if (li < 0) return false;
+      bool aff;
+      // (a value per reduce index that no output coordinate enters -- a row statistic --
+      // is the same for every lane: it does not decide the mapping)
+      uint64_t out_bits = 0;
+      for (int r : groups_[0].ranges) out_bits |= (uint64_t)1 << r;
+      if (!(g_.n(g_.n(g_.n(i).src[0]).src[1]).deps & out_bits)) continue;
+      if (g_.lin_range_coef(g_.lins[(size_t)li], QF, &aff) == 1 && aff) return false;
+      if (g_.lin_range_coef(g_.lins[(size_t)li], F, &aff) == 1 && aff) along_out = true;
+    }
+    return along_out;
+  }
+
+  std::string render_ordered(RenderedKernel *out) {
+    const Group &gr = groups_[0];
+    const int T = top_reduces_[0];
+    const KNode &tk = g_.n(T);
+    const PolyOps rop = reduce_op(tk);
+    const std::vector<int> order = fastest_first(gr);
+    double outs = 1;
+    for (int r : gr.ranges) outs *= (double)g_.ranges[(size_t)r].extent;
+    int64_t K = 1;
+    std::vector<int> rr;
+    for (size_t i = 1; i < tk.src.size(); i++) { rr.push_back(g_.range_ord.at(tk.src[i])); K *= g_.ranges[(size_t)rr.back()].extent; }
+    const char *ct = dt_cname(tk.dt);
+    std::string body;
+    line(body, 1, strf("__shared__ %s poly_terms[32][64];", ct));
+    line(body, 1, "const int lane = threadIdx.x & 63, w = threadIdx.x >> 6;");
+    line(body, 1, strf("const long long out_id = (long long)blockIdx.x * 64 + lane;"));
+    line(body, 1, strf("const bool live = out_id < %.0fll;", outs));
+    line(body, 1, "{");
+    Scope S0;
+    S0.indent = 2;
+    for (int r : gr.ranges) S0.avail |= (uint64_t)1 << r;
+    std::string decomp;
+    line(decomp, 2, strf("long long t_ = live ? out_id : %.0fll;", outs - 1));   // idle lanes redo the last output, store nothing
+    for (size_t oi = 0; oi < order.size(); oi++) {
+      const int ord = order[oi];
+      const long long e = (long long)g_.ranges[(size_t)ord].extent;
+      if (oi + 1 == order.size()) line(decomp, 2, strf("const int r%d = (int)t_;", ord));
+      else line(decomp, 2, strf("const int r%d = (int)(t_ %% %lld); t_ /= %lld;", ord, e, e));
+      em_.bind_range(ord, strf("r%d", ord));
+    }
+    Scope L;
+    L.parent = &S0;
+    L.avail = S0.avail;
+    L.indent = 4;
+    std::string qdecomp;
+    line(qdecomp, 4, "int q_ = k0 + w * 8 + t8;");
+    for (size_t i = rr.size(); i-- > 0;) {
+      const int ord = rr[i];
+      const long long e = (long long)g_.ranges[(size_t)ord].extent;
+      if (i == 0) line(qdecomp, 4, strf("const int r%d = q_;", ord));
+      else line(qdecomp, 4, strf("const int r%d = q_ %% %lld; q_ /= %lld;", ord, e, e));
+      em_.bind_range(ord, strf("r%d", ord));
+      L.avail |= (uint64_t)1 << ord;
+    }
+    const std::string term = em_.emit(tk.src[0], &L);
+    line(L.code, 4, strf("poly_terms[w * 8 + t8][lane] = %s;", term.c_str()));
+    const std::string acc = strf("acc%d", T);
+    std::string loop;
+    line(loop, 2, strf("%s %s = %s;", ct, acc.c_str(), Emitter::reduce_identity(rop, tk.dt).c_str()));
+    line(loop, 2, strf("for (int k0 = 0; k0 < %lld; k0 += 32) {", (long long)K));
+    line(loop, 3, "#pragma unroll");
+    line(loop, 3, "for (int t8 = 0; t8 < 8; t8++) {");
+    loop += qdecomp + L.code;
+    line(loop, 3, "}");
+    line(loop, 3, "__syncthreads();");
+    line(loop, 3, "if (w == 0) {");
+    line(loop, 4, "#pragma unroll");
+    line(loop, 4, strf("for (int t = 0; t < 32; t++) %s = %s;", acc.c_str(),
+                       Emitter::reduce_combine(rop, tk.dt, acc, "poly_terms[t][lane]").c_str()));
+    line(loop, 3, "}");
+    line(loop, 3, "__syncthreads();");
+    line(loop, 2, "}");
+    const std::string pre_loop = S0.code;
+    S0.code.clear();
+    em_.preset(T, acc);
+    std::string tail_stores;
+    for (int si : gr.stores) {
+      const StoreInfo &st = g_.stores[(size_t)si];
+      std::string v = em_.emit(st.value, &S0);
+      std::string idx = em_.emit(g_.n(st.index).src[1], &S0);
+      int p = g_.param_slot(st.param);
+      std::string cond = "w == 0 && live";
+      if (st.gate >= 0) cond += " && " + em_.emit(st.gate, &S0);
+      line(tail_stores, 2, strf("if (%s) data%d[%s] = %s;", cond.c_str(), p, idx.c_str(), v.c_str()));
+    }
+    body += decomp + pre_loop + loop + S0.code + tail_stores;
+    line(body, 1, "}");
+    out->launch.grid[0] = (unsigned)std::ceil(outs / 64.0);
+    out->launch.block[0] = 256;
+    out->klass = KernelClass::THREAD_REDUCE;
+    out->strategy = strf("ordered reduce: 64 outputs per workgroup, terms of K=%lld computed by four waves, added in order by one;", (long long)K);
     return body;
   }
 

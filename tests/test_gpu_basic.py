@@ -129,3 +129,29 @@ def test_random_graphs_match_reference(seed):
     c.close()
     scale = float(np.nanmax(np.abs(want[bo][np.isfinite(want[bo])]))) if np.isfinite(want[bo]).any() else 1.0
     assert_close(got[bo], want[bo], rtol=1e-4, atol=1e-5 * max(scale, 1.0), what=f"random graph {seed}")
+
+
+@pytest.mark.parametrize("rows,cols", [(4096, 1024), (512, 192), (1024, 100), (500, 128)])
+def test_bf16_column_sums_keep_the_reference_order(rows, cols):
+    """Sums over the rows of a bf16 matrix accumulate in bf16: every addition rounds, so the
+    result depends on the order.  The order-preserving lowering (terms computed by four
+    waves, added in index order by one) must give the reference's bits; so must whatever
+    lowering takes a shape it declines."""
+    c = R.Ctx()
+    g = rng(11)
+    x = c.buffer((rows, cols), R.BF16, name="x")
+    w = c.buffer((rows, cols), R.BF16, name="w")
+    s = c.buffer((rows, 1), R.F32, name="s")
+    o1, o2 = c.buffer((cols,), R.BF16, name="o1"), c.buffer((cols,), R.BF16, name="o2")
+    bits = lambda shape: R.f32_to_bf16_bits(g.normal(0, 1, int(np.prod(shape))).astype(np.float32))
+    arrays = {x: bits((rows, cols)), w: bits((rows, cols)), s: g.uniform(0.5, 2, rows).astype(np.float32)}
+    for out, val in ((o1, x.sum(axis=0)), (o2, ((x.cast(R.F32) * s).cast(R.BF16) * w).sum(axis=0))):
+        sink = c.sink((out, val))
+        sub = {t: a for t, a in arrays.items()}
+        sub[out] = np.zeros(cols, np.uint16)
+        want = run_ref(c, sink, sub)
+        got, info = run_hip(c, sink, sub)
+        if rows >= 512 and rows % 32 == 0 and cols >= 64:
+            assert any("ordered reduce" in i["desc"] for i in info), [i["desc"] for i in info]
+        assert np.array_equal(np.asarray(got[out]).view(np.uint16), np.asarray(want[out]).view(np.uint16)), (rows, cols)
+    c.close()
