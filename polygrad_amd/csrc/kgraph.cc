@@ -321,15 +321,24 @@ bool KernelGraph::build(const PolyUOp *root) {
   if (!root || root->op != POLY_OP_SINK) { error = "kernel root is not a SINK"; return false; }
 
   // iterative post-order DFS
+  auto src_of = [&](const PolyUOp *u, int i) -> const PolyUOp * {
+    return slab_value && u->op == POLY_OP_STORE && i == 1 ? slab_value : u->src[i];
+  };
   struct Frame { const PolyUOp *u; int next; };
   std::vector<Frame> stack;
-  stack.push_back({root, 0});
   std::unordered_map<const PolyUOp *, char> state;  // 1 = on stack, 2 = done
+  for (const PolyUOp *p : slab_params) {
+    if (p->op != POLY_OP_PARAM || p->n_src != 0) { error = "slab parameter is not a plain PARAM"; return false; }
+    if (!state.count(p)) { state[p] = 1; stack.push_back({p, 0}); }
+  }
+  std::reverse(stack.begin(), stack.end());
+  stack.insert(stack.begin(), {root, 0});
   state[root] = 1;
   while (!stack.empty()) {
     Frame &f = stack.back();
     if (f.next < (int)f.u->n_src) {
-      const PolyUOp *s = f.u->src[f.next++];
+      const PolyUOp *s = src_of(f.u, f.next);
+      f.next++;
       if (!s) { error = "null source pointer"; return false; }
       auto it = state.find(s);
       if (it == state.end()) { state[s] = 1; stack.push_back({s, 0}); }
@@ -343,7 +352,7 @@ bool KernelGraph::build(const PolyUOp *root) {
         error = strf("vector dtype on %s in a scheduled kernel", op_name(u->op));
         return false;
       }
-      for (int i = 0; i < (int)u->n_src; i++) kn.src.push_back(ids[u->src[i]]);
+      for (int i = 0; i < (int)u->n_src; i++) kn.src.push_back(ids[src_of(u, i)]);
       ids[u] = (int)nodes.size();
       nodes.push_back(std::move(kn));
       state[u] = 2;
@@ -376,6 +385,10 @@ bool KernelGraph::build(const PolyUOp *root) {
       r.node = i; r.bound_node = k.src[0]; r.is_reduce = false; r.extent = -1;
       const PolyUOp *b = nodes[(size_t)k.src[0]].u;
       if (b->op == POLY_OP_CONST) r.extent = b->arg.i;
+      if (k.u == slab_range) {
+        if (r.extent < 0 || slab_lo < 0 || slab_extent <= 0 || slab_lo + slab_extent > r.extent) { error = "slab outside its range"; return false; }
+        r.extent = slab_extent;
+      }
       r.axis_id = k.u->arg.kind == POLY_ARG_RANGE ? k.u->arg.range.axis_id
                   : (k.u->arg.kind == POLY_ARG_INT ? k.u->arg.i : -1);
       if (ranges.size() >= 64) { error = "more than 64 ranges in one kernel"; return false; }
@@ -510,6 +523,7 @@ bool KernelGraph::build(const PolyUOp *root) {
           hi = bh - 1;
         }
         out = lin_atom(atom_for_node(i, Atom::RANGE, 0, hi < 0 ? 0 : hi));
+        if (k.u == slab_range) out.c0 = slab_lo;
         ok = true;
         break;
       }
@@ -600,7 +614,7 @@ struct RawEval {
     auto S = [&](size_t i) { return node(k.src[i]); };
     switch (k.op) {
       case POLY_OP_CONST: return k.u->arg.i;
-      case POLY_OP_RANGE: return rv[(size_t)g.range_ord.at(id)];
+      case POLY_OP_RANGE: return rv[(size_t)g.range_ord.at(id)] + (g.slab_range && k.u == g.slab_range ? g.slab_lo : 0);
       case POLY_OP_ADD: return S(0) + S(1);
       case POLY_OP_SUB: return S(0) - S(1);
       case POLY_OP_MUL: return S(0) * S(1);

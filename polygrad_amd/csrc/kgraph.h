@@ -94,6 +94,13 @@ struct KernelGraph {
   std::vector<Lin> lins;
   std::string error;
 
+  // One slab of a kernel, set before build(): RANGE `slab_range` runs over
+  // [slab_lo, slab_lo + slab_extent) only (the graph's range counts from 0 and every use
+  // sees range + slab_lo), and every STORE takes `slab_value` in place of its value.
+  const PolyUOp *slab_range = nullptr, *slab_value = nullptr;
+  int64_t slab_lo = 0, slab_extent = 0;
+  std::vector<const PolyUOp *> slab_params;   // every PARAM of the whole kernel: a slab keeps its argument list
+
   bool build(const PolyUOp *root);
 
   // canonical-expression helpers

@@ -966,12 +966,145 @@ static bool split_in_two(const KernelGraph &g, const std::string &fn_name, const
   return true;
 }
 
+// For which values of range ordinal R can boolean node `id` (negated when `neg`) hold?
+// Narrows [*lo, *hi) and returns true when the answer is that interval exactly: conjunctions
+// of comparisons of R with constants, and comparisons that the bounds of their operands decide.
+static bool cond_interval(const KernelGraph &g, int id, bool neg, int R, int64_t *lo, int64_t *hi) {
+  const KNode &k = g.n(id);
+  auto is_true = [&](int n) { return g.n(n).op == POLY_OP_CONST && g.n(n).dt == DT_BOOL && g.n(n).u->arg.b; };
+  if (k.op == POLY_OP_CONST && k.dt == DT_BOOL) {
+    if (k.u->arg.b == neg) *hi = *lo;
+    return true;
+  }
+  if (k.dt == DT_BOOL && k.op == POLY_OP_NEG) return cond_interval(g, k.src[0], !neg, R, lo, hi);
+  if (k.dt == DT_BOOL && (k.op == POLY_OP_CMPNE || k.op == POLY_OP_XOR) && k.src.size() == 2 && g.n(k.src[0]).dt == DT_BOOL) {
+    if (is_true(k.src[1])) return cond_interval(g, k.src[0], !neg, R, lo, hi);
+    if (is_true(k.src[0])) return cond_interval(g, k.src[1], !neg, R, lo, hi);
+    return false;
+  }
+  if (k.op == POLY_OP_AND && k.dt == DT_BOOL && !neg)
+    return cond_interval(g, k.src[0], false, R, lo, hi) && cond_interval(g, k.src[1], false, R, lo, hi);
+  if (k.op == POLY_OP_CMPLT && k.src.size() == 2) {
+    const int la = g.n(k.src[0]).lin, lb = g.n(k.src[1]).lin;
+    if (la < 0 || lb < 0) return false;
+    const Lin d = g.lin_add(g.lins[(size_t)la], g.lins[(size_t)lb], -1);      // holds when d < 0
+    int64_t dl, dh;
+    g.lin_bounds(d, &dl, &dh);
+    if (dh < 0) { if (neg) *hi = *lo; return true; }
+    if (dl >= 0) { if (!neg) *hi = *lo; return true; }
+    if (d.terms.size() != 1) return false;
+    const Atom &a = g.atoms[(size_t)d.terms[0].atom];
+    if (a.kind != Atom::RANGE || g.range_ord.at(a.node) != R) return false;
+    if (d.terms[0].coef == 1) {            // R + c0 < 0  <=>  R < -c0
+      if (!neg) *hi = std::min(*hi, -d.c0); else *lo = std::max(*lo, -d.c0);
+    } else if (d.terms[0].coef == -1) {    // c0 - R < 0  <=>  R > c0
+      if (!neg) *lo = std::max(*lo, d.c0 + 1); else *hi = std::min(*hi, d.c0 + 1);
+    } else return false;
+    if (*hi < *lo) *hi = *lo;
+    return true;
+  }
+  return false;
+}
+
+// A kernel whose stored value is a sum of where(cond_i, X_i, 0) with the conditions cutting
+// one output range into adjacent slabs -- the derivative of a concatenation, e.g. of the
+// q | k | v columns of an attention block, every X_i its own batched matmul -- computes, as
+// one kernel, every sum in every thread.  It is rendered as one kernel per slab instead
+// (range restricted, value X_i), run one after the other: each is then a plain kernel that
+// the matmul lowerings can take.  x + 0 + 0 is x, so the values are the same (a -0 result
+// stays -0 instead of becoming +0).  Done only when every slab lands on the matrix pipe.
+static bool fis_reject(int line) {
+  if (getenv("POLY_HIP_DEBUG")) fprintf(stderr, "polygrad: render_hip: slab fission rejected at render_hip.cc:%d\n", line);
+  return false;
+}
+
+static bool try_slab_fission(const KernelGraph &g, const std::string &fn_name, const RenderOptions &opt, RenderedKernel *out) {
+  if (!opt.allow_templates || !opt.reduce_override.empty() || opt.exit_if_flag || opt.exit_unless_flag || opt.promote_reduce >= 0 ||
+      opt.slice_reduce >= 0 || opt.scratch_param || g.slab_range || getenv("POLY_HIP_NO_FISSION"))
+    return false;
+  if (g.stores.size() != 1 || g.stores[0].gate >= 0 || !g.vars.empty() || g.reduces.size() < 2) return false;
+  const StoreInfo &st = g.stores[0];
+  // leaves of the sum
+  struct Piece { int cond, value; int64_t lo, hi; };
+  std::vector<Piece> pieces;
+  std::vector<int> stack{st.value};
+  while (!stack.empty()) {
+    const int id = stack.back();
+    stack.pop_back();
+    const KNode &k = g.n(id);
+    if (k.op == POLY_OP_ADD && dt_is_float(k.dt) && k.dt == g.n(st.value).dt) { stack.push_back(k.src[1]); stack.push_back(k.src[0]); continue; }
+    if (k.op != POLY_OP_WHERE || k.src.size() != 3) return fis_reject(__LINE__);
+    const KNode &z = g.n(k.src[2]);
+    if (z.op != POLY_OP_CONST || !dt_is_float(z.dt) || z.u->arg.f != 0.0 || g.n(k.src[1]).dt != k.dt) return fis_reject(__LINE__);
+    pieces.push_back({k.src[0], k.src[1], 0, 0});
+  }
+  if (pieces.size() < 2 || pieces.size() > 8) return fis_reject(__LINE__);
+  for (const int R : st.ranges) {
+    const int64_t ext = g.ranges[(size_t)R].extent;
+    if (ext <= 0) continue;
+    bool ok = true;
+    for (Piece &p : pieces) {
+      p.lo = 0; p.hi = ext;
+      if (!cond_interval(g, p.cond, false, R, &p.lo, &p.hi) || p.hi <= p.lo) { ok = false; break; }
+    }
+    if (!ok) continue;
+    std::vector<Piece> order = pieces;
+    std::sort(order.begin(), order.end(), [](const Piece &a, const Piece &b) { return a.lo < b.lo; });
+    int64_t at = 0;
+    for (const Piece &p : order) { if (p.lo != at) { ok = false; break; } at = p.hi; }
+    if (!ok || at != ext) continue;
+    // one kernel per slab
+    std::vector<RenderedKernel> parts(order.size());
+    const PolyUOp *root = g.nodes.back().u;
+    for (size_t i = 0; i < order.size() && ok; i++) {
+      KernelGraph sub;
+      sub.slab_range = g.n(g.ranges[(size_t)R].node).u;
+      sub.slab_lo = order[i].lo;
+      sub.slab_extent = order[i].hi - order[i].lo;
+      sub.slab_value = g.n(order[i].value).u;
+      for (const ParamInfo &pi : g.params) sub.slab_params.push_back(g.n(pi.node).u);
+      std::string err;
+      if (!sub.build(root) || !render_kernel(sub, fn_name, opt, &parts[i], &err)) {
+        if (getenv("POLY_HIP_DEBUG")) fprintf(stderr, "polygrad: render_hip: slab %zu: %s%s\n", i, sub.error.c_str(), err.c_str());
+        ok = false;
+        break;
+      }
+      const RenderedKernel &pk = parts[i];
+      if (pk.klass != KernelClass::MATMUL_MFMA || !pk.guards.empty() || !pk.tables.empty() || !pk.fallback_source.empty() ||
+          pk.n_vars != 0 || pk.n_params != parts[0].n_params)
+        ok = false;
+    }
+    if (!ok) return fis_reject(__LINE__);
+    *out = parts.back();
+    out->variants.clear();
+    out->pres.clear();
+    out->scratch_bytes = 256;
+    out->strategy = "";
+    out->bytes = 0;
+    out->flops = 0;
+    for (size_t i = 0; i < parts.size(); i++) {
+      const RenderedKernel &pk = parts[i];
+      for (const RenderedKernel::Pre &pp : pk.pres) out->pres.push_back(pp);
+      if (i + 1 < parts.size()) out->pres.push_back({pk.source, pk.entry, pk.launch});
+      out->scratch_bytes = std::max(out->scratch_bytes, pk.scratch_bytes);
+      out->strategy += strf("%s[%lld,%lld) %s", i ? "; " : "", (long long)order[i].lo, (long long)order[i].hi, pk.strategy.c_str());
+      out->bytes += pk.bytes;
+      out->flops += pk.flops;
+    }
+    out->strategy = strf("%zu slabs of one output range, one kernel each: ", parts.size()) + out->strategy;
+    return true;
+  }
+  return fis_reject(__LINE__);
+}
+
 bool render_kernel(const KernelGraph &g, const std::string &fn_name, const RenderOptions &opt,
                    RenderedKernel *out, std::string *err) {
   if (opt.allow_templates) {
     if (try_render_matmul(g, fn_name, opt, out)) return true;
     if (try_render_gather(g, fn_name, opt, out)) return true;
     if (try_render_matmul_generic(g, fn_name, opt, out)) return true;
+    *out = RenderedKernel();
+    if (try_slab_fission(g, fn_name, opt, out)) return true;
   }
   *out = RenderedKernel();
   if (try_split_reduce(g, fn_name, opt, out)) return true;

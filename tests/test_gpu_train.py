@@ -79,7 +79,7 @@ def test_adamw_update_matches_reference():
     assert got[bufs["g"]].tobytes() == arrays[bufs["g"]].tobytes()
 
 
-@pytest.mark.parametrize("B,T,D,H,V", [(1, 32, 64, 2, 97), (2, 64, 128, 4, 301)])
+@pytest.mark.parametrize("B,T,D,H,V", [(1, 32, 64, 2, 97), (2, 64, 128, 4, 301), (1, 128, 128, 2, 97)])
 def test_gpt2_block_train_step_matches_reference(B, T, D, H, V):
     """Benchmark configuration 5 at a reduced size: one transformer block, final LayerNorm,
     vocabulary projection, next-token cross-entropy (sparse targets), reverse-mode
@@ -97,6 +97,8 @@ def test_gpt2_block_train_step_matches_reference(B, T, D, H, V):
     assert len(info) >= 100
     if D >= 128:      # large enough for the backward matmuls to leave the generic reductions
         assert sum("operands as expressions" in k["desc"] for k in info) >= 4, [k["desc"] for k in info if "reduce" in k["desc"]]
+    if T >= 128:      # the derivative of the q | k | v concatenation: one batched matmul per slab of columns
+        assert any("3 slabs of one output range" in k["desc"] for k in info)
     assert_close(got[bufs["loss"]], want[bufs["loss"]], rtol=1e-4, what="loss")
     assert abs(float(want[bufs["loss"]][0]) - np.log(V)) < 0.05       # random init: loss is ln(vocab)
     for name in graphs.BLOCK_PARAMS:

@@ -33,7 +33,7 @@ def test_fixture_kernels_stay_in_bounds(hiplib):
 
 
 @pytest.mark.skipif(not R.available(), reason="reference library not built")
-@pytest.mark.parametrize("B,T,D,H,V", [(1, 32, 64, 2, 97), (2, 64, 128, 4, 301)])
+@pytest.mark.parametrize("B,T,D,H,V", [(1, 32, 64, 2, 97), (2, 64, 128, 4, 301), (1, 128, 128, 2, 97)])
 def test_training_step_kernels_stay_in_bounds(B, T, D, H, V, hiplib):
     """The backward kernels of the one-block training step: among them the derivative of a
     pad, `where(valid, reduce(...), 0)`, whose index arithmetic goes negative on the masked
