@@ -131,7 +131,10 @@ class Generic {
     if (coop) {
       body = render_coop(out);
     } else if (plan_ordered()) {
-      body = render_ordered(out);
+      body = opt_.ordered_stage ? render_ordered_stage(out) : render_ordered(out);
+    } else if (opt_.ordered_stage) {
+      *err = "not an ordered reduction";
+      return false;
     } else {
       body = render_flat(out);
     }
@@ -689,6 +692,7 @@ class Generic {
     const KNode &T = g_.n(top_reduces_[0]);
     const int sz = dt_size(T.dt);
     if (sz != 2 && sz != 4) return false;
+    if (opt_.ordered_stage && !dt_is_float(T.dt)) return false;    // terms travel as fp32
     int64_t K = 1;
     for (size_t i = 1; i < T.src.size(); i++) {
       const int64_t e = g_.ranges[(size_t)g_.range_ord.at(T.src[i])].extent;
@@ -804,6 +808,117 @@ class Generic {
     out->launch.block[0] = 256;
     out->klass = KernelClass::THREAD_REDUCE;
     out->strategy = strf("ordered reduce: 64 outputs per workgroup, terms of K=%lld computed by four waves, added in order by one;", (long long)K);
+    return body;
+  }
+
+  // The two kernels of the same reduction with the terms passing through memory: every
+  // term is computed by a thread of its own (the whole chip instead of outputs / 64
+  // workgroups), and the adder only walks a column of finished terms.
+  std::string render_ordered_stage(RenderedKernel *out) {
+    const Group &gr = groups_[0];
+    const int T = top_reduces_[0];
+    const KNode &tk = g_.n(T);
+    const PolyOps rop = reduce_op(tk);
+    const std::vector<int> order = fastest_first(gr);
+    double outs = 1;
+    for (int r : gr.ranges) outs *= (double)g_.ranges[(size_t)r].extent;
+    int64_t K = 1;
+    std::vector<int> rr;
+    for (size_t i = 1; i < tk.src.size(); i++) { rr.push_back(g_.range_ord.at(tk.src[i])); K *= g_.ranges[(size_t)rr.back()].extent; }
+    const char *ct = dt_cname(tk.dt);
+    const bool first = opt_.ordered_stage == 1;
+    std::string body;
+    Scope S0;
+    S0.indent = 2;
+    for (int r : gr.ranges) S0.avail |= (uint64_t)1 << r;
+    std::string decomp;
+    if (first) {
+      line(body, 1, "const long long gid = (long long)blockIdx.x * 256 + threadIdx.x;");
+      line(body, 1, strf("if (gid < %.0fll) {", outs * (double)K));
+      line(decomp, 2, strf("long long t_ = gid %% %.0fll;", outs));
+    } else {
+      line(body, 1, "const long long out_id = (long long)blockIdx.x * 64 + threadIdx.x;");
+      line(body, 1, strf("const bool live = out_id < %.0fll;", outs));
+      line(body, 1, "{");
+      line(decomp, 2, strf("const long long col_ = live ? out_id : %.0fll;", outs - 1));   // idle lanes redo the last output, store nothing
+      line(decomp, 2, "long long t_ = col_;");
+    }
+    for (size_t oi = 0; oi < order.size(); oi++) {
+      const int ord = order[oi];
+      const long long e = (long long)g_.ranges[(size_t)ord].extent;
+      if (oi + 1 == order.size()) line(decomp, 2, strf("const int r%d = (int)t_;", ord));
+      else line(decomp, 2, strf("const int r%d = (int)(t_ %% %lld); t_ /= %lld;", ord, e, e));
+      em_.bind_range(ord, strf("r%d", ord));
+    }
+    if (first) {
+      Scope L;
+      L.parent = &S0;
+      L.avail = S0.avail;
+      L.indent = 2;
+      std::string qdecomp;
+      line(qdecomp, 2, strf("int q_ = (int)(gid / %.0fll);", outs));
+      for (size_t i = rr.size(); i-- > 0;) {
+        const int ord = rr[i];
+        const long long e = (long long)g_.ranges[(size_t)ord].extent;
+        if (i == 0) line(qdecomp, 2, strf("const int r%d = q_;", ord));
+        else line(qdecomp, 2, strf("const int r%d = q_ %% %lld; q_ /= %lld;", ord, e, e));
+        em_.bind_range(ord, strf("r%d", ord));
+        L.avail |= (uint64_t)1 << ord;
+      }
+      const std::string term = em_.emit(tk.src[0], &L);
+      line(L.code, 2, strf("poly_scratch[gid] = (float)(%s);", term.c_str()));
+      body += decomp + qdecomp + S0.code + L.code;
+      line(body, 1, "}");
+      out->launch.grid[0] = (unsigned)std::ceil(outs * (double)K / 256.0);
+      out->launch.block[0] = 256;
+      out->klass = KernelClass::ELEMENTWISE;
+      out->strategy = strf("ordered reduce, stage 1: the %.0f x %lld terms, one thread each;", outs, (long long)K);
+      return body;
+    }
+    const std::string acc = strf("acc%d", T);
+    std::string loop;
+    line(loop, 2, strf("%s %s = %s;", ct, acc.c_str(), Emitter::reduce_identity(rop, tk.dt).c_str()));
+    // The additions form one dependent chain; what can overlap is the memory latency of
+    // the terms: 64 are loaded ahead while the previous 64 are added.
+    const long long NB = K / 64;
+    const std::string at = strf("poly_scratch[(long long)(%%s) * %.0fll + col_]", outs);
+    auto term_at = [&](const std::string &k) { std::string e = at; e.replace(e.find("%s"), 2, k); return e; };
+    if (NB > 0) {
+      line(loop, 2, "float cur_[64], nxt_[64];");
+      line(loop, 2, "#pragma unroll");
+      line(loop, 2, strf("for (int j = 0; j < 64; j++) cur_[j] = %s;", term_at("j").c_str()));
+      line(loop, 2, strf("for (int b = 0; b < %lld; b++) {", NB));
+      line(loop, 3, strf("if (b + 1 < %lld) {", NB));
+      line(loop, 4, "#pragma unroll");
+      line(loop, 4, strf("for (int j = 0; j < 64; j++) nxt_[j] = %s;", term_at("(b + 1) * 64 + j").c_str()));
+      line(loop, 3, "}");
+      line(loop, 3, "#pragma unroll");
+      line(loop, 3, strf("for (int j = 0; j < 64; j++) %s = %s;", acc.c_str(),
+                         Emitter::reduce_combine(rop, tk.dt, acc, strf("(%s)cur_[j]", ct)).c_str()));
+      line(loop, 3, "#pragma unroll");
+      line(loop, 3, "for (int j = 0; j < 64; j++) cur_[j] = nxt_[j];");
+      line(loop, 2, "}");
+    }
+    if (K % 64)
+      line(loop, 2, strf("for (int k = %lld; k < %lld; k++) %s = %s;", NB * 64, (long long)K, acc.c_str(),
+                         Emitter::reduce_combine(rop, tk.dt, acc, strf("(%s)%s", ct, term_at("k").c_str())).c_str()));
+    em_.preset(T, acc);
+    std::string tail_stores;
+    for (int si : gr.stores) {
+      const StoreInfo &st = g_.stores[(size_t)si];
+      std::string v = em_.emit(st.value, &S0);
+      std::string idx = em_.emit(g_.n(st.index).src[1], &S0);
+      int p = g_.param_slot(st.param);
+      std::string cond = "live";
+      if (st.gate >= 0) cond += " && " + em_.emit(st.gate, &S0);
+      line(tail_stores, 2, strf("if (%s) data%d[%s] = %s;", cond.c_str(), p, idx.c_str(), v.c_str()));
+    }
+    body += decomp + loop + S0.code + tail_stores;
+    line(body, 1, "}");
+    out->launch.grid[0] = (unsigned)std::ceil(outs / 64.0);
+    out->launch.block[0] = 64;
+    out->klass = KernelClass::THREAD_REDUCE;
+    out->strategy = strf("stage 2: K=%lld terms per output added in index order, one thread per output;", (long long)K);
     return body;
   }
 
@@ -966,6 +1081,32 @@ static bool split_in_two(const KernelGraph &g, const std::string &fn_name, const
   return true;
 }
 
+// The order-preserving reduction (a sum that rounds to 16 bits at every step) with its terms
+// computed by a first kernel over the whole chip; the second only adds, in index order.
+static bool try_ordered_two_stage(const KernelGraph &g, const std::string &fn_name, const RenderOptions &opt, RenderedKernel *out) {
+  if (opt.ordered_stage || opt.scratch_param || !opt.reduce_override.empty() || opt.exit_if_flag || opt.exit_unless_flag ||
+      opt.promote_reduce >= 0 || opt.slice_reduce >= 0 || getenv("POLY_HIP_NO_SPLIT_REDUCE"))
+    return false;
+  if (g.stores.empty() || g.reduces.size() != 1 || !g.vars.empty()) return false;
+  double terms = 1;
+  for (const RangeInfo &r : g.ranges) { if (r.extent <= 0) return false; terms *= (double)r.extent; }
+  if (terms * 4 > 268435456.0) return false;        // scratch: at most 256 MiB
+  RenderOptions o1 = opt, o2 = opt;
+  o1.ordered_stage = 1; o1.scratch_param = true;
+  o2.ordered_stage = 2; o2.scratch_param = true;
+  RenderedKernel pre;
+  std::string err;
+  Generic g1(g, fn_name, o1);
+  if (!g1.run(&pre, &err)) return false;
+  Generic g2(g, fn_name, o2);
+  if (!g2.run(out, &err)) return false;
+  out->pres.push_back({pre.source, pre.entry, pre.launch});
+  out->scratch_bytes = (size_t)terms * sizeof(float);
+  out->strategy = pre.strategy + " " + out->strategy;
+  out->bytes = pre.bytes;
+  return true;
+}
+
 // For which values of range ordinal R can boolean node `id` (negated when `neg`) hold?
 // Narrows [*lo, *hi) and returns true when the answer is that interval exactly: conjunctions
 // of comparisons of R with constants, and comparisons that the bounds of their operands decide.
@@ -1110,6 +1251,8 @@ bool render_kernel(const KernelGraph &g, const std::string &fn_name, const Rende
   if (try_split_reduce(g, fn_name, opt, out)) return true;
   *out = RenderedKernel();
   if (try_slice_reduce(g, fn_name, opt, out)) return true;
+  *out = RenderedKernel();
+  if (try_ordered_two_stage(g, fn_name, opt, out)) return true;
   *out = RenderedKernel();
   Generic gen(g, fn_name, opt);
   return gen.run(out, err);
