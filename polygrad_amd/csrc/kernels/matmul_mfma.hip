@@ -17,6 +17,7 @@
 //   POLY_SIGNATURE      the kernel's parameter list
 //   POLY_EPILOGUE(acc, m, n, z)   stores one finished element (generated from the
 //                       UOps around the REDUCE: casts, bias, activation, index)
+//   POLY_KSPLIT         (optional) workgroups sharing the K tiles of one output tile
 //   POLY_EP_CONTIG      1 when consecutive n of a row are consecutive in memory; then
 //                       POLY_EP_TYPE, POLY_EP_VALUE(acc, m, n, z) and POLY_EP_PTR(m, n, z)
 //                       give the element type, value and address separately and the
@@ -79,7 +80,13 @@ typedef float poly_f32x4 __attribute__((ext_vector_type(4)));
 #define POLY_LDK POLY_BK
 #define POLY_NCOL (POLY_BK / 8)
 __device__ __forceinline__ int poly_swz(int row) { return (row ^ (row >> 3)) & (POLY_NCOL - 1); }
-#define POLY_KT (POLY_K / POLY_BK)
+#ifndef POLY_KSPLIT
+#define POLY_KSPLIT 1
+#endif
+// K tiles one workgroup walks: with POLY_KSPLIT > 1 the K tiles of an output tile are dealt
+// to that many workgroups (blockIdx.y = z * POLY_KSPLIT + part), each leaving its fp32
+// accumulators where the epilogue macros put them (they may use `poly_ks`, the part).
+#define POLY_KT (POLY_K / POLY_BK / POLY_KSPLIT)
 // row pitch (floats) of the 32x32 output staging tile: 16-byte aligned rows, and rows 4
 // apart (the two halves of a wave) land on different banks
 #define POLY_STAGE_LD 36
@@ -211,7 +218,13 @@ extern "C" __global__ void __launch_bounds__(POLY_NTHREADS) poly_k(POLY_SIGNATUR
     tile_n = in_group / gsz;
 #endif
   }
+#if POLY_KSPLIT > 1
+  const int z = blockIdx.y / POLY_KSPLIT, poly_ks = blockIdx.y % POLY_KSPLIT;
+  const int k_base = poly_ks * (POLY_KT * POLY_BK);
+#else
   const int z = blockIdx.y;
+  constexpr int k_base = 0;
+#endif
   const int m0 = tile_m * POLY_BM, n0 = tile_n * POLY_BN;
 
   const POLY_TIN *__restrict__ gA = POLY_A_PTR + poly_a_z(z);
@@ -264,7 +277,7 @@ extern "C" __global__ void __launch_bounds__(POLY_NTHREADS) poly_k(POLY_SIGNATUR
 #endif
 
   auto load_tiles = [&](int kt, auto &ra, auto &rb) {
-    const int k0 = kt * POLY_BK;
+    const int k0 = k_base + kt * POLY_BK;
 #if POLY_A_KC
     StageA::load(gA, a_off, poly_a_k(k0), ra);
 #else
@@ -292,7 +305,7 @@ extern "C" __global__ void __launch_bounds__(POLY_NTHREADS) poly_k(POLY_SIGNATUR
   // of the tile held in (ra, rb) to LDS buffer `buf` (if st) and then refill those
   // registers from tile kt_load (if ld).
   auto stage_part = [&](int part, int nparts, bool st, int buf, bool ld, int kt_load, auto &ra, auto &rb) {
-    const int k0 = kt_load * POLY_BK;
+    const int k0 = k_base + kt_load * POLY_BK;
 #pragma unroll
     for (int u = 0; u < StageA::UNITS; u++) {
       if (u * nparts / StageA::UNITS != part) continue;

@@ -376,9 +376,10 @@ extern "C" __global__ void __launch_bounds__(256) poly_k(POLY_SIGNATURE) {
   const long long gid = (long long)blockIdx.x * 256 + threadIdx.x;
   if (gid >= (long long)POLY_Z * POLY_M * POLY_N) return;
   const int n = (int)(gid % POLY_N), m = (int)((gid / POLY_N) % POLY_M), z = (int)(gid / ((long long)POLY_N * POLY_M));
-  float acc = poly_scratch[gid];
+  const float *__restrict__ part = POLY_PARTIALS;
+  float acc = part[gid];
 #pragma unroll
-  for (int s = 1; s < POLY_KSPLIT; s++) acc += poly_scratch[(size_t)s * POLY_Z * POLY_M * POLY_N + gid];
+  for (int s = 1; s < POLY_KSPLIT; s++) acc += part[(size_t)s * POLY_Z * POLY_M * POLY_N + gid];
   POLY_EPILOGUE(acc, m, n, z);
 }
 )HIP";
@@ -454,7 +455,7 @@ static bool render_matmul_f32(const MatmulMatch &mm, const MatmulEpilogue &ep, R
   cfg += matmul_k_fn("poly_a_k", mm.ka, K);
   cfg += matmul_k_fn("poly_b_k", mm.kb, K);
   cfg += strf("#define POLY_SIGNATURE %s%s\n", ep.signature.c_str(), S > 1 ? ", float* poly_scratch" : "");
-  cfg += strf("#define POLY_KSPLIT %d\n", S);
+  cfg += strf("#define POLY_KSPLIT %d\n#define POLY_PARTIALS poly_scratch\n", S);
   cfg += ep.code;
   cfg += strf("#define POLY_EPILOGUE(acc, m, n, z) %s\n", ep.call.c_str());
   *out = RenderedKernel();
@@ -537,6 +538,26 @@ bool render_matmul(const MatmulMatch &mm, const MatmulEpilogue &ep, RenderedKern
   int pipe = (BM * BN >= 256 * 256) ? 2 : 3;
   if (const char *e = getenv("POLY_HIP_MM_PIPE")) pipe = atoi(e) == 2 ? 2 : 3;
 
+  // A deep product on so few tiles that half the chip would idle: the K tiles of a tile are
+  // dealt to S workgroups, which leave fp32 partial results in scratch memory, and a second
+  // kernel adds them in split order and runs the epilogue.  S minimises rounds over the
+  // chip / S among the divisors of the K tile count that leave every part 64 tiles or more.
+  int S = 1;
+  size_t part_off = 0;
+  if (!getenv("POLY_HIP_NO_SPLIT_K") && !getenv("POLY_HIP_MM_NOEPI") && M > 64 && N > 64) {
+    const int64_t t = ((M + BM - 1) / BM) * ((N + BN - 1) / BN) * Z, kt = K / BK;
+    double best = 0.75;      // worth a second kernel only from a quarter of the time saved
+    for (int s = 2; s <= 16 && t <= 128; s++) {
+      if (kt % s != 0 || kt / s < 64 || Z * s > 65535) continue;
+      const double r = std::ceil((double)(t * s) / 256.0) / (double)s;
+      if (r < best) { best = r; S = s; }
+    }
+    part_off = (ep.scratch_used + 255) / 256 * 256;
+    if ((double)S * (double)Z * (double)M * (double)N * 4.0 > 1073741824.0) S = 1;
+  }
+  const std::string partials = ep.scratch_type.empty() ? std::string("poly_scratch") : strf("((float*)((char*)poly_scratch + %zuull))", part_off);
+  const std::string signature = ep.signature + (S > 1 && ep.scratch_type.empty() ? ", float* poly_scratch" : "");
+
   auto emit = [&](int bm, int bn, int wvm, int wvn, int pp, RenderedKernel *rk) {
     const int64_t tiles = ((M + bm - 1) / bm) * ((N + bn - 1) / bn);
     if (tiles > 2147483647LL / 2) return reject(__LINE__);
@@ -563,13 +584,19 @@ bool render_matmul(const MatmulMatch &mm, const MatmulEpilogue &ep, RenderedKern
     }
     cfg += matmul_k_fn("poly_a_k", ka, K);
     cfg += matmul_k_fn("poly_b_k", kb, K);
-    cfg += strf("#define POLY_SIGNATURE %s\n", ep.signature.c_str());
+    cfg += strf("#define POLY_SIGNATURE %s\n", signature.c_str());
     cfg += ep.code;
+    if (S > 1) {
+      cfg += strf("#define POLY_KSPLIT %d\n#define POLY_PARTIALS %s\n", S, partials.c_str());
+      cfg += "#define POLY_EP_CONTIG 1\n#define POLY_EP_TYPE float\n#define POLY_EP_VALUE(acc, m, n, z) (acc)\n";
+      cfg += "#define POLY_EP_PTR(m, n, z) (POLY_PARTIALS + (((size_t)poly_ks * POLY_Z + (z)) * POLY_M + (m)) * POLY_N + (n))\n";
+      cfg += "#define POLY_EPILOGUE(acc, m, n, z) *POLY_EP_PTR(m, n, z) = (acc)\n";
+    } else
     if (getenv("POLY_HIP_MM_NOEPI")) cfg += strf("#define POLY_EPILOGUE(acc, m, n, z) do { if (((m) | (n)) == -1) { %s; } } while (0)\n", ep.call.c_str());
     else
     cfg += strf("#define POLY_EPILOGUE(acc, m, n, z) %s\n", ep.call.c_str());
-    const bool split = ep.contiguous_n && !getenv("POLY_HIP_MM_NOEPI") && (ep.out_type == "__bf16" || ep.out_type == "_Float16" || ep.out_type == "float");
-    cfg += strf("#define POLY_EP_CONTIG %d\n", split ? 1 : 0);
+    const bool split = S == 1 && ep.contiguous_n && !getenv("POLY_HIP_MM_NOEPI") && (ep.out_type == "__bf16" || ep.out_type == "_Float16" || ep.out_type == "float");
+    if (S == 1) cfg += strf("#define POLY_EP_CONTIG %d\n", split ? 1 : 0);
     if (split) {
       cfg += strf("#define POLY_EP_TYPE %s\n", ep.out_type.c_str());
       cfg += strf("#define POLY_EP_VALUE(acc, m, n, z) %s\n", ep.value_call.c_str());
@@ -580,7 +607,7 @@ bool render_matmul(const MatmulMatch &mm, const MatmulEpilogue &ep, RenderedKern
     rk->source = std::string(hip_prelude()) + cfg + kMatmulTemplate;
     rk->entry = "poly_k";
     rk->launch.grid[0] = (unsigned)tiles;
-    rk->launch.grid[1] = (unsigned)Z;
+    rk->launch.grid[1] = (unsigned)(Z * S);
     rk->launch.block[0] = (unsigned)(64 * wvm * wvn);
     rk->klass = KernelClass::MATMUL_MFMA;
     rk->strategy = strf("mfma 32x32x16 %s M=%lld N=%lld K=%lld Z=%lld tile %dx%dx%d A:%s B:%s", A.dt == DT_BF16 ? "bf16" : "f16",
@@ -593,6 +620,23 @@ bool render_matmul(const MatmulMatch &mm, const MatmulEpilogue &ep, RenderedKern
     return true;
   };
   if (!emit(BM, BN, WVM, WVN, pipe, out)) return false;
+  if (S > 1) {
+    // the template becomes a first stage; the kernel proper adds the partial results up
+    RenderedKernel::Pre pre{out->source, out->entry, out->launch};
+    out->pres.push_back(pre);
+    out->scratch_bytes = part_off + (size_t)S * (size_t)Z * (size_t)M * (size_t)N * sizeof(float);
+    std::string cfg;
+    cfg += strf("#define POLY_M %lld\n#define POLY_N %lld\n#define POLY_Z %lld\n#define POLY_KSPLIT %d\n", (long long)M, (long long)N, (long long)Z, S);
+    cfg += strf("#define POLY_PARTIALS %s\n#define POLY_SIGNATURE %s\n", partials.c_str(), signature.c_str());
+    cfg += ep.code;
+    cfg += strf("#define POLY_EPILOGUE(acc, m, n, z) %s\n", ep.call.c_str());
+    out->source = std::string(hip_prelude()) + cfg + kSplitKCombine;
+    out->launch = LaunchSpec();
+    out->launch.grid[0] = (unsigned)(((double)Z * M * N + 255) / 256);
+    out->launch.block[0] = 256;
+    out->strategy += strf(", K dealt to %d workgroups per tile, partial results added by a second kernel", S);
+    return true;
+  }
   // Candidates for on-device tuning: the same kernel in the other tile shapes and
   // pipeline depths; the plan times them on its first run when POLY_BEAM is set.
   if (matmul_tuning_enabled() && M > 64 && N > 64 && !(!a_kc && M % 8)) {
@@ -901,14 +945,15 @@ bool try_render_matmul_generic(const KernelGraph &g, const std::string &fn, cons
       m2.md_full = mm.md_full; m2.nd_full = mm.nd_full; m2.zd_full = mm.zd_full;
       MatmulEpilogue ep2 = ep;
       ep2.signature += ", __bf16* poly_scratch";
+      ep2.scratch_type = "__bf16";
+      ep2.scratch_used = scratch_bytes;
       ep2.a_ptr = "((const __bf16*)poly_scratch)";
       ep2.b_ptr = strf("((const __bf16*)((const char*)poly_scratch + %zuull))", off_b);
       RenderedKernel main;
       if (render_matmul(m2, ep2, &main)) {
         *out = main;
-        out->pres.push_back(pre[0]);
-        out->pres.push_back(pre[1]);
-        out->scratch_bytes = scratch_bytes;
+        out->pres.insert(out->pres.begin(), {pre[0], pre[1]});      // planes first, then a split product's first stage
+        out->scratch_bytes = std::max(scratch_bytes, main.scratch_bytes);
         out->flops = 2.0 * (double)M * (double)N * (double)K * (double)Z;
         out->strategy = strf("operands as expressions, written as bf16 planes first (%d + %d planes of K=%lld, %.0f MB): ", parts[0], parts[1],
                              (long long)KP, (double)scratch_bytes / 1e6) + out->strategy;

@@ -62,6 +62,11 @@ struct MatmulEpilogue {
   bool contiguous_n = false;
   int n_params = 0;
   double bytes = 0;    // algorithmic bytes of the whole kernel
+  // When `signature` already ends in a `poly_scratch` parameter (operands staged there by
+  // first-stage kernels): its element type and the bytes in use, so that a split-K product
+  // can put its partial results behind them.  Empty: no such parameter yet.
+  std::string scratch_type;
+  size_t scratch_used = 0;
 };
 // Is element (m, n + 1) of the kernel's output stored right after (m, n), for every n
 // that is not the last of an aligned group of 8?  (store index affine with coefficient 1

@@ -40,6 +40,35 @@ def test_matmul_bf16_layouts(m, n, k, tb):
     c.close()
 
 
+@pytest.mark.parametrize("tb", [False, True])
+def test_matmul_bf16_deep_product_on_few_tiles_is_split_along_k(tb):
+    """A deep product with few output tiles: the K tiles of a tile are dealt to several
+    workgroups and a second kernel adds their fp32 partial results in split order (ragged
+    M and N, so the partial stores meet both edges).  Against the reference, and against
+    the unsplit kernel of the same graph (POLY_HIP_NO_SPLIT_K)."""
+    import os
+    m, n, k = 200, 328, 8192
+    c = R.Ctx()
+    g = np.random.default_rng(31 + tb)
+    A, Bm, O, sink = graphs.matmul_bf16(c, m, n, k, transposed_b=tb)
+    arrays = {A: bf16(g, (m, k), 1.0), Bm: bf16(g, (k, n), 1.0), O: np.zeros(m * n, np.float32)}
+    want = run_ref(c, sink, arrays)
+    got, info = run_hip(c, sink, arrays)
+    assert any("K dealt to" in k_["desc"] and "32x32x16" in k_["desc"] for k_ in info), [k_["desc"] for k_ in info]
+    os.environ["POLY_HIP_NO_SPLIT_K"] = "1"
+    try:
+        got1, info1 = run_hip(c, sink, arrays)
+    finally:
+        del os.environ["POLY_HIP_NO_SPLIT_K"]
+    c.close()
+    assert not any("K dealt to" in k_["desc"] for k_ in info1)
+    w = want[O].astype(np.float64)
+    bound = 1e-4 * float(np.abs(w).mean())
+    assert_close(got[O], want[O], rtol=1e-4, atol=bound, what="split-K vs reference")
+    assert_close(got1[O], want[O], rtol=1e-4, atol=bound, what="unsplit vs reference")
+    assert float(np.abs(got[O].astype(np.float64) - got1[O]).max()) <= 2e-5 * float(np.abs(w).max())
+
+
 def test_matmul_broadcast_batch():
     c = R.Ctx()
     g = np.random.default_rng(11)

@@ -64,16 +64,36 @@ def test_benchmark_plan_kernels_stay_in_bounds(name, hiplib):
 
 @pytest.mark.skipif(not R.available(), reason="reference library not built")
 def test_bf16_plane_kernels_stay_in_bounds(hiplib):
-    """The three kernels of a matmul whose fp32 operand is cut into bf16 planes (two
-    first-stage kernels writing the planes, the 16-bit MFMA template reading them), with a
-    depth that is not a multiple of the K tile."""
+    """The four kernels of a matmul whose fp32 operand is cut into bf16 planes (two
+    first-stage kernels writing the planes, the 16-bit MFMA template reading them with its
+    K tiles dealt to three workgroups per output tile, the kernel adding their partial
+    results behind the planes in scratch memory), with a depth that is not a multiple of
+    the K tile."""
     import numpy as np
     import test_gpu_matmul as T
     c = R.Ctx()
     sink, _, _ = T._planes_case(c, np.random.default_rng(0))
     sched = c.schedule(sink)
     try:
-        assert hostcheck.check_schedule(hiplib, sched) == 3
+        assert hostcheck.check_schedule(hiplib, sched) == 4
+    finally:
+        c.L.poly_schedule_free(sched)
+        c.close()
+
+
+@pytest.mark.skipif(not R.available(), reason="reference library not built")
+@pytest.mark.parametrize("tb", [False, True])
+def test_split_k_matmul_stays_in_bounds(tb, hiplib):
+    """A bf16 product with ragged M and N whose K tiles are dealt to two workgroups per
+    tile: the template writing partial results to scratch memory and the adder."""
+    import graphs
+    c = R.Ctx()
+    _, _, _, sink = graphs.matmul_bf16(c, 200, 328, 8192, transposed_b=tb)
+    sched = c.schedule(sink)
+    try:
+        sp = C.cast(sched, C.POINTER(_ffi.PolySchedule)).contents
+        assert "K dealt to 2" in _ffi.take_string(hiplib.poly_hip_describe(sp.items[0].root, 0))
+        assert hostcheck.check_schedule(hiplib, sched) == 2
     finally:
         c.L.poly_schedule_free(sched)
         c.close()
