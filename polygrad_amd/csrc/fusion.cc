@@ -835,6 +835,7 @@ static bool match_row_chain_impl(const Sched &sc, int a_item, const std::vector<
     const std::vector<int> roots{ph.is_map ? g.stores[0].value : g.n(ph.red).src[0]};
     // vector width along the row
     int V = 1;
+    bool ragged = false;             // vectors up to the last full one, then R mod V lanes take one element each
     {
       int maxsz = 1;
       std::vector<char> mark(g.nodes.size(), 0);
@@ -848,13 +849,22 @@ static bool match_row_chain_impl(const Sched &sc, int a_item, const std::vector<
       for (auto &kv : ph.m.preset) if (kv.second.find("[it]") != std::string::npos) reads_row = true;
       if (reads_row) V = row_V;   // positions must line up with the phase that made the row
       while (V > 1 && (R % V != 0 || R < (int64_t)G * V)) V /= 2;
+      // long rows of an extent that is no multiple of the vector width (a vocabulary of
+      // 50257): vector accesses at element alignment and a scalar tail
+      if (V == 1 && !reads_row && !ph.keeps_row && !getenv("POLY_HIP_NO_RAGGED_VEC")) {
+        int vr = std::max(1, 16 / maxsz);
+        while (vr > 1 && R < (int64_t)G * vr * 16) vr /= 2;
+        if (vr > 1) { V = vr; ragged = true; }
+      }
       if (reads_row && V != row_V) FA_REJECT();
       if (ph.is_map) {
         const int li = g.n(g.n(g.stores[0].index).src[1]).lin;
-        while (V > 1 && (li < 0 || !lin_vec_ok(g, g.lins[(size_t)li], own_f, V) ||
+        while (V > 1 && (li < 0 || !lin_vec_ok(g, g.lins[(size_t)li], own_f, V, ragged) ||
                          dt_size(g.n(g.stores[0].value).dt) != dt_size(g.n(g.stores[0].param).dt))) V /= 2;
       }
+      if (V == 1) ragged = false;
     }
+    const int64_t R_main = ragged ? R - R % V : R;
     const std::string fv = strf("f%d", own_f);           // C name of the position along the row
     Scope L;                          // loop body, one vector per step
     L.parent = &S0;
@@ -887,7 +897,8 @@ static bool match_row_chain_impl(const Sched &sc, int a_item, const std::vector<
       cache.push_back({key, strf("poly_vec<%s,%d>", dt_cname(g.n(node).dt), V), nit});
       return strf("(c%zu[it] = %s)", cache.size() - 1, ld.c_str());
     };
-    if (V > 1) pres = hoist_vector_loads(g, em, roots, own_f, V, fv + "_0", &L, unrolled ? &keep : nullptr);
+    if (ragged && unrolled) FA_REJECT();
+    if (V > 1) pres = hoist_vector_loads(g, em, roots, own_f, V, fv + "_0", &L, unrolled ? &keep : nullptr, ragged);
     // the row loop: positions fv_0 = lane * V, + G * V, ...
     // q: position in the row; the phase's own variable starts there (or, for a flat phase,
     // at the row's first element plus q)
@@ -895,8 +906,26 @@ static bool match_row_chain_impl(const Sched &sc, int a_item, const std::vector<
     const std::string loop_open = unrolled
         ? strf("#pragma unroll\n  for (int it = 0; it < %d; it++) {\n  const int q_0 = lane * %d + it * %d;\n  if (q_0 < %lld) {\n  const int %s_0 = %s;\n", nit, V, G * V,
                (long long)R, fv.c_str(), start.c_str())
-        : strf("  for (int q_0 = lane * %d; q_0 < %lld; q_0 += %d) {\n  const int %s_0 = %s;\n", V, (long long)R, G * V, fv.c_str(), start.c_str());
+        : strf("  for (int q_0 = lane * %d; q_0 < %lld; q_0 += %d) {\n  const int %s_0 = %s;\n", V, (long long)R_main, G * V, fv.c_str(), start.c_str());
     const std::string loop_close = unrolled ? "  }\n  }\n" : "  }\n";
+    // the scalar tail of a ragged row: the phase's value emitted once more for one element
+    auto ragged_tail = [&](int root, const std::function<std::string(Scope *, const std::string &)> &use) {
+      for (int n : pres) em.clear_preset(n);
+      pres.clear();
+      Scope Tl;
+      Tl.parent = &S0;
+      Tl.avail = S0.avail | ((uint64_t)1 << own_f);
+      Tl.indent = 2;
+      em.bind_range(own_f, fv);
+      const std::string v = em.emit(root, &Tl);
+      const std::string last = use(&Tl, v);
+      std::string t = S0.code;       // (row-invariant values the vector form did not need)
+      S0.code.clear();
+      t += strf("  if (lane < %lld) {\n    const int %s = %s%lld + lane;\n", (long long)(R % V), fv.c_str(), flat_base.empty() ? "" : (flat_base + " + ").c_str(),
+                (long long)R_main);
+      t += Tl.code + last + "  }\n";
+      return t;
+    };
     Scope U;                          // one element
     U.parent = &L;
     U.avail = L.avail | ((uint64_t)1 << own_f);
@@ -917,6 +946,8 @@ static bool match_row_chain_impl(const Sched &sc, int a_item, const std::vector<
       loop += L.code;
       loop += strf("#pragma unroll\n    for (int u = 0; u < %d; u++) {\n      const int %s = %s_0 + u;\n", V, fv.c_str(), fv.c_str());
       loop += U.code + "    }\n" + loop_close;
+      if (ragged)
+        loop += ragged_tail(Rn.src[0], [&](Scope *, const std::string &v2) { return strf("    acc = %s;\n", Emitter::reduce_combine(op, Rn.dt, "acc", v2).c_str()); });
       loop += strf("  acc = %s;\n", wave_reduce_call(op, Rn.dt, "acc").c_str());
       if (G == 256) {
         loop += strf("  __shared__ %s red[4];\n  __syncthreads();\n  if ((threadIdx.x & 63) == 0) red[threadIdx.x >> 6] = acc;\n  __syncthreads();\n",
@@ -955,6 +986,11 @@ static bool match_row_chain_impl(const Sched &sc, int a_item, const std::vector<
       loop += U.code + "    }\n";
       if (V > 1 && !ph.keeps_row) loop += strf("    poly_vstore<%s,%d>(data%d + %s, out);\n", odt, V, p, addr.c_str());
       loop += loop_close;
+      if (ragged)
+        loop += ragged_tail(st.value, [&](Scope *tl, const std::string &v2) {
+          const std::string idx = em.emit(g.n(st.index).src[1], tl);
+          return strf("    data%d[%s] = %s;\n", p, idx.c_str(), v2.c_str());
+        });
     }
     if (em.failed() || em.uses_threefry) FA_REJECT();
     std::string cache_params, cache_args;
@@ -986,7 +1022,7 @@ static bool match_row_chain_impl(const Sched &sc, int a_item, const std::vector<
     } else {
       calls += strf("    %s(row, lane%s%s, %s);\n", fn.c_str(), lead_call.c_str(), cache_args.c_str(), call_args(ph.m.item).c_str());
     }
-    strat += strf("%s%s vec%d", pi ? ", " : "", ph.is_map ? "map" : "reduce", V);
+    strat += strf("%s%s vec%d%s", pi ? ", " : "", ph.is_map ? "map" : "reduce", V, ragged ? " unaligned + tail" : "");
   }
   std::string body = strf("extern \"C\" __global__ void __launch_bounds__(256) poly_k(%s) {\n", sig.c_str());
   if (G == 64) {

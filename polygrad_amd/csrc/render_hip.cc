@@ -21,8 +21,8 @@
 
 namespace polyhip {
 
-bool lin_vec_ok(const KernelGraph &g_, const Lin &l, int F, int V) {
-  if (l.c0 % V) return false;
+bool lin_vec_ok(const KernelGraph &g_, const Lin &l, int F, int V, bool any_alignment) {
+  if (l.c0 % V && !any_alignment) return false;
   bool seenF = false;
   for (const Term &t : l.terms) {
     const Atom &a = g_.atoms[(size_t)t.atom];
@@ -31,7 +31,7 @@ bool lin_vec_ok(const KernelGraph &g_, const Lin &l, int F, int V) {
       seenF = true;
     } else {
       if (g_.atom_deps(t.atom) & ((uint64_t)1 << F)) return false;
-      if (t.coef % V) return false;
+      if (t.coef % V && !any_alignment) return false;
     }
   }
   return seenF;
@@ -49,7 +49,7 @@ void mark_reachable(const KernelGraph &g_, int root, std::vector<char> &mark) {
 
 std::vector<int> hoist_vector_loads(const KernelGraph &g_, Emitter &em_, const std::vector<int> &roots, int F, int V,
                                     const std::string &f0, Scope *outer,
-                                    const std::function<std::string(int, const std::string &)> *wrap) {
+                                    const std::function<std::string(int, const std::string &)> *wrap, bool any_alignment) {
   std::vector<char> mark(g_.nodes.size(), 0);
   for (int r : roots) mark_reachable(g_, r, mark);
   std::vector<int> done;
@@ -64,7 +64,7 @@ std::vector<int> hoist_vector_loads(const KernelGraph &g_, Emitter &em_, const s
     if (k.deps & ~(outer->avail | ((uint64_t)1 << F))) continue;
     const KNode &ix = g_.n(k.src[0]);
     int li = g_.n(ix.src[1]).lin;
-    if (li < 0 || !lin_vec_ok(g_, g_.lins[(size_t)li], F, V)) continue;
+    if (li < 0 || !lin_vec_ok(g_, g_.lins[(size_t)li], F, V, any_alignment)) continue;
     if (ix.src.size() >= 3 && (g_.n(ix.src[2]).deps & ((uint64_t)1 << F))) continue;
     if (k.guard >= 0 && (g_.n(k.guard).deps & ((uint64_t)1 << F))) continue;
     if (dt_size(k.dt) * V > 16) continue;
@@ -265,8 +265,8 @@ class Generic {
 
   bool node_under(int root, std::vector<char> &mark) const { mark_reachable(g_, root, mark); return true; }
   std::vector<int> hoist_vector_loads(const std::vector<int> &roots, int F, int V, const std::string &f0,
-                                      Scope *outer, bool) {
-    return polyhip::hoist_vector_loads(g_, em_, roots, F, V, f0, outer);
+                                      Scope *outer, bool, bool any_alignment = false) {
+    return polyhip::hoist_vector_loads(g_, em_, roots, F, V, f0, outer, nullptr, any_alignment);
   }
 
   static void line(std::string &code, int indent, const std::string &s) {
@@ -536,6 +536,7 @@ class Generic {
     int QF = coop_ranges_.back();
     int64_t eF = g_.ranges[(size_t)QF].extent;
     int V = 1;
+    bool ragged = false;
     if (opt_.allow_vectorize) {
       int maxsz = 1;
       std::vector<char> mark(g_.nodes.size(), 0);
@@ -545,6 +546,14 @@ class Generic {
           maxsz = std::max(maxsz, dt_size(g_.n(i).dt));
       V = std::max(1, 16 / maxsz);
       while (V > 1 && (eF % V != 0 || coop_R_ < (int64_t)G * V)) V /= 2;
+      // A single reduce range whose extent is no multiple of the vector width (a vocabulary
+      // of 50257): vectors up to the last full one, wherever the row starts, and the
+      // remaining R mod V elements one lane each.
+      if (V == 1 && coop_ranges_.size() == 1 && !getenv("POLY_HIP_NO_RAGGED_VEC")) {
+        int vr = std::max(1, 16 / maxsz);
+        while (vr > 1 && coop_R_ < (int64_t)G * vr * 4) vr /= 2;
+        if (vr > 1) { V = vr; ragged = true; }
+      }
     }
     // accumulators
     std::string accs;
@@ -575,7 +584,7 @@ class Generic {
     std::vector<int> pres;
     std::string loop_body;
     if (V > 1) {
-      pres = hoist_vector_loads(roots, QF, V, strf("r%d_0", QF), &L, true);
+      pres = hoist_vector_loads(roots, QF, V, strf("r%d_0", QF), &L, true, ragged);
       Scope U;
       U.parent = &L;
       U.avail = L.avail | ((uint64_t)1 << QF);
@@ -603,6 +612,24 @@ class Generic {
       loop_body = L.code;
     }
     for (int n : pres) em_.clear_preset(n);
+    std::string ragged_tail;
+    if (ragged) {
+      Scope Tl;
+      Tl.parent = &S0;
+      Tl.avail = S0.avail | ((uint64_t)1 << QF);
+      Tl.indent = 3;
+      em_.bind_range(QF, strf("r%d", QF));
+      for (int id : top_reduces_) {
+        const KNode &k = g_.n(id);
+        std::string v = em_.emit(k.src[0], &Tl);
+        std::string acc = strf("acc%d", id);
+        line(Tl.code, 3, strf("%s = %s;", acc.c_str(), Emitter::reduce_combine(reduce_op(k), k.dt, acc, v).c_str()));
+      }
+      line(ragged_tail, 2, strf("if (lane < %lld) {", (long long)(coop_R_ % V)));
+      line(ragged_tail, 3, strf("const int r%d = %lld + lane;", QF, (long long)(coop_R_ - coop_R_ % V)));
+      ragged_tail += Tl.code;
+      line(ragged_tail, 2, "}");
+    }
     // S0.code now holds everything hoisted out of the loop (row-invariant values)
     std::string pre_loop = S0.code;
     S0.code.clear();
@@ -660,10 +687,10 @@ class Generic {
       line(body, 1, strf("if (row < %lldll) {", (long long)rows));
     }
     body += decomp + accs + pre_loop;
-    line(body, 2, strf("for (int q0 = lane * %d; q0 < %lld; q0 += %d) {", V, (long long)coop_R_, G * V));
+    line(body, 2, strf("for (int q0 = lane * %d; q0 < %lld; q0 += %d) {", V, (long long)(coop_R_ - (ragged ? coop_R_ % V : 0)), G * V));
     body += qdecomp + loop_body;
     line(body, 2, "}");
-    body += red + tail;
+    body += ragged_tail + red + tail;
     line(body, 1, "}");
     (void)nred;
 
@@ -672,7 +699,7 @@ class Generic {
     out->launch.grid[0] = (unsigned)std::max(1.0, blocks);
     out->launch.block[0] = (unsigned)opt_.block;
     out->klass = KernelClass::ROW_REDUCE;
-    out->strategy = strf("row-reduce G=%d vec%d R=%lld rows=%.0f", G, V, (long long)coop_R_, rows);
+    out->strategy = strf("row-reduce G=%d vec%d%s R=%lld rows=%.0f", G, V, ragged ? " (unaligned, scalar tail)" : "", (long long)coop_R_, rows);
     return body;
   }
 

@@ -180,8 +180,9 @@ class Emitter {
 
 // Pieces of the generic lowering that fused kernels reuse.
 // Can `l` be accessed as a V-wide vector along range ordinal F (unit stride in F, every
-// other contribution a multiple of V)?
-bool lin_vec_ok(const KernelGraph &g, const Lin &l, int F, int V);
+// other contribution a multiple of V)?  With `any_alignment` only the unit stride is asked
+// for: vector loads and stores to global memory need no more than element alignment.
+bool lin_vec_ok(const KernelGraph &g, const Lin &l, int F, int V, bool any_alignment = false);
 void mark_reachable(const KernelGraph &g, int root, std::vector<char> &mark);
 // Emits V-wide vector loads into `outer` for every LOAD under `roots` that is unit-stride
 // along F (starting at the C expression f0) and presets those nodes to "<name>.v[u]";
@@ -190,7 +191,8 @@ void mark_reachable(const KernelGraph &g, int root, std::vector<char> &mark);
 // value kept from an earlier pass over the same addresses).
 std::vector<int> hoist_vector_loads(const KernelGraph &g, Emitter &em, const std::vector<int> &roots, int F, int V,
                                     const std::string &f0, Scope *outer,
-                                    const std::function<std::string(int, const std::string &)> *wrap = nullptr);
+                                    const std::function<std::string(int, const std::string &)> *wrap = nullptr,
+                                    bool any_alignment = false);
 // C expression reducing `v` over the 64 lanes of a wave.
 std::string wave_reduce_call(PolyOps op, DT dt, const std::string &v);
 

@@ -33,6 +33,42 @@ def test_fused_chain_fp32():
     c.close()
 
 
+@pytest.mark.parametrize("cols,dt", [(20001, "f32"), (16387, "f32"), (50257, "f32"), (33333, "bf16")])
+def test_ragged_long_rows_take_unaligned_vectors_and_a_scalar_tail(cols, dt):
+    """Rows whose length is no multiple of the vector width (a vocabulary of 50257): row sum,
+    row max and softmax read vectors at element alignment up to the last full one and leave
+    the remaining elements to single lanes.  Every row starts at a different alignment; the
+    last elements of each row carry the extreme values, so a dropped tail shows."""
+    c = R.Ctx()
+    g = rng(cols)
+    rows = 24
+    shape = (rows, cols)
+    xf = g.uniform(-1, 1, shape).astype(np.float32)
+    xf[:, -1] = 3.0          # the maximum of every row sits in the scalar tail
+    xf[:, -2] = -2.5
+    if dt == "bf16":
+        x = c.buffer(shape, R.BF16, name="x")
+        xv = x.cast(R.F32)
+        xa = R.f32_to_bf16_bits(xf.ravel()).reshape(shape)
+    else:
+        x = c.buffer(shape, name="x")
+        xv = x
+        xa = xf
+    s_out, m_out, o = c.buffer((rows,), name="sum"), c.buffer((rows,), name="max"), c.buffer(shape, name="o")
+    atol = 1e-6 * float(np.abs(xf).sum(axis=1).max())
+    for out, val, zero, what in ((s_out, xv.sum(), np.zeros(rows, np.float32), "sum"), (m_out, xv.max(), np.zeros(rows, np.float32), "max"),
+                                 (o, xv.softmax(), np.zeros(shape, np.float32), "softmax")):
+        sink = c.sink((out, val))
+        sub = {x: xa, out: zero}
+        want = run_ref(c, sink, sub)
+        got, info = run_hip(c, sink, sub)
+        assert any("tail" in k["desc"] for k in info), [k["desc"] for k in info]
+        assert_close(got[out], want[out], rtol=1e-4, atol=atol if what == "sum" else 1e-9, what=f"{what} cols={cols} {dt}")
+        if what == "max":
+            assert np.array_equal(got[out], want[out])
+    c.close()
+
+
 @pytest.mark.parametrize("cols", [8, 100, 128, 1024, 4096, 5000])
 def test_row_reductions_fp32(cols):
     c = R.Ctx()

@@ -82,6 +82,25 @@ def test_bf16_plane_kernels_stay_in_bounds(hiplib):
 
 
 @pytest.mark.skipif(not R.available(), reason="reference library not built")
+@pytest.mark.parametrize("cols,bf", [(20001, False), (50257, False), (33333, True)])
+def test_ragged_row_kernels_stay_in_bounds(cols, bf, hiplib):
+    """Row sum and softmax over rows whose length is no multiple of the vector width:
+    unaligned vector accesses up to the last full vector, single lanes for the rest."""
+    c = R.Ctx()
+    shape = (6, cols)
+    x = c.buffer(shape, R.BF16 if bf else R.F32, name="x")
+    xv = x.cast(R.F32) if bf else x
+    s_out, o = c.buffer((6,), name="s"), c.buffer(shape, name="o")
+    for out, val in ((s_out, xv.sum()), (o, xv.softmax())):
+        sched = c.schedule(c.sink((out, val)))
+        try:
+            assert hostcheck.check_schedule(hiplib, sched) >= 1
+        finally:
+            c.L.poly_schedule_free(sched)
+    c.close()
+
+
+@pytest.mark.skipif(not R.available(), reason="reference library not built")
 @pytest.mark.parametrize("tb", [False, True])
 def test_split_k_matmul_stays_in_bounds(tb, hiplib):
     """A bf16 product with ragged M and N whose K tiles are dealt to two workgroups per
