@@ -838,9 +838,9 @@ class Generic {
     return body;
   }
 
-  // The two kernels of the same reduction with the terms passing through memory: every
-  // term is computed by a thread of its own (the whole chip instead of outputs / 64
-  // workgroups), and the adder only walks a column of finished terms.
+  // The two kernels of the same reduction with the terms passing through memory: a first
+  // kernel computes them, four consecutive terms of an output per thread (the whole chip
+  // instead of outputs / 64 workgroups), and the adder only walks a column of finished terms.
   std::string render_ordered_stage(RenderedKernel *out) {
     const Group &gr = groups_[0];
     const int T = top_reduces_[0];
@@ -861,7 +861,7 @@ class Generic {
     std::string decomp;
     if (first) {
       line(body, 1, "const long long gid = (long long)blockIdx.x * 256 + threadIdx.x;");
-      line(body, 1, strf("if (gid < %.0fll) {", outs * (double)K));
+      line(body, 1, strf("if (gid < %.0fll) {", outs * (double)(K / 4)));
       line(decomp, 2, strf("long long t_ = gid %% %.0fll;", outs));
     } else {
       line(body, 1, "const long long out_id = (long long)blockIdx.x * 64 + threadIdx.x;");
@@ -881,54 +881,73 @@ class Generic {
       Scope L;
       L.parent = &S0;
       L.avail = S0.avail;
-      L.indent = 2;
+      L.indent = 3;
       std::string qdecomp;
-      line(qdecomp, 2, strf("int q_ = (int)(gid / %.0fll);", outs));
+      line(qdecomp, 3, strf("int q_ = (int)(gid / %.0fll) * 4 + e_;", outs));
       for (size_t i = rr.size(); i-- > 0;) {
         const int ord = rr[i];
         const long long e = (long long)g_.ranges[(size_t)ord].extent;
-        if (i == 0) line(qdecomp, 2, strf("const int r%d = q_;", ord));
-        else line(qdecomp, 2, strf("const int r%d = q_ %% %lld; q_ /= %lld;", ord, e, e));
+        if (i == 0) line(qdecomp, 3, strf("const int r%d = q_;", ord));
+        else line(qdecomp, 3, strf("const int r%d = q_ %% %lld; q_ /= %lld;", ord, e, e));
         em_.bind_range(ord, strf("r%d", ord));
         L.avail |= (uint64_t)1 << ord;
       }
       const std::string term = em_.emit(tk.src[0], &L);
-      line(L.code, 2, strf("poly_scratch[gid] = (float)(%s);", term.c_str()));
-      body += decomp + qdecomp + S0.code + L.code;
+      line(L.code, 3, strf("four_[e_] = (float)(%s);", term.c_str()));
+      body += decomp + S0.code;
+      line(body, 2, "poly_f32x4 four_;");
+      line(body, 2, "#pragma unroll");
+      line(body, 2, "for (int e_ = 0; e_ < 4; e_++) {");
+      body += qdecomp + L.code;
+      line(body, 2, "}");
+      line(body, 2, "*(poly_f32x4 *)(poly_scratch + gid * 4) = four_;");
       line(body, 1, "}");
-      out->launch.grid[0] = (unsigned)std::ceil(outs * (double)K / 256.0);
+      out->launch.grid[0] = (unsigned)std::ceil(outs * (double)(K / 4) / 256.0);
       out->launch.block[0] = 256;
       out->klass = KernelClass::ELEMENTWISE;
-      out->strategy = strf("ordered reduce, stage 1: the %.0f x %lld terms, one thread each;", outs, (long long)K);
+      out->strategy = strf("ordered reduce, stage 1: the %.0f x %lld terms, four of an output per thread;", outs, (long long)K);
       return body;
     }
     const std::string acc = strf("acc%d", T);
     std::string loop;
     line(loop, 2, strf("%s %s = %s;", ct, acc.c_str(), Emitter::reduce_identity(rop, tk.dt).c_str()));
     // The additions form one dependent chain; what can overlap is the memory latency of
-    // the terms: 64 are loaded ahead while the previous 64 are added.
-    const long long NB = K / 64;
-    const std::string at = strf("poly_scratch[(long long)(%%s) * %.0fll + col_]", outs);
-    auto term_at = [&](const std::string &k) { std::string e = at; e.replace(e.find("%s"), 2, k); return e; };
-    if (NB > 0) {
-      line(loop, 2, "float cur_[64], nxt_[64];");
+    // the terms.  They lie as [k / 4][output][4], so a thread fetches four of its terms
+    // with one 16-byte load; two sets of 16 such loads alternate, one in flight while the
+    // 64 terms of the other are added (the load after the last pair fetches block 0
+    // again, unused, so that no branch separates a load from the waits that count it).
+    const long long NP = K / 128;
+    line(loop, 2, "const poly_f32x4 *const col4_ = (const poly_f32x4 *)poly_scratch + col_;");
+    auto consume = [&](const char *set) {
+      line(loop, 3, "#pragma unroll");
+      line(loop, 3, "for (int j = 0; j < 16; j++)");
+      line(loop, 3, "#pragma unroll");
+      line(loop, 4, strf("for (int e = 0; e < 4; e++) %s = %s;", acc.c_str(),
+                         Emitter::reduce_combine(rop, tk.dt, acc, strf("(%s)%s[j][e]", ct, set)).c_str()));
+    };
+    if (NP > 0) {
+      line(loop, 2, "poly_f32x4 a_[16], b_[16];");
       line(loop, 2, "#pragma unroll");
-      line(loop, 2, strf("for (int j = 0; j < 64; j++) cur_[j] = %s;", term_at("j").c_str()));
-      line(loop, 2, strf("for (int b = 0; b < %lld; b++) {", NB));
-      line(loop, 3, strf("if (b + 1 < %lld) {", NB));
-      line(loop, 4, "#pragma unroll");
-      line(loop, 4, strf("for (int j = 0; j < 64; j++) nxt_[j] = %s;", term_at("(b + 1) * 64 + j").c_str()));
-      line(loop, 3, "}");
+      line(loop, 2, strf("for (int j = 0; j < 16; j++) a_[j] = col4_[(long long)j * %.0fll];", outs));
+      line(loop, 2, strf("for (int p = 0; p < %lld; p++) {", NP));
       line(loop, 3, "#pragma unroll");
-      line(loop, 3, strf("for (int j = 0; j < 64; j++) %s = %s;", acc.c_str(),
-                         Emitter::reduce_combine(rop, tk.dt, acc, strf("(%s)cur_[j]", ct)).c_str()));
+      line(loop, 3, strf("for (int j = 0; j < 16; j++) b_[j] = col4_[(long long)((2 * p + 1) * 16 + j) * %.0fll];", outs));
+      // (the compiler would gather all 32 loads at the top of the iteration and wait for
+      // them there: the fences keep each set of loads behind the additions before it)
+      line(loop, 3, "__builtin_amdgcn_sched_barrier(0);");
+      consume("a_");
+      line(loop, 3, "__builtin_amdgcn_sched_barrier(0);");
+      line(loop, 3, strf("const int nb_ = p + 1 < %lld ? 2 * p + 2 : 0;", NP));
       line(loop, 3, "#pragma unroll");
-      line(loop, 3, "for (int j = 0; j < 64; j++) cur_[j] = nxt_[j];");
+      line(loop, 3, strf("for (int j = 0; j < 16; j++) a_[j] = col4_[(long long)(nb_ * 16 + j) * %.0fll];", outs));
+      line(loop, 3, "__builtin_amdgcn_sched_barrier(0);");
+      consume("b_");
+      line(loop, 3, "__builtin_amdgcn_sched_barrier(0);");
       line(loop, 2, "}");
     }
-    if (K % 64)
-      line(loop, 2, strf("for (int k = %lld; k < %lld; k++) %s = %s;", NB * 64, (long long)K, acc.c_str(),
-                         Emitter::reduce_combine(rop, tk.dt, acc, strf("(%s)%s", ct, term_at("k").c_str())).c_str()));
+    if (K % 128)
+      line(loop, 2, strf("for (int k = %lld; k < %lld; k++) %s = %s;", NP * 128, (long long)K, acc.c_str(),
+                         Emitter::reduce_combine(rop, tk.dt, acc, strf("(%s)poly_scratch[((long long)(k >> 2) * %.0fll + col_) * 4 + (k & 3)]", ct, outs)).c_str()));
     em_.preset(T, acc);
     std::string tail_stores;
     for (int si : gr.stores) {

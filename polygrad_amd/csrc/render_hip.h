@@ -102,8 +102,9 @@ struct RenderOptions {
   // partial result goes to poly_scratch[output * slice_parts + part].
   int slice_reduce = -1, slice_range = -1, slice_parts = 0;
   // The order-preserving reduction as two kernels: stage 1 writes every term to
-  // poly_scratch[k * outputs + output] (one thread per term, lanes along the outputs),
-  // stage 2 adds them in index order, one thread per output.  0: one kernel.
+  // poly_scratch[((k / 4) * outputs + output) * 4 + k % 4] (four terms per thread, lanes
+  // along the outputs), stage 2 adds them in index order, one thread per output.
+  // 0: one kernel.
   int ordered_stage = 0;
   // Lanes along the reduce range only when some load is contiguous along it, however few
   // rows there are (otherwise: only from 65536 rows up).
