@@ -167,12 +167,14 @@ def test_random_graphs_match_reference(seed):
     assert_close(got[bo], want[bo], rtol=1e-4, atol=1e-5 * max(scale, 1.0), what=f"random graph {seed}")
 
 
-@pytest.mark.parametrize("rows,cols", [(4096, 1024), (512, 192), (1024, 100), (500, 128)])
+@pytest.mark.parametrize("rows,cols", [(4096, 1024), (512, 192), (1024, 100), (500, 128), (544, 192), (608, 64)])
 def test_bf16_column_sums_keep_the_reference_order(rows, cols):
     """Sums over the rows of a bf16 matrix accumulate in bf16: every addition rounds, so the
-    result depends on the order.  The order-preserving lowering (terms computed by four
-    waves, added in index order by one) must give the reference's bits; so must whatever
-    lowering takes a shape it declines."""
+    result depends on the order.  The order-preserving lowering (a kernel that writes the
+    terms, four per thread, and one that adds them in index order: blocks of 128 terms
+    through alternating load sets, then a tail of single terms when the row count is no
+    multiple of 128) must give the reference's bits; so must whatever lowering takes a
+    shape it declines."""
     c = R.Ctx()
     g = rng(11)
     x = c.buffer((rows, cols), R.BF16, name="x")

@@ -119,7 +119,7 @@ def test_split_k_matmul_stays_in_bounds(tb, hiplib):
 
 
 @pytest.mark.skipif(not R.available(), reason="reference library not built")
-@pytest.mark.parametrize("rows,cols", [(512, 192), (1024, 100)])
+@pytest.mark.parametrize("rows,cols", [(512, 192), (1024, 100), (544, 192)])
 def test_ordered_column_sum_stays_in_bounds(rows, cols, hiplib):
     """The order-preserving bf16 column sum (a kernel that writes the terms, one that adds
     them in order), with a column count that leaves the adder's last workgroup partly idle."""
