@@ -128,6 +128,12 @@ class Generic {
     std::string body;
     bool coop = false;
     if (n_loop_reduces() > 0 && opt_.allow_coop_reduce && groups_.size() == 1 && opt_.reduce_override.empty()) coop = plan_coop();
+    if (coop && opt_.ordered_stage) {
+      // the cooperative form is the better lowering; rendering it under a stage number
+      // would hand back the whole kernel as "stage one" and again as "stage two"
+      *err = "not an ordered reduction";
+      return false;
+    }
     if (coop) {
       body = render_coop(out);
     } else if (plan_ordered()) {
