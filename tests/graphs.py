@@ -63,8 +63,10 @@ def _layernorm(x, w, b, eps, wdt):
     return y * w.reshape(bc).expand(x.shape) + b.reshape(bc).expand(x.shape)
 
 
-def gpt2_forward(c, cfg, wdt=R.BF16):
-    """Returns (sink, bufs) where bufs maps names to buffer T's; logits go to bufs['output']."""
+def gpt2_forward(c, cfg, wdt=R.BF16, hidden_only=False):
+    """Returns (sink, bufs) where bufs maps names to buffer T's; logits go to bufs['output'].
+    With hidden_only the graph ends after the last block: the residual stream [B, T, D] goes
+    to bufs['hidden'] and the final LayerNorm and the vocabulary projection are left out."""
     V, D, H, L, T, B = cfg.vocab, cfg.d_model, cfg.n_head, cfg.n_layer, cfg.ctx, cfg.batch
     hd = D // H
     bufs = {}
@@ -132,6 +134,9 @@ def gpt2_forward(c, cfg, wdt=R.BF16):
         ff = _linear(ff, lp["fc2_w"], lp["fc2_b"], wdt).contiguous()
         h = (h + ff).contiguous()
 
+    if hidden_only:
+        hidden = P("hidden", (B, T, D))
+        return c.sink((hidden, h)), bufs
     h = _layernorm(h, lnf_w, lnf_b, cfg.eps, wdt).contiguous()
     wte_t = wte.reshape((V, D)).permute((1, 0))
     if wdt != R.F32:

@@ -22,13 +22,13 @@ TOL = {
     # attention: the default single-pass kernel rounds exp-terms where the reference rounds
     # probabilities; for the first queries (a handful of keys, outputs up to 1) that is two
     # 16-bit steps of the output scale.  The exact two-pass form is held to 2e-3 below.
-    "mlp_train_b32": (1e-4, 1e-5), "attention_bf16_t256": (2e-2, 8e-3), "bf16_matmul_gelu": (2e-2, 2e-3),
+    "mlp_train_b32": (1e-4, 1e-5), "attention_bf16_t256": (2e-2, 8e-3), "attention_bf16_t1024": (2e-2, 8e-3), "bf16_matmul_gelu": (2e-2, 2e-3),
     "bf16_layernorm_rows": (2e-2, 2e-3),
 }
 # plans that update their inputs in place: a second run would start from other parameters
 STATEFUL = {"mlp_train_b32"}
 # fixtures whose plan must come out as one of the fused kernel groups
-FUSED = {"attention_bf16_t256": "attention-mfma", "bf16_matmul_gelu": "lookup table", "bf16_layernorm_rows": "row chain of 3"}
+FUSED = {"attention_bf16_t256": "attention-mfma", "attention_bf16_t1024": "attention-mfma", "bf16_matmul_gelu": "lookup table", "bf16_layernorm_rows": "row chain of 3"}
 
 
 def run_fixture_on_gpu(fx, env_flags=None):
@@ -62,10 +62,11 @@ def test_fixture_on_gpu(name):
             assert_close(F.as_float(got[slot]), F.as_float(want), rtol=rtol, atol=atol, what=f"{name} slot {slot} ({fx.plan.names[slot]})")
 
 
-def test_attention_fixture_exact_form(monkeypatch):
+@pytest.mark.parametrize("name", ["attention_bf16_t256", "attention_bf16_t1024"])
+def test_attention_fixture_exact_form(monkeypatch, name):
     """The two-pass attention kernel keeps every rounding of the unfused kernels."""
     monkeypatch.setenv("POLY_HIP_EXACT_ATTENTION", "1")
-    fx = F.Fixture("attention_bf16_t256")
+    fx = F.Fixture(name)
     got, info = run_fixture_on_gpu(fx)
     assert any("two passes" in k["desc"] for k in info), [k["desc"] for k in info]
     for slot in fx.external:
