@@ -38,6 +38,19 @@ int poly_hip_lower_item(PolyCtx *ctx, PolyUOp *scheduled_root, const char *fn_na
  * without waiting; copy_out / poly_hip_sync make results visible. */
 int poly_hip_execute(PolyRunner *runner, void **args, int n_args);
 
+/* No counterpart in the reference.  For callers that cannot allocate device memory
+ * (code under HIP graph capture, tight serving loops, harnesses that forbid hipMalloc):
+ * poly_hip_execute for a runner whose kernel runs in two stages (partial sums, split-K
+ * accumulators, operand planes), with the stage-one results in a static device array of
+ * POLY_HIP_STATIC_SCRATCH_BYTES inside the library instead of memory the runner
+ * allocates on its first poly_hip_execute.  Calls no hipMalloc/hipFree once
+ * poly_hip_init() (or a first call on the device) has looked the array up.  Returns -1
+ * with a "polygrad: execute_static:" message when the kernel needs more scratch than the
+ * array holds; a one-stage kernel is simply launched.  Every call on a GPU uses the
+ * same array: calls that overlap on one GPU (other streams, other threads) race. */
+#define POLY_HIP_STATIC_SCRATCH_BYTES (32u << 20)
+int poly_hip_execute_static(PolyRunner *runner, void **args, int n_args);
+
 /* Replaces cuda_free_runner (src/exec_plan.c:611-617). */
 void poly_hip_free_runner(PolyRunner *runner);
 

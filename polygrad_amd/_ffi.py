@@ -72,6 +72,7 @@ SYMBOLS = {
     "poly_hip_backend_desc": (C.POINTER(PolyBackendDesc), []),
     "poly_hip_lower_item": (C.c_int, [C.c_void_p, C.c_void_p, C.c_char_p, C.POINTER(PolyRunner)]),
     "poly_hip_execute": (C.c_int, [C.POINTER(PolyRunner), C.POINTER(C.c_void_p), C.c_int]),
+    "poly_hip_execute_static": (C.c_int, [C.POINTER(PolyRunner), C.POINTER(C.c_void_p), C.c_int]),
     "poly_hip_free_runner": (None, [C.POINTER(PolyRunner)]),
     "poly_hip_get_allocator": (C.POINTER(PolyAllocator), []),
     "poly_hip_init": (C.c_int, []),

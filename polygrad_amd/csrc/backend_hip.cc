@@ -2,11 +2,20 @@
 // execute / free_runner / get_allocator), the allocator, the runtime wrappers
 // and the render-only entry points.  Declarations and the reference interfaces
 // they replace are in include/polygrad_hip.h.
+#include <hip/hip_runtime.h>
+
 #include <cstdlib>
 #include <cstring>
 
 #include "polygrad_hip.h"
 #include "runtime_hip.h"
+
+// Scratch memory of poly_hip_execute_static: stage-one results of a two-stage kernel go
+// here instead of into memory the runner allocates.  Every GPU the library runs on holds
+// its own copy of the array, at its own address, until the process ends.  In host code
+// the name below only stands for the symbol; the device address comes from
+// hipGetSymbolAddress (static_scratch()).
+static __device__ __align__(256) unsigned char poly_static_scratch[POLY_HIP_STATIC_SCRATCH_BYTES];
 
 namespace polyhip {
 
@@ -94,8 +103,9 @@ HipRunner *runner_from_rendered(const RenderedKernel &rk, const char *fn_name, b
       if (!p) { runner_destroy(r); return nullptr; }
       r->pres.push_back(p);
     }
-    r->scratch = runtime_alloc(r->rk.scratch_bytes);
-    if (!r->scratch) { runner_destroy(r); return nullptr; }
+    // the scratch memory itself is allocated by the first ordinary launch
+    // (runner_ensure_scratch): a runner that only ever runs on scratch memory handed in
+    // from outside never holds any of its own
   }
   for (const RenderedKernel::Table &t : r->rk.tables) {
     std::shared_ptr<void> tab = runtime_table(t.source, t.entry, t.bytes, t.launch);
@@ -128,6 +138,13 @@ int runner_use_variant(HipRunner *r, int idx) {
   return 0;
 }
 
+int runner_ensure_scratch(HipRunner *r) {
+  if (!r || r->pres.empty() || r->scratch) return 0;
+  r->scratch = runtime_alloc(r->rk.scratch_bytes);
+  r->owns_scratch = true;
+  return r->scratch ? 0 : -1;
+}
+
 void runner_share_scratch(HipRunner *r, void *pool) {
   if (!r || !pool || r->rk.scratch_bytes == 0) return;
   if (r->scratch && r->owns_scratch) runtime_free(r->scratch);
@@ -146,7 +163,7 @@ void runner_destroy(HipRunner *r) {
   delete r;
 }
 
-int runner_launch(HipRunner *r, void **args, int n_args) {
+int runner_launch(HipRunner *r, void **args, int n_args, void *scratch_from_caller) {
   const int np = r->rk.n_params, nv = r->rk.n_vars;
   if (n_args < np + nv) {
     log_err("execute", "%s: expected %d args, got %d", r->name.c_str(), np + nv, n_args);
@@ -169,7 +186,12 @@ int runner_launch(HipRunner *r, void **args, int n_args) {
     r->arg_ptrs[(size_t)(np + nv + t)] = &r->ptr_store[(size_t)(np + nv + t)];
   }
   if (!r->pres.empty()) {
-    r->ptr_store[(size_t)(np + nv + nt)] = r->scratch;
+    void *scratch = scratch_from_caller;
+    if (!scratch) {
+      if (runner_ensure_scratch(r) != 0) { log_err("execute", "%s: no scratch memory", r->name.c_str()); return -1; }
+      scratch = r->scratch;
+    }
+    r->ptr_store[(size_t)(np + nv + nt)] = scratch;
     r->arg_ptrs[(size_t)(np + nv + nt)] = &r->ptr_store[(size_t)(np + nv + nt)];
     for (size_t i = 0; i < r->pres.size(); i++)
       if (program_launch(r->pres[i], r->arg_ptrs.data(), r->rk.pres[i].launch) != 0) return -1;
@@ -182,14 +204,14 @@ int runner_launch(HipRunner *r, void **args, int n_args) {
   r->arg_ptrs[(size_t)(np + nv + nt)] = &r->ptr_store[(size_t)(np + nv + nt)];
   for (size_t gi = 0; gi < r->guards.size(); gi++) {
     const RenderedKernel::Guard &gd = r->rk.guards[gi];
-    std::vector<void *> gargs;
-    void *flagp = r->flag;
-    gargs.push_back(&flagp);
-    std::vector<void *> vals;
-    vals.reserve(gd.arg_params.size());
-    for (int p : gd.arg_params) vals.push_back(args[p]);
-    for (size_t i = 0; i < vals.size(); i++) gargs.push_back(&vals[i]);
-    if (program_launch(r->guards[gi], gargs.data(), gd.launch) != 0) return -1;
+    enum { kMaxGuardArgs = 8 };     // a guard reads one or two buffers; no heap use per launch
+    if (gd.arg_params.size() > kMaxGuardArgs) { log_err("execute", "%s: guard with %zu arguments", r->name.c_str(), gd.arg_params.size()); return -1; }
+    void *vals[kMaxGuardArgs + 1];
+    void *gargs[kMaxGuardArgs + 1];
+    vals[0] = r->flag;
+    gargs[0] = &vals[0];
+    for (size_t i = 0; i < gd.arg_params.size(); i++) { vals[i + 1] = args[gd.arg_params[i]]; gargs[i + 1] = &vals[i + 1]; }
+    if (program_launch(r->guards[gi], gargs, gd.launch) != 0) return -1;
   }
   if (program_launch(r->main, r->arg_ptrs.data(), r->rk.launch) != 0) return -1;
   return program_launch(r->fallback, r->arg_ptrs.data(), r->rk.fallback_launch);
@@ -199,9 +221,34 @@ int runner_launch(HipRunner *r, void **args, int n_args) {
 
 using namespace polyhip;
 
+// Device address of poly_static_scratch on the current device, looked up once per device
+// (with that device current) and kept; NULL after an error message when the lookup fails.
+static void *static_scratch() {
+  enum { kMaxDevices = 64 };
+  static void *ptr_of[kMaxDevices];
+  int dev = -1;
+  if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= kMaxDevices) {
+    log_err("execute_static", "no current HIP device");
+    return nullptr;
+  }
+  if (!ptr_of[dev]) {
+    void *p = nullptr;
+    hipError_t e = hipGetSymbolAddress(&p, HIP_SYMBOL(poly_static_scratch));
+    if (e != hipSuccess || !p) {
+      log_err("execute_static", "hipGetSymbolAddress failed: %s", hipGetErrorString(e));
+      return nullptr;
+    }
+    ptr_of[dev] = p;
+  }
+  return ptr_of[dev];
+}
+
 extern "C" {
 
-int poly_hip_init(void) { return runtime_init(); }
+int poly_hip_init(void) {
+  if (runtime_init() != 0) return -1;
+  return static_scratch() ? 0 : -1;
+}
 int poly_hip_available(void) { return runtime_init() == 0 ? 1 : 0; }
 void *poly_hip_alloc(size_t nbytes) { return runtime_alloc(nbytes); }
 void poly_hip_free(void *p) { runtime_free(p); }
@@ -257,6 +304,21 @@ int poly_hip_lower_item(PolyCtx *ctx, PolyUOp *scheduled_root, const char *fn_na
 int poly_hip_execute(PolyRunner *runner, void **args, int n_args) {
   if (!runner || !runner->handle) { log_err("execute", "runner has no handle"); return -1; }
   return runner_launch((HipRunner *)runner->handle, args, n_args);
+}
+
+int poly_hip_execute_static(PolyRunner *runner, void **args, int n_args) {
+  if (!runner || !runner->handle) { log_err("execute_static", "runner has no handle"); return -1; }
+  HipRunner *r = (HipRunner *)runner->handle;
+  if (r->rk.scratch_bytes > (size_t)POLY_HIP_STATIC_SCRATCH_BYTES) {
+    log_err("execute_static", "%s needs %zu bytes of scratch memory, the static array holds %u", r->name.c_str(),
+            r->rk.scratch_bytes, (unsigned)POLY_HIP_STATIC_SCRATCH_BYTES);
+    return -1;
+  }
+  void *scratch = static_scratch();
+  if (!scratch) return -1;
+  // Stage one writes every scratch element stage two reads, so what an earlier call left
+  // in the array needs no clearing.
+  return runner_launch(r, args, n_args, scratch);
 }
 
 void poly_hip_free_runner(PolyRunner *runner) {

@@ -299,6 +299,8 @@ PolyHipPlan *poly_hip_compile_schedule(PolyCtx *ctx, const PolySchedule *s) {
       if (!plan->scratch_pool) return nullptr;
       for (Unit &u : plan->units) runner_share_scratch(u.runner, plan->scratch_pool);
     }
+    // a lone user owns its scratch memory; it must exist before the launches are captured
+    for (Unit &u : plan->units) if (runner_ensure_scratch(u.runner) != 0) return nullptr;
   }
   plan->kargs.resize((size_t)n_units);
   plan->var_vals.resize((size_t)n_units);

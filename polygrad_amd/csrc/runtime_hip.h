@@ -54,7 +54,13 @@ HipRunner *runner_from_rendered(const RenderedKernel &rk, const char *fn_name, b
 // Replaces the runner's own scratch memory by `pool` (at least rk.scratch_bytes large, owned
 // by the caller, who runs the runners sharing it one after the other on the stream).
 void runner_share_scratch(HipRunner *r, void *pool);
-int runner_launch(HipRunner *r, void **args, int n_args);
+// Allocates the runner's own scratch memory if its kernel runs in two stages and it has
+// none yet (neither its own nor a shared pool).  Launches under stream capture need it in
+// place beforehand.
+int runner_ensure_scratch(HipRunner *r);
+// `scratch_from_caller`, when non-NULL, is used as the two-stage scratch memory of this
+// launch (at least rk.scratch_bytes large) and the runner allocates none of its own.
+int runner_launch(HipRunner *r, void **args, int n_args, void *scratch_from_caller = nullptr);
 // Switches the runner to rk.variants[idx] (compiles it if needed); the runner is unchanged
 // when that fails.
 int runner_use_variant(HipRunner *r, int idx);
