@@ -112,8 +112,8 @@ int poly_hip_check_index_simplification(PolyUOp *scheduled_root, int samples);
 
 /* MI355X-native counterparts of poly_compile_schedule / poly_compiled_plan_run /
  * poly_compiled_plan_free.  Differences from the reference, all internal:
- * intermediates that are dead share memory, nothing is zero-filled per run
- * (every intermediate is fully written by its producer), launches are
+ * intermediates that are dead share memory, only the intermediates that their
+ * producers leave holes in are cleared per run (poly_hip_unwritten_slots), launches are
  * asynchronous on one stream and the launch sequence is replayed from a
  * hipGraph when the bound pointers repeat. */
 typedef struct PolyHipPlan PolyHipPlan;
@@ -145,6 +145,13 @@ int poly_hip_fused_groups(const PolySchedule *schedule, int index, char **source
  * launch_out[0..3] = grid x, y, z and workgroup size.  Returns the number of buffer
  * arguments, <0 on error.  No reference counterpart. */
 int poly_hip_fused_group_launch(const PolySchedule *schedule, int index, int *slots_out, int cap, int *launch_out);
+/* Intermediate slots of `schedule` that its kernels do not write completely (padded or
+ * gated stores): poly_hip_compile_schedule clears each of them with a fill kernel right
+ * before its first use on every run, which is what keeps the reference's rule that an
+ * intermediate reads as zero where nothing was stored (src/exec_plan.c:946-963 zeroes
+ * all of them, every run).  At most cap slot numbers go to slots_out; returns how many
+ * there are, <0 on a malformed schedule.  Needs no device. */
+int poly_hip_unwritten_slots(const PolySchedule *schedule, int *slots_out, int cap);
 /* Introspection for benches and tests. */
 int poly_hip_plan_n_kernels(const PolyHipPlan *plan);
 /* Fills at most cap entries; per kernel (in execution order): class id

@@ -576,14 +576,20 @@ static Val eval_load(Kern *k, Node *n) {
 static Val eval_reduce(Kern *k, Node *n, int id) {
   (void)id;
   PolyOps op = reduce_op_of(n->u);
-  int nr = n->n_src - 1;
+  int nr = 0;
   int ords[16];
   int64_t ext[16];
-  if (nr > 16) { snprintf(k->err, sizeof(k->err), "REDUCE over more than 16 ranges"); Val z; z.u = 0; return z; }
-  for (int i = 0; i < nr; i++) {
-    ords[i] = range_ord(k, n->src[i + 1]);
-    ext[i] = eval(k, k->nodes[n->src[i + 1]].src[0]).i;
+  if (n->n_src - 1 > 16) { snprintf(k->err, sizeof(k->err), "REDUCE over more than 16 ranges"); Val z; z.u = 0; return z; }
+  /* only RANGE sources loop; an axis of extent 1 may arrive as a constant instead
+   * (src/codegen.c:1431-1439), and with no loop at all the result is the value itself,
+   * not identity-op-value (src/codegen.c:1444-1450) */
+  for (int i = 1; i < n->n_src; i++) {
+    if (k->nodes[n->src[i]].u->op != POLY_OP_RANGE) continue;
+    ords[nr] = range_ord(k, n->src[i]);
+    ext[nr] = eval(k, k->nodes[n->src[i]].src[0]).i;
+    nr++;
   }
+  if (nr == 0) return eval(k, n->src[0]);
   Val acc = reduce_identity(op, n->ty);
   int64_t total = 1;
   for (int i = 0; i < nr; i++) total *= ext[i] > 0 ? ext[i] : 0;

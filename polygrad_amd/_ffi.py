@@ -98,6 +98,7 @@ SYMBOLS = {
     "poly_hip_plan_free": (None, [C.c_void_p]),
     "poly_hip_fused_groups": (C.c_int, [C.c_void_p, C.c_int, C.POINTER(C.c_void_p), C.POINTER(C.c_int)]),
     "poly_hip_fused_group_launch": (C.c_int, [C.c_void_p, C.c_int, C.POINTER(C.c_int), C.c_int, C.POINTER(C.c_int)]),
+    "poly_hip_unwritten_slots": (C.c_int, [C.c_void_p, C.POINTER(C.c_int), C.c_int]),
     "poly_hip_plan_n_kernels": (C.c_int, [C.c_void_p]),
     "poly_hip_plan_kernel_info": (C.c_int, [C.c_void_p, C.c_int, C.POINTER(C.c_int), C.POINTER(C.c_double), C.POINTER(C.c_double)]),
     "poly_hip_plan_profile": (C.c_int, [C.c_void_p, C.POINTER(C.c_void_p), C.c_int, C.POINTER(C.c_float), C.c_int]),

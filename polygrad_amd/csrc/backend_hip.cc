@@ -113,6 +113,7 @@ HipRunner *runner_from_rendered(const RenderedKernel &rk, const char *fn_name, b
     r->tables.push_back(tab);
   }
   size_t n = (size_t)r->rk.n_params + (size_t)r->rk.n_vars + r->rk.tables.size() + 2;
+  r->vetted.assign((size_t)r->rk.n_params, nullptr);
   r->ptr_store.resize(n);
   r->var_store.resize(n);
   r->arg_ptrs.resize(n);
@@ -171,6 +172,18 @@ int runner_launch(HipRunner *r, void **args, int n_args, void *scratch_from_call
   }
   for (int i = 0; i < np; i++) {
     if (!args[i]) { log_err("execute", "%s: null buffer for param %d", r->name.c_str(), i); return -1; }
+    // The reference's callers hand some slots over as host addresses whatever the device
+    // (constants of the frontend's registry, src/frontend.c:2231-2232; the loss and the
+    // bias corrections of a training step, src/instance.c:1299-1311).  A kernel would
+    // fault on them: refuse, once per new pointer.
+    if (args[i] != r->vetted[(size_t)i]) {
+      if (!runtime_device_can_read(args[i])) {
+        log_err("execute", "%s: param %d (%p) is not device memory; upload it with the allocator's copy_in first",
+                r->name.c_str(), i, args[i]);
+        return -1;
+      }
+      r->vetted[(size_t)i] = args[i];
+    }
     r->ptr_store[(size_t)i] = args[i];
     r->arg_ptrs[(size_t)i] = &r->ptr_store[(size_t)i];
   }
@@ -367,8 +380,7 @@ char *poly_hip_render(PolyUOp *scheduled_root, const char *fn_name, int flags, i
 char *poly_hip_describe(PolyUOp *scheduled_root, int flags) {
   RenderedKernel rk;
   if (!scheduled_root || !render_root(scheduled_root, "kernel", flags, &rk)) return nullptr;
-  static const char *const kn[] = {"elementwise", "row-reduce", "thread-reduce", "matmul-mfma", "gather", "copy"};
-  return dup_string(strf("%s: %s bytes=%.0f flops=%.0f grid=%u,%u,%u block=%u", kn[(int)rk.klass],
+  return dup_string(strf("%s: %s bytes=%.0f flops=%.0f grid=%u,%u,%u block=%u", kernel_class_name(rk.klass),
                          rk.strategy.c_str(), rk.bytes, rk.flops, rk.launch.grid[0], rk.launch.grid[1],
                          rk.launch.grid[2], rk.launch.block[0]));
 }

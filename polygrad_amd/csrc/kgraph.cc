@@ -417,14 +417,28 @@ bool KernelGraph::build(const PolyUOp *root) {
   for (int i = 0; i < (int)nodes.size(); i++) {
     KNode &k = nodes[(size_t)i];
     if (k.op != POLY_OP_REDUCE) continue;
-    if (k.src.size() < 2) { error = "REDUCE without ranges"; return false; }
+    if (k.src.empty()) { error = "REDUCE without a value"; return false; }
     if (k.u->arg.kind != POLY_ARG_INT && k.u->arg.kind != POLY_ARG_OPS) {
       error = "REDUCE without an op argument"; return false;
     }
+    // Axes of extent 1 arrive as constants in place of ranges (or as no source at all); only
+    // real RANGEs make a loop, as in the reference's lowering (src/codegen.c:1431-1439).
+    std::vector<int> kept{k.src[0]};
     for (size_t s = 1; s < k.src.size(); s++) {
       auto it = range_ord.find(k.src[s]);
-      if (it == range_ord.end()) { error = "REDUCE source is not a RANGE"; return false; }
+      if (it == range_ord.end()) {
+        if (nodes[(size_t)k.src[s]].op == POLY_OP_CONST) continue;
+        error = "REDUCE source is neither a RANGE nor a constant";
+        return false;
+      }
       ranges[(size_t)it->second].is_reduce = true;
+      kept.push_back(k.src[s]);
+    }
+    k.src = kept;
+    if (k.src.size() == 1) {
+      // nothing to loop over: the value itself, not identity-op-value (src/codegen.c:1444-1450)
+      k.op = POLY_OP_CAST;
+      continue;
     }
     reduces.push_back(i);
   }

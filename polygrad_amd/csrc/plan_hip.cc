@@ -66,6 +66,8 @@ struct PolyHipPlan {
   std::vector<void *> slot_ptr;              // device pointer per slot (intermediates fixed)
   std::vector<size_t> slot_off;
   std::vector<char> slot_needs_zero;
+  std::vector<void *> vetted_slot;              // per external slot: the last pointer found to be device memory
+  std::vector<std::vector<int>> fills_before;   // per unit: slots to clear right before it runs
   void *arena = nullptr;
   size_t arena_bytes = 0;
   void *scratch_pool = nullptr;              // shared by the two-stage kernels of the plan (they run one after the other)
@@ -94,12 +96,14 @@ namespace {
 
 size_t align_up(size_t v, size_t a) { return (v + a - 1) / a * a; }
 
-// Does the producer of `slot` write every element?  Counts, over every STORE
-// into the slot's PARAM, the product of the extents of the store's ranges when
-// the store is ungated and its index is injective enough to be a full cover
-// (affine with non-zero coefficient on every range).
+// Do the producers of `slot` write every element?  Every ungated STORE into the slot's
+// PARAM whose index is affine in its ranges with strides that nest (sorted by stride,
+// each stride is the previous stride times the previous extent, the smallest is 1)
+// writes exactly one contiguous interval of elements; the slot is covered when the union
+// of those intervals is [0, numel).  Gated stores, strided stores and indices with
+// divisions count for nothing: the answer errs towards "needs a fill".
 bool slot_fully_written(const PolySchedule *s, int slot, const std::vector<KernelGraph> &graphs) {
-  double covered = 0;
+  std::vector<std::pair<int64_t, int64_t>> spans;    // [first, end)
   for (int k = 0; k < s->n_items; k++) {
     const PolyExecItem &it = s->items[k];
     const KernelGraph &g = graphs[(size_t)k];
@@ -109,35 +113,68 @@ bool slot_fully_written(const PolySchedule *s, int slot, const std::vector<Kerne
       if (st.gate >= 0) continue;
       int li = g.n(g.n(st.index).src[1]).lin;
       if (li < 0) continue;
-      double n = 1;
+      const Lin &l = g.lins[(size_t)li];
+      if (!g.lin_is_affine(l)) continue;
+      std::vector<std::pair<int64_t, int64_t>> dims;   // (|stride|, extent)
+      int64_t base = l.c0;
       bool ok = true;
+      uint64_t seen = 0;
       for (int r : st.ranges) {
         bool aff;
-        int64_t c = g.lin_range_coef(g.lins[(size_t)li], r, &aff);
-        if (!aff || c == 0 || g.ranges[(size_t)r].extent < 0) { ok = false; break; }
-        n *= (double)g.ranges[(size_t)r].extent;
+        int64_t c = g.lin_range_coef(l, r, &aff);
+        const int64_t ext = g.ranges[(size_t)r].extent;
+        if (!aff || ext <= 0) { ok = false; break; }
+        seen |= 1ull << r;
+        if (c == 0 || ext == 1) continue;              // rewrites the same elements / a single value
+        if (c < 0) { base += c * (ext - 1); c = -c; }  // walks downwards: the interval starts at its last step
+        dims.push_back({c, ext});
       }
-      if (ok) covered += n;
+      // anything else the index depends on (a variable, a range of an enclosing loop)
+      if (ok && (g.lin_deps(l) & ~seen) != 0) ok = false;
+      if (ok) for (const Term &t : l.terms) if (g.atoms[(size_t)t.atom].kind != Atom::RANGE) ok = false;
+      if (!ok) continue;
+      std::sort(dims.begin(), dims.end());
+      int64_t expect = 1;
+      for (const auto &d : dims) {
+        if (d.first != expect) { ok = false; break; }
+        expect *= d.second;
+      }
+      if (ok) spans.push_back({base, base + expect});
     }
   }
-  return covered >= (double)s->buf_slots[slot].numel;
+  std::sort(spans.begin(), spans.end());
+  int64_t covered_to = 0;
+  for (const auto &sp : spans) {
+    if (sp.first > covered_to) break;
+    covered_to = std::max(covered_to, sp.second);
+  }
+  return covered_to >= s->buf_slots[slot].numel;
+}
+
+// The fill kernel over one slot (a slot whose producers leave holes reads as zero there,
+// as every intermediate does in the reference, src/exec_plan.c:946-963).
+int launch_fill(PolyHipPlan *plan, int slot) {
+  const PolySchedule *s = plan->sched;
+  void *p = plan->slot_ptr[(size_t)slot];
+  long long words = (long long)(align_up((size_t)std::max<int64_t>(s->buf_slots[slot].nbytes, 4), 4) / 4);
+  void *args[2] = {&p, &words};
+  LaunchSpec ls;
+  ls.grid[0] = (unsigned)std::min<long long>((words + 255) / 256, 65536);
+  return program_launch(plan->fill, args, ls);
+}
+
+// Launches unit `u` after the fills that belong in front of it.  A slot shares its bytes
+// with intermediates that die before its first use, so it can only be cleared then.
+int launch_unit(PolyHipPlan *plan, size_t u) {
+  for (int slot : plan->fills_before[u])
+    if (launch_fill(plan, slot) != 0) return -1;
+  std::vector<void *> &a = plan->kargs[u];
+  return runner_launch(plan->units[u].runner, a.data(), (int)a.size());
 }
 
 int enqueue_all(PolyHipPlan *plan) {
-  const PolySchedule *s = plan->sched;
-  // zero-fill the few slots whose producers leave holes
-  for (int i = 0; i < s->n_buf_slots; i++) {
-    if (!plan->slot_needs_zero[(size_t)i]) continue;
-    void *p = plan->slot_ptr[(size_t)i];
-    long long words = (long long)(align_up((size_t)std::max<int64_t>(s->buf_slots[i].nbytes, 4), 4) / 4);
-    void *args[2] = {&p, &words};
-    LaunchSpec ls;
-    ls.grid[0] = (unsigned)std::min<long long>((words + 255) / 256, 65536);
-    if (program_launch(plan->fill, args, ls) != 0) return -1;
-  }
   for (size_t u = 0; u < plan->units.size(); u++) {
-    std::vector<void *> &a = plan->kargs[u];
-    if (runner_launch(plan->units[u].runner, a.data(), (int)a.size()) != 0) {
+    if (launch_unit(plan, u) != 0) {
       log_err("plan_run", "kernel %d failed to launch", plan->units[u].item);
       return -1;
     }
@@ -280,10 +317,17 @@ PolyHipPlan *poly_hip_compile_schedule(PolyCtx *ctx, const PolySchedule *s) {
   }
   plan->slot_ptr.assign((size_t)ns, nullptr);
   plan->slot_needs_zero.assign((size_t)ns, 0);
+  plan->fills_before.assign((size_t)n_units, std::vector<int>());
   bool any_zero = false;
   for (int sl : order) {
     plan->slot_ptr[(size_t)sl] = (char *)plan->arena + plan->slot_off[(size_t)sl];
-    if (!slot_fully_written(s, sl, graphs)) { plan->slot_needs_zero[(size_t)sl] = 1; any_zero = true; }
+    if (first[(size_t)sl] < 0 || slot_fully_written(s, sl, graphs)) continue;
+    plan->slot_needs_zero[(size_t)sl] = 1;
+    plan->fills_before[(size_t)first[(size_t)sl]].push_back(sl);
+    any_zero = true;
+    if (getenv("POLY_HIP_DEBUG"))
+      fprintf(stderr, "polygrad: compile_schedule: slot %d (%lld bytes) is not fully written by its producers: cleared before launch %d\n",
+              sl, (long long)s->buf_slots[sl].nbytes, first[(size_t)sl]);
   }
   if (any_zero) {
     plan->fill = program_create(kFillSrc, "poly_fill0");
@@ -315,10 +359,22 @@ static int bind_args(PolyHipPlan *plan, void **slot_data, int n_slots, const Pol
                      uint64_t *key_out) {
   const PolySchedule *s = plan->sched;
   uint64_t key = 1469598103934665603ull;
+  if (plan->vetted_slot.size() != (size_t)s->n_buf_slots) plan->vetted_slot.assign((size_t)s->n_buf_slots, nullptr);
   for (int i = 0; i < s->n_buf_slots; i++) {
     if (s->buf_slots[i].is_intermediate) continue;
     plan->slot_ptr[(size_t)i] = (i < n_slots && slot_data) ? slot_data[i] : nullptr;
     key = fnv1a(&plan->slot_ptr[(size_t)i], sizeof(void *), key);
+    // A host address in a device plan (the frontend's constant registry, src/frontend.c:2231-2232,
+    // or a training step's loss slot, src/instance.c:1299-1311) would fault in the first kernel
+    // that touches it; looked up once per new pointer, outside any stream capture.
+    void *p = plan->slot_ptr[(size_t)i];
+    if (p && p != plan->vetted_slot[(size_t)i]) {
+      if (!runtime_device_can_read(p)) {
+        log_err("plan_run", "slot %d (%p) is not device memory; upload it with the allocator's copy_in first", i, p);
+        return -1;
+      }
+      plan->vetted_slot[(size_t)i] = p;
+    }
   }
   // default vars first, runtime overrides win (src/exec_plan.c:984-996)
   plan->merged.clear();
@@ -340,6 +396,7 @@ static int bind_args(PolyHipPlan *plan, void **slot_data, int n_slots, const Pol
         return -1;
       }
       a[i] = p;
+      if (i < un.runner->vetted.size()) un.runner->vetted[i] = p;     // vetted above, or the plan's own arena
     }
     (void)it;
     for (int v = 0; v < un.n_vars; v++) {
@@ -395,15 +452,12 @@ static int tuned_first_run(PolyHipPlan *plan) {
   plan->tuned = true;
   static std::map<uint64_t, std::string> decided;   // per process: identical kernels are timed once
   const std::string dir = runtime_cache_dir();
-  const PolySchedule *s = plan->sched;
-  for (int i = 0; i < s->n_buf_slots; i++) {
-    if (!plan->slot_needs_zero[(size_t)i]) continue;
-    if (runtime_memset(plan->slot_ptr[(size_t)i], 0, (size_t)std::max<int64_t>(s->buf_slots[i].nbytes, 4)) != 0) return -1;
-  }
   hipEvent_t e0 = nullptr, e1 = nullptr;
   int rc = 0;
   for (size_t ui = 0; ui < plan->units.size() && rc == 0; ui++) {
     Unit &u = plan->units[ui];
+    for (int slot : plan->fills_before[ui]) if (launch_fill(plan, slot) != 0) rc = -1;
+    if (rc != 0) break;
     HipRunner *r = u.runner;
     std::vector<void *> &args = plan->kargs[ui];
     const std::vector<RenderedKernel::Variant> &vs = r->rk.variants;
@@ -552,6 +606,24 @@ int poly_hip_fused_group_launch(const PolySchedule *s, int index, int *slots_out
   return (int)fg.arg_slots.size();
 }
 
+int poly_hip_unwritten_slots(const PolySchedule *s, int *slots_out, int cap) {
+  if (!s) return -1;
+  std::vector<KernelGraph> graphs((size_t)s->n_items);
+  for (int k = 0; k < s->n_items; k++)
+    if (s->items[k].kind != POLY_EXEC_COMPUTE || !graphs[(size_t)k].build(s->items[k].root)) return -1;
+  std::vector<FusedGroup> groups;
+  find_fused_groups(s, graphs, &groups);
+  std::vector<char> internal((size_t)s->n_buf_slots, 0);
+  for (const FusedGroup &fg : groups) for (int sl : fg.internal_slots) internal[(size_t)sl] = 1;
+  int n = 0;
+  for (int sl = 0; sl < s->n_buf_slots; sl++) {
+    if (!s->buf_slots[sl].is_intermediate || internal[(size_t)sl] || slot_fully_written(s, sl, graphs)) continue;
+    if (slots_out && n < cap) slots_out[n] = sl;
+    n++;
+  }
+  return n;
+}
+
 void poly_hip_plan_free(PolyHipPlan *plan) {
   if (!plan) return;
   runtime_sync();
@@ -589,8 +661,7 @@ int poly_hip_plan_profile(PolyHipPlan *plan, void **slot_data, int n_slots, floa
   int rc = 0;
   (void)hipEventRecord(ev[0], stream);
   for (int step = 0; step < n && rc == 0; step++) {
-    std::vector<void *> &a = plan->kargs[(size_t)step];
-    rc = runner_launch(plan->units[(size_t)step].runner, a.data(), (int)a.size());
+    rc = launch_unit(plan, (size_t)step);         // (a fill in front of the unit is timed with it)
     (void)hipEventRecord(ev[(size_t)step + 1], stream);
   }
   (void)hipStreamSynchronize(stream);
@@ -603,8 +674,7 @@ int poly_hip_plan_profile(PolyHipPlan *plan, void **slot_data, int n_slots, floa
 char *poly_hip_plan_kernel_desc(const PolyHipPlan *plan, int step) {
   if (!plan || step < 0 || step >= (int)plan->units.size()) return nullptr;
   const HipRunner *r = plan->units[(size_t)step].runner;
-  static const char *const kn[] = {"elementwise", "row-reduce", "thread-reduce", "matmul-mfma", "gather", "copy", "attention-mfma"};
-  std::string d = strf("%s %s: %s grid=%u,%u,%u bytes=%.0f flops=%.0f", r->name.c_str(), kn[(int)r->rk.klass],
+  std::string d = strf("%s %s: %s grid=%u,%u,%u bytes=%.0f flops=%.0f", r->name.c_str(), kernel_class_name(r->rk.klass),
                        r->rk.strategy.c_str(), r->rk.launch.grid[0], r->rk.launch.grid[1], r->rk.launch.grid[2],
                        r->rk.bytes, r->rk.flops);
   char *p = (char *)malloc(d.size() + 1);

@@ -24,6 +24,11 @@ struct LaunchSpec {
 };
 
 enum class KernelClass { ELEMENTWISE, ROW_REDUCE, THREAD_REDUCE, MATMUL_MFMA, GATHER, COPY, ATTENTION };
+inline const char *kernel_class_name(KernelClass k) {
+  static const char *const names[] = {"elementwise", "row-reduce", "thread-reduce", "matmul-mfma", "gather", "copy", "attention-mfma"};
+  const int i = (int)k;
+  return i >= 0 && i < (int)(sizeof(names) / sizeof(names[0])) ? names[i] : "unknown";
+}
 
 struct RenderedKernel {
   std::string source;      // complete HIP C translation unit

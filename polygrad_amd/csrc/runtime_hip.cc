@@ -78,6 +78,9 @@ bool compile_to_code_object(const std::string &source, std::vector<char> *code, 
   const int n_opts = (int)(sizeof(opts) / sizeof(opts[0]));
   uint64_t h = fnv1a(source.data(), source.size());
   for (int i = 0; i < n_opts; i++) h = h * 1099511628211ULL ^ fnv1a(opts[i], strlen(opts[i]));
+  // a code object on disk belongs to the compiler that made it
+  int rtc_major = 0, rtc_minor = 0;
+  if (hiprtcVersion(&rtc_major, &rtc_minor) == HIPRTC_SUCCESS) h = h * 1099511628211ULL ^ (uint64_t)(rtc_major * 100000 + rtc_minor);
   Runtime &r = rt();
   auto it = r.code_cache.find(h);
   if (it != r.code_cache.end()) { *code = it->second; return true; }
@@ -169,6 +172,19 @@ int runtime_memset(void *p, int value, size_t n) {
   if (runtime_init() != 0) return -1;
   if (n == 0) return 0;
   return check(hipMemsetAsync(p, value, n, rt().stream), "hipMemsetAsync") ? 0 : -1;
+}
+
+bool runtime_device_can_read(const void *p) {
+  if (!p || runtime_init() != 0) return false;
+  hipPointerAttribute_t a;
+  memset(&a, 0, sizeof(a));
+  if (hipPointerGetAttributes(&a, p) != hipSuccess) {
+    (void)hipGetLastError();      // an address HIP knows nothing about; the error must not stick
+    return false;
+  }
+  // device memory, managed memory, or host memory that HIP pinned (hipHostMalloc)
+  return a.type == hipMemoryTypeDevice || a.type == hipMemoryTypeManaged || a.type == hipMemoryTypeHost ||
+         a.type == hipMemoryTypeArray;
 }
 
 int runtime_sync() {

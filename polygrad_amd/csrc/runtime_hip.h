@@ -19,6 +19,9 @@ void runtime_free(void *p);
 int runtime_copy(void *dst, const void *src, size_t n, int kind);
 int runtime_memset(void *p, int value, size_t n);
 int runtime_sync();
+// Can a kernel dereference `p`?  False for pageable host memory (malloc, numpy arrays, the
+// host-side constant registry of the frontend) and for addresses HIP does not know.
+bool runtime_device_can_read(const void *p);
 // A device buffer of `bytes` bytes filled once by running kernel `entry(T* out)` of
 // `source` with the given launch; identical sources share one buffer.
 std::shared_ptr<void> runtime_table(const std::string &source, const std::string &entry, size_t bytes, const LaunchSpec &ls);
@@ -42,6 +45,7 @@ struct HipRunner {
   void *flag = nullptr;            // device int written by the guards
   std::vector<std::shared_ptr<void>> tables;   // filled lookup tables (shared between identical kernels)
   std::string name;
+  std::vector<void *> vetted;      // per buffer parameter: the last pointer found to be device-readable
   std::vector<void *> ptr_store;   // argument storage reused by every launch
   std::vector<int> var_store;
   std::vector<void *> arg_ptrs;

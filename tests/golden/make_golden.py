@@ -48,8 +48,82 @@ def emit(name, c, sink, arrays):
     print(f"{name}: {n} slots, {sum(v.nbytes for v in data.values())} bytes of vectors")
 
 
+def emit_assembled(name):
+    """A schedule put together by hand from kernels the reference scheduled, run through the
+    reference's own poly_compile_schedule / poly_compiled_plan_run: an intermediate twice
+    as large as what its producer writes.  The reference clears every intermediate at the
+    start of every run (src/exec_plan.c:946-963), so the half nobody writes reads as zero.
+    The reference frontend itself never builds such a schedule (poly_assign always targets
+    a whole buffer, src/frontend.c:98-120); the case pins the rule for callers that do.
+
+        J[0:2N]  = x2 * 3         (k0; J dies after k1, so I may take its bytes)
+        out2     = J + 1          (k1)
+        I[0:N]   = x * 2          (k2: writes the first half of I only)
+        out      = I + 1          (k3: reads all 2N elements of I)
+    """
+    if ONLY and name not in ONLY:
+        return
+    from polygrad_amd import _ffi
+    N = 1536
+    c = R.Ctx()
+    x, o1 = c.buffer((N,), name="x"), c.buffer((N,), name="o1")
+    x2, o2 = c.buffer((2 * N,), name="x2"), c.buffer((2 * N,), name="o2")
+    y, o3 = c.buffer((2 * N,), name="y"), c.buffer((2 * N,), name="o3")
+    scheds = [c.schedule(c.sink((o2, x2 * c.const(3.0)))), c.schedule(c.sink((o3, y + c.const(1.0)))),
+              c.schedule(c.sink((o1, x * c.const(2.0))))]
+    parts = [C.cast(p, C.POINTER(_ffi.PolySchedule)).contents for p in scheds]
+    for p, sp, out_t in zip(parts, scheds, (o2, o3, o1)):
+        assert p.n_items == 1 and p.items[0].n_buf_slots == 2 and p.n_buf_slots == 2
+        by_slot, _ = schedule_slots(c, sp)
+        assert by_slot[p.items[0].buf_slot_indices[0]][0] == out_t, "PARAM 0 is expected to be the output"
+    mul3, add1, mul2 = (p.items[0] for p in parts)
+    f32_2n = parts[0].buf_slots[0]          # a float32 slot of 2N elements to copy dtype and sizes from
+    # slots: 0 x2 (ext), 1 x (ext), 2 out2 (ext), 3 out (ext), 4 J (tmp), 5 I (tmp)
+    slots = (_ffi.PolyScheduleBufSlot * 6)()
+    for i, (numel, tmp) in enumerate(((2 * N, False), (N, False), (2 * N, False), (2 * N, False), (2 * N, True), (2 * N, True))):
+        slots[i].dtype = f32_2n.dtype
+        slots[i].numel, slots[i].nbytes = numel, 4 * numel
+        slots[i].buf_uop = None
+        slots[i].is_intermediate = tmp
+        slots[i].external_buf_idx = -1
+    items = (_ffi.PolyExecItem * 4)()
+    keep = []
+    for i, (src, (dst_slot, src_slot)) in enumerate(((mul3, (4, 0)), (add1, (2, 4)), (mul2, (5, 1)), (add1, (3, 5)))):
+        idx = (C.c_int * 2)(dst_slot, src_slot)       # PARAM 0 is the output (checked above)
+        keep.append(idx)
+        items[i].kind = src.kind
+        items[i].root = src.root
+        items[i].buf_slot_indices = idx
+        items[i].n_buf_slots = 2
+    order = (C.c_int * 4)(0, 1, 2, 3)
+    sched = _ffi.PolySchedule()
+    sched.entrypoint_name = b"assembled"
+    sched.buf_slots, sched.n_buf_slots = slots, 6
+    sched.items, sched.n_items = items, 4
+    sched.exec_order = order
+    sched.loss_buf_slot = -1
+    names = ["x2", "x", "out2", "out", None, None]
+    g = np.random.default_rng(77)
+    ins = [g.uniform(-1, 1, 2 * N).astype(np.float32), g.uniform(-1, 1, N).astype(np.float32),
+           np.zeros(2 * N, np.float32), np.zeros(2 * N, np.float32)]
+    outs = [a.copy() for a in ins]
+    for _ in range(2):       # twice: the second run must find the holes cleared again
+        c.run_schedule_ref(C.addressof(sched), outs + [None, None])
+    assert np.array_equal(outs[3][:N], ins[1] * np.float32(2) + np.float32(1)) and np.all(outs[3][N:] == 1.0)
+    data = {}
+    for i in range(4):
+        data[f"in{i}"], data[f"out{i}"] = ins[i], outs[i]
+    save_schedule(C.addressof(sched), names, os.path.join(HERE, name + ".polyplan"))
+    np.savez_compressed(os.path.join(HERE, name + ".npz"), **data)
+    for p in scheds:
+        c.L.poly_schedule_free(p)
+    c.close()
+    print(f"{name}: hand-assembled, 6 slots")
+
+
 def main():
     g = np.random.default_rng(1234)
+    emit_assembled("assembled_partial_store")
 
     # reference KAT: (2,3)@(3,4) = [[38,44,50,56],[83,98,113,128]]  (test/test_nn.c:417-439)
     c = R.Ctx()
@@ -74,6 +148,14 @@ def main():
     onehot[np.arange(4), [0, 1, 2, 1]] = 1
     emit("kat_xent_uniform", c, c.sink((o, lg.cross_entropy(tg))),
          {lg: np.full((4, 3), 0.7, np.float32), tg: onehot, o: np.zeros(1, np.float32)})
+    c.close()
+
+    # reductions over an axis of extent 1 (a batch of one): no loop, the value itself passes
+    # through -- -0.0 stays -0.0, NaN stays NaN (src/codegen.c:1444-1450)
+    c = R.Ctx()
+    x, o1, o2 = c.buffer((8, 1), name="x"), c.buffer((8,), name="sum"), c.buffer((8,), name="max")
+    xs = np.array([0.0, -0.0, 1.5, -2.25, np.nan, np.inf, -np.inf, 1e-40], np.float32)
+    emit("reduce_singleton_axis", c, c.sink((o1, x.sum(1)), (o2, x.max(1))), {x: xs, o1: np.ones(8, np.float32), o2: np.ones(8, np.float32)})
     c.close()
 
     # fused chain + row ops (config 2 at a reduced shape)

@@ -11,7 +11,8 @@ from polygrad_amd import HipPlan
 pytestmark = pytest.mark.gpu
 
 # bit-exact: integer, index and movement work
-BIT_EXACT = {"kat_threefry_u32", "kat_threefry_u64", "movement_i32", "int_alu"}
+BIT_EXACT = {"kat_threefry_u32", "kat_threefry_u64", "movement_i32", "int_alu", "assembled_partial_store",
+             "reduce_singleton_axis"}
 # tolerance per case: (rtol, atol)
 TOL = {
     "kat_matmul_2x3x4": (1e-4, 0), "kat_xent_uniform": (1e-4, 1e-6),
