@@ -3,7 +3,7 @@ reference CPU backend (oracle/_ref/libpolygrad.so, built from /root/reference). 
 10-20 minutes on one core, so it is separate from make_golden.py.
 
 Run from the repository root in the build container:
-    python tests/golden/make_golden_fullsize.py [attention] [block0] [logits]
+    python tests/golden/make_golden_fullsize.py [attention] [block0] [logits] [truth]
 
 Writes
   tests/golden/attention_bf16_t1024.{polyplan,npz}
@@ -18,6 +18,9 @@ Writes
       `logits_rows` = their full logit rows [len(rows), 50257], `cols` = sampled vocabulary
       columns, `logits_cols` = those columns at every position [1024, len(cols)]; bf16 bit
       patterns.  The plan is polygrad_amd/plans/gpt2_small_bf16_b1_t1024.polyplan.
+  tests/golden/fullsize/gpt2_small_f32_b1_t1024_logits.npz
+      the same network and sequence evaluated in fp32 by the reference (fp32 graph, the
+      same bf16-valued weights), same rows and columns, float32.
 Inputs are not stored: tests/gpt2_data.py regenerates them from seed 3.
 """
 import os
@@ -87,6 +90,28 @@ def block0():
     c.close()
 
 
+def block0_truth():
+    """Block 0 evaluated in fp32 by the reference (fp32 graph, same bf16-valued weights).
+    Stored as float16: an 11-bit mantissa, eight times finer than the bf16 values that are
+    compared against it, on values below 2."""
+    cfg = graphs.GPT2Config(n_layer=1, batch=1)
+    named = gpt2_data.gpt2_named_arrays(12, cfg.d_model, cfg.vocab, cfg.ctx, 1, seed=3)
+    named = {k: (gpt2_data.bf16_bits_to_f32(a) if a.dtype == np.uint16 else a) for k, a in named.items()}
+    c = R.Ctx()
+    sink, bufs = graphs.gpt2_forward(c, cfg, R.F32, hidden_only=True)
+    hidden = np.zeros(cfg.ctx * cfg.d_model, np.float32)
+    arrays = bind(bufs, named, {"hidden": hidden})
+    sched = c.schedule(sink)
+    slots, _ = schedule_slots(c, sched)
+    c.L.poly_schedule_free(sched)
+    used = {tn[0] for tn in slots.values() if tn is not None}
+    t0 = time.time()
+    c.realize_cpu(sink, {t: a for t, a in arrays.items() if t in used})
+    print(f"block0_truth: reference ran in {time.time() - t0:.0f} s")
+    np.savez_compressed(os.path.join(FULL, "gpt2_small_f32_b1_t1024_block0.npz"), hidden=hidden.astype(np.float16))
+    c.close()
+
+
 def logits():
     cfg = graphs.GPT2Config(batch=1)
     named = gpt2_data.gpt2_named_arrays(12, cfg.d_model, cfg.vocab, cfg.ctx, 1, seed=3)
@@ -103,8 +128,27 @@ def logits():
     c.close()
 
 
+def truth():
+    """The same network evaluated in fp32 by the reference (same bf16-valued weights): what
+    both bf16 evaluations approximate.  Stored at the same rows and columns."""
+    cfg = graphs.GPT2Config(batch=1)
+    named = gpt2_data.gpt2_named_arrays(12, cfg.d_model, cfg.vocab, cfg.ctx, 1, seed=3)
+    named = {k: (gpt2_data.bf16_bits_to_f32(a) if a.dtype == np.uint16 else a) for k, a in named.items()}
+    c = R.Ctx()
+    sink, bufs = graphs.gpt2_forward(c, cfg, R.F32)
+    out = np.zeros(cfg.ctx * cfg.vocab, np.float32)
+    arrays = bind(bufs, named, {"output": out})
+    t0 = time.time()
+    c.realize_cpu(sink, arrays)
+    print(f"truth: reference ran in {time.time() - t0:.0f} s")
+    lg = out.reshape(cfg.ctx, cfg.vocab)
+    np.savez_compressed(os.path.join(FULL, "gpt2_small_f32_b1_t1024_logits.npz"), rows=ROWS, logits_rows=lg[ROWS],
+                        cols=COLS, logits_cols=np.ascontiguousarray(lg[:, COLS]))
+    c.close()
+
+
 if __name__ == "__main__":
     os.makedirs(FULL, exist_ok=True)
-    which = sys.argv[1:] or ["attention", "block0", "logits"]
+    which = sys.argv[1:] or ["attention", "block0", "block0_truth", "logits", "truth"]
     for w in which:
-        {"attention": attention, "block0": block0, "logits": logits}[w]()
+        {"attention": attention, "block0": block0, "block0_truth": block0_truth, "logits": logits, "truth": truth}[w]()

@@ -16,6 +16,9 @@ import numpy as np
 
 _HERE = os.path.dirname(os.path.abspath(__file__))
 REF_LIB = os.path.join(_HERE, "..", "oracle", "_ref", "libpolygrad.so")
+# The same sources with the HIP backend wired in (oracle/hip_integration.py,
+# `make -C oracle ref_hip`): the reference's own callers driving libpolygrad_hip.so.
+HIP_REF_LIB = os.path.join(_HERE, "..", "oracle", "_ref", "libpolygrad_hip_ref.so")
 
 # dtype ids of the reference's FFI table (src/frontend.c:124-129)
 VOID, BOOL, I8, U8, I16, U16, I32, U32, I64, U64, F16, BF16, F32, F64 = range(14)
@@ -31,7 +34,7 @@ OPS = ("DEFINE_VAR BIND SPECIAL DEFINE_LOCAL DEFINE_REG NOOP REWRITE_ERROR PARAM
        "BARRIER RANGE IF END ENDIF VCONST CONST").split()
 OP = {name: i + 1 for i, name in enumerate(OPS)}
 
-DEVICE_CPU, DEVICE_INTERP = 1, 2
+DEVICE_CPU, DEVICE_INTERP, DEVICE_HIP = 1, 2, 7
 
 
 class PolyDType(C.Structure):
@@ -48,18 +51,26 @@ class PolyBufferBinding(C.Structure):
     _fields_ = [("buffer", C.c_void_p), ("handle", PolyBufferHandle)]
 
 
-_lib = None
+class PolyIOBinding(C.Structure):
+    _fields_ = [("name", C.c_char_p), ("data", C.c_void_p)]
+
+
+_libs = {}
 
 
 def available():
     return os.path.exists(REF_LIB)
 
 
-def lib():
-    global _lib
-    if _lib is not None:
-        return _lib
-    L = C.CDLL(os.path.abspath(REF_LIB))
+def hip_ref_available():
+    return os.path.exists(HIP_REF_LIB)
+
+
+def lib(path=None):
+    path = os.path.abspath(path or REF_LIB)
+    if path in _libs:
+        return _libs[path]
+    L = C.CDLL(path)
     P = C.c_void_p
     I64P = C.POINTER(C.c_int64)
     sig = {
@@ -99,20 +110,32 @@ def lib():
         "poly_define_var": (P, [P, C.c_char_p, C.c_int64, C.c_int64]), "poly_bind_var": (P, [P, P, C.c_int64]),
         "poly_buffer_var": (P, [P, PolyDType, P, I64P, C.c_int]),
         "poly_op_name": (C.c_char_p, [C.c_int]),
+        # PolyInstance (src/instance.h) and the MLP builder (src/model_mlp.h:31)
+        "poly_mlp_instance": (P, [C.c_char_p, C.c_int]), "poly_instance_free": (None, [P]),
+        "poly_instance_set_device": (C.c_int, [P, C.c_int]),
+        "poly_instance_param_count": (C.c_int, [P]), "poly_instance_buf_count": (C.c_int, [P]),
+        "poly_instance_param_data": (P, [P, C.c_int, I64P]), "poly_instance_buf_data": (P, [P, C.c_int, I64P]),
+        "poly_instance_buf_role": (C.c_int, [P, C.c_int]), "poly_instance_buf_name": (C.c_char_p, [P, C.c_int]),
+        "poly_instance_readback_buf": (C.c_int, [P, C.c_int, P, C.c_size_t]),
+        "poly_instance_readback_param": (C.c_int, [P, C.c_int, P, C.c_size_t]),
+        "poly_instance_forward": (C.c_int, [P, C.POINTER(PolyIOBinding), C.c_int]),
+        "poly_instance_value_and_grad": (C.c_int, [P, C.c_char_p, C.POINTER(PolyIOBinding), C.c_int, C.POINTER(C.c_float)]),
+        "poly_instance_train_step": (C.c_int, [P, C.POINTER(PolyIOBinding), C.c_int, C.POINTER(C.c_float)]),
+        "poly_instance_set_optimizer": (C.c_int, [P, C.c_int] + [C.c_float] * 5),
     }
     for name, (res, args) in sig.items():
         fn = getattr(L, name)
         fn.restype = res
         fn.argtypes = args
-    _lib = L
+    _libs[path] = L
     return L
 
 
-def dtype_struct(dt):
+def dtype_struct(dt, L=None):
     names = ["POLY_VOID", "POLY_BOOL", "POLY_INT8", "POLY_UINT8", "POLY_INT16", "POLY_UINT16", "POLY_INT32",
              "POLY_UINT32", "POLY_INT64", "POLY_UINT64", "POLY_FLOAT16", "POLY_BFLOAT16", "POLY_FLOAT32",
              "POLY_FLOAT64"]
-    return PolyDType.in_dll(lib(), names[dt])
+    return PolyDType.in_dll(L or lib(), names[dt])
 
 
 def _i64(vals):
@@ -123,8 +146,9 @@ def _i64(vals):
 class Ctx:
     """A reference PolyCtx plus the list of buffers created in it."""
 
-    def __init__(self):
-        self.L = lib()
+    def __init__(self, hip_ref=False):
+        """hip_ref: use the build of the reference that has the HIP backend in its table."""
+        self.L = lib(HIP_REF_LIB if hip_ref else None)
         self.ctx = self.L.poly_ctx_new()
         self.buffers = []   # (T, name)
 
@@ -152,7 +176,7 @@ class Ctx:
     def buffer_var(self, var, max_val, inner=(), dt=F32, name=None):
         """A buffer whose leading dimension is the variable `var` (allocated for max_val),
         as poly_buffer_var builds it (src/frontend.c:163-179)."""
-        u = self.L.poly_buffer_var(self.ctx, dtype_struct(dt), var, _i64(inner) if inner else None, len(inner))
+        u = self.L.poly_buffer_var(self.ctx, dtype_struct(dt, self.L), var, _i64(inner) if inner else None, len(inner))
         t = T(self, u, (max_val,) + tuple(inner), dt, buf=u)
         self.buffers.append((t, name or f"buf{len(self.buffers)}"))
         return t
@@ -160,7 +184,7 @@ class Ctx:
     def const(self, v, dt=F32):
         if dt in (F32,):
             return T(self, self.L.poly_const_float(self.ctx, float(v)), (), dt)
-        return T(self, self.L.poly_const_typed(self.ctx, dtype_struct(dt), float(v)), (), dt)
+        return T(self, self.L.poly_const_typed(self.ctx, dtype_struct(dt, self.L), float(v)), (), dt)
 
     def sink(self, *pairs):
         """pairs: (out_buffer T, value T) -> tensor-level SINK."""
@@ -208,6 +232,16 @@ class Ctx:
         rc = self.L.poly_realize(self.ctx, sink, b, n)
         if rc != 0:
             raise RuntimeError("reference poly_realize failed")
+
+    def realize_bound(self, sink, handles):
+        """poly_realize with explicit handles: {buffer T: (pointer, nbytes, device domain)}
+        -- the form the reference's own device tests use (test/test_cuda.c:438-516)."""
+        n = len(handles)
+        b = (PolyBufferBinding * n)()
+        for i, (t, (ptr, nbytes, domain)) in enumerate(handles.items()):
+            b[i].buffer = t.buf
+            b[i].handle = PolyBufferHandle(ptr, nbytes, domain, False)
+        return self.L.poly_realize(self.ctx, sink, b, n)
 
     def schedule(self, sink):
         s = self.L.poly_schedule_for(self.ctx, sink, 0)

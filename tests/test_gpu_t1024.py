@@ -1,0 +1,198 @@
+"""The benchmark's kernels at the benchmark's sequence length against the REAL reference:
+GPT-2 small (12 layers, d_model 768, 12 heads, vocab 50257), one sequence of 1024 tokens,
+computed once by the reference CPU backend in the build container
+(tests/golden/make_golden_fullsize.py) and stored as sampled logits and as the residual
+stream after block 0.  The GPU runs the same sequence through the one-sequence plan and
+through the B=8 plan the benchmark times (the sequence as batch element 5), in both
+attention forms, and the stand-alone B=8 x 12-head attention plan on the heads of the
+T=1024 attention fixture.
+
+Tolerances.  bf16 values: rtol 2e-2.  The attention kernel alone: plus an absolute term of
+2.5e-3 of the output's largest magnitude (what the T=256 attention fixture is held to:
+8e-3 on outputs up to 3.2).  Whole blocks: a bf16 rounding that falls differently (another
+summation order in a matmul) is one unit in the last place of a LayerNorm output, i.e.
+1/128 of the row's standard deviation, and the matmuls behind the LayerNorm spread it over
+the row; block 0's residual stream has entries around 0.03 with a few up to 2, so such a
+flip moves entries by several of their own bf16 steps.  The residual stream after one
+block is therefore held element-wise to 2e-2 of the tensor's scale (99.9 % of the entries
+to 2.5e-3 of it), the logits after twelve blocks to 2e-2 of theirs, and -- the sharper
+statement, position by position -- the GPU's result must be as close to the fp32
+evaluation of the same network (reference CPU backend, fp32 graph) as the reference's own
+bf16 result is."""
+import os
+
+import numpy as np
+import pytest
+
+import fixtures as F
+import gpt2_data
+from hipharness import assert_close, from_device, to_device
+from polygrad_amd import HipPlan
+
+pytestmark = pytest.mark.gpu
+
+HERE = os.path.dirname(os.path.abspath(__file__))
+FULL = os.path.join(HERE, "golden", "fullsize")
+PLANS = os.path.join(HERE, "..", "polygrad_amd", "plans")
+T, D, V, H = 1024, 768, 50257, 12
+
+
+@pytest.fixture(scope="module")
+def named():
+    return gpt2_data.gpt2_named_arrays(12, D, V, T, 1, seed=3)
+
+
+@pytest.fixture(scope="module")
+def weights_on_device(named):
+    return {k: to_device(a) for k, a in named.items() if k != "x"}
+
+
+def bind_by_name(plan, weights, extra):
+    data = [None] * len(plan.slots)
+    for s in plan.external_slots():
+        t = extra.get(s.name, weights.get(s.name))
+        assert t is not None, f"no data for slot {s.name}"
+        assert t.numel() * t.element_size() == s.nbytes, f"{s.name}: {t.numel() * t.element_size()} bytes bound, {s.nbytes} expected"
+        data[s.index] = t
+    return data
+
+
+def set_form(monkeypatch, form):
+    if form == "exact":
+        monkeypatch.setenv("POLY_HIP_EXACT_ATTENTION", "1")
+    else:
+        monkeypatch.delenv("POLY_HIP_EXACT_ATTENTION", raising=False)
+    return "two passes" if form == "exact" else "one pass"
+
+
+@pytest.mark.parametrize("form", ["online", "exact"])
+def test_block0_residual_stream_t1024_matches_reference(monkeypatch, named, weights_on_device, form):
+    import torch
+    marker = set_form(monkeypatch, form)
+    want = gpt2_data.bf16_bits_to_f32(np.load(os.path.join(FULL, "gpt2_small_bf16_b1_t1024_block0.npz"))["hidden"]).reshape(T, D)
+    plan = HipPlan.from_file(os.path.join(FULL, "gpt2_small_bf16_b1_t1024_block0.polyplan"))
+    hidden = torch.zeros(T * D, dtype=torch.int16, device="cuda")
+    data = bind_by_name(plan, weights_on_device, {"x": to_device(named["x"]), "hidden": hidden})
+    plan.run(data)
+    plan.run(data)
+    info = plan.kernel_info()
+    plan.close()
+    attn = [k["desc"] for k in info if k["klass"] == "attention-mfma"]
+    assert len(attn) == 1 and marker in attn[0], attn
+    got = gpt2_data.bf16_bits_to_f32(from_device(hidden, np.uint16)).reshape(T, D).astype(np.float64)
+    want = want.astype(np.float64)
+    scale = float(np.abs(want).max())
+    what = f"residual stream after block 0, T=1024, {form} attention"
+    assert np.isfinite(got).all()
+    assert_close(got, want, rtol=2e-2, atol=2e-2 * scale, what=what)
+    tight = np.abs(got - want) <= 2e-2 * np.abs(want) + 2.5e-3 * scale
+    assert tight.mean() >= 0.999, f"{what}: only {tight.mean():.5f} of the entries within 2.5e-3 of the scale"
+    truth_path = os.path.join(FULL, "gpt2_small_f32_b1_t1024_block0.npz")
+    if os.path.exists(truth_path):
+        truth = np.load(truth_path)["hidden"].astype(np.float64).reshape(T, D)
+        e_gpu = np.sqrt(((got - truth) ** 2).mean(axis=1))        # per position
+        e_ref = np.sqrt(((want - truth) ** 2).mean(axis=1))
+        worst = int(np.argmax(e_gpu / e_ref))
+        assert (e_gpu <= 1.5 * e_ref).all(), f"{what}: position {worst}: rms error {e_gpu[worst]:.3e} against the fp32 network, the reference's own is {e_ref[worst]:.3e}"
+        assert e_gpu.mean() <= 1.1 * e_ref.mean(), f"{what}: mean rms error {e_gpu.mean():.3e} vs the reference's {e_ref.mean():.3e}"
+
+
+def _check_logits(got_rows, got_cols, what):
+    ref = np.load(os.path.join(FULL, "gpt2_small_bf16_b1_t1024_logits.npz"))
+    w_rows = gpt2_data.bf16_bits_to_f32(ref["logits_rows"]).astype(np.float64)
+    w_cols = gpt2_data.bf16_bits_to_f32(ref["logits_cols"]).astype(np.float64)
+    scale = max(float(np.abs(w_rows).max()), float(np.abs(w_cols).max()))
+    assert np.isfinite(got_rows).all() and np.isfinite(got_cols).all()
+    assert_close(got_rows, w_rows, rtol=2e-2, atol=2e-2 * scale, what=f"{what}: logits of the sampled positions")
+    assert_close(got_cols, w_cols, rtol=2e-2, atol=2e-2 * scale, what=f"{what}: sampled vocabulary columns at every position")
+    truth_path = os.path.join(FULL, "gpt2_small_f32_b1_t1024_logits.npz")
+    if os.path.exists(truth_path):
+        tr = np.load(truth_path)
+        rms = lambda d: float(np.sqrt((d ** 2).mean()))
+        for g_, w_, t_, part in ((got_rows, w_rows, tr["logits_rows"].astype(np.float64), "rows"),
+                                 (got_cols, w_cols, tr["logits_cols"].astype(np.float64), "columns")):
+            e_gpu, e_ref = rms(g_ - t_), rms(w_ - t_)
+            assert e_gpu <= 1.25 * e_ref, f"{what} ({part}): GPU rms error {e_gpu:.3e} vs reference rms error {e_ref:.3e} against the fp32 network"
+    return ref
+
+
+@pytest.mark.parametrize("form", ["online", "exact"])
+def test_logits_t1024_one_sequence_plan_matches_reference(monkeypatch, named, weights_on_device, form):
+    import torch
+    marker = set_form(monkeypatch, form)
+    ref = np.load(os.path.join(FULL, "gpt2_small_bf16_b1_t1024_logits.npz"))
+    plan = HipPlan.from_file(os.path.join(PLANS, "gpt2_small_bf16_b1_t1024.polyplan"))
+    out = torch.zeros(T * V, dtype=torch.int16, device="cuda")
+    data = bind_by_name(plan, weights_on_device, {"x": to_device(named["x"]), "output": out})
+    plan.run(data)
+    info = plan.kernel_info()
+    plan.close()
+    attn = [k["desc"] for k in info if k["klass"] == "attention-mfma"]
+    assert len(attn) == 12 and all(marker in d for d in attn), attn
+    lg = out.view(T, V)
+    rows = gpt2_data.bf16_bits_to_f32(from_device(lg[torch.as_tensor(ref["rows"], device="cuda")].contiguous(), np.uint16)).astype(np.float64)
+    cols = gpt2_data.bf16_bits_to_f32(from_device(lg[:, torch.as_tensor(ref["cols"], device="cuda")].contiguous(), np.uint16)).astype(np.float64)
+    _check_logits(rows, cols, f"B=1 plan, {form} attention")
+
+
+@pytest.mark.parametrize("form", ["online", "exact"])
+def test_logits_t1024_benchmark_plan_matches_reference(monkeypatch, named, weights_on_device, form):
+    """The plan bench.py times (B=8): the reference's sequence is batch element 5, the
+    other seven are random tokens."""
+    import torch
+    marker = set_form(monkeypatch, form)
+    ref = np.load(os.path.join(FULL, "gpt2_small_bf16_b1_t1024_logits.npz"))
+    plan = HipPlan.from_file(os.path.join(PLANS, "gpt2_small_bf16_b8_t1024.polyplan"))
+    g = np.random.default_rng(8)
+    tokens = g.integers(0, V, 8 * T).astype(np.float32).reshape(8, T)
+    tokens[5] = named["x"]
+    out = torch.zeros(8 * T * V, dtype=torch.int16, device="cuda")
+    data = bind_by_name(plan, weights_on_device, {"x": to_device(tokens.reshape(-1)), "output": out})
+    plan.run(data)
+    plan.run(data)      # the replayed hipGraph is what the benchmark times
+    info = plan.kernel_info()
+    plan.close()
+    attn = [k["desc"] for k in info if k["klass"] == "attention-mfma"]
+    assert len(attn) == 12 and all(marker in d for d in attn), attn
+    lg = out.view(8, T, V)[5]
+    rows = gpt2_data.bf16_bits_to_f32(from_device(lg[torch.as_tensor(ref["rows"], device="cuda")].contiguous(), np.uint16)).astype(np.float64)
+    cols = gpt2_data.bf16_bits_to_f32(from_device(lg[:, torch.as_tensor(ref["cols"], device="cuda")].contiguous(), np.uint16)).astype(np.float64)
+    _check_logits(rows, cols, f"B=8 plan, {form} attention")
+
+
+@pytest.mark.parametrize("form", ["online", "exact"])
+def test_attention_b8_h12_t1024_plan_on_the_fixture_heads(monkeypatch, form):
+    """The stand-alone attention plan at the benchmark's shape (8 sequences, 12 heads): the
+    two heads of the T=1024 fixture sit at (sequence 3, heads 4 and 5) and (sequence 7,
+    heads 10 and 11), everything around them is random."""
+    import torch
+    marker = set_form(monkeypatch, form)
+    fx = F.Fixture("attention_bf16_t1024")
+    by = {fx.plan.names[i]: i for i in fx.external}
+    plan = HipPlan.from_file(os.path.join(PLANS, "attention_bf16_b8_h12_t1024_d64.polyplan"))
+    g = np.random.default_rng(12)
+    host = {}
+    spots = ((3, 4), (7, 10))
+    for nm in ("q", "k", "v"):
+        a = gpt2_data.f32_to_bf16_bits(g.normal(0, 1.0, 8 * T * H * 64).astype(np.float32)).reshape(8, T, H, 64)
+        two = fx.inputs[by[nm]].reshape(T, 2, 64)
+        for b, h in spots:
+            a[b, :, h:h + 2, :] = two
+        host[nm] = a
+    out = torch.zeros(8 * T * H * 64, dtype=torch.int16, device="cuda")
+    extra = {nm: to_device(host[nm].reshape(-1)) for nm in host}
+    extra["out"] = out
+    extra["arange"] = to_device(np.arange(T, dtype=np.float32))
+    data = bind_by_name(plan, {}, extra)
+    plan.run(data)
+    plan.run(data)
+    info = plan.kernel_info()
+    plan.close()
+    attn = [k["desc"] for k in info if k["klass"] == "attention-mfma"]
+    assert len(attn) == 1 and marker in attn[0], attn
+    got = gpt2_data.bf16_bits_to_f32(from_device(out, np.uint16)).reshape(8, T, H, 64)
+    want = gpt2_data.bf16_bits_to_f32(fx.expected[by["out"]]).reshape(T, 2, 64)
+    scale = float(np.abs(want).max())
+    for b, h in spots:
+        assert_close(got[b, :, h:h + 2, :], want, rtol=2e-2, atol=(2.5e-3 if form == "online" else 6.5e-4) * scale,
+                     what=f"attention B=8 H=12 T=1024, sequence {b} heads {h},{h + 1}, {form}")

@@ -7,6 +7,7 @@
 3. Where the reference library is built, random graphs against it, bit for bit.
 """
 import math
+import os
 
 import numpy as np
 import pytest
@@ -84,8 +85,15 @@ def test_threefry_known_answers():
         assert v & 0xFFFFFFFF == ref32[i]
 
 
+# Minutes of interpreted evaluation (2 x 1024 x 1024 scores, each through the whole softmax
+# chain); the same kernels are pinned bit for bit at 256 positions (attention_bf16_t256).
+SLOW_ON_THE_ORACLE = {"attention_bf16_t1024"}
+
+
 @pytest.mark.parametrize("name", F.case_names())
 def test_oracle_reproduces_reference_fixture(name):
+    if name in SLOW_ON_THE_ORACLE and not os.environ.get("POLY_SLOW_TESTS"):
+        pytest.skip("set POLY_SLOW_TESTS=1 to run the T=1024 attention fixture through the oracle (about 2 minutes)")
     fx = F.Fixture(name)
     got = F.run_oracle_schedule(fx.plan.schedule, fx.n_slots, fx.inputs)
     for slot in fx.external:
