@@ -86,7 +86,9 @@ __device__ __forceinline__ int poly_swz(int row) { return (row ^ (row >> 3)) & (
 // K tiles one workgroup walks: with POLY_KSPLIT > 1 the K tiles of an output tile are dealt
 // to that many workgroups (blockIdx.y = z * POLY_KSPLIT + part), each leaving its fp32
 // accumulators where the epilogue macros put them (they may use `poly_ks`, the part).
+#ifndef POLY_KT
 #define POLY_KT (POLY_K / POLY_BK / POLY_KSPLIT)
+#endif
 // row pitch (floats) of the 32x32 output staging tile: 16-byte aligned rows, and rows 4
 // apart (the two halves of a wave) land on different banks
 #define POLY_STAGE_LD 36

@@ -571,6 +571,8 @@ bool render_matmul(const MatmulMatch &mm, const MatmulEpilogue &ep, RenderedKern
     // each XCD (own L2) works on a contiguous run of tiles: let it re-read the smaller operand
     cfg += strf("#define POLY_GROUP_ALONG_N %d\n", (N > 2 * M && !getenv("POLY_HIP_MM_GROUP_M")) ? 1 : 0);
     cfg += strf("#define POLY_PIPE %d\n", pp);
+    // timing experiments only (wrong results): walk just the first n K tiles
+    if (const char *e = getenv("POLY_HIP_MM_KT")) if (atoi(e) > 0 && atoi(e) <= K / BK) cfg += strf("#define POLY_KT %d\n", atoi(e));
     cfg += strf("#define POLY_A_KC %d\n#define POLY_B_KC %d\n", a_kc ? 1 : 0, b_kc ? 1 : 0);
     cfg += strf("#define POLY_A_PTR %s\n#define POLY_B_PTR %s\n", ep.a_ptr.c_str(), ep.b_ptr.c_str());
     cfg += offset_fn("poly_a_row", md, true, 0);

@@ -9,6 +9,7 @@ the GPU box, where the reference frontend is not part of the product path:
     polygrad_amd/plans/mlp_train_f32_b4096.polyplan        config 1: MLP forward + backward + SGD step
     polygrad_amd/plans/adamw_f32_355m.polyplan             config 5: AdamW update of 355 M fp32 parameters
     polygrad_amd/plans/gpt2_medium_block_train_b4_t1024.polyplan   config 5: one block + head, backward, AdamW
+    polygrad_amd/plans/gpt2_small_layer_matmuls_b8_t1024.polyplan  the four weight matmuls of a GPT-2 small layer with their tails
 
 The graphs are built with the REAL reference frontend and scheduler
 (oracle/_ref/libpolygrad.so through tests/refpoly.py); only the scheduled kernel
@@ -80,6 +81,20 @@ def main():
     c = R.Ctx()
     _, _, _, sink = graphs.matmul_bf16(c, 1024, 1024, 1024, batch=16)
     save(c, sink, "matmul_bf16_b16_1024x1024x1024")
+    c.close()
+    # the four weight matmuls of one GPT-2 small layer with their pointwise tails (bias, residual,
+    # GELU), as gpt2_forward schedules them, without LayerNorm and attention: for timing them alone
+    c = R.Ctx()
+    BT, D = 8192, 768
+    P = lambda name, shape: c.buffer(shape, R.BF16, name=name)
+    x, o_qkv, o_h = P("x", (BT, D)), P("qkv", (BT, 3 * D)), P("h", (BT, D))
+    qkv = graphs._linear(x, P("attn_w", (D, 3 * D)), P("attn_b", (3 * D,)), R.BF16).contiguous()
+    a = graphs._linear(x, P("proj_w", (D, D)), P("proj_b", (D,)), R.BF16).contiguous()
+    h = (x + a).contiguous()
+    ff = graphs._linear(h, P("fc_w", (D, 4 * D)), P("fc_b", (4 * D,)), R.BF16).contiguous()
+    ff = ff.gelu().contiguous()
+    ff = graphs._linear(ff, P("fc2_w", (4 * D, D)), P("fc2_b", (D,)), R.BF16).contiguous()
+    save(c, c.sink((o_qkv, qkv), (o_h, (h + ff).contiguous())), "gpt2_small_layer_matmuls_b8_t1024")
     c.close()
     c = R.Ctx()
     _, sink = graphs.gpt2_block_train_step(c, batch=4, ctx=1024, d_model=1024, heads=16, vocab=50257)
