@@ -2,6 +2,7 @@
 
 #include <algorithm>
 #include <climits>
+#include <cstdint>
 #include <cstdlib>
 #include <cstring>
 
@@ -39,18 +40,31 @@ static std::string lin_key(const Lin &l) {
   return k;
 }
 
+// a * b and a + b in 64 bits; on overflow *flag is set and the result is harmless
+static int64_t ck_mul(int64_t a, int64_t b, bool *flag) {
+  int64_t r;
+  if (__builtin_mul_overflow(a, b, &r)) { *flag = true; return 0; }
+  return r;
+}
+static int64_t ck_add(int64_t a, int64_t b, bool *flag) {
+  int64_t r;
+  if (__builtin_add_overflow(a, b, &r)) { *flag = true; return 0; }
+  return r;
+}
+
 Lin KernelGraph::lin_add(const Lin &a, const Lin &b, int64_t sb) const {
   Lin r;
-  r.c0 = a.c0 + sb * b.c0;
+  bool *of = &lin_overflow;
+  r.c0 = ck_add(a.c0, ck_mul(sb, b.c0, of), of);
   size_t i = 0, j = 0;
   while (i < a.terms.size() || j < b.terms.size()) {
     if (j >= b.terms.size() || (i < a.terms.size() && a.terms[i].atom < b.terms[j].atom)) {
       r.terms.push_back(a.terms[i++]);
     } else if (i >= a.terms.size() || b.terms[j].atom < a.terms[i].atom) {
-      r.terms.push_back({sb * b.terms[j].coef, b.terms[j].atom});
+      r.terms.push_back({ck_mul(sb, b.terms[j].coef, of), b.terms[j].atom});
       j++;
     } else {
-      int64_t c = a.terms[i].coef + sb * b.terms[j].coef;
+      int64_t c = ck_add(a.terms[i].coef, ck_mul(sb, b.terms[j].coef, of), of);
       if (c != 0) r.terms.push_back({c, a.terms[i].atom});
       i++; j++;
     }
@@ -97,8 +111,11 @@ Lin KernelGraph::lin_recombine(const Lin &a) const {
 Lin KernelGraph::lin_scale(const Lin &a, int64_t s) const {
   Lin r;
   if (s == 0) return r;
-  r.c0 = a.c0 * s;
-  for (const Term &t : a.terms) r.terms.push_back({t.coef * s, t.atom});
+  r.c0 = ck_mul(a.c0, s, &lin_overflow);
+  for (const Term &t : a.terms) {
+    const int64_t c = ck_mul(t.coef, s, &lin_overflow);
+    if (c != 0) r.terms.push_back({c, t.atom});
+  }
   return r;
 }
 
@@ -385,6 +402,7 @@ bool KernelGraph::build(const PolyUOp *root) {
       r.node = i; r.bound_node = k.src[0]; r.is_reduce = false; r.extent = -1;
       const PolyUOp *b = nodes[(size_t)k.src[0]].u;
       if (b->op == POLY_OP_CONST) r.extent = b->arg.i;
+      if (r.extent > ((int64_t)1 << 40)) { error = "RANGE with an extent beyond 2^40"; return false; }
       if (k.u == slab_range) {
         if (r.extent < 0 || slab_lo < 0 || slab_extent <= 0 || slab_lo + slab_extent > r.extent) { error = "slab outside its range"; return false; }
         r.extent = slab_extent;
@@ -420,6 +438,11 @@ bool KernelGraph::build(const PolyUOp *root) {
     if (k.src.empty()) { error = "REDUCE without a value"; return false; }
     if (k.u->arg.kind != POLY_ARG_INT && k.u->arg.kind != POLY_ARG_OPS) {
       error = "REDUCE without an op argument"; return false;
+    }
+    {
+      // read as an integer: the value is checked before anything treats it as a PolyOps
+      const int64_t rop = k.u->arg.kind == POLY_ARG_OPS ? (int64_t)(int)k.u->arg.ops : k.u->arg.i;
+      if (rop != POLY_OP_ADD && rop != POLY_OP_MUL && rop != POLY_OP_MAX) { error = "REDUCE with an op other than ADD, MUL, MAX"; return false; }
     }
     // Axes of extent 1 arrive as constants in place of ranges (or as no source at all); only
     // real RANGEs make a loop, as in the reference's lowering (src/codegen.c:1431-1439).
@@ -612,6 +635,7 @@ bool KernelGraph::build(const PolyUOp *root) {
       }
     k.deps = d;
   }
+  if (lin_overflow) { error = "index arithmetic leaves the 64-bit range"; return false; }
   return true;
 }
 
@@ -629,13 +653,15 @@ struct RawEval {
     switch (k.op) {
       case POLY_OP_CONST: return k.u->arg.i;
       case POLY_OP_RANGE: return rv[(size_t)g.range_ord.at(id)] + (g.slab_range && k.u == g.slab_range ? g.slab_lo : 0);
-      case POLY_OP_ADD: return S(0) + S(1);
-      case POLY_OP_SUB: return S(0) - S(1);
-      case POLY_OP_MUL: return S(0) * S(1);
-      case POLY_OP_NEG: return -S(0);
-      case POLY_OP_IDIV: { int64_t b = S(1); if (b == 0) { ok = false; return 0; } return (int64_t)((int32_t)S(0) / (int32_t)b); }
-      case POLY_OP_MOD: { int64_t b = S(1); if (b == 0) { ok = false; return 0; } return (int64_t)((int32_t)S(0) % (int32_t)b); }
-      case POLY_OP_SHL: return S(0) << (S(1) & 31);
+      // (wrapping arithmetic: the check compares two evaluations, it must not trip over
+      // what a damaged graph makes them compute)
+      case POLY_OP_ADD: return (int64_t)((uint64_t)S(0) + (uint64_t)S(1));
+      case POLY_OP_SUB: return (int64_t)((uint64_t)S(0) - (uint64_t)S(1));
+      case POLY_OP_MUL: return (int64_t)((uint64_t)S(0) * (uint64_t)S(1));
+      case POLY_OP_NEG: return (int64_t)(0 - (uint64_t)S(0));
+      case POLY_OP_IDIV: { const int32_t a = (int32_t)S(0), b = (int32_t)S(1); if (b == 0 || (a == INT32_MIN && b == -1)) { ok = false; return 0; } return (int64_t)(a / b); }
+      case POLY_OP_MOD: { const int32_t a = (int32_t)S(0), b = (int32_t)S(1); if (b == 0 || (a == INT32_MIN && b == -1)) { ok = false; return 0; } return (int64_t)(a % b); }
+      case POLY_OP_SHL: return (int64_t)((uint64_t)S(0) << (S(1) & 31));
       case POLY_OP_SHR: return S(0) >> (S(1) & 31);
       case POLY_OP_CAST:
         if (g.n(k.src[0]).dt == DT_I32 || g.n(k.src[0]).dt == DT_INDEX) return S(0);
@@ -647,17 +673,17 @@ struct RawEval {
     const Atom &at = g.atoms[(size_t)a];
     switch (at.kind) {
       case Atom::RANGE: return rv[(size_t)g.range_ord.at(at.node)];
-      case Atom::DIV: return lin(at.inner) / at.c;
-      case Atom::MOD: return lin(at.inner) % at.c;
+      case Atom::DIV: { const int64_t v = lin(at.inner); if (at.c == 0 || (v == INT64_MIN && at.c == -1)) { ok = false; return 0; } return v / at.c; }
+      case Atom::MOD: { const int64_t v = lin(at.inner); if (at.c == 0 || (v == INT64_MIN && at.c == -1)) { ok = false; return 0; } return v % at.c; }
       case Atom::OPAQUE: return node_raw_opaque(at.node);
       default: ok = false; return 0;
     }
   }
   int64_t node_raw_opaque(int id) { return node(id); }
   int64_t lin(const Lin &l) {
-    int64_t v = l.c0;
-    for (const Term &t : l.terms) v += t.coef * atom(t.atom);
-    return v;
+    uint64_t v = (uint64_t)l.c0;
+    for (const Term &t : l.terms) v += (uint64_t)t.coef * (uint64_t)atom(t.atom);
+    return (int64_t)v;
   }
 };
 }  // namespace

@@ -114,6 +114,9 @@ struct KernelGraph {
   Lin lin_div(const Lin &a, int64_t c);
   Lin lin_mod(const Lin &a, int64_t c);
   void lin_bounds(const Lin &a, int64_t *lo, int64_t *hi) const;
+  // Set when a coefficient or constant of a canonical form left the 64-bit range (only a
+  // damaged graph gets there): build() then fails instead of lowering nonsense.
+  mutable bool lin_overflow = false;
   // coefficient of RANGE ordinal `ord` in `l`; *affine=false when `l` holds a
   // non-affine atom that depends on that range.
   int64_t lin_range_coef(const Lin &l, int ord, bool *affine) const;

@@ -256,7 +256,9 @@ PolyHipPlanFile *poly_hip_planfile_load(const char *path) {
   }
   for (uint32_t i = 0; i < n_slots && !r.bad; i++) {
     PolyScheduleBufSlot b{};
-    b.dtype = dtype_of_code(r.get<uint8_t>());
+    const uint8_t slot_dt = r.get<uint8_t>();
+    if (slot_dt >= POLYHIP_DT_COUNT) { r.bad = true; break; }
+    b.dtype = dtype_of_code(slot_dt);
     b.is_intermediate = r.get<uint8_t>() != 0;
     b.external_buf_idx = r.get<int32_t>();
     b.numel = r.get<int64_t>();
@@ -290,9 +292,15 @@ PolyHipPlanFile *poly_hip_planfile_load(const char *path) {
     nodes.reserve(nn);
     for (uint32_t j = 0; j < nn && !r.bad; j++) {
       PolyUOp u{};
-      u.op = (PolyOps)r.get<uint16_t>();
-      u.dtype = dtype_of_code(r.get<uint8_t>());
+      // every enumeration read from the file is range-checked before it becomes one
+      const uint16_t op_code = r.get<uint16_t>();
+      if (op_code < 1 || op_code >= (uint16_t)POLY_OP_COUNT) { r.bad = true; break; }
+      u.op = (PolyOps)op_code;
+      const uint8_t dt_code = r.get<uint8_t>();
+      if (dt_code >= POLYHIP_DT_COUNT) { r.bad = true; break; }
+      u.dtype = dtype_of_code(dt_code);
       uint8_t flags = r.get<uint8_t>();
+      if (((flags >> 1) & 3) > (uint8_t)POLY_ADDR_REG) { r.bad = true; break; }
       u.dtype.count = r.get<uint16_t>();
       if (u.dtype.count > 1) u.dtype.bitsize = (uint16_t)(u.dtype.bitsize * u.dtype.count);
       u.dtype.vcount = r.get<uint16_t>();
@@ -308,14 +316,21 @@ PolyHipPlanFile *poly_hip_planfile_load(const char *path) {
         pf->srcs.back().push_back(nodes[si]);
       }
       u.src = pf->srcs.back().empty() ? nullptr : pf->srcs.back().data();
-      u.arg.kind = (PolyArgKind)r.get<uint8_t>();
+      const uint8_t kind_code = r.get<uint8_t>();
+      if (kind_code > (uint8_t)POLY_ARG_INVALID) { r.bad = true; break; }
+      u.arg.kind = (PolyArgKind)kind_code;
+      auto get_op = [&]() {
+        const uint32_t v = r.get<uint32_t>();
+        if (v < 1 || v >= (uint32_t)POLY_OP_COUNT) { r.bad = true; return POLY_OP_NOOP; }
+        return (PolyOps)v;
+      };
       bool is_var = false;
       switch (u.arg.kind) {
         case POLY_ARG_NONE: case POLY_ARG_INVALID: break;
         case POLY_ARG_INT: u.arg.i = r.get<int64_t>(); break;
         case POLY_ARG_FLOAT: u.arg.f = r.get<double>(); break;
         case POLY_ARG_BOOL: u.arg.b = r.get<uint8_t>() != 0; break;
-        case POLY_ARG_OPS: u.arg.ops = (PolyOps)r.get<uint32_t>(); break;
+        case POLY_ARG_OPS: u.arg.ops = get_op(); break;
         case POLY_ARG_STRING: pf->strings.push_back(r.str()); u.arg.str = pf->strings.back().c_str(); break;
         case POLY_ARG_INT_TUPLE: {
           uint32_t c = r.get<uint32_t>();
@@ -336,7 +351,7 @@ PolyHipPlanFile *poly_hip_planfile_load(const char *path) {
           break;
         }
         case POLY_ARG_REDUCE_AXIS: {
-          u.arg.reduce_axis.op = (PolyOps)r.get<uint32_t>();
+          u.arg.reduce_axis.op = get_op();
           uint32_t c = r.get<uint32_t>();
           if (c > (1u << 20)) { r.bad = true; break; }
           pf->ints.emplace_back();
@@ -347,7 +362,9 @@ PolyHipPlanFile *poly_hip_planfile_load(const char *path) {
         }
         case POLY_ARG_RANGE: {
           u.arg.range.axis_id = r.get<int64_t>();
-          u.arg.range.axis_type = (PolyAxisType)r.get<uint32_t>();
+          const uint32_t axis_type = r.get<uint32_t>();
+          if (axis_type > (uint32_t)POLY_AXIS_PLACEHOLDER) { r.bad = true; break; }
+          u.arg.range.axis_type = (PolyAxisType)axis_type;
           uint32_t c = r.get<uint32_t>();
           if (c > (1u << 20)) { r.bad = true; break; }
           pf->ints.emplace_back();
