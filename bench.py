@@ -59,7 +59,7 @@ def run_gpu(workload, steps, warmup):
     t0 = time.perf_counter()
     plan = HipPlan.from_file(path)
     compile_s = time.perf_counter() - t0
-    if workload.startswith("gpt2_medium_block_train"):
+    if workload.startswith("gpt2_medium_block_train") or workload.startswith("gpt2_medium_train"):
         data, _ = block_train_slot_tensors(plan)
         tokens = None
     elif workload.startswith("gpt2"):

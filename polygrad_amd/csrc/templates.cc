@@ -1127,6 +1127,9 @@ extern "C" __global__ void __launch_bounds__(1024) poly_guard(int* flag, const %
   if (threadIdx.x == 0) bad = 0;
   __syncthreads();
   int mine = 0;
+  // (unrolled: the loads of all steps are in flight together -- one memory latency for the
+  // whole check instead of one per step)
+#pragma unroll 16
   for (long long i = (long long)threadIdx.x * 4; i < %lldll; i += 4096) {
 #pragma unroll
     for (int j = 0; j < 4; j++)

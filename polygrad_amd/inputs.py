@@ -92,7 +92,7 @@ def block_train_slot_tensors(plan, vocab=50257, seed=4, device="cuda"):
             t = torch.full((n,), 1.0 / (1.0 - 0.999), dtype=dt, device=device)
         elif name.endswith(".m") or name.endswith(".v") or name == "loss" or name.endswith("_b"):
             t = torch.zeros(n, dtype=dt, device=device)
-        elif name in ("ln1_w", "ln2_w", "lnf_w"):
+        elif name.split(".")[-1] in ("ln1_w", "ln2_w", "lnf_w"):     # (blocks of a deeper stack are named h<i>.<parameter>)
             t = torch.ones(n, dtype=dt, device=device)
         else:
             t = (torch.randn(n, generator=g, device=device, dtype=torch.float32) * 0.02).to(dt)

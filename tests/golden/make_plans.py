@@ -10,6 +10,8 @@ the GPU box, where the reference frontend is not part of the product path:
     polygrad_amd/plans/adamw_f32_355m.polyplan             config 5: AdamW update of 355 M fp32 parameters
     polygrad_amd/plans/gpt2_medium_block_train_b4_t1024.polyplan   config 5: one block + head, backward, AdamW
     polygrad_amd/plans/gpt2_small_layer_matmuls_b8_t1024.polyplan  the four weight matmuls of a GPT-2 small layer with their tails
+    polygrad_amd/plans/gpt2_medium_train_24l_b4_t1024.polyplan     config 5 whole: 24 blocks, head, loss, backward, AdamW
+                                                                   (`python tests/golden/make_plans.py train24`)
 
 The graphs are built with the REAL reference frontend and scheduler
 (oracle/_ref/libpolygrad.so through tests/refpoly.py); only the scheduled kernel
@@ -102,5 +104,19 @@ def main():
     c.close()
 
 
+def train_24_layers():
+    """Config 5 whole: 24 blocks of GPT-2 medium above the embedding, head, loss, backward,
+    AdamW.  Needs the build of the reference with raised buffer caps
+    (oracle/_ref/libpolygrad_hip_ref.so, `make -C oracle ref_hip`): the stock limits stop at
+    256 buffers (src/frontend_internal.h:23).  Scheduling takes about six minutes."""
+    c = R.Ctx(hip_ref=True)
+    _, sink = graphs.gpt2_block_train_step(c, batch=4, ctx=1024, d_model=1024, heads=16, vocab=50257, n_blocks=24)
+    save(c, sink, "gpt2_medium_train_24l_b4_t1024")
+    c.close()
+
+
 if __name__ == "__main__":
-    main()
+    if sys.argv[1:] == ["train24"]:
+        train_24_layers()
+    else:
+        main()

@@ -298,26 +298,40 @@ BLOCK_PARAMS = ("ln1_w", "ln1_b", "attn_w", "attn_b", "proj_w", "proj_b", "ln2_w
                 "lnf_w", "lnf_b", "head_w")
 
 
+LAYER_PARAMS = BLOCK_PARAMS[:12]
+
+
+def train_param_names(n_blocks):
+    """Parameter names of gpt2_block_train_step: one block keeps the bare names, several
+    blocks prefix theirs with h<i>. (the final LayerNorm and the head stay bare)."""
+    if n_blocks == 1:
+        return list(BLOCK_PARAMS)
+    return [f"h{i}.{n}" for i in range(n_blocks) for n in LAYER_PARAMS] + ["lnf_w", "lnf_b", "head_w"]
+
+
 def gpt2_block_train_step(c, batch=4, ctx=1024, d_model=1024, heads=16, vocab=50257, lr=3e-4, beta1=0.9, beta2=0.999,
-                          eps=1e-8, weight_decay=0.1, ln_eps=1e-5, head_vd=True):
-    """One transformer block of config 5 (GPT-2 medium shapes) with the final LayerNorm,
-    the vocabulary projection and next-token cross-entropy, reverse-mode gradients from the
-    reference's poly_grad (src/autograd.c:773) and an AdamW update of every parameter
-    (src/instance.c:1162-1224).  Mixed precision: fp32 master parameters and optimizer
-    state, bf16 copies of the weights and bf16 activations for the matmuls, fp32
-    reductions.  The block's input activations stand in for the layers below it.
-    Returns (bufs, sink): the sink stores the loss and updates p, m, v of all 15 parameters."""
+                          eps=1e-8, weight_decay=0.1, ln_eps=1e-5, head_vd=True, n_blocks=1):
+    """n_blocks transformer blocks of config 5 (GPT-2 medium shapes; 24 of them are the
+    whole model above the embedding) with the final LayerNorm, the vocabulary projection and
+    next-token cross-entropy, reverse-mode gradients from the reference's poly_grad
+    (src/autograd.c:773) and an AdamW update of every parameter (src/instance.c:1162-1224).
+    Mixed precision: fp32 master parameters and optimizer state, bf16 copies of the weights
+    and bf16 activations for the matmuls, fp32 reductions.  The first block's input
+    activations stand in for the embedding below it.
+    Returns (bufs, sink): the sink stores the loss and updates p, m, v of every parameter."""
     B, T, D, H, V = batch, ctx, d_model, heads, vocab
     hd = D // H
     shapes = dict(ln1_w=(D,), ln1_b=(D,), attn_w=(D, 3 * D), attn_b=(3 * D,), proj_w=(D, D), proj_b=(D,), ln2_w=(D,),
                   ln2_b=(D,), fc_w=(D, 4 * D), fc_b=(4 * D,), fc2_w=(4 * D, D), fc2_b=(D,), lnf_w=(D,), lnf_b=(D,),
                   head_w=(V, D) if head_vd else (D, V))      # (V, D): tied-embedding layout, as GPT-2 stores it
+    names = train_param_names(n_blocks)
     bufs = {}
     P = {}
-    for name in BLOCK_PARAMS:
-        P[name] = bufs[name] = c.buffer(shapes[name], R.F32, name=name)
-        bufs[name + ".m"] = c.buffer(shapes[name], R.F32, name=name + ".m")
-        bufs[name + ".v"] = c.buffer(shapes[name], R.F32, name=name + ".v")
+    for name in names:
+        shape = shapes[name.split(".")[-1]]
+        P[name] = bufs[name] = c.buffer(shape, R.F32, name=name)
+        bufs[name + ".m"] = c.buffer(shape, R.F32, name=name + ".m")
+        bufs[name + ".v"] = c.buffer(shape, R.F32, name=name + ".v")
     h0 = bufs["h0"] = c.buffer((B, T, D), R.BF16, name="h0")
     target = bufs["target"] = c.buffer((B * T,), R.F32, name="target")     # class ids as floats (sparse cross-entropy)
     arange = bufs["arange"] = c.buffer((T,), R.F32, name="arange")
@@ -330,29 +344,44 @@ def gpt2_block_train_step(c, batch=4, ctx=1024, d_model=1024, heads=16, vocab=50
     col = arange.reshape((1, T)).expand((T, T))
     mask = row.lt(col).where(c.const(-1e9, R.BF16), c.const(0.0, R.BF16)).reshape((1, 1, T, T)).contiguous()
     wdt = R.BF16
-    ln1 = _layernorm(h0, W["ln1_w"], W["ln1_b"], ln_eps, wdt).contiguous()
-    qkv = _linear(ln1, W["attn_w"], W["attn_b"], wdt).contiguous()
-    q = qkv.shrink(((0, B), (0, T), (0, D))).contiguous().reshape((B, T, H, hd)).permute((0, 2, 1, 3))
-    k = qkv.shrink(((0, B), (0, T), (D, 2 * D))).contiguous().reshape((B, T, H, hd)).permute((0, 2, 1, 3))
-    v = qkv.shrink(((0, B), (0, T), (2 * D, 3 * D))).contiguous().reshape((B, T, H, hd)).permute((0, 2, 1, 3))
-    scores = q.cast(R.F32).dot(k.permute((0, 1, 3, 2)).cast(R.F32)).cast(wdt).contiguous()
-    scores = (scores * c.const(1.0 / math.sqrt(hd), wdt) + mask.expand((B, H, T, T))).contiguous()
-    attn = scores.cast(R.F32).softmax(-1).cast(wdt).contiguous()
-    ctxv = attn.cast(R.F32).dot(v.cast(R.F32)).cast(wdt).contiguous()
-    merged = ctxv.permute((0, 2, 1, 3)).reshape((B, T, D))
-    h1 = (h0 + _linear(merged, W["proj_w"], W["proj_b"], wdt).contiguous()).contiguous()
-    ln2 = _layernorm(h1, W["ln2_w"], W["ln2_b"], ln_eps, wdt).contiguous()
-    ff = _linear(ln2, W["fc_w"], W["fc_b"], wdt).contiguous().gelu().contiguous()
-    h2 = (h1 + _linear(ff, W["fc2_w"], W["fc2_b"], wdt).contiguous()).contiguous()
-    lnf = _layernorm(h2, W["lnf_w"], W["lnf_b"], ln_eps, wdt).contiguous()
+    h = h0
+    for i in range(n_blocks):
+        w = (lambda n: W[n]) if n_blocks == 1 else (lambda n, i=i: W[f"h{i}.{n}"])
+        ln1 = _layernorm(h, w("ln1_w"), w("ln1_b"), ln_eps, wdt).contiguous()
+        qkv = _linear(ln1, w("attn_w"), w("attn_b"), wdt).contiguous()
+        q = qkv.shrink(((0, B), (0, T), (0, D))).contiguous().reshape((B, T, H, hd)).permute((0, 2, 1, 3))
+        k = qkv.shrink(((0, B), (0, T), (D, 2 * D))).contiguous().reshape((B, T, H, hd)).permute((0, 2, 1, 3))
+        v = qkv.shrink(((0, B), (0, T), (2 * D, 3 * D))).contiguous().reshape((B, T, H, hd)).permute((0, 2, 1, 3))
+        scores = q.cast(R.F32).dot(k.permute((0, 1, 3, 2)).cast(R.F32)).cast(wdt).contiguous()
+        scores = (scores * c.const(1.0 / math.sqrt(hd), wdt) + mask.expand((B, H, T, T))).contiguous()
+        attn = scores.cast(R.F32).softmax(-1).cast(wdt).contiguous()
+        ctxv = attn.cast(R.F32).dot(v.cast(R.F32)).cast(wdt).contiguous()
+        merged = ctxv.permute((0, 2, 1, 3)).reshape((B, T, D))
+        h1 = (h + _linear(merged, w("proj_w"), w("proj_b"), wdt).contiguous()).contiguous()
+        ln2 = _layernorm(h1, w("ln2_w"), w("ln2_b"), ln_eps, wdt).contiguous()
+        ff = _linear(ln2, w("fc_w"), w("fc_b"), wdt).contiguous().gelu().contiguous()
+        h = (h1 + _linear(ff, w("fc2_w"), w("fc2_b"), wdt).contiguous()).contiguous()
+    lnf = _layernorm(h, W["lnf_w"], W["lnf_b"], ln_eps, wdt).contiguous()
     hw = W["head_w"].permute((1, 0)) if head_vd else W["head_w"]
     logits = lnf.reshape((B * T, D)).cast(R.F32).dot(hw.cast(R.F32)).contiguous()   # fp32 logits
     loss = logits.cross_entropy(target)
     assigns = []
-    for name in BLOCK_PARAMS:
+    grads = {}
+    if n_blocks > 1:
+        # one reverse pass for all parameters, as the reference's own training graph takes
+        # them (poly_grad_many, src/instance.c:876-963); a pass per parameter grows with the
+        # square of the depth
+        import ctypes as C
+        wrts = (C.c_void_p * len(names))(*[P[nm].buf for nm in names])
+        outs = (C.c_void_p * len(names))()
+        if c.L.poly_grad_many(c.ctx, loss.u, None, wrts, len(names), outs) != 0:
+            raise RuntimeError("poly_grad_many failed")
+        for nm, u in zip(names, outs):
+            grads[nm] = R.T(c, u, P[nm].shape, P[nm].dt).reshape((int(np.prod(P[nm].shape)),))
+    for name in names:
         p, m, vv = P[name], bufs[name + ".m"], bufs[name + ".v"]
         n = int(np.prod(p.shape))
-        g = T_grad(c, loss, p, n)
+        g = grads[name] if name in grads else T_grad(c, loss, p, n)
         pf, mf, vf = p.reshape((n,)), m.reshape((n,)), vv.reshape((n,))
         m_new = c.const(beta1) * mf + c.const(1.0 - beta1) * g
         v_new = c.const(beta2) * vf + c.const(1.0 - beta2) * (g * g)
@@ -381,7 +410,7 @@ def gpt2_block_train_inputs(bufs, batch, ctx, vocab, seed=4):
             a = np.array([1.0 / (1.0 - 0.999)], np.float32)
         elif name.endswith(".m") or name.endswith(".v") or name == "loss" or name.endswith("_b"):
             a = np.zeros(n, np.float32)
-        elif name in ("ln1_w", "ln2_w", "lnf_w"):
+        elif name.split(".")[-1] in ("ln1_w", "ln2_w", "lnf_w"):
             a = np.ones(n, np.float32)
         else:
             a = g.normal(0.0, 0.02, n).astype(np.float32)

@@ -106,6 +106,7 @@ def lib(path=None):
         "poly_compiled_plan_run": (C.c_int, [P, C.POINTER(P), C.c_int, P, C.c_int]),
         "poly_compiled_plan_free": (None, [P]),
         "poly_grad": (P, [P, P, P]),
+        "poly_grad_many": (C.c_int, [P, P, P, C.POINTER(P), C.c_int, C.POINTER(P)]),
         "poly_const_buffer_data": (P, [P, P]),
         "poly_define_var": (P, [P, C.c_char_p, C.c_int64, C.c_int64]), "poly_bind_var": (P, [P, P, C.c_int64]),
         "poly_buffer_var": (P, [P, PolyDType, P, I64P, C.c_int]),
