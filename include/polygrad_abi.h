@@ -3,7 +3,7 @@
  * consumes, re-declared so that this backend builds without polygrad's headers.
  *
  * Every type below must stay layout-identical (x86-64 SysV) to the reference
- * declaration it cites; tests/test_abi_layout.py checks sizes and offsets
+ * declaration it cites; tests/test_render_cpu.py checks sizes and offsets
  * against the real library where it is available.  Names are kept identical
  * on purpose: a translation unit inside polygrad that includes both this file
  * and polygrad's own headers must define POLYGRAD_ABI_USE_NATIVE_HEADERS and

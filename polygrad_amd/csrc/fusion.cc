@@ -1543,6 +1543,7 @@ static bool match_attention(const Sched &sc, int s_item, const std::vector<char>
     score = strf("%s(%s, m, n, z, %s)", fn.c_str(), score.c_str(), call_args(m.item).c_str());
   }
   cfg += strf("#define POLY_FA_SCORE(acc, m, n, z) %s\n", score.c_str());
+  bool mask_table = false;   // a kernel ahead of this one looks at the mask once for all z
   // An additive mask: the stored score is cast(f(acc) + mask[...]) with f made of casts
   // and products with positive constants, and the mask a bf16 buffer read at consecutive
   // positions for consecutive keys.  The kernel then loads the mask entries of a tile
@@ -1558,6 +1559,7 @@ static bool match_attention(const Sched &sc, int s_item, const std::vector<char>
     auto strip = [&](int v) { while (g.n(v).op == POLY_OP_CAST && dt_is_float(g.n(v).dt) && dt_is_float(g.n(g.n(v).src[0]).dt)) v = g.n(v).src[0]; return v; };
     const int top = strip(n_chain ? g.stores[0].value : stS.value);
     int mask_ld = -1, other = -1;
+    bool mask_z_free = false;   // the mask entry does not depend on z
     if (g.n(top).op == POLY_OP_ADD && g.n(top).dt == tin)
       for (int side = 0; side < 2; side++) {
         const int cand = g.n(top).src[(size_t)side];
@@ -1569,6 +1571,11 @@ static bool match_attention(const Sched &sc, int s_item, const std::vector<char>
         if (it == a.c.end() || it->second != 1) continue;
         mask_ld = cand;
         other = g.n(top).src[(size_t)(1 - side)];
+        mask_z_free = true;
+        for (const auto &d : mS.zd) {
+          auto zc = a.c.find(d.ord);
+          if (zc != a.c.end() && zc->second != 0) mask_z_free = false;
+        }
       }
     // f: from acc (or the chain input x) through casts and products with positive constants
     std::function<bool(int)> plain = [&](int id) -> bool {
@@ -1622,6 +1629,7 @@ static bool match_attention(const Sched &sc, int s_item, const std::vector<char>
       value_fn(lm, "poly_fa_score_nomask", "float", n_chain ? strf("%s x", tn).c_str() : "float acc", other, pre_acc);
       cfg += strf("#define POLY_FA_SCORE_NOMASK(acc, m, n, z) poly_fa_score_nomask(%s, m, n, z, %s)\n", head.c_str(), call_args(lm.item).c_str());
       if (failed && !failed_before) { failed = false; cfg.resize(before); }
+      else if (!failed && mask_z_free && !getenv("POLY_HIP_NO_MASK_TABLE")) mask_table = true;
     }
   }
   // Single-pass form when the group is a plain softmax: p = cast(term / sum) with
@@ -1664,6 +1672,34 @@ static bool match_attention(const Sched &sc, int s_item, const std::vector<char>
   out->arg_slots = arg_slots;
   RenderedKernel &rk = out->rk;
   rk = RenderedKernel();
+  // timing experiments: extra macro definitions, "NAME=VALUE;NAME=VALUE"
+  if (const char *e = getenv("POLY_HIP_FA_DEFS")) {
+    std::string d(e);
+    size_t pos = 0;
+    while (pos < d.size()) {
+      size_t end = d.find(';', pos);
+      if (end == std::string::npos) end = d.size();
+      std::string item = d.substr(pos, end - pos);
+      const size_t eq = item.find('=');
+      if (!item.empty()) cfg += "#define " + (eq == std::string::npos ? item + " 1" : item.substr(0, eq) + " " + item.substr(eq + 1)) + "\n";
+      pos = end + 1;
+    }
+  }
+  if (mask_table) {
+    // One word per 32 x 32 tile and one per block of 128 queries x 64 keys, written by a
+    // first kernel into scratch memory that the main kernel takes as its last argument.
+    const std::string from = strf("#define POLY_SIGNATURE %s\n", sig.c_str());
+    const size_t at = cfg.find(from);
+    if (at == std::string::npos) FA_REJECT();
+    cfg.replace(at, from.size(), strf("#define POLY_SIGNATURE %s, unsigned int* poly_scratch\n#define POLY_FA_MASK_TABLE poly_scratch\n", sig.c_str()));
+    RenderedKernel::Pre pre;
+    pre.source = std::string(hip_prelude()) + cfg + "#define POLY_FA_CLASSIFY 1\n" + kAttentionTemplate;
+    pre.entry = "poly_k";
+    pre.launch.grid[0] = (unsigned)((mS.M / 128) * (mS.N / 64));
+    pre.launch.block[0] = 512;
+    rk.pres.push_back(pre);
+    rk.scratch_bytes = (size_t)((mS.M / 32) * (mS.N / 32) + (mS.M / 128) * (mS.N / 64)) * sizeof(unsigned);
+  }
   rk.source = std::string(hip_prelude()) + cfg + kAttentionTemplate;
   rk.entry = "poly_k";
   rk.launch.grid[0] = (unsigned)((mS.M / 128) * mS.Z);
@@ -1672,6 +1708,7 @@ static bool match_attention(const Sched &sc, int s_item, const std::vector<char>
   rk.strategy = strf("fused attention (%zu kernels): mfma 32x32x16 %s Z=%lld M=%lld N=%lld D=64, %s", all.size() + copy_items.size(),
                      tin == DT_BF16 ? "bf16" : "f16", (long long)mS.Z, (long long)mS.M, (long long)mS.N,
                      cfg.find("#define POLY_FA_ONLINE 1") != std::string::npos ? "one pass, online softmax" : "two passes over keys, exact roundings");
+  if (mask_table) rk.strategy += ", mask tiles classified by a first kernel";
   rk.n_params = (int)arg_slots.size();
   rk.n_vars = 0;
   rk.flops = 2.0 * (double)mS.Z * (double)mS.M * (double)mS.N * (double)(mS.K + mV.N);

@@ -48,6 +48,13 @@
 //   POLY_FA_ONLINE                     1: single pass (needs p = cast(term / sum),
 //                                      term(x, mx) = exp2((x - mx) * POLY_FA_C) and the
 //                                      maximum taken over the scores themselves)
+//   POLY_FA_MASK_TABLE                 (optional, with POLY_FA_MASK_PTR, when the mask does
+//                                      not depend on z) pointer to the words that the
+//                                      classifying kernel below writes: the mask is then
+//                                      looked at once for all z instead of by every wave
+//   POLY_FA_CLASSIFY                   compile the classifying kernel instead of the
+//                                      attention kernel (same configuration block, the
+//                                      same arguments)
 //
 // Online form: one pass.  Per 32-key tile a wave computes the scores x exactly as the
 // pointwise chain stores them (POLY_FA_SCORE, roundings included), the new running
@@ -55,9 +62,10 @@
 // the output accumulators by exp2((m_old - m) * c) when a maximum moved, and accumulates
 // O^T += V^T cast(t)^T; the division by the sum happens once at the end.  Against the
 // unfused kernels the 16-bit rounding of the probabilities moves from t / sum to t (the
-// output differs from theirs by about one 16-bit rounding), and a key tile whose terms are
-// all exact zeros against the running maxima (as under a causal mask) is skipped after
-// its scores, so a non-finite V under zero probability does not propagate.
+// output differs from theirs by about one 16-bit rounding).  A key tile whose mask entries
+// are all -inf is passed over before its scores, and one whose terms are all exact zeros
+// against the running maxima after them: a non-finite product or V under probabilities
+// that are all zero does not propagate.
 // The output is transposed relative to the exact form: a lane holds ONE query in both
 // MFMAs, so maximum, sum and rescaling factor are per-lane scalars.
 //
@@ -78,11 +86,22 @@
 #define POLY_Q_PTR data1
 #define POLY_K_PTR data2
 #define POLY_V_PTR data3
+#ifdef POLY_STANDALONE_QKV   // q, k, v as column blocks of one [8192, 2304] buffer
+__device__ __forceinline__ int poly_q_off(int z, int m) { return (z / 12) * 2359296 + (z % 12) * 64 + m * 2304; }
+__device__ __forceinline__ int poly_k_off(int z, int n) { return (z / 12) * 2359296 + (z % 12) * 64 + n * 2304 + 768; }
+__device__ __forceinline__ int poly_v_off(int z, int n) { return (z / 12) * 2359296 + (z % 12) * 64 + n * 2304 + 1536; }
+#else
 __device__ __forceinline__ int poly_q_off(int z, int m) { return (z / 12) * 786432 + (z % 12) * 64 + m * 768; }
 __device__ __forceinline__ int poly_k_off(int z, int n) { return (z / 12) * 786432 + (z % 12) * 64 + n * 768; }
 __device__ __forceinline__ int poly_v_off(int z, int n) { return (z / 12) * 786432 + (z % 12) * 64 + n * 768; }
+#endif
+#ifdef POLY_STANDALONE_MASK_TABLE
+#define POLY_SIGNATURE __bf16 *data0, const __bf16 *__restrict__ data1, const __bf16 *__restrict__ data2, const __bf16 *__restrict__ data3, const __bf16 *__restrict__ data4, unsigned int *poly_scratch
+#define POLY_FA_MASK_TABLE poly_scratch
+#else
 #define POLY_SIGNATURE __bf16 *data0, const __bf16 *__restrict__ data1, const __bf16 *__restrict__ data2, const __bf16 *__restrict__ data3, const __bf16 *__restrict__ data4
-#define POLY_FA_SCORE(acc, m, n, z) ((__bf16)((float)(__bf16)((float)(__bf16)(acc) * 0.125f) + (float)data4[(m) * 1024 + (n)]))
+#endif
+#define POLY_FA_SCORE(acc, m, n, z) ((__bf16)((float)(__bf16)(acc) * 0.125f + (float)data4[(m) * 1024 + (n)]))
 #define POLY_FA_MAXV(x, m, n, z) ((float)(x))
 #define POLY_FA_TERM(x, mx, m, n, z) __builtin_amdgcn_exp2f(((float)(x) - (mx)) * 0x1.715476p+0f)
 #define POLY_FA_P(x, mx, sum, m, n, z) ((__bf16)(__builtin_amdgcn_exp2f(((float)(x) - (mx)) * 0x1.715476p+0f) / (sum)))
@@ -90,6 +109,9 @@ __device__ __forceinline__ int poly_v_off(int z, int n) { return (z / 12) * 7864
 #define POLY_FA_SKIP_DEAD_BLOCKS 1
 #define POLY_FA_ONLINE 1
 #define POLY_FA_C 0x1.715476p+0f
+#define POLY_FA_MASK_PTR(m, n, z) (data4 + (m) * 1024 + (n))
+#define POLY_FA_SCORE_MASK(acc, mk, m, n, z) ((__bf16)((float)(__bf16)(acc) * 0.125f + (float)(mk)))
+#define POLY_FA_SCORE_NOMASK(acc, m, n, z) ((float)(__bf16)(acc) * 0.125f)
 #endif
 #ifndef POLY_FA_ONLINE
 #define POLY_FA_ONLINE 0
@@ -113,11 +135,49 @@ typedef fa_u32x2 fa_u32x2_u __attribute__((aligned(2)));
 __device__ __forceinline__ int fa_swz(int row) { return (row ^ (row >> 3)) & 7; }
 
 __device__ __forceinline__ float fa_other_half(float v) {
-  // value held by lane ^ 32
-  const int lane = (int)(threadIdx.x & 63);
-  return __builtin_bit_cast(float, __builtin_amdgcn_ds_bpermute(((lane ^ 32) << 2), __builtin_bit_cast(int, v)));
+  // value held by lane ^ 32: v_permlane32_swap exchanges lanes 32..63 of its first operand
+  // with lanes 0..31 of its second (written as assembly: the compiler's builtin for it
+  // returned the first exchange's result for every later one)
+#ifdef POLY_HOST_ADDRESS_CHECK   // the kernel compiled for the host to check its indexing: lanes run one by one
+  return v;
+#else
+  float a = v, b = v;
+  asm volatile("s_nop 1\n\tv_permlane32_swap_b32 %0, %1\n\ts_nop 1" : "+v"(a), "+v"(b));
+  return (threadIdx.x & 32) ? a : b;
+#endif
 }
 
+#ifdef POLY_FA_CLASSIFY
+// The kernel that looks at a z-independent mask once for all z (see POLY_FA_MASK_TABLE
+// below for the layout it writes).  One workgroup of 8 waves per block of 128 queries x
+// 64 keys, one wave per 32 x 32 tile.
+extern "C" __global__ void __launch_bounds__(512) poly_k(POLY_SIGNATURE) {
+  __shared__ int dead_tiles;
+  if (threadIdx.x == 0) dead_tiles = 0;
+  __syncthreads();
+  constexpr int NB = POLY_FA_N / 64;
+  const int rb = blockIdx.x / NB, cb = blockIdx.x % NB;
+  const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
+  const int qt = 4 * rb + (wave >> 1), kt = 2 * cb + (wave & 1);
+  fa_u32x4 look[2];
+#pragma unroll
+  for (int i = 0; i < 2; i++) look[i] = *(const fa_u32x4_u *)POLY_FA_MASK_PTR(32 * qt + 16 * i + (lane >> 2), 32 * kt + 8 * (lane & 3), 0);
+  const unsigned s0 = (unsigned)__builtin_amdgcn_readfirstlane((int)((look[0][0] & 0xffffu) * 0x10001u));
+  unsigned diff = 0;
+#pragma unroll
+  for (int i = 0; i < 2; i++)
+#pragma unroll
+    for (int j = 0; j < 4; j++) diff |= look[i][j] ^ s0;
+  const bool uniform = __builtin_amdgcn_ballot_w64(diff != 0) == 0;
+  unsigned *const table = (unsigned *)(POLY_FA_MASK_TABLE);
+  if (lane == 0) {
+    table[qt * (POLY_FA_N / 32) + kt] = (s0 & 0xffffu) | (uniform ? 0x10000u : 0u);
+    if (uniform && __builtin_bit_cast(float, s0 << 16) == -__builtin_inff()) atomicAdd(&dead_tiles, 1);
+  }
+  __syncthreads();
+  if (threadIdx.x == 0) table[(POLY_FA_M / 32) * (POLY_FA_N / 32) + rb * NB + cb] = dead_tiles == 8 ? 1u : 0u;
+}
+#else
 // Three workgroups per CU (three waves per SIMD): the arithmetic on the scores is VALU work,
 // and it is the other resident waves that hide its latencies.
 extern "C" __global__ void __launch_bounds__(FA_THREADS) __attribute__((amdgpu_waves_per_eu(3, 3))) poly_k(POLY_SIGNATURE) {
@@ -231,17 +291,17 @@ extern "C" __global__ void __launch_bounds__(FA_THREADS) __attribute__((amdgpu_w
   {
     const float c = POLY_FA_C;
     fa_u32x4 rk[2], rv[4];
-    load_k(0, rk);
-    load_v(0, rv);
-    store_k(0, rk);
-    store_v(0, rv);
-    __syncthreads();
-    for (int kb = 0; kb < FA_NKB; kb++) {
-      const int cur = kb & 1;
-      if (kb + 1 < FA_NKB) { load_k(kb + 1, rk); load_v(kb + 1, rv); }
+#ifdef POLY_FA_MASK_PTR
+    // this lane's 16 keys of a tile: four runs of 4 consecutive keys, 8 bytes each (the
+    // entries of one query are consecutive in memory)
+    const POLY_TIN *const mask_row = POLY_FA_MASK_PTR(mq, 4 * half, z);
+#endif
+    // One 32 x 32 tile: tile t of key block kb, staged in LDS buffer cur.  With a mask,
+    // `uniform` says that all its 32 x 32 entries hold the one value `cmask`.
+    auto tile = [&](int cur, int kb, int t, bool uniform, float cmask) {
       // V^T fragment (A operand): feature row 32 dt + lq, the 8 keys of this lane's half
       // of the 16 keys 32t + 16u .., in the key order of the score registers
-      auto v_frag = [&](int t, int u, int dt) {
+      auto v_frag = [&](int u, int dt) {
         const int col0 = 4 * t + 2 * u;
         const int d = 32 * dt + lq;
         const POLY_TIN *row = lds_v[cur] + d * FA_BN;
@@ -252,109 +312,199 @@ extern "C" __global__ void __launch_bounds__(FA_THREADS) __attribute__((amdgpu_w
         both[0] = lo[0]; both[1] = lo[1]; both[2] = hi[0]; both[3] = hi[1];
         return __builtin_bit_cast(fa_in8, both);
       };
-#pragma unroll
-      for (int t = 0; t < 2; t++) {
+      float x[16];
 #ifdef POLY_FA_MASK_PTR
-        // mask entries of this lane's 16 keys: four runs of 4 consecutive keys, 8 bytes each
-        // (issued ahead of the MFMAs)
+      // -inf everywhere: every score of the tile is -inf whatever the (finite) product,
+      // every term an exact zero and no maximum moves; a query that has seen nothing but
+      // such tiles keeps sum 0 and ends as 0 / 0 like in the unfused kernels.  (A
+      // non-finite product goes unseen here: its key is masked out for every query of
+      // the tile, and would have made the unfused kernels' rows NaN.)
+      if (uniform && cmask == -__builtin_inff()) return;
+      asm volatile("" ::: "memory");   // (keeps the fragment reads and MFMAs below the test)
+      fa_acc16 st;
+      scores(cur, t, st);
+      if (uniform && cmask == 0.0f) {
+        // nothing is added: the score is f(acc), already a 16-bit value
+#pragma unroll
+        for (int r = 0; r < 16; r++) x[r] = POLY_FA_SCORE_NOMASK(st[r], mq, key_of(kb, t, r), z);
+      } else {
+        if (uniform) {
+          // One value c is added everywhere: the score of the largest product bounds this
+          // lane's scores.  If even its term is an exact zero against the running maximum
+          // for all 32 queries, the tile adds nothing and moves no maximum.  (A NaN product
+          // goes unseen here, as above.)
+          float amax = st[0];
+#pragma unroll
+          for (int r = 1; r < 16; r++) amax = __builtin_fmaxf(amax, st[r]);
+          const int n0 = key_of(kb, t, 0);
+          const float bound = POLY_FA_MAXV(POLY_FA_SCORE_MASK(amax, (POLY_TIN)cmask, mq, n0, z), mq, n0, z);
+          const bool early_dead = __builtin_amdgcn_exp2f((bound - m_run) * c) == 0.0f;
+          if (__builtin_amdgcn_ballot_w64(!early_dead) == 0) return;
+        }
+        // entries in the layout of the score registers
         fa_u32x2 mraw[4];
 #pragma unroll
-        for (int gq = 0; gq < 4; gq++) mraw[gq] = *(const fa_u32x2_u *)POLY_FA_MASK_PTR(mq, key_of(kb, t, 4 * gq), z);
-#endif
-        fa_acc16 st;
-        scores(cur, t, st);
-        float x[16];
-#ifdef POLY_FA_MASK_PTR
-        // Do all 32 x 32 entries hold one value?  (compared as bit patterns)
-        const unsigned s0 = (unsigned)__builtin_amdgcn_readfirstlane((int)((mraw[0][0] & 0xffffu) * 0x10001u));
-        unsigned diff = 0;
-#pragma unroll
-        for (int gq = 0; gq < 4; gq++) diff |= (mraw[gq][0] ^ s0) | (mraw[gq][1] ^ s0);
-        const bool uniform = __builtin_amdgcn_ballot_w64(diff != 0) == 0;
-        const float cmask = __builtin_bit_cast(float, s0 << 16);
-        auto mask_of = [&](int r) {   // entry of register r as the 16-bit type
-          const unsigned d = mraw[r >> 2][(r >> 1) & 1];
-          return __builtin_bit_cast(POLY_TIN, (unsigned short)((r & 1) ? (d >> 16) : (d & 0xffffu)));
-        };
-        if (uniform && cmask == 0.0f) {
-          // nothing is added: the score is f(acc), already a 16-bit value
-#pragma unroll
-          for (int r = 0; r < 16; r++) x[r] = POLY_FA_SCORE_NOMASK(st[r], mq, key_of(kb, t, r), z);
-        } else {
-          if (uniform) {
-            // One value c is added everywhere: the score of the largest product bounds this
-            // lane's scores.  If even its term is an exact zero against the running maximum
-            // for all 32 queries, the tile adds nothing and moves no maximum.  (A NaN product
-            // goes unseen here: the key it belongs to is masked out for every query of the
-            // tile, and would have made the unfused kernels' rows NaN.)
-            float amax = st[0];
-#pragma unroll
-            for (int r = 1; r < 16; r++) amax = __builtin_fmaxf(amax, st[r]);
-            const int n0 = key_of(kb, t, 0);
-            const float bound = POLY_FA_MAXV(POLY_FA_SCORE_MASK(amax, mask_of(0), mq, n0, z), mq, n0, z);
-            const bool early_dead = __builtin_amdgcn_exp2f((bound - m_run) * c) == 0.0f;
-            if (__builtin_amdgcn_ballot_w64(!early_dead) == 0) continue;
-          }
-#pragma unroll
-          for (int r = 0; r < 16; r++) {
-            const int n = key_of(kb, t, r);
-            x[r] = POLY_FA_MAXV(POLY_FA_SCORE_MASK(st[r], mask_of(r), mq, n, z), mq, n, z);
-          }
-        }
-#else
+        for (int gq = 0; gq < 4; gq++) mraw[gq] = *(const fa_u32x2_u *)(mask_row + 32 * (2 * kb + t) + 8 * gq);
 #pragma unroll
         for (int r = 0; r < 16; r++) {
           const int n = key_of(kb, t, r);
-          x[r] = POLY_FA_MAXV(POLY_FA_SCORE(st[r], mq, n, z), mq, n, z);
-        }
-#endif
-        float bm = -__builtin_inff(), nan_probe = 0.0f;
-#pragma unroll
-        for (int r = 0; r < 16; r++) {
-          bm = __builtin_fmaxf(bm, x[r]);     // ignores a NaN ...
-          nan_probe = nan_probe + x[r];        // ... which this catches (as does +inf meeting -inf)
-        }
-        bm = __builtin_fmaxf(bm, fa_other_half(bm));
-        // Against the running maximum the largest term of this tile is exactly zero (the
-        // exponential underflows, or the scores are -inf) for all 32 queries: the maxima
-        // do not move and every term is an exact zero.  (A query with no finite score yet
-        // has m_run = -inf and counts as live.)
-        const bool lane_dead = (__builtin_amdgcn_exp2f((bm - m_run) * c) == 0.0f) && (nan_probe == nan_probe);
-        if (__builtin_amdgcn_ballot_w64(!lane_dead) == 0) continue;
-        const float m_new = __builtin_fmaxf(m_run, bm);
-        // a query whose keys were all -inf so far: subtract 0 instead (its terms come out 0,
-        // not NaN; if the row stays empty the final 0 / 0 is the NaN the unfused kernels give)
-        const float m_use = (m_new == -__builtin_inff()) ? 0.0f : m_new;
-        const float mc = m_use * c;
-        const float alpha = __builtin_amdgcn_exp2f((m_run - m_use) * c);
-        float sum = 0.0f;
-        POLY_TIN p[16];
-#pragma unroll
-        for (int r = 0; r < 16; r++) {
-          const float tt = __builtin_amdgcn_exp2f(__builtin_fmaf(x[r], c, -mc));
-          sum = sum + tt;
-          p[r] = (POLY_TIN)tt;
-        }
-        l_run = l_run * alpha + sum;
-        m_run = m_new;
-        if (__builtin_amdgcn_ballot_w64(alpha != 1.0f) != 0) {
-#pragma unroll
-          for (int dt = 0; dt < 2; dt++)
-#pragma unroll
-            for (int r = 0; r < 16; r++) o[dt][r] = o[dt][r] * alpha;
-        }
-#pragma unroll
-        for (int u = 0; u < 2; u++) {
-          fa_in8 pf;
-#pragma unroll
-          for (int i = 0; i < 8; i++) pf[i] = p[8 * u + i];
-#pragma unroll
-          for (int dt = 0; dt < 2; dt++) o[dt] = POLY_MFMA(v_frag(t, u, dt), pf, o[dt]);
+          const unsigned d = mraw[r >> 2][(r >> 1) & 1];
+          const POLY_TIN mk = __builtin_bit_cast(POLY_TIN, (unsigned short)((r & 1) ? (d >> 16) : (d & 0xffffu)));
+          x[r] = POLY_FA_MAXV(POLY_FA_SCORE_MASK(st[r], mk, mq, n, z), mq, n, z);
         }
       }
+#else
+      fa_acc16 st;
+      scores(cur, t, st);
+#pragma unroll
+      for (int r = 0; r < 16; r++) {
+        const int n = key_of(kb, t, r);
+        x[r] = POLY_FA_MAXV(POLY_FA_SCORE(st[r], mq, n, z), mq, n, z);
+      }
+#endif
+      // largest score of this lane's keys; a NaN among them makes it NaN (v_maximum3_f32)
+      float bm = x[0];
+#pragma unroll
+      for (int r = 1; r < 16; r++) bm = __builtin_elementwise_maximum(bm, x[r]);
+      bm = __builtin_elementwise_maximum(bm, fa_other_half(bm));
+      // Against the running maximum the largest term of this tile is exactly zero (the
+      // exponential underflows, or the scores are -inf) for all 32 queries: the maxima
+      // do not move and every term is an exact zero.  (A query with no finite score yet
+      // has m_run = -inf and counts as live, and so does one with a NaN score: both make
+      // the exponential NaN.)
+      const bool lane_dead = __builtin_amdgcn_exp2f((bm - m_run) * c) == 0.0f;
+      if (__builtin_amdgcn_ballot_w64(!lane_dead) == 0) return;
+      const float m_new = __builtin_fmaxf(m_run, bm);   // ignores a NaN: the terms carry it
+      // a query whose keys were all -inf so far: subtract 0 instead (its terms come out 0,
+      // not NaN; if the row stays empty the final 0 / 0 is the NaN the unfused kernels give)
+      const float m_use = (m_new == -__builtin_inff()) ? 0.0f : m_new;
+      const float mc = m_use * c;
+      const float alpha = __builtin_amdgcn_exp2f((m_run - m_use) * c);
+      float sum = 0.0f;
+      POLY_TIN p[16];
+#pragma unroll
+      for (int r = 0; r < 16; r++) {
+        const float tt = __builtin_amdgcn_exp2f(__builtin_fmaf(x[r], c, -mc));
+        sum = sum + tt;
+        p[r] = (POLY_TIN)tt;
+      }
+      l_run = l_run * alpha + sum;
+      m_run = m_new;
+      if (__builtin_amdgcn_ballot_w64(alpha != 1.0f) != 0) {
+#pragma unroll
+        for (int dt = 0; dt < 2; dt++)
+#pragma unroll
+          for (int r = 0; r < 16; r++) o[dt][r] = o[dt][r] * alpha;
+      }
+#pragma unroll
+      for (int u = 0; u < 2; u++) {
+        fa_in8 pf;
+#pragma unroll
+        for (int i = 0; i < 8; i++) pf[i] = p[8 * u + i];
+#pragma unroll
+        for (int dt = 0; dt < 2; dt++) o[dt] = POLY_MFMA(v_frag(u, dt), pf, o[dt]);
+      }
+    };
+#ifdef POLY_FA_MASK_TABLE
+    // The mask does not depend on z, and a kernel ahead of this one has looked at it once
+    // for all z: POLY_FA_MASK_TABLE points at one word per 32 x 32 tile ([M/32][N/32]:
+    // bit 16 set when all entries of the tile hold one value, that value in the low 16
+    // bits), followed by one word per block of 128 queries x 64 keys ([M/128][N/64]:
+    // non-zero when every entry of the block is -inf).  All of it is read through scalar
+    // loads, and the key blocks that are -inf for the whole workgroup are neither loaded
+    // nor waited for.
+    const unsigned *const tile_words = (const unsigned *)(POLY_FA_MASK_TABLE) + (m0 / 32 + __builtin_amdgcn_readfirstlane(wave)) * (POLY_FA_N / 32);
+    const unsigned *const block_words = (const unsigned *)(POLY_FA_MASK_TABLE) + (POLY_FA_M / 32) * (POLY_FA_N / 32) + mb * FA_NKB;
+#if POLY_FA_N / 32 <= 64
+    // up to 64 tiles along the keys: lane l fetches the word of tile l and of block l once,
+    // and the loop below picks them out of the lanes (no load, no wait per tile)
+    const unsigned my_tile_word = lane < POLY_FA_N / 32 ? tile_words[lane] : 0u;
+    const unsigned my_block_word = lane < FA_NKB ? block_words[lane] : 1u;
+    const unsigned long long live_blocks = __builtin_amdgcn_ballot_w64(my_block_word == 0u);
+    auto tile_word = [&](int ti) { return (unsigned)__builtin_amdgcn_readlane((int)my_tile_word, ti); };
+    auto next_block = [&](int kb) {
+      const unsigned long long rest = kb < 64 ? (live_blocks >> kb) : 0ull;
+      return rest ? kb + __builtin_ctzll(rest) : FA_NKB;
+    };
+#else
+    auto tile_word = [&](int ti) { return tile_words[ti]; };
+    auto next_block = [&](int kb) {
+      while (kb < FA_NKB && block_words[kb] != 0) kb++;
+      return kb;
+    };
+#endif
+    int kb = next_block(0), cur = 0;
+    if (kb < FA_NKB) {
+      load_k(kb, rk);
+      load_v(kb, rv);
+      store_k(0, rk);
+      store_v(0, rv);
+    }
+    __syncthreads();
+    while (kb < FA_NKB) {
+      const int nb = next_block(kb + 1);
+      if (nb < FA_NKB) { load_k(nb, rk); load_v(nb, rv); }
+#pragma unroll
+      for (int t = 0; t < 2; t++) {
+        const unsigned w = tile_word(2 * kb + t);
+        tile(cur, kb, t, (w >> 16) != 0, __builtin_bit_cast(float, w << 16));
+      }
+      if (nb < FA_NKB) { store_k(cur ^ 1, rk); store_v(cur ^ 1, rv); }
+      __syncthreads();
+      kb = nb;
+      cur ^= 1;
+    }
+#else
+    load_k(0, rk);
+    load_v(0, rv);
+    store_k(0, rk);
+    store_v(0, rv);
+    __syncthreads();
+#ifdef POLY_FA_MASK_PTR
+    // Is the mask one value over a 32 x 32 tile?  Any lane can look at any entries for that,
+    // so the tile is read the cheap way: 16 bytes per lane, four lanes along a query's 64
+    // bytes, 16 queries per load (16 cache lines per instruction; in the layout of the
+    // score registers, 8 bytes per lane with 32 queries per load, the same tile takes four
+    // times as many line accesses, and those were what the memory pipeline spent its time
+    // on).  The entries in score layout are fetched only for a tile that is not uniform.
+    const POLY_TIN *const look_row0 = POLY_FA_MASK_PTR(m0 + wave * 32 + (lane >> 2), 8 * (lane & 3), z);
+    const POLY_TIN *const look_row1 = POLY_FA_MASK_PTR(m0 + wave * 32 + 16 + (lane >> 2), 8 * (lane & 3), z);
+    auto load_look = [&](int tl, fa_u32x4 (&lk)[2]) {
+      lk[0] = *(const fa_u32x4_u *)(look_row0 + 32 * tl);
+      lk[1] = *(const fa_u32x4_u *)(look_row1 + 32 * tl);
+    };
+    fa_u32x4 look[2];
+    load_look(0, look);
+#endif
+    for (int kb = 0; kb < FA_NKB; kb++) {
+      const int cur = kb & 1;
+      if (kb + 1 < FA_NKB) { load_k(kb + 1, rk); load_v(kb + 1, rv); }
+#ifdef POLY_FA_MASK_PTR
+#pragma unroll
+      for (int t = 0; t < 2; t++) {
+        // the entries of the tile after this one are requested now, a tile ahead of their use
+        fa_u32x4 look_next[2];
+        load_look((2 * kb + t + 1 < 2 * FA_NKB) ? 2 * kb + t + 1 : 2 * kb + t, look_next);
+        // Do all 32 x 32 entries hold one value?  (compared as bit patterns)
+        const unsigned s0 = (unsigned)__builtin_amdgcn_readfirstlane((int)((look[0][0] & 0xffffu) * 0x10001u));
+        unsigned diff = 0;
+#pragma unroll
+        for (int i = 0; i < 2; i++)
+#pragma unroll
+          for (int j = 0; j < 4; j++) diff |= look[i][j] ^ s0;
+        const bool uniform = __builtin_amdgcn_ballot_w64(diff != 0) == 0;
+        tile(cur, kb, t, uniform, __builtin_bit_cast(float, s0 << 16));
+        look[0] = look_next[0];
+        look[1] = look_next[1];
+      }
+#else
+      tile(cur, kb, 0, false, 0.0f);
+      tile(cur, kb, 1, false, 0.0f);
+#endif
       if (kb + 1 < FA_NKB) { store_k(cur ^ 1, rk); store_v(cur ^ 1, rv); }
       __syncthreads();
     }
+#endif
   }
   // the two lanes of a query each summed half of the keys (a + b == b + a bit for bit)
   const float l_tot = l_run + fa_other_half(l_run);
@@ -503,3 +653,4 @@ extern "C" __global__ void __launch_bounds__(FA_THREADS) __attribute__((amdgpu_w
     }
 #endif
 }
+#endif

@@ -577,9 +577,16 @@ int poly_hip_fused_groups(const PolySchedule *s, int index, char **source_out, i
   if (index >= 0 && index < (int)groups.size()) {
     if (n_items_out) *n_items_out = (int)groups[(size_t)index].items.size();
     if (source_out) {
-      // the main kernel, then the kernels that fill its tables, as separate translation units
+      // the main kernel, then the kernels that fill its tables and those that run ahead of
+      // it, as separate translation units
       std::string src = groups[(size_t)index].rk.source;
       for (const RenderedKernel::Table &t : groups[(size_t)index].rk.tables) src += "\n// ---- table " + t.entry + "\n" + t.source;
+      for (const RenderedKernel::Pre &pk : groups[(size_t)index].rk.pres) {
+        char head[160];
+        snprintf(head, sizeof head, "\n// ---- first stage ---- grid=%u,%u block=%u scratch=%zu\n", pk.launch.grid[0], pk.launch.grid[1],
+                 pk.launch.block[0], groups[(size_t)index].rk.scratch_bytes);
+        src += head + pk.source;
+      }
       const std::vector<RenderedKernel::Variant> &vs = groups[(size_t)index].rk.variants;
       for (size_t i = 1; i < vs.size(); i++) src += "\n// ---- variant " + vs[i].label + "\n" + vs[i].source;
       *source_out = (char *)malloc(src.size() + 1);

@@ -25,6 +25,7 @@ SHIM = r"""
 #include <cstdint>
 struct poly_dim3 { unsigned x, y, z; };
 static poly_dim3 threadIdx, blockIdx, blockDim, gridDim;
+#define POLY_HOST_ADDRESS_CHECK 1
 #define __device__
 #define __global__
 #define __forceinline__ inline
@@ -43,6 +44,7 @@ static poly_dim3 threadIdx, blockIdx, blockDim, gridDim;
 #define __builtin_amdgcn_wave_barrier() ((void)0)
 #define __builtin_amdgcn_sched_barrier(m) ((void)0)
 #define __builtin_amdgcn_exp2f(x) exp2f(x)
+template <class T> static T atomicAdd(T *p, T v) { T old = *p; *p += v; return old; }
 #define __builtin_amdgcn_mfma_f32_32x32x16_bf16(a, b, c, x, y, z) (c)
 #define __builtin_amdgcn_mfma_f32_32x32x16_f16(a, b, c, x, y, z) (c)
 #define __builtin_amdgcn_mfma_f32_32x32x2f32(a, b, c, x, y, z) (c)
@@ -162,7 +164,8 @@ def _jobs(lib, schedule, max_threads, only, groups):
     for gi in range(lib.poly_hip_fused_groups(schedule, -1, None, None)):
         src = C.c_void_p()
         lib.poly_hip_fused_groups(schedule, gi, C.byref(src), None)
-        main = _ffi.take_string(src.value).split("\n// ---- ")[0]
+        text = _ffi.take_string(src.value)
+        main = text.split("\n// ---- ")[0]
         slots = (C.c_int * 64)()
         launch = (C.c_int * 4)()
         n = lib.poly_hip_fused_group_launch(schedule, gi, slots, 64, launch)
@@ -171,7 +174,13 @@ def _jobs(lib, schedule, max_threads, only, groups):
         if (main, sizes) in seen:
             continue
         seen.add((main, sizes))
-        yield f"group {gi}", main, (launch[0], launch[1], launch[2]), launch[3], sizes, 0
+        scratch = 0
+        for unit in text.split("\n// ---- ")[1:]:
+            m = re.match(r"first stage ---- grid=(\d+),(\d+) block=(\d+) scratch=(\d+)\n", unit)
+            if m:
+                scratch = int(m.group(4))
+                yield f"group {gi} (first stage)", unit[m.end():], (int(m.group(1)), int(m.group(2)), 1), int(m.group(3)), sizes, scratch
+        yield f"group {gi}", main, (launch[0], launch[1], launch[2]), launch[3], sizes, scratch
 
 
 def check_schedule(lib, schedule, max_threads=1 << 21, only=None, groups=True, workers=6):

@@ -93,12 +93,15 @@ def test_fused_attention_matches_unfused_and_reference(qk_gain, form):
     c.close()
 
 
-@pytest.mark.parametrize("form", ["online", "exact"])
+@pytest.mark.parametrize("form", ["online", "online, mask looked at by every wave", "exact"])
 def test_attention_with_infinite_mask_entries(form):
     """An additive mask handed in as a buffer, with -inf entries: causal; the first 64 keys
     hidden from the last 128 queries (their first key tiles are fully masked, so the running
     maximum starts at -inf); a band of keys hidden from everybody; one query with no key at
-    all, whose output row is NaN in the reference."""
+    all, whose output row is NaN in the reference.  The single-pass form runs both ways of
+    finding the tiles whose mask entries are all one value: a first kernel that looks at the
+    mask once for all heads (the default for a mask that does not depend on batch or head),
+    and every wave looking at its own tiles (POLY_HIP_NO_MASK_TABLE=1)."""
     ctx, heads, hd, batch = 256, 2, 64, 1
     c = R.Ctx()
     bufs, sink = graphs.attention_bf16(c, batch=batch, heads=heads, ctx=ctx, hd=hd, mask_buffer=True)
@@ -115,16 +118,20 @@ def test_attention_with_infinite_mask_entries(form):
     want = R.bf16_bits_to_f32(run_ref(c, sink, arrays)[bufs["out"]]).reshape(ctx, heads * hd)
     if form == "exact":
         os.environ["POLY_HIP_EXACT_ATTENTION"] = "1"
+    if "every wave" in form:
+        os.environ["POLY_HIP_NO_MASK_TABLE"] = "1"
     try:
         got, info = run_hip(c, sink, arrays)
     finally:
         os.environ.pop("POLY_HIP_EXACT_ATTENTION", None)
+        os.environ.pop("POLY_HIP_NO_MASK_TABLE", None)
     c.close()
-    assert any(k["klass"] == "attention-mfma" and ("one pass" if form == "online" else "two passes") in k["desc"] for k in info), [k["desc"] for k in info]
+    assert any(k["klass"] == "attention-mfma" and ("one pass" if form.startswith("online") else "two passes") in k["desc"] for k in info), [k["desc"] for k in info]
+    assert any("classified by a first kernel" in k["desc"] for k in info) == (form == "online"), [k["desc"] for k in info]
     have = R.bf16_bits_to_f32(got[bufs["out"]]).reshape(ctx, heads * hd)
     assert np.isnan(want[5]).all() and np.isnan(have[5]).all()
     assert np.isfinite(np.delete(want, 5, axis=0)).all() and np.isfinite(np.delete(have, 5, axis=0)).all()
-    assert_close(have, want, rtol=2e-2, atol=8e-3 if form == "online" else 2e-3, what=f"{form} attention with -inf mask entries")
+    assert_close(have, want, rtol=2e-2, atol=8e-3 if form.startswith("online") else 2e-3, what=f"{form} attention with -inf mask entries")
 
 
 @pytest.mark.parametrize("form", ["online", "exact"])

@@ -58,10 +58,17 @@ def bind_by_name(plan, weights, extra):
 
 
 def set_form(monkeypatch, form):
+    """ "online": the single pass, mask tiles classified by a first kernel; "online, every
+    wave looks at the mask": the single pass with POLY_HIP_NO_MASK_TABLE=1; "exact": two
+    passes with the reference's roundings."""
     if form == "exact":
         monkeypatch.setenv("POLY_HIP_EXACT_ATTENTION", "1")
     else:
         monkeypatch.delenv("POLY_HIP_EXACT_ATTENTION", raising=False)
+    if "every wave" in form:
+        monkeypatch.setenv("POLY_HIP_NO_MASK_TABLE", "1")
+    else:
+        monkeypatch.delenv("POLY_HIP_NO_MASK_TABLE", raising=False)
     return "two passes" if form == "exact" else "one pass"
 
 
@@ -160,7 +167,7 @@ def test_logits_t1024_benchmark_plan_matches_reference(monkeypatch, named, weigh
     _check_logits(rows, cols, f"B=8 plan, {form} attention")
 
 
-@pytest.mark.parametrize("form", ["online", "exact"])
+@pytest.mark.parametrize("form", ["online", "online, every wave looks at the mask", "exact"])
 def test_attention_b8_h12_t1024_plan_on_the_fixture_heads(monkeypatch, form):
     """The stand-alone attention plan at the benchmark's shape (8 sequences, 12 heads): the
     two heads of the T=1024 fixture sit at (sequence 3, heads 4 and 5) and (sequence 7,
@@ -190,9 +197,10 @@ def test_attention_b8_h12_t1024_plan_on_the_fixture_heads(monkeypatch, form):
     plan.close()
     attn = [k["desc"] for k in info if k["klass"] == "attention-mfma"]
     assert len(attn) == 1 and marker in attn[0], attn
+    assert ("classified by a first kernel" in attn[0]) == (form == "online"), attn
     got = gpt2_data.bf16_bits_to_f32(from_device(out, np.uint16)).reshape(8, T, H, 64)
     want = gpt2_data.bf16_bits_to_f32(fx.expected[by["out"]]).reshape(T, 2, 64)
     scale = float(np.abs(want).max())
     for b, h in spots:
-        assert_close(got[b, :, h:h + 2, :], want, rtol=2e-2, atol=(2.5e-3 if form == "online" else 6.5e-4) * scale,
+        assert_close(got[b, :, h:h + 2, :], want, rtol=2e-2, atol=(2.5e-3 if form.startswith("online") else 6.5e-4) * scale,
                      what=f"attention B=8 H=12 T=1024, sequence {b} heads {h},{h + 1}, {form}")
