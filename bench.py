@@ -29,15 +29,18 @@ GPT2_PLAN = "gpt2_small_bf16_b8_t1024"
 
 # HBM bytes per launch measured with `rocprofv3 --pmc FETCH_SIZE` and `--pmc WRITE_SIZE`
 # (two runs of this script, counters scaled by what a plain copy of known size reads:
-# FETCH_SIZE x 2.0 KiB, WRITE_SIZE x 1.0 KiB); keyed by the start of the kernel description.
-# The summaries with the commands are under profiles/.
+# FETCH_SIZE x 2.0 KiB, WRITE_SIZE x 1.0 KiB).  A counter run cannot be made from inside
+# this script, so the figures are a table; each key is the start of a kernel description
+# INCLUDING its tile shape or form, so that a kernel built differently from the one that
+# was measured finds no entry and reports null.  The summaries with the commands are
+# under profiles/ (…hbm_traffic_pmc.md).
 MEASURED_TRAFFIC = {
-    "attention-mfma: fused attention (9 kernels): mfma 32x32x16 bf16 Z=96 M=1024 N=1024 D=64, one pass": 56.4e6 + 15.0e6,
-    "attention-mfma: fused attention (9 kernels): mfma 32x32x16 bf16 Z=96 M=1024 N=1024 D=64, two passes": 73.9e6 + 12.6e6,
-    "matmul-mfma: mfma 32x32x16 bf16 M=8192 N=3072 K=768 Z=1": 74.0e6 + 51.1e6,
-    "matmul-mfma: mfma 32x32x16 bf16 M=8192 N=2304 K=768 Z=1": 64.1e6 + 37.8e6,
-    "matmul-mfma: mfma 32x32x16 bf16 M=8192 N=768 K=3072 Z=1": 101.0e6 + 15.8e6,
-    "matmul-mfma: mfma 32x32x16 bf16 M=8192 N=50257 K=768 Z=1": 988e6 + 948e6,
+    "attention-mfma: fused attention (9 kernels): mfma 32x32x16 bf16 Z=96 M=1024 N=1024 D=64, one pass, online softmax, mask tiles classified by a first kernel": 39.1e6 + 12.6e6 + 2.1e6,
+    "matmul-mfma: mfma 32x32x16 bf16 M=8192 N=3072 K=768 Z=1 tile 128x256x64 A:k-major B:n-major": 74.0e6 + 51.1e6,
+    "matmul-mfma: mfma 32x32x16 bf16 M=8192 N=2304 K=768 Z=1 tile 128x256x64 A:k-major B:n-major": 63.8e6 + 37.8e6,
+    "matmul-mfma: mfma 32x32x16 bf16 M=8192 N=768 K=3072 Z=1 tile 128x256x64 A:k-major B:n-major": 101.0e6 + 15.8e6,
+    "matmul-mfma: mfma 32x32x16 bf16 M=8192 N=768 K=768 Z=1 tile 128x256x64 A:k-major B:n-major": 35.0e6 + 15.5e6,
+    "matmul-mfma: mfma 32x32x16 bf16 M=8192 N=50257 K=768 Z=1 tile 256x256x64 A:k-major B:k-major": 987.5e6 + 952.0e6,
 }
 
 

@@ -206,7 +206,7 @@ int runner_launch(HipRunner *r, void **args, int n_args, void *scratch_from_call
     }
     r->ptr_store[(size_t)(np + nv + nt)] = scratch;
     r->arg_ptrs[(size_t)(np + nv + nt)] = &r->ptr_store[(size_t)(np + nv + nt)];
-    for (size_t i = 0; i < r->pres.size(); i++)
+    for (size_t i = 0; i < r->pres.size() && !r->skip_pres; i++)
       if (program_launch(r->pres[i], r->arg_ptrs.data(), r->rk.pres[i].launch) != 0) return -1;
     return program_launch(r->main, r->arg_ptrs.data(), r->rk.launch);
   }

@@ -1544,6 +1544,7 @@ static bool match_attention(const Sched &sc, int s_item, const std::vector<char>
   }
   cfg += strf("#define POLY_FA_SCORE(acc, m, n, z) %s\n", score.c_str());
   bool mask_table = false;   // a kernel ahead of this one looks at the mask once for all z
+  int mask_arg = -1;         // which argument of the fused kernel the mask is
   // An additive mask: the stored score is cast(f(acc) + mask[...]) with f made of casts
   // and products with positive constants, and the mask a bf16 buffer read at consecutive
   // positions for consecutive keys.  The kernel then loads the mask entries of a tile
@@ -1571,6 +1572,7 @@ static bool match_attention(const Sched &sc, int s_item, const std::vector<char>
         if (it == a.c.end() || it->second != 1) continue;
         mask_ld = cand;
         other = g.n(top).src[(size_t)(1 - side)];
+        mask_arg = arg_of(sc.slot(lm.item, g.param_slot(ix.src[0])));
         mask_z_free = true;
         for (const auto &d : mS.zd) {
           auto zc = a.c.find(d.ord);
@@ -1699,6 +1701,9 @@ static bool match_attention(const Sched &sc, int s_item, const std::vector<char>
     pre.launch.block[0] = 512;
     rk.pres.push_back(pre);
     rk.scratch_bytes = (size_t)((mS.M / 32) * (mS.N / 32) + (mS.M / 128) * (mS.N / 64)) * sizeof(unsigned);
+    // the words depend on the mask buffer alone
+    rk.pres_key = pre.source;
+    rk.pre_reads.assign(1, mask_arg);
   }
   rk.source = std::string(hip_prelude()) + cfg + kAttentionTemplate;
   rk.entry = "poly_k";

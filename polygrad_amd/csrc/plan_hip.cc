@@ -58,6 +58,7 @@ struct Unit {
   std::vector<const PolyUOp *> var_uops;   // which variable each of them is
   int n_items = 1;               // schedule items this launch stands for
   bool repeatable = false;       // writes no buffer it also reads: running it twice changes nothing
+  std::vector<int> writes;       // slots the launch writes
 };
 
 struct PolyHipPlan {
@@ -262,7 +263,10 @@ PolyHipPlan *poly_hip_compile_schedule(PolyCtx *ctx, const PolySchedule *s) {
         }
       }
       u.repeatable = true;
-      for (int sl = 0; sl < s->n_buf_slots; sl++) if (wr[(size_t)sl] && rd[(size_t)sl]) u.repeatable = false;
+      for (int sl = 0; sl < s->n_buf_slots; sl++) {
+        if (wr[(size_t)sl] && rd[(size_t)sl]) u.repeatable = false;
+        if (wr[(size_t)sl]) u.writes.push_back(sl);
+      }
     }
     plan->units.push_back(u);
   }
@@ -333,15 +337,50 @@ PolyHipPlan *poly_hip_compile_schedule(PolyCtx *ctx, const PolySchedule *s) {
     plan->fill = program_create(kFillSrc, "poly_fill0");
     if (!plan->fill) return nullptr;
   }
-  // one scratch pool for all two-stage kernels: the largest need
+  // First stages whose result depends only on buffers that nothing writes in between run
+  // once: the first launch of such a family keeps its scratch memory to itself, the later
+  // ones read it and skip their first stages.
+  std::vector<char> keeps_scratch((size_t)n_units, 0);
+  if (!getenv("POLY_HIP_NO_SHARED_FIRST_STAGE")) {
+    std::map<std::pair<std::string, std::vector<int>>, int> leader_of;
+    for (int ui = 0; ui < n_units; ui++) {
+      HipRunner *r = plan->units[(size_t)ui].runner;
+      if (r->rk.pres_key.empty() || r->pres.empty()) continue;
+      std::vector<int> read_slots;
+      bool known = true;
+      for (int a : r->rk.pre_reads) {
+        if (a < 0 || a >= (int)plan->units[(size_t)ui].slots.size()) { known = false; break; }
+        read_slots.push_back(plan->units[(size_t)ui].slots[(size_t)a]);
+      }
+      if (!known) continue;
+      const auto key = std::make_pair(r->rk.pres_key, read_slots);
+      auto it = leader_of.find(key);
+      bool reuse = it != leader_of.end();
+      for (int w = reuse ? it->second : ui; reuse && w < ui; w++)
+        for (int sl : plan->units[(size_t)w].writes)
+          if (std::find(read_slots.begin(), read_slots.end(), sl) != read_slots.end()) reuse = false;
+      if (!reuse) { leader_of[key] = ui; continue; }
+      HipRunner *lead = plan->units[(size_t)it->second].runner;
+      if (runner_ensure_scratch(lead) != 0) return nullptr;
+      runner_share_scratch(r, lead->scratch);
+      r->skip_pres = true;
+      keeps_scratch[(size_t)it->second] = keeps_scratch[(size_t)ui] = 1;
+      if (getenv("POLY_HIP_DEBUG"))
+        fprintf(stderr, "polygrad: compile_schedule: launch %d reads what the first stage of launch %d leaves\n", ui, it->second);
+    }
+  }
+  // one scratch pool for all other two-stage kernels: the largest need
   {
     int users = 0;
-    for (const Unit &u : plan->units)
-      if (u.runner->rk.scratch_bytes > 0) { users++; plan->scratch_bytes = std::max(plan->scratch_bytes, u.runner->rk.scratch_bytes); }
+    for (int ui = 0; ui < n_units; ui++) {
+      const Unit &u = plan->units[(size_t)ui];
+      if (u.runner->rk.scratch_bytes > 0 && !keeps_scratch[(size_t)ui]) { users++; plan->scratch_bytes = std::max(plan->scratch_bytes, u.runner->rk.scratch_bytes); }
+    }
     if (users > 1) {
       plan->scratch_pool = runtime_alloc(plan->scratch_bytes);
       if (!plan->scratch_pool) return nullptr;
-      for (Unit &u : plan->units) runner_share_scratch(u.runner, plan->scratch_pool);
+      for (int ui = 0; ui < n_units; ui++)
+        if (!keeps_scratch[(size_t)ui]) runner_share_scratch(plan->units[(size_t)ui].runner, plan->scratch_pool);
     }
     // a lone user owns its scratch memory; it must exist before the launches are captured
     for (Unit &u : plan->units) if (runner_ensure_scratch(u.runner) != 0) return nullptr;

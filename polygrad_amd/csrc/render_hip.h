@@ -79,6 +79,14 @@ struct RenderedKernel {
   };
   std::vector<Pre> pres;
   size_t scratch_bytes = 0;
+  // Set when what the first stages leave in the scratch memory depends on nothing but the
+  // contents of the buffers bound to the arguments `pre_reads` (indices into the kernel's
+  // buffer parameters) and the main kernel only reads it: `pres_key` then identifies the
+  // computation (the text of the first stages before they get their symbol names), and a
+  // plan runs it once for all launches that share key and buffers, as long as nothing
+  // writes those buffers in between.
+  std::string pres_key;
+  std::vector<int> pre_reads;
 };
 
 struct Scope;

@@ -42,6 +42,7 @@ struct HipRunner {
   std::vector<Program *> pres;     // first stage(s) of a two-stage kernel
   void *scratch = nullptr;         // what they leave for the main kernel
   bool owns_scratch = true;        // false: the memory belongs to a pool shared with other runners
+  bool skip_pres = false;          // the scratch memory already holds what the first stages would write
   void *flag = nullptr;            // device int written by the guards
   std::vector<std::shared_ptr<void>> tables;   // filled lookup tables (shared between identical kernels)
   std::string name;
