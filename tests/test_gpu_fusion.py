@@ -160,6 +160,29 @@ def test_attention_fp16(form):
     assert_close(got[bufs["out"]].astype(np.float32), want, rtol=2e-2, atol=2e-3, what=f"{form} attention in fp16")
 
 
+@pytest.mark.parametrize("mask_value", ["-inf", "-1e9"])
+def test_attention_with_more_than_64_key_tiles(mask_value):
+    """2176 keys are 68 tiles of 32: a wave keeps the words of up to 64 mask tiles in its
+    lanes and reads them one by one beyond that.  One head, causal; with -inf above the
+    diagonal (tiles and key blocks passed over unseen) and with the reference's -1e9."""
+    ctx, heads, hd, batch = 2176, 1, 64, 1
+    c = R.Ctx()
+    bufs, sink = graphs.attention_bf16(c, batch=batch, heads=heads, ctx=ctx, hd=hd, mask_buffer=True)
+    g = np.random.default_rng(17)
+    fill = np.float32(-np.inf) if mask_value == "-inf" else np.float32(-1e9)
+    mask = np.where(np.arange(ctx)[:, None] < np.arange(ctx)[None, :], fill, np.float32(0.0)).astype(np.float32)
+    arrays = {bufs["mask"]: R.f32_to_bf16_bits(mask), bufs["out"]: np.zeros(batch * ctx * heads * hd, np.uint16)}
+    for n in ("q", "k", "v"):
+        arrays[bufs[n]] = R.f32_to_bf16_bits(g.uniform(-1, 1, batch * ctx * heads * hd).astype(np.float32) * (2.0 if n != "v" else 1.0))
+    want = R.bf16_bits_to_f32(run_ref(c, sink, arrays)[bufs["out"]]).reshape(ctx, heads * hd)
+    got, info = run_hip(c, sink, arrays)
+    c.close()
+    assert any(k["klass"] == "attention-mfma" and "classified by a first kernel" in k["desc"] for k in info), [k["desc"] for k in info]
+    have = R.bf16_bits_to_f32(got[bufs["out"]]).reshape(ctx, heads * hd)
+    assert np.isfinite(want).all() and np.isfinite(have).all()
+    assert_close(have, want, rtol=2e-2, atol=8e-3, what=f"attention over 2176 keys, mask {mask_value}")
+
+
 def test_lookup_table_epilogue_is_bit_identical_to_the_arithmetic():
     """A pointwise kernel of one 16-bit input fused behind a matmul is evaluated through a
     65536-entry table filled by its own expression: results must not change by a bit."""
