@@ -1624,10 +1624,45 @@ static bool match_attention(const Sched &sc, int s_item, const std::vector<char>
       const char *lead = n_chain ? "%s x, %s mk" : "float acc, %s mk";
       std::map<int, std::string> pre_mask{{mask_ld, "mk"}};
       if (!n_chain) pre_mask[mS.red] = "acc";
-      value_fn(lm, "poly_fa_score_mask", tn, n_chain ? strf(lead, tn, tn).c_str() : strf(lead, tn).c_str(), n_chain ? g.stores[0].value : stS.value, pre_mask);
-      cfg += strf("#define POLY_FA_SCORE_MASK(acc, mk, m, n, z) poly_fa_score_mask(%s, mk, m, n, z, %s)\n", head.c_str(), call_args(lm.item).c_str());
+      // f(acc) = cast(acc) * 2^k with nothing else in it: the kernel multiplies Q by 2^k
+      // once when it stages it instead (products and sums of a dot product scale exactly
+      // with a power of two, and so does every rounding on the way, as long as nothing
+      // becomes subnormal), and the chain is emitted with that constant as 1.
+      int scale_const = -1;
+      double qscale = 1.0;
+      if (!getenv("POLY_HIP_NO_QSCALE")) {
+        int muls = 0, v = other;
+        while (true) {
+          const KNode &k = g.n(v);
+          if (k.op == POLY_OP_CAST) { v = k.src[0]; continue; }
+          if (k.op != POLY_OP_MUL) break;
+          int side = -1;
+          for (int sd = 0; sd < 2; sd++) {
+            const KNode &cn = g.n(k.src[(size_t)sd]);
+            if (cn.op == POLY_OP_CONST && cn.u->arg.kind == POLY_ARG_FLOAT && cn.u->arg.f > 0) side = sd;
+          }
+          if (side < 0) break;
+          muls++;
+          scale_const = k.src[(size_t)side];
+          qscale = g.n(scale_const).u->arg.f;
+          v = k.src[(size_t)(1 - side)];
+        }
+        int e2 = 0;
+        const bool pow2 = muls == 1 && std::frexp(qscale, &e2) == 0.5 && e2 > -100 && e2 < 100;
+        int uses = 0;
+        if (pow2)
+          for (const KNode &k : g.nodes) for (int sN : k.src) if (sN == scale_const) uses++;
+        if (!pow2 || uses != 1) scale_const = -1;
+      }
       std::map<int, std::string> pre_acc;
       if (!n_chain) pre_acc[mS.red] = "acc";
+      if (scale_const >= 0) {
+        pre_mask[scale_const] = "1.0f";
+        pre_acc[scale_const] = "1.0f";
+        cfg += strf("#define POLY_FA_QSCALE %s\n", Emitter::float_literal(qscale, DT_F32).c_str());
+      }
+      value_fn(lm, "poly_fa_score_mask", tn, n_chain ? strf(lead, tn, tn).c_str() : strf(lead, tn).c_str(), n_chain ? g.stores[0].value : stS.value, pre_mask);
+      cfg += strf("#define POLY_FA_SCORE_MASK(acc, mk, m, n, z) poly_fa_score_mask(%s, mk, m, n, z, %s)\n", head.c_str(), call_args(lm.item).c_str());
       value_fn(lm, "poly_fa_score_nomask", "float", n_chain ? strf("%s x", tn).c_str() : "float acc", other, pre_acc);
       cfg += strf("#define POLY_FA_SCORE_NOMASK(acc, m, n, z) poly_fa_score_nomask(%s, m, n, z, %s)\n", head.c_str(), call_args(lm.item).c_str());
       if (failed && !failed_before) { failed = false; cfg.resize(before); }

@@ -48,6 +48,9 @@
 //   POLY_FA_ONLINE                     1: single pass (needs p = cast(term / sum),
 //                                      term(x, mx) = exp2((x - mx) * POLY_FA_C) and the
 //                                      maximum taken over the scores themselves)
+//   POLY_FA_QSCALE                     (optional, with POLY_FA_MASK_PTR) a power of two that
+//                                      the kernel multiplies Q by when it stages it; the
+//                                      score hooks are then generated without it
 //   POLY_FA_MASK_TABLE                 (optional, with POLY_FA_MASK_PTR, when the mask does
 //                                      not depend on z) pointer to the words that the
 //                                      classifying kernel below writes: the mask is then
@@ -110,8 +113,9 @@ __device__ __forceinline__ int poly_v_off(int z, int n) { return (z / 12) * 7864
 #define POLY_FA_ONLINE 1
 #define POLY_FA_C 0x1.715476p+0f
 #define POLY_FA_MASK_PTR(m, n, z) (data4 + (m) * 1024 + (n))
-#define POLY_FA_SCORE_MASK(acc, mk, m, n, z) ((__bf16)((float)(__bf16)(acc) * 0.125f + (float)(mk)))
-#define POLY_FA_SCORE_NOMASK(acc, m, n, z) ((float)(__bf16)(acc) * 0.125f)
+#define POLY_FA_QSCALE 0.125f
+#define POLY_FA_SCORE_MASK(acc, mk, m, n, z) ((__bf16)((float)(__bf16)(acc) + (float)(mk)))
+#define POLY_FA_SCORE_NOMASK(acc, m, n, z) ((float)(__bf16)(acc))
 #endif
 #ifndef POLY_FA_ONLINE
 #define POLY_FA_ONLINE 0
@@ -129,6 +133,9 @@ typedef fa_u32x2 fa_u32x2_u __attribute__((aligned(2)));
 #define FA_D 64          // head features
 #define FA_THREADS 256
 #define FA_NKB (POLY_FA_N / FA_BN)
+#ifndef FA_LAG
+#define FA_LAG 8.0f      // online form: how many powers of two a score may exceed the reference before it moves
+#endif
 
 // LDS tiles are [row][64] 16-bit values; the eight 16-byte columns of a row are
 // XOR-swizzled by the row number so fragment reads and staging writes spread over banks.
@@ -210,7 +217,16 @@ extern "C" __global__ void __launch_bounds__(FA_THREADS) __attribute__((amdgpu_w
   for (int i = 0; i < 4; i++) {
     const int c = threadIdx.x + i * FA_THREADS;
     const int q = c >> 3, col = c & 7;
-    const fa_u32x4 v = *(const fa_u32x4_u *)(POLY_Q_PTR + poly_q_off(z, m0 + q) + col * 8);
+    fa_u32x4 v = *(const fa_u32x4_u *)(POLY_Q_PTR + poly_q_off(z, m0 + q) + col * 8);
+#ifdef POLY_FA_QSCALE
+    // the power of two that the score chain would multiply every cast(acc) by, applied to Q
+    {
+      fa_in8 qv = __builtin_bit_cast(fa_in8, v);
+#pragma unroll
+      for (int e = 0; e < 8; e++) qv[e] = (POLY_TIN)((float)qv[e] * POLY_FA_QSCALE);
+      v = __builtin_bit_cast(fa_u32x4, qv);
+    }
+#endif
     *(fa_u32x4 *)(lds_q + q * FA_D + ((col ^ fa_swz(q)) * 8)) = v;
   }
   const POLY_TIN *q_row = lds_q + (wave * 32 + lq) * FA_D;
@@ -372,14 +388,34 @@ extern "C" __global__ void __launch_bounds__(FA_THREADS) __attribute__((amdgpu_w
       // do not move and every term is an exact zero.  (A query with no finite score yet
       // has m_run = -inf and counts as live, and so does one with a NaN score: both make
       // the exponential NaN.)
-      const bool lane_dead = __builtin_amdgcn_exp2f((bm - m_run) * c) == 0.0f;
+      const float dist = (bm - m_run) * c;   // how far above the reference the tile reaches, in powers of two
+      const bool lane_dead = __builtin_amdgcn_exp2f(dist) == 0.0f;
       if (__builtin_amdgcn_ballot_w64(!lane_dead) == 0) return;
-      const float m_new = __builtin_fmaxf(m_run, bm);   // ignores a NaN: the terms carry it
-      // a query whose keys were all -inf so far: subtract 0 instead (its terms come out 0,
-      // not NaN; if the row stays empty the final 0 / 0 is the NaN the unfused kernels give)
-      const float m_use = (m_new == -__builtin_inff()) ? 0.0f : m_new;
-      const float mc = m_use * c;
-      const float alpha = __builtin_amdgcn_exp2f((m_run - m_use) * c);
+      // m_run is the reference the terms are taken against.  It follows the largest score
+      // lazily: only when some query's tile maximum lies more than 2^FA_LAG above it (or it
+      // is still -inf, or a NaN is involved) do all queries of the wave move theirs, with
+      // the usual rescaling of sum and accumulators; otherwise terms simply come out as
+      // large as 2^FA_LAG, which fp32 sums and a 16-bit float hold as well as values below
+      // one, and the final division takes out whatever reference was used.  After the
+      // first tiles of a row this is rare, and the rescaling was a sixth of the tile's
+      // vector instructions.
+      const bool move = !(dist <= FA_LAG);
+      if (__builtin_amdgcn_ballot_w64(move) != 0) {
+        const float m_new = __builtin_fmaxf(m_run, bm);   // ignores a NaN: the terms carry it
+        // a query whose keys were all -inf so far: subtract 0 instead (its terms come out 0,
+        // not NaN; if the row stays empty the final 0 / 0 is the NaN the unfused kernels give)
+        const float m_to = (m_new == -__builtin_inff()) ? 0.0f : m_new;
+        const float alpha = __builtin_amdgcn_exp2f((m_run - m_to) * c);
+        l_run = l_run * alpha;
+        m_run = m_new;
+        if (__builtin_amdgcn_ballot_w64(alpha != 1.0f) != 0) {
+#pragma unroll
+          for (int dt = 0; dt < 2; dt++)
+#pragma unroll
+            for (int r = 0; r < 16; r++) o[dt][r] = o[dt][r] * alpha;
+        }
+      }
+      const float mc = ((m_run == -__builtin_inff()) ? 0.0f : m_run) * c;
       float sum = 0.0f;
       POLY_TIN p[16];
 #pragma unroll
@@ -388,14 +424,7 @@ extern "C" __global__ void __launch_bounds__(FA_THREADS) __attribute__((amdgpu_w
         sum = sum + tt;
         p[r] = (POLY_TIN)tt;
       }
-      l_run = l_run * alpha + sum;
-      m_run = m_new;
-      if (__builtin_amdgcn_ballot_w64(alpha != 1.0f) != 0) {
-#pragma unroll
-        for (int dt = 0; dt < 2; dt++)
-#pragma unroll
-          for (int r = 0; r < 16; r++) o[dt][r] = o[dt][r] * alpha;
-      }
+      l_run = l_run + sum;
 #pragma unroll
       for (int u = 0; u < 2; u++) {
         fa_in8 pf;
