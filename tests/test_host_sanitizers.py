@@ -47,5 +47,9 @@ def test_benchmark_schedules(driver):
     files = sorted(glob.glob(os.path.join(HERE, "..", "polygrad_amd", "plans", "*.polyplan")))
     files += sorted(glob.glob(os.path.join(HERE, "golden", "fullsize", "*.polyplan")))
     files = [f for f in files if "b1_t1024" not in os.path.basename(f) or "block0" in f]   # the B=1 twin of the B=8 plan adds a minute and nothing new
+    if not os.environ.get("POLY_SLOW_TESTS"):
+        # the 24-layer training step is the one-block step 24 times over (2770 kernels, five
+        # minutes under the sanitizers); the one-block plan goes through the same code
+        files = [f for f in files if "train_24l" not in os.path.basename(f)]
     out = run(driver, files, 900)
     assert "0 problems" in out
