@@ -19,6 +19,7 @@
 #include <algorithm>
 #include <cmath>
 #include <cstdlib>
+#include <cstring>
 #include <map>
 #include <set>
 
@@ -288,7 +289,7 @@ static bool only_depends_on_presets(const KernelGraph &g, const Member &m, int n
 // possible results: a table filled once by the kernel's own expression replaces the
 // arithmetic (bit-identical by construction, and a gather instead of dozens of VALU
 // instructions per element when the expression rounds to 16 bits after every step).
-static bool make_unary_table(const Sched &sc, const Member &m, RenderedKernel::Table *t, std::string *out_type) {
+static bool make_unary_table(const Sched &sc, const Member &m, RenderedKernel::Table *t, std::string *out_type, bool *bf16_in) {
   const KernelGraph &g = sc.graphs[(size_t)m.item];
   const StoreInfo &st = g.stores[0];
   if (m.preset.size() != 1) return false;
@@ -315,7 +316,55 @@ static bool make_unary_table(const Sched &sc, const Member &m, RenderedKernel::T
   t->launch.grid[0] = 256;
   t->launch.block[0] = 256;
   *out_type = dt_cname(odt);
+  *bf16_in = in.dt == DT_BF16;
   return true;
+}
+
+// Most values that reach such a table are of moderate size, and a gather from memory costs
+// the address path a cycle for every cache line a wave instruction touches.  The matmul
+// template therefore keeps the entries of 2^-24 <= |x| < 256 (bf16 inputs: 32 binades of 128
+// entries per sign) in LDS when it has the room (it says how much in POLY_EP_WIN_ROOM).
+// A lookup then comes in two modes: from the window alone, recording in *tmax how far
+// outside the window the inputs went (mode 1), or from the table in memory (mode 0); the
+// template computes a group of values in mode 1 and, if any input was outside, again in
+// mode 0.
+static const char *const kNoWindow = "0, (unsigned int*)0";
+static const char *const kWindow = "1, &poly_tmax";
+static std::string table_window_helpers(const std::vector<RenderedKernel::Table> &tables, const std::vector<std::string> &types) {
+  size_t bytes = 0;
+  std::string fill;
+  for (size_t i = 0; i < tables.size(); i++) {
+    fill += strf(" poly_win_fill<%s>(poly_win_raw + %zu, poly_lut%zu, tid, nthreads);", types[i].c_str(), bytes, i);
+    bytes += tables[i].bytes / 8;
+  }
+  // (the window is read through a pointer that names the LDS address space: with a plain
+  // pointer the compiler picks between window and table by address and issues one flat load)
+  return strf("#define POLY_LDS __attribute__((address_space(3)))\n"
+              "#if defined(POLY_EP_WIN_ROOM) && POLY_EP_WIN_ROOM >= %zu\n#define POLY_EP_WIN_BYTES %zu\n"
+              "#define POLY_EP_WIN(off, T) ((POLY_LDS const T*)(poly_win_raw + (off)))\n"
+              "#define POLY_EP_WIN_FILL(tid, nthreads) do {%s } while (0)\n"
+              "#else\n#define POLY_EP_WIN(off, T) ((POLY_LDS const T*)0)\n#endif\n", bytes, bytes, fill.c_str()) +
+         "#define POLY_WIN_FIRST (103u << 7)   /* code of 2^-24 */\n"
+         "#define POLY_WIN_CODES 4096u         /* per sign */\n"
+         "typedef unsigned int poly_win_u32x4 __attribute__((ext_vector_type(4)));\n"
+         "template <typename T> __device__ __forceinline__ void poly_win_fill(unsigned char* win, const T* __restrict__ lut, int tid, int nthreads) {\n"
+         "  constexpr int HALF = (int)POLY_WIN_CODES * (int)sizeof(T);   // bytes per sign\n"
+         "  for (int b = tid * 16; b < 2 * HALF; b += nthreads * 16) {\n"
+         "    const int first = ((b / HALF) * 0x8000 + (int)POLY_WIN_FIRST) * (int)sizeof(T);\n"
+         "    *(poly_win_u32x4*)(win + b) = *(const poly_win_u32x4*)((const unsigned char*)lut + first + b % HALF);\n"
+         "  }\n}\n"
+         "template <typename T, typename X> __device__ __forceinline__ T poly_lut_get(const T* __restrict__ lut, POLY_LDS const T* win, const int mode, unsigned int* tmax, X x) {\n"
+         "  const unsigned int u = __builtin_bit_cast(unsigned short, x);\n"
+         "#ifdef POLY_EP_WIN_BYTES\n"
+         "  if (mode) {\n"
+         "    const unsigned int t = (u & 0x7fffu) - POLY_WIN_FIRST;\n"
+         "    *tmax = t > *tmax ? t : *tmax;\n"
+         "    return win[(t & (POLY_WIN_CODES - 1u)) | ((u >> 3) & POLY_WIN_CODES)];\n"
+         "  }\n"
+         "#endif\n"
+         "  (void)win; (void)mode; (void)tmax;\n"
+         "  return lut[u];\n"
+         "}\n";
 }
 
 // A matmul whose result only feeds a chain of pointwise kernels (bias/activation/residual
@@ -389,7 +438,10 @@ static bool match_matmul_tail(const Sched &sc, int s_item, const std::vector<cha
   DT prev_dt = gS.n(stS.value).dt;
   std::vector<RenderedKernel::Table> tables;
   std::map<size_t, int> table_of;     // member -> table index
-  std::map<size_t, std::string> lead_of, lut_arg_of;
+  std::map<size_t, std::string> lead_of, lut_arg_of, lookup_of;
+  std::vector<std::string> table_types;
+  size_t win_bytes = 0;               // LDS windows of the tables so far
+  bool windowed = false;              // some table takes bf16 codes: its lookups know the window
   for (size_t e = 1; e < members.size(); e++) {
     const Member &m = members[e];
     const KernelGraph &g = sc.graphs[(size_t)m.item];
@@ -399,13 +451,18 @@ static bool match_matmul_tail(const Sched &sc, int s_item, const std::vector<cha
     std::map<int, std::string> extra;
     RenderedKernel::Table tab;
     std::string tab_type;
-    if (!getenv("POLY_HIP_NO_LUT") && make_unary_table(sc, m, &tab, &tab_type)) {
+    bool bf16_in = false;
+    if (!getenv("POLY_HIP_NO_LUT") && make_unary_table(sc, m, &tab, &tab_type, &bf16_in)) {
       table_of[e] = (int)tables.size();
-      lead += strf(", const %s* __restrict__ poly_lut", tab_type.c_str());
-      lut_arg_of[e] = strf(", poly_lut%zu", tables.size());
-      extra[g.stores[0].value] = "poly_lut[__builtin_bit_cast(unsigned short, x)]";
+      lead += strf(", const %s* __restrict__ poly_lut, POLY_LDS const %s* poly_win, const int poly_mode, unsigned int* poly_tmax", tab_type.c_str(), tab_type.c_str());
+      lut_arg_of[e] = strf(", poly_lut%zu, POLY_EP_WIN(%zu, %s), %s", tables.size(), win_bytes, tab_type.c_str(), kNoWindow);
+      lookup_of[e] = bf16_in ? "poly_lut_get(poly_lut, poly_win, poly_mode, poly_tmax, x)" : "poly_lut[__builtin_bit_cast(unsigned short, x)]";
+      if (bf16_in) windowed = true;
+      extra[g.stores[0].value] = lookup_of[e];
       ep.signature += strf(", const %s* __restrict__ poly_lut%zu", tab_type.c_str(), tables.size());
+      win_bytes += tab.bytes / 8;
       tables.push_back(tab);
+      table_types.push_back(tab_type);
     }
     lead_of[e] = lead;
     if (!emit_member_fn(sc, m, master_decomp, fn.c_str(), dt_cname(g.n(g.stores[0].value).dt), lead, g.stores[0].value, extra, false, last,
@@ -414,6 +471,7 @@ static bool match_matmul_tail(const Sched &sc, int s_item, const std::vector<cha
     prev_dt = g.n(g.stores[0].value).dt;
   }
   ep.call = call;
+  if (!tables.empty()) ep.code = table_window_helpers(tables, table_types) + ep.code;
   {
     // value and address of the last kernel's store, separately, when rows are contiguous
     const Member &m = members.back();
@@ -438,7 +496,7 @@ static bool match_matmul_tail(const Sched &sc, int s_item, const std::vector<cha
       (void)before;
       const size_t le = members.size() - 1;
       std::map<int, std::string> extra;
-      if (table_of.count(le)) extra[st.value] = "poly_lut[__builtin_bit_cast(unsigned short, x)]";
+      if (table_of.count(le)) extra[st.value] = lookup_of[le];
       bool ok = emit_member_fn(sc, m, master_decomp, fn.c_str(), dt_cname(g.n(st.value).dt), lead_of[le], st.value, extra, false, false, &code2);
       // address: the store index in master coordinates
       Emitter ea(g);
@@ -458,6 +516,11 @@ static bool match_matmul_tail(const Sched &sc, int s_item, const std::vector<cha
         code2 += master_decomp + flat_decl + Sa.code + strf("  return data%d + %s;\n}\n", g.param_slot(st.param), idx.c_str());
         ep.code += code2;
         ep.value_call = vcall;
+        if (windowed) {
+          ep.value_call_win = vcall;
+          for (size_t at = 0; (at = ep.value_call_win.find(kNoWindow, at)) != std::string::npos; at += strlen(kWindow))
+            ep.value_call_win.replace(at, strlen(kNoWindow), kWindow);
+        }
         ep.ptr_call = strf("poly_ep_ptr(m, n, z, %s)", call_args(m.item).c_str());
         ep.contiguous_n = true;
       }

@@ -22,6 +22,12 @@
 //                       POLY_EP_TYPE, POLY_EP_VALUE(acc, m, n, z) and POLY_EP_PTR(m, n, z)
 //                       give the element type, value and address separately and the
 //                       template writes 8 values of a row with one store
+//   POLY_EP_WIN_BYTES   (optional, set by the epilogue's own code when POLY_EP_WIN_ROOM, the
+//                       LDS left beside the operand tiles, suffices) bytes of LDS that
+//                       POLY_EP_WIN_FILL(tid, nthreads) fills with the middle of the
+//                       epilogue's lookup tables; POLY_EP_VALUE_WIN is then POLY_EP_VALUE
+//                       with lookups from there, raising poly_tmax to POLY_WIN_CODES or
+//                       more when an input lies outside
 //
 // Data path: global --16B loads--> registers --(transpose if needed)--> LDS
 // [row][K] with padded rows, double buffered; each wave reads 16-byte A and B
@@ -181,6 +187,12 @@ struct PolyXC {
 extern "C" __global__ void __launch_bounds__(POLY_NTHREADS) poly_k(POLY_SIGNATURE) {
   // one allocation: the operand tiles during the K loop, the per-wave output staging after it
   __shared__ __attribute__((aligned(16))) POLY_TIN lds_raw[2 * (POLY_BM + POLY_BN) * POLY_LDK];
+#ifdef POLY_EP_WIN_BYTES
+  // the entries of the epilogue's lookup tables that most values hit; the barriers of the K
+  // loop lie between this copy and the epilogue's reads
+  __shared__ __attribute__((aligned(16))) unsigned char poly_win_raw[POLY_EP_WIN_BYTES];
+  POLY_EP_WIN_FILL((int)threadIdx.x, POLY_NTHREADS);
+#endif
   auto lds_a = [&](int buf) { return lds_raw + buf * (POLY_BM * POLY_LDK); };
   auto lds_b = [&](int buf) { return lds_raw + 2 * POLY_BM * POLY_LDK + buf * (POLY_BN * POLY_LDK); };
 
@@ -515,6 +527,17 @@ extern "C" __global__ void __launch_bounds__(POLY_NTHREADS) poly_k(POLY_SIGNATUR
           typedef POLY_EP_TYPE poly_out8 __attribute__((ext_vector_type(8)));
           typedef poly_out8 poly_out8_u __attribute__((aligned(sizeof(POLY_EP_TYPE))));
           poly_out8 o;
+#if defined(POLY_EP_WIN_BYTES) && defined(POLY_EP_VALUE_WIN)
+          // table lookups from the LDS windows first; a lane with an input outside them
+          // computes its group again with lookups in memory
+          unsigned int poly_tmax = 0;
+#pragma unroll
+          for (int e = 0; e < 8; e++) {
+            const int ne = (POLY_N % 8 == 0 || n + e < POLY_N) ? n + e : n;
+            o[e] = POLY_EP_VALUE_WIN(v[e], m, ne, z);
+          }
+          if (poly_tmax >= POLY_WIN_CODES)
+#endif
 #pragma unroll
           for (int e = 0; e < 8; e++) {
             // (keep n + e plain when every group is full: whatever the epilogue loads

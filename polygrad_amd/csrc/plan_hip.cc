@@ -73,6 +73,7 @@ struct PolyHipPlan {
   size_t arena_bytes = 0;
   void *scratch_pool = nullptr;              // shared by the two-stage kernels of the plan (they run one after the other)
   size_t scratch_bytes = 0;
+  size_t kept_scratch_bytes = 0;            // scratch memory of first stages that later launches read
   std::vector<std::vector<void *>> kargs;    // per unit: args array handed to runner_launch
   std::vector<std::vector<int>> var_vals;    // per unit: storage for var ints
   std::vector<PolyVarBinding> merged;
@@ -364,6 +365,7 @@ PolyHipPlan *poly_hip_compile_schedule(PolyCtx *ctx, const PolySchedule *s) {
       if (runner_ensure_scratch(lead) != 0) return nullptr;
       runner_share_scratch(r, lead->scratch);
       r->skip_pres = true;
+      if (!keeps_scratch[(size_t)it->second]) plan->kept_scratch_bytes += lead->rk.scratch_bytes;
       keeps_scratch[(size_t)it->second] = keeps_scratch[(size_t)ui] = 1;
       if (getenv("POLY_HIP_DEBUG"))
         fprintf(stderr, "polygrad: compile_schedule: launch %d reads what the first stage of launch %d leaves\n", ui, it->second);
@@ -734,6 +736,6 @@ void *poly_hip_plan_slot_ptr(const PolyHipPlan *plan, int slot) {
 }
 
 void poly_hip_plan_set_graph(PolyHipPlan *plan, int enabled) { if (plan) plan->use_graph = enabled != 0; }
-size_t poly_hip_plan_workspace_bytes(const PolyHipPlan *plan) { return plan ? plan->arena_bytes + plan->scratch_bytes : 0; }
+size_t poly_hip_plan_workspace_bytes(const PolyHipPlan *plan) { return plan ? plan->arena_bytes + plan->scratch_bytes + plan->kept_scratch_bytes : 0; }
 
 }  // extern "C"

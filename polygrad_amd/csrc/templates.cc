@@ -587,6 +587,8 @@ bool render_matmul(const MatmulMatch &mm, const MatmulEpilogue &ep, RenderedKern
     cfg += matmul_k_fn("poly_a_k", ka, K);
     cfg += matmul_k_fn("poly_b_k", kb, K);
     cfg += strf("#define POLY_SIGNATURE %s\n", signature.c_str());
+    // LDS beside the operand tiles that an epilogue may use for the middle of its lookup tables
+    if (S == 1 && !getenv("POLY_HIP_NO_LUT_WINDOW")) cfg += strf("#define POLY_EP_WIN_ROOM %d\n", 163840 - 2 * (bm + bn) * BK * 2);
     cfg += ep.code;
     if (S > 1) {
       cfg += strf("#define POLY_KSPLIT %d\n#define POLY_PARTIALS %s\n", S, partials.c_str());
@@ -602,6 +604,7 @@ bool render_matmul(const MatmulMatch &mm, const MatmulEpilogue &ep, RenderedKern
     if (split) {
       cfg += strf("#define POLY_EP_TYPE %s\n", ep.out_type.c_str());
       cfg += strf("#define POLY_EP_VALUE(acc, m, n, z) %s\n", ep.value_call.c_str());
+      if (!ep.value_call_win.empty()) cfg += strf("#define POLY_EP_VALUE_WIN(acc, m, n, z) %s\n", ep.value_call_win.c_str());
       cfg += strf("#define POLY_EP_PTR(m, n, z) %s\n", ep.ptr_call.c_str());
     }
 

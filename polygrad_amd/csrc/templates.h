@@ -57,6 +57,7 @@ struct MatmulEpilogue {
   // Optional split of `call` into value and address, for outputs that are contiguous
   // along n: the template then stores 8 values of a row with one 16-byte store.
   std::string value_call;  // expression of type out_type: uses acc, m, n, z
+  std::string value_call_win;   // the same value with table lookups served from LDS windows (sets poly_tmax), or empty
   std::string ptr_call;    // expression of type out_type*: uses m, n, z
   std::string out_type;
   bool contiguous_n = false;

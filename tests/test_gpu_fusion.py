@@ -185,7 +185,11 @@ def test_attention_with_more_than_64_key_tiles(mask_value):
 
 def test_lookup_table_epilogue_is_bit_identical_to_the_arithmetic():
     """A pointwise kernel of one 16-bit input fused behind a matmul is evaluated through a
-    65536-entry table filled by its own expression: results must not change by a bit."""
+    65536-entry table filled by its own expression: results must not change by a bit.  The
+    matmul keeps the table's entries for 2^-24 <= |x| < 256 in LDS and goes to the table in
+    memory for a group of values with an input outside that range: rows of zeros, of huge,
+    of undefined and of tiny products are among the inputs, and the result must be the same
+    with the LDS copy switched off."""
     m, n, k = 512, 768, 256
     g = np.random.default_rng(21)
     c = R.Ctx()
@@ -194,10 +198,22 @@ def test_lookup_table_epilogue_is_bit_identical_to_the_arithmetic():
     O = c.buffer((m, n), R.BF16, name="O")
     y = A.cast(R.F32).dot(W.cast(R.F32)).cast(R.BF16).contiguous()
     sink = c.sink((O, y.gelu()))
-    arrays = {A: R.f32_to_bf16_bits(g.normal(0, 1.0, m * k).astype(np.float32)),
+    a = g.normal(0, 1.0, (m, k)).astype(np.float32)
+    a[3] = 0.0                 # products exactly 0
+    a[40:44] *= 1e3            # |x| beyond 256
+    a[77] = np.inf             # inf - inf: NaN in any order of summation
+    a[130:133] *= 1e-9         # |x| below 2^-24
+    a[200, ::2] = 0.0
+    arrays = {A: R.f32_to_bf16_bits(a.reshape(-1)),
               W: R.f32_to_bf16_bits(g.normal(0, 0.2, k * n).astype(np.float32)), O: np.zeros(m * n, np.uint16)}
     with_table, info = run_hip(c, sink, arrays)
     assert any("lookup table" in kk["desc"] for kk in info), [kk["desc"] for kk in info]
+    os.environ["POLY_HIP_NO_LUT_WINDOW"] = "1"
+    try:
+        from_memory, _ = run_hip(c, sink, arrays)
+    finally:
+        del os.environ["POLY_HIP_NO_LUT_WINDOW"]
+    assert with_table[O].tobytes() == from_memory[O].tobytes()
     os.environ["POLY_HIP_NO_LUT"] = "1"
     try:
         plain, info2 = run_hip(c, sink, arrays)
@@ -205,6 +221,8 @@ def test_lookup_table_epilogue_is_bit_identical_to_the_arithmetic():
         del os.environ["POLY_HIP_NO_LUT"]
     assert not any("lookup table" in kk["desc"] for kk in info2) and len(info2) == len(info)
     assert with_table[O].tobytes() == plain[O].tobytes()
+    got = R.bf16_bits_to_f32(with_table[O]).reshape(m, n)
+    assert (got[3] == 0).all() and np.isnan(got[77]).all() and (np.abs(got[40:44]) > 256).any()
     want = run_ref(c, sink, arrays)
     c.close()
     assert_close(R.bf16_bits_to_f32(with_table[O]), R.bf16_bits_to_f32(want[O]), rtol=2e-2, atol=2e-2, what="matmul + GELU vs reference")
