@@ -89,6 +89,12 @@ __device__ __forceinline__ int poly_swz(int row) { return (row ^ (row >> 3)) & (
 #ifndef POLY_KSPLIT
 #define POLY_KSPLIT 1
 #endif
+// columns [POLY_N_LO, POLY_N_HI) are this launch's (another launch has the others);
+// POLY_N_LO is a multiple of POLY_BN, and so is POLY_N_HI unless it is POLY_N
+#ifndef POLY_N_LO
+#define POLY_N_LO 0
+#define POLY_N_HI POLY_N
+#endif
 // K tiles one workgroup walks: with POLY_KSPLIT > 1 the K tiles of an output tile are dealt
 // to that many workgroups (blockIdx.y = z * POLY_KSPLIT + part), each leaving its fp32
 // accumulators where the epilogue macros put them (they may use `poly_ks`, the part).
@@ -201,7 +207,7 @@ extern "C" __global__ void __launch_bounds__(POLY_NTHREADS) poly_k(POLY_SIGNATUR
   // contiguous run of tiles, and runs walk down M within a band of columns so the
   // B panel stays resident in that XCD's L2.
   constexpr int TILES_M = (POLY_M + POLY_BM - 1) / POLY_BM;
-  constexpr int TILES_N = (POLY_N + POLY_BN - 1) / POLY_BN;
+  constexpr int TILES_N = (POLY_N_HI - POLY_N_LO + POLY_BN - 1) / POLY_BN;
   constexpr int NT = TILES_M * TILES_N;
   int bid = blockIdx.x;
   {
@@ -239,7 +245,7 @@ extern "C" __global__ void __launch_bounds__(POLY_NTHREADS) poly_k(POLY_SIGNATUR
   const int z = blockIdx.y;
   constexpr int k_base = 0;
 #endif
-  const int m0 = tile_m * POLY_BM, n0 = tile_n * POLY_BN;
+  const int m0 = tile_m * POLY_BM, n0 = POLY_N_LO + tile_n * POLY_BN;
 
   const POLY_TIN *__restrict__ gA = POLY_A_PTR + poly_a_z(z);
   const POLY_TIN *__restrict__ gB = POLY_B_PTR + poly_b_z(z);

@@ -558,8 +558,11 @@ bool render_matmul(const MatmulMatch &mm, const MatmulEpilogue &ep, RenderedKern
   const std::string partials = ep.scratch_type.empty() ? std::string("poly_scratch") : strf("((float*)((char*)poly_scratch + %zuull))", part_off);
   const std::string signature = ep.signature + (S > 1 && ep.scratch_type.empty() ? ", float* poly_scratch" : "");
 
-  auto emit = [&](int bm, int bn, int wvm, int wvn, int pp, RenderedKernel *rk) {
-    const int64_t tiles = ((M + bm - 1) / bm) * ((N + bn - 1) / bn);
+  // (n_lo, n_hi: the columns this launch covers; n_lo and, unless it is N, n_hi are
+  // multiples of bn)
+  auto emit = [&](int bm, int bn, int wvm, int wvn, int pp, RenderedKernel *rk, int64_t n_lo = 0, int64_t n_hi = -1) {
+    if (n_hi < 0) n_hi = N;
+    const int64_t tiles = ((M + bm - 1) / bm) * ((n_hi - n_lo + bn - 1) / bn);
     if (tiles > 2147483647LL / 2) return reject(__LINE__);
     // ── configuration block ─────────────────────────────────────────────────
     std::string cfg;
@@ -567,6 +570,7 @@ bool render_matmul(const MatmulMatch &mm, const MatmulEpilogue &ep, RenderedKern
     cfg += strf("#define POLY_MFMA(a, b, c) __builtin_amdgcn_mfma_f32_32x32x16_%s(a, b, c, 0, 0, 0)\n", A.dt == DT_BF16 ? "bf16" : "f16");
     cfg += strf("#define POLY_M %lld\n#define POLY_N %lld\n#define POLY_K %lld\n#define POLY_Z %lld\n", (long long)M, (long long)N, (long long)K, (long long)Z);
     cfg += strf("#define POLY_BM %d\n#define POLY_BN %d\n#define POLY_BK %d\n#define POLY_WAVES_M %d\n#define POLY_WAVES_N %d\n", bm, bn, BK, wvm, wvn);
+    if (n_lo != 0 || n_hi != N) cfg += strf("#define POLY_N_LO %lld\n#define POLY_N_HI %lld\n", (long long)n_lo, (long long)n_hi);
     cfg += strf("#define POLY_GROUP_M %d\n", bm >= 256 ? 4 : 8);
     // each XCD (own L2) works on a contiguous run of tiles: let it re-read the smaller operand
     cfg += strf("#define POLY_GROUP_ALONG_N %d\n", (N > 2 * M && !getenv("POLY_HIP_MM_GROUP_M")) ? 1 : 0);
@@ -641,6 +645,48 @@ bool render_matmul(const MatmulMatch &mm, const MatmulEpilogue &ep, RenderedKern
     out->launch.block[0] = 256;
     out->strategy += strf(", K dealt to %d workgroups per tile, partial results added by a second kernel", S);
     return true;
+  }
+  // A last round over the chip that is at most half full (8192 x 2304 in 128 x 256 tiles:
+  // 576 tiles, two rounds and a quarter) costs a whole round.  The launch then keeps the
+  // columns whose tiles make whole rounds, and the columns left over go to a launch of
+  // their own ahead of it, in tiles a quarter or half the size, so that they fill the chip
+  // once with short workgroups.  Taken when the estimate (rounds, a small tile's round
+  // weighted by its area and by what its narrower wave tiles cost, plus a launch) saves
+  // a quarter of a round or more.
+  if (Z == 1 && M > 64 && N > 64 && !matmul_tuning_enabled() && !getenv("POLY_HIP_NO_TAIL_LAUNCH") && !getenv("POLY_HIP_MM_NOEPI")) {
+    const int64_t tm = (M + BM - 1) / BM, tn = (N + BN - 1) / BN, T = tm * tn;
+    const int64_t whole = T / 256, rest = T % 256;
+    const int64_t keep = std::min<int64_t>(whole * 256 / tm, tn - 1);     // column tiles of the main launch
+    if (whole >= 1 && rest > 0 && keep >= 1 && (!a_kc ? M % 8 == 0 : true)) {
+      struct Small { int bm, bn, wm, wn; double cost; };
+      // cost of a launch of one round of such tiles relative to a round of 128 x 256 tiles
+      // (measured at K = 768: 12.6 and 10.5 us against 18.6; most of it does not depend on
+      // the tile: the launch, the first loads, the epilogue)
+      static const Small smalls[] = {{128, 128, 2, 2, 0.68}, {128, 64, 4, 1, 0.56}};
+      const int64_t n_lo = keep * BN;
+      const double before = std::ceil((double)T / 256.0);
+      double best = before - 0.25;
+      const Small *pick = nullptr;
+      for (const Small &c : smalls) {
+        if (c.bm > BM || c.bn > BN) continue;
+        const double scale = (128.0 * 256.0) / ((double)BM * BN);
+        const int64_t tt = ((M + c.bm - 1) / c.bm) * ((N - n_lo + c.bn - 1) / c.bn);
+        const double after = std::ceil((double)(tm * keep) / 256.0) + std::ceil((double)tt / 256.0) * c.cost * scale + 0.1;
+        if (after < best) { best = after; pick = &c; }
+      }
+      Small forced{0, 0, 0, 0, 0};
+      if (const char *ov = getenv("POLY_HIP_MM_TAIL_TILE"))    // "BM,BN,WVM,WVN": tuning experiments
+        if (sscanf(ov, "%d,%d,%d,%d", &forced.bm, &forced.bn, &forced.wm, &forced.wn) == 4 && BN % forced.bn == 0) pick = &forced;
+      RenderedKernel main, tail;
+      if (pick && emit(BM, BN, WVM, WVN, pipe, &main, 0, n_lo) && emit(pick->bm, pick->bn, pick->wm, pick->wn, 3, &tail, n_lo, N)) {
+        const std::string strategy = out->strategy;
+        *out = main;
+        out->pres.push_back({tail.source, tail.entry, tail.launch});
+        out->scratch_bytes = 256;      // (a kernel with a first stage owns scratch memory; this one uses none)
+        out->strategy = strategy + strf(", columns from %lld on by a launch of %dx%d tiles ahead of it", (long long)n_lo, pick->bm, pick->bn);
+        return true;
+      }
+    }
   }
   // Candidates for on-device tuning: the same kernel in the other tile shapes and
   // pipeline depths; the plan times them on its first run when POLY_BEAM is set.
