@@ -36,11 +36,11 @@ GPT2_PLAN = "gpt2_small_bf16_b8_t1024"
 # under profiles/ (…hbm_traffic_pmc.md).
 MEASURED_TRAFFIC = {
     "attention-mfma: fused attention (9 kernels): mfma 32x32x16 bf16 Z=96 M=1024 N=1024 D=64, one pass, online softmax, mask tiles classified by a first kernel": 39.1e6 + 12.6e6 + 2.1e6,
-    "matmul-mfma: mfma 32x32x16 bf16 M=8192 N=3072 K=768 Z=1 tile 128x256x64 A:k-major B:n-major": 74.0e6 + 51.1e6,
-    "matmul-mfma: mfma 32x32x16 bf16 M=8192 N=2304 K=768 Z=1 tile 128x256x64 A:k-major B:n-major": 63.8e6 + 37.8e6,
+    "matmul-mfma: mfma 32x32x16 bf16 M=8192 N=3072 K=768 Z=1 tile 128x256x64 A:k-major B:n-major": 74.4e6 + 51.1e6,
+    "matmul-mfma: mfma 32x32x16 bf16 M=8192 N=2304 K=768 Z=1 tile 128x256x64 A:k-major B:n-major": 49.9e6 + 15.9e6 + 33.6e6 + 4.2e6,
     "matmul-mfma: mfma 32x32x16 bf16 M=8192 N=768 K=3072 Z=1 tile 128x256x64 A:k-major B:n-major": 101.0e6 + 15.8e6,
     "matmul-mfma: mfma 32x32x16 bf16 M=8192 N=768 K=768 Z=1 tile 128x256x64 A:k-major B:n-major": 35.0e6 + 15.5e6,
-    "matmul-mfma: mfma 32x32x16 bf16 M=8192 N=50257 K=768 Z=1 tile 256x256x64 A:k-major B:k-major": 987.5e6 + 952.0e6,
+    "matmul-mfma: mfma 32x32x16 bf16 M=8192 N=50257 K=768 Z=1 tile 256x256x64 A:k-major B:k-major": 992.7e6 + 948.8e6,
 }
 
 
