@@ -65,7 +65,7 @@ def run_gpu(workload, steps, warmup):
     if workload.startswith("gpt2_medium_block_train") or workload.startswith("gpt2_medium_train"):
         data, _ = block_train_slot_tensors(plan)
         tokens = None
-    elif workload.startswith("gpt2"):
+    elif workload.startswith("gpt2_small_bf16"):
         data, _ = gpt2_slot_tensors(plan)
         tokens = [s for s in plan.slots if s.name == "x"][0].numel
     else:
