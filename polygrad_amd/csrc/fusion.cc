@@ -1170,6 +1170,39 @@ static bool match_copy(const Sched &sc, int item, CopyMap *cm) {
 }
 
 // Tries to grow an attention group from the matmul at schedule item `s_item`.
+// Which (block of 128 queries, z) each workgroup of the attention kernel takes.  Under a
+// causal mask block b has b + 1 times the work of block 0, every workgroup is resident from
+// the start (three per CU) and the hardware puts workgroups j, j + 32, j + 64 of an XCD on
+// the same CU (ids go round the 8 XCDs first), so the order decides how evenly the CUs are
+// loaded: heaviest first, and within each later round of 32 the heaviest goes to the CU
+// that has the least so far.  For 8 blocks x 12 z per XCD the CUs then carry 13 or 14 units
+// each instead of 10 to 17.  (Without such a mask all workgroups weigh the same and any
+// order does.)  Emitted as a table indexed by the workgroup's number within its XCD.
+static std::string attention_order(int64_t MB, int64_t Z) {
+  if (getenv("POLY_HIP_FA_PLAIN_ORDER") || Z % 8 != 0 || MB < 2) return "";
+  const int64_t ZX = Z / 8, n = MB * ZX;
+  if (n > 8192) return "";
+  constexpr int CUS = 32;
+  std::vector<int> items((size_t)n);                 // mb * ZX + z', heaviest first
+  for (int64_t i = 0; i < n; i++) items[(size_t)i] = (int)((MB - 1 - i / ZX) * ZX + i % ZX);
+  std::vector<int> order((size_t)n);
+  std::vector<int64_t> load(CUS, 0);
+  for (int64_t r0 = 0; r0 < n; r0 += CUS) {
+    const int k = (int)std::min<int64_t>(CUS, n - r0);
+    std::vector<int> cu((size_t)k);
+    for (int c = 0; c < k; c++) cu[(size_t)c] = c;
+    std::stable_sort(cu.begin(), cu.end(), [&](int a, int b) { return load[(size_t)a] < load[(size_t)b]; });
+    for (int i = 0; i < k; i++) {
+      const int item = items[(size_t)(r0 + i)];
+      order[(size_t)(r0 + cu[(size_t)i])] = item;
+      load[(size_t)cu[(size_t)i]] += item / ZX + 1;
+    }
+  }
+  std::string t = strf("#define POLY_FA_ORDER 1\n__constant__ unsigned short poly_fa_order[%lld] = {", (long long)n);
+  for (int64_t i = 0; i < n; i++) t += strf("%s%d", i ? "," : "", order[(size_t)i]);
+  return t + "};\n";
+}
+
 static bool match_attention(const Sched &sc, int s_item, const std::vector<char> &taken, FusedGroup *out) {
   const PolySchedule *s = sc.s;
   const KernelGraph &gS = sc.graphs[(size_t)s_item];
@@ -1532,6 +1565,7 @@ static bool match_attention(const Sched &sc, int s_item, const std::vector<char>
   cfg += strf("#define POLY_TIN %s\n", tn);
   cfg += strf("#define POLY_MFMA(a, b, c) __builtin_amdgcn_mfma_f32_32x32x16_%s(a, b, c, 0, 0, 0)\n", tin == DT_BF16 ? "bf16" : "f16");
   cfg += strf("#define POLY_FA_M %lld\n#define POLY_FA_N %lld\n#define POLY_FA_Z %lld\n", (long long)mS.M, (long long)mS.N, (long long)mS.Z);
+  cfg += attention_order(mS.M / 128, mS.Z);
   auto operand_arg = [&](int o) { return arg_of(folded[o].item >= 0 ? folded[o].src_slot : op_slot[o]); };
   cfg += strf("#define POLY_Q_PTR fa%d\n#define POLY_K_PTR fa%d\n#define POLY_V_PTR fa%d\n", operand_arg(0), operand_arg(1), operand_arg(2));
   // position in the operand's own buffer -> position in the buffer it was copied from

@@ -201,8 +201,16 @@ extern "C" __global__ void __launch_bounds__(FA_THREADS) __attribute__((amdgpu_w
   if (POLY_FA_Z % 8 == 0) {
     constexpr int ZX = POLY_FA_Z / 8 > 0 ? POLY_FA_Z / 8 : 1;   // z per XCD
     const int xcd = blockIdx.x & 7, j = blockIdx.x >> 3;
+#ifdef POLY_FA_ORDER
+    // (a table from the renderer: the same blocks, dealt so that the three workgroups that
+    // share a CU carry about the same number of key blocks together)
+    const int item = poly_fa_order[j];
+    mb = item / ZX;
+    z = xcd * ZX + item % ZX;
+#else
     mb = MB - 1 - j / ZX;
     z = xcd * ZX + j % ZX;
+#endif
   } else {
     mb = MB - 1 - (int)blockIdx.x / POLY_FA_Z;
     z = (int)blockIdx.x % POLY_FA_Z;

@@ -32,6 +32,7 @@ static poly_dim3 threadIdx, blockIdx, blockDim, gridDim;
 #define __launch_bounds__(...)
 #define amdgpu_waves_per_eu(...)
 #define __shared__ static
+#define __constant__ static const
 #define __syncthreads() ((void)0)
 #define __lane_id() (threadIdx.x & 63u)
 #define __builtin_amdgcn_update_dpp(old, src, ctrl, rm, bm, bc) (src)
