@@ -330,29 +330,27 @@ static bool make_unary_table(const Sched &sc, const Member &m, RenderedKernel::T
 // mode 0.
 static const char *const kNoWindow = "0, (unsigned int*)0";
 static const char *const kWindow = "1, &poly_tmax";
-static std::string table_window_helpers(const std::vector<RenderedKernel::Table> &tables, const std::vector<std::string> &types) {
+static std::string table_window_helpers(const std::vector<RenderedKernel::Table> &tables) {
   size_t bytes = 0;
-  std::string fill;
-  for (size_t i = 0; i < tables.size(); i++) {
-    fill += strf(" poly_win_fill<%s>(poly_win_raw + %zu, poly_lut%zu, tid, nthreads);", types[i].c_str(), bytes, i);
-    bytes += tables[i].bytes / 8;
-  }
+  std::string src = "(const unsigned char*)0";     // nested ?: from the last table to the first
+  std::vector<size_t> offs;
+  for (size_t i = 0; i < tables.size(); i++) { offs.push_back(bytes); bytes += tables[i].bytes / 8; }
+  for (size_t i = tables.size(); i-- > 0;)
+    src = i + 1 == tables.size() ? strf("poly_win_src(poly_lut%zu, (b) - %zu)", i, offs[i])
+                                 : strf("((b) < %zu ? poly_win_src(poly_lut%zu, (b) - %zu) : %s)", offs[i + 1], i, offs[i], src.c_str());
   // (the window is read through a pointer that names the LDS address space: with a plain
   // pointer the compiler picks between window and table by address and issues one flat load)
   return strf("#define POLY_LDS __attribute__((address_space(3)))\n"
               "#if defined(POLY_EP_WIN_ROOM) && POLY_EP_WIN_ROOM >= %zu\n#define POLY_EP_WIN_BYTES %zu\n"
               "#define POLY_EP_WIN(off, T) ((POLY_LDS const T*)(poly_win_raw + (off)))\n"
-              "#define POLY_EP_WIN_FILL(tid, nthreads) do {%s } while (0)\n"
-              "#else\n#define POLY_EP_WIN(off, T) ((POLY_LDS const T*)0)\n#endif\n", bytes, bytes, fill.c_str()) +
+              "#define POLY_EP_WIN_SRC(b) %s   /* where byte b of the windows comes from */\n"
+              "#else\n#define POLY_EP_WIN(off, T) ((POLY_LDS const T*)0)\n#endif\n", bytes, bytes, src.c_str()) +
          "#define POLY_WIN_FIRST (103u << 7)   /* code of 2^-24 */\n"
          "#define POLY_WIN_CODES 4096u         /* per sign */\n"
-         "typedef unsigned int poly_win_u32x4 __attribute__((ext_vector_type(4)));\n"
-         "template <typename T> __device__ __forceinline__ void poly_win_fill(unsigned char* win, const T* __restrict__ lut, int tid, int nthreads) {\n"
+         "template <typename T> __device__ __forceinline__ const unsigned char* poly_win_src(const T* __restrict__ lut, int b) {\n"
          "  constexpr int HALF = (int)POLY_WIN_CODES * (int)sizeof(T);   // bytes per sign\n"
-         "  for (int b = tid * 16; b < 2 * HALF; b += nthreads * 16) {\n"
-         "    const int first = ((b / HALF) * 0x8000 + (int)POLY_WIN_FIRST) * (int)sizeof(T);\n"
-         "    *(poly_win_u32x4*)(win + b) = *(const poly_win_u32x4*)((const unsigned char*)lut + first + b % HALF);\n"
-         "  }\n}\n"
+         "  return (const unsigned char*)lut + ((b / HALF) * 0x8000 + (int)POLY_WIN_FIRST) * (int)sizeof(T) + b % HALF;\n"
+         "}\n"
          "template <typename T, typename X> __device__ __forceinline__ T poly_lut_get(const T* __restrict__ lut, POLY_LDS const T* win, const int mode, unsigned int* tmax, X x) {\n"
          "  const unsigned int u = __builtin_bit_cast(unsigned short, x);\n"
          "#ifdef POLY_EP_WIN_BYTES\n"
@@ -439,7 +437,6 @@ static bool match_matmul_tail(const Sched &sc, int s_item, const std::vector<cha
   std::vector<RenderedKernel::Table> tables;
   std::map<size_t, int> table_of;     // member -> table index
   std::map<size_t, std::string> lead_of, lut_arg_of, lookup_of;
-  std::vector<std::string> table_types;
   size_t win_bytes = 0;               // LDS windows of the tables so far
   bool windowed = false;              // some table takes bf16 codes: its lookups know the window
   for (size_t e = 1; e < members.size(); e++) {
@@ -462,7 +459,6 @@ static bool match_matmul_tail(const Sched &sc, int s_item, const std::vector<cha
       ep.signature += strf(", const %s* __restrict__ poly_lut%zu", tab_type.c_str(), tables.size());
       win_bytes += tab.bytes / 8;
       tables.push_back(tab);
-      table_types.push_back(tab_type);
     }
     lead_of[e] = lead;
     if (!emit_member_fn(sc, m, master_decomp, fn.c_str(), dt_cname(g.n(g.stores[0].value).dt), lead, g.stores[0].value, extra, false, last,
@@ -471,7 +467,7 @@ static bool match_matmul_tail(const Sched &sc, int s_item, const std::vector<cha
     prev_dt = g.n(g.stores[0].value).dt;
   }
   ep.call = call;
-  if (!tables.empty()) ep.code = table_window_helpers(tables, table_types) + ep.code;
+  if (!tables.empty()) ep.code = table_window_helpers(tables) + ep.code;
   {
     // value and address of the last kernel's store, separately, when rows are contiguous
     const Member &m = members.back();

@@ -24,8 +24,8 @@
 //                       template writes 8 values of a row with one store
 //   POLY_EP_WIN_BYTES   (optional, set by the epilogue's own code when POLY_EP_WIN_ROOM, the
 //                       LDS left beside the operand tiles, suffices) bytes of LDS that
-//                       POLY_EP_WIN_FILL(tid, nthreads) fills with the middle of the
-//                       epilogue's lookup tables; POLY_EP_VALUE_WIN is then POLY_EP_VALUE
+//                       the kernel fills from POLY_EP_WIN_SRC(byte) with the middle of
+//                       the epilogue's lookup tables; POLY_EP_VALUE_WIN is then POLY_EP_VALUE
 //                       with lookups from there, raising poly_tmax to POLY_WIN_CODES or
 //                       more when an input lies outside
 //
@@ -194,10 +194,27 @@ extern "C" __global__ void __launch_bounds__(POLY_NTHREADS) poly_k(POLY_SIGNATUR
   // one allocation: the operand tiles during the K loop, the per-wave output staging after it
   __shared__ __attribute__((aligned(16))) POLY_TIN lds_raw[2 * (POLY_BM + POLY_BN) * POLY_LDK];
 #ifdef POLY_EP_WIN_BYTES
-  // the entries of the epilogue's lookup tables that most values hit; the barriers of the K
-  // loop lie between this copy and the epilogue's reads
+  // The entries of the epilogue's lookup tables that most values hit.  Their loads are the
+  // first the kernel issues; they go to LDS once the loads of the first operand tiles are
+  // on their way (nothing waits for them alone), and the barriers of the K loop lie
+  // between that and the epilogue's reads.
   __shared__ __attribute__((aligned(16))) unsigned char poly_win_raw[POLY_EP_WIN_BYTES];
-  POLY_EP_WIN_FILL((int)threadIdx.x, POLY_NTHREADS);
+  constexpr int WIN_VECS = (POLY_EP_WIN_BYTES / 16 + POLY_NTHREADS - 1) / POLY_NTHREADS;
+  poly_u32x4 win_regs[WIN_VECS];
+#pragma unroll
+  for (int v = 0; v < WIN_VECS; v++) {
+    const int b = ((int)threadIdx.x + v * POLY_NTHREADS) * 16;
+    if (POLY_EP_WIN_BYTES / 16 % POLY_NTHREADS == 0 || b < POLY_EP_WIN_BYTES) win_regs[v] = *(const poly_u32x4 *)POLY_EP_WIN_SRC(b);
+  }
+  auto win_store = [&]() {
+#pragma unroll
+    for (int v = 0; v < WIN_VECS; v++) {
+      const int b = ((int)threadIdx.x + v * POLY_NTHREADS) * 16;
+      if (POLY_EP_WIN_BYTES / 16 % POLY_NTHREADS == 0 || b < POLY_EP_WIN_BYTES) *(poly_u32x4 *)(poly_win_raw + b) = win_regs[v];
+    }
+  };
+#else
+  auto win_store = [&]() {};
 #endif
   auto lds_a = [&](int buf) { return lds_raw + buf * (POLY_BM * POLY_LDK); };
   auto lds_b = [&](int buf) { return lds_raw + 2 * POLY_BM * POLY_LDK + buf * (POLY_BN * POLY_LDK); };
@@ -441,6 +458,7 @@ extern "C" __global__ void __launch_bounds__(POLY_NTHREADS) poly_k(POLY_SIGNATUR
   // iterations to land.  Tile t always uses register set t & 1, hence the loop is
   // unrolled by two.
   load_tiles(0, ra0, rb0);
+  win_store();
   StageA::store(lds_a(0), ra0);
   StageB::store(lds_b(0), rb0);
   if (POLY_KT > 1) load_tiles(1, ra1, rb1);
@@ -468,6 +486,7 @@ extern "C" __global__ void __launch_bounds__(POLY_NTHREADS) poly_k(POLY_SIGNATUR
   // register set): the global loads of tile kt+1 are issued at the top of iteration kt
   // and move to the other LDS buffer during the second half of its slots.
   load_tiles(0, ra0, rb0);
+  win_store();
   StageA::store(lds_a(0), ra0);
   StageB::store(lds_b(0), rb0);
   __syncthreads();
