@@ -20,9 +20,10 @@
 //   POLY_SP_OUT                            the kernel argument that receives the planes
 //   POLY_SIGNATURE
 //
-// One workgroup of 256 threads handles a 64 (rows) x 64 (k) tile: values are computed
-// with lanes along whichever axis the source is contiguous in, pass through LDS, and
-// leave with lanes along k.
+// One workgroup of 256 threads handles a 64 (rows) x 64 (k) tile, 16 values per thread: two
+// groups of 8 neighbours along k when the source is contiguous in k and K a multiple of 8;
+// otherwise with lanes along the source's contiguous axis and through LDS, to leave with
+// lanes along k.
 #ifdef POLY_TEMPLATE_STANDALONE
 #include <hip/hip_runtime.h>
 #define POLY_SP_ROWS 4096
@@ -39,11 +40,59 @@
 #endif
 
 extern "C" __global__ void __launch_bounds__(256) poly_k(POLY_SIGNATURE) {
-  __shared__ float tile[64][65];
   constexpr int TILES_K = POLY_SP_KP / 64;
   const int tk = blockIdx.x % TILES_K, tr = blockIdx.x / TILES_K, z = blockIdx.y;
   const int row0 = tr * 64, k0 = tk * 64;
-  // 16 elements per thread
+  __bf16 *const out = (POLY_SP_OUT) + (size_t)z * POLY_SP_ROWS * (POLY_SP_PARTS * POLY_SP_KP);
+  typedef __bf16 sp_out8 __attribute__((ext_vector_type(8)));
+  // 8 consecutive k of one row leave as one 16-byte store per plane (rows of the planes
+  // start on multiples of 64 elements from a 256-byte aligned base)
+  auto write_planes = [&](int row, int lk, const float (&x)[8]) {
+    __bf16 *const dst = out + (size_t)row * (POLY_SP_PARTS * POLY_SP_KP) + k0 + lk;
+    sp_out8 hi, mid, lo;
+#pragma unroll
+    for (int e = 0; e < 8; e++) {
+      hi[e] = (__bf16)x[e];
+      if (POLY_SP_PARTS == 3) {
+        // (an infinite or NaN x is all in hi: no inf - inf in the residuals)
+        const float r1 = __builtin_isfinite((float)hi[e]) ? x[e] - (float)hi[e] : 0.0f;
+        mid[e] = (__bf16)r1;
+        lo[e] = (__bf16)(r1 - (float)mid[e]);
+      }
+    }
+    *(sp_out8 *)dst = hi;
+    if (POLY_SP_PARTS == 3) {
+      *(sp_out8 *)(dst + POLY_SP_KP) = mid;
+      *(sp_out8 *)(dst + 2 * POLY_SP_KP) = lo;
+    }
+  };
+#if POLY_SP_WALK_K && POLY_SP_K % 8 == 0
+  // along k, rows a multiple of 8 long: a thread takes 8 neighbours, so that what the operand's expression loads for
+  // them sits side by side and can be fetched together, and they are a row's piece as the
+  // planes store it: no exchange needed
+#pragma unroll
+  for (int i = 0; i < 2; i++) {
+    const int g = threadIdx.x + i * 256;
+    const int lr = g / 8, lk = (g % 8) * 8;
+    const int row = row0 + lr;
+    if (row >= POLY_SP_ROWS) continue;
+    float x[8];
+#pragma unroll
+    for (int e = 0; e < 8; e++) {
+      const int k = k0 + lk + e;
+      x[e] = 0.0f;
+      if (k < POLY_SP_K) {
+        unsigned int raw[POLY_SP_NRAW];
+        POLY_SP_LOAD(row, k, z, raw);
+        x[e] = POLY_SP_MATH(row, k, z, raw);
+      }
+    }
+    write_planes(row, lk, x);
+  }
+#else
+  // along the rows, or along rows of k of any length: lanes along that axis (64 neighbours
+  // per load), through LDS, to leave with lanes along k
+  __shared__ float tile[64][65];
 #pragma unroll 4
   for (int i = 0; i < 16; i++) {
     const int c = threadIdx.x + i * 256;
@@ -58,24 +107,16 @@ extern "C" __global__ void __launch_bounds__(256) poly_k(POLY_SIGNATURE) {
     tile[lr][lk] = v;
   }
   __syncthreads();
-  __bf16 *const out = (POLY_SP_OUT) + (size_t)z * POLY_SP_ROWS * (POLY_SP_PARTS * POLY_SP_KP);
-#pragma unroll 4
-  for (int i = 0; i < 16; i++) {
-    const int c = threadIdx.x + i * 256;
-    const int lr = c / 64, lk = c % 64;
+#pragma unroll
+  for (int i = 0; i < 2; i++) {
+    const int g = threadIdx.x + i * 256;
+    const int lr = g / 8, lk = (g % 8) * 8;
     const int row = row0 + lr;
     if (row >= POLY_SP_ROWS) continue;
-    const float x = tile[lr][lk];
-    __bf16 *const dst = out + (size_t)row * (POLY_SP_PARTS * POLY_SP_KP) + k0 + lk;
-    const __bf16 hi = (__bf16)x;
-    dst[0] = hi;
-    if (POLY_SP_PARTS == 3) {
-      // (an infinite or NaN x is all in hi: no inf - inf in the residuals)
-      const float r1 = __builtin_isfinite((float)hi) ? x - (float)hi : 0.0f;
-      const __bf16 mid = (__bf16)r1;
-      const float r2 = r1 - (float)mid;
-      dst[POLY_SP_KP] = mid;
-      dst[2 * POLY_SP_KP] = (__bf16)r2;
-    }
+    float x[8];
+#pragma unroll
+    for (int e = 0; e < 8; e++) x[e] = tile[lr][lk + e];
+    write_planes(row, lk, x);
   }
+#endif
 }
