@@ -171,6 +171,11 @@ void *poly_hip_plan_slot_ptr(const PolyHipPlan *plan, int slot);
 /* Enable (1, default) or disable (0) hipGraph replay for this plan. */
 void poly_hip_plan_set_graph(PolyHipPlan *plan, int enabled);
 size_t poly_hip_plan_workspace_bytes(const PolyHipPlan *plan);
+/* How many launches of the plan its captured graph runs on a second stream beside the
+ * main sequence (small launches that are a chain of dependent steps; 0 for most plans).
+ * No counterpart in the reference, whose plans run kernel by kernel with a sync after
+ * each (src/exec_plan.c:1000-1057). */
+int poly_hip_plan_side_launches(const PolyHipPlan *plan);
 
 /* ── Serialized schedules ("plan files") ─────────────────────────────────── */
 

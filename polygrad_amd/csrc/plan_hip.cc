@@ -77,6 +77,17 @@ struct PolyHipPlan {
   std::vector<std::vector<void *>> kargs;    // per unit: args array handed to runner_launch
   std::vector<std::vector<int>> var_vals;    // per unit: storage for var ints
   std::vector<PolyVarBinding> merged;
+  // Launches that a captured graph runs beside the main sequence, on a second stream: small
+  // launches whose time is a dependent chain, not throughput (the in-order adders of the
+  // bf16 column sums: 1024 threads for 48 us each, 194 of them in a 24-layer training step).
+  // wait_for[u]: the latest launch on the other stream that u's buffers depend on (-1: none
+  // that an earlier wait does not already cover); records[u]: someone waits for u.
+  std::vector<char> on_side;
+  std::vector<int> wait_for;
+  std::vector<char> records;
+  std::vector<hipEvent_t> events;            // per launch (those with records), then fork and join
+  bool forked = false;
+  void *side_scratch_pool = nullptr;         // the two-stage kernels among them share this one
   Program *fill = nullptr;
   bool use_graph = true;
   bool tuned = false;            // candidates of the tunable kernels have been timed (or there are none)
@@ -91,6 +102,8 @@ struct PolyHipPlan {
     if (fill) program_destroy(fill);
     if (arena) runtime_free(arena);
     if (scratch_pool) runtime_free(scratch_pool);
+    if (side_scratch_pool) runtime_free(side_scratch_pool);
+    for (hipEvent_t e : events) if (e) (void)hipEventDestroy(e);
   }
 };
 
@@ -184,6 +197,49 @@ int enqueue_all(PolyHipPlan *plan) {
   return 0;
 }
 
+// The same launches under stream capture, with those marked on_side going to the second
+// stream: it joins the capture by waiting for an event recorded at the start of the main
+// sequence, every dependence between the two streams is an event recorded behind the
+// producer and waited for in front of the consumer (edges of the graph), and the main
+// stream waits for the last side launch before the capture ends.
+int enqueue_captured(PolyHipPlan *plan) {
+  hipStream_t main_s = (hipStream_t)runtime_stream(), side_s = (hipStream_t)runtime_side_stream();
+  if (!side_s) return enqueue_all(plan);
+  const size_t n = plan->units.size();
+  if (plan->events.size() != n + 2) plan->events.assign(n + 2, nullptr);
+  auto event = [&](size_t i) -> hipEvent_t {
+    if (!plan->events[i] && hipEventCreateWithFlags(&plan->events[i], hipEventDisableTiming) != hipSuccess) plan->events[i] = nullptr;
+    return plan->events[i];
+  };
+  int rc = 0;
+  hipEvent_t fork = event(n), join = event(n + 1);
+  if (!fork || !join || hipEventRecord(fork, main_s) != hipSuccess || hipStreamWaitEvent(side_s, fork, 0) != hipSuccess) rc = -1;
+  long last_side = -1;
+  for (size_t u = 0; u < n && rc == 0; u++) {
+    hipStream_t st = plan->on_side[u] ? side_s : main_s;
+    if (plan->wait_for[u] >= 0) {
+      hipEvent_t e = event((size_t)plan->wait_for[u]);
+      if (!e || hipStreamWaitEvent(st, e, 0) != hipSuccess) { rc = -1; break; }
+    }
+    runtime_launch_on(plan->on_side[u] ? (void *)side_s : nullptr);
+    if (launch_unit(plan, u) != 0) {
+      log_err("plan_run", "kernel %d failed to launch", plan->units[u].item);
+      rc = -1;
+      break;
+    }
+    if (plan->on_side[u]) last_side = (long)u;
+    if (plan->records[u]) {
+      hipEvent_t e = event(u);
+      if (!e || hipEventRecord(e, st) != hipSuccess) { rc = -1; break; }
+    }
+  }
+  runtime_launch_on(nullptr);
+  // (the side stream rejoins whatever happened, or the capture cannot end)
+  if (hipEventRecord(join, side_s) != hipSuccess || hipStreamWaitEvent(main_s, join, 0) != hipSuccess) rc = -1;
+  (void)last_side;
+  return rc;
+}
+
 }  // namespace
 
 extern "C" {
@@ -273,10 +329,39 @@ PolyHipPlan *poly_hip_compile_schedule(PolyCtx *ctx, const PolySchedule *s) {
   }
   plan_counter++;
 
+  const int n_units = (int)plan->units.size();
+  // Which launches may run beside the main sequence (what orders the two streams follows
+  // further down, once the intermediates have their places).
+  plan->on_side.assign((size_t)n_units, 0);
+  plan->wait_for.assign((size_t)n_units, -1);
+  plan->records.assign((size_t)n_units, 0);
+  if (!getenv("POLY_HIP_NO_SIDE_STREAM") && n_units > 1) {
+    auto threads_of = [](const LaunchSpec &l) {
+      return (uint64_t)l.grid[0] * l.grid[1] * l.grid[2] * l.block[0] * l.block[1] * l.block[2];
+    };
+    // The seeds are the small thread reductions; a small launch of any kind that reads what
+    // a side launch left (the cast of a column sum, the optimizer update of a bias) follows
+    // its producer, so that the main sequence does not wait for the chain one step later.
+    std::vector<char> side_wrote((size_t)s->n_buf_slots, 0);     // the slot's current contents come from a side launch
+    for (int ui = 0; ui < n_units; ui++) {
+      const Unit &u = plan->units[(size_t)ui];
+      const HipRunner *r = u.runner;
+      bool small = threads_of(r->rk.launch) <= 16384 && r->guards.empty() && r->rk.variants.size() < 2 && r->rk.pres_key.empty();
+      for (const RenderedKernel::Pre &pk : r->rk.pres) small = small && (r->rk.klass == KernelClass::THREAD_REDUCE || threads_of(pk.launch) <= 16384);
+      bool follows = false;
+      for (int sl : u.slots) follows = follows || side_wrote[(size_t)sl];
+      const bool side = small && (r->rk.klass == KernelClass::THREAD_REDUCE || follows);
+      if (side) { plan->on_side[(size_t)ui] = 1; plan->forked = true; }
+      for (int sl : u.writes) side_wrote[(size_t)sl] = side ? 1 : 0;
+    }
+    // (a plan that is mostly such launches is one chain of small steps: nothing to run beside)
+    int n_side = 0;
+    for (int ui = 0; ui < n_units; ui++) n_side += plan->on_side[(size_t)ui];
+    if (2 * n_side > n_units) { plan->on_side.assign((size_t)n_units, 0); plan->forked = false; }
+  }
   // ── lifetimes of intermediates in execution order ──────────────────────
   const int ns = s->n_buf_slots;
   std::vector<int> first((size_t)ns, -1), last((size_t)ns, -1);
-  const int n_units = (int)plan->units.size();
   for (int step = 0; step < n_units; step++) {
     for (int sl : plan->units[(size_t)step].slots) {
       if (sl < 0 || sl >= ns) { log_err("compile_schedule", "bad slot index %d", sl); return nullptr; }
@@ -284,6 +369,19 @@ PolyHipPlan *poly_hip_compile_schedule(PolyCtx *ctx, const PolySchedule *s) {
       last[(size_t)sl] = step;
     }
   }
+  // What a side launch reads or writes stays where it is for a while after its turn in the
+  // sequence: the main sequence runs on meanwhile, and a later launch given the same bytes
+  // would have to wait for it.  Small buffers (column sums, their casts) keep their place
+  // for good, larger ones for the next 32 launches.
+  if (plan->forked)
+    for (int step = 0; step < n_units; step++) {
+      if (!plan->on_side[(size_t)step]) continue;
+      for (int sl : plan->units[(size_t)step].slots) {
+        if (!s->buf_slots[sl].is_intermediate) continue;
+        const int keep = s->buf_slots[sl].nbytes <= 65536 ? n_units : std::min(n_units, step + 32);
+        last[(size_t)sl] = std::max(last[(size_t)sl], keep);
+      }
+    }
   // ── place intermediates in one arena; overlapping lifetimes never share ──
   struct Placed { size_t off, size; int first, last; };
   std::vector<Placed> placed;
@@ -371,19 +469,86 @@ PolyHipPlan *poly_hip_compile_schedule(PolyCtx *ctx, const PolySchedule *s) {
         fprintf(stderr, "polygrad: compile_schedule: launch %d reads what the first stage of launch %d leaves\n", ui, it->second);
     }
   }
-  // one scratch pool for all other two-stage kernels: the largest need
-  {
-    int users = 0;
+  // What orders the two streams.
+  if (plan->forked) {
+    // what a launch touches, as byte ranges: intermediates by their place in the arena (two
+    // slots that share bytes are one resource), every other slot as a range of its own
+    struct Span { uint64_t lo, hi; bool w; };
+    std::vector<std::vector<Span>> spans((size_t)n_units);
     for (int ui = 0; ui < n_units; ui++) {
       const Unit &u = plan->units[(size_t)ui];
-      if (u.runner->rk.scratch_bytes > 0 && !keeps_scratch[(size_t)ui]) { users++; plan->scratch_bytes = std::max(plan->scratch_bytes, u.runner->rk.scratch_bytes); }
+      for (int sl : u.slots) {
+        const bool in_arena = s->buf_slots[sl].is_intermediate && !internal[(size_t)sl];
+        const uint64_t lo = in_arena ? (uint64_t)plan->slot_off[(size_t)sl] : ((uint64_t)(sl + 1) << 44);
+        const uint64_t size = (uint64_t)std::max<int64_t>(s->buf_slots[sl].nbytes, 4);
+        bool w = std::find(u.writes.begin(), u.writes.end(), sl) != u.writes.end();
+        for (int f : plan->fills_before[(size_t)ui]) w = w || f == sl;
+        spans[(size_t)ui].push_back({lo, lo + size, w});
+      }
+    }
+    auto conflict = [&](int a, int b) {
+      for (const Span &x : spans[(size_t)a])
+        for (const Span &y : spans[(size_t)b])
+          if ((x.w || y.w) && x.lo < y.hi && y.lo < x.hi) return true;
+      return false;
+    };
+    int synced[2] = {-1, -1};     // [stream]: the latest launch of the OTHER stream that this stream has waited for
+    for (int i = 0; i < n_units; i++) {
+      const int me = plan->on_side[(size_t)i];
+      for (int j = i - 1; j > synced[me]; j--) {
+        if (plan->on_side[(size_t)j] == me || !conflict(i, j)) continue;
+        plan->wait_for[(size_t)i] = j;
+        plan->records[(size_t)j] = 1;
+        synced[me] = j;
+        break;
+      }
+    }
+    if (getenv("POLY_HIP_DEBUG")) {
+      int ns = 0, nw = 0;
+      for (int i = 0; i < n_units; i++) { ns += plan->on_side[(size_t)i]; nw += plan->wait_for[(size_t)i] >= 0; }
+      fprintf(stderr, "polygrad: compile_schedule: %d of %d launches on the second stream, %d waits between the streams\n", ns, n_units, nw);
+      // every pair of launches on different streams that touch the same bytes, one of them
+      // writing, must be ordered by the waits (checked here from scratch, pair by pair)
+      {
+        std::vector<int> seen_other((size_t)n_units, -1);   // latest launch of the other stream known to be over when i starts
+        int last_on[2] = {-1, -1};
+        long long unordered = 0, pairs = 0;
+        for (int i = 0; i < n_units; i++) {
+          const int me = plan->on_side[(size_t)i];
+          int so = last_on[me] >= 0 ? seen_other[(size_t)last_on[me]] : -1;
+          if (plan->wait_for[(size_t)i] >= 0) so = std::max(so, plan->wait_for[(size_t)i]);
+          seen_other[(size_t)i] = so;
+          last_on[me] = i;
+          for (int j = 0; j < i; j++)
+            if (plan->on_side[(size_t)j] != me && conflict(i, j)) { pairs++; if (j > so) unordered++; }
+        }
+        fprintf(stderr, "polygrad: compile_schedule: %lld pairs of launches across the streams share bytes, %lld of them unordered\n", pairs, unordered);
+      }
+    }
+  }
+  // one scratch pool for all other two-stage kernels of a stream: the largest need
+  {
+    int users = 0, side_users = 0;
+    size_t side_bytes = 0;
+    for (int ui = 0; ui < n_units; ui++) {
+      const Unit &u = plan->units[(size_t)ui];
+      if (u.runner->rk.scratch_bytes == 0 || keeps_scratch[(size_t)ui]) continue;
+      if (plan->on_side[(size_t)ui]) { side_users++; side_bytes = std::max(side_bytes, u.runner->rk.scratch_bytes); }
+      else { users++; plan->scratch_bytes = std::max(plan->scratch_bytes, u.runner->rk.scratch_bytes); }
     }
     if (users > 1) {
       plan->scratch_pool = runtime_alloc(plan->scratch_bytes);
       if (!plan->scratch_pool) return nullptr;
       for (int ui = 0; ui < n_units; ui++)
-        if (!keeps_scratch[(size_t)ui]) runner_share_scratch(plan->units[(size_t)ui].runner, plan->scratch_pool);
+        if (!keeps_scratch[(size_t)ui] && !plan->on_side[(size_t)ui]) runner_share_scratch(plan->units[(size_t)ui].runner, plan->scratch_pool);
     }
+    if (side_users > 1) {
+      plan->side_scratch_pool = runtime_alloc(side_bytes);
+      if (!plan->side_scratch_pool) return nullptr;
+      for (int ui = 0; ui < n_units; ui++)
+        if (!keeps_scratch[(size_t)ui] && plan->on_side[(size_t)ui]) runner_share_scratch(plan->units[(size_t)ui].runner, plan->side_scratch_pool);
+    }
+    plan->kept_scratch_bytes += side_bytes;
     // a lone user owns its scratch memory; it must exist before the launches are captured
     for (Unit &u : plan->units) if (runner_ensure_scratch(u.runner) != 0) return nullptr;
   }
@@ -581,7 +746,18 @@ int poly_hip_plan_run(PolyHipPlan *plan, void **slot_data, int n_slots, const Po
     plan->use_graph = false;
     return enqueue_all(plan);
   }
-  int rc = enqueue_all(plan);
+  // (the order between the two streams was worked out with every bound buffer a resource
+  // of its own: two bound buffers that share bytes put everything on one stream)
+  bool disjoint = true;
+  if (plan->forked) {
+    std::vector<std::pair<uintptr_t, uintptr_t>> ext;
+    for (int i = 0; i < plan->sched->n_buf_slots; i++)
+      if (!plan->sched->buf_slots[i].is_intermediate && plan->slot_ptr[(size_t)i])
+        ext.push_back({(uintptr_t)plan->slot_ptr[(size_t)i], (uintptr_t)plan->slot_ptr[(size_t)i] + (uintptr_t)std::max<int64_t>(plan->sched->buf_slots[i].nbytes, 4)});
+    std::sort(ext.begin(), ext.end());
+    for (size_t i = 1; i < ext.size(); i++) if (ext[i].first < ext[i - 1].second) disjoint = false;
+  }
+  int rc = plan->forked && disjoint ? enqueue_captured(plan) : enqueue_all(plan);
   hipError_t e = hipStreamEndCapture(stream, &ge.graph);
   if (rc != 0 || e != hipSuccess || !ge.graph) {
     if (ge.graph) (void)hipGraphDestroy(ge.graph);
@@ -736,6 +912,12 @@ void *poly_hip_plan_slot_ptr(const PolyHipPlan *plan, int slot) {
 }
 
 void poly_hip_plan_set_graph(PolyHipPlan *plan, int enabled) { if (plan) plan->use_graph = enabled != 0; }
+int poly_hip_plan_side_launches(const PolyHipPlan *plan) {
+  int n = 0;
+  if (plan) for (char c : plan->on_side) n += c;
+  return n;
+}
+
 size_t poly_hip_plan_workspace_bytes(const PolyHipPlan *plan) { return plan ? plan->arena_bytes + plan->scratch_bytes + plan->kept_scratch_bytes : 0; }
 
 }  // extern "C"

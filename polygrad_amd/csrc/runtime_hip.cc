@@ -36,6 +36,8 @@ struct Runtime {
   bool ok = false;
   int device = 0;
   hipStream_t stream = nullptr;
+  hipStream_t side = nullptr;          // second stream of a plan's captured graphs, made on first use
+  hipStream_t launch_on = nullptr;     // where program_launch puts kernels when not the main stream
   std::map<uint64_t, std::weak_ptr<Module>> modules;   // keyed by source hash
   std::map<uint64_t, std::vector<char>> code_cache;    // compiled, not yet loaded
 };
@@ -141,6 +143,15 @@ int runtime_init() {
 }
 
 void *runtime_stream() { return runtime_init() == 0 ? (void *)rt().stream : nullptr; }
+
+void *runtime_side_stream() {
+  if (runtime_init() != 0) return nullptr;
+  Runtime &r = rt();
+  if (!r.side && !check(hipStreamCreateWithFlags(&r.side, hipStreamNonBlocking), "hipStreamCreate")) r.side = nullptr;
+  return (void *)r.side;
+}
+
+void runtime_launch_on(void *stream) { rt().launch_on = (hipStream_t)stream; }
 
 void *runtime_alloc(size_t nbytes) {
   if (runtime_init() != 0) return nullptr;
@@ -256,7 +267,7 @@ std::shared_ptr<void> runtime_table(const std::string &source, const std::string
 int program_launch(Program *p, void **kernel_args, const LaunchSpec &ls) {
   if (!p || runtime_init() != 0) return -1;
   hipError_t e = hipModuleLaunchKernel(p->fn, ls.grid[0], ls.grid[1], ls.grid[2], ls.block[0], ls.block[1],
-                                       ls.block[2], ls.lds_bytes, rt().stream, kernel_args, nullptr);
+                                       ls.block[2], ls.lds_bytes, rt().launch_on ? rt().launch_on : rt().stream, kernel_args, nullptr);
   return check(e, "hipModuleLaunchKernel") ? 0 : -1;
 }
 

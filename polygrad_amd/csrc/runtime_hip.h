@@ -13,6 +13,11 @@ struct Program;  // one kernel entry inside a loaded (shared) module
 
 int runtime_init();
 void *runtime_stream();
+// A second stream (same priority) for launches that a plan's captured graph lets run beside
+// the main sequence, and the switch that sends the following program_launch calls to it
+// (nullptr: back to the main stream).
+void *runtime_side_stream();
+void runtime_launch_on(void *stream);
 void *runtime_alloc(size_t nbytes);
 void runtime_free(void *p);
 // kind: 0 host->device, 1 device->host, 2 device->device; returns once done

@@ -147,6 +147,10 @@ class HipPlan:
     def workspace_bytes(self):
         return int(self.lib.poly_hip_plan_workspace_bytes(self.handle))
 
+    def side_launches(self):
+        """Launches that the plan's captured graph runs on a second stream."""
+        return int(self.lib.poly_hip_plan_side_launches(self.handle))
+
     def slot_ptr(self, slot):
         return self.lib.poly_hip_plan_slot_ptr(self.handle, slot)
 

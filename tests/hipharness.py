@@ -111,6 +111,7 @@ def run_hip(c, sink, arrays, graph=True, repeats=1):
         plan.run(dev)
     out = {owner[i]: from_device(dev[i], arrays[owner[i]].dtype) for i in owner}
     info = plan.kernel_info()
+    run_hip.side_launches = plan.side_launches()      # of the last plan run (tests of the second stream read it)
     plan.close()
     c.L.poly_schedule_free(sched)
     return out, info

@@ -143,3 +143,32 @@ def test_gpt2_multi_block_train_step_matches_reference(n_blocks):
     info = check_train_step(c, bufs, sink, B, T, V, lr, graphs.train_param_names(n_blocks), 100 * n_blocks)
     c.close()
     assert sum("3 slabs of one output range" in k["desc"] for k in info) == n_blocks
+
+
+def test_launches_on_the_second_stream_change_nothing():
+    """The in-order adders of the bf16 column sums (one thread per output, a chain of 4096
+    dependent additions each) run on a second stream of the captured graph, ordered against
+    the main sequence by the buffers they share.  Three replays of the graph must give what
+    the single-stream graph gives, bit for bit (the optimizer state advances with every run,
+    so a launch that ran too early or too late would show)."""
+    import os
+    # (large enough for most launches to fill more than a quarter of the chip: a plan of
+    # small launches only is one chain and stays on one stream)
+    B, T, D, H, V, lr = 4, 256, 256, 4, 1000, 3e-4
+    outs = []
+    for single in (False, True):
+        c = R.Ctx()
+        bufs, sink = graphs.gpt2_block_train_step(c, B, T, D, H, V, lr=lr)
+        arrays = graphs.gpt2_block_train_inputs(bufs, B, T, V)
+        if single:
+            os.environ["POLY_HIP_NO_SIDE_STREAM"] = "1"
+        try:
+            got, info = run_hip(c, sink, arrays, repeats=3)
+        finally:
+            os.environ.pop("POLY_HIP_NO_SIDE_STREAM", None)
+        n_side = run_hip.side_launches
+        assert (n_side == 0) if single else (n_side >= 4), n_side
+        outs.append({name: got[t] for name, t in bufs.items()})
+        c.close()
+    for name in outs[0]:
+        assert outs[0][name].tobytes() == outs[1][name].tobytes(), name
