@@ -115,7 +115,9 @@ int poly_hip_check_index_simplification(PolyUOp *scheduled_root, int samples);
  * intermediates that are dead share memory, only the intermediates that their
  * producers leave holes in are cleared per run (poly_hip_unwritten_slots), launches are
  * asynchronous on one stream and the launch sequence is replayed from a
- * hipGraph when the bound pointers repeat. */
+ * hipGraph when the bound pointers repeat (in that graph, small launches that are
+ * chains of dependent steps may run on a second branch beside the others, ordered by
+ * the buffers they share: poly_hip_plan_side_launches). */
 typedef struct PolyHipPlan PolyHipPlan;
 PolyHipPlan *poly_hip_compile_schedule(PolyCtx *ctx, const PolySchedule *schedule);
 /* slot_data[i]: device pointer for every external slot (ignored for

@@ -11,7 +11,8 @@
 //   * kernels are enqueued on one stream with no per-kernel synchronisation and
 //     no per-launch allocation (src/exec_plan.c:590-607 does both);
 //   * the launch sequence is captured into a hipGraph and replayed while the
-//     bound pointers and variable values repeat;
+//     bound pointers and variable values repeat; in the graph, small launches that are
+//     chains of dependent steps run on a second stream beside the main sequence;
 //   * kernel groups that fusion.cc recognises run as one launch and their
 //     intermediates get no memory at all.
 #include <hip/hip_runtime.h>
