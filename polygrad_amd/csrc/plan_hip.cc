@@ -215,7 +215,6 @@ int enqueue_captured(PolyHipPlan *plan) {
   int rc = 0;
   hipEvent_t fork = event(n), join = event(n + 1);
   if (!fork || !join || hipEventRecord(fork, main_s) != hipSuccess || hipStreamWaitEvent(side_s, fork, 0) != hipSuccess) rc = -1;
-  long last_side = -1;
   for (size_t u = 0; u < n && rc == 0; u++) {
     hipStream_t st = plan->on_side[u] ? side_s : main_s;
     if (plan->wait_for[u] >= 0) {
@@ -228,7 +227,6 @@ int enqueue_captured(PolyHipPlan *plan) {
       rc = -1;
       break;
     }
-    if (plan->on_side[u]) last_side = (long)u;
     if (plan->records[u]) {
       hipEvent_t e = event(u);
       if (!e || hipEventRecord(e, st) != hipSuccess) { rc = -1; break; }
@@ -237,7 +235,6 @@ int enqueue_captured(PolyHipPlan *plan) {
   runtime_launch_on(nullptr);
   // (the side stream rejoins whatever happened, or the capture cannot end)
   if (hipEventRecord(join, side_s) != hipSuccess || hipStreamWaitEvent(main_s, join, 0) != hipSuccess) rc = -1;
-  (void)last_side;
   return rc;
 }
 
