@@ -908,6 +908,10 @@ static bool match_row_chain_impl(const Sched &sc, int a_item, const std::vector<
       for (auto &kv : ph.m.preset) if (kv.second.find("[it]") != std::string::npos) reads_row = true;
       if (reads_row) V = row_V;   // positions must line up with the phase that made the row
       while (V > 1 && (R % V != 0 || R < (int64_t)G * V)) V /= 2;
+      // a row that half the vector width deals out evenly (768 = 3 x 64 x 4, against one
+      // and a half steps of 64 x 8) is walked that way: no step with half the lanes idle
+      // (LayerNorm of 8192 x 768: 12.3 -> 11.2 us)
+      if (!reads_row && V >= 8 && R % ((int64_t)G * V) != 0 && R % ((int64_t)G * V / 2) == 0) V /= 2;
       // long rows of an extent that is no multiple of the vector width (a vocabulary of
       // 50257): vector accesses at element alignment and a scalar tail
       if (V == 1 && !reads_row && !ph.keeps_row && !getenv("POLY_HIP_NO_RAGGED_VEC")) {
