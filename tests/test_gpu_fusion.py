@@ -226,3 +226,32 @@ def test_lookup_table_epilogue_is_bit_identical_to_the_arithmetic():
     want = run_ref(c, sink, arrays)
     c.close()
     assert_close(R.bf16_bits_to_f32(with_table[O]), R.bf16_bits_to_f32(want[O]), rtol=2e-2, atol=2e-2, what="matmul + GELU vs reference")
+
+
+def test_table_epilogue_on_both_launches_of_a_product_with_leftover_columns():
+    """8192 x 2304 with a GELU behind it: the columns from 2048 on are a launch of small tiles
+    of their own, and both launches serve the table's middle from their LDS.  Every switch
+    (one launch, table in memory only, no table) must give the same bits."""
+    m, n, k = 8192, 2304, 64
+    g = np.random.default_rng(77)
+    c = R.Ctx()
+    A = c.buffer((m, k), R.BF16, name="A")
+    W = c.buffer((k, n), R.BF16, name="W")
+    O = c.buffer((m, n), R.BF16, name="O")
+    y = A.cast(R.F32).dot(W.cast(R.F32)).cast(R.BF16).contiguous()
+    sink = c.sink((O, y.gelu()))
+    a = g.normal(0, 1.0, (m, k)).astype(np.float32)
+    a[5] = 0.0
+    a[4000:4003] *= 1e3
+    arrays = {A: R.f32_to_bf16_bits(a.reshape(-1)), W: R.f32_to_bf16_bits(g.normal(0, 0.2, k * n).astype(np.float32)),
+              O: np.zeros(m * n, np.uint16)}
+    got, info = run_hip(c, sink, arrays)
+    assert any("lookup table" in kk["desc"] and "columns from 2048 on by a launch of" in kk["desc"] for kk in info), [kk["desc"] for kk in info]
+    for switch in ("POLY_HIP_NO_TAIL_LAUNCH", "POLY_HIP_NO_LUT_WINDOW", "POLY_HIP_NO_LUT"):
+        os.environ[switch] = "1"
+        try:
+            other, _ = run_hip(c, sink, arrays)
+        finally:
+            del os.environ[switch]
+        assert got[O].tobytes() == other[O].tobytes(), switch
+    c.close()
