@@ -1855,6 +1855,212 @@ static bool match_attention(const Sched &sc, int s_item, const std::vector<char>
   return true;
 }
 
+// ── pointwise kernels over the same positions ─────────────────────────────────
+//
+// An optimizer step reaches the backend as four kernels per parameter (reference:
+// src/instance.c:1152-1224): the new parameter into a temporary, the copy back, the two
+// moments -- each walks the same N positions with one flat range and reads and writes
+// element p of its buffers only.  Run back to back they move 13 streams of N floats; one
+// launch in which a thread does all four for its positions moves 7 (p, m, v, g in; p, m, v
+// out) and never materialises the temporary.  In general: consecutive kernels of the
+// schedule, each without a reduction and with a single ungated store at the flat position,
+// all of the same extent, whose loads are at the flat position or at a fixed index, and no
+// buffer written twice.  A member's load of what an earlier member stored takes that
+// value; a load of what a later member will store reads memory, and every store happens
+// after every load of the thread.
+static bool match_pointwise_group(const Sched &sc, int a_item, const std::vector<char> &taken, FusedGroup *out) {
+  const PolySchedule *s = sc.s;
+  if (getenv("POLY_HIP_NO_POINTWISE_GROUPS")) return false;
+  struct Pw { int item, ord, out_slot; };
+  auto flat_member = [&](int item, int64_t *extent, Pw *pw) {
+    const KernelGraph &g = sc.graphs[(size_t)item];
+    if (!g.reduces.empty() || g.stores.size() != 1 || g.stores[0].gate >= 0 || !g.vars.empty()) return false;
+    if (g.stores[0].ranges.size() != 1 || g.ranges.size() != 1) return false;
+    const int ord = g.stores[0].ranges[0];
+    auto is_flat = [&](const Lin &l) {
+      if (l.c0 != 0 || l.terms.size() != 1 || l.terms[0].coef != 1) return false;
+      const Atom &a = g.atoms[(size_t)l.terms[0].atom];
+      return a.kind == Atom::RANGE && g.range_ord.at(a.node) == ord;
+    };
+    const int li = g.n(g.n(g.stores[0].index).src[1]).lin;
+    if (li < 0 || !is_flat(g.lins[(size_t)li])) return false;
+    if (g.n(g.stores[0].value).dt != g.n(g.stores[0].param).dt) return false;
+    for (size_t p = 0; p < g.params.size(); p++) {
+      std::vector<LoadRef> lds;
+      if (!loads_of(g, (int)p, &lds)) return false;
+      for (const LoadRef &l : lds) {
+        const Lin &lin = g.lins[(size_t)l.lin];
+        if (!is_flat(lin) && !lin.terms.empty()) return false;
+      }
+    }
+    *extent = g.ranges[(size_t)ord].extent;
+    *pw = {item, ord, sc.slot(item, g.param_slot(g.stores[0].param))};
+    return *extent > 0 && *extent < 2147483647LL;
+  };
+  int64_t E = 0;
+  Pw first;
+  if (!flat_member(a_item, &E, &first)) return false;
+  std::vector<Pw> members{first};
+  std::set<int> touched;
+  for (int i = 0; i < s->items[a_item].n_buf_slots; i++) touched.insert(s->items[a_item].buf_slot_indices[i]);
+  for (int st = sc.step_of[(size_t)a_item] + 1; st < s->n_items && members.size() < 8; st++) {
+    const int k = s->exec_order[st];
+    int64_t e2 = 0;
+    Pw pw;
+    if (taken[(size_t)k] || !flat_member(k, &e2, &pw) || e2 != E) break;
+    bool shares = false;
+    for (int i = 0; i < s->items[k].n_buf_slots; i++) shares = shares || touched.count(s->items[k].buf_slot_indices[i]);
+    if (!shares) break;
+    bool twice = false;
+    for (const Pw &m : members) twice = twice || m.out_slot == pw.out_slot;
+    if (twice) break;
+    for (int i = 0; i < s->items[k].n_buf_slots; i++) touched.insert(s->items[k].buf_slot_indices[i]);
+    members.push_back(pw);
+  }
+  if (members.size() < 2) return false;
+  // what the group writes it may only read at the flat position (a fixed index would be
+  // another thread's element)
+  for (const Pw &w : members)
+    for (const Pw &m : members) {
+      const KernelGraph &g = sc.graphs[(size_t)m.item];
+      const int p = sc.param_of(m.item, w.out_slot);
+      if (p < 0) continue;
+      std::vector<LoadRef> lds;
+      loads_of(g, p, &lds);
+      for (const LoadRef &l : lds) if (g.lins[(size_t)l.lin].terms.empty()) return false;
+    }
+  // a slot is internal when the group writes it and nobody outside ever touches it
+  std::set<int> in_group;
+  for (const Pw &m : members) in_group.insert(m.item);
+  std::set<int> internal;
+  for (const Pw &m : members) {
+    if (!s->buf_slots[m.out_slot].is_intermediate) continue;
+    bool outside = false;
+    for (int r : sc.readers[(size_t)m.out_slot]) outside = outside || !in_group.count(r);
+    for (int w : sc.writers[(size_t)m.out_slot]) outside = outside || !in_group.count(w);
+    if (!outside) internal.insert(m.out_slot);
+  }
+  // every buffer position must hold numel == E elements for the flat index to mean the same in all members
+  for (int sl : touched) {
+    bool flat_use = false;
+    for (const Pw &m : members) {
+      const KernelGraph &g = sc.graphs[(size_t)m.item];
+      const int p = sc.param_of(m.item, sl);
+      if (p < 0) continue;
+      std::vector<LoadRef> lds;
+      loads_of(g, p, &lds);
+      for (const LoadRef &l : lds) flat_use = flat_use || !g.lins[(size_t)l.lin].terms.empty();
+      if (m.out_slot == sl) flat_use = true;
+    }
+    if (flat_use && s->buf_slots[sl].numel < E) return false;
+  }
+  std::vector<int> arg_slots;
+  for (const Pw &m : members)
+    for (int i = 0; i < s->items[m.item].n_buf_slots; i++) {
+      const int sl = s->items[m.item].buf_slot_indices[i];
+      if (!internal.count(sl) && std::find(arg_slots.begin(), arg_slots.end(), sl) == arg_slots.end()) arg_slots.push_back(sl);
+    }
+  auto arg_of = [&](int sl) { return (int)(std::find(arg_slots.begin(), arg_slots.end(), sl) - arg_slots.begin()); };
+  // vector width: 16 bytes of the widest element touched at the flat position
+  int maxsz = 1;
+  std::map<int, DT> slot_dt;
+  std::set<int> written;
+  for (const Pw &m : members) {
+    const KernelGraph &g = sc.graphs[(size_t)m.item];
+    for (size_t p = 0; p < g.params.size(); p++) {
+      maxsz = std::max(maxsz, dt_size(g.params[p].dt));
+      slot_dt[sc.slot(m.item, (int)p)] = g.params[p].dt;
+    }
+    written.insert(m.out_slot);
+  }
+  int V = std::max(1, 16 / maxsz);
+  while (V > 1 && E % V != 0) V /= 2;
+  // the members as functions of the flat position (passed as `m`)
+  std::string code, body;
+  std::map<int, std::string> value_of_slot;   // what the group has stored so far, by slot
+  std::set<int> read_from_memory;
+  double bytes = 0;
+  for (size_t mi = 0; mi < members.size(); mi++) {
+    const Pw &pw = members[mi];
+    const KernelGraph &g = sc.graphs[(size_t)pw.item];
+    Member m;
+    m.item = pw.item;
+    m.range_expr[pw.ord] = "m";
+    std::string lead, lead_call;
+    for (size_t p = 0; p < g.params.size(); p++) {
+      const int sl = sc.slot(pw.item, (int)p);
+      std::vector<LoadRef> lds;
+      loads_of(g, (int)p, &lds);
+      if (lds.empty()) continue;
+      if (!value_of_slot.count(sl)) { read_from_memory.insert(sl); continue; }
+      const std::string nm = strf("fw%zu", p);
+      for (const LoadRef &l : lds) {
+        if (g.lins[(size_t)l.lin].terms.empty()) return false;     // a fixed index into what the group itself writes
+        m.preset[l.node] = nm;
+      }
+      lead += strf("%s%s %s", lead.empty() ? "" : ", ", dt_cname(g.params[p].dt), nm.c_str());
+      lead_call += strf("%s%s", lead_call.empty() ? "" : ", ", value_of_slot[sl].c_str());
+    }
+    if (!internal_loads_replaced(sc, m, internal, -1)) return false;
+    if (lead.empty()) { lead = "int poly_unused"; lead_call = "0"; }
+    const std::string fn = strf("poly_pw_%zu", mi);
+    const DT odt = g.n(g.stores[0].value).dt;
+    if (!emit_member_fn(sc, m, "", fn.c_str(), dt_cname(odt), lead, g.stores[0].value, {}, false, false, &code)) return false;
+    std::string args;
+    for (size_t p = 0; p < g.params.size(); p++) {
+      const int sl = sc.slot(pw.item, (int)p);
+      if (p) args += ", ";
+      if (internal.count(sl)) args += strf("(%s%s*)0", g.params[p].written ? "" : "const ", dt_cname(g.params[p].dt));
+      else args += strf("fa%d", arg_of(sl));
+    }
+    body += strf("    o%zu[u] = %s(%s, pos + u, 0, 0, %s);\n", mi, fn.c_str(), lead_call.c_str(), args.c_str());
+    value_of_slot[pw.out_slot] = strf("o%zu[u]", mi);
+  }
+  std::string sig;
+  for (size_t j = 0; j < arg_slots.size(); j++) {
+    const int sl = arg_slots[j];
+    if (j) sig += ", ";
+    // (a buffer the group both reads and writes is not declared restrict)
+    if (written.count(sl)) sig += strf("%s* fa%zu", dt_cname(slot_dt[sl]), j);
+    else sig += strf("const %s* __restrict__ fa%zu", dt_cname(slot_dt[sl]), j);
+    // (a buffer updated in place moves twice: in and out)
+    bytes += (double)s->buf_slots[sl].nbytes * ((read_from_memory.count(sl) ? 1 : 0) + (written.count(sl) ? 1 : 0));
+  }
+  std::string src = std::string(hip_prelude()) + code;
+  src += strf("extern \"C\" __global__ void __launch_bounds__(256) poly_k(%s) {\n", sig.c_str());
+  src += strf("  const long long pos_ll = ((long long)blockIdx.x * 256 + threadIdx.x) * %d;\n  if (pos_ll >= %lldll) return;\n  const int pos = (int)pos_ll;\n", V, (long long)E);
+  for (size_t mi = 0; mi < members.size(); mi++)
+    src += strf("  %s o%zu[%d];\n", dt_cname(sc.graphs[(size_t)members[mi].item].n(sc.graphs[(size_t)members[mi].item].stores[0].value).dt), mi, V);
+  src += strf("#pragma unroll\n  for (int u = 0; u < %d; u++) {\n", V) + body + "  }\n";
+  for (size_t mi = 0; mi < members.size(); mi++) {
+    const Pw &pw = members[mi];
+    if (internal.count(pw.out_slot)) continue;
+    const char *tn = dt_cname(slot_dt[pw.out_slot]);
+    src += strf("  { poly_vec<%s, %d> st; for (int u = 0; u < %d; u++) st.v[u] = o%zu[u]; poly_vstore<%s, %d>(fa%d + pos, st); }\n", tn, V, V, mi, tn, V,
+                arg_of(pw.out_slot));
+  }
+  src += "}\n";
+  out->items.clear();
+  for (const Pw &m : members) out->items.push_back(m.item);
+  out->launch_item = members.back().item;
+  out->internal_slots.assign(internal.begin(), internal.end());
+  out->arg_slots = arg_slots;
+  RenderedKernel &rk = out->rk;
+  rk = RenderedKernel();
+  rk.source = src;
+  rk.entry = "poly_k";
+  rk.launch.grid[0] = (unsigned)((E / V + 255) / 256);
+  rk.launch.block[0] = 256;
+  rk.klass = KernelClass::ELEMENTWISE;
+  rk.strategy = strf("%zu pointwise kernels over the same %lld positions as one, vec%d, %zu buffers never written out", members.size(), (long long)E, V,
+                     internal.size());
+  rk.n_params = (int)arg_slots.size();
+  rk.n_vars = 0;
+  rk.bytes = bytes;
+  rk.flops = 0;
+  return true;
+}
+
 void find_fused_groups(const PolySchedule *s, const std::vector<KernelGraph> &graphs, std::vector<FusedGroup> *out) {
   out->clear();
   if (getenv("POLY_HIP_NO_FUSION")) return;
@@ -1881,6 +2087,15 @@ void find_fused_groups(const PolySchedule *s, const std::vector<KernelGraph> &gr
     if (taken[(size_t)k] || graphs[(size_t)k].reduces.size() != 1) continue;
     FusedGroup fg;
     if (!match_attention(sc, k, taken, &fg) && !match_matmul_tail(sc, k, taken, &fg) && !match_row_chain(sc, k, taken, &fg)) continue;
+    for (int it : fg.items) taken[(size_t)it] = 1;
+    out->push_back(std::move(fg));
+  }
+  // what is left of the pointwise kernels, in runs over the same positions
+  for (int st = 0; st < s->n_items; st++) {
+    const int k = s->exec_order[st];
+    if (taken[(size_t)k] || !graphs[(size_t)k].reduces.empty()) continue;
+    FusedGroup fg;
+    if (!match_pointwise_group(sc, k, taken, &fg)) continue;
     for (int it : fg.items) taken[(size_t)it] = 1;
     out->push_back(std::move(fg));
   }
