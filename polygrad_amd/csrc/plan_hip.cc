@@ -502,7 +502,7 @@ PolyHipPlan *poly_hip_compile_schedule(PolyCtx *ctx, const PolySchedule *s) {
       }
     }
     // A wait between the streams costs a few microseconds of its own: worth it when the
-    // side launches run for long stretches without one (three waits for 970 launches in the
+    // side launches run for long stretches without one (two waits for 388 launches in the
     // 24-layer training step), not when every other side launch needs one (an MLP step of
     // 22 launches came out 13 % slower on two streams).
     {
