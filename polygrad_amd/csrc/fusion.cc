@@ -1886,6 +1886,7 @@ static bool match_pointwise_group(const Sched &sc, int a_item, const std::vector
     if (li < 0 || !is_flat(g.lins[(size_t)li])) return false;
     if (g.n(g.stores[0].value).dt != g.n(g.stores[0].param).dt) return false;
     for (size_t p = 0; p < g.params.size(); p++) {
+      if (!dt_is_float(g.params[p].dt)) return false;      // (float buffers only: what the vector helpers are used with elsewhere)
       std::vector<LoadRef> lds;
       if (!loads_of(g, (int)p, &lds)) return false;
       for (const LoadRef &l : lds) {
