@@ -168,9 +168,16 @@ bool match_matmul(const KernelGraph &g, MatmulMatch *mm, int *reject_line) {
   if (st.gate >= 0) MM_REJECT();
   const int red = g.reduces[0];
   const KNode &R = g.n(red);
-  if (reduce_op(R) != POLY_OP_ADD || R.dt != DT_F32 || R.src.size() != 2) MM_REJECT();
-  const int kr = g.range_ord.at(R.src[1]);
-  const int64_t K = g.ranges[(size_t)kr].extent;
+  if (reduce_op(R) != POLY_OP_ADD || R.dt != DT_F32 || (R.src.size() != 2 && R.src.size() != 3)) MM_REJECT();
+  const bool two_k = R.src.size() == 3;
+  if (two_k && getenv("POLY_HIP_MM_ONE_K_RANGE")) MM_REJECT();
+  const int kr = two_k ? -1 : g.range_ord.at(R.src[1]);
+  int64_t K = 1;
+  for (size_t i = 1; i < R.src.size(); i++) {
+    const int64_t e = g.ranges[(size_t)g.range_ord.at(R.src[i])].extent;
+    if (e <= 0 || K > 2147483647LL / e) MM_REJECT();
+    K *= e;
+  }
   if (K < 16) MM_REJECT();
   const KNode &mul = g.n(R.src[0]);
   if (mul.op != POLY_OP_MUL || mul.dt != DT_F32) MM_REJECT();
@@ -180,7 +187,28 @@ bool match_matmul(const KernelGraph &g, MatmulMatch *mm, int *reject_line) {
   for (const ParamInfo &p : g.params) if (p.numel >= ((int64_t)1 << 31)) MM_REJECT();
   const Lin &la = g.lins[(size_t)A.lin], &lb = g.lins[(size_t)B.lin];
   KSplit ka, kb;
-  if (!k_dependence(g, la, kr, K, &ka) || !k_dependence(g, lb, kr, K, &kb)) MM_REJECT();
+  if (!two_k) {
+    if (!k_dependence(g, la, kr, K, &ka) || !k_dependence(g, lb, kr, K, &kb)) MM_REJECT();
+  } else {
+    // Two reduce ranges p, q that both operands index plainly: k = p * |q| + q walks them as
+    // one depth of two levels (one level where the strides nest).  The sum runs over the
+    // same products in either nesting; the one whose inner stride in A is smaller is taken.
+    const int r1 = g.range_ord.at(R.src[1]), r2 = g.range_ord.at(R.src[2]);
+    const int64_t e1 = g.ranges[(size_t)r1].extent, e2 = g.ranges[(size_t)r2].extent;
+    KSplit a1, a2, b1, b2;
+    if (!k_dependence(g, la, r1, e1, &a1) || !k_dependence(g, la, r2, e2, &a2)) MM_REJECT();
+    if (!k_dependence(g, lb, r1, e1, &b1) || !k_dependence(g, lb, r2, e2, &b2)) MM_REJECT();
+    if (a1.kb != e1 || a2.kb != e2 || b1.kb != e1 || b2.kb != e2) MM_REJECT();   // plain uses only
+    const bool q_inner = std::llabs(a2.s_lo) <= std::llabs(a1.s_lo);
+    const int64_t ei = q_inner ? e2 : e1;
+    auto level = [&](const KSplit &p, const KSplit &q) {
+      const int64_t hi = q_inner ? p.s_lo : q.s_lo, lo = q_inner ? q.s_lo : p.s_lo;
+      return KSplit{ei, hi, lo};
+    };
+    ka = level(a1, a2);
+    kb = level(b1, b2);
+    if (ka.s_hi == ka.s_lo * ei && kb.s_hi == kb.s_lo * ei) { ka = {K, 0, ka.s_lo}; kb = {K, 0, kb.s_lo}; }
+  }
 
   // classify the END ranges of the store
   std::vector<Dim> md, nd, zd;
@@ -514,21 +542,27 @@ bool render_matmul(const MatmulMatch &mm, const MatmulEpilogue &ep, RenderedKern
   // relative to the 256x256 tile as measured on 8192^3).  Pick the smallest estimated
   // time = rounds over the chip * time of one tile.
   int BM = 128, BN = 128, WVM = 2, WVN = 2;
-  if (N <= 64) { BN = 64; BM = 256; WVM = 4; WVN = 1; }
-  else if (M <= 64) { BM = 64; BN = 256; WVM = 1; WVN = 4; }
-  else {
-    struct Cand { int bm, bn, wm, wn, per_cu; double thr; };
+  // (`alone`: the same with one workgroup on the CU, which is all a launch of at most 256
+  // tiles gives it: 4096x1024x4096 took 65 us on 256 tiles of 128x128 and 78 us on 128
+  // tiles of 128x256.)
+  auto pick_tile = [&](bool count_alone) {
+    struct Cand { int bm, bn, wm, wn, per_cu; double thr, alone; };
     // (128x256 before 256x128: equal by the estimate, 1-4 % faster when timed on the device)
-    static const Cand cands[] = {{256, 256, 4, 2, 1, 1.00}, {128, 256, 2, 4, 1, 0.84}, {256, 128, 4, 2, 1, 0.84}, {128, 128, 2, 2, 2, 0.80}};
+    static const Cand cands[] = {{256, 256, 4, 2, 1, 1.00, 1.00}, {128, 256, 2, 4, 1, 0.84, 0.84}, {256, 128, 4, 2, 1, 0.84, 0.84}, {128, 128, 2, 2, 2, 0.80, 0.52}};
     double best = 0;
     for (const Cand &c : cands) {
       if (!a_kc && M % 8) continue;
       double t = (double)((M + c.bm - 1) / c.bm) * (double)((N + c.bn - 1) / c.bn) * (double)Z;
       double rounds = std::ceil(t / (256.0 * c.per_cu));
       double est = rounds * (double)c.bm * c.bn / (c.thr / c.per_cu);
+      if (count_alone && t <= 256.0) est = (double)c.bm * c.bn / c.alone;
       if (best == 0 || est < best) { best = est; BM = c.bm; BN = c.bn; WVM = c.wm; WVN = c.wn; }
     }
-  }
+  };
+  const bool fixed_tile = N <= 64 || M <= 64;
+  if (N <= 64) { BN = 64; BM = 256; WVM = 4; WVN = 1; }
+  else if (M <= 64) { BM = 64; BN = 256; WVM = 1; WVN = 4; }
+  else pick_tile(false);
   if (const char *ov = getenv("POLY_HIP_MM_TILE")) {   // "BM,BN,WVM,WVN": tuning experiments
     int a, b2, c2, d2;
     if (sscanf(ov, "%d,%d,%d,%d", &a, &b2, &c2, &d2) == 4) { BM = a; BN = b2; WVM = c2; WVN = d2; }
@@ -542,18 +576,36 @@ bool render_matmul(const MatmulMatch &mm, const MatmulEpilogue &ep, RenderedKern
   // dealt to S workgroups, which leave fp32 partial results in scratch memory, and a second
   // kernel adds them in split order and runs the epilogue.  S minimises rounds over the
   // chip / S among the divisors of the K tile count that leave every part 64 tiles or more.
+  // A product of few tiles and moderate depth (no split by that rule) runs on the tile that is
+  // fastest with a CU to itself, and may then be split down to parts of 32 K tiles.
   int S = 1;
   size_t part_off = 0;
-  if (!getenv("POLY_HIP_NO_SPLIT_K") && !getenv("POLY_HIP_MM_NOEPI") && M > 64 && N > 64) {
+  auto pick_split = [&](int64_t min_part) {
     const int64_t t = ((M + BM - 1) / BM) * ((N + BN - 1) / BN) * Z, kt = K / BK;
     double best = 0.75;      // worth a second kernel only from a quarter of the time saved
+    S = 1;
     for (int s = 2; s <= 16 && t <= 128; s++) {
-      if (kt % s != 0 || kt / s < 64 || Z * s > 65535) continue;
+      if (kt % s != 0 || kt / s < min_part || Z * s > 65535) continue;
       const double r = std::ceil((double)(t * s) / 256.0) / (double)s;
       if (r < best) { best = r; S = s; }
     }
-    part_off = (ep.scratch_used + 255) / 256 * 256;
     if ((double)S * (double)Z * (double)M * (double)N * 4.0 > 1073741824.0) S = 1;
+  };
+  const bool may_split = !getenv("POLY_HIP_NO_SPLIT_K") && !getenv("POLY_HIP_MM_NOEPI") && M > 64 && N > 64;
+  if (may_split) pick_split(64);
+  if (S == 1 && !fixed_tile && !getenv("POLY_HIP_MM_TILE") && !getenv("POLY_HIP_MM_OLD_ESTIMATE")) {
+    pick_tile(true);
+    pipe = (BM * BN >= 256 * 256) ? 2 : 3;
+    if (const char *e = getenv("POLY_HIP_MM_PIPE")) pipe = atoi(e) == 2 ? 2 : 3;
+    if (may_split) pick_split(32);
+  }
+  if (may_split) {
+    const int64_t kt = K / BK;
+    if (const char *e = getenv("POLY_HIP_MM_KSPLIT")) {   // tuning experiments: a given split
+      const int s = atoi(e);
+      if (s >= 1 && s <= 64 && kt % s == 0 && Z * s <= 65535) S = s;
+    }
+    part_off = (ep.scratch_used + 255) / 256 * 256;
   }
   const std::string partials = ep.scratch_type.empty() ? std::string("poly_scratch") : strf("((float*)((char*)poly_scratch + %zuull))", part_off);
   const std::string signature = ep.signature + (S > 1 && ep.scratch_type.empty() ? ", float* poly_scratch" : "");

@@ -212,6 +212,19 @@ def matmul_bf16(c, m, n, k, transposed_b=False, batch=None, transposed_a=False):
     return A, Bm, O, sink
 
 
+def matmul_bf16_over_two_ranges(c, b, t, m, n, time_major_a=False):
+    """C[m, n] = sum over (b, t) of X[b, t, m] * Y[b, t, n]: the weight gradient of a linear
+    layer over a batch of sequences, as one REDUCE over two ranges.  time_major_a: X is
+    stored [t, b, m] and permuted in the graph, so its two reduce strides do not nest in
+    the order Y's do."""
+    X = c.buffer((t, b, m) if time_major_a else (b, t, m), R.BF16, name="A")
+    Y = c.buffer((b, t, n), R.BF16, name="B")
+    O = c.buffer((m, n), R.F32, name="C")
+    x = X.permute((1, 0, 2)) if time_major_a else X
+    p = x.cast(R.F32).reshape((b, t, m, 1)).expand((b, t, m, n)) * Y.cast(R.F32).reshape((b, t, 1, n)).expand((b, t, m, n))
+    return X, Y, O, c.sink((O, p.reduce_axes("ADD", (0, 1)).reshape((m, n))))
+
+
 def attention_bf16(c, batch=8, heads=12, ctx=1024, hd=64, mask_buffer=False, dt=None):
     """The attention block of gpt2_forward on its own: q, k, v as [B, T, H*hd] bf16 buffers
     (heads interleaved along the feature axis, as the qkv projection leaves them), additive

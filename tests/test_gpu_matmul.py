@@ -69,6 +69,31 @@ def test_matmul_bf16_deep_product_on_few_tiles_is_split_along_k(tb):
     assert float(np.abs(got[O].astype(np.float64) - got1[O]).max()) <= 2e-5 * float(np.abs(w).max())
 
 
+@pytest.mark.parametrize("b,t,m,n,tm", [(4, 64, 256, 384, False), (4, 64, 256, 384, True), (3, 64, 136, 200, False)])
+def test_matmul_bf16_reduce_over_two_ranges(b, t, m, n, tm):
+    """dW = X^T dY summed over batch and position: the REDUCE runs over two ranges.  Where
+    the strides of both operands nest they are one depth; where they do not (X stored time
+    major) the depth has two levels.  Either way the operands are read where they lie: no
+    launch that rewrites them first."""
+    c = R.Ctx()
+    g = np.random.default_rng(b * 1000 + m + tm)
+    X, Y, O, sink = graphs.matmul_bf16_over_two_ranges(c, b, t, m, n, time_major_a=tm)
+    arrays = {X: bf16(g, (b, t, m), 1.0), Y: bf16(g, (b, t, n), 1.0), O: np.zeros(m * n, np.float32)}
+    want = run_ref(c, sink, arrays)
+    got, info = run_hip(c, sink, arrays)
+    c.close()
+    assert len(info) == 1 and info[0]["klass"] == "matmul-mfma" and "planes" not in info[0]["desc"], [k_["desc"] for k_ in info]
+    bound = 1e-4 * float(np.abs(want[O]).mean())
+    assert_close(got[O], want[O], rtol=1e-4, atol=bound, what="two reduce ranges vs reference")
+    # the definition, in float64 (the products of bf16 values are exact there)
+    x = R.bf16_bits_to_f32(arrays[X]).astype(np.float64).reshape((t, b, m) if tm else (b, t, m))
+    if tm:
+        x = x.transpose(1, 0, 2)
+    y = R.bf16_bits_to_f32(arrays[Y]).astype(np.float64).reshape(b, t, n)
+    exact = np.einsum("btm,btn->mn", x, y)
+    assert float(np.abs(got[O].reshape(m, n) - exact).max()) <= 1e-5 * float(np.abs(exact).max()) + 1e-4 * float(np.abs(exact).mean())
+
+
 def test_matmul_broadcast_batch():
     c = R.Ctx()
     g = np.random.default_rng(11)
