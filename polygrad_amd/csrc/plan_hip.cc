@@ -19,6 +19,7 @@
 #include <unistd.h>
 
 #include <algorithm>
+#include <array>
 #include <cstdio>
 #include <cstdlib>
 #include <cstring>
@@ -78,17 +79,19 @@ struct PolyHipPlan {
   std::vector<std::vector<void *>> kargs;    // per unit: args array handed to runner_launch
   std::vector<std::vector<int>> var_vals;    // per unit: storage for var ints
   std::vector<PolyVarBinding> merged;
-  // Launches that a captured graph runs beside the main sequence, on a second stream: small
+  // Launches that a captured graph runs beside the main sequence, on further streams: small
   // launches whose time is a dependent chain, not throughput (the in-order adders of the
   // bf16 column sums: 1024 threads for 48 us each, 194 of them in a 24-layer training step).
-  // wait_for[u]: the latest launch on the other stream that u's buffers depend on (-1: none
-  // that an earlier wait does not already cover); records[u]: someone waits for u.
+  // on_side[u]: 0 = main sequence, k = side stream k - 1; waits[u]: launches on other streams
+  // that u's buffers depend on (those that an earlier wait of u's stream does not already
+  // cover); records[u]: someone waits for u.
   std::vector<char> on_side;
-  std::vector<int> wait_for;
+  std::vector<std::vector<int>> waits;
   std::vector<char> records;
-  std::vector<hipEvent_t> events;            // per launch (those with records), then fork and join
+  std::vector<hipEvent_t> events;            // per launch (those with records), then fork and one join per side stream
   bool forked = false;
-  void *side_scratch_pool = nullptr;         // the two-stage kernels among them share this one
+  int n_side_streams = 0;
+  void *side_scratch_pool[kSideStreams] = {nullptr, nullptr, nullptr};   // the two-stage kernels of a side stream share one
   Program *fill = nullptr;
   bool use_graph = true;
   bool tuned = false;            // candidates of the tunable kernels have been timed (or there are none)
@@ -103,7 +106,7 @@ struct PolyHipPlan {
     if (fill) program_destroy(fill);
     if (arena) runtime_free(arena);
     if (scratch_pool) runtime_free(scratch_pool);
-    if (side_scratch_pool) runtime_free(side_scratch_pool);
+    for (void *p : side_scratch_pool) if (p) runtime_free(p);
     for (hipEvent_t e : events) if (e) (void)hipEventDestroy(e);
   }
 };
@@ -198,30 +201,39 @@ int enqueue_all(PolyHipPlan *plan) {
   return 0;
 }
 
-// The same launches under stream capture, with those marked on_side going to the second
-// stream: it joins the capture by waiting for an event recorded at the start of the main
-// sequence, every dependence between the two streams is an event recorded behind the
-// producer and waited for in front of the consumer (edges of the graph), and the main
-// stream waits for the last side launch before the capture ends.
+// The same launches under stream capture, with those marked on_side going to the side
+// streams: each joins the capture by waiting for an event recorded at the start of the main
+// sequence, every dependence between two streams is an event recorded behind the producer
+// and waited for in front of the consumer (edges of the graph), and the main stream waits
+// for the last launch of every side stream before the capture ends.
 int enqueue_captured(PolyHipPlan *plan) {
-  hipStream_t main_s = (hipStream_t)runtime_stream(), side_s = (hipStream_t)runtime_side_stream();
-  if (!side_s) return enqueue_all(plan);
+  hipStream_t main_s = (hipStream_t)runtime_stream();
+  hipStream_t side_s[kSideStreams];
+  const int ns = plan->n_side_streams;
+  for (int k = 0; k < ns; k++) {
+    side_s[k] = (hipStream_t)runtime_side_stream(k);
+    if (!side_s[k]) return enqueue_all(plan);
+  }
   const size_t n = plan->units.size();
-  if (plan->events.size() != n + 2) plan->events.assign(n + 2, nullptr);
+  if (plan->events.size() != n + 1 + kSideStreams) plan->events.assign(n + 1 + kSideStreams, nullptr);
   auto event = [&](size_t i) -> hipEvent_t {
     if (!plan->events[i] && hipEventCreateWithFlags(&plan->events[i], hipEventDisableTiming) != hipSuccess) plan->events[i] = nullptr;
     return plan->events[i];
   };
   int rc = 0;
-  hipEvent_t fork = event(n), join = event(n + 1);
-  if (!fork || !join || hipEventRecord(fork, main_s) != hipSuccess || hipStreamWaitEvent(side_s, fork, 0) != hipSuccess) rc = -1;
+  hipEvent_t fork = event(n);
+  if (!fork || hipEventRecord(fork, main_s) != hipSuccess) rc = -1;
+  int joined = 0;       // side streams that are part of the capture
+  for (; joined < ns && rc == 0; joined++)
+    if (hipStreamWaitEvent(side_s[joined], fork, 0) != hipSuccess) { rc = -1; break; }
   for (size_t u = 0; u < n && rc == 0; u++) {
-    hipStream_t st = plan->on_side[u] ? side_s : main_s;
-    if (plan->wait_for[u] >= 0) {
-      hipEvent_t e = event((size_t)plan->wait_for[u]);
+    hipStream_t st = plan->on_side[u] ? side_s[plan->on_side[u] - 1] : main_s;
+    for (int w : plan->waits[u]) {
+      hipEvent_t e = event((size_t)w);
       if (!e || hipStreamWaitEvent(st, e, 0) != hipSuccess) { rc = -1; break; }
     }
-    runtime_launch_on(plan->on_side[u] ? (void *)side_s : nullptr);
+    if (rc != 0) break;
+    runtime_launch_on(plan->on_side[u] ? (void *)st : nullptr);
     if (launch_unit(plan, u) != 0) {
       log_err("plan_run", "kernel %d failed to launch", plan->units[u].item);
       rc = -1;
@@ -233,8 +245,11 @@ int enqueue_captured(PolyHipPlan *plan) {
     }
   }
   runtime_launch_on(nullptr);
-  // (the side stream rejoins whatever happened, or the capture cannot end)
-  if (hipEventRecord(join, side_s) != hipSuccess || hipStreamWaitEvent(main_s, join, 0) != hipSuccess) rc = -1;
+  // (the side streams rejoin whatever happened, or the capture cannot end)
+  for (int k = 0; k < joined; k++) {
+    hipEvent_t join = event(n + 1 + (size_t)k);
+    if (!join || hipEventRecord(join, side_s[k]) != hipSuccess || hipStreamWaitEvent(main_s, join, 0) != hipSuccess) rc = -1;
+  }
   return rc;
 }
 
@@ -331,30 +346,38 @@ PolyHipPlan *poly_hip_compile_schedule(PolyCtx *ctx, const PolySchedule *s) {
   // Which launches may run beside the main sequence (what orders the two streams follows
   // further down, once the intermediates have their places).
   plan->on_side.assign((size_t)n_units, 0);
-  plan->wait_for.assign((size_t)n_units, -1);
+  plan->waits.assign((size_t)n_units, std::vector<int>());
   plan->records.assign((size_t)n_units, 0);
+  // (chain_of: which seed a side launch follows; the chains are dealt to the side streams in
+  // turn once it is known how many streams pay, further down)
+  std::vector<int> chain_of((size_t)n_units, -1);
   if (!getenv("POLY_HIP_NO_SIDE_STREAM") && n_units > 1) {
     auto threads_of = [](const LaunchSpec &l) {
       return (uint64_t)l.grid[0] * l.grid[1] * l.grid[2] * l.block[0] * l.block[1] * l.block[2];
     };
-    // The seeds are the small thread reductions; a small launch of any kind that reads what
-    // a side launch left (the cast of a column sum, the optimizer update of a bias) follows
-    // its producer, so that the main sequence does not wait for the chain one step later.
-    std::vector<char> side_wrote((size_t)s->n_buf_slots, 0);     // the slot's current contents come from a side launch
+    // The seeds are the small thread reductions (each is one dependent chain on a handful of
+    // waves: several run side by side); a small launch of any kind that reads what a side
+    // launch left (the cast of a column sum, the optimizer update of a bias) follows its
+    // producer on the same stream, so that the main sequence does not wait for the chain one
+    // step later.
+    std::vector<int> side_wrote((size_t)s->n_buf_slots, 0);     // the chain (1-based) that the slot's current contents come from
+    int next = 0;
     for (int ui = 0; ui < n_units; ui++) {
       const Unit &u = plan->units[(size_t)ui];
       const HipRunner *r = u.runner;
       bool small = threads_of(r->rk.launch) <= 16384 && r->guards.empty() && r->rk.variants.size() < 2 && r->rk.pres_key.empty();
       for (const RenderedKernel::Pre &pk : r->rk.pres) small = small && (r->rk.klass == KernelClass::THREAD_REDUCE || threads_of(pk.launch) <= 16384);
-      bool follows = false;
-      for (int sl : u.slots) follows = follows || side_wrote[(size_t)sl];
-      const bool side = small && (r->rk.klass == KernelClass::THREAD_REDUCE || follows);
-      if (side) { plan->on_side[(size_t)ui] = 1; plan->forked = true; }
-      for (int sl : u.writes) side_wrote[(size_t)sl] = side ? 1 : 0;
+      int follows = 0;
+      for (int sl : u.slots) if (!follows) follows = side_wrote[(size_t)sl];
+      int side = 0;
+      if (small && follows) side = follows;
+      else if (small && r->rk.klass == KernelClass::THREAD_REDUCE) side = 1 + next++;
+      if (side) { plan->on_side[(size_t)ui] = 1; chain_of[(size_t)ui] = side - 1; plan->forked = true; }
+      for (int sl : u.writes) side_wrote[(size_t)sl] = side;
     }
     // (a plan that is mostly such launches is one chain of small steps: nothing to run beside)
     int n_side = 0;
-    for (int ui = 0; ui < n_units; ui++) n_side += plan->on_side[(size_t)ui];
+    for (int ui = 0; ui < n_units; ui++) n_side += plan->on_side[(size_t)ui] != 0;
     if (2 * n_side > n_units) { plan->on_side.assign((size_t)n_units, 0); plan->forked = false; }
   }
   // ── lifetimes of intermediates in execution order ──────────────────────
@@ -490,51 +513,83 @@ PolyHipPlan *poly_hip_compile_schedule(PolyCtx *ctx, const PolySchedule *s) {
           if ((x.w || y.w) && x.lo < y.hi && y.lo < x.hi) return true;
       return false;
     };
-    int synced[2] = {-1, -1};     // [stream]: the latest launch of the OTHER stream that this stream has waited for
-    for (int i = 0; i < n_units; i++) {
-      const int me = plan->on_side[(size_t)i];
-      for (int j = i - 1; j > synced[me]; j--) {
-        if (plan->on_side[(size_t)j] == me || !conflict(i, j)) continue;
-        plan->wait_for[(size_t)i] = j;
-        plan->records[(size_t)j] = 1;
-        synced[me] = j;
-        break;
-      }
-    }
     // A wait between the streams costs a few microseconds of its own: worth it when the
-    // side launches run for long stretches without one (two waits for 388 launches in the
-    // 24-layer training step), not when every other side launch needs one (an MLP step of
-    // 22 launches came out 13 % slower on two streams).
-    {
-      int ns = 0, nw = 0;
-      for (int i = 0; i < n_units; i++) { ns += plan->on_side[(size_t)i]; nw += plan->wait_for[(size_t)i] >= 0; }
-      if (8 * nw > ns) {
-        if (getenv("POLY_HIP_DEBUG"))
-          fprintf(stderr, "polygrad: compile_schedule: %d waits for %d side launches: everything stays on one stream\n", nw, ns);
+    // side launches run for long stretches without one (a handful of waits for 388 launches
+    // in the 24-layer training step), not when every other side launch needs one (an MLP
+    // step of 22 launches came out 13 % slower on two streams).  The most side streams
+    // whose waits stay under one for eight side launches are taken.
+    int n_on_side = 0, n_waits = 0, n_main_waits = 0;
+    for (int i = 0; i < n_units; i++) n_on_side += plan->on_side[(size_t)i] != 0;
+    // (two by default: with the main stream and the default stream of the process they take
+    // the four hardware queues a process gets; a third side stream shares a queue with one
+    // of the others, and the 24-layer step came out 3 ms slower than on two)
+    int max_streams = 2;
+    if (const char *e = getenv("POLY_HIP_SIDE_STREAMS")) max_streams = std::max(1, std::min(kSideStreams, atoi(e)));
+    for (int n_streams = max_streams; n_streams >= 1; n_streams--) {
+      plan->n_side_streams = 0;
+      for (int i = 0; i < n_units; i++) {
+        plan->on_side[(size_t)i] = chain_of[(size_t)i] < 0 ? 0 : (char)(1 + chain_of[(size_t)i] % n_streams);
+        plan->n_side_streams = std::max(plan->n_side_streams, (int)plan->on_side[(size_t)i]);
+      }
+      plan->waits.assign((size_t)n_units, std::vector<int>());
+      plan->records.assign((size_t)n_units, 0);
+      // synced[a][b]: the latest launch of stream b that stream a has waited for
+      int synced[kSideStreams + 1][kSideStreams + 1];
+      for (auto &row : synced) for (int &v : row) v = -1;
+      n_waits = n_main_waits = 0;
+      for (int i = 0; i < n_units; i++) {
+        const int me = plan->on_side[(size_t)i];
+        for (int other = 0; other <= plan->n_side_streams; other++) {
+          if (other == me) continue;
+          for (int j = i - 1; j > synced[me][other]; j--) {
+            if (plan->on_side[(size_t)j] != other || !conflict(i, j)) continue;
+            plan->waits[(size_t)i].push_back(j);
+            plan->records[(size_t)j] = 1;
+            synced[me][other] = j;
+            n_waits++;
+            n_main_waits += me == 0;
+            break;
+          }
+        }
+      }
+      if (8 * n_main_waits <= n_on_side) break;
+      if (getenv("POLY_HIP_DEBUG"))
+        fprintf(stderr, "polygrad: compile_schedule: the main sequence would wait %d times for %d side launches on %d side streams: too many\n", n_main_waits, n_on_side, n_streams);
+      if (n_streams == 1) {   // everything stays on one stream
         plan->on_side.assign((size_t)n_units, 0);
-        plan->wait_for.assign((size_t)n_units, -1);
+        plan->waits.assign((size_t)n_units, std::vector<int>());
         plan->records.assign((size_t)n_units, 0);
+        plan->n_side_streams = 0;
         plan->forked = false;
       }
     }
     if (plan->forked && getenv("POLY_HIP_DEBUG")) {
-      int ns = 0, nw = 0;
-      for (int i = 0; i < n_units; i++) { ns += plan->on_side[(size_t)i]; nw += plan->wait_for[(size_t)i] >= 0; }
-      fprintf(stderr, "polygrad: compile_schedule: %d of %d launches on the second stream, %d waits between the streams\n", ns, n_units, nw);
+      fprintf(stderr, "polygrad: compile_schedule: %d of %d launches on %d side streams, %d waits between the streams, %d of them by the main sequence\n",
+              n_on_side, n_units, plan->n_side_streams, n_waits, n_main_waits);
+      for (int i = 0; i < n_units; i++)
+        for (int w : plan->waits[(size_t)i])
+          if (plan->on_side[(size_t)i] == 0 || n_waits <= 16) fprintf(stderr, "polygrad: compile_schedule: launch %d (stream %d) waits for launch %d (stream %d)\n", i, plan->on_side[(size_t)i], w,
+                  plan->on_side[(size_t)w]);
       // every pair of launches on different streams that touch the same bytes, one of them
       // writing, must be ordered by the waits (checked here from scratch, pair by pair)
       {
-        std::vector<int> seen_other((size_t)n_units, -1);   // latest launch of the other stream known to be over when i starts
-        int last_on[2] = {-1, -1};
+        // seen[i][b]: latest launch of stream b known to be over when i starts
+        std::vector<std::array<int, kSideStreams + 1>> seen((size_t)n_units);
+        int last_on[kSideStreams + 1];
+        for (int &v : last_on) v = -1;
         long long unordered = 0, pairs = 0;
         for (int i = 0; i < n_units; i++) {
           const int me = plan->on_side[(size_t)i];
-          int so = last_on[me] >= 0 ? seen_other[(size_t)last_on[me]] : -1;
-          if (plan->wait_for[(size_t)i] >= 0) so = std::max(so, plan->wait_for[(size_t)i]);
-          seen_other[(size_t)i] = so;
+          for (int b = 0; b <= kSideStreams; b++) seen[(size_t)i][(size_t)b] = last_on[me] >= 0 ? seen[(size_t)last_on[me]][(size_t)b] : -1;
+          for (int w : plan->waits[(size_t)i]) {
+            int &v = seen[(size_t)i][(size_t)plan->on_side[(size_t)w]];
+            v = std::max(v, w);
+          }
           last_on[me] = i;
-          for (int j = 0; j < i; j++)
-            if (plan->on_side[(size_t)j] != me && conflict(i, j)) { pairs++; if (j > so) unordered++; }
+          for (int j = 0; j < i; j++) {
+            const int sj = plan->on_side[(size_t)j];
+            if (sj != me && conflict(i, j)) { pairs++; if (j > seen[(size_t)i][(size_t)sj]) unordered++; }
+          }
         }
         fprintf(stderr, "polygrad: compile_schedule: %lld pairs of launches across the streams share bytes, %lld of them unordered\n", pairs, unordered);
       }
@@ -542,12 +597,13 @@ PolyHipPlan *poly_hip_compile_schedule(PolyCtx *ctx, const PolySchedule *s) {
   }
   // one scratch pool for all other two-stage kernels of a stream: the largest need
   {
-    int users = 0, side_users = 0;
-    size_t side_bytes = 0;
+    int users = 0, side_users[kSideStreams] = {0, 0, 0};
+    size_t side_bytes[kSideStreams] = {0, 0, 0};
     for (int ui = 0; ui < n_units; ui++) {
       const Unit &u = plan->units[(size_t)ui];
       if (u.runner->rk.scratch_bytes == 0 || keeps_scratch[(size_t)ui]) continue;
-      if (plan->on_side[(size_t)ui]) { side_users++; side_bytes = std::max(side_bytes, u.runner->rk.scratch_bytes); }
+      const int st = plan->on_side[(size_t)ui];
+      if (st) { side_users[st - 1]++; side_bytes[st - 1] = std::max(side_bytes[st - 1], u.runner->rk.scratch_bytes); }
       else { users++; plan->scratch_bytes = std::max(plan->scratch_bytes, u.runner->rk.scratch_bytes); }
     }
     if (users > 1) {
@@ -556,13 +612,15 @@ PolyHipPlan *poly_hip_compile_schedule(PolyCtx *ctx, const PolySchedule *s) {
       for (int ui = 0; ui < n_units; ui++)
         if (!keeps_scratch[(size_t)ui] && !plan->on_side[(size_t)ui]) runner_share_scratch(plan->units[(size_t)ui].runner, plan->scratch_pool);
     }
-    if (side_users > 1) {
-      plan->side_scratch_pool = runtime_alloc(side_bytes);
-      if (!plan->side_scratch_pool) return nullptr;
-      for (int ui = 0; ui < n_units; ui++)
-        if (!keeps_scratch[(size_t)ui] && plan->on_side[(size_t)ui]) runner_share_scratch(plan->units[(size_t)ui].runner, plan->side_scratch_pool);
+    for (int k = 0; k < kSideStreams; k++) {
+      if (side_users[k] > 1) {
+        plan->side_scratch_pool[k] = runtime_alloc(side_bytes[k]);
+        if (!plan->side_scratch_pool[k]) return nullptr;
+        for (int ui = 0; ui < n_units; ui++)
+          if (!keeps_scratch[(size_t)ui] && plan->on_side[(size_t)ui] == k + 1) runner_share_scratch(plan->units[(size_t)ui].runner, plan->side_scratch_pool[k]);
+      }
+      plan->kept_scratch_bytes += side_bytes[k];
     }
-    plan->kept_scratch_bytes += side_bytes;
     // a lone user owns its scratch memory; it must exist before the launches are captured
     for (Unit &u : plan->units) if (runner_ensure_scratch(u.runner) != 0) return nullptr;
   }
@@ -928,7 +986,7 @@ void *poly_hip_plan_slot_ptr(const PolyHipPlan *plan, int slot) {
 void poly_hip_plan_set_graph(PolyHipPlan *plan, int enabled) { if (plan) plan->use_graph = enabled != 0; }
 int poly_hip_plan_side_launches(const PolyHipPlan *plan) {
   int n = 0;
-  if (plan) for (char c : plan->on_side) n += c;
+  if (plan) for (char c : plan->on_side) n += c != 0;
   return n;
 }
 

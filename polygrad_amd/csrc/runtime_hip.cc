@@ -36,7 +36,7 @@ struct Runtime {
   bool ok = false;
   int device = 0;
   hipStream_t stream = nullptr;
-  hipStream_t side = nullptr;          // second stream of a plan's captured graphs, made on first use
+  hipStream_t side[3] = {nullptr, nullptr, nullptr};   // further streams of a plan's captured graphs, made on first use
   hipStream_t launch_on = nullptr;     // where program_launch puts kernels when not the main stream
   std::map<uint64_t, std::weak_ptr<Module>> modules;   // keyed by source hash
   std::map<uint64_t, std::vector<char>> code_cache;    // compiled, not yet loaded
@@ -144,11 +144,11 @@ int runtime_init() {
 
 void *runtime_stream() { return runtime_init() == 0 ? (void *)rt().stream : nullptr; }
 
-void *runtime_side_stream() {
-  if (runtime_init() != 0) return nullptr;
+void *runtime_side_stream(int k) {
+  if (runtime_init() != 0 || k < 0 || k >= kSideStreams) return nullptr;
   Runtime &r = rt();
-  if (!r.side && !check(hipStreamCreateWithFlags(&r.side, hipStreamNonBlocking), "hipStreamCreate")) r.side = nullptr;
-  return (void *)r.side;
+  if (!r.side[k] && !check(hipStreamCreateWithFlags(&r.side[k], hipStreamNonBlocking), "hipStreamCreate")) r.side[k] = nullptr;
+  return (void *)r.side[k];
 }
 
 void runtime_launch_on(void *stream) { rt().launch_on = (hipStream_t)stream; }

@@ -13,10 +13,11 @@ struct Program;  // one kernel entry inside a loaded (shared) module
 
 int runtime_init();
 void *runtime_stream();
-// A second stream (same priority) for launches that a plan's captured graph lets run beside
-// the main sequence, and the switch that sends the following program_launch calls to it
-// (nullptr: back to the main stream).
-void *runtime_side_stream();
+// Further streams (same priority; k in [0, kSideStreams)) for launches that a plan's
+// captured graph lets run beside the main sequence, and the switch that sends the following
+// program_launch calls to one of them (nullptr: back to the main stream).
+constexpr int kSideStreams = 3;
+void *runtime_side_stream(int k);
 void runtime_launch_on(void *stream);
 void *runtime_alloc(size_t nbytes);
 void runtime_free(void *p);

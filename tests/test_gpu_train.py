@@ -157,12 +157,14 @@ def test_gpt2_multi_block_train_step_matches_reference(n_blocks):
     assert sum("3 slabs of one output range" in k["desc"] for k in info) == n_blocks
 
 
-def test_launches_on_the_second_stream_change_nothing():
+@pytest.mark.parametrize("streams", ["1", "2", "3"])
+def test_launches_on_the_second_stream_change_nothing(streams):
     """The in-order adders of the bf16 column sums (one thread per output, a chain of 4096
-    dependent additions each) run on a second stream of the captured graph, ordered against
-    the main sequence by the buffers they share.  Three replays of the graph must give what
-    the single-stream graph gives, bit for bit (the optimizer state advances with every run,
-    so a launch that ran too early or too late would show)."""
+    dependent additions each) run on side streams of the captured graph (dealt to them in
+    turn), ordered against the main sequence and each other by the buffers they share.  Three
+    replays of the graph must give what the single-stream graph gives, bit for bit (the
+    optimizer state advances with every run, so a launch that ran too early or too late
+    would show)."""
     import os
     # (large enough for most launches to fill more than a quarter of the chip: a plan of
     # small launches only is one chain and stays on one stream)
@@ -172,12 +174,14 @@ def test_launches_on_the_second_stream_change_nothing():
         c = R.Ctx()
         bufs, sink = graphs.gpt2_block_train_step(c, B, T, D, H, V, lr=lr)
         arrays = graphs.gpt2_block_train_inputs(bufs, B, T, V)
+        os.environ["POLY_HIP_SIDE_STREAMS"] = streams
         if single:
             os.environ["POLY_HIP_NO_SIDE_STREAM"] = "1"
         try:
             got, info = run_hip(c, sink, arrays, repeats=3)
         finally:
             os.environ.pop("POLY_HIP_NO_SIDE_STREAM", None)
+            os.environ.pop("POLY_HIP_SIDE_STREAMS", None)
         n_side = run_hip.side_launches
         assert (n_side == 0) if single else (n_side >= 4), n_side
         outs.append({name: got[t] for name, t in bufs.items()})
