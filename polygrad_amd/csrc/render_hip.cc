@@ -1249,6 +1249,9 @@ static bool try_slab_fission(const KernelGraph &g, const std::string &fn_name, c
     // one kernel per slab
     std::vector<RenderedKernel> parts(order.size());
     const PolyUOp *root = g.nodes.back().u;
+    // (operand planes that an earlier slab left in the scratch memory and nothing has
+    // overwritten since: a later slab may read them)
+    const RenderedKernel::OperandPlanes *planes = nullptr;
     for (size_t i = 0; i < order.size() && ok; i++) {
       KernelGraph sub;
       sub.slab_range = g.n(g.ranges[(size_t)R].node).u;
@@ -1257,7 +1260,9 @@ static bool try_slab_fission(const KernelGraph &g, const std::string &fn_name, c
       sub.slab_value = g.n(order[i].value).u;
       for (const ParamInfo &pi : g.params) sub.slab_params.push_back(g.n(pi.node).u);
       std::string err;
-      if (!sub.build(root) || !render_kernel(sub, fn_name, opt, &parts[i], &err)) {
+      RenderOptions sopt = opt;
+      sopt.planes_before = planes;
+      if (!sub.build(root) || !render_kernel(sub, fn_name, sopt, &parts[i], &err)) {
         if (getenv("POLY_HIP_DEBUG")) fprintf(stderr, "polygrad: render_hip: slab %zu: %s%s\n", i, sub.error.c_str(), err.c_str());
         ok = false;
         break;
@@ -1266,6 +1271,7 @@ static bool try_slab_fission(const KernelGraph &g, const std::string &fn_name, c
       if (pk.klass != KernelClass::MATMUL_MFMA || !pk.guards.empty() || !pk.tables.empty() || !pk.fallback_source.empty() ||
           pk.n_vars != 0 || pk.n_params != parts[0].n_params)
         ok = false;
+      if (!pk.reads_planes_before) planes = pk.a_planes.valid ? &parts[i].a_planes : nullptr;
     }
     if (!ok) return fis_reject(__LINE__);
     *out = parts.back();

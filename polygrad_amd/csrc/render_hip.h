@@ -87,6 +87,22 @@ struct RenderedKernel {
   // writes those buffers in between.
   std::string pres_key;
   std::vector<int> pre_reads;
+  // What the first stages of a product of computed operands leave at the start of the
+  // scratch memory: operand A as `parts` bf16 planes per row ([z][row][part][k]), with a
+  // description of the operand that does not name ranges -- its arithmetic over its loads,
+  // and every load's address as base + by_row[row] + by_k[k] + by_z[z].  A later kernel
+  // of the same launch whose operand A is the same values with rows and depth exchanged
+  // reads these planes instead of writing its own (the slabs of the derivative of a
+  // q | k | v split: dS K and dS^T Q).
+  struct OperandPlanes {
+    bool valid = false;
+    std::string dag;
+    struct Load { int param, dt; int64_t base; std::vector<int64_t> by_row, by_k, by_z; };
+    std::vector<Load> loads;
+    int64_t rows = 0, k = 0, z = 0;
+    int parts = 0;
+  } a_planes;
+  bool reads_planes_before = false;   // this kernel's operand A is the planes of RenderOptions::planes_before
 };
 
 struct Scope;
@@ -122,6 +138,9 @@ struct RenderOptions {
   // Lanes along the reduce range only when some load is contiguous along it, however few
   // rows there are (otherwise: only from 65536 rows up).
   bool coop_needs_unit_stride = false;
+  // Operand planes that an earlier kernel of the same launch leaves at the start of the
+  // scratch memory (see RenderedKernel::OperandPlanes).
+  const RenderedKernel::OperandPlanes *planes_before = nullptr;
 };
 
 // Returns false and sets *err on unsupported graphs (never falls back to a

@@ -7,6 +7,9 @@
 #include <algorithm>
 #include <cmath>
 #include <cstdlib>
+#include <cstring>
+#include <functional>
+#include <map>
 
 #include "templates.h"
 
@@ -768,8 +771,129 @@ bool render_matmul(const MatmulMatch &mm, const MatmulEpilogue &ep, RenderedKern
 // runs it with the operands evaluated on the way into LDS: the loads of an element are
 // issued K tiles ahead (phase 1, raw bits kept in registers), the arithmetic on them runs
 // when the tile is stored to LDS (phase 2).  Products are exact fp32, accumulation fp32.
+// Value of canonical index expression `l` at range values `rv` (false: not a function of
+// ranges alone).
+static bool eval_lin(const KernelGraph &g, const Lin &l, const std::vector<int64_t> &rv, int64_t *out) {
+  int64_t v = l.c0;
+  for (const Term &t : l.terms) {
+    const Atom &a = g.atoms[(size_t)t.atom];
+    int64_t x;
+    if (a.kind == Atom::RANGE) x = rv[(size_t)g.range_ord.at(a.node)];
+    else if (a.kind == Atom::DIV || a.kind == Atom::MOD) {
+      int64_t in;
+      if (!eval_lin(g, a.inner, rv, &in) || in < 0 || a.c <= 0) return false;
+      x = a.kind == Atom::DIV ? in / a.c : in % a.c;
+    } else return false;
+    v += t.coef * x;
+  }
+  *out = v;
+  return true;
+}
+
+// Describes operand `node` of a product without naming ranges (RenderedKernel::OperandPlanes):
+// `loads` are its LOADs, `rows` / `kd` / `zd` the digits that make up its row, depth and
+// batch coordinates.
+static void describe_operand(const KernelGraph &g, int node, const std::vector<int> &loads, const std::vector<Dim> &rows,
+                             const std::vector<Dim> &kd, const std::vector<Dim> &zd, int64_t M, int64_t K, int64_t Z,
+                             RenderedKernel::OperandPlanes *out) {
+  out->valid = false;
+  out->rows = M; out->k = K; out->z = Z;
+  if (loads.empty() || M + K + Z > 1048576) return;
+  // the arithmetic, nodes numbered in the order they are met
+  std::map<int, int> seen;
+  std::vector<int> load_order;
+  bool ok = true;
+  std::string text;
+  std::function<void(int)> walk = [&](int id) {
+    if (!ok) return;
+    auto it = seen.find(id);
+    if (it != seen.end()) { text += strf("@%d ", it->second); return; }
+    const int my = (int)seen.size();
+    seen[id] = my;
+    const KNode &k = g.n(id);
+    if (k.op == POLY_OP_LOAD) {
+      const KNode &ix = g.n(k.src[0]);
+      if (k.guard >= 0 || ix.op != POLY_OP_INDEX || ix.src.size() != 2 || g.n(ix.src[1]).lin < 0) { ok = false; return; }
+      text += strf("L%zu ", load_order.size());
+      load_order.push_back(id);
+      return;
+    }
+    if (k.op == POLY_OP_CONST) {
+      const PolyArg &a = k.u->arg;
+      long long bits = 0;
+      if (a.kind == POLY_ARG_FLOAT) memcpy(&bits, &a.f, sizeof bits);
+      else if (a.kind == POLY_ARG_INT) bits = (long long)a.i;
+      else if (a.kind == POLY_ARG_BOOL) bits = a.b ? 1 : 0;
+      else { ok = false; return; }
+      text += strf("C%d:%d:%llx ", (int)k.dt, (int)a.kind, bits);
+      return;
+    }
+    if (k.op == POLY_OP_RANGE || k.op == POLY_OP_INDEX || k.op == POLY_OP_PARAM || k.op == POLY_OP_DEFINE_VAR || k.op == POLY_OP_REDUCE ||
+        k.op == POLY_OP_SPECIAL || k.op == POLY_OP_BIND || k.op == POLY_OP_STORE || k.u->arg.kind != POLY_ARG_NONE || k.src.empty()) { ok = false; return; }
+    text += strf("(%d:%d ", (int)k.op, (int)k.dt);
+    for (int c : k.src) walk(c);
+    text += ") ";
+  };
+  walk(node);
+  if (!ok || load_order.size() != loads.size()) return;
+  // the addresses
+  std::vector<int64_t> rv(g.ranges.size());
+  auto address = [&](const Lin &l, int64_t m, int64_t k, int64_t z, int64_t *a) {
+    std::fill(rv.begin(), rv.end(), 0);
+    auto put = [&](const std::vector<Dim> &dims, int64_t x) {
+      for (size_t i = dims.size(); i-- > 0;) {
+        const int64_t digit = i == 0 ? x : x % dims[i].extent;
+        if (i) x /= dims[i].extent;
+        rv[(size_t)dims[i].ord] += digit * dims[i].cut;
+      }
+    };
+    put(rows, m); put(kd, k); put(zd, z);
+    return eval_lin(g, l, rv, a);
+  };
+  out->loads.clear();
+  for (int id : load_order) {
+    const KNode &ld = g.n(id);
+    const KNode &ix = g.n(ld.src[0]);
+    const Lin &l = g.lins[(size_t)g.n(ix.src[1]).lin];
+    RenderedKernel::OperandPlanes::Load d;
+    d.param = g.param_slot(ix.src[0]);
+    d.dt = (int)ld.dt;
+    if (d.param < 0 || !address(l, 0, 0, 0, &d.base)) return;
+    d.by_row.resize((size_t)M); d.by_k.resize((size_t)K); d.by_z.resize((size_t)Z);
+    int64_t a;
+    for (int64_t m = 0; m < M; m++) { if (!address(l, m, 0, 0, &a)) return; d.by_row[(size_t)m] = a - d.base; }
+    for (int64_t k = 0; k < K; k++) { if (!address(l, 0, k, 0, &a)) return; d.by_k[(size_t)k] = a - d.base; }
+    for (int64_t z = 0; z < Z; z++) { if (!address(l, 0, 0, z, &a)) return; d.by_z[(size_t)z] = a - d.base; }
+    // the address is the sum of the three parts: every atom of a canonical index depends on
+    // one range, and every use of a range is a sum over its digits; checked at scattered
+    // points and the far corner all the same
+    uint64_t rnd = 0x9e3779b97f4a7c15ull;
+    for (int t = 0; t < 256; t++) {
+      rnd = rnd * 6364136223846793005ull + 1442695040888963407ull;
+      int64_t m = (int64_t)((rnd >> 33) % (uint64_t)M), k = (int64_t)((rnd >> 13) % (uint64_t)K), z = (int64_t)((rnd >> 3) % (uint64_t)Z);
+      if (t == 0) { m = M - 1; k = K - 1; z = Z - 1; }
+      if (!address(l, m, k, z, &a) || a != d.base + d.by_row[(size_t)m] + d.by_k[(size_t)k] + d.by_z[(size_t)z]) return;
+    }
+    out->loads.push_back(std::move(d));
+  }
+  out->dag = text;
+  out->valid = true;
+}
+
+// Is operand `mine` the operand behind `theirs` with rows and depth exchanged?
+static bool exchanged(const RenderedKernel::OperandPlanes &mine, const RenderedKernel::OperandPlanes &theirs) {
+  if (!mine.valid || !theirs.valid || mine.parts != theirs.parts || mine.rows != theirs.k || mine.k != theirs.rows || mine.z != theirs.z ||
+      mine.dag != theirs.dag || mine.loads.size() != theirs.loads.size())
+    return false;
+  for (size_t j = 0; j < mine.loads.size(); j++) {
+    const auto &a = mine.loads[j], &b = theirs.loads[j];
+    if (a.param != b.param || a.dt != b.dt || a.base != b.base || a.by_row != b.by_k || a.by_k != b.by_row || a.by_z != b.by_z) return false;
+  }
+  return true;
+}
+
 bool try_render_matmul_generic(const KernelGraph &g, const std::string &fn, const RenderOptions &opt, RenderedKernel *out) {
-  (void)fn; (void)opt;
+  (void)fn;
   if (getenv("POLY_HIP_NO_F32_MFMA") || getenv("POLY_HIP_NO_GENERIC_MM")) return reject(__LINE__);
   if (g.stores.size() != 1 || g.reduces.size() != 1 || !g.vars.empty()) return reject(__LINE__);
   const StoreInfo &st = g.stores[0];
@@ -915,6 +1039,7 @@ bool try_render_matmul_generic(const KernelGraph &g, const std::string &fn, cons
   };
   int n_loads[2] = {0, 0};
   bool walk_k[2] = {true, true};
+  std::vector<int> a_loads;
   std::string code;
   for (int side = 0; side < 2; side++) {
     const char *nm = side == 0 ? "a" : "b";
@@ -932,6 +1057,7 @@ bool try_render_matmul_generic(const KernelGraph &g, const std::string &fn, cons
       }
     if (loads.size() > 6) return reject(__LINE__);
     n_loads[side] = (int)loads.size();
+    if (side == 0) a_loads = loads;
     // which way memory runs: along k when the first load has unit stride in the innermost
     // reduce range, along the rows when it has unit stride in the innermost row range
     if (!loads.empty()) {
@@ -1013,10 +1139,20 @@ bool try_render_matmul_generic(const KernelGraph &g, const std::string &fn, cons
     // (int offsets inside the template; and the planes should stay a small part of the card's memory)
     const bool fits = elems_a < 2147483647.0 && elems_b < 2147483647.0 && (elems_a + elems_b) * 2.0 <= 8.0 * 1073741824.0;
     // worth the extra pass over the operands only for deep or large products
-    const bool large = (double)M * (double)N * (double)K * (double)Z >= 1073741824.0;
+    double min_work = 1073741824.0;
+    if (const char *e = getenv("POLY_HIP_BF16_SPLIT_MIN")) min_work = std::max(1.0, atof(e));   // tests: small products through this path
+    const bool large = (double)M * (double)N * (double)K * (double)Z >= min_work;
     if (!getenv("POLY_HIP_NO_BF16_SPLIT") && parts[0] + parts[1] <= 4 && fits && large) {
       const size_t off_b = ((size_t)elems_a * 2 + 255) / 256 * 256;       // bytes
       const size_t scratch_bytes = off_b + (size_t)elems_b * 2;
+      // Operand A may already lie in the scratch memory with rows and depth exchanged (an
+      // earlier kernel of the same launch wrote it): read row m, plane p, depth k at
+      // [z][k][p][m] then, and write no planes.  Sizes in whole K tiles, so that both
+      // kernels put operand B behind the same number of bytes and no padding is read.
+      RenderedKernel::OperandPlanes mine;
+      if (!getenv("POLY_HIP_NO_SHARED_PLANES")) describe_operand(g, opnd[0], a_loads, mm.md_full, k_dims, mm.zd_full, M, K, Z, &mine);
+      mine.parts = parts[0];
+      const bool shared = opt.planes_before && M % 64 == 0 && K % 64 == 0 && exchanged(mine, *opt.planes_before);
       RenderedKernel::Pre pre[2];
       for (int side = 0; side < 2; side++) {
         const char *nm = side == 0 ? "a" : "b";
@@ -1045,6 +1181,11 @@ bool try_render_matmul_generic(const KernelGraph &g, const std::string &fn, cons
       m2.md.push_back(Dim{-1, M, parts[0] * KP, 0, 1});
       m2.nd.push_back(Dim{-1, N, 0, parts[1] * KP, 1});
       if (Z > 1) m2.zd.push_back(Dim{-1, Z, M * parts[0] * KP, N * parts[1] * KP, 1});
+      if (shared) {
+        // (the planes were written for K rows of M: M is the padded depth there)
+        m2.ka = KSplit{KP, parts[0] == P ? M : 0, parts[0] * M};
+        m2.md[0].ca = 1;
+      }
       m2.md_full = mm.md_full; m2.nd_full = mm.nd_full; m2.zd_full = mm.zd_full;
       MatmulEpilogue ep2 = ep;
       ep2.signature += ", __bf16* poly_scratch";
@@ -1055,11 +1196,16 @@ bool try_render_matmul_generic(const KernelGraph &g, const std::string &fn, cons
       RenderedKernel main;
       if (render_matmul(m2, ep2, &main)) {
         *out = main;
-        out->pres.insert(out->pres.begin(), {pre[0], pre[1]});      // planes first, then a split product's first stage
+        // planes first, then a split product's first stage
+        if (shared) out->pres.insert(out->pres.begin(), pre[1]);
+        else out->pres.insert(out->pres.begin(), {pre[0], pre[1]});
         out->scratch_bytes = std::max(scratch_bytes, main.scratch_bytes);
         out->flops = 2.0 * (double)M * (double)N * (double)K * (double)Z;
-        out->strategy = strf("operands as expressions, written as bf16 planes first (%d + %d planes of K=%lld, %.0f MB): ", parts[0], parts[1],
-                             (long long)KP, (double)scratch_bytes / 1e6) + out->strategy;
+        out->strategy = strf("operands as expressions, written as bf16 planes first (%d + %d planes of K=%lld, %.0f MB%s): ", parts[0], parts[1],
+                             (long long)KP, (double)scratch_bytes / 1e6,
+                             shared ? "; A is what the kernel before left as its A, rows and depth exchanged, and is not written again" : "") + out->strategy;
+        out->reads_planes_before = shared;
+        if (!shared) out->a_planes = mine;
         for (RenderedKernel::Variant &v : out->variants) v.strategy = out->strategy;
         return true;
       }

@@ -141,6 +141,38 @@ def test_gpt2_block_train_step_matches_reference(B, T, D, H, V):
         assert any("3 slabs of one output range" in k["desc"] for k in info)
 
 
+def test_slabs_of_the_qkv_derivative_share_operand_planes():
+    """Two slabs of the derivative of the q | k | v split multiply by the same fp32 tensor
+    (the softmax derivative dS: dq = dS K, dk = dS^T Q).  At full size both products run on
+    the bf16 MFMA over three bf16 planes of dS; the second slab reads the planes the first
+    one wrote (as rows along the depth) instead of writing its own.  Here at a size the
+    reference CPU backend finishes quickly, with the size threshold of that path lowered:
+    against the reference, and bit for bit against the same step with every slab writing
+    its own planes."""
+    import os
+    B, T, D, H, V, lr = 1, 128, 128, 2, 97, 3e-4
+    os.environ["POLY_HIP_BF16_SPLIT_MIN"] = "1048576"
+    try:
+        c = R.Ctx()
+        bufs, sink = graphs.gpt2_block_train_step(c, B, T, D, H, V, lr=lr)
+        info = check_train_step(c, bufs, sink, B, T, V, lr, graphs.BLOCK_PARAMS, 60)
+        slabs = [k["desc"] for k in info if "3 slabs of one output range" in k["desc"]]
+        assert len(slabs) == 1 and "rows and depth exchanged" in slabs[0] and slabs[0].count("bf16 planes first") == 3, slabs
+        arrays = graphs.gpt2_block_train_inputs(bufs, B, T, V)
+        got, _ = run_hip(c, sink, arrays)
+        os.environ["POLY_HIP_NO_SHARED_PLANES"] = "1"
+        try:
+            own, info1 = run_hip(c, sink, arrays)
+        finally:
+            del os.environ["POLY_HIP_NO_SHARED_PLANES"]
+        assert not any("rows and depth exchanged" in k["desc"] for k in info1)
+        for name, t in bufs.items():
+            assert got[t].tobytes() == own[t].tobytes(), name
+        c.close()
+    finally:
+        del os.environ["POLY_HIP_BF16_SPLIT_MIN"]
+
+
 @pytest.mark.parametrize("n_blocks", [2, 3])
 def test_gpt2_multi_block_train_step_matches_reference(n_blocks):
     """The same with several blocks stacked (configuration 5 has 24): gradients flow through
