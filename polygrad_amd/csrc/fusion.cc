@@ -31,8 +31,9 @@ const char *const kAttentionTemplate =
 #include "attention_mfma.hip.inc"
     ;
 
+int fa_item = -1;     // the schedule item a group is being grown from (for the message below)
 bool fa_reject(int line) {
-  if (getenv("POLY_HIP_DEBUG")) fprintf(stderr, "polygrad: fusion: attention group rejected at fusion.cc:%d\n", line);
+  if (getenv("POLY_HIP_DEBUG")) fprintf(stderr, "polygrad: fusion: group from kernel %d rejected at fusion.cc:%d\n", fa_item, line);
   return false;
 }
 #define FA_REJECT() return fa_reject(__LINE__)
@@ -789,7 +790,12 @@ static bool match_row_chain_impl(const Sched &sc, int a_item, const std::vector<
       for (int r : sc.readers[(size_t)c_out]) {
         if (taken[(size_t)r]) row_goes_on = false;
         else if (sc.graphs[(size_t)r].reduces.empty()) rm++;
-        else rr++;
+        else {
+          rr++;
+          // (a reduction of another shape -- a matmul over the rows -- ends the chain here)
+          int red, ord;
+          if (!reduce_shape(sc.graphs[(size_t)r], &red, &ord) || sc.graphs[(size_t)r].ranges[(size_t)ord].extent != R) row_goes_on = false;
+        }
       }
       if (rr != 1 || rm > 1) row_goes_on = false;
     }
@@ -1118,6 +1124,7 @@ static bool match_row_chain_impl(const Sched &sc, int a_item, const std::vector<
 }
 
 static bool match_row_chain(const Sched &sc, int a_item, const std::vector<char> &taken, FusedGroup *out) {
+  fa_item = a_item;
   // first with maps in the middle of the chain (their rows kept in registers), then the plain form
   return match_row_chain_impl(sc, a_item, taken, out, true) || match_row_chain_impl(sc, a_item, taken, out, false);
 }

@@ -390,19 +390,25 @@ PolyHipPlan *poly_hip_compile_schedule(PolyCtx *ctx, const PolySchedule *s) {
       last[(size_t)sl] = step;
     }
   }
-  // What a side launch reads or writes stays where it is for a while after its turn in the
-  // sequence: the main sequence runs on meanwhile, and a later launch given the same bytes
-  // would have to wait for it.  Small buffers (column sums, their casts) keep their place
-  // for good, larger ones for the next 32 launches.
-  if (plan->forked)
+  // What a side launch reads or writes keeps its place to the end of the sequence: the main
+  // sequence runs on meanwhile, and a later launch given the same bytes would have to wait
+  // for the side stream.  A wait by the main sequence in the middle of the graph costs far
+  // more than the wait itself (one such wait made the 24-layer training step 2 ms slower),
+  // the memory little (the buffers are the terms of the column sums, alive up to their
+  // adder anyway, and the sums).  POLY_HIP_SIDE_KEEP=n releases buffers above 64 KB n
+  // launches after their side launch instead.
+  if (plan->forked) {
+    int keep_for = n_units;
+    if (const char *e = getenv("POLY_HIP_SIDE_KEEP")) keep_for = std::max(0, atoi(e));
     for (int step = 0; step < n_units; step++) {
       if (!plan->on_side[(size_t)step]) continue;
       for (int sl : plan->units[(size_t)step].slots) {
         if (!s->buf_slots[sl].is_intermediate) continue;
-        const int keep = s->buf_slots[sl].nbytes <= 65536 ? n_units : std::min(n_units, step + 32);
+        const int keep = s->buf_slots[sl].nbytes <= 65536 ? n_units : std::min(n_units, step + keep_for);
         last[(size_t)sl] = std::max(last[(size_t)sl], keep);
       }
     }
+  }
   // ── place intermediates in one arena; overlapping lifetimes never share ──
   struct Placed { size_t off, size; int first, last; };
   std::vector<Placed> placed;
