@@ -116,7 +116,7 @@ int poly_hip_check_index_simplification(PolyUOp *scheduled_root, int samples);
  * producers leave holes in are cleared per run (poly_hip_unwritten_slots), launches are
  * asynchronous on one stream and the launch sequence is replayed from a
  * hipGraph when the bound pointers repeat (in that graph, small launches that are
- * chains of dependent steps may run on a second branch beside the others, ordered by
+ * chains of dependent steps may run on side branches beside the others, ordered by
  * the buffers they share: poly_hip_plan_side_launches). */
 typedef struct PolyHipPlan PolyHipPlan;
 PolyHipPlan *poly_hip_compile_schedule(PolyCtx *ctx, const PolySchedule *schedule);
@@ -173,7 +173,7 @@ void *poly_hip_plan_slot_ptr(const PolyHipPlan *plan, int slot);
 /* Enable (1, default) or disable (0) hipGraph replay for this plan. */
 void poly_hip_plan_set_graph(PolyHipPlan *plan, int enabled);
 size_t poly_hip_plan_workspace_bytes(const PolyHipPlan *plan);
-/* How many launches of the plan its captured graph runs on a second stream beside the
+/* How many launches of the plan its captured graph runs on side streams beside the
  * main sequence (small launches that are a chain of dependent steps; 0 for most plans).
  * No counterpart in the reference, whose plans run kernel by kernel with a sync after
  * each (src/exec_plan.c:1000-1057). */
