@@ -119,6 +119,47 @@ def test_split_k_matmul_stays_in_bounds(tb, hiplib):
 
 
 @pytest.mark.skipif(not R.available(), reason="reference library not built")
+@pytest.mark.parametrize("b,t,m,n,tm", [(4, 64, 256, 384, False), (4, 64, 256, 384, True), (3, 64, 136, 200, False)])
+def test_matmul_over_two_reduce_ranges_stays_in_bounds(b, t, m, n, tm, hiplib):
+    """dW = X^T dY summed over batch and position on the plain bf16 template: the two reduce
+    ranges as one depth (nested strides) or as a depth of two levels (X stored time major),
+    a row-contiguous A and a column-contiguous B, ragged M and N in the last case."""
+    import graphs
+    c = R.Ctx()
+    _, _, _, sink = graphs.matmul_bf16_over_two_ranges(c, b, t, m, n, time_major_a=tm)
+    sched = c.schedule(sink)
+    try:
+        sp = C.cast(sched, C.POINTER(_ffi.PolySchedule)).contents
+        d = _ffi.take_string(hiplib.poly_hip_describe(sp.items[0].root, 0))
+        assert d.startswith("matmul-mfma: mfma 32x32x16 bf16") and "A:m-major B:n-major" in d, d
+        assert hostcheck.check_schedule(hiplib, sched) == 1
+    finally:
+        c.L.poly_schedule_free(sched)
+        c.close()
+
+
+@pytest.mark.skipif(not R.available(), reason="reference library not built")
+def test_slabs_that_share_operand_planes_stay_in_bounds(hiplib, monkeypatch):
+    """The training step with the bf16-planes path taken at this small size: the second slab
+    of the q/k/v derivative reads the first slab's planes of dS out of the scratch memory,
+    rows along the depth."""
+    import graphs
+    monkeypatch.setenv("POLY_HIP_BF16_SPLIT_MIN", "1048576")
+    c = R.Ctx()
+    _, sink = graphs.gpt2_block_train_step(c, 1, 128, 128, 2, 97)
+    sched = c.schedule(sink)
+    try:
+        sp = C.cast(sched, C.POINTER(_ffi.PolySchedule)).contents
+        descs = [_ffi.take_string(hiplib.poly_hip_describe(sp.items[i].root, 0)) for i in range(sp.n_items)]
+        slabs = [d for d in descs if "3 slabs of one output range" in d]
+        assert len(slabs) == 1 and "rows and depth exchanged" in slabs[0], slabs
+        assert hostcheck.check_schedule(hiplib, sched) > 60
+    finally:
+        c.L.poly_schedule_free(sched)
+        c.close()
+
+
+@pytest.mark.skipif(not R.available(), reason="reference library not built")
 @pytest.mark.parametrize("rows,cols", [(512, 192), (1024, 100), (544, 192)])
 def test_ordered_column_sum_stays_in_bounds(rows, cols, hiplib):
     """The order-preserving bf16 column sum (a kernel that writes the terms, one that adds
