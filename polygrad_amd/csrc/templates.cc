@@ -1153,6 +1153,68 @@ bool try_render_matmul_generic(const KernelGraph &g, const std::string &fn, cons
       if (!getenv("POLY_HIP_NO_SHARED_PLANES")) describe_operand(g, opnd[0], a_loads, mm.md_full, k_dims, mm.zd_full, M, K, Z, &mine);
       mine.parts = parts[0];
       const bool shared = opt.planes_before && M % 64 == 0 && K % 64 == 0 && exchanged(mine, *opt.planes_before);
+      // An operand that is a bf16 buffer read at an index of the plain template's kind needs
+      // no plane: the template reads it where it lies (the probabilities P in dv = P^T dO
+      // are 134 MB per layer that a copy would read and write again).  Needs whole K tiles
+      // (a padded depth would be read outside the buffer) and one reduce range.
+      struct InPlace { bool ok = false; Operand op; KSplit ks{0, 0, 0}; std::vector<Dim> rows, z; int64_t c0 = 0; };
+      InPlace in_place[2];
+      for (int side = 0; side < 2 && !getenv("POLY_HIP_NO_IN_PLACE_OPERAND"); side++) {
+        InPlace &ip = in_place[side];
+        if (parts[side] != 1 || K % 64 != 0 || kr.size() > 2 || (side == 0 && shared)) continue;
+        if (!match_operand(g, opnd[side], &ip.op) || ip.op.dt != DT_BF16) continue;
+        const Lin &l = g.lins[(size_t)ip.op.lin];
+        if (kr.size() == 1) {
+          if (!k_dependence(g, l, kr[0], K, &ip.ks) || ip.ks.kb < K) continue;
+        } else {
+          // two reduce ranges whose strides nest are one depth
+          const int64_t e0 = g.ranges[(size_t)kr[0]].extent, e1 = g.ranges[(size_t)kr[1]].extent;
+          KSplit k0, k1;
+          if (!k_dependence(g, l, kr[0], e0, &k0) || !k_dependence(g, l, kr[1], e1, &k1) || k0.kb != e0 || k1.kb != e1 || k0.s_lo != k1.s_lo * e1) continue;
+          ip.ks = KSplit{K, 0, k1.s_lo};
+        }
+        bool ok = true;
+        auto coefs = [&](const std::vector<Dim> &dims, std::vector<Dim> *out) {
+          for (const Dim &d : dims) {
+            std::vector<DigitUse> u;
+            if (!digit_uses(g, l, d.ord, &u)) { ok = false; return; }
+            int64_t c = 0;
+            for (const DigitUse &x : u)
+              if (d.cut >= x.a && (x.b == 0 || d.cut < x.a * x.b)) c += x.coef * (d.cut / x.a);
+            Dim e = d;
+            e.ca = side == 0 ? c : 0;
+            e.cb = side == 0 ? 0 : c;
+            out->push_back(e);
+          }
+        };
+        coefs(side == 0 ? mm.md_full : mm.nd_full, &ip.rows);
+        coefs(mm.zd_full, &ip.z);
+        // (the digits must be all there is to the index: checked against the canonical form
+        // at the far corner and at scattered points)
+        std::vector<int64_t> rv(g.ranges.size());
+        uint64_t rnd = 0x2545f4914f6cdd1dull;
+        for (int t = 0; t < 64 && ok; t++) {
+          std::fill(rv.begin(), rv.end(), 0);
+          int64_t want = l.c0, got = 0;
+          auto put = [&](const std::vector<Dim> &dims) {
+            for (const Dim &d : dims) {
+              rnd = rnd * 6364136223846793005ull + 1442695040888963407ull;
+              const int64_t digit = t == 0 ? d.extent - 1 : (int64_t)((rnd >> 33) % (uint64_t)d.extent);
+              rv[(size_t)d.ord] += digit * d.cut;
+              want += digit * (side == 0 ? d.ca : d.cb);
+            }
+          };
+          put(ip.rows); put(ip.z);
+          rnd = rnd * 6364136223846793005ull + 1442695040888963407ull;
+          const int64_t kk = t == 0 ? K - 1 : (int64_t)((rnd >> 33) % (uint64_t)K);
+          if (kr.size() == 1) rv[(size_t)kr[0]] = kk;
+          else { const int64_t e1 = g.ranges[(size_t)kr[1]].extent; rv[(size_t)kr[0]] = kk / e1; rv[(size_t)kr[1]] = kk % e1; }
+          want += kk * ip.ks.s_lo;
+          if (!eval_lin(g, l, rv, &got) || got != want) ok = false;
+        }
+        ip.c0 = l.c0;
+        ip.ok = ok;
+      }
       RenderedKernel::Pre pre[2];
       for (int side = 0; side < 2; side++) {
         const char *nm = side == 0 ? "a" : "b";
@@ -1172,7 +1234,13 @@ bool try_render_matmul_generic(const KernelGraph &g, const std::string &fn, cons
         pre[side].launch.grid[1] = (unsigned)Z;
         pre[side].launch.block[0] = 256;
       }
-      // the product of the planes, as the 16-bit template sees it
+      // the product of the planes, as the 16-bit template sees it (a second time with every
+      // operand as planes if the template does not take an operand where it lies)
+      for (int attempt = 0; attempt < 2; attempt++) {
+      if (attempt == 1) {
+        if (!in_place[0].ok && !in_place[1].ok) break;
+        in_place[0].ok = in_place[1].ok = false;
+      }
       MatmulMatch m2;
       m2.red = red; m2.K = P * KP; m2.M = M; m2.N = N; m2.Z = Z;
       m2.A.dt = m2.B.dt = DT_BF16;
@@ -1186,28 +1254,61 @@ bool try_render_matmul_generic(const KernelGraph &g, const std::string &fn, cons
         m2.ka = KSplit{KP, parts[0] == P ? M : 0, parts[0] * M};
         m2.md[0].ca = 1;
       }
+      if (in_place[0].ok || in_place[1].ok) {
+        // batch digits one by one: a plane operand's stride of a digit is the plane stride
+        // times the extents of the digits inside it
+        m2.zd.clear();
+        int64_t inner = 1;
+        std::vector<Dim> zs(mm.zd_full.size());
+        for (size_t i = mm.zd_full.size(); i-- > 0;) {
+          Dim d = mm.zd_full[i];
+          d.ca = in_place[0].ok ? in_place[0].z[i].ca : M * parts[0] * KP * inner;
+          d.cb = in_place[1].ok ? in_place[1].z[i].cb : N * parts[1] * KP * inner;
+          inner *= d.extent;
+          zs[i] = d;
+        }
+        m2.zd = zs;
+        if (in_place[0].ok) {
+          m2.md = in_place[0].rows;
+          collapse(m2.md);
+          m2.ka = KSplit{KP, 0, in_place[0].ks.s_lo};
+          m2.a_c0 = in_place[0].c0;
+          m2.A = in_place[0].op;
+        }
+        if (in_place[1].ok) {
+          m2.nd = in_place[1].rows;
+          collapse(m2.nd);
+          m2.kb = KSplit{KP, 0, in_place[1].ks.s_lo};
+          m2.b_c0 = in_place[1].c0;
+        }
+      }
       m2.md_full = mm.md_full; m2.nd_full = mm.nd_full; m2.zd_full = mm.zd_full;
       MatmulEpilogue ep2 = ep;
       ep2.signature += ", __bf16* poly_scratch";
       ep2.scratch_type = "__bf16";
-      ep2.scratch_used = scratch_bytes;
+      const size_t planes_bytes = in_place[1].ok ? std::max<size_t>(off_b, 256) : scratch_bytes;
+      ep2.scratch_used = planes_bytes;
       ep2.a_ptr = "((const __bf16*)poly_scratch)";
       ep2.b_ptr = strf("((const __bf16*)((const char*)poly_scratch + %zuull))", off_b);
+      if (in_place[0].ok) ep2.a_ptr = strf("data%d", in_place[0].op.param);
+      if (in_place[1].ok) ep2.b_ptr = strf("data%d", in_place[1].op.param);
       RenderedKernel main;
       if (render_matmul(m2, ep2, &main)) {
         *out = main;
         // planes first, then a split product's first stage
-        if (shared) out->pres.insert(out->pres.begin(), pre[1]);
-        else out->pres.insert(out->pres.begin(), {pre[0], pre[1]});
-        out->scratch_bytes = std::max(scratch_bytes, main.scratch_bytes);
+        if (!in_place[1].ok) out->pres.insert(out->pres.begin(), pre[1]);
+        if (!shared && !in_place[0].ok) out->pres.insert(out->pres.begin(), pre[0]);
+        out->scratch_bytes = std::max(planes_bytes, main.scratch_bytes);
         out->flops = 2.0 * (double)M * (double)N * (double)K * (double)Z;
         out->strategy = strf("operands as expressions, written as bf16 planes first (%d + %d planes of K=%lld, %.0f MB%s): ", parts[0], parts[1],
-                             (long long)KP, (double)scratch_bytes / 1e6,
-                             shared ? "; A is what the kernel before left as its A, rows and depth exchanged, and is not written again" : "") + out->strategy;
+                             (long long)KP, (double)planes_bytes / 1e6,
+                             shared ? "; A is what the kernel before left as its A, rows and depth exchanged, and is not written again"
+                             : in_place[0].ok ? "; A read in place" : in_place[1].ok ? "; B read in place" : "") + out->strategy;
         out->reads_planes_before = shared;
-        if (!shared) out->a_planes = mine;
+        if (!shared && !in_place[0].ok) out->a_planes = mine;
         for (RenderedKernel::Variant &v : out->variants) v.strategy = out->strategy;
         return true;
+      }
       }
     }
   }
