@@ -285,3 +285,39 @@ def test_matmul_of_fp32_operand_as_three_bf16_planes():
     assert_close(got32[O], want[O], rtol=1e-4, atol=bound, what="fp32 MFMA vs reference")
     # the two device paths agree far more closely than either needs to
     assert float(np.abs(got[O].astype(np.float64) - got32[O]).max()) <= 2e-5 * float(np.abs(w).max())
+
+
+@pytest.mark.parametrize("tb,batch", [(False, None), (True, None), (False, 3)])
+def test_plain_bf16_operand_beside_a_computed_one_is_read_in_place(tb, batch):
+    """fp32 x bf16 with a depth of whole K tiles: the fp32 operand goes to three bf16 planes,
+    the bf16 one is a buffer the template can read where it lies (rows along n, or along k
+    when stored transposed; also per batch) and gets no plane.  Against the reference, and
+    bit for bit against the same product with both operands as planes."""
+    import os
+    M, N, K = 256, 320, 4096 if batch is None else 2048
+    g = np.random.default_rng(5 + tb)
+    c = R.Ctx()
+    lead = () if batch is None else (batch,)
+    A = c.buffer(lead + (M, K), R.F32, name="A")
+    Bm = c.buffer(lead + ((N, K) if tb else (K, N)), R.BF16, name="B")
+    O = c.buffer(lead + (M, N), R.F32, name="C")
+    b = Bm.permute(tuple(range(len(lead))) + (len(lead) + 1, len(lead))) if tb else Bm
+    sink = c.sink((O, (A * c.const(0.75)).dot(b.cast(R.F32))))
+    arrays = {A: g.normal(0, 1, lead + (M, K)).astype(np.float32), Bm: bf16(g, lead + (K, N), 1.0), O: np.zeros(lead + (M, N), np.float32)}
+    os.environ["POLY_HIP_BF16_SPLIT_MIN"] = "1048576"
+    try:
+        want = run_ref(c, sink, arrays)
+        got, info = run_hip(c, sink, arrays)
+        assert any("B read in place" in k["desc"] for k in info), [k["desc"] for k in info]
+        os.environ["POLY_HIP_NO_IN_PLACE_OPERAND"] = "1"
+        try:
+            planes, info1 = run_hip(c, sink, arrays)
+        finally:
+            del os.environ["POLY_HIP_NO_IN_PLACE_OPERAND"]
+    finally:
+        del os.environ["POLY_HIP_BF16_SPLIT_MIN"]
+    c.close()
+    assert any("bf16 planes" in k["desc"] and "in place" not in k["desc"] for k in info1), [k["desc"] for k in info1]
+    bound = 1e-4 * float(np.abs(want[O]).mean()) * 8
+    assert_close(got[O], want[O], rtol=1e-4, atol=bound, what="operand in place vs reference")
+    assert got[O].tobytes() == planes[O].tobytes()

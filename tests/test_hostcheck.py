@@ -139,6 +139,29 @@ def test_matmul_over_two_reduce_ranges_stays_in_bounds(b, t, m, n, tm, hiplib):
 
 
 @pytest.mark.skipif(not R.available(), reason="reference library not built")
+@pytest.mark.parametrize("tb,batch", [(False, None), (True, None), (False, 3)])
+def test_operand_read_in_place_beside_planes_stays_in_bounds(tb, batch, hiplib, monkeypatch):
+    """fp32 x bf16 with the fp32 operand as three bf16 planes and the bf16 buffer read where
+    it lies (rows along n, rows along k, per batch), K dealt to three workgroups per tile."""
+    monkeypatch.setenv("POLY_HIP_BF16_SPLIT_MIN", "1048576")
+    M, N, K = 256, 320, 4096 if batch is None else 2048
+    c = R.Ctx()
+    lead = () if batch is None else (batch,)
+    A = c.buffer(lead + (M, K), R.F32, name="A")
+    Bm = c.buffer(lead + ((N, K) if tb else (K, N)), R.BF16, name="B")
+    O = c.buffer(lead + (M, N), R.F32, name="C")
+    b = Bm.permute(tuple(range(len(lead))) + (len(lead) + 1, len(lead))) if tb else Bm
+    sched = c.schedule(c.sink((O, (A * c.const(0.75)).dot(b.cast(R.F32)))))
+    try:
+        sp = C.cast(sched, C.POINTER(_ffi.PolySchedule)).contents
+        assert "B read in place" in _ffi.take_string(hiplib.poly_hip_describe(sp.items[0].root, 0))
+        assert hostcheck.check_schedule(hiplib, sched) == 3      # A's planes, the template, the adder of the partial results
+    finally:
+        c.L.poly_schedule_free(sched)
+        c.close()
+
+
+@pytest.mark.skipif(not R.available(), reason="reference library not built")
 def test_slabs_that_share_operand_planes_stay_in_bounds(hiplib, monkeypatch):
     """The training step with the bf16-planes path taken at this small size: the second slab
     of the q/k/v derivative reads the first slab's planes of dS out of the scratch memory,
