@@ -146,7 +146,7 @@ def run_gpu(workload, steps, warmup):
     if tokens is not None:
         ctx = [s for s in plan.slots if s.name == "positions"]
         extra["seq_len"] = ctx[0].numel if ctx else None
-    top = sorted(groups.items(), key=lambda kv: -kv[1]["ms"])[:8]
+    top = sorted(groups.items(), key=lambda kv: -kv[1]["ms"])[:int(os.environ.get("POLY_BENCH_GROUPS", "8"))]
     for key, g in top:
         log(f"  {g['ms']:8.3f} ms  x{g['launches']:3d}  {key[:150]}")
     plan.close()
