@@ -730,6 +730,7 @@ static bool match_row_chain_impl(const Sched &sc, int a_item, const std::vector<
   }
   collect_ref_loads(sc, A.m, &ref_loads);
   // grow: the readers of the latest result decide what comes next
+  const bool exports_ok = !getenv("POLY_HIP_NO_ROW_CHAIN_EXPORTS");
   std::vector<char> row_result{0};   // per result: a whole row (kept in registers) instead of one value per row
   int n_reduces = 1;
   for (;;) {
@@ -738,6 +739,9 @@ static bool match_row_chain_impl(const Sched &sc, int a_item, const std::vector<
     internal.insert(cur);
     int next_reduce = -1, next_map = -1;
     for (int r : sc.readers[(size_t)cur]) {
+      // (a reader far down the schedule -- the backward pass reading a statistic of the
+      // forward pass -- does not belong to the chain: the value is stored for it, below)
+      if (exports_ok && !row_result.back() && sc.step_of[(size_t)r] > sc.step_of[(size_t)a_item] + 16) continue;
       if (taken[(size_t)r]) return false;
       const KernelGraph &g = sc.graphs[(size_t)r];
       if (g.reduces.empty()) { if (next_map >= 0 && next_map != r) return false; next_map = r; }
@@ -811,23 +815,32 @@ static bool match_row_chain_impl(const Sched &sc, int a_item, const std::vector<
     phases.push_back(C);
     break;
   }
-  // every result is read inside the group only
+  // A result is read inside the group only, or it is one value per row that kernels
+  // behind the whole group read as well (the row maximum and the sum of a softmax, the mean
+  // and the variance of a LayerNorm in a training step, which the backward pass reads): the
+  // phase that makes such a value stores it, too.
   std::vector<int> items;
   for (const RowPhase &p : phases) items.push_back(p.m.item);
-  for (const auto &res : results)
-    for (int r : sc.readers[(size_t)res.first])
-      if (std::find(items.begin(), items.end(), r) == items.end()) FA_REJECT();
+  std::set<int> exported;
+  for (size_t ri = 0; ri < results.size(); ri++)
+    for (int r : sc.readers[(size_t)results[ri].first]) {
+      if (std::find(items.begin(), items.end(), r) != items.end()) continue;
+      if (!exports_ok || row_result[ri] || phases[ri].is_map || sc.step_of[(size_t)r] <= sc.step_of[(size_t)items.back()]) FA_REJECT();
+      exported.insert(results[ri].first);
+    }
   const int last_item = items.back();
   const int out_slot = out_slot_of(last_item);
   std::set<int> inputs;
   if (!group_is_schedulable(sc, items, a_item, last_item, internal, out_slot, &inputs)) FA_REJECT();
   for (const RowPhase &p : phases) if (!internal_loads_replaced(sc, p.m, internal, -1)) FA_REJECT();
+  for (int sl : exported) internal.erase(sl);      // they have memory, and the kernel gets them as arguments
 
   // ── code generation ────────────────────────────────────────────────────
   const int G = (R >= 4096 || (rows < 2048 && R >= 1024)) ? 256 : 64;
   std::vector<int> arg_slots;
   arg_slots.push_back(out_slot);
   for (int sl : inputs) arg_slots.push_back(sl);
+  for (int sl : exported) arg_slots.push_back(sl);
   auto arg_of = [&](int sl) { return (int)(std::find(arg_slots.begin(), arg_slots.end(), sl) - arg_slots.begin()); };
   auto call_args = [&](int item) {
     const KernelGraph &g = sc.graphs[(size_t)item];
@@ -849,7 +862,7 @@ static bool match_row_chain_impl(const Sched &sc, int a_item, const std::vector<
       if (p >= 0) dt = sc.graphs[(size_t)it].params[(size_t)p].dt;
     }
     if (j) sig += ", ";
-    sig += j == 0 ? strf("%s* fa%zu", dt_cname(dt), j) : strf("const %s* __restrict__ fa%zu", dt_cname(dt), j);
+    sig += j == 0 || exported.count(arg_slots[j]) ? strf("%s* fa%zu", dt_cname(dt), j) : strf("const %s* __restrict__ fa%zu", dt_cname(dt), j);
     bytes += (double)s->buf_slots[arg_slots[j]].nbytes;
   }
   // master row decomposition: fastest row range = smallest stride in the first result
@@ -877,7 +890,7 @@ static bool match_row_chain_impl(const Sched &sc, int a_item, const std::vector<
   // being repeated (the row is then read from memory once, not once per phase).
   struct RowCache { std::string key, type; int nit; };
   std::vector<RowCache> cache;
-  int n_cached_uses = 0;
+  int n_cached_uses = 0, n_exported = 0;
   int row_V = 0, row_nit = 0;       // vector width and step count of the rows kept between phases
   std::string row_decls;             // their declarations in the kernel body
   for (size_t pi = 0; pi < phases.size(); pi++) {
@@ -1028,8 +1041,17 @@ static bool match_row_chain_impl(const Sched &sc, int a_item, const std::vector<
       for (int n : pres) em.clear_preset(n);
       em.preset(ph.red, "acc");
       result_expr = em.emit(g.stores[0].value, &S0);
-      tail = S0.code + strf("  return %s;\n", result_expr.c_str());
       ret = dt_cname(g.n(g.stores[0].value).dt);
+      if (exported.count(results[pi].first)) {
+        // (phase pi makes result pi: every phase before the last map makes one)
+        const StoreInfo &st = g.stores[0];
+        const std::string idx = em.emit(g.n(st.index).src[1], &S0);
+        tail = S0.code + strf("  const %s res_ = %s;\n  if (lane == 0) data%d[%s] = res_;\n  return res_;\n", ret.c_str(), result_expr.c_str(),
+                              g.param_slot(st.param), idx.c_str());
+        n_exported++;
+      } else {
+        tail = S0.code + strf("  return %s;\n", result_expr.c_str());
+      }
     } else {
       const StoreInfo &st = g.stores[0];
       const int li = g.n(g.n(st.index).src[1]).lin;
@@ -1118,6 +1140,7 @@ static bool match_row_chain_impl(const Sched &sc, int a_item, const std::vector<
   rk.strategy = strf("row chain of %zu kernels (%s) G=%d R=%lld rows=%.0f", phases.size(), strat.c_str(), G, (long long)R, rows);
   if (n_cached_uses) rk.strategy += strf(", %d row loads kept in registers", n_cached_uses);
   if (row_V) rk.strategy += ", intermediate rows kept in registers";
+  if (n_exported) rk.strategy += strf(", %d row values stored for later kernels", n_exported);
   rk.n_params = (int)arg_slots.size();
   rk.bytes = bytes;
   return true;

@@ -141,6 +141,30 @@ def test_gpt2_block_train_step_matches_reference(B, T, D, H, V):
         assert any("3 slabs of one output range" in k["desc"] for k in info)
 
 
+def test_row_chains_store_the_row_values_that_the_backward_pass_reads():
+    """In a training step the statistics of the forward pass (mean and variance of every
+    LayerNorm, maximum and sum of the softmax) are read again by the backward pass, far
+    down the schedule.  The forward kernels still run as one row chain each: the phase that
+    makes such a value stores it as well.  Bit for bit against the same step with those
+    kernels launched one by one."""
+    import os
+    B, T, D, H, V, lr = 1, 128, 128, 2, 97, 3e-4
+    c = R.Ctx()
+    bufs, sink = graphs.gpt2_block_train_step(c, B, T, D, H, V, lr=lr)
+    arrays = graphs.gpt2_block_train_inputs(bufs, B, T, V)
+    got, info = run_hip(c, sink, arrays)
+    assert sum("row values stored for later kernels" in k["desc"] for k in info) >= 4, [k["desc"] for k in info if "row chain" in k["desc"]]
+    os.environ["POLY_HIP_NO_ROW_CHAIN_EXPORTS"] = "1"
+    try:
+        apart, info1 = run_hip(c, sink, arrays)
+    finally:
+        del os.environ["POLY_HIP_NO_ROW_CHAIN_EXPORTS"]
+    c.close()
+    assert not any("row values stored" in k["desc"] for k in info1) and len(info1) > len(info)
+    for name, t in bufs.items():
+        assert got[t].tobytes() == apart[t].tobytes(), name
+
+
 @pytest.mark.parametrize("T", [128, 1024])
 def test_slabs_of_the_qkv_derivative_share_operand_planes(T):
     """Two slabs of the derivative of the q | k | v split multiply by the same fp32 tensor
