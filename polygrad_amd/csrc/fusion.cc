@@ -2092,6 +2092,140 @@ static bool match_pointwise_group(const Sched &sc, int a_item, const std::vector
   return true;
 }
 
+// ── small independent pointwise kernels, side by side ──────────────────────────
+//
+// A training step casts every fp32 bias and LayerNorm parameter to bf16 before the forward
+// pass uses it: a kernel of one workgroup each, six per block of the model, spread over the
+// schedule, and a launch costs more than its work.  Kernels of at most 16 384 positions
+// without a reduction, with one ungated store at the flat position, that read only buffers
+// nobody has written before them in the schedule (parameters, inputs) and whose output
+// nobody else writes can run at the place of the first of them, in one launch: member i
+// owns the workgroups [first_i, first_i+1) of the grid.
+static bool match_side_by_side(const Sched &sc, int a_item, const std::vector<char> &taken, FusedGroup *out) {
+  const PolySchedule *s = sc.s;
+  if (getenv("POLY_HIP_NO_SIDE_BY_SIDE")) return false;
+  struct Sb { int item, ord, out_slot, V; int64_t E; unsigned blocks; };
+  auto candidate = [&](int item, Sb *sb) {
+    const KernelGraph &g = sc.graphs[(size_t)item];
+    if (!g.reduces.empty() || g.stores.size() != 1 || g.stores[0].gate >= 0 || !g.vars.empty()) return false;
+    if (g.stores[0].ranges.size() != 1 || g.ranges.size() != 1) return false;
+    const int ord = g.stores[0].ranges[0];
+    const int64_t E = g.ranges[(size_t)ord].extent;
+    if (E <= 0 || E > 16384) return false;
+    auto is_flat = [&](const Lin &l) {
+      if (l.c0 != 0 || l.terms.size() != 1 || l.terms[0].coef != 1) return false;
+      const Atom &a = g.atoms[(size_t)l.terms[0].atom];
+      return a.kind == Atom::RANGE && g.range_ord.at(a.node) == ord;
+    };
+    const int li = g.n(g.n(g.stores[0].index).src[1]).lin;
+    if (li < 0 || !is_flat(g.lins[(size_t)li])) return false;
+    if (g.n(g.stores[0].value).dt != g.n(g.stores[0].param).dt) return false;
+    const int out_slot = sc.slot(item, g.param_slot(g.stores[0].param));
+    if (!s->buf_slots[out_slot].is_intermediate || sc.writers[(size_t)out_slot].size() != 1 || s->buf_slots[out_slot].numel < E) return false;
+    int maxsz = 1;
+    for (size_t p = 0; p < g.params.size(); p++) {
+      if (!dt_is_float(g.params[p].dt)) return false;
+      maxsz = std::max(maxsz, dt_size(g.params[p].dt));
+      const int sl = sc.slot(item, (int)p);
+      if (sl == out_slot) { if (g.params[p].read) return false; continue; }
+      // nobody writes what it reads before it runs (then it may as well run earlier)
+      for (int w : sc.writers[(size_t)sl]) if (sc.step_of[(size_t)w] <= sc.step_of[(size_t)item]) return false;
+      std::vector<LoadRef> lds;
+      if (!loads_of(g, (int)p, &lds)) return false;
+      for (const LoadRef &l : lds) {
+        const Lin &lin = g.lins[(size_t)l.lin];
+        if (!is_flat(lin) && !lin.terms.empty()) return false;
+        if (is_flat(lin) && s->buf_slots[sl].numel < E) return false;
+      }
+    }
+    // the output is not read before the member's own place in the schedule anyway; nobody
+    // may read it in front of the launch either (nobody can: it has one writer, this kernel)
+    int V = std::max(1, 16 / maxsz);
+    while (V > 1 && E % V != 0) V /= 2;
+    *sb = {item, ord, out_slot, V, E, (unsigned)((E / V + 255) / 256)};
+    return true;
+  };
+  Sb first;
+  if (!candidate(a_item, &first)) return false;
+  std::vector<Sb> members{first};
+  for (int st = sc.step_of[(size_t)a_item] + 1; st < s->n_items && members.size() < 24; st++) {
+    const int k = s->exec_order[st];
+    Sb sb;
+    if (taken[(size_t)k] || !candidate(k, &sb)) continue;
+    members.push_back(sb);
+  }
+  if (members.size() < 2) return false;
+  std::vector<int> arg_slots;
+  std::map<int, DT> slot_dt;
+  std::set<int> written;
+  for (const Sb &m : members) {
+    const KernelGraph &g = sc.graphs[(size_t)m.item];
+    for (size_t p = 0; p < g.params.size(); p++) {
+      const int sl = sc.slot(m.item, (int)p);
+      if (written.count(sl)) return false;        // (a member reading another member's output: not independent)
+      slot_dt[sl] = g.params[p].dt;
+      if (std::find(arg_slots.begin(), arg_slots.end(), sl) == arg_slots.end()) arg_slots.push_back(sl);
+    }
+    written.insert(m.out_slot);
+  }
+  for (const Sb &m : members) {
+    const KernelGraph &g = sc.graphs[(size_t)m.item];
+    for (size_t p = 0; p < g.params.size(); p++) {
+      const int sl = sc.slot(m.item, (int)p);
+      if (sl != m.out_slot && written.count(sl)) return false;
+    }
+  }
+  auto arg_of = [&](int sl) { return (int)(std::find(arg_slots.begin(), arg_slots.end(), sl) - arg_slots.begin()); };
+  std::string code, body;
+  double bytes = 0;
+  unsigned first_block = 0;
+  for (size_t mi = 0; mi < members.size(); mi++) {
+    const Sb &sb = members[mi];
+    const KernelGraph &g = sc.graphs[(size_t)sb.item];
+    Member m;
+    m.item = sb.item;
+    m.range_expr[sb.ord] = "m";
+    const std::string fn = strf("poly_sb_%zu", mi);
+    const DT odt = g.n(g.stores[0].value).dt;
+    if (!emit_member_fn(sc, m, "", fn.c_str(), dt_cname(odt), "int poly_unused", g.stores[0].value, {}, false, false, &code)) return false;
+    std::string args;
+    for (size_t p = 0; p < g.params.size(); p++) args += strf("%sfa%d", p ? ", " : "", arg_of(sc.slot(sb.item, (int)p)));
+    const char *tn = dt_cname(odt);
+    body += strf("  %sif (blockIdx.x < %uu) {\n", mi ? "else " : "", first_block + sb.blocks);
+    body += strf("    const int pos = (int)((blockIdx.x - %uu) * 256u + threadIdx.x) * %d;\n    if (pos < %lld) {\n", first_block, sb.V, (long long)sb.E);
+    body += strf("      poly_vec<%s, %d> st;\n#pragma unroll\n      for (int u = 0; u < %d; u++) st.v[u] = %s(0, pos + u, 0, 0, %s);\n", tn, sb.V, sb.V, fn.c_str(), args.c_str());
+    body += strf("      poly_vstore<%s, %d>(fa%d + pos, st);\n    }\n  }\n", tn, sb.V, arg_of(sb.out_slot));
+    first_block += sb.blocks;
+  }
+  std::string sig;
+  for (size_t j = 0; j < arg_slots.size(); j++) {
+    const int sl = arg_slots[j];
+    if (j) sig += ", ";
+    if (written.count(sl)) sig += strf("%s* fa%zu", dt_cname(slot_dt[sl]), j);
+    else sig += strf("const %s* __restrict__ fa%zu", dt_cname(slot_dt[sl]), j);
+    bytes += (double)s->buf_slots[sl].nbytes;
+  }
+  std::string src = std::string(hip_prelude()) + code;
+  src += strf("extern \"C\" __global__ void __launch_bounds__(256) poly_k(%s) {\n", sig.c_str()) + body + "}\n";
+  out->items.clear();
+  for (const Sb &m : members) out->items.push_back(m.item);
+  out->launch_item = members.front().item;
+  out->internal_slots.clear();
+  out->arg_slots = arg_slots;
+  RenderedKernel &rk = out->rk;
+  rk = RenderedKernel();
+  rk.source = src;
+  rk.entry = "poly_k";
+  rk.launch.grid[0] = first_block;
+  rk.launch.block[0] = 256;
+  rk.klass = KernelClass::ELEMENTWISE;
+  rk.strategy = strf("%zu small independent pointwise kernels side by side in one launch", members.size());
+  rk.n_params = (int)arg_slots.size();
+  rk.n_vars = 0;
+  rk.bytes = bytes;
+  return true;
+}
+
 void find_fused_groups(const PolySchedule *s, const std::vector<KernelGraph> &graphs, std::vector<FusedGroup> *out) {
   out->clear();
   if (getenv("POLY_HIP_NO_FUSION")) return;
@@ -2127,6 +2261,15 @@ void find_fused_groups(const PolySchedule *s, const std::vector<KernelGraph> &gr
     if (taken[(size_t)k] || !graphs[(size_t)k].reduces.empty()) continue;
     FusedGroup fg;
     if (!match_pointwise_group(sc, k, taken, &fg)) continue;
+    for (int it : fg.items) taken[(size_t)it] = 1;
+    out->push_back(std::move(fg));
+  }
+  // small kernels that depend on nothing computed in the plan, wherever they stand
+  for (int st = 0; st < s->n_items; st++) {
+    const int k = s->exec_order[st];
+    if (taken[(size_t)k] || !graphs[(size_t)k].reduces.empty()) continue;
+    FusedGroup fg;
+    if (!match_side_by_side(sc, k, taken, &fg)) continue;
     for (int it : fg.items) taken[(size_t)it] = 1;
     out->push_back(std::move(fg));
   }

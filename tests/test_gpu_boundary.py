@@ -61,6 +61,7 @@ def test_partly_written_intermediate_reads_zero_where_nothing_was_stored(monkeyp
     for i in fx.external:
         assert fused[i].tobytes() == fx.expected[i].tobytes(), f"slot {i} ({fx.plan.names[i]}), pointwise kernels as one launch"
     monkeypatch.setenv("POLY_HIP_NO_POINTWISE_GROUPS", "1")
+    monkeypatch.setenv("POLY_HIP_NO_SIDE_BY_SIDE", "1")      # (kernels one by one, each at its place in the schedule)
     got, work, _ = _run(fx, runs=3)
     for i in fx.external:
         assert got[i].tobytes() == fx.expected[i].tobytes(), f"slot {i} ({fx.plan.names[i]})"

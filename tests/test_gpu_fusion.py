@@ -255,3 +255,41 @@ def test_table_epilogue_on_both_launches_of_a_product_with_leftover_columns():
             del os.environ[switch]
         assert got[O].tobytes() == other[O].tobytes(), switch
     c.close()
+
+
+def test_small_independent_kernels_run_side_by_side_in_one_launch():
+    """Casts of small fp32 parameters to bf16 that stand between larger kernels of a schedule
+    (as in a training step, where every bias and LayerNorm parameter is cast before use) read
+    nothing that the plan computes: they run as one launch at the place of the first, each
+    on its own workgroups.  Against the reference, and bit for bit against the kernels
+    launched one by one, where they stand."""
+    import os
+    c = R.Ctx()
+    g = np.random.default_rng(12)
+    rows, d = 512, 768
+    x = c.buffer((rows, d), R.BF16, name="x")
+    params = [c.buffer((n,), R.F32, name=f"p{i}") for i, n in enumerate((d, d, 3 * d, 1000))]
+    out = c.buffer((rows, d), R.BF16, name="out")
+    aux = c.buffer((1000,), R.BF16, name="aux")
+    h = x
+    for i, p in enumerate(params[:3]):
+        pc = p.cast(R.BF16).contiguous()                       # one small kernel each
+        pc = pc.shrink(((0, d),)) if pc.shape[0] != d else pc
+        h = ((h.cast(R.F32) * c.const(0.5 + i)).cast(R.BF16) + pc.reshape((1, d)).expand((rows, d))).contiguous()
+    sink = c.sink((out, h), (aux, (params[3] * c.const(3.0)).cast(R.BF16)))
+    arrays = {x: R.f32_to_bf16_bits(g.normal(0, 1, rows * d).astype(np.float32)), out: np.zeros(rows * d, np.uint16), aux: np.zeros(1000, np.uint16)}
+    for p in params:
+        arrays[p] = g.normal(0, 1, p.shape[0]).astype(np.float32)
+    want = run_ref(c, sink, arrays)
+    got, info = run_hip(c, sink, arrays)
+    assert any("small independent pointwise kernels side by side" in k["desc"] for k in info), [k["desc"] for k in info]
+    os.environ["POLY_HIP_NO_SIDE_BY_SIDE"] = "1"
+    try:
+        apart, info1 = run_hip(c, sink, arrays)
+    finally:
+        del os.environ["POLY_HIP_NO_SIDE_BY_SIDE"]
+    c.close()
+    assert len(info1) > len(info) and not any("side by side" in k["desc"] for k in info1)
+    for t in (out, aux):
+        assert got[t].tobytes() == apart[t].tobytes()
+        assert got[t].tobytes() == want[t].tobytes()
