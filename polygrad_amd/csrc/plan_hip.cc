@@ -526,9 +526,9 @@ PolyHipPlan *poly_hip_compile_schedule(PolyCtx *ctx, const PolySchedule *s) {
     // whose waits stay under one for eight side launches are taken.
     int n_on_side = 0, n_waits = 0, n_main_waits = 0;
     for (int i = 0; i < n_units; i++) n_on_side += plan->on_side[(size_t)i] != 0;
-    // (two by default: with the main stream and the default stream of the process they take
-    // the four hardware queues a process gets; a third side stream shares a queue with one
-    // of the others, and the 24-layer step came out 3 ms slower than on two)
+    // (two by default: on three the 24-layer step came out 1.6-3 ms slower than on two, with
+    // four hardware queues for the process and with eight alike -- the chains slow each
+    // other down, an adder that takes 48 us alone takes up to 110 us beside others)
     int max_streams = 2;
     if (const char *e = getenv("POLY_HIP_SIDE_STREAMS")) max_streams = std::max(1, std::min(kSideStreams, atoi(e)));
     for (int n_streams = max_streams; n_streams >= 1; n_streams--) {
