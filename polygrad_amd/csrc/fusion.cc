@@ -2226,6 +2226,151 @@ static bool match_side_by_side(const Sched &sc, int a_item, const std::vector<ch
   return true;
 }
 
+// ── ordered column sums, side by side ─────────────────────────────────────────
+//
+// The order-preserving column sums of a training step (bias and LayerNorm-parameter
+// gradients that accumulate in bf16) are two kernels each: the terms, over the whole chip,
+// and an adder of one thread per output whose time is a chain of dependent additions
+// (48 us for 4096 terms) however few outputs there are.  Several of them that depend on
+// nothing between them run as one pair of launches at the place of the first: the terms
+// kernels on consecutive ranges of workgroups, and so the adders, each with its own part of
+// the scratch memory.  The members are rendered as they would be alone and called as device
+// functions with their workgroup number passed in.
+static bool match_ordered_sums_side_by_side(const Sched &sc, int a_item, const std::vector<char> &taken, FusedGroup *out) {
+  const PolySchedule *s = sc.s;
+  if (getenv("POLY_HIP_NO_MERGED_ADDERS")) return false;
+  struct Ad { int item, out_slot; RenderedKernel rk; };
+  auto candidate = [&](int item, Ad *ad) {
+    const KernelGraph &g = sc.graphs[(size_t)item];
+    if (g.reduces.size() != 1 || g.stores.size() != 1 || !g.vars.empty()) return false;
+    const int out_slot = sc.slot(item, g.param_slot(g.stores[0].param));
+    if (s->buf_slots[out_slot].numel > 16384 || sc.writers[(size_t)out_slot].size() != 1) return false;
+    std::string err;
+    RenderedKernel rk;
+    if (!render_kernel(g, "poly_m", RenderOptions(), &rk, &err)) return false;
+    if (rk.klass != KernelClass::THREAD_REDUCE || rk.pres.size() != 1 || rk.strategy.rfind("ordered reduce, stage 1", 0) != 0 || !rk.guards.empty() ||
+        !rk.tables.empty() || rk.variants.size() > 1 || rk.n_vars != 0 || !rk.fallback_source.empty() || rk.n_params != (int)g.params.size())
+      return false;
+    if (rk.launch.block[0] != 64 || rk.pres[0].launch.block[0] != 256 || rk.launch.grid[1] != 1 || rk.pres[0].launch.grid[1] != 1) return false;
+    ad->item = item;
+    ad->out_slot = out_slot;
+    ad->rk = std::move(rk);
+    return true;
+  };
+  std::vector<Ad> members(1);
+  if (!candidate(a_item, &members[0])) return false;
+  const int first_step = sc.step_of[(size_t)a_item];
+  std::set<int> outs{members[0].out_slot};
+  uint64_t threads = (uint64_t)members[0].rk.launch.grid[0] * 64;
+  for (int st = first_step + 1; st < s->n_items && st < first_step + 96 && members.size() < 8; st++) {
+    const int k = s->exec_order[st];
+    if (taken[(size_t)k] || sc.graphs[(size_t)k].reduces.size() != 1) continue;
+    // what it reads is there before the first member runs, and is no member's output
+    const KernelGraph &g = sc.graphs[(size_t)k];
+    bool ready = true;
+    for (size_t p = 0; p < g.params.size() && ready; p++) {
+      const int sl = sc.slot(k, (int)p);
+      if (outs.count(sl)) ready = false;
+      if (!g.params[p].read) continue;
+      for (int w : sc.writers[(size_t)sl]) if (w != k && sc.step_of[(size_t)w] >= first_step) ready = false;
+    }
+    if (!ready) continue;
+    Ad ad;
+    if (!candidate(k, &ad)) continue;
+    if (threads + (uint64_t)ad.rk.launch.grid[0] * 64 > 65536) break;
+    threads += (uint64_t)ad.rk.launch.grid[0] * 64;
+    outs.insert(ad.out_slot);
+    members.push_back(std::move(ad));
+  }
+  if (members.size() < 2) return false;
+  // a kernel as a device function of its workgroup number
+  const std::string prelude = hip_prelude();
+  auto as_device_fn = [&](const std::string &src, const std::string &entry, const std::string &name, std::string *fn) {
+    if (src.compare(0, prelude.size(), prelude) != 0) return false;
+    std::string t = src.substr(prelude.size());
+    const std::string head = "extern \"C\" __global__ void __launch_bounds__(";
+    if (t.compare(0, head.size(), head) != 0) return false;        // (helpers of its own in front: names could clash)
+    const size_t open = t.find(entry + "(");
+    if (open == std::string::npos || open > 128) return false;
+    t = "__device__ __forceinline__ void " + name + "(const unsigned int poly_bid, " + t.substr(open + entry.size() + 1);
+    for (size_t at = t.find("blockIdx.x"); at != std::string::npos; at = t.find("blockIdx.x", at)) t.replace(at, 10, "poly_bid");
+    if (t.find("blockIdx") != std::string::npos || t.find("__shared__") != std::string::npos) return false;
+    *fn = t;
+    return true;
+  };
+  std::vector<int> arg_slots;
+  std::map<int, DT> slot_dt;
+  std::set<int> written;
+  for (const Ad &m : members) {
+    const KernelGraph &g = sc.graphs[(size_t)m.item];
+    for (size_t p = 0; p < g.params.size(); p++) {
+      const int sl = sc.slot(m.item, (int)p);
+      if (slot_dt.count(sl) && slot_dt[sl] != g.params[p].dt) return false;
+      slot_dt[sl] = g.params[p].dt;
+      if (g.params[p].written) written.insert(sl);
+      if (std::find(arg_slots.begin(), arg_slots.end(), sl) == arg_slots.end()) arg_slots.push_back(sl);
+    }
+  }
+  auto arg_of = [&](int sl) { return (int)(std::find(arg_slots.begin(), arg_slots.end(), sl) - arg_slots.begin()); };
+  std::string code, pre_body, main_body;
+  size_t scratch = 0;
+  unsigned pre_blocks = 0, main_blocks = 0;
+  double bytes = 0;
+  for (size_t mi = 0; mi < members.size(); mi++) {
+    const Ad &m = members[mi];
+    const KernelGraph &g = sc.graphs[(size_t)m.item];
+    std::string f1, f2;
+    if (!as_device_fn(m.rk.pres[0].source, m.rk.pres[0].entry, strf("poly_terms_%zu", mi), &f1) ||
+        !as_device_fn(m.rk.source, m.rk.entry, strf("poly_adder_%zu", mi), &f2))
+      return false;
+    code += f1 + f2;
+    std::string args;
+    for (size_t p = 0; p < g.params.size(); p++) args += strf("fa%d, ", arg_of(sc.slot(m.item, (int)p)));
+    args += strf("(float*)((char*)poly_scratch + %zuull)", scratch);
+    pre_body += strf("  %sif (blockIdx.x < %uu) poly_terms_%zu(blockIdx.x - %uu, %s);\n", mi ? "else " : "", pre_blocks + m.rk.pres[0].launch.grid[0], mi,
+                     pre_blocks, args.c_str());
+    main_body += strf("  %sif (blockIdx.x < %uu) poly_adder_%zu(blockIdx.x - %uu, %s);\n", mi ? "else " : "", main_blocks + m.rk.launch.grid[0], mi,
+                      main_blocks, args.c_str());
+    pre_blocks += m.rk.pres[0].launch.grid[0];
+    main_blocks += m.rk.launch.grid[0];
+    scratch += (m.rk.scratch_bytes + 255) / 256 * 256;
+    bytes += m.rk.bytes;
+  }
+  if (scratch > ((size_t)1 << 30)) return false;
+  std::string sig;
+  for (size_t j = 0; j < arg_slots.size(); j++) {
+    const int sl = arg_slots[j];
+    if (written.count(sl)) sig += strf("%s* fa%zu, ", dt_cname(slot_dt[sl]), j);
+    else sig += strf("const %s* __restrict__ fa%zu, ", dt_cname(slot_dt[sl]), j);
+  }
+  sig += "float* poly_scratch";
+  const std::string common = prelude + code;
+  out->items.clear();
+  for (const Ad &m : members) out->items.push_back(m.item);
+  out->launch_item = members.front().item;
+  out->internal_slots.clear();
+  out->arg_slots = arg_slots;
+  RenderedKernel &rk = out->rk;
+  rk = RenderedKernel();
+  RenderedKernel::Pre pre;
+  pre.source = common + strf("extern \"C\" __global__ void __launch_bounds__(256) poly_k(%s) {\n", sig.c_str()) + pre_body + "}\n";
+  pre.entry = "poly_k";
+  pre.launch.grid[0] = pre_blocks;
+  pre.launch.block[0] = 256;
+  rk.pres.push_back(pre);
+  rk.source = common + strf("extern \"C\" __global__ void __launch_bounds__(64) poly_k(%s) {\n", sig.c_str()) + main_body + "}\n";
+  rk.entry = "poly_k";
+  rk.launch.grid[0] = main_blocks;
+  rk.launch.block[0] = 64;
+  rk.scratch_bytes = scratch;
+  rk.klass = KernelClass::THREAD_REDUCE;
+  rk.strategy = strf("%zu ordered column sums side by side (terms in one launch, adders in one): ", members.size()) + members[0].rk.strategy;
+  rk.n_params = (int)arg_slots.size();
+  rk.n_vars = 0;
+  rk.bytes = bytes;
+  return true;
+}
+
 void find_fused_groups(const PolySchedule *s, const std::vector<KernelGraph> &graphs, std::vector<FusedGroup> *out) {
   out->clear();
   if (getenv("POLY_HIP_NO_FUSION")) return;
@@ -2261,6 +2406,15 @@ void find_fused_groups(const PolySchedule *s, const std::vector<KernelGraph> &gr
     if (taken[(size_t)k] || !graphs[(size_t)k].reduces.empty()) continue;
     FusedGroup fg;
     if (!match_pointwise_group(sc, k, taken, &fg)) continue;
+    for (int it : fg.items) taken[(size_t)it] = 1;
+    out->push_back(std::move(fg));
+  }
+  // the order-preserving column sums that are left, several to a launch
+  for (int st = 0; st < s->n_items; st++) {
+    const int k = s->exec_order[st];
+    if (taken[(size_t)k] || graphs[(size_t)k].reduces.size() != 1) continue;
+    FusedGroup fg;
+    if (!match_ordered_sums_side_by_side(sc, k, taken, &fg)) continue;
     for (int it : fg.items) taken[(size_t)it] = 1;
     out->push_back(std::move(fg));
   }

@@ -365,7 +365,9 @@ PolyHipPlan *poly_hip_compile_schedule(PolyCtx *ctx, const PolySchedule *s) {
     for (int ui = 0; ui < n_units; ui++) {
       const Unit &u = plan->units[(size_t)ui];
       const HipRunner *r = u.runner;
-      bool small = threads_of(r->rk.launch) <= 16384 && r->guards.empty() && r->rk.variants.size() < 2 && r->rk.pres_key.empty();
+      // (several column sums as one launch are still a chain: up to 65 536 threads there)
+      const uint64_t most = r->rk.klass == KernelClass::THREAD_REDUCE ? 65536 : 16384;
+      bool small = threads_of(r->rk.launch) <= most && r->guards.empty() && r->rk.variants.size() < 2 && r->rk.pres_key.empty();
       for (const RenderedKernel::Pre &pk : r->rk.pres) small = small && (r->rk.klass == KernelClass::THREAD_REDUCE || threads_of(pk.launch) <= 16384);
       int follows = 0;
       for (int sl : u.slots) if (!follows) follows = side_wrote[(size_t)sl];

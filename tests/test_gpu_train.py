@@ -165,6 +165,31 @@ def test_row_chains_store_the_row_values_that_the_backward_pass_reads():
         assert got[t].tobytes() == apart[t].tobytes(), name
 
 
+def test_ordered_column_sums_of_a_step_run_side_by_side():
+    """The order-preserving bf16 column sums of the backward pass (bias and LayerNorm-parameter
+    gradients: a terms kernel and an in-order adder each) that depend on nothing between
+    them run as one pair of launches, every member on its own workgroups and its own part
+    of the scratch memory.  Bit for bit against the same step with every sum launched by
+    itself."""
+    import os
+    B, T, D, H, V, lr = 2, 256, 128, 4, 301, 3e-4      # 512 rows: long enough for the ordered form
+    c = R.Ctx()
+    bufs, sink = graphs.gpt2_block_train_step(c, B, T, D, H, V, lr=lr)
+    arrays = graphs.gpt2_block_train_inputs(bufs, B, T, V)
+    got, info = run_hip(c, sink, arrays)
+    merged = [k["desc"] for k in info if "ordered column sums side by side" in k["desc"]]
+    assert merged, [k["desc"] for k in info if "ordered" in k["desc"]]
+    os.environ["POLY_HIP_NO_MERGED_ADDERS"] = "1"
+    try:
+        apart, info1 = run_hip(c, sink, arrays)
+    finally:
+        del os.environ["POLY_HIP_NO_MERGED_ADDERS"]
+    c.close()
+    assert not any("side by side (terms" in k["desc"] for k in info1) and len(info1) > len(info)
+    for name, t in bufs.items():
+        assert got[t].tobytes() == apart[t].tobytes(), name
+
+
 @pytest.mark.parametrize("T", [128, 1024])
 def test_slabs_of_the_qkv_derivative_share_operand_planes(T):
     """Two slabs of the derivative of the q | k | v split multiply by the same fp32 tensor
