@@ -177,6 +177,33 @@ def test_gpt2_medium_train_matmul_shapes(m, n, k, ta, tb):
     assert bool((err <= 1e-4 * bound + 1e-30).all()), f"max err/bound {float((err / bound).max()):.3e}"
 
 
+@pytest.mark.parametrize("m,n", [(1024, 1024), (3072, 1024), (1024, 4096)])
+def test_gpt2_medium_weight_gradient_over_batch_and_position(m, n):
+    """dW = sum over (b, t) of X[b, t, :]^T dY[b, t, :] at the shapes of the train step, as the
+    scheduler hands it over: one REDUCE over two ranges.  On the plain template (operands read
+    in place; 1024 x 1024 has its depth dealt to two workgroups per tile), against float64 on
+    sampled rows."""
+    import torch
+    b, t = 4, 1024
+    c = R.Ctx()
+    X, Y, O, sink = graphs.matmul_bf16_over_two_ranges(c, b, t, m, n)
+    g = np.random.default_rng(m + 3 * n)
+    x_bits = R.f32_to_bf16_bits(g.normal(0, 0.05, b * t * m).astype(np.float32))
+    y_bits = R.f32_to_bf16_bits(g.normal(0, 0.05, b * t * n).astype(np.float32))
+    got, info = run_hip(c, sink, {X: x_bits, Y: y_bits, O: np.full(m * n, np.nan, np.float32)})
+    c.close()
+    assert all(k_["klass"] == "matmul-mfma" and "planes" not in k_["desc"] for k_ in info), [k_["desc"] for k_ in info]
+    C = torch.from_numpy(got[O]).view(m, n)
+    assert bool(torch.isfinite(C).all())
+    x = torch.from_numpy(R.bf16_bits_to_f32(x_bits)).double().view(b * t, m)
+    y = torch.from_numpy(R.bf16_bits_to_f32(y_bits)).double().view(b * t, n)
+    rows = sorted({0, 1, 127, 128, 255, 256, m // 2, m - 129, m - 1})
+    want = x[:, rows].t() @ y
+    bound = x[:, rows].abs().t() @ y.abs()
+    err = (C[rows].double() - want).abs()
+    assert bool((err <= 1e-4 * bound + 1e-30).all()), f"max err/bound {float((err / bound).max()):.3e}"
+
+
 # fp32 operands: the 32x32x2 MFMA template.  (m, n, k, A stored (k, m), B stored (n, k), batch)
 F32_SHAPES = [
     (4096, 512, 784, False, True, None),    # config 1 forward: X W1^T
