@@ -1,5 +1,5 @@
 #!/usr/bin/env python3
-"""Applies the HIP-backend integration edits (the ones INTEGRATION.md describes) to a
+"""Applies the HIP-backend integration edits (a device id, a table row, the whole-plan hook) to a
 SCRATCH COPY of the polygrad source tree.  Test infrastructure: `make -C oracle ref_hip`
 copies the tree to a temporary directory, runs this script on the copy, compiles it into
 oracle/_ref/libpolygrad_hip_ref.so linked against libpolygrad_hip.so, and deletes the

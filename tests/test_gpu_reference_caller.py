@@ -5,7 +5,7 @@ staging of host-resident bindings, device-resident training state) and linked ag
 libpolygrad_hip.so.  The tests follow the reference's own pattern for a device backend:
 test/test_cuda.c:438-516 (poly_realize with device-domain bindings next to the same graph
 with host bindings) and :533-652 (poly_instance_set_device, forward parity, CPU <-> device
-round trips), plus what SURVEY lists as broken on any device today: training steps whose
+round trips), plus what is broken in the reference on any device today: training steps whose
 loss and bias-correction slots are host addresses (src/instance.c:1299-1311), value_and_grad
 with host-resident outputs (src/instance.c:1027-1043), constants of the frontend's registry
 (src/frontend.c:2231-2232).  Each test runs the whole-plan hook and, with
