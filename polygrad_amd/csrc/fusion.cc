@@ -2122,6 +2122,8 @@ static bool match_side_by_side(const Sched &sc, int a_item, const std::vector<ch
     if (g.n(g.stores[0].value).dt != g.n(g.stores[0].param).dt) return false;
     const int out_slot = sc.slot(item, g.param_slot(g.stores[0].param));
     if (!s->buf_slots[out_slot].is_intermediate || sc.writers[(size_t)out_slot].size() != 1 || s->buf_slots[out_slot].numel < E) return false;
+    // (nobody reads the output in front of the kernel: such a reader would see it filled early)
+    for (int r : sc.readers[(size_t)out_slot]) if (sc.step_of[(size_t)r] <= sc.step_of[(size_t)item]) return false;
     int maxsz = 1;
     for (size_t p = 0; p < g.params.size(); p++) {
       if (!dt_is_float(g.params[p].dt)) return false;
@@ -2245,6 +2247,8 @@ static bool match_ordered_sums_side_by_side(const Sched &sc, int a_item, const s
     if (g.reduces.size() != 1 || g.stores.size() != 1 || !g.vars.empty()) return false;
     const int out_slot = sc.slot(item, g.param_slot(g.stores[0].param));
     if (s->buf_slots[out_slot].numel > 16384 || sc.writers[(size_t)out_slot].size() != 1) return false;
+    // (nobody reads the output in front of the kernel: such a reader would see it filled early)
+    for (int r : sc.readers[(size_t)out_slot]) if (sc.step_of[(size_t)r] <= sc.step_of[(size_t)item]) return false;
     std::string err;
     RenderedKernel rk;
     if (!render_kernel(g, "poly_m", RenderOptions(), &rk, &err)) return false;
