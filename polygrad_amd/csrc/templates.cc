@@ -327,12 +327,92 @@ bool matmul_store_contiguous(const KernelGraph &g, const MatmulMatch &mm, const 
 // value/address split when rows are contiguous along n).
 static bool epilogue_from_graph(const KernelGraph &g, const MatmulMatch &mm, MatmulEpilogue *epo) {
   const StoreInfo &st = g.stores[0];
+  // Parts of the epilogue that are functions of ONE 16-bit value it loads (the derivative of
+  // GELU at the saved pre-activation, in bf16 arithmetic: an exponential and three divisions
+  // among some twenty operations, each rounded to bf16) have 65 536 possible values: a table
+  // filled once by the same expression replaces the arithmetic, bit for bit.  Taken are the
+  // largest such parts of six operations or more, four tables at most.
+  struct Part { int node, load; };
+  std::vector<Part> parts;
+  if (!getenv("POLY_HIP_NO_LUT")) {
+    struct Info { bool known = false, impure = false; int load = -1, n_alu = 0; };
+    std::vector<Info> info(g.nodes.size());
+    std::function<const Info &(int)> look = [&](int id) -> const Info & {
+      Info &f = info[(size_t)id];
+      if (f.known) return f;
+      f.known = true;
+      const KNode &k = g.n(id);
+      if (k.op == POLY_OP_CONST) return f;
+      if (k.op == POLY_OP_LOAD) {
+        const KNode &ix = g.n(k.src[0]);
+        if ((k.dt == DT_BF16 || k.dt == DT_F16) && k.guard < 0 && ix.op == POLY_OP_INDEX && ix.src.size() == 2) f.load = id;
+        else f.impure = true;
+        return f;
+      }
+      if (id == mm.red || k.src.empty() || k.op == POLY_OP_RANGE || k.op == POLY_OP_INDEX || k.op == POLY_OP_PARAM || k.op == POLY_OP_DEFINE_VAR ||
+          k.op == POLY_OP_REDUCE || k.op == POLY_OP_SPECIAL || k.op == POLY_OP_BIND) { f.impure = true; return f; }
+      f.n_alu = 1;
+      for (int c : k.src) {
+        const Info ci = look(c);
+        if (ci.impure) f.impure = true;
+        if (ci.load >= 0) { if (f.load >= 0 && f.load != ci.load) f.impure = true; f.load = ci.load; }
+        f.n_alu += ci.n_alu;
+      }
+      return f;
+    };
+    std::vector<char> seen(g.nodes.size(), 0);
+    std::function<void(int)> visit = [&](int id) {
+      if (seen[(size_t)id]) return;
+      seen[(size_t)id] = 1;
+      const Info f = look(id);
+      const KNode &k = g.n(id);
+      if (!f.impure && f.load >= 0 && f.n_alu >= 6 && dt_is_float(k.dt) && dt_size(k.dt) <= 4) {
+        if (parts.size() < 4) parts.push_back({id, f.load});
+        return;
+      }
+      if (id == mm.red || k.op == POLY_OP_LOAD) return;
+      for (int c : k.src) visit(c);
+    };
+    visit(st.value);
+  }
+  MatmulEpilogue &ep0 = *epo;
+  std::vector<std::pair<int, int>> lut_of;       // (node, load) of table i
+  for (const Part &pt : parts) {
+    Emitter et(g);
+    Scope St;
+    St.indent = 1;
+    et.preset(pt.load, "x");
+    const std::string v = et.emit(pt.node, &St);
+    if (et.failed() || et.uses_threefry) continue;
+    const DT odt = g.n(pt.node).dt, idt = g.n(pt.load).dt;
+    RenderedKernel::Table t;
+    t.source = std::string(hip_prelude()) +
+               strf("extern \"C\" __global__ void __launch_bounds__(256) poly_lut_fill(%s* out) {\n"
+                    "  const unsigned int i = blockIdx.x * 256u + threadIdx.x;\n"
+                    "  const %s x = __builtin_bit_cast(%s, (unsigned short)i);\n",
+                    dt_cname(odt), dt_cname(idt), dt_cname(idt)) +
+               St.code + strf("  out[i] = %s;\n}\n", v.c_str());
+    t.entry = "poly_lut_fill";
+    t.bytes = (size_t)65536 * (size_t)dt_size(odt);
+    t.launch.grid[0] = 256;
+    t.launch.block[0] = 256;
+    ep0.tables.push_back(t);
+    lut_of.push_back({pt.node, pt.load});
+  }
+  // (an emitter reads a table entry in place of the part: the load first, then the lookup)
+  auto use_tables = [&](Emitter &e, Scope *S) {
+    for (size_t i = 0; i < lut_of.size(); i++) {
+      const std::string x = e.emit(lut_of[i].second, S);
+      e.preset(lut_of[i].first, strf("poly_lut%zu[__builtin_bit_cast(unsigned short, %s)]", i, x.c_str()));
+    }
+  };
   Emitter em(g);
   Scope S0;
   S0.indent = 1;
   for (int r : st.ranges) S0.avail |= (uint64_t)1 << r;
   std::string decomp = matmul_decompose(mm, &em);
   em.preset(mm.red, "acc");
+  use_tables(em, &S0);
   std::string val = em.emit(st.value, &S0);
   std::string idx = em.emit(g.n(st.index).src[1], &S0);
   if (em.failed()) return reject(__LINE__);
@@ -346,6 +426,11 @@ static bool epilogue_from_graph(const KernelGraph &g, const MatmulMatch &mm, Mat
     else ep.signature += strf("const %s* __restrict__ data%zu", dt_cname(p.dt), i);
     params_call += strf("data%zu", i);
   }
+  for (size_t i = 0; i < ep.tables.size(); i++) {
+    ep.signature += strf(", const %s* __restrict__ poly_lut%zu", dt_cname(g.n(lut_of[i].first).dt), i);
+    params_call += strf(", poly_lut%zu", i);
+  }
+  ep.params_call = params_call;
   ep.code = strf("__device__ __forceinline__ void poly_epilogue(float acc, int m, int n, int z, %s) {\n", ep.signature.c_str());
   ep.code += decomp + S0.code;
   ep.code += strf("  data%d[%s] = %s;\n}\n", pout, idx.c_str(), val.c_str());
@@ -362,6 +447,7 @@ static bool epilogue_from_graph(const KernelGraph &g, const MatmulMatch &mm, Mat
       matmul_decompose(mm, &ev);
       matmul_decompose(mm, &ea);
       ev.preset(mm.red, "acc");
+      use_tables(ev, &Sv);
       std::string v2 = ev.emit(st.value, &Sv);
       std::string i2 = ea.emit(g.n(st.index).src[1], &Sa);
       if (!ev.failed() && !ea.failed()) {
@@ -397,7 +483,14 @@ bool try_render_matmul(const KernelGraph &g, const std::string &fn, const Render
   if (!epilogue_from_graph(g, mm, &ep)) return false;
   ep.a_ptr = strf("data%d", mm.A.param);
   ep.b_ptr = strf("data%d", mm.B.param);
-  return render_matmul(mm, ep, out);
+  if (!render_matmul(mm, ep, out)) return false;
+  out->tables = ep.tables;
+  if (!ep.tables.empty()) {
+    const std::string note = strf(", %zu parts of the epilogue as 16-bit lookup tables", ep.tables.size());
+    out->strategy += note;
+    for (RenderedKernel::Variant &v : out->variants) v.strategy += note;
+  }
+  return true;
 }
 
 // Second stage of a split-K product: adds the S partial accumulators of an output element
@@ -1003,8 +1096,7 @@ bool try_render_matmul_generic(const KernelGraph &g, const std::string &fn, cons
 
   MatmulEpilogue ep;
   if (!epilogue_from_graph(g, mm, &ep)) return reject(__LINE__);
-  std::string params_call;
-  for (size_t i = 0; i < g.params.size(); i++) params_call += strf("%sdata%zu", i ? ", " : "", i);
+  const std::string params_call = ep.params_call;
 
   // C text that splits flattened coordinate `var` into digits (last one fastest); the
   // value of a range is the sum of its digits times their cuts over the coordinates a
@@ -1304,6 +1396,8 @@ bool try_render_matmul_generic(const KernelGraph &g, const std::string &fn, cons
                              (long long)KP, (double)planes_bytes / 1e6,
                              shared ? "; A is what the kernel before left as its A, rows and depth exchanged, and is not written again"
                              : in_place[0].ok ? "; A read in place" : in_place[1].ok ? "; B read in place" : "") + out->strategy;
+        out->tables = ep.tables;
+        if (!ep.tables.empty()) out->strategy += strf(", %zu parts of the epilogue as 16-bit lookup tables", ep.tables.size());
         out->reads_planes_before = shared;
         if (!shared && !in_place[0].ok) out->a_planes = mine;
         for (RenderedKernel::Variant &v : out->variants) v.strategy = out->strategy;
@@ -1344,6 +1438,8 @@ bool try_render_matmul_generic(const KernelGraph &g, const std::string &fn, cons
   out->n_vars = 0;
   out->flops = 2.0 * (double)M * (double)N * (double)K * (double)Z;
   out->bytes = ep.bytes;
+  out->tables = ep.tables;
+  if (!ep.tables.empty()) out->strategy += strf(", %zu parts of the epilogue as 16-bit lookup tables", ep.tables.size());
   return true;
 }
 

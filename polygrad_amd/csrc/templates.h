@@ -68,6 +68,10 @@ struct MatmulEpilogue {
   // can put its partial results behind them.  Empty: no such parameter yet.
   std::string scratch_type;
   size_t scratch_used = 0;
+  // Lookup tables the epilogue reads (parameters `poly_lut<i>` at the end of `signature`,
+  // in front of any scratch pointer), and the argument list that goes with `signature`.
+  std::vector<RenderedKernel::Table> tables;
+  std::string params_call;
 };
 // Is element (m, n + 1) of the kernel's output stored right after (m, n), for every n
 // that is not the last of an aligned group of 8?  (store index affine with coefficient 1
