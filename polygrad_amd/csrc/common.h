@@ -2,6 +2,7 @@
 // ("polygrad: <area>: message" on stderr, negative int / NULL returns, never
 // abort) and a tiny printf-style string builder.
 #pragma once
+#include <cstdlib>
 #include <cstdarg>
 #include <cstdint>
 #include <cstdio>
@@ -11,6 +12,15 @@
 #include "polygrad_abi.h"
 
 namespace polyhip {
+
+// Switches that change results (they skip work so that the rest can be timed) exist only
+// in a measurement build of the library (make MEASURE=1); the default build ignores them.
+#ifdef POLY_HIP_MEASUREMENT_BUILD
+inline const char *measurement_env(const char *name) { return getenv(name); }
+#else
+inline const char *measurement_env(const char *) { return nullptr; }
+#endif
+
 
 inline void log_err(const char *area, const char *fmt, ...) {
   va_list ap;

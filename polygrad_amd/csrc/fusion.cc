@@ -1837,7 +1837,7 @@ static bool match_attention(const Sched &sc, int s_item, const std::vector<char>
   RenderedKernel &rk = out->rk;
   rk = RenderedKernel();
   // timing experiments: extra macro definitions, "NAME=VALUE;NAME=VALUE"
-  if (const char *e = getenv("POLY_HIP_FA_DEFS")) {
+  if (const char *e = measurement_env("POLY_HIP_FA_DEFS")) {
     std::string d(e);
     size_t pos = 0;
     while (pos < d.size()) {

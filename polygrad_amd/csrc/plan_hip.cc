@@ -49,6 +49,18 @@ extern "C" __global__ void __launch_bounds__(256) poly_fill0(unsigned int* p, lo
 }
 )HIP";
 
+// Reads one word of every 64 bytes of a buffer and drops it: what the launch leaves behind
+// is the buffer in the memory-side cache.
+const char *const kTouchSrc = R"HIP(
+extern "C" __global__ void __launch_bounds__(256) poly_touch(const unsigned int* p, long long n_lines) {
+  long long i = (long long)blockIdx.x * 256 + threadIdx.x;
+  const long long stride = (long long)gridDim.x * 256;
+  unsigned int a = 0;
+  for (; i < n_lines; i += stride) a ^= p[i * 16];
+  asm volatile("" ::"v"(a));
+}
+)HIP";
+
 }  // namespace
 
 // One launch of the plan: a scheduled kernel, or a fused group of them.
@@ -93,6 +105,14 @@ struct PolyHipPlan {
   int n_side_streams = 0;
   void *side_scratch_pool[kSideStreams] = {nullptr, nullptr, nullptr};   // the two-stage kernels of a side stream share one
   Program *fill = nullptr;
+  // Buffers that no launch of the plan writes (weights) and that a matrix product reads are
+  // read once by a small launch shortly before the product: it then finds them in the
+  // memory-side cache instead of waiting for HBM with the first tiles of every workgroup (a
+  // product of 8192 x 3072 x 768 whose 4.7 MB of weights come from HBM takes 54 us, 43 us
+  // after such a read, which itself takes 2-3 us).  touch_at[u]: slots to read right
+  // before launch u.
+  std::vector<std::vector<int>> touch_at;
+  Program *touch = nullptr;
   bool use_graph = true;
   bool tuned = false;            // candidates of the tunable kernels have been timed (or there are none)
   std::vector<GraphEntry> graphs;
@@ -104,6 +124,7 @@ struct PolyHipPlan {
     }
     for (Unit &u : units) runner_destroy(u.runner);
     if (fill) program_destroy(fill);
+    if (touch) program_destroy(touch);
     if (arena) runtime_free(arena);
     if (scratch_pool) runtime_free(scratch_pool);
     for (void *p : side_scratch_pool) if (p) runtime_free(p);
@@ -184,7 +205,25 @@ int launch_fill(PolyHipPlan *plan, int slot) {
 
 // Launches unit `u` after the fills that belong in front of it.  A slot shares its bytes
 // with intermediates that die before its first use, so it can only be cleared then.
+// The touches that belong in front of launch `u`, as launches of the main sequence.  (On a
+// stream of their own, beside the launch before the product, they cost more than they
+// saved: every edge between two streams of a captured graph costs a few microseconds, and
+// the attention kernel ran 7 us longer with a touch beside it.)
+void launch_touches(PolyHipPlan *plan, size_t u) {
+  if (u >= plan->touch_at.size() || plan->touch_at[u].empty() || !plan->touch) return;
+  for (int slot : plan->touch_at[u]) {
+    void *p = plan->slot_ptr[(size_t)slot];
+    long long lines = (long long)(plan->sched->buf_slots[slot].nbytes / 64);
+    if (!p || lines <= 0) continue;
+    void *args[2] = {&p, &lines};
+    LaunchSpec ls;
+    ls.grid[0] = (unsigned)std::min<long long>((lines + 255) / 256, 2048);
+    (void)program_launch(plan->touch, args, ls);
+  }
+}
+
 int launch_unit(PolyHipPlan *plan, size_t u) {
+  launch_touches(plan, u);
   for (int slot : plan->fills_before[u])
     if (launch_fill(plan, slot) != 0) return -1;
   std::vector<void *> &a = plan->kargs[u];
@@ -192,13 +231,14 @@ int launch_unit(PolyHipPlan *plan, size_t u) {
 }
 
 int enqueue_all(PolyHipPlan *plan) {
-  for (size_t u = 0; u < plan->units.size(); u++) {
+  int rc = 0;
+  for (size_t u = 0; u < plan->units.size() && rc == 0; u++) {
     if (launch_unit(plan, u) != 0) {
       log_err("plan_run", "kernel %d failed to launch", plan->units[u].item);
-      return -1;
+      rc = -1;
     }
   }
-  return 0;
+  return rc;
 }
 
 // The same launches under stream capture, with those marked on_side going to the side
@@ -631,6 +671,37 @@ PolyHipPlan *poly_hip_compile_schedule(PolyCtx *ctx, const PolySchedule *s) {
     }
     // a lone user owns its scratch memory; it must exist before the launches are captured
     for (Unit &u : plan->units) if (runner_ensure_scratch(u.runner) != 0) return nullptr;
+  }
+  // Which buffers are read ahead of which launch: the inputs of a matrix product that no
+  // launch of the plan writes (the weights), from 128 KB up, `lead` launches ahead of it,
+  // and not again while an earlier touch is recent.
+  plan->touch_at.assign((size_t)n_units, std::vector<int>());
+  if (!getenv("POLY_HIP_NO_PREFETCH")) {
+    int lead = 1;
+    if (const char *e = getenv("POLY_HIP_PREFETCH_LEAD")) lead = std::max(0, atoi(e));
+    int64_t most = 128ll << 20;
+    if (const char *e = getenv("POLY_HIP_PREFETCH_MAX_MB")) most = (int64_t)std::max(0, atoi(e)) << 20;
+    std::vector<char> written((size_t)ns, 0);
+    for (const Unit &u : plan->units) for (int sl : u.writes) written[(size_t)sl] = 1;
+    std::vector<int> touched_for((size_t)ns, -1000);
+    bool any = false;
+    for (int t = 0; t < n_units; t++) {
+      const Unit &u = plan->units[(size_t)t];
+      if (u.runner->rk.klass != KernelClass::MATMUL_MFMA || plan->on_side[(size_t)t]) continue;
+      for (int sl : u.slots) {
+        const PolyScheduleBufSlot &b = s->buf_slots[sl];
+        if (b.is_intermediate || written[(size_t)sl] || b.nbytes < (128 << 10) || b.nbytes > most) continue;
+        if (t - touched_for[(size_t)sl] <= 8) continue;
+        touched_for[(size_t)sl] = t;
+        auto &at = plan->touch_at[(size_t)std::max(0, t - lead)];
+        if (std::find(at.begin(), at.end(), sl) == at.end()) at.push_back(sl);
+        any = true;
+      }
+    }
+    if (any) {
+      plan->touch = program_create(kTouchSrc, "poly_touch");
+      if (!plan->touch) return nullptr;
+    }
   }
   plan->kargs.resize((size_t)n_units);
   plan->var_vals.resize((size_t)n_units);

@@ -20,6 +20,9 @@ namespace {
 const char *const kMatmulTemplate =
 #include "matmul_mfma.hip.inc"
     ;
+const char *const kMatmulDmaTemplate =
+#include "matmul_dma.hip.inc"
+    ;
 const char *const kMatmulF32Template =
 #include "matmul_f32_mfma.hip.inc"
     ;
@@ -230,7 +233,13 @@ bool match_matmul(const KernelGraph &g, MatmulMatch *mm, int *reject_line) {
   if (md.empty() || nd.empty()) MM_REJECT();
 #undef MM_REJECT
 
-  // dims keep END order (outermost first); the innermost one is the fast coordinate
+  // N and Z digits keep END order (outermost first); the innermost one is the fast
+  // coordinate.  The M digits are put in the order of their strides in A, largest first, so
+  // that consecutive rows of a tile are neighbours in memory whatever order the kernel's
+  // ranges came in (a [B, T, d] activation whose ranges arrive as (t, b) would otherwise
+  // deal the rows of a tile to B distant streams); the epilogue finds every range value
+  // from the digits, so the order is free.
+  std::stable_sort(md.begin(), md.end(), [](const Dim &x, const Dim &y) { return std::llabs(x.ca) > std::llabs(y.ca); });
   mm->md_full = md; mm->nd_full = nd; mm->zd_full = zd;
   collapse(md); collapse(nd); collapse(zd);
   mm->md = md; mm->nd = nd; mm->zd = zd;
@@ -687,7 +696,7 @@ bool render_matmul(const MatmulMatch &mm, const MatmulEpilogue &ep, RenderedKern
     }
     if ((double)S * (double)Z * (double)M * (double)N * 4.0 > 1073741824.0) S = 1;
   };
-  const bool may_split = !getenv("POLY_HIP_NO_SPLIT_K") && !getenv("POLY_HIP_MM_NOEPI") && M > 64 && N > 64;
+  const bool may_split = !getenv("POLY_HIP_NO_SPLIT_K") && !measurement_env("POLY_HIP_MM_NOEPI") && M > 64 && N > 64;
   if (may_split) pick_split(64);
   if (S == 1 && !fixed_tile && !getenv("POLY_HIP_MM_TILE") && !getenv("POLY_HIP_MM_OLD_ESTIMATE")) {
     pick_tile(true);
@@ -708,8 +717,41 @@ bool render_matmul(const MatmulMatch &mm, const MatmulEpilogue &ep, RenderedKern
 
   // (n_lo, n_hi: the columns this launch covers; n_lo and, unless it is N, n_hi are
   // multiples of bn)
-  auto emit = [&](int bm, int bn, int wvm, int wvn, int pp, RenderedKernel *rk, int64_t n_lo = 0, int64_t n_hi = -1) {
+  // The template whose operand tiles go from memory straight into LDS (matmul_dma.hip)
+  // takes a tile shape with its own wave layout, K tile, number of LDS stages and
+  // workgroups per CU: 256x256 as 8 waves on four stages of 32; 128x256 and 256x128 as 4
+  // waves on three stages of 32, two workgroups to a CU, so that one's epilogue runs
+  // under the other's K loop; 128x128 as 4 waves on two stages of 64; narrow tiles as 4
+  // waves in a row.  `dma_for` says whether a shape has such a form.
+  struct Dma { int bk, stages, wg, wvm, wvn; };
+  auto dma_for = [&](int bm, int bn, Dma *d) {
+    if (getenv("POLY_HIP_NO_DMA")) return false;
+    Dma c;
+    if (bm * bn >= 256 * 256) c = Dma{32, 4, 1, 4, 2};
+    else if (bm * bn >= 128 * 256) c = Dma{32, 3, 2, 2, 2};
+    else if (bm * bn >= 128 * 128) c = Dma{64, 2, 2, 2, 2};
+    else c = Dma{32, 4, 2, bm >= bn ? 4 : 1, bm >= bn ? 1 : 4};
+    if (const char *ov = bm * bn < 256 * 256 ? getenv("POLY_HIP_MM_DMA") : getenv("POLY_HIP_MM_DMA_256")) {   // "BK,STAGES,WG,WVM,WVN": tuning experiments
+      int v[5];
+      if (sscanf(ov, "%d,%d,%d,%d,%d", &v[0], &v[1], &v[2], &v[3], &v[4]) == 5) c = Dma{v[0], v[1], v[2], v[3], v[4]};
+    }
+    const int nw = c.wvm * c.wvn;
+    if ((c.bk != 32 && c.bk != 64) || c.stages < 2 || c.wg < 1 || nw < 1 || nw > 16) return false;
+    if (bm % (32 * c.wvm) || bn % (32 * c.wvn) || K % c.bk) return false;
+    if ((a_kc && ka.kb % c.bk) || (b_kc && kb.kb % c.bk)) return false;
+    if ((bm * c.bk * 2) % (1024 * nw) || (bn * c.bk * 2) % (1024 * nw)) return false;      // whole LDS loads per wave
+    if ((!a_kc && bm < 64) || (!b_kc && bn < 64)) return false;                            // 8 chunks per k-row for the swizzle
+    const int stage_bytes = (bm + bn) * c.bk * 2;
+    if (c.stages * stage_bytes > 163840 / c.wg || nw * 32 * 36 * 4 > c.stages * stage_bytes) return false;
+    *d = c;
+    return true;
+  };
+  auto emit = [&](int bm, int bn, int wvm, int wvn, int pp, RenderedKernel *rk, int64_t n_lo = 0, int64_t n_hi = -1, bool may_dma = true) {
     if (n_hi < 0) n_hi = N;
+    Dma dma{0, 0, 0, 0, 0};
+    const bool use_dma = may_dma && dma_for(bm, bn, &dma);
+    const int bk = use_dma ? dma.bk : BK;
+    if (use_dma) { wvm = dma.wvm; wvn = dma.wvn; }
     const int64_t tiles = ((M + bm - 1) / bm) * ((n_hi - n_lo + bn - 1) / bn);
     if (tiles > 2147483647LL / 2) return reject(__LINE__);
     // ── configuration block ─────────────────────────────────────────────────
@@ -717,14 +759,15 @@ bool render_matmul(const MatmulMatch &mm, const MatmulEpilogue &ep, RenderedKern
     cfg += strf("#define POLY_TIN %s\n", dt_cname(A.dt));
     cfg += strf("#define POLY_MFMA(a, b, c) __builtin_amdgcn_mfma_f32_32x32x16_%s(a, b, c, 0, 0, 0)\n", A.dt == DT_BF16 ? "bf16" : "f16");
     cfg += strf("#define POLY_M %lld\n#define POLY_N %lld\n#define POLY_K %lld\n#define POLY_Z %lld\n", (long long)M, (long long)N, (long long)K, (long long)Z);
-    cfg += strf("#define POLY_BM %d\n#define POLY_BN %d\n#define POLY_BK %d\n#define POLY_WAVES_M %d\n#define POLY_WAVES_N %d\n", bm, bn, BK, wvm, wvn);
+    cfg += strf("#define POLY_BM %d\n#define POLY_BN %d\n#define POLY_BK %d\n#define POLY_WAVES_M %d\n#define POLY_WAVES_N %d\n", bm, bn, bk, wvm, wvn);
+    if (use_dma) cfg += strf("#define POLY_STAGES %d\n#define POLY_WG_PER_CU %d\n", dma.stages, dma.wg);
     if (n_lo != 0 || n_hi != N) cfg += strf("#define POLY_N_LO %lld\n#define POLY_N_HI %lld\n", (long long)n_lo, (long long)n_hi);
     cfg += strf("#define POLY_GROUP_M %d\n", bm >= 256 ? 4 : 8);
     // each XCD (own L2) works on a contiguous run of tiles: let it re-read the smaller operand
     cfg += strf("#define POLY_GROUP_ALONG_N %d\n", (N > 2 * M && !getenv("POLY_HIP_MM_GROUP_M")) ? 1 : 0);
     cfg += strf("#define POLY_PIPE %d\n", pp);
     // timing experiments only (wrong results): walk just the first n K tiles
-    if (const char *e = getenv("POLY_HIP_MM_KT")) if (atoi(e) > 0 && atoi(e) <= K / BK) cfg += strf("#define POLY_KT %d\n", atoi(e));
+    if (const char *e = measurement_env("POLY_HIP_MM_KT")) if (atoi(e) > 0 && atoi(e) <= K / bk) cfg += strf("#define POLY_KT %d\n", atoi(e));
     cfg += strf("#define POLY_A_KC %d\n#define POLY_B_KC %d\n", a_kc ? 1 : 0, b_kc ? 1 : 0);
     cfg += strf("#define POLY_A_PTR %s\n#define POLY_B_PTR %s\n", ep.a_ptr.c_str(), ep.b_ptr.c_str());
     cfg += offset_fn("poly_a_row", md, true, 0);
@@ -740,7 +783,17 @@ bool render_matmul(const MatmulMatch &mm, const MatmulEpilogue &ep, RenderedKern
     cfg += matmul_k_fn("poly_b_k", kb, K);
     cfg += strf("#define POLY_SIGNATURE %s\n", signature.c_str());
     // LDS beside the operand tiles that an epilogue may use for the middle of its lookup tables
-    if (S == 1 && !getenv("POLY_HIP_NO_LUT_WINDOW")) cfg += strf("#define POLY_EP_WIN_ROOM %d\n", 163840 - 2 * (bm + bn) * BK * 2);
+    if (S == 1 && !getenv("POLY_HIP_NO_LUT_WINDOW")) {
+      if (!use_dma) cfg += strf("#define POLY_EP_WIN_ROOM %d\n", 163840 - 2 * (bm + bn) * BK * 2);
+      else {
+        // the window moves into the stage that tile KT - STAGES leaves; the output staging
+        // must fit before or behind that stage
+        const int kt = (int)(K / bk), stage_bytes = (bm + bn) * bk * 2, out_bytes = wvm * wvn * 32 * 36 * 4;
+        const int win_stage = kt >= dma.stages ? (kt - dma.stages) % dma.stages : 0;
+        const bool fits = kt >= dma.stages && (out_bytes <= win_stage * stage_bytes || out_bytes <= (dma.stages - 1 - win_stage) * stage_bytes);
+        cfg += strf("#define POLY_EP_WIN_ROOM %d\n", fits ? stage_bytes / 1024 * 1024 : 0);
+      }
+    }
     cfg += ep.code;
     if (S > 1) {
       cfg += strf("#define POLY_KSPLIT %d\n#define POLY_PARTIALS %s\n", S, partials.c_str());
@@ -748,10 +801,10 @@ bool render_matmul(const MatmulMatch &mm, const MatmulEpilogue &ep, RenderedKern
       cfg += "#define POLY_EP_PTR(m, n, z) (POLY_PARTIALS + (((size_t)poly_ks * POLY_Z + (z)) * POLY_M + (m)) * POLY_N + (n))\n";
       cfg += "#define POLY_EPILOGUE(acc, m, n, z) *POLY_EP_PTR(m, n, z) = (acc)\n";
     } else
-    if (getenv("POLY_HIP_MM_NOEPI")) cfg += strf("#define POLY_EPILOGUE(acc, m, n, z) do { if (((m) | (n)) == -1) { %s; } } while (0)\n", ep.call.c_str());
+    if (measurement_env("POLY_HIP_MM_NOEPI")) cfg += strf("#define POLY_EPILOGUE(acc, m, n, z) do { if (((m) | (n)) == -1) { %s; } } while (0)\n", ep.call.c_str());
     else
     cfg += strf("#define POLY_EPILOGUE(acc, m, n, z) %s\n", ep.call.c_str());
-    const bool split = S == 1 && ep.contiguous_n && !getenv("POLY_HIP_MM_NOEPI") && (ep.out_type == "__bf16" || ep.out_type == "_Float16" || ep.out_type == "float");
+    const bool split = S == 1 && ep.contiguous_n && !measurement_env("POLY_HIP_MM_NOEPI") && (ep.out_type == "__bf16" || ep.out_type == "_Float16" || ep.out_type == "float");
     if (S == 1) cfg += strf("#define POLY_EP_CONTIG %d\n", split ? 1 : 0);
     if (split) {
       cfg += strf("#define POLY_EP_TYPE %s\n", ep.out_type.c_str());
@@ -761,15 +814,16 @@ bool render_matmul(const MatmulMatch &mm, const MatmulEpilogue &ep, RenderedKern
     }
 
     *rk = RenderedKernel();
-    rk->source = std::string(hip_prelude()) + cfg + kMatmulTemplate;
+    rk->source = std::string(hip_prelude()) + cfg + (use_dma ? kMatmulDmaTemplate : kMatmulTemplate);
     rk->entry = "poly_k";
     rk->launch.grid[0] = (unsigned)tiles;
     rk->launch.grid[1] = (unsigned)(Z * S);
     rk->launch.block[0] = (unsigned)(64 * wvm * wvn);
     rk->klass = KernelClass::MATMUL_MFMA;
     rk->strategy = strf("mfma 32x32x16 %s M=%lld N=%lld K=%lld Z=%lld tile %dx%dx%d A:%s B:%s", A.dt == DT_BF16 ? "bf16" : "f16",
-                        (long long)M, (long long)N, (long long)K, (long long)Z, bm, bn, BK, a_kc ? "k-major" : "m-major",
+                        (long long)M, (long long)N, (long long)K, (long long)Z, bm, bn, bk, a_kc ? "k-major" : "m-major",
                         b_kc ? "k-major" : "n-major");
+    if (use_dma) rk->strategy += strf(", operands straight into LDS: %d waves, %d stages, %d per CU", wvm * wvn, dma.stages, dma.wg);
     rk->n_params = ep.n_params;
     rk->n_vars = 0;
     rk->flops = 2.0 * (double)M * (double)N * (double)K * (double)Z;
@@ -801,7 +855,7 @@ bool render_matmul(const MatmulMatch &mm, const MatmulEpilogue &ep, RenderedKern
   // once with short workgroups.  Taken when the estimate (rounds, a small tile's round
   // weighted by its area and by what its narrower wave tiles cost, plus a launch) saves
   // a quarter of a round or more.
-  if (Z == 1 && M > 64 && N > 64 && !matmul_tuning_enabled() && !getenv("POLY_HIP_NO_TAIL_LAUNCH") && !getenv("POLY_HIP_MM_NOEPI")) {
+  if (Z == 1 && M > 64 && N > 64 && !matmul_tuning_enabled() && !getenv("POLY_HIP_NO_TAIL_LAUNCH") && !measurement_env("POLY_HIP_MM_NOEPI")) {
     const int64_t tm = (M + BM - 1) / BM, tn = (N + BN - 1) / BN, T = tm * tn;
     const int64_t whole = T / 256, rest = T % 256;
     const int64_t keep = std::min<int64_t>(whole * 256 / tm, tn - 1);     // column tiles of the main launch
