@@ -526,6 +526,10 @@ static bool match_matmul_tail(const Sched &sc, int s_item, const std::vector<cha
   ep.a_ptr = strf("fa%d", arg_of(sc.slot(s_item, mS.A.param)));
   ep.b_ptr = strf("fa%d", arg_of(sc.slot(s_item, mS.B.param)));
   ep.n_params = (int)arg_slots.size();
+  {
+    const int bs = sc.slot(s_item, mS.B.param);
+    ep.b_from_hbm = !s->buf_slots[bs].is_intermediate && sc.writers[(size_t)bs].empty();
+  }
   if (!render_matmul(mS, ep, &out->rk)) return false;
   out->rk.tables = tables;
   std::string tail = strf(" + %zu pointwise kernel%s in the epilogue", members.size() - 1, members.size() > 2 ? "s" : "");

@@ -14,6 +14,12 @@
 //                       POLY_STAGES - 1 tiles ahead of the multiplication
 //   POLY_WG_PER_CU      workgroups meant to share a CU (sets the register budget), so
 //                       that one's epilogue runs under another's K loop
+//   POLY_TOUCH_WGS      (optional) that many extra workgroups at the front of the grid, which
+//                       multiply nothing: they read one word of every 64 bytes of the
+//                       POLY_TOUCH_LINES * 64 bytes from element POLY_TOUCH_FIRST of B on and
+//                       leave.  When B comes from HBM (weights), they run ahead of the others
+//                       through B, which then find it in the memory-side cache instead of
+//                       waiting for HBM at every K tile
 //   POLY_EP_WIN_BYTES   (optional, set by the epilogue's own code when POLY_EP_WIN_ROOM
 //                       suffices) bytes of the epilogue's lookup tables that the kernel
 //                       keeps in LDS, read from POLY_EP_WIN_SRC(byte): they are loaded
@@ -184,7 +190,21 @@ extern "C" __global__ void __launch_bounds__(POLY_NTHREADS) POLY_WAVES_ATTR poly
   constexpr int TILES_M = (POLY_M + POLY_BM - 1) / POLY_BM;
   constexpr int TILES_N = (POLY_N_HI - POLY_N_LO + POLY_BN - 1) / POLY_BN;
   constexpr int NT = TILES_M * TILES_N;
+#ifdef POLY_TOUCH_WGS
+  static_assert(POLY_TOUCH_WGS % 8 == 0, "the workgroups behind keep their XCDs");
+  if (blockIdx.x < POLY_TOUCH_WGS) {
+    if (blockIdx.y == 0) {
+      const unsigned int *const p = (const unsigned int *)(POLY_B_PTR + (POLY_TOUCH_FIRST));
+      unsigned int a = 0;
+      for (long long i = (long long)blockIdx.x * POLY_NTHREADS + threadIdx.x; i < (POLY_TOUCH_LINES); i += (long long)POLY_TOUCH_WGS * POLY_NTHREADS) a ^= p[i * 16];
+      asm volatile("" ::"v"(a));
+    }
+    return;
+  }
+  int bid = blockIdx.x - POLY_TOUCH_WGS;
+#else
   int bid = blockIdx.x;
+#endif
   {
     constexpr int PER = NT / 8, REM = NT % 8;
     const int xcd = bid & 7, idx = bid >> 3;

@@ -338,7 +338,24 @@ PolyHipPlan *poly_hip_compile_schedule(PolyCtx *ctx, const PolySchedule *s) {
       u.slots = fg.arg_slots;
       u.n_items = (int)fg.items.size();
     } else {
-      u.runner = runner_create(it.root, name.c_str(), 0);
+      {
+        // (which of the kernel's buffers are inputs of the plan that nothing in it writes)
+        uint64_t mask = 0;
+        for (int p = 0; p < it.n_buf_slots && p < 64; p++) {
+          const int sl = it.buf_slot_indices[p];
+          bool written = s->buf_slots[sl].is_intermediate;
+          for (int k2 = 0; k2 < s->n_items && !written; k2++) {
+            const PolyExecItem &o = s->items[k2];
+            const KernelGraph &g2 = graphs[(size_t)k2];
+            for (size_t q = 0; q < g2.params.size() && (int)q < o.n_buf_slots; q++)
+              if (o.buf_slot_indices[q] == sl && g2.params[q].written) written = true;
+          }
+          if (!written) mask |= (uint64_t)1 << p;
+        }
+        matmul_hint_input_params(mask);
+        u.runner = runner_create(it.root, name.c_str(), 0);
+        matmul_hint_input_params(0);
+      }
       // (a kernel may use fewer variables than the schedule lists for it: a buffer sized by
       // a variable that the kernel itself walks over its full allocation)
       if (u.runner && (u.runner->rk.n_params != it.n_buf_slots || u.runner->rk.n_vars > it.n_var_uops)) {
@@ -687,7 +704,7 @@ PolyHipPlan *poly_hip_compile_schedule(PolyCtx *ctx, const PolySchedule *s) {
     bool any = false;
     for (int t = 0; t < n_units; t++) {
       const Unit &u = plan->units[(size_t)t];
-      if (u.runner->rk.klass != KernelClass::MATMUL_MFMA || plan->on_side[(size_t)t]) continue;
+      if (u.runner->rk.klass != KernelClass::MATMUL_MFMA || plan->on_side[(size_t)t] || u.runner->rk.reads_b_ahead) continue;
       for (int sl : u.slots) {
         const PolyScheduleBufSlot &b = s->buf_slots[sl];
         if (b.is_intermediate || written[(size_t)sl] || b.nbytes < (128 << 10) || b.nbytes > most) continue;

@@ -69,6 +69,9 @@ struct RenderedKernel {
     LaunchSpec launch;
   };
   std::vector<Variant> variants;
+  // A matrix product whose own first workgroups read operand B into the memory-side cache
+  // (the plan then launches nothing ahead of it for that).
+  bool reads_b_ahead = false;
   // Kernels in two stages (reductions through partial results, matmuls whose operands are
   // prepared first): `pres` run first, in order, with the same arguments plus one more
   // pointer to `scratch_bytes` bytes of device memory that the runner owns; the main

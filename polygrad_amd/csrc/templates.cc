@@ -30,6 +30,8 @@ const char *const kOperandSplitTemplate =
 #include "operand_split.hip.inc"
     ;
 
+thread_local uint64_t g_input_params = 0;
+
 PolyOps reduce_op(const KNode &k) {
   return k.u->arg.kind == POLY_ARG_OPS ? k.u->arg.ops : (PolyOps)k.u->arg.i;
 }
@@ -492,6 +494,7 @@ bool try_render_matmul(const KernelGraph &g, const std::string &fn, const Render
   if (!epilogue_from_graph(g, mm, &ep)) return false;
   ep.a_ptr = strf("data%d", mm.A.param);
   ep.b_ptr = strf("data%d", mm.B.param);
+  ep.b_from_hbm = mm.B.param >= 0 && mm.B.param < 64 && ((g_input_params >> mm.B.param) & 1);
   if (!render_matmul(mm, ep, out)) return false;
   out->tables = ep.tables;
   if (!ep.tables.empty()) {
@@ -617,6 +620,8 @@ static bool render_matmul_f32(const MatmulMatch &mm, const MatmulEpilogue &ep, R
   }
   return true;
 }
+
+void matmul_hint_input_params(uint64_t mask) { g_input_params = mask; }
 
 bool matmul_tuning_enabled() {
   const char *e = getenv("POLY_BEAM");
@@ -761,6 +766,15 @@ bool render_matmul(const MatmulMatch &mm, const MatmulEpilogue &ep, RenderedKern
     cfg += strf("#define POLY_M %lld\n#define POLY_N %lld\n#define POLY_K %lld\n#define POLY_Z %lld\n", (long long)M, (long long)N, (long long)K, (long long)Z);
     cfg += strf("#define POLY_BM %d\n#define POLY_BN %d\n#define POLY_BK %d\n#define POLY_WAVES_M %d\n#define POLY_WAVES_N %d\n", bm, bn, bk, wvm, wvn);
     if (use_dma) cfg += strf("#define POLY_STAGES %d\n#define POLY_WG_PER_CU %d\n", dma.stages, dma.wg);
+    // B in HBM as one dense block of K x N elements: extra workgroups at the front of the
+    // grid run ahead through it, so that the others wait for HBM once and not at every K tile
+    int touch_wgs = 0;
+    if (use_dma && ep.b_from_hbm && S == 1 && Z == 1 && zd.empty() && nd.size() == 1 && kb.kb >= K && !getenv("POLY_HIP_NO_PREFETCH") &&
+        ((b_kc && kb.s_lo == 1 && nd[0].cb == K) || (!b_kc && nd[0].cb == 1 && kb.s_lo == N)) && K * N * 2 >= (128 << 10) && tiles >= 64) {
+      touch_wgs = K * N * 2 >= (2 << 20) ? 64 : 32;
+      cfg += strf("#define POLY_TOUCH_WGS %d\n#define POLY_TOUCH_FIRST %lld\n#define POLY_TOUCH_LINES %lldll\n", touch_wgs,
+                  (long long)(mm.b_c0 & ~1ll), (long long)((K * N * 2 - 64) / 64));
+    }
     if (n_lo != 0 || n_hi != N) cfg += strf("#define POLY_N_LO %lld\n#define POLY_N_HI %lld\n", (long long)n_lo, (long long)n_hi);
     cfg += strf("#define POLY_GROUP_M %d\n", bm >= 256 ? 4 : 8);
     // each XCD (own L2) works on a contiguous run of tiles: let it re-read the smaller operand
@@ -816,14 +830,16 @@ bool render_matmul(const MatmulMatch &mm, const MatmulEpilogue &ep, RenderedKern
     *rk = RenderedKernel();
     rk->source = std::string(hip_prelude()) + cfg + (use_dma ? kMatmulDmaTemplate : kMatmulTemplate);
     rk->entry = "poly_k";
-    rk->launch.grid[0] = (unsigned)tiles;
+    rk->launch.grid[0] = (unsigned)(tiles + touch_wgs);
     rk->launch.grid[1] = (unsigned)(Z * S);
     rk->launch.block[0] = (unsigned)(64 * wvm * wvn);
     rk->klass = KernelClass::MATMUL_MFMA;
+    rk->reads_b_ahead = touch_wgs > 0;
     rk->strategy = strf("mfma 32x32x16 %s M=%lld N=%lld K=%lld Z=%lld tile %dx%dx%d A:%s B:%s", A.dt == DT_BF16 ? "bf16" : "f16",
                         (long long)M, (long long)N, (long long)K, (long long)Z, bm, bn, bk, a_kc ? "k-major" : "m-major",
                         b_kc ? "k-major" : "n-major");
     if (use_dma) rk->strategy += strf(", operands straight into LDS: %d waves, %d stages, %d per CU", wvm * wvn, dma.stages, dma.wg);
+    if (touch_wgs) rk->strategy += strf(", %d workgroups read B ahead", touch_wgs);
     rk->n_params = ep.n_params;
     rk->n_vars = 0;
     rk->flops = 2.0 * (double)M * (double)N * (double)K * (double)Z;

@@ -72,7 +72,13 @@ struct MatmulEpilogue {
   // in front of any scratch pointer), and the argument list that goes with `signature`.
   std::vector<RenderedKernel::Table> tables;
   std::string params_call;
+  // Operand B is a buffer that nothing in the plan writes (weights): at the time of the
+  // launch it is in HBM, not in the caches.
+  bool b_from_hbm = false;
 };
+// Set by the plan compiler around the lowering of one scheduled kernel: bit p says that
+// buffer parameter p is an input of the plan that none of its kernels writes.
+void matmul_hint_input_params(uint64_t mask);
 // Is element (m, n + 1) of the kernel's output stored right after (m, n), for every n
 // that is not the last of an aligned group of 8?  (store index affine with coefficient 1
 // on the innermost digit of n, digits not crossed inside a group)
