@@ -733,9 +733,10 @@ bool render_matmul(const MatmulMatch &mm, const MatmulEpilogue &ep, RenderedKern
     if (getenv("POLY_HIP_NO_DMA")) return false;
     Dma c;
     if (bm * bn >= 256 * 256) c = Dma{32, 4, 1, 4, 2};
-    else if (bm * bn >= 128 * 256) c = Dma{32, 3, 2, 2, 2};
+    else if (bm * bn >= 128 * 192) c = Dma{32, 3, 2, 2, 2};
     else if (bm * bn >= 128 * 128) c = Dma{64, 2, 2, 2, 2};
     else c = Dma{32, 4, 2, bm >= bn ? 4 : 1, bm >= bn ? 1 : 4};
+    if (d->bk) c = *d;      // the caller's own choice
     if (const char *ov = bm * bn < 256 * 256 ? getenv("POLY_HIP_MM_DMA") : getenv("POLY_HIP_MM_DMA_256")) {   // "BK,STAGES,WG,WVM,WVN": tuning experiments
       int v[5];
       if (sscanf(ov, "%d,%d,%d,%d,%d", &v[0], &v[1], &v[2], &v[3], &v[4]) == 5) c = Dma{v[0], v[1], v[2], v[3], v[4]};
@@ -751,9 +752,9 @@ bool render_matmul(const MatmulMatch &mm, const MatmulEpilogue &ep, RenderedKern
     *d = c;
     return true;
   };
-  auto emit = [&](int bm, int bn, int wvm, int wvn, int pp, RenderedKernel *rk, int64_t n_lo = 0, int64_t n_hi = -1, bool may_dma = true) {
+  auto emit = [&](int bm, int bn, int wvm, int wvn, int pp, RenderedKernel *rk, int64_t n_lo = 0, int64_t n_hi = -1, bool may_dma = true,
+                  Dma dma = Dma{0, 0, 0, 0, 0}) {
     if (n_hi < 0) n_hi = N;
-    Dma dma{0, 0, 0, 0, 0};
     const bool use_dma = may_dma && dma_for(bm, bn, &dma);
     const int bk = use_dma ? dma.bk : BK;
     if (use_dma) { wvm = dma.wvm; wvn = dma.wvn; }
@@ -846,6 +847,22 @@ bool render_matmul(const MatmulMatch &mm, const MatmulEpilogue &ep, RenderedKern
     rk->bytes = ep.bytes;
     return true;
   };
+  // Tile shapes of the straight-into-LDS template, from timings inside the GPT-2 forward
+  // plan (M = 8192, K = 768 or 3072): a launch of at most 256 tiles of 128x256 leaves a CU
+  // one workgroup of four waves, which is too little to hide anything: 128x128 tiles, two
+  // workgroups to a CU (N = 768: 21.7 -> 19.6 us at K = 768, 47.8 -> 46.2 us at K = 3072);
+  // between one and one and a quarter rounds of 512 workgroups, 128x192 tiles when they
+  // divide N and give a round and a half (N = 2304: 43.6 -> 39.9 us).
+  if (S == 1 && !fixed_tile && !getenv("POLY_HIP_MM_TILE") && BM * BN == 128 * 256) {
+    Dma probe{0, 0, 0, 0, 0};
+    auto count = [&](int bm, int bn) { return ((M + bm - 1) / bm) * ((N + bn - 1) / bn) * Z; };
+    const int64_t t = count(BM, BN);
+    if (dma_for(BM, BN, &probe)) {
+      Dma p2{0, 0, 0, 0, 0}, p3{0, 0, 0, 0, 0};
+      if (t <= 256 && M % 128 == 0 && dma_for(128, 128, &p2)) { BM = BN = 128; WVM = WVN = 2; }
+      else if (t > 512 && t < 640 && N % 192 == 0 && count(128, 192) >= 768 && dma_for(128, 192, &p3)) { BM = 128; BN = 192; WVM = WVN = 2; }
+    }
+  }
   if (!emit(BM, BN, WVM, WVN, pipe, out)) return false;
   if (S > 1) {
     // the template becomes a first stage; the kernel proper adds the partial results up
@@ -912,12 +929,22 @@ bool render_matmul(const MatmulMatch &mm, const MatmulEpilogue &ep, RenderedKern
     struct Shape { int bm, bn, wm, wn, pp; };
     static const Shape shapes[] = {{256, 256, 4, 2, 2}, {256, 128, 4, 2, 3}, {256, 128, 4, 2, 2}, {128, 256, 2, 4, 3},
                                    {128, 256, 2, 4, 2}, {128, 128, 2, 2, 3}, {128, 128, 2, 2, 2}};
-    out->variants.push_back({strf("%dx%dw%dx%dp%d", BM, BN, WVM, WVN, pipe), out->source, out->strategy, out->launch});
+    out->variants.push_back({"default", out->source, out->strategy, out->launch});
+    // the template with register staging
     for (const Shape &c : shapes) {
-      if (c.bm == BM && c.bn == BN && c.wm == WVM && c.wn == WVN && c.pp == pipe) continue;
       RenderedKernel v;
-      if (emit(c.bm, c.bn, c.wm, c.wn, c.pp, &v))
+      if (emit(c.bm, c.bn, c.wm, c.wn, c.pp, &v, 0, -1, false) && v.source != out->source)
         out->variants.push_back({strf("%dx%dw%dx%dp%d", c.bm, c.bn, c.wm, c.wn, c.pp), v.source, v.strategy, v.launch});
+    }
+    // the template that loads straight into LDS: tile, K tile, stages, workgroups per CU, waves
+    struct DShape { int bm, bn; Dma d; };
+    static const DShape dshapes[] = {{256, 256, {32, 4, 1, 4, 2}}, {256, 256, {64, 2, 1, 4, 2}}, {128, 256, {32, 3, 2, 2, 2}}, {256, 128, {32, 3, 2, 2, 2}},
+                                     {128, 256, {64, 3, 1, 2, 4}}, {256, 128, {64, 3, 1, 4, 2}}, {128, 192, {32, 3, 2, 2, 2}}, {128, 128, {64, 2, 2, 2, 2}},
+                                     {128, 128, {32, 4, 2, 2, 2}}};
+    for (const DShape &c : dshapes) {
+      RenderedKernel v;
+      if (emit(c.bm, c.bn, c.d.wvm, c.d.wvn, 3, &v, 0, -1, true, c.d) && v.source != out->source && v.strategy.find("straight into LDS") != std::string::npos)
+        out->variants.push_back({strf("%dx%dx%dw%dx%ds%dg%d", c.bm, c.bn, c.d.bk, c.d.wvm, c.d.wvn, c.d.stages, c.d.wg), v.source, v.strategy, v.launch});
     }
   }
   return true;

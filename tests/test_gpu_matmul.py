@@ -173,12 +173,15 @@ def test_full_size_row_block_matches_cpu_bit_pattern_of_sums():
     assert_close(h, w, rtol=1e-4, atol=1e-4 * float(np.abs(w).mean()), what="row block of 1024x4096x4096")
 
 
-@pytest.mark.parametrize("n,k,tb", [(2304, 64, False), (2296, 128, False), (2296, 64, True)])
-def test_columns_left_over_by_whole_rounds_go_to_a_launch_of_small_tiles(n, k, tb):
-    """8192 x 2304 in 128 x 256 tiles is 576 tiles, two rounds over 256 CUs and a quarter:
-    the columns from 2048 on are computed by a launch of 128 x 64 tiles of their own (here
-    also with a ragged last tile).  Sampled rows against the CPU backend on those rows, and
-    the whole result against the single launch of the same graph (POLY_HIP_NO_TAIL_LAUNCH)."""
+@pytest.mark.parametrize("n,k,tb,how", [(2304, 64, False, "tile 128x192"), (2296, 128, False, "columns from 2048 on by a launch of 128x64 tiles"),
+                                        (2296, 64, True, "columns from 2048 on by a launch of 128x64 tiles")])
+def test_columns_left_over_by_whole_rounds_go_to_a_launch_of_small_tiles(n, k, tb, how):
+    """8192 x 2304 in 128 x 256 tiles is 576 tiles, a round of 512 workgroups and an eighth:
+    128 x 192 tiles when they divide N (768 tiles, a round and a half); otherwise the columns
+    from 2048 on are computed by a launch of 128 x 64 tiles of their own (here with a ragged
+    last tile).  Sampled rows against the CPU backend on those rows, and the whole result
+    against the single launch of 128 x 256 tiles of the same graph (POLY_HIP_NO_TAIL_LAUNCH
+    and POLY_HIP_MM_TILE)."""
     import os
     m = 8192
     g = np.random.default_rng(n + k)
@@ -187,14 +190,16 @@ def test_columns_left_over_by_whole_rounds_go_to_a_launch_of_small_tiles(n, k, t
     A, Bm, O, sink = graphs.matmul_bf16(c, m, n, k, transposed_b=tb)
     arrays = {A: a_bits, Bm: b_bits, O: np.zeros(m * n, np.float32)}
     got, info = run_hip(c, sink, arrays)
-    assert "columns from 2048 on by a launch of 128x64 tiles" in info[0]["desc"], info[0]["desc"]
+    assert how in info[0]["desc"], info[0]["desc"]
     os.environ["POLY_HIP_NO_TAIL_LAUNCH"] = "1"
+    os.environ["POLY_HIP_MM_TILE"] = "128,256,2,4"
     try:
         one, info1 = run_hip(c, sink, arrays)
     finally:
         del os.environ["POLY_HIP_NO_TAIL_LAUNCH"]
+        del os.environ["POLY_HIP_MM_TILE"]
     c.close()
-    assert "by a launch of" not in info1[0]["desc"]
+    assert "by a launch of" not in info1[0]["desc"] and "tile 128x256" in info1[0]["desc"]
     rows = [0, 1, 127, 128, 4095, 4096, 5000, 8063, 8064, 8191]
     c = R.Ctx()
     A8, B8, O8, sink8 = graphs.matmul_bf16(c, len(rows), n, k, transposed_b=tb)
