@@ -274,6 +274,15 @@ def main():
     args = ap.parse_args()
     if args.gpus != 1:
         sys.exit("bench.py: this backend runs on one GPU; --gpus must be 1 (nothing here shards across devices)")
+    # The CPU baseline first, before anything touches the GPU: the reference's CPU backend
+    # forks and executes clang for every kernel (src/runtime_cpu.c:115-137), which a process
+    # that has initialised the GPU should not do.
+    cpu = None
+    if not args.no_cpu_baseline and args.workload == GPT2_PLAN and args.path == "plan":
+        try:
+            cpu = cpu_baseline_reference() or cpu_baseline_port()
+        except Exception as e:  # the baseline is reported, never required
+            log(f"cpu baseline failed: {e}")
     import torch
     if not torch.cuda.is_available():
         sys.exit("bench.py: no GPU available (there is no CPU path to benchmark)")
@@ -301,12 +310,6 @@ def main():
                                             "no fusion, no buffer sharing, no hipGraph (bench.py --path vtable)"}
         except Exception as e:
             log(f"vtable path failed: {e}")
-    cpu = None
-    if not args.no_cpu_baseline and args.workload == GPT2_PLAN:
-        try:
-            cpu = cpu_baseline_reference() or cpu_baseline_port()
-        except Exception as e:  # the baseline is reported, never required
-            log(f"cpu baseline failed: {e}")
     if tokens is not None:
         metric, value, unit = "GPT-2-small fwd tokens/s on 1 MI355X", tokens / (ms * 1e-3), "tokens/s"
         T = extra.get("seq_len") or 1024

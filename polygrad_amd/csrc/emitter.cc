@@ -70,18 +70,33 @@ __device__ __forceinline__ float poly_swz16_f32(float v) {
     float hi = __builtin_bit_cast(float, __builtin_amdgcn_readlane(__builtin_bit_cast(int, v), 32)); \
     return COMBINE(lo, hi);                                                   \
   }
+// The same over the 32 lanes of a half wave (two rows to a wave): every lane returns the
+// total of its own half.
+#define POLY_HALF_REDUCE_F32(NAME, COMBINE)                                   \
+  __device__ __forceinline__ float NAME(float v) {                            \
+    float o;                                                                  \
+    o = poly_dpp_f32<0xB1>(v); v = COMBINE(v, o);                             \
+    o = poly_dpp_f32<0x4E>(v); v = COMBINE(v, o);                             \
+    o = poly_dpp_f32<0x141>(v); v = COMBINE(v, o);                            \
+    o = poly_dpp_f32<0x140>(v); v = COMBINE(v, o);                            \
+    o = poly_swz16_f32(v); v = COMBINE(v, o);                                 \
+    return v;                                                                 \
+  }
 #define POLY_COMB_ADD(a, b) ((a) + (b))
 #define POLY_COMB_MUL(a, b) ((a) * (b))
 #define POLY_COMB_MAX(a, b) (((a) < (b)) ? (b) : (a))
 POLY_WAVE_REDUCE_F32(poly_wave_add_f32, POLY_COMB_ADD)
 POLY_WAVE_REDUCE_F32(poly_wave_mul_f32, POLY_COMB_MUL)
 POLY_WAVE_REDUCE_F32(poly_wave_max_f32, POLY_COMB_MAX)
+POLY_HALF_REDUCE_F32(poly_half_add_f32, POLY_COMB_ADD)
+POLY_HALF_REDUCE_F32(poly_half_mul_f32, POLY_COMB_MUL)
+POLY_HALF_REDUCE_F32(poly_half_max_f32, POLY_COMB_MAX)
 
 // Generic (any 4/8-byte type) fallback through ds_bpermute shuffles.
-template <typename T, typename F>
+template <typename T, typename F, int LANES = 64>
 __device__ __forceinline__ T poly_wave_reduce_any(T v, F f) {
 #pragma unroll
-  for (int m = 1; m < 64; m <<= 1) {
+  for (int m = 1; m < LANES; m <<= 1) {
     T o;
     if constexpr (sizeof(T) == 8) {
       long long x = __builtin_bit_cast(long long, v);

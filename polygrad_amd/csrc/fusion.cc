@@ -109,6 +109,9 @@ struct Sched {
   const std::vector<KernelGraph> &graphs;
   std::vector<int> step_of;                  // item -> position in exec_order
   std::vector<std::vector<int>> readers, writers;   // per slot: items
+  // item -> position at which what it writes exists: its own, or that of the launch of the
+  // group that has taken it (groups launch at their last item)
+  std::vector<int> launch_step;
   int slot(int item, int param) const { return s->items[item].buf_slot_indices[param]; }
   int param_of(int item, int sl) const {
     const PolyExecItem &it = s->items[item];
@@ -840,7 +843,19 @@ static bool match_row_chain_impl(const Sched &sc, int a_item, const std::vector<
   for (int sl : exported) internal.erase(sl);      // they have memory, and the kernel gets them as arguments
 
   // ── code generation ────────────────────────────────────────────────────
-  const int G = (R >= 4096 || (rows < 2048 && R >= 1024)) ? 256 : 64;
+  int G = (R >= 4096 || (rows < 2048 && R >= 1024)) ? 256 : 64;
+  // Rows of 16-bit elements that 64 lanes x 8 elements do not divide but 32 x 8 do (768 =
+  // 3 x 32 x 8): half a wave per row, two rows to a wave.  Every load is 16 bytes, a wave
+  // has twice the bytes in flight and the launch half the waves.  (Whatever the number of
+  // rows: the lanes a row is dealt to decide the order of its sums, and a plan for one
+  // sequence must round as the plan for eight does.)
+  if (G == 64 && R % 256 == 0 && R % 512 != 0 && R <= 4096 && !getenv("POLY_HIP_NO_HALF_WAVE_ROWS")) {
+    int maxsz = 1;
+    for (int it : items)
+      for (const auto &p : sc.graphs[(size_t)it].params)
+        if ((double)s->buf_slots[sc.slot(it, (int)(&p - &sc.graphs[(size_t)it].params[0]))].numel >= rows * (double)R) maxsz = std::max(maxsz, dt_size(p.dt));
+    if (maxsz == 2) G = 32;
+  }
   std::vector<int> arg_slots;
   arg_slots.push_back(out_slot);
   for (int sl : inputs) arg_slots.push_back(sl);
@@ -934,7 +949,7 @@ static bool match_row_chain_impl(const Sched &sc, int a_item, const std::vector<
       // a row that half the vector width deals out evenly (768 = 3 x 64 x 4, against one
       // and a half steps of 64 x 8) is walked that way: no step with half the lanes idle
       // (LayerNorm of 8192 x 768: 12.3 -> 11.2 us)
-      if (!reads_row && V >= 8 && R % ((int64_t)G * V) != 0 && R % ((int64_t)G * V / 2) == 0) V /= 2;
+      if (!reads_row && V >= 8 && G == 64 && R % ((int64_t)G * V) != 0 && R % ((int64_t)G * V / 2) == 0) V /= 2;
       // long rows of an extent that is no multiple of the vector width (a vocabulary of
       // 50257): vector accesses at element alignment and a scalar tail
       if (V == 1 && !reads_row && !ph.keeps_row && !getenv("POLY_HIP_NO_RAGGED_VEC")) {
@@ -959,7 +974,7 @@ static bool match_row_chain_impl(const Sched &sc, int a_item, const std::vector<
     std::vector<int> pres;
     const int nit = (int)((R + (int64_t)G * V - 1) / ((int64_t)G * V));
     // iterations as an unrolled loop over `it` (what is kept between phases is indexed by it)
-    const bool unrolled = (G == 64 && nit <= 4) || (G == 256 && nit <= 8);
+    const bool unrolled = (G <= 64 && nit <= 4) || (G == 256 && nit <= 8);
     {
       bool reads_row = false;
       for (auto &kv : ph.m.preset) if (kv.second.find("[it]") != std::string::npos) reads_row = true;
@@ -1034,7 +1049,7 @@ static bool match_row_chain_impl(const Sched &sc, int a_item, const std::vector<
       loop += U.code + "    }\n" + loop_close;
       if (ragged)
         loop += ragged_tail(Rn.src[0], [&](Scope *, const std::string &v2) { return strf("    acc = %s;\n", Emitter::reduce_combine(op, Rn.dt, "acc", v2).c_str()); });
-      loop += strf("  acc = %s;\n", wave_reduce_call(op, Rn.dt, "acc").c_str());
+      loop += strf("  acc = %s;\n", wave_reduce_call(op, Rn.dt, "acc", G == 32 ? 32 : 64).c_str());
       if (G == 256) {
         loop += strf("  __shared__ %s red[4];\n  __syncthreads();\n  if ((threadIdx.x & 63) == 0) red[threadIdx.x >> 6] = acc;\n  __syncthreads();\n",
                      dt_cname(Rn.dt));
@@ -1123,6 +1138,9 @@ static bool match_row_chain_impl(const Sched &sc, int a_item, const std::vector<
   if (G == 64) {
     body += "  const int lane = threadIdx.x & 63;\n  const long long row = (long long)blockIdx.x * 4 + (threadIdx.x >> 6);\n";
     body += strf("  if (row < %lldll) {\n", (long long)rows);
+  } else if (G == 32) {
+    body += "  const int lane = threadIdx.x & 31;\n  const long long row = (long long)blockIdx.x * 8 + (threadIdx.x >> 5);\n";
+    body += strf("  if (row < %lldll) {\n", (long long)rows);
   } else {
     body += "  const int lane = threadIdx.x;\n  const long long row = blockIdx.x;\n  {\n";
   }
@@ -1138,7 +1156,7 @@ static bool match_row_chain_impl(const Sched &sc, int a_item, const std::vector<
   rk = RenderedKernel();
   rk.source = std::string(hip_prelude()) + code + body;
   rk.entry = "poly_k";
-  rk.launch.grid[0] = (unsigned)(G == 256 ? rows : std::ceil(rows / 4));
+  rk.launch.grid[0] = (unsigned)(G == 256 ? rows : G == 32 ? std::ceil(rows / 8) : std::ceil(rows / 4));
   rk.launch.block[0] = 256;
   rk.klass = KernelClass::ROW_REDUCE;
   rk.strategy = strf("row chain of %zu kernels (%s) G=%d R=%lld rows=%.0f", phases.size(), strat.c_str(), G, (long long)R, rows);
@@ -1758,10 +1776,13 @@ static bool match_attention(const Sched &sc, int s_item, const std::vector<char>
       // f(acc) = cast(acc) * 2^k with nothing else in it: the kernel multiplies Q by 2^k
       // once when it stages it instead (products and sums of a dot product scale exactly
       // with a power of two, and so does every rounding on the way, as long as nothing
-      // becomes subnormal), and the chain is emitted with that constant as 1.
+      // becomes subnormal), and the chain is emitted with that constant as 1.  For bf16 only:
+      // it has the exponent range of fp32, so the scaled Q loses nothing; an fp16 Q below
+      // 2^-11 would lose mantissa bits, and the reference's cast of an unscaled sum to fp16
+      // can overflow where the scaled one does not.
       int scale_const = -1;
       double qscale = 1.0;
-      if (!getenv("POLY_HIP_NO_QSCALE")) {
+      if (!getenv("POLY_HIP_NO_QSCALE") && tin == DT_BF16) {
         int muls = 0, v = other;
         while (true) {
           const KNode &k = g.n(v);
@@ -2280,7 +2301,7 @@ static bool match_ordered_sums_side_by_side(const Sched &sc, int a_item, const s
       const int sl = sc.slot(k, (int)p);
       if (outs.count(sl)) ready = false;
       if (!g.params[p].read) continue;
-      for (int w : sc.writers[(size_t)sl]) if (w != k && sc.step_of[(size_t)w] >= first_step) ready = false;
+      for (int w : sc.writers[(size_t)sl]) if (w != k && sc.launch_step[(size_t)w] >= first_step) ready = false;
     }
     if (!ready) continue;
     Ad ad;
@@ -2379,12 +2400,56 @@ static bool match_ordered_sums_side_by_side(const Sched &sc, int a_item, const s
   return true;
 }
 
+// Which groups launch at a place that breaks a dependence of the schedule: for two items
+// that touch the same buffer, at least one of them writing, the launch of the earlier one
+// (its group's, if a group has taken it) must not come behind the launch of the later one.
+// A check of the matchers from scratch, on the host: they each reason about their own
+// members, this looks at every pair.
+std::vector<int> fused_groups_out_of_order(const PolySchedule *s, const std::vector<KernelGraph> &graphs, const std::vector<FusedGroup> &groups) {
+  std::vector<int> step_of((size_t)s->n_items, 0), group_of((size_t)s->n_items, -1), pos((size_t)s->n_items, 0);
+  for (int st = 0; st < s->n_items; st++) step_of[(size_t)s->exec_order[st]] = st;
+  for (size_t gi = 0; gi < groups.size(); gi++) for (int it : groups[gi].items) group_of[(size_t)it] = (int)gi;
+  for (int k = 0; k < s->n_items; k++) pos[(size_t)k] = group_of[(size_t)k] >= 0 ? step_of[(size_t)groups[(size_t)group_of[(size_t)k]].launch_item] : step_of[(size_t)k];
+  struct Use { int step, item; bool w; };
+  std::vector<std::vector<Use>> uses((size_t)s->n_buf_slots);
+  for (int k = 0; k < s->n_items; k++) {
+    const PolyExecItem &it = s->items[k];
+    const KernelGraph &g = graphs[(size_t)k];
+    for (int i = 0; i < it.n_buf_slots && i < (int)g.params.size(); i++) {
+      const int sl = it.buf_slot_indices[i];
+      if (sl < 0 || sl >= s->n_buf_slots) continue;
+      uses[(size_t)sl].push_back({step_of[(size_t)k], k, g.params[(size_t)i].written});
+    }
+  }
+  std::set<int> bad;
+  for (auto &u : uses) {
+    std::sort(u.begin(), u.end(), [](const Use &a, const Use &b) { return a.step < b.step; });
+    // (against every write only: two reads need no order)
+    for (size_t j = 0; j < u.size(); j++) {
+      if (!u[j].w) continue;
+      for (size_t i = 0; i < u.size(); i++) {
+        if (i == j || u[i].item == u[j].item) continue;
+        const Use &a = i < j ? u[i] : u[j], &b = i < j ? u[j] : u[i];
+        if (pos[(size_t)a.item] <= pos[(size_t)b.item]) continue;
+        if (group_of[(size_t)a.item] >= 0) bad.insert(group_of[(size_t)a.item]);
+        if (group_of[(size_t)b.item] >= 0) bad.insert(group_of[(size_t)b.item]);
+      }
+    }
+  }
+  return std::vector<int>(bad.begin(), bad.end());
+}
+
 void find_fused_groups(const PolySchedule *s, const std::vector<KernelGraph> &graphs, std::vector<FusedGroup> *out) {
   out->clear();
   if (getenv("POLY_HIP_NO_FUSION")) return;
-  Sched sc{s, graphs, {}, {}, {}};
+  Sched sc{s, graphs, {}, {}, {}, {}};
   sc.step_of.assign((size_t)s->n_items, 0);
   for (int st = 0; st < s->n_items; st++) sc.step_of[(size_t)s->exec_order[st]] = st;
+  sc.launch_step = sc.step_of;
+  auto accept = [&](FusedGroup &fg, std::vector<char> &taken) {
+    for (int it : fg.items) { taken[(size_t)it] = 1; sc.launch_step[(size_t)it] = sc.step_of[(size_t)fg.launch_item]; }
+    out->push_back(std::move(fg));
+  };
   sc.readers.assign((size_t)s->n_buf_slots, {});
   sc.writers.assign((size_t)s->n_buf_slots, {});
   for (int k = 0; k < s->n_items; k++) {
@@ -2405,8 +2470,7 @@ void find_fused_groups(const PolySchedule *s, const std::vector<KernelGraph> &gr
     if (taken[(size_t)k] || graphs[(size_t)k].reduces.size() != 1) continue;
     FusedGroup fg;
     if (!match_attention(sc, k, taken, &fg) && !match_matmul_tail(sc, k, taken, &fg) && !match_row_chain(sc, k, taken, &fg)) continue;
-    for (int it : fg.items) taken[(size_t)it] = 1;
-    out->push_back(std::move(fg));
+    accept(fg, taken);
   }
   // what is left of the pointwise kernels, in runs over the same positions
   for (int st = 0; st < s->n_items; st++) {
@@ -2414,8 +2478,7 @@ void find_fused_groups(const PolySchedule *s, const std::vector<KernelGraph> &gr
     if (taken[(size_t)k] || !graphs[(size_t)k].reduces.empty()) continue;
     FusedGroup fg;
     if (!match_pointwise_group(sc, k, taken, &fg)) continue;
-    for (int it : fg.items) taken[(size_t)it] = 1;
-    out->push_back(std::move(fg));
+    accept(fg, taken);
   }
   // the order-preserving column sums that are left, several to a launch
   for (int st = 0; st < s->n_items; st++) {
@@ -2423,8 +2486,7 @@ void find_fused_groups(const PolySchedule *s, const std::vector<KernelGraph> &gr
     if (taken[(size_t)k] || graphs[(size_t)k].reduces.size() != 1) continue;
     FusedGroup fg;
     if (!match_ordered_sums_side_by_side(sc, k, taken, &fg)) continue;
-    for (int it : fg.items) taken[(size_t)it] = 1;
-    out->push_back(std::move(fg));
+    accept(fg, taken);
   }
   // small kernels that depend on nothing computed in the plan, wherever they stand
   for (int st = 0; st < s->n_items; st++) {
@@ -2432,8 +2494,18 @@ void find_fused_groups(const PolySchedule *s, const std::vector<KernelGraph> &gr
     if (taken[(size_t)k] || !graphs[(size_t)k].reduces.empty()) continue;
     FusedGroup fg;
     if (!match_side_by_side(sc, k, taken, &fg)) continue;
-    for (int it : fg.items) taken[(size_t)it] = 1;
-    out->push_back(std::move(fg));
+    accept(fg, taken);
+  }
+  // every pair of items that share a buffer keeps its order; a group that breaks one is
+  // dropped and its kernels launch one by one at their own places
+  for (;;) {
+    const std::vector<int> bad = fused_groups_out_of_order(s, graphs, *out);
+    if (bad.empty()) break;
+    for (size_t i = bad.size(); i-- > 0;) {
+      log_err("compile_schedule", "fused group at kernel %d (%zu kernels: %s) would launch out of order with a kernel it shares a buffer with: dropped",
+              (*out)[(size_t)bad[i]].launch_item, (*out)[(size_t)bad[i]].items.size(), (*out)[(size_t)bad[i]].rk.strategy.substr(0, 60).c_str());
+      out->erase(out->begin() + bad[i]);
+    }
   }
 }
 

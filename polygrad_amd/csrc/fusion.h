@@ -19,5 +19,9 @@ struct FusedGroup {
 // Finds the fusable groups of a schedule.  graphs[k] is the analysed kernel of item k.
 // Setting POLY_HIP_NO_FUSION in the environment disables the search.
 void find_fused_groups(const PolySchedule *s, const std::vector<KernelGraph> &graphs, std::vector<FusedGroup> *out);
+// The groups (indices into `groups`) whose place of launch breaks the order of two kernels
+// of the schedule that share a buffer, one of them writing it; find_fused_groups drops such
+// groups itself, so that its result always passes.
+std::vector<int> fused_groups_out_of_order(const PolySchedule *s, const std::vector<KernelGraph> &graphs, const std::vector<FusedGroup> &groups);
 
 }  // namespace polyhip

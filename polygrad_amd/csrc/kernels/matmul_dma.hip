@@ -115,12 +115,14 @@ static_assert(POLY_A_NI % POLY_NW == 0 && POLY_B_NI % POLY_NW == 0, "every wave 
 static_assert(POLY_BK == 32 || POLY_BK == 64, "K tile of 32 or 64");
 
 // ── layouts ────────────────────────────────────────────────────────────────
-// K-contiguous operand, [row][BK]: BK/8 chunks of 16 bytes per row.  With 8 chunks a row
-// is 128 bytes and the chunk index is XORed with the row number; with 4 chunks two rows
-// share 128 bytes and the chunk index is XORed with bits 1-2 of the row number: either
-// way 8 consecutive rows reading the same logical chunk cover 128 distinct bytes.
+// K-contiguous operand, [row][BK]: BK/8 chunks of 16 bytes per row.  A 16-byte fragment
+// read is served 16 lanes at a time over 256 bytes of banks: the 16 lanes read the same
+// logical chunk of 16 consecutive rows, which must land on 16 different 16-byte slots
+// modulo 256 bytes.  With 8 chunks (rows of 128 bytes, two rows per 256) the chunk index
+// is XORed with the row number and with the row number / 8; with 4 chunks (rows of 64
+// bytes, four rows per 256) with the row number / 4.
 #define POLY_CH (POLY_BK / 8)
-__device__ __forceinline__ int poly_swz_k(int row) { return POLY_CH == 8 ? ((row ^ (row >> 3)) & 7) : ((row >> 1) & 3); }
+__device__ __forceinline__ int poly_swz_k(int row) { return POLY_CH == 8 ? ((row ^ (row >> 3)) & 7) : ((row >> 2) & 3); }
 // Row-contiguous operand, [k][ROWS]: the transposing read of 16 lanes touches 4
 // consecutive k-rows x 32 bytes (32 lanes: 4 x 64 bytes), all at the same logical chunk;
 // the XOR term spreads the four rows over bits 0-1 and bits 1-2 of the chunk index.
@@ -518,7 +520,11 @@ extern "C" __global__ void __launch_bounds__(POLY_NTHREADS) POLY_WAVES_ATTR poly
             o[e] = POLY_EP_VALUE(v[e], m, ne, z);
           }
           if (POLY_N % 8 == 0 || n + 7 < POLY_N) {
+#ifdef POLY_EP_NT
+            __builtin_nontemporal_store(o, (poly_out8_u *)POLY_EP_PTR(m, n, z));
+#else
             *(poly_out8_u *)POLY_EP_PTR(m, n, z) = o;
+#endif
           } else {
 #pragma unroll
             for (int e = 0; e < 8; e++)

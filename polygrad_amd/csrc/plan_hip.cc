@@ -163,7 +163,7 @@ bool slot_fully_written(const PolySchedule *s, int slot, const std::vector<Kerne
         bool aff;
         int64_t c = g.lin_range_coef(l, r, &aff);
         const int64_t ext = g.ranges[(size_t)r].extent;
-        if (!aff || ext <= 0) { ok = false; break; }
+        if (!aff || ext <= 0 || r >= 64) { ok = false; break; }
         seen |= 1ull << r;
         if (c == 0 || ext == 1) continue;              // rewrites the same elements / a single value
         if (c < 0) { base += c * (ext - 1); c = -c; }  // walks downwards: the interval starts at its last step
@@ -628,35 +628,46 @@ PolyHipPlan *poly_hip_compile_schedule(PolyCtx *ctx, const PolySchedule *s) {
         plan->forked = false;
       }
     }
-    if (plan->forked && getenv("POLY_HIP_DEBUG")) {
-      fprintf(stderr, "polygrad: compile_schedule: %d of %d launches on %d side streams, %d waits between the streams, %d of them by the main sequence\n",
-              n_on_side, n_units, plan->n_side_streams, n_waits, n_main_waits);
-      for (int i = 0; i < n_units; i++)
-        for (int w : plan->waits[(size_t)i])
-          if (plan->on_side[(size_t)i] == 0 || n_waits <= 16) fprintf(stderr, "polygrad: compile_schedule: launch %d (stream %d) waits for launch %d (stream %d)\n", i, plan->on_side[(size_t)i], w,
-                  plan->on_side[(size_t)w]);
-      // every pair of launches on different streams that touch the same bytes, one of them
-      // writing, must be ordered by the waits (checked here from scratch, pair by pair)
-      {
-        // seen[i][b]: latest launch of stream b known to be over when i starts
-        std::vector<std::array<int, kSideStreams + 1>> seen((size_t)n_units);
-        int last_on[kSideStreams + 1];
-        for (int &v : last_on) v = -1;
-        long long unordered = 0, pairs = 0;
-        for (int i = 0; i < n_units; i++) {
-          const int me = plan->on_side[(size_t)i];
-          for (int b = 0; b <= kSideStreams; b++) seen[(size_t)i][(size_t)b] = last_on[me] >= 0 ? seen[(size_t)last_on[me]][(size_t)b] : -1;
-          for (int w : plan->waits[(size_t)i]) {
-            int &v = seen[(size_t)i][(size_t)plan->on_side[(size_t)w]];
-            v = std::max(v, w);
-          }
-          last_on[me] = i;
-          for (int j = 0; j < i; j++) {
-            const int sj = plan->on_side[(size_t)j];
-            if (sj != me && conflict(i, j)) { pairs++; if (j > seen[(size_t)i][(size_t)sj]) unordered++; }
-          }
+    if (plan->forked) {
+      const bool debug = getenv("POLY_HIP_DEBUG") != nullptr;
+      if (debug) {
+        fprintf(stderr, "polygrad: compile_schedule: %d of %d launches on %d side streams, %d waits between the streams, %d of them by the main sequence\n",
+                n_on_side, n_units, plan->n_side_streams, n_waits, n_main_waits);
+        for (int i = 0; i < n_units; i++)
+          for (int w : plan->waits[(size_t)i])
+            if (plan->on_side[(size_t)i] == 0 || n_waits <= 16) fprintf(stderr, "polygrad: compile_schedule: launch %d (stream %d) waits for launch %d (stream %d)\n", i, plan->on_side[(size_t)i], w,
+                    plan->on_side[(size_t)w]);
+      }
+      // Every pair of launches on different streams that touch the same bytes, one of them
+      // writing, must be ordered by the waits: checked here from scratch, pair by pair,
+      // whenever a plan is forked (cheap next to compiling its kernels).  A plan that fails
+      // runs on one stream.
+      // seen[i][b]: latest launch of stream b known to be over when i starts
+      std::vector<std::array<int, kSideStreams + 1>> seen((size_t)n_units);
+      int last_on[kSideStreams + 1];
+      for (int &v : last_on) v = -1;
+      long long unordered = 0, pairs = 0;
+      for (int i = 0; i < n_units; i++) {
+        const int me = plan->on_side[(size_t)i];
+        for (int b = 0; b <= kSideStreams; b++) seen[(size_t)i][(size_t)b] = last_on[me] >= 0 ? seen[(size_t)last_on[me]][(size_t)b] : -1;
+        for (int w : plan->waits[(size_t)i]) {
+          int &v = seen[(size_t)i][(size_t)plan->on_side[(size_t)w]];
+          v = std::max(v, w);
         }
-        fprintf(stderr, "polygrad: compile_schedule: %lld pairs of launches across the streams share bytes, %lld of them unordered\n", pairs, unordered);
+        last_on[me] = i;
+        for (int j = 0; j < i; j++) {
+          const int sj = plan->on_side[(size_t)j];
+          if (sj != me && conflict(i, j)) { pairs++; if (j > seen[(size_t)i][(size_t)sj]) unordered++; }
+        }
+      }
+      if (debug) fprintf(stderr, "polygrad: compile_schedule: %lld pairs of launches across the streams share bytes, %lld of them unordered\n", pairs, unordered);
+      if (unordered != 0) {
+        log_err("compile_schedule", "%lld pairs of launches on different streams share bytes without an order between them: everything stays on one stream", unordered);
+        plan->on_side.assign((size_t)n_units, 0);
+        plan->waits.assign((size_t)n_units, std::vector<int>());
+        plan->records.assign((size_t)n_units, 0);
+        plan->n_side_streams = 0;
+        plan->forked = false;
       }
     }
   }

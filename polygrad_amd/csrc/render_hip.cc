@@ -90,13 +90,18 @@ std::vector<int> hoist_vector_loads(const KernelGraph &g_, Emitter &em_, const s
   return done;
 }
 
-std::string wave_reduce_call(PolyOps op, DT dt, const std::string &v) {
+std::string wave_reduce_call(PolyOps op, DT dt, const std::string &v, int lanes) {
   if (dt == DT_F32) {
-    const char *fn = op == POLY_OP_ADD ? "poly_wave_add_f32" : op == POLY_OP_MUL ? "poly_wave_mul_f32" : "poly_wave_max_f32";
-    return strf("%s(%s)", fn, v.c_str());
+    const char *fn = op == POLY_OP_ADD ? "add" : op == POLY_OP_MUL ? "mul" : "max";
+    return strf("poly_%s_%s_f32(%s)", lanes == 32 ? "half" : "wave", fn, v.c_str());
   }
   const char *ct = dt_cname(dt);
   std::string comb = Emitter::reduce_combine(op, dt, "a_", "b_");
+  if (lanes == 32) {
+    // (the lambda's type cannot be named in front of the lane count: the call goes through a variable)
+    return strf("[&]() { auto f_ = [](%s a_, %s b_) { return (%s)%s; }; return poly_wave_reduce_any<%s, decltype(f_), 32>(%s, f_); }()", ct, ct, ct, comb.c_str(),
+                ct, v.c_str());
+  }
   return strf("poly_wave_reduce_any<%s>(%s, [](%s a_, %s b_) { return (%s)%s; })", ct, v.c_str(), ct, ct, ct, comb.c_str());
 }
 
@@ -504,7 +509,7 @@ class Generic {
     return true;
   }
 
-  std::string wave_reduce_call(PolyOps op, DT dt, const std::string &v) const { return polyhip::wave_reduce_call(op, dt, v); }
+  std::string wave_reduce_call(PolyOps op, DT dt, const std::string &v) const { return polyhip::wave_reduce_call(op, dt, v, 64); }
 
   std::string render_coop(RenderedKernel *out) {
     const Group &gr = groups_[0];

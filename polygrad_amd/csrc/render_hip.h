@@ -230,7 +230,8 @@ std::vector<int> hoist_vector_loads(const KernelGraph &g, Emitter &em, const std
                                     const std::function<std::string(int, const std::string &)> *wrap = nullptr,
                                     bool any_alignment = false);
 // C expression reducing `v` over the 64 lanes of a wave.
-std::string wave_reduce_call(PolyOps op, DT dt, const std::string &v);
+// (lanes: 64, or 32 for a reduction over each half of the wave by itself)
+std::string wave_reduce_call(PolyOps op, DT dt, const std::string &v, int lanes = 64);
 
 // Prelude with the wave/workgroup reduction helpers and small utilities that
 // every generated kernel may use.

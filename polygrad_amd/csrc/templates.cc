@@ -980,6 +980,27 @@ static bool eval_lin(const KernelGraph &g, const Lin &l, const std::vector<int64
   return true;
 }
 
+// Does every atom of index `l` depend on ranges of only one of the three groups (bit masks
+// of range ordinals), and on no other range?  Then the index is a sum of a part per group.
+// A DIV or MOD atom whose inner expression mixes ranges of two groups fails here whatever
+// values a sampled comparison would happen to hit.  (An atom over a single range is fine
+// even when two groups own digits of that range: its uses are taken apart digit by digit.)
+static bool lin_separates(const KernelGraph &g, const Lin &l, uint64_t rows_mask, uint64_t k_mask, uint64_t z_mask) {
+  for (const Term &t : l.terms) {
+    const uint64_t deps = g.atom_deps(t.atom);
+    if (deps & ~(rows_mask | k_mask | z_mask)) return false;
+    if ((deps & (deps - 1)) == 0) continue;
+    const int groups = ((deps & rows_mask) != 0) + ((deps & k_mask) != 0) + ((deps & z_mask) != 0);
+    if (groups > 1) return false;
+  }
+  return true;
+}
+static uint64_t ord_mask(const std::vector<Dim> &dims) {
+  uint64_t m = 0;
+  for (const Dim &d : dims) if (d.ord >= 0 && d.ord < 64) m |= (uint64_t)1 << d.ord;
+  return m;
+}
+
 // Describes operand `node` of a product without naming ranges (RenderedKernel::OperandPlanes):
 // `loads` are its LOADs, `rows` / `kd` / `zd` the digits that make up its row, depth and
 // batch coordinates.
@@ -1049,14 +1070,14 @@ static void describe_operand(const KernelGraph &g, int node, const std::vector<i
     d.param = g.param_slot(ix.src[0]);
     d.dt = (int)ld.dt;
     if (d.param < 0 || !address(l, 0, 0, 0, &d.base)) return;
+    if (!lin_separates(g, l, ord_mask(rows), ord_mask(kd), ord_mask(zd))) return;
     d.by_row.resize((size_t)M); d.by_k.resize((size_t)K); d.by_z.resize((size_t)Z);
     int64_t a;
     for (int64_t m = 0; m < M; m++) { if (!address(l, m, 0, 0, &a)) return; d.by_row[(size_t)m] = a - d.base; }
     for (int64_t k = 0; k < K; k++) { if (!address(l, 0, k, 0, &a)) return; d.by_k[(size_t)k] = a - d.base; }
     for (int64_t z = 0; z < Z; z++) { if (!address(l, 0, 0, z, &a)) return; d.by_z[(size_t)z] = a - d.base; }
-    // the address is the sum of the three parts: every atom of a canonical index depends on
-    // one range, and every use of a range is a sum over its digits; checked at scattered
-    // points and the far corner all the same
+    // the address is the sum of the three parts (no atom mixes two of them: checked above by
+    // structure); compared at scattered points and the far corner all the same
     uint64_t rnd = 0x9e3779b97f4a7c15ull;
     for (int t = 0; t < 256; t++) {
       rnd = rnd * 6364136223846793005ull + 1442695040888963407ull;
@@ -1378,6 +1399,11 @@ bool try_render_matmul_generic(const KernelGraph &g, const std::string &fn, cons
         };
         coefs(side == 0 ? mm.md_full : mm.nd_full, &ip.rows);
         coefs(mm.zd_full, &ip.z);
+        {
+          uint64_t k_mask = 0;
+          for (int r : kr) if (r >= 0 && r < 64) k_mask |= (uint64_t)1 << r;
+          if (!lin_separates(g, l, ord_mask(ip.rows), k_mask, ord_mask(ip.z))) ok = false;
+        }
         // (the digits must be all there is to the index: checked against the canonical form
         // at the far corner and at scattered points)
         std::vector<int64_t> rv(g.ranges.size());

@@ -464,3 +464,41 @@ def test_gpt2_medium_24_layer_train_step_full_size():
         assert bool((torch.sign(step[big]) == -torch.sign(want[big])).float().mean() > 0.995), name
         assert float(step.abs().max()) <= 2.2 * 3e-4
     print("worst (mean, max) error over scale:", worst)
+
+
+def test_24_layer_side_streams_change_no_bit():
+    """The 24-layer training plan runs several hundred small launches on side streams of its
+    captured graph, in an arena whose buffers share bytes.  Three passes in a row (the first
+    captures the graph, the others replay it; every pass is an optimizer step on the state
+    the pass before left) must leave every tensor of the state, bit for bit, as the same
+    three passes on one stream do: a missing wait between two streams would show here even
+    where it stays inside the tolerances of the comparison with the torch restatement."""
+    import torch
+    from polygrad_amd.inputs import block_train_slot_tensors
+    path = os.path.join(PLANS, "gpt2_medium_train_24l_b4_t1024.polyplan")
+    if not os.path.exists(path):
+        pytest.skip("the 24-layer plan is not generated (python tests/golden/make_plans.py train24)")
+
+    def three_passes(one_stream):
+        if one_stream:
+            os.environ["POLY_HIP_NO_SIDE_STREAM"] = "1"
+        try:
+            plan = load("gpt2_medium_train_24l_b4_t1024")
+        finally:
+            os.environ.pop("POLY_HIP_NO_SIDE_STREAM", None)
+        data, t = block_train_slot_tensors(plan)
+        side = plan.side_launches()
+        for _ in range(3):
+            plan.run(data)
+        torch.cuda.synchronize()
+        plan.close()
+        return t, side
+
+    forked, n_side = three_passes(False)
+    assert n_side > 100, n_side
+    single, n_single = three_passes(True)
+    assert n_single == 0
+    assert set(forked) == set(single)
+    differing = [k for k in forked if not torch.equal(forked[k].view(torch.uint8), single[k].view(torch.uint8))]
+    assert not differing, differing[:10]
+    assert bool(torch.isfinite(forked["loss"].float()).all())

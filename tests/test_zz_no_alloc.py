@@ -94,17 +94,33 @@ def test_static_scratch_matches_allocated_scratch_two_calls_in_a_row():
     assert staged[big] > staged[small]
     kernels = [Kernel(plan, big, seed=11), Kernel(plan, small, seed=12)]
     try:
+        import torch
+        # the static path first, on runners that have never run and so own no scratch memory:
+        # the calls must leave the device's free memory where it was (the runner's own scratch
+        # of this size would show: hipMalloc takes whole 2 MiB pieces for it)
+        for kn in kernels:
+            kn.upload()
+        torch.cuda.synchronize()
+        free_before = torch.cuda.mem_get_info()[0]
+        got = []
+        for kn in kernels:                           # back to back on the shared array
+            rc = kn.lib.poly_hip_execute_static(C.byref(kn.runner), kn.args, len(kn.dev))
+            assert rc == 0
+        assert kn.lib.poly_hip_sync() == 0
+        free_after = torch.cuda.mem_get_info()[0]
+        # (the runtime may take a little memory of its own at a kernel's first launch; the
+        # runner's scratch for the larger kernel is 12 MiB)
+        assert staged[big] >= (8 << 20), "the larger kernel's scratch would be too small to show in the free memory"
+        assert free_before - free_after < staged[big] // 2, f"poly_hip_execute_static took {free_before - free_after} bytes of device memory"
+        for kn in kernels:
+            got.append(kn.download())
         want = []
         for kn in kernels:
             rc, out = kn.run(static=False)
             assert rc == 0
             want.append(out)
-        got = []
-        for kn in kernels:                           # back to back on the shared array
-            rc, out = kn.run(static=True)
-            assert rc == 0
-            got.append(out)
         for w, g_, kn, k in zip(want, got, kernels, (big, small)):
+            assert (g_[0] != kn.host[0]).any(), "the static path wrote nothing"
             assert (w[0] != kn.host[0]).any(), "the kernel wrote nothing"
             for a, b in zip(w, g_):
                 assert a.tobytes() == b.tobytes(), f"kernel {k}: static-scratch result differs"
