@@ -777,9 +777,11 @@ bool render_matmul(const MatmulMatch &mm, const MatmulEpilogue &ep, RenderedKern
                   (long long)(mm.b_c0 & ~1ll), (long long)((K * N * 2 - 64) / 64));
     }
     if (n_lo != 0 || n_hi != N) cfg += strf("#define POLY_N_LO %lld\n#define POLY_N_HI %lld\n", (long long)n_lo, (long long)n_hi);
-    cfg += strf("#define POLY_GROUP_M %d\n", bm >= 256 ? 4 : 8);
     // each XCD (own L2) works on a contiguous run of tiles: let it re-read the smaller operand
-    cfg += strf("#define POLY_GROUP_ALONG_N %d\n", (N > 2 * M && !getenv("POLY_HIP_MM_GROUP_M")) ? 1 : 0);
+    const bool along_n = N > 2 * M && !getenv("POLY_HIP_MM_GROUP_M");
+    // (bands of 8 tile columns for the wide product: the 50257-wide head 727 -> 710 us against bands of 4)
+    cfg += strf("#define POLY_GROUP_M %d\n", bm >= 256 && !(along_n && use_dma) ? 4 : 8);
+    cfg += strf("#define POLY_GROUP_ALONG_N %d\n", along_n ? 1 : 0);
     cfg += strf("#define POLY_PIPE %d\n", pp);
     // timing experiments only (wrong results): walk just the first n K tiles
     if (const char *e = measurement_env("POLY_HIP_MM_KT")) if (atoi(e) > 0 && atoi(e) <= K / bk) cfg += strf("#define POLY_KT %d\n", atoi(e));
@@ -848,22 +850,32 @@ bool render_matmul(const MatmulMatch &mm, const MatmulEpilogue &ep, RenderedKern
     return true;
   };
   // Tile shapes of the straight-into-LDS template, from timings inside the GPT-2 forward
-  // plan (M = 8192, K = 768 or 3072): a launch of at most 256 tiles of 128x256 leaves a CU
-  // one workgroup of four waves, which is too little to hide anything: 128x128 tiles, two
-  // workgroups to a CU (N = 768: 21.7 -> 19.6 us at K = 768, 47.8 -> 46.2 us at K = 3072);
-  // between one and one and a quarter rounds of 512 workgroups, 128x192 tiles when they
-  // divide N and give a round and a half (N = 2304: 43.6 -> 39.9 us).
-  if (S == 1 && !fixed_tile && !getenv("POLY_HIP_MM_TILE") && BM * BN == 128 * 256) {
+  // plan (M = 8192, K = 768 or 3072) and the GPT-2 medium training step (M = 4096, N = 1024,
+  // K = 4096).  A launch of at most 256 tiles of 128x256 leaves a CU one workgroup of four
+  // waves, too little to hide anything: 128x128 tiles -- two workgroups to a CU on two
+  // stages of 64 when there are more than 256 of them (N = 768: 21.7 -> 19.6 us at K = 768,
+  // 47.8 -> 46.2 us at K = 3072), one to a CU on four stages otherwise (4096x1024x4096: 32 us
+  // against 48 us on two stages and 44 us for the template that stages through registers).
+  // Between one and one and a quarter rounds of 512 workgroups, 128x192 tiles when they
+  // divide N and give a round and a half (N = 2304: 43.6 -> 39.9 us).  Narrow outputs (one
+  // tile of 64 across) stay with the template that stages through registers.
+  Dma chosen{0, 0, 0, 0, 0};
+  bool dma_ok = !fixed_tile;
+  if (!fixed_tile && !getenv("POLY_HIP_MM_TILE") && BM * BN <= 128 * 256) {
     Dma probe{0, 0, 0, 0, 0};
-    auto count = [&](int bm, int bn) { return ((M + bm - 1) / bm) * ((N + bn - 1) / bn) * Z; };
+    auto count = [&](int bm, int bn) { return ((M + bm - 1) / bm) * ((N + bn - 1) / bn) * Z * S; };   // workgroups of the launch
     const int64_t t = count(BM, BN);
     if (dma_for(BM, BN, &probe)) {
       Dma p2{0, 0, 0, 0, 0}, p3{0, 0, 0, 0, 0};
-      if (t <= 256 && M % 128 == 0 && dma_for(128, 128, &p2)) { BM = BN = 128; WVM = WVN = 2; }
-      else if (t > 512 && t < 640 && N % 192 == 0 && count(128, 192) >= 768 && dma_for(128, 192, &p3)) { BM = 128; BN = 192; WVM = WVN = 2; }
+      if (S == 1 && BM * BN == 128 * 256 && t <= 256 && M % 128 == 0 && dma_for(128, 128, &p2)) { BM = BN = 128; WVM = WVN = 2; }
+      else if (S == 1 && BM * BN == 128 * 256 && t > 512 && t < 640 && N % 192 == 0 && count(128, 192) >= 768 && dma_for(128, 192, &p3)) { BM = 128; BN = 192; WVM = WVN = 2; }
+      if (BM == 128 && BN == 128 && count(128, 128) <= 256) {
+        Dma deep{64, 4, 1, 2, 2};
+        if (dma_for(128, 128, &deep)) chosen = deep;
+      }
     }
   }
-  if (!emit(BM, BN, WVM, WVN, pipe, out)) return false;
+  if (!emit(BM, BN, WVM, WVN, pipe, out, 0, -1, dma_ok, chosen)) return false;
   if (S > 1) {
     // the template becomes a first stage; the kernel proper adds the partial results up
     RenderedKernel::Pre pre{out->source, out->entry, out->launch};
