@@ -178,6 +178,13 @@ size_t poly_hip_plan_workspace_bytes(const PolyHipPlan *plan);
  * No counterpart in the reference, whose plans run kernel by kernel with a sync after
  * each (src/exec_plan.c:1000-1057). */
 int poly_hip_plan_side_launches(const PolyHipPlan *plan);
+/* How the plan's graph met the bindings it has run with: *captures = times the launch
+ * sequence went through stream capture, *rebinds = times a binding (a set of buffer
+ * addresses and variable values) not seen before was served by instantiating the
+ * captured graph again and giving every kernel node the new argument values.  A binding
+ * seen before (all values compared, up to four kept) replays its graph and counts in
+ * neither.  No counterpart in the reference (src/exec_plan.c:1000-1057 has no graphs). */
+void poly_hip_plan_graph_counts(const PolyHipPlan *plan, long long *captures, long long *rebinds);
 
 /* ── Serialized schedules ("plan files") ─────────────────────────────────── */
 

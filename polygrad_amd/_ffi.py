@@ -107,6 +107,7 @@ SYMBOLS = {
     "poly_hip_plan_set_graph": (None, [C.c_void_p, C.c_int]),
     "poly_hip_plan_workspace_bytes": (C.c_size_t, [C.c_void_p]),
     "poly_hip_plan_side_launches": (C.c_int, [C.c_void_p]),
+    "poly_hip_plan_graph_counts": (None, [C.c_void_p, C.POINTER(C.c_longlong), C.POINTER(C.c_longlong)]),
     "poly_hip_planfile_save": (C.c_int, [C.c_void_p, C.POINTER(C.c_char_p), C.c_char_p]),
     "poly_hip_planfile_load": (C.c_void_p, [C.c_char_p]),
     "poly_hip_planfile_schedule": (C.POINTER(PolySchedule), [C.c_void_p]),

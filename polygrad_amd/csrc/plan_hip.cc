@@ -34,9 +34,10 @@ using namespace polyhip;
 
 namespace {
 
+// One instantiated graph of the plan's launch sequence, bound to one set of buffers and
+// variable values (compared value by value, not by a hash of them).
 struct GraphEntry {
-  uint64_t key = 0;
-  hipGraph_t graph = nullptr;
+  std::vector<uint64_t> bound;
   hipGraphExec_t exec = nullptr;
   uint64_t last_use = 0;
 };
@@ -115,13 +116,20 @@ struct PolyHipPlan {
   Program *touch = nullptr;
   bool use_graph = true;
   bool tuned = false;            // candidates of the tunable kernels have been timed (or there are none)
+  // The launch sequence is captured once (`captured`, with the kernel node of every launch
+  // in `launches`); a binding the plan has not seen gets a graph instantiated from it whose
+  // kernel nodes receive the new argument values, not a capture of its own.
+  hipGraph_t captured = nullptr;
+  GraphLaunches launches;
+  bool captured_forked = false;              // the capture put launches on side streams
   std::vector<GraphEntry> graphs;
+  std::vector<uint64_t> bound_now;           // the current binding: external pointers, then variable values
   uint64_t tick = 0;
+  long long n_captures = 0, n_rebinds = 0;   // (how often the sequence was captured / rebound by updating nodes)
   ~PolyHipPlan() {
-    for (GraphEntry &g : graphs) {
+    for (GraphEntry &g : graphs)
       if (g.exec) (void)hipGraphExecDestroy(g.exec);
-      if (g.graph) (void)hipGraphDestroy(g.graph);
-    }
+    if (captured) (void)hipGraphDestroy(captured);
     for (Unit &u : units) runner_destroy(u.runner);
     if (fill) program_destroy(fill);
     if (touch) program_destroy(touch);
@@ -744,10 +752,12 @@ static int bind_args(PolyHipPlan *plan, void **slot_data, int n_slots, const Pol
                      uint64_t *key_out) {
   const PolySchedule *s = plan->sched;
   uint64_t key = 1469598103934665603ull;
+  plan->bound_now.clear();
   if (plan->vetted_slot.size() != (size_t)s->n_buf_slots) plan->vetted_slot.assign((size_t)s->n_buf_slots, nullptr);
   for (int i = 0; i < s->n_buf_slots; i++) {
     if (s->buf_slots[i].is_intermediate) continue;
     plan->slot_ptr[(size_t)i] = (i < n_slots && slot_data) ? slot_data[i] : nullptr;
+    plan->bound_now.push_back((uint64_t)(uintptr_t)plan->slot_ptr[(size_t)i]);
     key = fnv1a(&plan->slot_ptr[(size_t)i], sizeof(void *), key);
     // A host address in a device plan (the frontend's constant registry, src/frontend.c:2231-2232,
     // or a training step's loss slot, src/instance.c:1299-1311) would fault in the first kernel
@@ -790,6 +800,7 @@ static int bind_args(PolyHipPlan *plan, void **slot_data, int n_slots, const Pol
         if (m.var == un.var_uops[(size_t)v]) { plan->var_vals[u][(size_t)v] = m.value; found = true; break; }
       if (!found) { log_err("plan_run", "no binding for DEFINE_VAR in kernel %d", un.item); return -1; }
       a[un.slots.size() + (size_t)v] = &plan->var_vals[u][(size_t)v];
+      plan->bound_now.push_back((uint64_t)(uint32_t)plan->var_vals[u][(size_t)v]);
       key = fnv1a(&plan->var_vals[u][(size_t)v], sizeof(int), key);
     }
   }
@@ -910,23 +921,15 @@ int poly_hip_plan_run(PolyHipPlan *plan, void **slot_data, int n_slots, const Po
   hipStream_t stream = (hipStream_t)runtime_stream();
   if (!plan->use_graph || getenv("POLY_HIP_NO_GRAPH")) return enqueue_all(plan);
   plan->tick++;
+  (void)key;
   for (GraphEntry &g : plan->graphs)
-    if (g.key == key && g.exec) {
+    if (g.exec && g.bound == plan->bound_now) {
       g.last_use = plan->tick;
       if (hipGraphLaunch(g.exec, stream) != hipSuccess) { log_err("plan_run", "hipGraphLaunch failed"); return -1; }
       return 0;
     }
-  // First sight of this binding: capture the launch sequence, then replay it.
-  GraphEntry ge;
-  ge.key = key;
-  ge.last_use = plan->tick;
-  if (hipStreamBeginCapture(stream, hipStreamCaptureModeThreadLocal) != hipSuccess) {
-    log_err("plan_run", "hipStreamBeginCapture failed; running without a graph");
-    plan->use_graph = false;
-    return enqueue_all(plan);
-  }
-  // (the order between the two streams was worked out with every bound buffer a resource
-  // of its own: two bound buffers that share bytes put everything on one stream)
+  // (the order between the streams was worked out with every bound buffer a resource of its
+  // own: two bound buffers that share bytes put everything on one stream)
   bool disjoint = true;
   if (plan->forked) {
     std::vector<std::pair<uintptr_t, uintptr_t>> ext;
@@ -936,29 +939,83 @@ int poly_hip_plan_run(PolyHipPlan *plan, void **slot_data, int n_slots, const Po
     std::sort(ext.begin(), ext.end());
     for (size_t i = 1; i < ext.size(); i++) if (ext[i].first < ext[i - 1].second) disjoint = false;
   }
-  int rc = plan->forked && disjoint ? enqueue_captured(plan) : enqueue_all(plan);
-  hipError_t e = hipStreamEndCapture(stream, &ge.graph);
-  if (rc != 0 || e != hipSuccess || !ge.graph) {
-    if (ge.graph) (void)hipGraphDestroy(ge.graph);
+  auto keep = [&](GraphEntry &ge) {
+    if (plan->graphs.size() >= 4) {
+      size_t victim = 0;
+      for (size_t i = 1; i < plan->graphs.size(); i++)
+        if (plan->graphs[i].last_use < plan->graphs[victim].last_use) victim = i;
+      (void)hipGraphExecDestroy(plan->graphs[victim].exec);
+      plan->graphs.erase(plan->graphs.begin() + (long)victim);
+    }
+    plan->graphs.push_back(ge);
+  };
+  GraphEntry ge;
+  ge.bound = plan->bound_now;
+  ge.last_use = plan->tick;
+  // A binding the plan has not run with, and the sequence is captured already: a graph
+  // instantiated from the capture, every kernel node given the arguments of this binding
+  // (the launches are walked as for a capture, but each call only updates its node).
+  if (plan->captured && !plan->launches.failed && !getenv("POLY_HIP_NO_GRAPH_REBIND") && (!plan->captured_forked || disjoint)) {
+    if (hipGraphInstantiate(&ge.exec, plan->captured, nullptr, nullptr, 0) == hipSuccess) {
+      plan->launches.exec = (void *)ge.exec;
+      plan->launches.next = 0;
+      runtime_graph_update(&plan->launches);
+      int rc = 0;
+      for (size_t u = 0; u < plan->units.size() && rc == 0; u++) rc = launch_unit(plan, u);
+      runtime_graph_update(nullptr);
+      const bool ok = rc == 0 && !plan->launches.failed && plan->launches.next == plan->launches.nodes.size();
+      plan->launches.failed = false;      // (a failed update says nothing about the capture)
+      if (ok) {
+        plan->n_rebinds++;
+        keep(ge);
+        if (hipGraphLaunch(ge.exec, stream) != hipSuccess) { log_err("plan_run", "hipGraphLaunch failed"); return -1; }
+        return 0;
+      }
+      (void)hipGraphExecDestroy(ge.exec);
+      ge.exec = nullptr;
+      log_err("plan_run", "the captured graph could not be bound to new buffers by updating its nodes; capturing again");
+    }
+    // the capture is replaced below
+    for (GraphEntry &g : plan->graphs) if (g.exec) (void)hipGraphExecDestroy(g.exec);
+    plan->graphs.clear();
+    (void)hipGraphDestroy(plan->captured);
+    plan->captured = nullptr;
+  } else if (plan->captured) {
+    // (bound buffers that overlap under a forked capture, or rebinding switched off: this
+    // binding gets a capture of its own, which replaces the old one)
+    for (GraphEntry &g : plan->graphs) if (g.exec) (void)hipGraphExecDestroy(g.exec);
+    plan->graphs.clear();
+    (void)hipGraphDestroy(plan->captured);
+    plan->captured = nullptr;
+  }
+  // First sight of the sequence: capture it, then replay it.
+  if (hipStreamBeginCapture(stream, hipStreamCaptureModeThreadLocal) != hipSuccess) {
+    log_err("plan_run", "hipStreamBeginCapture failed; running without a graph");
+    plan->use_graph = false;
+    return enqueue_all(plan);
+  }
+  plan->launches = GraphLaunches();
+  runtime_graph_record(&plan->launches);
+  plan->captured_forked = plan->forked && disjoint;
+  int rc = plan->captured_forked ? enqueue_captured(plan) : enqueue_all(plan);
+  runtime_graph_record(nullptr);
+  hipError_t e = hipStreamEndCapture(stream, &plan->captured);
+  if (rc != 0 || e != hipSuccess || !plan->captured) {
+    if (plan->captured) (void)hipGraphDestroy(plan->captured);
+    plan->captured = nullptr;
     log_err("plan_run", "graph capture failed; running without a graph");
     plan->use_graph = false;
     return rc != 0 ? rc : enqueue_all(plan);
   }
-  if (hipGraphInstantiate(&ge.exec, ge.graph, nullptr, nullptr, 0) != hipSuccess) {
-    (void)hipGraphDestroy(ge.graph);
+  plan->n_captures++;
+  if (hipGraphInstantiate(&ge.exec, plan->captured, nullptr, nullptr, 0) != hipSuccess) {
+    (void)hipGraphDestroy(plan->captured);
+    plan->captured = nullptr;
     log_err("plan_run", "hipGraphInstantiate failed; running without a graph");
     plan->use_graph = false;
     return enqueue_all(plan);
   }
-  if (plan->graphs.size() >= 4) {
-    size_t victim = 0;
-    for (size_t i = 1; i < plan->graphs.size(); i++)
-      if (plan->graphs[i].last_use < plan->graphs[victim].last_use) victim = i;
-    (void)hipGraphExecDestroy(plan->graphs[victim].exec);
-    (void)hipGraphDestroy(plan->graphs[victim].graph);
-    plan->graphs.erase(plan->graphs.begin() + (long)victim);
-  }
-  plan->graphs.push_back(ge);
+  keep(ge);
   if (hipGraphLaunch(ge.exec, stream) != hipSuccess) { log_err("plan_run", "hipGraphLaunch failed"); return -1; }
   return 0;
 }
@@ -1095,6 +1152,11 @@ int poly_hip_plan_side_launches(const PolyHipPlan *plan) {
   int n = 0;
   if (plan) for (char c : plan->on_side) n += c != 0;
   return n;
+}
+
+void poly_hip_plan_graph_counts(const PolyHipPlan *plan, long long *captures, long long *rebinds) {
+  if (captures) *captures = plan ? plan->n_captures : 0;
+  if (rebinds) *rebinds = plan ? plan->n_rebinds : 0;
 }
 
 size_t poly_hip_plan_workspace_bytes(const PolyHipPlan *plan) { return plan ? plan->arena_bytes + plan->scratch_bytes + plan->kept_scratch_bytes : 0; }

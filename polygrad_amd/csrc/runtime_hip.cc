@@ -37,6 +37,7 @@ struct Runtime {
   int device = 0;
   hipStream_t stream = nullptr;
   hipStream_t side[3] = {nullptr, nullptr, nullptr};   // further streams of a plan's captured graphs, made on first use
+  GraphLaunches *record = nullptr, *update = nullptr;   // see runtime_graph_record / runtime_graph_update
   hipStream_t launch_on = nullptr;     // where program_launch puts kernels when not the main stream
   std::map<uint64_t, std::weak_ptr<Module>> modules;   // keyed by source hash
   std::map<uint64_t, std::vector<char>> code_cache;    // compiled, not yet loaded
@@ -264,11 +265,45 @@ std::shared_ptr<void> runtime_table(const std::string &source, const std::string
   return owner;
 }
 
+void runtime_graph_record(GraphLaunches *g) { rt().record = g; rt().update = nullptr; }
+void runtime_graph_update(GraphLaunches *g) { rt().update = g; rt().record = nullptr; }
+
 int program_launch(Program *p, void **kernel_args, const LaunchSpec &ls) {
   if (!p || runtime_init() != 0) return -1;
+  Runtime &r = rt();
+  if (GraphLaunches *u = r.update) {
+    // the same launch as when the graph was captured, with other argument values: only the
+    // node's arguments change
+    if (u->failed || u->next >= u->nodes.size()) { u->failed = true; return -1; }
+    hipGraphNode_t node = (hipGraphNode_t)u->nodes[u->next++];
+    hipKernelNodeParams kp;
+    memset(&kp, 0, sizeof kp);
+    if (hipGraphKernelNodeGetParams(node, &kp) != hipSuccess) { (void)hipGetLastError(); u->failed = true; return -1; }
+    if (kp.func != (void *)p->fn || kp.blockDim.x != ls.block[0] || kp.sharedMemBytes != ls.lds_bytes) { u->failed = true; return -1; }
+    kp.gridDim = dim3(ls.grid[0], ls.grid[1], ls.grid[2]);     // (a grid may follow a variable's value)
+    kp.kernelParams = kernel_args;
+    kp.extra = nullptr;
+    if (hipGraphExecKernelNodeSetParams((hipGraphExec_t)u->exec, node, &kp) != hipSuccess) { (void)hipGetLastError(); u->failed = true; return -1; }
+    return 0;
+  }
+  hipStream_t stream = r.launch_on ? r.launch_on : r.stream;
   hipError_t e = hipModuleLaunchKernel(p->fn, ls.grid[0], ls.grid[1], ls.grid[2], ls.block[0], ls.block[1],
-                                       ls.block[2], ls.lds_bytes, rt().launch_on ? rt().launch_on : rt().stream, kernel_args, nullptr);
-  return check(e, "hipModuleLaunchKernel") ? 0 : -1;
+                                       ls.block[2], ls.lds_bytes, stream, kernel_args, nullptr);
+  if (!check(e, "hipModuleLaunchKernel")) return -1;
+  if (GraphLaunches *g = r.record) {
+    // which node of the graph under capture the launch became: the one the stream now depends on
+    hipStreamCaptureStatus status = hipStreamCaptureStatusNone;
+    const hipGraphNode_t *deps = nullptr;
+    size_t n_deps = 0;
+    if (hipStreamGetCaptureInfo_v2(stream, &status, nullptr, nullptr, &deps, &n_deps) != hipSuccess || status != hipStreamCaptureStatusActive ||
+        n_deps != 1) {
+      (void)hipGetLastError();
+      g->failed = true;
+    } else {
+      g->nodes.push_back((void *)deps[0]);
+    }
+  }
+  return 0;
 }
 
 }  // namespace polyhip

@@ -39,6 +39,22 @@ Program *program_create(const std::string &source, const std::string &entry);
 void program_destroy(Program *p);
 int program_launch(Program *p, void **kernel_args, const LaunchSpec &ls);
 
+// What program_launch does with a launch besides (or instead of) enqueueing it, for plans
+// that keep their launch sequence as a hipGraph:
+//   record: the stream is under capture; after the launch, the kernel node it became is
+//           appended to `nodes` (failed is set when the capture does not name exactly one);
+//   update: nothing is enqueued; the arguments of the call go to node nodes[next++] of the
+//           instantiated graph `exec` (hipGraphExecKernelNodeSetParams), the way to bind a
+//           captured sequence to other buffers without capturing it again.
+struct GraphLaunches {
+  std::vector<void *> nodes;     // hipGraphNode_t, in launch order
+  void *exec = nullptr;          // hipGraphExec_t (update)
+  size_t next = 0;
+  bool failed = false;
+};
+void runtime_graph_record(GraphLaunches *g);    // nullptr: back to plain launches
+void runtime_graph_update(GraphLaunches *g);
+
 // One lowered kernel: the program(s) plus how to call them.
 struct HipRunner {
   RenderedKernel rk;

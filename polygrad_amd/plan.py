@@ -151,6 +151,14 @@ class HipPlan:
         """Launches that the plan's captured graph runs on a second stream."""
         return int(self.lib.poly_hip_plan_side_launches(self.handle))
 
+    def graph_counts(self):
+        """(captures, rebinds): how often the launch sequence was captured, and how often a
+        new set of buffers was served by updating the captured graph's kernel nodes."""
+        import ctypes as C
+        c, r = C.c_longlong(0), C.c_longlong(0)
+        self.lib.poly_hip_plan_graph_counts(self.handle, C.byref(c), C.byref(r))
+        return int(c.value), int(r.value)
+
     def slot_ptr(self, slot):
         return self.lib.poly_hip_plan_slot_ptr(self.handle, slot)
 

@@ -81,3 +81,39 @@ def test_oracle_agrees_with_gpu_on_fixture_inputs():
     got, info = run_fixture_on_gpu(fx)
     out = [i for i in fx.external if fx.plan.names[i] == "output"][0]
     assert_close(F.as_float(got[out]), F.as_float(want[out]), rtol=2e-2, atol=2e-3, what="gpt2 tiny bf16 logits")
+
+
+def test_attention_with_a_non_finite_value_row(monkeypatch):
+    """Where the single-pass attention kernel and the reference part ways on non-finite data,
+    stated so that a change in either direction shows.  V of key 200 of head 0 is +inf.
+    The reference multiplies every probability with every value, so the zero probabilities of
+    the queries before key 200 meet the infinity (0 x inf = NaN) and every row of the head is
+    non-finite; the CPU oracle and the two-pass kernel do the same.  The single-pass kernel
+    never multiplies a key tile that the causal mask removes for a whole tile of queries: the
+    queries before that key's tile of 32 (rows 0..191) come out finite and exactly as
+    without the infinity; the rows from key 200 on are non-finite as in the reference (the
+    rows 192..199 share the key's tile and see 0 x inf like the reference).  Head 1 is
+    untouched in every form."""
+    fx = F.Fixture("attention_bf16_t256")
+    by = {fx.plan.names[i]: i for i in fx.external}
+    T, J = 256, 200
+    clean, _ = run_fixture_on_gpu(fx)
+    clean = F.as_float(clean[by["out"]]).reshape(T, 2, 64)
+    v = fx.inputs[by["v"]].copy().reshape(T, 2, 64)
+    v[J, 0, :] = 0x7F80                      # +inf as a bf16 bit pattern
+    fx.inputs[by["v"]] = v.reshape(-1)
+    want = F.as_float(F.run_oracle_schedule(fx.plan.schedule, fx.n_slots, fx.inputs)[by["out"]]).reshape(T, 2, 64)
+    assert not np.isfinite(want[:, 0, :]).any() and np.isfinite(want[:, 1, :]).all()
+    online, info = run_fixture_on_gpu(fx)
+    assert any("one pass" in k["desc"] for k in info), [k["desc"] for k in info]
+    online = F.as_float(online[by["out"]]).reshape(T, 2, 64)
+    assert np.isfinite(online[:, 1, :]).all() and (online[:, 1, :] == clean[:, 1, :]).all()
+    assert not np.isfinite(online[J:, 0, :]).any(), "rows from the key on: non-finite, as in the reference"
+    assert np.isfinite(online[:192, 0, :]).all() and (online[:192, 0, :] == clean[:192, 0, :]).all(), \
+        "rows before the key's tile: the masked tile is never multiplied"
+    monkeypatch.setenv("POLY_HIP_EXACT_ATTENTION", "1")
+    exact, info = run_fixture_on_gpu(fx)
+    assert any("two passes" in k["desc"] for k in info), [k["desc"] for k in info]
+    exact = F.as_float(exact[by["out"]]).reshape(T, 2, 64)
+    assert not np.isfinite(exact[:, 0, :]).any(), "the two-pass form propagates like the reference"
+    assert np.isfinite(exact[:, 1, :]).all()

@@ -144,15 +144,18 @@ def test_logits_t1024_one_sequence_plan_matches_reference(monkeypatch, named, we
 
 @pytest.mark.parametrize("form", ["online", "exact"])
 def test_logits_t1024_benchmark_plan_matches_reference(monkeypatch, named, weights_on_device, form):
-    """The plan bench.py times (B=8): the reference's sequence is batch element 5, the
-    other seven are random tokens."""
+    """The plan bench.py times (B=8): the reference's sequence is batch element 0, 5 and 7
+    (first, middle and last: other rows of the same tiles, other workgroups), the other five
+    are random tokens; each of the three is held to the reference's logits."""
     import torch
     marker = set_form(monkeypatch, form)
     ref = np.load(os.path.join(FULL, "gpt2_small_bf16_b1_t1024_logits.npz"))
     plan = HipPlan.from_file(os.path.join(PLANS, "gpt2_small_bf16_b8_t1024.polyplan"))
     g = np.random.default_rng(8)
     tokens = g.integers(0, V, 8 * T).astype(np.float32).reshape(8, T)
-    tokens[5] = named["x"]
+    where = (0, 5, 7)
+    for b in where:
+        tokens[b] = named["x"]
     out = torch.zeros(8 * T * V, dtype=torch.int16, device="cuda")
     data = bind_by_name(plan, weights_on_device, {"x": to_device(tokens.reshape(-1)), "output": out})
     plan.run(data)
@@ -161,10 +164,14 @@ def test_logits_t1024_benchmark_plan_matches_reference(monkeypatch, named, weigh
     plan.close()
     attn = [k["desc"] for k in info if k["klass"] == "attention-mfma"]
     assert len(attn) == 12 and all(marker in d for d in attn), attn
-    lg = out.view(8, T, V)[5]
-    rows = gpt2_data.bf16_bits_to_f32(from_device(lg[torch.as_tensor(ref["rows"], device="cuda")].contiguous(), np.uint16)).astype(np.float64)
-    cols = gpt2_data.bf16_bits_to_f32(from_device(lg[:, torch.as_tensor(ref["cols"], device="cuda")].contiguous(), np.uint16)).astype(np.float64)
-    _check_logits(rows, cols, f"B=8 plan, {form} attention")
+    for b in where:
+        lg = out.view(8, T, V)[b]
+        rows = gpt2_data.bf16_bits_to_f32(from_device(lg[torch.as_tensor(ref["rows"], device="cuda")].contiguous(), np.uint16)).astype(np.float64)
+        cols = gpt2_data.bf16_bits_to_f32(from_device(lg[:, torch.as_tensor(ref["cols"], device="cuda")].contiguous(), np.uint16)).astype(np.float64)
+        _check_logits(rows, cols, f"B=8 plan, batch element {b}, {form} attention")
+    # the same sequence at three places of the batch: the same bits
+    l3 = out.view(8, T, V)
+    assert torch.equal(l3[0], l3[5]) and torch.equal(l3[0], l3[7]), "one sequence, three batch elements: logits differ"
 
 
 @pytest.mark.parametrize("form", ["online", "online, every wave looks at the mask", "exact"])
