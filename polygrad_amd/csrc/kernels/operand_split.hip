@@ -4,7 +4,8 @@
 //
 // An fp32 value x is cut into three bf16 pieces hi + mid + lo (each the bf16 rounding of
 // what the previous ones left over; the two residuals are exact in fp32 and the last
-// rounding is below 2^-25 |x|).  A bf16 x bf16 product is exact in fp32, so
+// rounding is below 2^-25 |x|), or into the first two of them (what is left is below
+// 2^-17 |x|) for a product whose result is stored as a 16-bit float.  A bf16 x bf16 product is exact in fp32, so
 //     sum_k x[k] * b[k]  =  sum over the 3 K_p-long planes of  piece[k'] * b[k' mod K_p]
 // on the bf16 MFMA with fp32 accumulation carries the same information as the fp32
 // product at about a third of the bf16 rate (the fp32 MFMA runs at a sixteenth).  An
@@ -13,7 +14,7 @@
 // Configuration (prepended by templates.cc):
 //   POLY_SP_ROWS / POLY_SP_K / POLY_SP_Z   operand extents (rows = M or N)
 //   POLY_SP_KP                             K rounded up to the K tile of the matmul
-//   POLY_SP_PARTS                          3 (fp32 value) or 1 (already a bf16 value)
+//   POLY_SP_PARTS                          3 or 2 (fp32 value) or 1 (already a bf16 value)
 //   POLY_SP_WALK_K                         1: the source is contiguous along k, 0: along rows
 //   POLY_SP_NRAW, POLY_SP_LOAD(row, k, z, raw), POLY_SP_MATH(row, k, z, raw)
 //                                          the operand as the computed-operand matmul has it
@@ -53,7 +54,7 @@ extern "C" __global__ void __launch_bounds__(256) poly_k(POLY_SIGNATURE) {
 #pragma unroll
     for (int e = 0; e < 8; e++) {
       hi[e] = (__bf16)x[e];
-      if (POLY_SP_PARTS == 3) {
+      if (POLY_SP_PARTS >= 2) {
         // (an infinite or NaN x is all in hi: no inf - inf in the residuals)
         const float r1 = __builtin_isfinite((float)hi[e]) ? x[e] - (float)hi[e] : 0.0f;
         mid[e] = (__bf16)r1;
@@ -61,10 +62,8 @@ extern "C" __global__ void __launch_bounds__(256) poly_k(POLY_SIGNATURE) {
       }
     }
     *(sp_out8 *)dst = hi;
-    if (POLY_SP_PARTS == 3) {
-      *(sp_out8 *)(dst + POLY_SP_KP) = mid;
-      *(sp_out8 *)(dst + 2 * POLY_SP_KP) = lo;
-    }
+    if (POLY_SP_PARTS >= 2) *(sp_out8 *)(dst + POLY_SP_KP) = mid;
+    if (POLY_SP_PARTS == 3) *(sp_out8 *)(dst + 2 * POLY_SP_KP) = lo;
   };
 #if POLY_SP_WALK_K && POLY_SP_K % 8 == 0
   // along k, rows a multiple of 8 long: a thread takes 8 neighbours, so that what the operand's expression loads for

@@ -449,6 +449,7 @@ static bool epilogue_from_graph(const KernelGraph &g, const MatmulMatch &mm, Mat
   {
     const int li = g.n(g.n(st.index).src[1]).lin;
     const DT odt = g.n(st.param).dt;
+    ep.out_16bit = odt == DT_BF16 || odt == DT_F16;
     if (li >= 0 && g.n(st.value).dt == odt && matmul_store_contiguous(g, mm, g.lins[(size_t)li])) {
       // the same code once more, split into the value and the address of an element
       Emitter ev(g), ea(g);
@@ -1354,7 +1355,10 @@ bool try_render_matmul_generic(const KernelGraph &g, const std::string &fn, cons
       const KNode &k = g.n(node);
       return k.op == POLY_OP_CAST && k.dt == DT_F32 && g.n(k.src[0]).dt == DT_BF16;
     };
-    const int parts[2] = {exact16(opnd[0]) ? 1 : 3, exact16(opnd[1]) ? 1 : 3};
+    // (two pieces, hi + lo, leave an error below 2^-17 |x|: enough where the result is
+    // stored as a 16-bit float, whose own rounding is 2^-9 or 2^-12 of it)
+    const int pieces = ep.out_16bit && !getenv("POLY_HIP_SPLIT_THREE") ? 2 : 3;
+    const int parts[2] = {exact16(opnd[0]) ? 1 : pieces, exact16(opnd[1]) ? 1 : pieces};
     const int P = std::max(parts[0], parts[1]);
     const int64_t KP = (K + 63) / 64 * 64;
     const double elems_a = (double)Z * (double)M * parts[0] * (double)KP, elems_b = (double)Z * (double)N * parts[1] * (double)KP;
@@ -1364,7 +1368,8 @@ bool try_render_matmul_generic(const KernelGraph &g, const std::string &fn, cons
     double min_work = 1073741824.0;
     if (const char *e = getenv("POLY_HIP_BF16_SPLIT_MIN")) min_work = std::max(1.0, atof(e));   // tests: small products through this path
     const bool large = (double)M * (double)N * (double)K * (double)Z >= min_work;
-    if (!getenv("POLY_HIP_NO_BF16_SPLIT") && parts[0] + parts[1] <= 4 && fits && large) {
+    // (planes meet plane by plane along K: one side has to be a single plane)
+    if (!getenv("POLY_HIP_NO_BF16_SPLIT") && (parts[0] == 1 || parts[1] == 1) && fits && large) {
       const size_t off_b = ((size_t)elems_a * 2 + 255) / 256 * 256;       // bytes
       const size_t scratch_bytes = off_b + (size_t)elems_b * 2;
       // Operand A may already lie in the scratch memory with rows and depth exchanged (an

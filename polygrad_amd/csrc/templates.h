@@ -60,6 +60,7 @@ struct MatmulEpilogue {
   std::string value_call_win;   // the same value with table lookups served from LDS windows (sets poly_tmax), or empty
   std::string ptr_call;    // expression of type out_type*: uses m, n, z
   std::string out_type;
+  bool out_16bit = false;  // the stored element is a 16-bit float, whatever the form of the store
   bool contiguous_n = false;
   int n_params = 0;
   double bytes = 0;    // algorithmic bytes of the whole kernel
