@@ -2412,6 +2412,46 @@ static bool match_ordered_sums_side_by_side(const Sched &sc, int a_item, const s
 // (its group's, if a group has taken it) must not come behind the launch of the later one.
 // A check of the matchers from scratch, on the host: they each reason about their own
 // members, this looks at every pair.
+// Does buffer `slot` only ever receive bf16 values cast to fp32?  (an intermediate with one
+// writer, whose one ungated store has such a cast as its value; what the writer leaves out
+// is either never read or filled with zeros)
+static bool slot_holds_bf16_values(const PolySchedule *s, const std::vector<KernelGraph> &graphs, int slot) {
+  if (slot < 0 || slot >= s->n_buf_slots || !s->buf_slots[slot].is_intermediate) return false;
+  int writer = -1;
+  for (int k = 0; k < s->n_items; k++) {
+    const PolyExecItem &it = s->items[k];
+    const KernelGraph &g = graphs[(size_t)k];
+    for (size_t q = 0; q < g.params.size() && (int)q < it.n_buf_slots; q++)
+      if (it.buf_slot_indices[q] == slot && g.params[q].written) {
+        if (writer >= 0 && writer != k) return false;
+        writer = k;
+      }
+  }
+  if (writer < 0) return false;
+  const KernelGraph &g = graphs[(size_t)writer];
+  if (g.stores.size() != 1 || g.stores[0].gate >= 0) return false;
+  const StoreInfo &st = g.stores[0];
+  const int p = g.param_slot(st.param);
+  if (p < 0 || p >= s->items[writer].n_buf_slots || s->items[writer].buf_slot_indices[p] != slot) return false;
+  const KNode &v = g.n(st.value);
+  return g.n(st.param).dt == DT_F32 && v.op == POLY_OP_CAST && v.dt == DT_F32 && v.src.size() == 1 && g.n(v.src[0]).dt == DT_BF16;
+}
+
+std::vector<int> matmul_param_kinds_of(const PolySchedule *s, const std::vector<KernelGraph> &graphs, int item, const std::vector<int> &narrow_slots) {
+  std::vector<int> kinds;
+  if (getenv("POLY_HIP_NO_EXACT16_BUFFERS")) return kinds;
+  const PolyExecItem &it = s->items[item];
+  const KernelGraph &g = graphs[(size_t)item];
+  kinds.assign((size_t)it.n_buf_slots, 0);
+  for (int p = 0; p < it.n_buf_slots && (size_t)p < g.params.size(); p++) {
+    if (g.params[(size_t)p].dt != DT_F32 || g.params[(size_t)p].written) continue;
+    const int sl = it.buf_slot_indices[p];
+    if (!slot_holds_bf16_values(s, graphs, sl)) continue;
+    kinds[(size_t)p] = std::find(narrow_slots.begin(), narrow_slots.end(), sl) != narrow_slots.end() ? 2 : 1;
+  }
+  return kinds;
+}
+
 std::vector<int> fused_groups_out_of_order(const PolySchedule *s, const std::vector<KernelGraph> &graphs, const std::vector<FusedGroup> &groups) {
   std::vector<int> step_of((size_t)s->n_items, 0), group_of((size_t)s->n_items, -1), pos((size_t)s->n_items, 0);
   for (int st = 0; st < s->n_items; st++) step_of[(size_t)s->exec_order[st]] = st;

@@ -24,4 +24,10 @@ void find_fused_groups(const PolySchedule *s, const std::vector<KernelGraph> &gr
 // groups itself, so that its result always passes.
 std::vector<int> fused_groups_out_of_order(const PolySchedule *s, const std::vector<KernelGraph> &graphs, const std::vector<FusedGroup> &groups);
 
+// What matmul_hint_param_kinds takes for the lowering of item `item`: 1 for every fp32
+// buffer parameter that is an intermediate of the plan with one writer, whose one store
+// puts a bf16 value cast to fp32 there (2 where `narrow_slots` names the buffer: its writer
+// has been made to store the bf16 values themselves).
+std::vector<int> matmul_param_kinds_of(const PolySchedule *s, const std::vector<KernelGraph> &graphs, int item, const std::vector<int> &narrow_slots);
+
 }  // namespace polyhip

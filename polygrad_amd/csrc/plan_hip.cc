@@ -361,8 +361,10 @@ PolyHipPlan *poly_hip_compile_schedule(PolyCtx *ctx, const PolySchedule *s) {
           if (!written) mask |= (uint64_t)1 << p;
         }
         matmul_hint_input_params(mask);
+        matmul_hint_param_kinds(matmul_param_kinds_of(s, graphs, k, {}));
         u.runner = runner_create(it.root, name.c_str(), 0);
         matmul_hint_input_params(0);
+        matmul_hint_param_kinds({});
       }
       // (a kernel may use fewer variables than the schedule lists for it: a buffer sized by
       // a variable that the kernel itself walks over its full allocation)

@@ -1282,6 +1282,7 @@ static bool try_slab_fission(const KernelGraph &g, const std::string &fn_name, c
     *out = parts.back();
     out->variants.clear();
     out->pres.clear();
+    out->narrow_loads = -1;      // (each slab passed render_kernel's check by itself)
     out->scratch_bytes = 256;
     out->strategy = "";
     out->bytes = 0;
@@ -1301,7 +1302,28 @@ static bool try_slab_fission(const KernelGraph &g, const std::string &fn_name, c
   return fis_reject(__LINE__);
 }
 
+static bool render_kernel_any(const KernelGraph &g, const std::string &fn_name, const RenderOptions &opt, RenderedKernel *out, std::string *err);
+
 bool render_kernel(const KernelGraph &g, const std::string &fn_name, const RenderOptions &opt,
+                   RenderedKernel *out, std::string *err) {
+  // loads from fp32 buffers that hold bf16 values at the time of the launch
+  // (matmul_hint_param_kinds, kind 2): the lowering has to read every one of them as such
+  int narrow_loads = 0;
+  for (int id = 0; id < (int)g.nodes.size(); id++) {
+    const KNode &k = g.n(id);
+    if (k.op != POLY_OP_LOAD) continue;
+    const KNode &ix = g.n(k.src[0]);
+    if (!ix.src.empty() && matmul_param_kind(g.param_slot(ix.src[0])) == 2) narrow_loads++;
+  }
+  if (!render_kernel_any(g, fn_name, opt, out, err)) return false;
+  if (narrow_loads > 0 && out->narrow_loads != -1 && out->narrow_loads != narrow_loads) {
+    if (err) *err = "a buffer of bf16 values would be read as fp32 values";
+    return false;
+  }
+  return true;
+}
+
+static bool render_kernel_any(const KernelGraph &g, const std::string &fn_name, const RenderOptions &opt,
                    RenderedKernel *out, std::string *err) {
   if (opt.allow_templates) {
     if (try_render_matmul(g, fn_name, opt, out)) return true;

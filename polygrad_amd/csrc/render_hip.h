@@ -106,6 +106,9 @@ struct RenderedKernel {
     int parts = 0;
   } a_planes;
   bool reads_planes_before = false;   // this kernel's operand A is the planes of RenderOptions::planes_before
+  // loads from fp32 buffers that hold bf16 values instead (matmul_hint_param_kinds, kind 2)
+  // that the kernel reads as such; -1: a launch of several kernels, each checked by itself
+  int narrow_loads = 0;
 };
 
 struct Scope;

@@ -31,6 +31,8 @@ const char *const kOperandSplitTemplate =
     ;
 
 thread_local uint64_t g_input_params = 0;
+// What the plan knows about the kernel's fp32 buffer parameters; see matmul_hint_param_kinds.
+thread_local std::vector<int> g_param_kinds;
 
 PolyOps reduce_op(const KNode &k) {
   return k.u->arg.kind == POLY_ARG_OPS ? k.u->arg.ops : (PolyOps)k.u->arg.i;
@@ -623,6 +625,10 @@ static bool render_matmul_f32(const MatmulMatch &mm, const MatmulEpilogue &ep, R
 }
 
 void matmul_hint_input_params(uint64_t mask) { g_input_params = mask; }
+void matmul_hint_param_kinds(const std::vector<int> &kinds) { g_param_kinds = kinds; }
+int matmul_param_kind(int param) {
+  return param >= 0 && (size_t)param < g_param_kinds.size() ? g_param_kinds[(size_t)param] : 0;
+}
 
 bool matmul_tuning_enabled() {
   const char *e = getenv("POLY_BEAM");
@@ -1351,14 +1357,21 @@ bool try_render_matmul_generic(const KernelGraph &g, const std::string &fn, cons
   // a first stage writes both operands as k-contiguous bf16 planes into scratch memory and
   // the 16-bit template multiplies them (K' = planes x K rounded up to its K tile).
   {
-    auto exact16 = [&](int node) {
-      const KNode &k = g.n(node);
-      return k.op == POLY_OP_CAST && k.dt == DT_F32 && g.n(k.src[0]).dt == DT_BF16;
+    // (a plain load from an fp32 buffer that only ever receives bf16 values, or holds them
+    // as bf16 in the first place: matmul_hint_param_kinds)
+    int kind[2] = {0, 0};
+    for (int side = 0; side < 2; side++) {
+      Operand o;
+      if (g.n(opnd[side]).op == POLY_OP_LOAD && g.n(opnd[side]).dt == DT_F32 && match_operand(g, opnd[side], &o)) kind[side] = matmul_param_kind(o.param);
+    }
+    auto exact16 = [&](int side) {
+      const KNode &k = g.n(opnd[side]);
+      return kind[side] != 0 || (k.op == POLY_OP_CAST && k.dt == DT_F32 && g.n(k.src[0]).dt == DT_BF16);
     };
     // (two pieces, hi + lo, leave an error below 2^-17 |x|: enough where the result is
     // stored as a 16-bit float, whose own rounding is 2^-9 or 2^-12 of it)
     const int pieces = ep.out_16bit && !getenv("POLY_HIP_SPLIT_THREE") ? 2 : 3;
-    const int parts[2] = {exact16(opnd[0]) ? 1 : pieces, exact16(opnd[1]) ? 1 : pieces};
+    const int parts[2] = {exact16(0) ? 1 : pieces, exact16(1) ? 1 : pieces};
     const int P = std::max(parts[0], parts[1]);
     const int64_t KP = (K + 63) / 64 * 64;
     const double elems_a = (double)Z * (double)M * parts[0] * (double)KP, elems_b = (double)Z * (double)N * parts[1] * (double)KP;
@@ -1388,8 +1401,12 @@ bool try_render_matmul_generic(const KernelGraph &g, const std::string &fn, cons
       InPlace in_place[2];
       for (int side = 0; side < 2 && !getenv("POLY_HIP_NO_IN_PLACE_OPERAND"); side++) {
         InPlace &ip = in_place[side];
+        // (a buffer that holds bf16 values where the schedule has fp32 ones is read as the
+        // 16-bit buffer it is, at the same element indices)
+        const bool narrow = kind[side] == 2;
         if (parts[side] != 1 || K % 64 != 0 || kr.size() > 2 || (side == 0 && shared)) continue;
-        if (!match_operand(g, opnd[side], &ip.op) || ip.op.dt != DT_BF16) continue;
+        if (!match_operand(g, opnd[side], &ip.op) || ip.op.dt != (narrow ? DT_F32 : DT_BF16)) continue;
+        if (!narrow && kind[side] != 0) continue;
         const Lin &l = g.lins[(size_t)ip.op.lin];
         if (kr.size() == 1) {
           if (!k_dependence(g, l, kr[0], K, &ip.ks) || ip.ks.kb < K) continue;
@@ -1445,6 +1462,7 @@ bool try_render_matmul_generic(const KernelGraph &g, const std::string &fn, cons
           if (!eval_lin(g, l, rv, &got) || got != want) ok = false;
         }
         ip.c0 = l.c0;
+        if (narrow) ip.op.dt = DT_BF16;
         ip.ok = ok;
       }
       RenderedKernel::Pre pre[2];
@@ -1518,12 +1536,12 @@ bool try_render_matmul_generic(const KernelGraph &g, const std::string &fn, cons
       MatmulEpilogue ep2 = ep;
       ep2.signature += ", __bf16* poly_scratch";
       ep2.scratch_type = "__bf16";
-      const size_t planes_bytes = in_place[1].ok ? std::max<size_t>(off_b, 256) : scratch_bytes;
+      const size_t planes_bytes = in_place[1].ok ? (in_place[0].ok ? (size_t)256 : std::max<size_t>(off_b, 256)) : scratch_bytes;
       ep2.scratch_used = planes_bytes;
       ep2.a_ptr = "((const __bf16*)poly_scratch)";
       ep2.b_ptr = strf("((const __bf16*)((const char*)poly_scratch + %zuull))", off_b);
-      if (in_place[0].ok) ep2.a_ptr = strf("data%d", in_place[0].op.param);
-      if (in_place[1].ok) ep2.b_ptr = strf("data%d", in_place[1].op.param);
+      if (in_place[0].ok) ep2.a_ptr = strf(kind[0] == 2 ? "((const __bf16*)data%d)" : "data%d", in_place[0].op.param);
+      if (in_place[1].ok) ep2.b_ptr = strf(kind[1] == 2 ? "((const __bf16*)data%d)" : "data%d", in_place[1].op.param);
       RenderedKernel main;
       if (render_matmul(m2, ep2, &main)) {
         *out = main;
@@ -1535,7 +1553,8 @@ bool try_render_matmul_generic(const KernelGraph &g, const std::string &fn, cons
         out->strategy = strf("operands as expressions, written as bf16 planes first (%d + %d planes of K=%lld, %.0f MB%s): ", parts[0], parts[1],
                              (long long)KP, (double)planes_bytes / 1e6,
                              shared ? "; A is what the kernel before left as its A, rows and depth exchanged, and is not written again"
-                             : in_place[0].ok ? "; A read in place" : in_place[1].ok ? "; B read in place" : "") + out->strategy;
+                             : in_place[0].ok && in_place[1].ok ? "; both read in place" : in_place[0].ok ? "; A read in place" : in_place[1].ok ? "; B read in place" : "") + out->strategy;
+        out->narrow_loads = (in_place[0].ok && kind[0] == 2 ? 1 : 0) + (in_place[1].ok && kind[1] == 2 ? 1 : 0);
         out->tables = ep.tables;
         if (!ep.tables.empty()) out->strategy += strf(", %zu parts of the epilogue as 16-bit lookup tables", ep.tables.size());
         out->reads_planes_before = shared;

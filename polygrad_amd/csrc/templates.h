@@ -80,6 +80,15 @@ struct MatmulEpilogue {
 // Set by the plan compiler around the lowering of one scheduled kernel: bit p says that
 // buffer parameter p is an input of the plan that none of its kernels writes.
 void matmul_hint_input_params(uint64_t mask);
+// Also set around a lowering: what the plan knows of the kernel's buffer parameters that
+// are fp32 in the schedule.  kinds[p] = 1: every value the buffer receives is a bf16 value
+// cast to fp32 (its one writer stores such a cast), so that a product may take it as the
+// one bf16 plane it is.  kinds[p] = 2: the writer was made to store those bf16 values
+// themselves, at the same element indices (the buffer read as a 16-bit one); only a product
+// that takes the buffer as a plain operand can read that, and render_kernel refuses every
+// other use.
+void matmul_hint_param_kinds(const std::vector<int> &kinds);
+int matmul_param_kind(int param);
 // Is element (m, n + 1) of the kernel's output stored right after (m, n), for every n
 // that is not the last of an aligned group of 8?  (store index affine with coefficient 1
 // on the innermost digit of n, digits not crossed inside a group)
