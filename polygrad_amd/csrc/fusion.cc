@@ -688,6 +688,11 @@ static void collect_ref_loads(const Sched &sc, const Member &m, std::vector<std:
   }
 }
 
+// The buffer (slot) whose values the chain being built is to store as the bf16 values they
+// are casts of, at the same element indices of the buffer read as a 16-bit one; -1: none.
+// (set by find_fused_groups once it knows that the one reader of the buffer takes that)
+static thread_local int g_narrow_store_slot = -1;
+
 static bool match_row_chain_impl(const Sched &sc, int a_item, const std::vector<char> &taken, FusedGroup *out, bool allow_rows) {
   const PolySchedule *s = sc.s;
   const KernelGraph &gA = sc.graphs[(size_t)a_item];
@@ -910,6 +915,7 @@ static bool match_row_chain_impl(const Sched &sc, int a_item, const std::vector<
   struct RowCache { std::string key, type; int nit; };
   std::vector<RowCache> cache;
   int n_cached_uses = 0, n_exported = 0;
+  bool narrow_stored = false;
   int row_V = 0, row_nit = 0;       // vector width and step count of the rows kept between phases
   std::string row_decls;             // their declarations in the kernel body
   for (size_t pi = 0; pi < phases.size(); pi++) {
@@ -1075,15 +1081,26 @@ static bool match_row_chain_impl(const Sched &sc, int a_item, const std::vector<
       const StoreInfo &st = g.stores[0];
       const int li = g.n(g.n(st.index).src[1]).lin;
       const int p = g.param_slot(st.param);
-      std::string v = em.emit(st.value, &U);
-      const char *odt = dt_cname(g.n(st.param).dt);
+      // (a buffer whose reader takes bf16 values: what the cast to fp32 is applied to goes
+      // there, into the buffer read as a 16-bit one)
+      const bool narrow = !ph.keeps_row && g_narrow_store_slot >= 0 && sc.slot(ph.m.item, p) == g_narrow_store_slot;
+      if (narrow) {
+        const KNode &cv = g.n(st.value);
+        if (pi + 1 != phases.size() || cv.op != POLY_OP_CAST || cv.dt != DT_F32 || cv.src.size() != 1 || g.n(cv.src[0]).dt != DT_BF16 ||
+            g.n(st.param).dt != DT_F32)
+          FA_REJECT();
+        narrow_stored = true;
+      }
+      std::string v = em.emit(narrow ? g.n(st.value).src[0] : st.value, &U);
+      const char *odt = narrow ? "__bf16" : dt_cname(g.n(st.param).dt);
+      const std::string dst = narrow ? strf("((__bf16*)data%d)", p) : strf("data%d", p);
       if (ph.keeps_row) {
         U.code += strf("      %s = %s;\n", names[pi].c_str(), v.c_str());
       } else if (V > 1) {
         U.code += strf("      out.v[u] = %s;\n", v.c_str());
       } else {
         std::string idx = em.emit(g.n(st.index).src[1], &U);
-        U.code += strf("      data%d[%s] = %s;\n", p, idx.c_str(), v.c_str());
+        U.code += strf("      %s[%s] = %s;\n", dst.c_str(), idx.c_str(), v.c_str());
       }
       std::string addr;
       if (V > 1) { em.bind_range(own_f, fv + "_0"); addr = em.emit_lin(g.lins[(size_t)li], &L); em.bind_range(own_f, fv); }
@@ -1094,12 +1111,12 @@ static bool match_row_chain_impl(const Sched &sc, int a_item, const std::vector<
       if (V > 1 && !ph.keeps_row) loop += strf("    poly_vec<%s,%d> out;\n", odt, V);
       loop += strf("#pragma unroll\n    for (int u = 0; u < %d; u++) {\n      const int %s = %s_0 + u;\n", V, fv.c_str(), fv.c_str());
       loop += U.code + "    }\n";
-      if (V > 1 && !ph.keeps_row) loop += strf("    poly_vstore<%s,%d>(data%d + %s, out);\n", odt, V, p, addr.c_str());
+      if (V > 1 && !ph.keeps_row) loop += strf("    poly_vstore<%s,%d>(%s + %s, out);\n", odt, V, dst.c_str(), addr.c_str());
       loop += loop_close;
       if (ragged)
-        loop += ragged_tail(st.value, [&](Scope *tl, const std::string &v2) {
+        loop += ragged_tail(narrow ? g.n(st.value).src[0] : st.value, [&](Scope *tl, const std::string &v2) {
           const std::string idx = em.emit(g.n(st.index).src[1], tl);
-          return strf("    data%d[%s] = %s;\n", p, idx.c_str(), v2.c_str());
+          return strf("    %s[%s] = %s;\n", dst.c_str(), idx.c_str(), v2.c_str());
         });
     }
     if (em.failed() || em.uses_threefry) FA_REJECT();
@@ -1163,6 +1180,13 @@ static bool match_row_chain_impl(const Sched &sc, int a_item, const std::vector<
   if (n_cached_uses) rk.strategy += strf(", %d row loads kept in registers", n_cached_uses);
   if (row_V) rk.strategy += ", intermediate rows kept in registers";
   if (n_exported) rk.strategy += strf(", %d row values stored for later kernels", n_exported);
+  if (g_narrow_store_slot >= 0 && !narrow_stored) FA_REJECT();
+  if (narrow_stored) rk.strategy += ", result stored as the bf16 values that its fp32 values are casts of";
+  out->row_chain_from = a_item;
+  {
+    const KernelGraph &gl = sc.graphs[(size_t)phases.back().m.item];
+    out->row_chain_stores = phases.back().is_map ? sc.slot(phases.back().m.item, gl.param_slot(gl.stores[0].param)) : -1;
+  }
   rk.n_params = (int)arg_slots.size();
   rk.bytes = bytes;
   return true;
@@ -2542,6 +2566,40 @@ void find_fused_groups(const PolySchedule *s, const std::vector<KernelGraph> &gr
     FusedGroup fg;
     if (!match_side_by_side(sc, k, taken, &fg)) continue;
     accept(fg, taken);
+  }
+  // A row chain whose result is an fp32 buffer of bf16 values (the derivative of the scores
+  // of attention: a cast of a bf16 product), read by one product that can take it as a
+  // 16-bit operand where it lies: the chain stores the bf16 values, the product reads them,
+  // and nothing writes or reads the values as fp32 (half the bytes written, no planes).
+  for (size_t gi = 0, n0 = out->size(); gi < n0 && !getenv("POLY_HIP_NO_NARROW_STORE"); gi++) {
+    const int slot = (*out)[gi].row_chain_stores;
+    if (slot < 0 || !slot_holds_bf16_values(s, graphs, slot)) continue;
+    if (std::find((*out)[gi].internal_slots.begin(), (*out)[gi].internal_slots.end(), slot) != (*out)[gi].internal_slots.end()) continue;
+    const std::vector<int> &rd = sc.readers[(size_t)slot];
+    if (rd.size() != 1 || sc.writers[(size_t)slot].size() != 1 || taken[(size_t)rd[0]]) continue;
+    const int reader = rd[0];
+    if (sc.step_of[(size_t)reader] <= sc.step_of[(size_t)(*out)[gi].launch_item]) continue;
+    FusedGroup rg;
+    matmul_hint_param_kinds(matmul_param_kinds_of(s, graphs, reader, {slot}));
+    std::string err;
+    const bool reads = render_kernel(graphs[(size_t)reader], "poly_k", RenderOptions(), &rg.rk, &err) && rg.rk.klass == KernelClass::MATMUL_MFMA &&
+                       rg.rk.guards.empty() && rg.rk.n_vars == 0 && rg.rk.n_params == s->items[reader].n_buf_slots;
+    matmul_hint_param_kinds({});
+    if (!reads) continue;
+    // the chain once more, with the other store
+    std::vector<char> free_again = taken;
+    for (int it : (*out)[gi].items) free_again[(size_t)it] = 0;
+    FusedGroup chain;
+    g_narrow_store_slot = slot;
+    const bool stores = match_row_chain(sc, (*out)[gi].row_chain_from, free_again, &chain) && chain.items == (*out)[gi].items &&
+                        chain.launch_item == (*out)[gi].launch_item;
+    g_narrow_store_slot = -1;
+    if (!stores) continue;
+    (*out)[gi] = std::move(chain);
+    rg.items = {reader};
+    rg.launch_item = reader;
+    rg.arg_slots.assign(s->items[reader].buf_slot_indices, s->items[reader].buf_slot_indices + s->items[reader].n_buf_slots);
+    accept(rg, taken);
   }
   // every pair of items that share a buffer keeps its order; a group that breaks one is
   // dropped and its kernels launch one by one at their own places

@@ -14,6 +14,8 @@ struct FusedGroup {
   std::vector<int> internal_slots;  // buffers that are never materialised
   std::vector<int> arg_slots;       // slot of each kernel argument, in order
   RenderedKernel rk;
+  // a row chain: the item it was grown from and the buffer its last kernel stores (-1: none)
+  int row_chain_from = -1, row_chain_stores = -1;
 };
 
 // Finds the fusable groups of a schedule.  graphs[k] is the analysed kernel of item k.

@@ -214,14 +214,16 @@ def test_ordered_column_sums_of_a_step_run_side_by_side():
 
 
 @pytest.mark.parametrize("T", [128, 1024])
-def test_slabs_of_the_qkv_derivative_share_operand_planes(T):
-    """Two slabs of the derivative of the q | k | v split multiply by the same fp32 tensor
-    (the softmax derivative dS: dq = dS K, dk = dS^T Q).  At full size both products run on
-    the bf16 MFMA over three bf16 planes of dS; the second slab reads the planes the first
-    one wrote (as rows along the depth) instead of writing its own.  Here at a size the
-    reference CPU backend finishes quickly (one short sequence, and one of the full 1024
-    positions), with the size threshold of that path lowered: against the reference, and
-    bit for bit against the same step with every slab writing its own planes."""
+def test_slabs_of_the_qkv_derivative_read_the_score_derivative_as_bf16(T):
+    """Two slabs of the derivative of the q | k | v split multiply by the same tensor (the
+    derivative of the scores dS: dq = dS K, dk = dS^T Q), an fp32 buffer in the schedule
+    whose values are casts of bf16 products.  The row chain that makes dS stores the bf16
+    values themselves and both products read them where they lie, on the bf16 MFMA.  Here
+    at a size the reference CPU backend finishes quickly (one short sequence, and one of the
+    full 1024 positions), with the size threshold of that path lowered: against the
+    reference, and bit for bit against the same step with dS stored as fp32 and written
+    as one bf16 plane first (which the second slab reads as the first one left it, rows
+    along the depth, or writes again itself)."""
     import os
     B, D, H, V, lr = 1, 128, 2, 97, 3e-4
     os.environ["POLY_HIP_BF16_SPLIT_MIN"] = "1048576"
@@ -243,15 +245,33 @@ def test_slabs_of_the_qkv_derivative_share_operand_planes(T):
                 m_ref, m_got = want[bufs[name + ".m"]], got[bufs[name + ".m"]]
                 assert float(np.abs(m_got - m_ref).mean()) <= 2e-3 * float(np.abs(m_ref).max()), name
         slabs = [k["desc"] for k in info if "3 slabs of one output range" in k["desc"]]
-        assert len(slabs) == 1 and "rows and depth exchanged" in slabs[0] and slabs[0].count("bf16 planes first") == 3, slabs
-        os.environ["POLY_HIP_NO_SHARED_PLANES"] = "1"
-        try:
-            own, info1 = run_hip(c, sink, arrays)
-        finally:
-            del os.environ["POLY_HIP_NO_SHARED_PLANES"]
-        assert not any("rows and depth exchanged" in k["desc"] for k in info1)
+        assert len(slabs) == 1 and slabs[0].count("read in place") == 3 and "rows and depth exchanged" not in slabs[0], slabs
+        assert slabs[0].count("(1 + 1 planes") == 3, slabs
+        assert sum("result stored as the bf16 values" in k["desc"] for k in info) == 1
+
+        def again(*switches):
+            for e in switches:
+                os.environ[e] = "1"
+            try:
+                return run_hip(c, sink, arrays)
+            finally:
+                for e in switches:
+                    del os.environ[e]
+
+        wide, info1 = again("POLY_HIP_NO_NARROW_STORE")
+        assert sum("rows and depth exchanged" in k["desc"] for k in info1) == 1
+        assert not any("result stored as the bf16 values" in k["desc"] for k in info1)
+        own, info2 = again("POLY_HIP_NO_NARROW_STORE", "POLY_HIP_NO_SHARED_PLANES")
+        assert not any("rows and depth exchanged" in k["desc"] for k in info2)
+        # every value of dS in three bf16 pieces, of which two are zero
+        three, info3 = again("POLY_HIP_NO_EXACT16_BUFFERS", "POLY_HIP_SPLIT_THREE")
+        assert any("(3 + 1 planes" in k["desc"] for k in info3)
         for name, t in bufs.items():
+            assert got[t].tobytes() == wide[t].tobytes(), name
             assert got[t].tobytes() == own[t].tobytes(), name
+        # (the pieces that are zero add nothing, but a product three times as deep may be dealt
+        # to workgroups another way and add its terms in another order)
+        assert_close(three[bufs["loss"]], got[bufs["loss"]], rtol=1e-5, what="loss")
         c.close()
     finally:
         del os.environ["POLY_HIP_BF16_SPLIT_MIN"]
