@@ -1917,6 +1917,7 @@ static bool match_attention(const Sched &sc, int s_item, const std::vector<char>
     rk.pre_reads.assign(1, mask_arg);
   }
   rk.source = std::string(hip_prelude()) + cfg + kAttentionTemplate;
+  const std::string fa_cfg = cfg;
   rk.entry = "poly_k";
   rk.launch.grid[0] = (unsigned)((mS.M / 128) * mS.Z);
   rk.launch.block[0] = 256;
@@ -1925,6 +1926,14 @@ static bool match_attention(const Sched &sc, int s_item, const std::vector<char>
                      tin == DT_BF16 ? "bf16" : "f16", (long long)mS.Z, (long long)mS.M, (long long)mS.N,
                      cfg.find("#define POLY_FA_ONLINE 1") != std::string::npos ? "one pass, online softmax" : "two passes over keys, exact roundings");
   if (mask_table) rk.strategy += ", mask tiles classified by a first kernel";
+  if (matmul_tuning_enabled()) {
+    // the register budget (waves per SIMD) changes the schedule of the instructions, not
+    // one value: candidates of the search that POLY_BEAM switches on
+    rk.variants.push_back({"default", rk.source, rk.strategy, rk.launch});
+    for (int occ : {2, 4})
+      rk.variants.push_back({strf("attn_occ%d", occ), std::string(hip_prelude()) + strf("#define POLY_FA_OCC %d\n", occ) + fa_cfg + kAttentionTemplate,
+                             rk.strategy + strf(", %d waves per SIMD", occ), rk.launch});
+  }
   rk.n_params = (int)arg_slots.size();
   rk.n_vars = 0;
   rk.flops = 2.0 * (double)mS.Z * (double)mS.M * (double)mS.N * (double)(mS.K + mV.N);
@@ -2113,20 +2122,29 @@ static bool match_pointwise_group(const Sched &sc, int a_item, const std::vector
     // (a buffer updated in place moves twice: in and out)
     bytes += (double)s->buf_slots[sl].nbytes * ((read_from_memory.count(sl) ? 1 : 0) + (written.count(sl) ? 1 : 0));
   }
-  std::string src = std::string(hip_prelude()) + code;
-  src += strf("extern \"C\" __global__ void __launch_bounds__(256) poly_k(%s) {\n", sig.c_str());
-  src += strf("  const long long pos_ll = ((long long)blockIdx.x * 256 + threadIdx.x) * %d;\n  if (pos_ll >= %lldll) return;\n  const int pos = (int)pos_ll;\n", V, (long long)E);
-  for (size_t mi = 0; mi < members.size(); mi++)
-    src += strf("  %s o%zu[%d];\n", dt_cname(sc.graphs[(size_t)members[mi].item].n(sc.graphs[(size_t)members[mi].item].stores[0].value).dt), mi, V);
-  src += strf("#pragma unroll\n  for (int u = 0; u < %d; u++) {\n", V) + body + "  }\n";
-  for (size_t mi = 0; mi < members.size(); mi++) {
-    const Pw &pw = members[mi];
-    if (internal.count(pw.out_slot)) continue;
-    const char *tn = dt_cname(slot_dt[pw.out_slot]);
-    src += strf("  { poly_vec<%s, %d> st; for (int u = 0; u < %d; u++) st.v[u] = o%zu[u]; poly_vstore<%s, %d>(fa%d + pos, st); }\n", tn, V, V, mi, tn, V,
-                arg_of(pw.out_slot));
-  }
-  src += "}\n";
+  // the kernel for V positions per thread (the members themselves are per position)
+  const auto kernel_for = [&](int V) {
+    std::string src = std::string(hip_prelude()) + code;
+    src += strf("extern \"C\" __global__ void __launch_bounds__(256) poly_k(%s) {\n", sig.c_str());
+    src += strf("  const long long pos_ll = ((long long)blockIdx.x * 256 + threadIdx.x) * %d;\n  if (pos_ll >= %lldll) return;\n  const int pos = (int)pos_ll;\n", V, (long long)E);
+    for (size_t mi = 0; mi < members.size(); mi++)
+      src += strf("  %s o%zu[%d];\n", dt_cname(sc.graphs[(size_t)members[mi].item].n(sc.graphs[(size_t)members[mi].item].stores[0].value).dt), mi, V);
+    src += strf("#pragma unroll\n  for (int u = 0; u < %d; u++) {\n", V) + body + "  }\n";
+    for (size_t mi = 0; mi < members.size(); mi++) {
+      const Pw &pw = members[mi];
+      if (internal.count(pw.out_slot)) continue;
+      const char *tn = dt_cname(slot_dt[pw.out_slot]);
+      src += strf("  { poly_vec<%s, %d> st; for (int u = 0; u < %d; u++) st.v[u] = o%zu[u]; poly_vstore<%s, %d>(fa%d + pos, st); }\n", tn, V, V, mi, tn, V,
+                  arg_of(pw.out_slot));
+    }
+    src += "}\n";
+    return src;
+  };
+  const auto strategy_for = [&](int V) {
+    return strf("%zu pointwise kernels over the same %lld positions as one, vec%d, %zu buffers never written out", members.size(), (long long)E, V,
+                internal.size());
+  };
+  const std::string src = kernel_for(V);
   out->items.clear();
   for (const Pw &m : members) out->items.push_back(m.item);
   out->launch_item = members.back().item;
@@ -2139,12 +2157,25 @@ static bool match_pointwise_group(const Sched &sc, int a_item, const std::vector
   rk.launch.grid[0] = (unsigned)((E / V + 255) / 256);
   rk.launch.block[0] = 256;
   rk.klass = KernelClass::ELEMENTWISE;
-  rk.strategy = strf("%zu pointwise kernels over the same %lld positions as one, vec%d, %zu buffers never written out", members.size(), (long long)E, V,
-                     internal.size());
+  rk.strategy = strategy_for(V);
   rk.n_params = (int)arg_slots.size();
   rk.n_vars = 0;
   rk.bytes = bytes;
   rk.flops = 0;
+  if (matmul_tuning_enabled()) {
+    // other widths of a thread's accesses: candidates of the search that POLY_BEAM switches on
+    rk.variants.push_back({"default", rk.source, rk.strategy, rk.launch});
+    for (int bytes_per : {16, 8, 4}) {
+      const int v = std::max(1, bytes_per / maxsz);
+      bool seen = v == V || E % v != 0;
+      for (const RenderedKernel::Variant &o : rk.variants) if (o.label == strf("pw_vec%d", v)) seen = true;
+      if (seen) continue;
+      LaunchSpec ls = rk.launch;
+      ls.grid[0] = (unsigned)((E / v + 255) / 256);
+      rk.variants.push_back({strf("pw_vec%d", v), kernel_for(v), strategy_for(v), ls});
+    }
+    if (rk.variants.size() < 2) rk.variants.clear();
+  }
   return true;
 }
 

@@ -128,6 +128,9 @@ typedef unsigned int fa_u32x2 __attribute__((ext_vector_type(2)));
 typedef fa_u32x4 fa_u32x4_u __attribute__((aligned(2)));
 typedef fa_u32x2 fa_u32x2_u __attribute__((aligned(2)));
 
+#ifndef POLY_FA_OCC
+#define POLY_FA_OCC 3    // waves per SIMD the register budget is set for (a tuning candidate: no effect on the values)
+#endif
 #define FA_BM 128        // queries per workgroup: 4 waves x 32
 #define FA_BN 64         // keys per step
 #define FA_D 64          // head features
@@ -187,7 +190,7 @@ extern "C" __global__ void __launch_bounds__(512) poly_k(POLY_SIGNATURE) {
 #else
 // Three workgroups per CU (three waves per SIMD): the arithmetic on the scores is VALU work,
 // and it is the other resident waves that hide its latencies.
-extern "C" __global__ void __launch_bounds__(FA_THREADS) __attribute__((amdgpu_waves_per_eu(3, 3))) poly_k(POLY_SIGNATURE) {
+extern "C" __global__ void __launch_bounds__(FA_THREADS) __attribute__((amdgpu_waves_per_eu(POLY_FA_OCC, POLY_FA_OCC))) poly_k(POLY_SIGNATURE) {
   __shared__ __attribute__((aligned(16))) POLY_TIN lds_k[2][FA_BN * FA_D];   // [key][feature]
   __shared__ __attribute__((aligned(16))) POLY_TIN lds_v[2][FA_D * FA_BN];   // [feature][key]
   __shared__ __attribute__((aligned(16))) POLY_TIN lds_q[FA_BM * FA_D];      // [query][feature]

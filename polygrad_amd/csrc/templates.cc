@@ -551,6 +551,28 @@ static void f32_tile(int64_t M, int64_t N, int64_t Z, int *bm, int *bn, int *wvm
   *bm = BM; *bn = BN; *wvm = WVM; *wvn = WVN;
 }
 
+// The other tile shapes of the fp32 template as tuning candidates (same sums in the same
+// order: a tile's shape does not change the order of the terms of an output).  `build`
+// renders one shape; the default shape comes first, as the kernel itself.
+struct F32Shape { int bm, bn, wvm, wvn; };
+static void f32_variants(int64_t M, int64_t N, const F32Shape &chosen, const std::function<void(const F32Shape &, RenderedKernel *)> &build,
+                         RenderedKernel *out) {
+  if (!matmul_tuning_enabled()) return;
+  static const F32Shape shapes[] = {{128, 128, 2, 2}, {128, 128, 4, 2}, {64, 64, 2, 2}, {128, 64, 2, 2}, {64, 128, 2, 2}, {256, 128, 4, 2}, {128, 256, 2, 4},
+                                    {32, 64, 1, 2}, {256, 32, 4, 1}, {128, 64, 4, 1}, {32, 256, 1, 4}, {64, 128, 1, 4}};
+  out->variants.clear();
+  out->variants.push_back({"default", out->source, out->strategy, out->launch});
+  for (const F32Shape &sh : shapes) {
+    if (sh.bm == chosen.bm && sh.bn == chosen.bn && sh.wvm == chosen.wvm && sh.wvn == chosen.wvn) continue;
+    if ((sh.bm > 64 && M <= sh.bm / 2) || (sh.bn > 64 && N <= sh.bn / 2)) continue;       // (mostly padding)
+    RenderedKernel v;
+    build(sh, &v);
+    if (v.source.empty()) continue;
+    out->variants.push_back({strf("f32_%dx%dw%dx%d", sh.bm, sh.bn, sh.wvm, sh.wvn), v.source, v.strategy, v.launch});
+  }
+  if (out->variants.size() < 2) out->variants.clear();
+}
+
 // fp32 operands: kernels/matmul_f32_mfma.hip (v_mfma_f32_32x32x2_f32, exact fp32 products).
 static bool render_matmul_f32(const MatmulMatch &mm, const MatmulEpilogue &ep, RenderedKernel *out) {
   const int64_t K = mm.K, M = mm.M, N = mm.N, Z = mm.Z;
@@ -575,11 +597,9 @@ static bool render_matmul_f32(const MatmulMatch &mm, const MatmulEpilogue &ep, R
     if (s128 > 1 && t128 * s128 >= 128) { BM = BN = 128; WVM = WVN = 2; S = s128; }
     else if (s64 > 1) { BM = BN = 64; WVM = WVN = 2; S = s64; }
   }
-  const int64_t tiles = ((M + BM - 1) / BM) * ((N + BN - 1) / BN);
-  if (tiles > 2147483647LL / 2) return reject(__LINE__);
-  std::string cfg;
+  if (((M + BM - 1) / BM) * ((N + BN - 1) / BN) > 2147483647LL / 2) return reject(__LINE__);
+  std::string cfg;     // (all but the shape of the tile)
   cfg += strf("#define POLY_M %lld\n#define POLY_N %lld\n#define POLY_K %lld\n#define POLY_Z %lld\n", (long long)M, (long long)N, (long long)K, (long long)Z);
-  cfg += strf("#define POLY_BM %d\n#define POLY_BN %d\n#define POLY_WAVES_M %d\n#define POLY_WAVES_N %d\n#define POLY_GROUP_M 8\n", BM, BN, WVM, WVN);
   cfg += strf("#define POLY_A_KC %d\n#define POLY_B_KC %d\n", a_kc ? 1 : 0, b_kc ? 1 : 0);
   cfg += strf("#define POLY_A_PTR %s\n#define POLY_B_PTR %s\n", ep.a_ptr.c_str(), ep.b_ptr.c_str());
   cfg += offset_fn("poly_a_row", mm.md, true, 0);
@@ -597,25 +617,32 @@ static bool render_matmul_f32(const MatmulMatch &mm, const MatmulEpilogue &ep, R
   cfg += strf("#define POLY_KSPLIT %d\n#define POLY_PARTIALS poly_scratch\n", S);
   cfg += ep.code;
   cfg += strf("#define POLY_EPILOGUE(acc, m, n, z) %s\n", ep.call.c_str());
-  *out = RenderedKernel();
-  out->source = std::string(hip_prelude()) + cfg + kMatmulF32Template;
-  out->entry = "poly_k";
-  out->launch.grid[0] = (unsigned)tiles;
-  out->launch.grid[1] = (unsigned)(Z * S);
-  out->launch.block[0] = (unsigned)(64 * WVM * WVN);
-  out->klass = KernelClass::MATMUL_MFMA;
-  out->strategy = strf("mfma 32x32x2 f32 M=%lld N=%lld K=%lld Z=%lld tile %dx%dx16 A:%s B:%s", (long long)M, (long long)N, (long long)K,
-                       (long long)Z, BM, BN, a_kc ? "k-major" : "m-major", b_kc ? "k-major" : "n-major");
-  out->n_params = ep.n_params;
-  out->n_vars = 0;
-  out->flops = 2.0 * (double)M * (double)N * (double)K * (double)Z;
-  out->bytes = ep.bytes;
+  const auto build = [&](const F32Shape &sh, RenderedKernel *rk) {
+    const int64_t tiles = ((M + sh.bm - 1) / sh.bm) * ((N + sh.bn - 1) / sh.bn);
+    *rk = RenderedKernel();
+    rk->source = std::string(hip_prelude()) +
+                 strf("#define POLY_BM %d\n#define POLY_BN %d\n#define POLY_WAVES_M %d\n#define POLY_WAVES_N %d\n#define POLY_GROUP_M 8\n", sh.bm, sh.bn, sh.wvm, sh.wvn) +
+                 cfg + kMatmulF32Template;
+    rk->entry = "poly_k";
+    rk->launch.grid[0] = (unsigned)tiles;
+    rk->launch.grid[1] = (unsigned)(Z * S);
+    rk->launch.block[0] = (unsigned)(64 * sh.wvm * sh.wvn);
+    rk->klass = KernelClass::MATMUL_MFMA;
+    rk->strategy = strf("mfma 32x32x2 f32 M=%lld N=%lld K=%lld Z=%lld tile %dx%dx16 A:%s B:%s", (long long)M, (long long)N, (long long)K,
+                        (long long)Z, sh.bm, sh.bn, a_kc ? "k-major" : "m-major", b_kc ? "k-major" : "n-major");
+    rk->n_params = ep.n_params;
+    rk->n_vars = 0;
+    rk->flops = 2.0 * (double)M * (double)N * (double)K * (double)Z;
+    rk->bytes = ep.bytes;
+  };
+  build(F32Shape{BM, BN, WVM, WVN}, out);
+  if (S == 1) f32_variants(M, N, F32Shape{BM, BN, WVM, WVN}, build, out);
   if (S > 1) {
     // the template becomes the first stage; the kernel proper adds the partial results up
     RenderedKernel::Pre pre{out->source, out->entry, out->launch};
     out->pres.push_back(pre);
     out->scratch_bytes = (size_t)S * (size_t)Z * (size_t)M * (size_t)N * sizeof(float);
-    out->source = std::string(hip_prelude()) + cfg + kSplitKCombine;
+    out->source = std::string(hip_prelude()) + strf("#define POLY_BM %d\n#define POLY_BN %d\n", BM, BN) + cfg + kSplitKCombine;
     out->launch = LaunchSpec();
     out->launch.grid[0] = (unsigned)(((double)Z * M * N + 255) / 256);
     out->launch.block[0] = 256;
@@ -1568,12 +1595,10 @@ bool try_render_matmul_generic(const KernelGraph &g, const std::string &fn, cons
 
   int BM, BN, WVM, WVN;
   f32_tile(M, N, Z, &BM, &BN, &WVM, &WVN);
-  const int64_t tiles = ((M + BM - 1) / BM) * ((N + BN - 1) / BN);
-  if (tiles > 2147483647LL / 2) return reject(__LINE__);
+  if (((M + BM - 1) / BM) * ((N + BN - 1) / BN) > 2147483647LL / 2) return reject(__LINE__);
   const int depth = n_loads[0] + n_loads[1] <= 2 ? 4 : n_loads[0] + n_loads[1] <= 4 ? 2 : 1;
-  std::string cfg;
+  std::string cfg;     // (all but the shape of the tile)
   cfg += strf("#define POLY_M %lld\n#define POLY_N %lld\n#define POLY_K %lld\n#define POLY_Z %lld\n", (long long)M, (long long)N, (long long)K, (long long)Z);
-  cfg += strf("#define POLY_BM %d\n#define POLY_BN %d\n#define POLY_WAVES_M %d\n#define POLY_WAVES_N %d\n#define POLY_GROUP_M 8\n", BM, BN, WVM, WVN);
   cfg += strf("#define POLY_GEN 1\n#define POLY_PF_DEPTH %d\n#define POLY_A_KC %d\n#define POLY_B_KC %d\n", depth, walk_k[0] ? 1 : 0, walk_k[1] ? 1 : 0);
   cfg += strf("#define POLY_A_NLOADS %d\n#define POLY_B_NLOADS %d\n", std::max(1, n_loads[0]), std::max(1, n_loads[1]));
   cfg += strf("#define POLY_SIGNATURE %s\n", ep.signature.c_str());
@@ -1583,22 +1608,28 @@ bool try_render_matmul_generic(const KernelGraph &g, const std::string &fn, cons
   cfg += strf("#define POLY_B_LOAD(n, k, z, raw) poly_b_load(n, k, z, raw, %s)\n#define POLY_B_MATH(n, k, z, raw) poly_b_math(n, k, z, raw, %s)\n",
               params_call.c_str(), params_call.c_str());
   cfg += strf("#define POLY_EPILOGUE(acc, m, n, z) %s\n", ep.call.c_str());
-  *out = RenderedKernel();
-  out->source = std::string(hip_prelude()) + cfg + kMatmulF32Template;
-  out->entry = "poly_k";
-  out->launch.grid[0] = (unsigned)tiles;
-  out->launch.grid[1] = (unsigned)Z;
-  out->launch.block[0] = (unsigned)(64 * WVM * WVN);
-  out->klass = KernelClass::MATMUL_MFMA;
-  out->strategy = strf("mfma 32x32x2 f32, operands as expressions (%d + %d loads per element pair, %d tiles ahead) M=%lld N=%lld K=%lld Z=%lld tile %dx%dx16 A:%s B:%s",
-                       n_loads[0], n_loads[1], depth, (long long)M, (long long)N, (long long)K, (long long)Z, BM, BN,
-                       walk_k[0] ? "k-major" : "m-major", walk_k[1] ? "k-major" : "n-major");
-  out->n_params = ep.n_params;
-  out->n_vars = 0;
-  out->flops = 2.0 * (double)M * (double)N * (double)K * (double)Z;
-  out->bytes = ep.bytes;
-  out->tables = ep.tables;
-  if (!ep.tables.empty()) out->strategy += strf(", %zu parts of the epilogue as 16-bit lookup tables", ep.tables.size());
+  const auto build = [&](const F32Shape &sh, RenderedKernel *rk) {
+    *rk = RenderedKernel();
+    rk->source = std::string(hip_prelude()) +
+                 strf("#define POLY_BM %d\n#define POLY_BN %d\n#define POLY_WAVES_M %d\n#define POLY_WAVES_N %d\n#define POLY_GROUP_M 8\n", sh.bm, sh.bn, sh.wvm, sh.wvn) +
+                 cfg + kMatmulF32Template;
+    rk->entry = "poly_k";
+    rk->launch.grid[0] = (unsigned)(((M + sh.bm - 1) / sh.bm) * ((N + sh.bn - 1) / sh.bn));
+    rk->launch.grid[1] = (unsigned)Z;
+    rk->launch.block[0] = (unsigned)(64 * sh.wvm * sh.wvn);
+    rk->klass = KernelClass::MATMUL_MFMA;
+    rk->strategy = strf("mfma 32x32x2 f32, operands as expressions (%d + %d loads per element pair, %d tiles ahead) M=%lld N=%lld K=%lld Z=%lld tile %dx%dx16 A:%s B:%s",
+                        n_loads[0], n_loads[1], depth, (long long)M, (long long)N, (long long)K, (long long)Z, sh.bm, sh.bn,
+                        walk_k[0] ? "k-major" : "m-major", walk_k[1] ? "k-major" : "n-major");
+    rk->n_params = ep.n_params;
+    rk->n_vars = 0;
+    rk->flops = 2.0 * (double)M * (double)N * (double)K * (double)Z;
+    rk->bytes = ep.bytes;
+    rk->tables = ep.tables;
+    if (!ep.tables.empty()) rk->strategy += strf(", %zu parts of the epilogue as 16-bit lookup tables", ep.tables.size());
+  };
+  build(F32Shape{BM, BN, WVM, WVN}, out);
+  f32_variants(M, N, F32Shape{BM, BN, WVM, WVN}, build, out);
   return true;
 }
 
