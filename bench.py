@@ -148,7 +148,7 @@ def run_gpu(workload, steps, warmup):
         extra["seq_len"] = ctx[0].numel if ctx else None
     top = sorted(groups.items(), key=lambda kv: -kv[1]["ms"])[:int(os.environ.get("POLY_BENCH_GROUPS", "8"))]
     for key, g in top:
-        log(f"  {g['ms']:8.3f} ms  x{g['launches']:3d}  {key[:150]}")
+        log(f"  {g['ms']:8.3f} ms  x{g['launches']:3d}  {key[:int(os.environ.get('POLY_BENCH_DESC_CHARS', '150'))]}")
     plan.close()
     return ms_per_step, tokens, roofline, extra
 
