@@ -271,7 +271,19 @@ def main():
     ap.add_argument("--path", choices=["plan", "vtable"], default="plan",
                     help="plan: poly_hip_compile_schedule + poly_hip_plan_run (default, what the metric is quoted on); "
                          "vtable: the descriptor row alone, one launch per scheduled kernel")
+    ap.add_argument("--copy-calibration", action="store_true",
+                    help="instead of a benchmark: three device-to-device copies of 1 GiB, the kernel of known traffic "
+                         "that the FETCH_SIZE / WRITE_SIZE counters of a rocprofv3 --pmc run are scaled by")
     args = ap.parse_args()
+    if args.copy_calibration:
+        import torch
+        x = torch.empty(1 << 28, dtype=torch.float32, device="cuda").fill_(1.0)
+        y = torch.empty_like(x)
+        for _ in range(3):
+            y.copy_(x)
+        torch.cuda.synchronize()
+        print(json.dumps({"copied_bytes_per_launch": x.numel() * 4, "launches": 3}), flush=True)
+        return
     if args.gpus != 1:
         sys.exit("bench.py: this backend runs on one GPU; --gpus must be 1 (nothing here shards across devices)")
     # The CPU baseline first, before anything touches the GPU: the reference's CPU backend

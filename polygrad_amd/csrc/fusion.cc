@@ -1181,14 +1181,16 @@ static bool match_row_chain_impl(const Sched &sc, int a_item, const std::vector<
   if (row_V) rk.strategy += ", intermediate rows kept in registers";
   if (n_exported) rk.strategy += strf(", %d row values stored for later kernels", n_exported);
   if (g_narrow_store_slot >= 0 && !narrow_stored) FA_REJECT();
-  if (narrow_stored) rk.strategy += ", result stored as the bf16 values that its fp32 values are casts of";
+  if (narrow_stored) {
+    rk.strategy += ", result stored as the bf16 values that its fp32 values are casts of";
+  }
   out->row_chain_from = a_item;
   {
     const KernelGraph &gl = sc.graphs[(size_t)phases.back().m.item];
     out->row_chain_stores = phases.back().is_map ? sc.slot(phases.back().m.item, gl.param_slot(gl.stores[0].param)) : -1;
   }
   rk.n_params = (int)arg_slots.size();
-  rk.bytes = bytes;
+  rk.bytes = bytes - (narrow_stored ? (double)s->buf_slots[g_narrow_store_slot].nbytes / 2 : 0.0);      // (a buffer stored as bf16 values is half written)
   return true;
 }
 
