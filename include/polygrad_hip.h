@@ -162,8 +162,12 @@ int poly_hip_plan_n_kernels(const PolyHipPlan *plan);
  * launch: a fused group counts once.  Returns the number of launches. */
 int poly_hip_plan_kernel_info(const PolyHipPlan *plan, int cap, int *klass, double *bytes,
                               double *flops);
-/* Times each kernel of one plan run with HIP events on the backend stream;
- * ms_out[k] for k in execution order.  Returns the number of kernels or <0. */
+/* Runs the plan once, launch by launch on the backend stream, and times every
+ * kernel with the pair of HIP events its own dispatch stamps at its start and end
+ * (hipExtModuleLaunchKernel): ms_out[k], k in execution order, is the sum over the
+ * kernels of launch k (a fill or first stage in front of it included) -- what a
+ * profiler's kernel trace reports, without the waits between launches.  Returns
+ * the number of launches or <0. */
 int poly_hip_plan_profile(PolyHipPlan *plan, void **slot_data, int n_slots, float *ms_out, int cap);
 /* Malloc'd description ("lower0_k3 matmul-mfma ...") of kernel k; free with
  * poly_hip_free_string. */

@@ -1116,20 +1116,34 @@ int poly_hip_plan_profile(PolyHipPlan *plan, void **slot_data, int n_slots, floa
     if (any && tuned_first_run(plan) != 0) return -1;
     plan->tuned = true;
   }
+  // One pass of the launches in order on the one stream, every kernel launch with the pair
+  // of events its own dispatch stamps (runtime_time_launches): a step's time is the sum of
+  // the durations of its kernels (a fill or a first stage in front of it included), as a
+  // profiler's kernel trace would give them, without the gaps between launches.
   const int n = (int)plan->units.size();
   hipStream_t stream = (hipStream_t)runtime_stream();
-  std::vector<hipEvent_t> ev((size_t)n + 1);
-  for (hipEvent_t &e : ev) if (hipEventCreate(&e) != hipSuccess) return -1;
+  LaunchTimes times;
+  std::vector<size_t> first((size_t)n + 1, 0);
   int rc = 0;
-  (void)hipEventRecord(ev[0], stream);
+  runtime_time_launches(&times);
   for (int step = 0; step < n && rc == 0; step++) {
-    rc = launch_unit(plan, (size_t)step);         // (a fill in front of the unit is timed with it)
-    (void)hipEventRecord(ev[(size_t)step + 1], stream);
+    first[(size_t)step] = times.events.size();
+    rc = launch_unit(plan, (size_t)step);
   }
-  (void)hipStreamSynchronize(stream);
-  for (int step = 0; step < n && step < cap && rc == 0; step++)
-    (void)hipEventElapsedTime(&ms_out[step], ev[(size_t)step], ev[(size_t)step + 1]);
-  for (hipEvent_t &e : ev) (void)hipEventDestroy(e);
+  runtime_time_launches(nullptr);
+  first[(size_t)n] = times.events.size();
+  if (times.failed) rc = -1;
+  if (hipStreamSynchronize(stream) != hipSuccess) rc = -1;
+  for (int step = 0; step < n && step < cap && rc == 0; step++) {
+    float total = 0;
+    for (size_t i = first[(size_t)step]; i + 1 < first[(size_t)step + 1]; i += 2) {
+      float ms = 0;
+      if (hipEventElapsedTime(&ms, (hipEvent_t)times.events[i], (hipEvent_t)times.events[i + 1]) != hipSuccess) { rc = -1; break; }
+      total += ms;
+    }
+    ms_out[step] = total;
+  }
+  for (void *e : times.events) (void)hipEventDestroy((hipEvent_t)e);
   return rc == 0 ? n : -1;
 }
 

@@ -10,6 +10,7 @@
 #include "runtime_hip.h"
 
 #include <hip/hip_runtime.h>
+#include <hip/hip_ext.h>
 #include <hip/hiprtc.h>
 #include <sys/stat.h>
 #include <unistd.h>
@@ -38,6 +39,7 @@ struct Runtime {
   hipStream_t stream = nullptr;
   hipStream_t side[3] = {nullptr, nullptr, nullptr};   // further streams of a plan's captured graphs, made on first use
   GraphLaunches *record = nullptr, *update = nullptr;   // see runtime_graph_record / runtime_graph_update
+  LaunchTimes *times = nullptr;                         // see runtime_time_launches
   hipStream_t launch_on = nullptr;     // where program_launch puts kernels when not the main stream
   std::map<uint64_t, std::weak_ptr<Module>> modules;   // keyed by source hash
   std::map<uint64_t, std::vector<char>> code_cache;    // compiled, not yet loaded
@@ -265,6 +267,7 @@ std::shared_ptr<void> runtime_table(const std::string &source, const std::string
   return owner;
 }
 
+void runtime_time_launches(LaunchTimes *t) { rt().times = t; }
 void runtime_graph_record(GraphLaunches *g) { rt().record = g; rt().update = nullptr; }
 void runtime_graph_update(GraphLaunches *g) { rt().update = g; rt().record = nullptr; }
 
@@ -287,6 +290,17 @@ int program_launch(Program *p, void **kernel_args, const LaunchSpec &ls) {
     return 0;
   }
   hipStream_t stream = r.launch_on ? r.launch_on : r.stream;
+  if (LaunchTimes *t = r.times) {
+    hipEvent_t e0 = nullptr, e1 = nullptr;
+    if (hipEventCreate(&e0) != hipSuccess || hipEventCreate(&e1) != hipSuccess) { t->failed = true; return -1; }
+    t->events.push_back((void *)e0);
+    t->events.push_back((void *)e1);
+    // (this entry point takes the grid in threads, not in workgroups)
+    hipError_t e = hipExtModuleLaunchKernel(p->fn, ls.grid[0] * ls.block[0], ls.grid[1] * ls.block[1], ls.grid[2] * ls.block[2], ls.block[0], ls.block[1],
+                                            ls.block[2], ls.lds_bytes, stream, kernel_args, nullptr, e0, e1, 0);
+    if (!check(e, "hipExtModuleLaunchKernel")) { t->failed = true; return -1; }
+    return 0;
+  }
   hipError_t e = hipModuleLaunchKernel(p->fn, ls.grid[0], ls.grid[1], ls.grid[2], ls.block[0], ls.block[1],
                                        ls.block[2], ls.lds_bytes, stream, kernel_args, nullptr);
   if (!check(e, "hipModuleLaunchKernel")) return -1;

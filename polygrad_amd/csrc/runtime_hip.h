@@ -54,6 +54,12 @@ struct GraphLaunches {
 };
 void runtime_graph_record(GraphLaunches *g);    // nullptr: back to plain launches
 void runtime_graph_update(GraphLaunches *g);
+// While `t` is set every kernel launch carries a pair of events that the dispatch itself
+// stamps at the kernel's first and last cycle (hipExtModuleLaunchKernel), appended to
+// t->events as (start, stop): what a profiler reports as the kernel's duration, without
+// the time a launch waits in the queue.  The caller destroys the events.
+struct LaunchTimes { std::vector<void *> events; bool failed = false; };
+void runtime_time_launches(LaunchTimes *t);
 
 // One lowered kernel: the program(s) plus how to call them.
 struct HipRunner {

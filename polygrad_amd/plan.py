@@ -136,7 +136,8 @@ class HipPlan:
                 for i in range(n)]
 
     def profile(self, slot_data):
-        """Per-kernel milliseconds of one eager pass (HIP events on the backend stream)."""
+        """Per-launch milliseconds of one eager pass: the durations of each launch's kernels,
+        from the HIP events that their dispatches stamp at start and end."""
         arr = self._ptr_array(slot_data)
         ms = (C.c_float * self.n_kernels)()
         rc = self.lib.poly_hip_plan_profile(self.handle, arr, len(self.slots), ms, self.n_kernels)
