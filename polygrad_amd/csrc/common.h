@@ -13,8 +13,12 @@
 
 namespace polyhip {
 
-// Switches that change results (they skip work so that the rest can be timed) exist only
+// Switches that change results (they skip work so that the rest can be timed), and the knobs
+// of tuning experiments (a forced tile, pipeline depth, prefetch distance, ...), exist only
 // in a measurement build of the library (make MEASURE=1); the default build ignores them.
+// What the default build reads from the environment are the switches that the tests use
+// for the other leg of a comparison (POLY_HIP_NO_...), the tuning switch POLY_BEAM, and the
+// cache and debugging settings.
 #ifdef POLY_HIP_MEASUREMENT_BUILD
 inline const char *measurement_env(const char *name) { return getenv(name); }
 #else

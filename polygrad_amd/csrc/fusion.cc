@@ -1257,7 +1257,7 @@ static bool match_copy(const Sched &sc, int item, CopyMap *cm) {
 // each instead of 10 to 17.  (Without such a mask all workgroups weigh the same and any
 // order does.)  Emitted as a table indexed by the workgroup's number within its XCD.
 static std::string attention_order(int64_t MB, int64_t Z) {
-  if (getenv("POLY_HIP_FA_PLAIN_ORDER") || Z % 8 != 0 || MB < 2) return "";
+  if (measurement_env("POLY_HIP_FA_PLAIN_ORDER") || Z % 8 != 0 || MB < 2) return "";
   const int64_t ZX = Z / 8, n = MB * ZX;
   if (n > 8192) return "";
   constexpr int CUS = 32;
@@ -2071,7 +2071,7 @@ static bool match_pointwise_group(const Sched &sc, int a_item, const std::vector
   // 32 bytes: 1.87 ms); the per-tensor updates of a training step (4 M positions each) do not
   // change.
   if (E >= ((int64_t)1 << 25) && arg_slots.size() >= 4) V = std::max(1, 4 / maxsz);
-  if (const char *e = getenv("POLY_HIP_PW_BYTES")) V = std::max(1, atoi(e) / maxsz);   // tuning experiments: bytes per thread and buffer
+  if (const char *e = measurement_env("POLY_HIP_PW_BYTES")) V = std::max(1, atoi(e) / maxsz);   // tuning experiments: bytes per thread and buffer
   while (V > 1 && E % V != 0) V /= 2;
   // the members as functions of the flat position (passed as `m`)
   std::string code, body;

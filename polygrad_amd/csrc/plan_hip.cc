@@ -468,7 +468,7 @@ PolyHipPlan *poly_hip_compile_schedule(PolyCtx *ctx, const PolySchedule *s) {
   // launches after their side launch instead.
   if (plan->forked) {
     int keep_for = n_units;
-    if (const char *e = getenv("POLY_HIP_SIDE_KEEP")) keep_for = std::max(0, atoi(e));
+    if (const char *e = measurement_env("POLY_HIP_SIDE_KEEP")) keep_for = std::max(0, atoi(e));
     for (int step = 0; step < n_units; step++) {
       if (!plan->on_side[(size_t)step]) continue;
       for (int sl : plan->units[(size_t)step].slots) {
@@ -716,9 +716,9 @@ PolyHipPlan *poly_hip_compile_schedule(PolyCtx *ctx, const PolySchedule *s) {
   plan->touch_at.assign((size_t)n_units, std::vector<int>());
   if (!getenv("POLY_HIP_NO_PREFETCH")) {
     int lead = 1;
-    if (const char *e = getenv("POLY_HIP_PREFETCH_LEAD")) lead = std::max(0, atoi(e));
+    if (const char *e = measurement_env("POLY_HIP_PREFETCH_LEAD")) lead = std::max(0, atoi(e));
     int64_t most = 128ll << 20;
-    if (const char *e = getenv("POLY_HIP_PREFETCH_MAX_MB")) most = (int64_t)std::max(0, atoi(e)) << 20;
+    if (const char *e = measurement_env("POLY_HIP_PREFETCH_MAX_MB")) most = (int64_t)std::max(0, atoi(e)) << 20;
     std::vector<char> written((size_t)ns, 0);
     for (const Unit &u : plan->units) for (int sl : u.writes) written[(size_t)sl] = 1;
     std::vector<int> touched_for((size_t)ns, -1000);

@@ -670,7 +670,7 @@ bool render_matmul(const MatmulMatch &mm, const MatmulEpilogue &ep, RenderedKern
   if (M > 2147483647LL || N > 2147483647LL || Z > 65535) return reject(__LINE__);
   if (A.dt == DT_F32) return render_matmul_f32(mm, ep, out);
   int BK = 64;
-  if (const char *e = getenv("POLY_HIP_MM_BK")) BK = atoi(e) == 32 ? 32 : 64;
+  if (const char *e = measurement_env("POLY_HIP_MM_BK")) BK = atoi(e) == 32 ? 32 : 64;
   // operand layout: contiguous along K, or along its row axis
   auto layout = [&](const KSplit &ks, const std::vector<Dim> &dims, bool is_a, int64_t rows, bool *kc) {
     int64_t inner_c = is_a ? dims.back().ca : dims.back().cb;
@@ -714,7 +714,7 @@ bool render_matmul(const MatmulMatch &mm, const MatmulEpilogue &ep, RenderedKern
   // a 256x256 tile holds 128 accumulator registers per lane: no room for the second
   // staging register set of the three-deep pipeline
   int pipe = (BM * BN >= 256 * 256) ? 2 : 3;
-  if (const char *e = getenv("POLY_HIP_MM_PIPE")) pipe = atoi(e) == 2 ? 2 : 3;
+  if (const char *e = measurement_env("POLY_HIP_MM_PIPE")) pipe = atoi(e) == 2 ? 2 : 3;
 
   // A deep product on so few tiles that half the chip would idle: the K tiles of a tile are
   // dealt to S workgroups, which leave fp32 partial results in scratch memory, and a second
@@ -737,15 +737,15 @@ bool render_matmul(const MatmulMatch &mm, const MatmulEpilogue &ep, RenderedKern
   };
   const bool may_split = !getenv("POLY_HIP_NO_SPLIT_K") && !measurement_env("POLY_HIP_MM_NOEPI") && M > 64 && N > 64;
   if (may_split) pick_split(64);
-  if (S == 1 && !fixed_tile && !getenv("POLY_HIP_MM_TILE") && !getenv("POLY_HIP_MM_OLD_ESTIMATE")) {
+  if (S == 1 && !fixed_tile && !getenv("POLY_HIP_MM_TILE") && !measurement_env("POLY_HIP_MM_OLD_ESTIMATE")) {
     pick_tile(true);
     pipe = (BM * BN >= 256 * 256) ? 2 : 3;
-    if (const char *e = getenv("POLY_HIP_MM_PIPE")) pipe = atoi(e) == 2 ? 2 : 3;
+    if (const char *e = measurement_env("POLY_HIP_MM_PIPE")) pipe = atoi(e) == 2 ? 2 : 3;
     if (may_split) pick_split(32);
   }
   if (may_split) {
     const int64_t kt = K / BK;
-    if (const char *e = getenv("POLY_HIP_MM_KSPLIT")) {   // tuning experiments: a given split
+    if (const char *e = measurement_env("POLY_HIP_MM_KSPLIT")) {   // tuning experiments: a given split
       const int s = atoi(e);
       if (s >= 1 && s <= 64 && kt % s == 0 && Z * s <= 65535) S = s;
     }
@@ -771,7 +771,7 @@ bool render_matmul(const MatmulMatch &mm, const MatmulEpilogue &ep, RenderedKern
     else if (bm * bn >= 128 * 128) c = Dma{64, 2, 2, 2, 2};
     else c = Dma{32, 4, 2, bm >= bn ? 4 : 1, bm >= bn ? 1 : 4};
     if (d->bk) c = *d;      // the caller's own choice
-    if (const char *ov = bm * bn < 256 * 256 ? getenv("POLY_HIP_MM_DMA") : getenv("POLY_HIP_MM_DMA_256")) {   // "BK,STAGES,WG,WVM,WVN": tuning experiments
+    if (const char *ov = bm * bn < 256 * 256 ? measurement_env("POLY_HIP_MM_DMA") : measurement_env("POLY_HIP_MM_DMA_256")) {   // "BK,STAGES,WG,WVM,WVN": tuning experiments
       int v[5];
       if (sscanf(ov, "%d,%d,%d,%d,%d", &v[0], &v[1], &v[2], &v[3], &v[4]) == 5) c = Dma{v[0], v[1], v[2], v[3], v[4]};
     }
@@ -812,7 +812,7 @@ bool render_matmul(const MatmulMatch &mm, const MatmulEpilogue &ep, RenderedKern
     }
     if (n_lo != 0 || n_hi != N) cfg += strf("#define POLY_N_LO %lld\n#define POLY_N_HI %lld\n", (long long)n_lo, (long long)n_hi);
     // each XCD (own L2) works on a contiguous run of tiles: let it re-read the smaller operand
-    const bool along_n = N > 2 * M && !getenv("POLY_HIP_MM_GROUP_M");
+    const bool along_n = N > 2 * M && !measurement_env("POLY_HIP_MM_GROUP_M");
     // (bands of 8 tile columns for the wide product: the 50257-wide head 727 -> 710 us against bands of 4)
     cfg += strf("#define POLY_GROUP_M %d\n", bm >= 256 && !(along_n && use_dma) ? 4 : 8);
     cfg += strf("#define POLY_GROUP_ALONG_N %d\n", along_n ? 1 : 0);
@@ -956,7 +956,7 @@ bool render_matmul(const MatmulMatch &mm, const MatmulEpilogue &ep, RenderedKern
         if (after < best) { best = after; pick = &c; }
       }
       Small forced{0, 0, 0, 0, 0};
-      if (const char *ov = getenv("POLY_HIP_MM_TAIL_TILE"))    // "BM,BN,WVM,WVN": tuning experiments
+      if (const char *ov = measurement_env("POLY_HIP_MM_TAIL_TILE"))    // "BM,BN,WVM,WVN": tuning experiments
         if (sscanf(ov, "%d,%d,%d,%d", &forced.bm, &forced.bn, &forced.wm, &forced.wn) == 4 && BN % forced.bn == 0) pick = &forced;
       RenderedKernel main, tail;
       if (pick && emit(BM, BN, WVM, WVN, pipe, &main, 0, n_lo) && emit(pick->bm, pick->bn, pick->wm, pick->wn, 3, &tail, n_lo, N)) {
