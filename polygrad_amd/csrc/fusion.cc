@@ -2629,6 +2629,8 @@ void find_fused_groups(const PolySchedule *s, const std::vector<KernelGraph> &gr
     g_narrow_store_slot = -1;
     if (!stores) continue;
     (*out)[gi] = std::move(chain);
+    (*out)[gi].needs_group_at = reader;
+    rg.needs_group_at = (*out)[gi].launch_item;
     rg.items = {reader};
     rg.launch_item = reader;
     rg.arg_slots.assign(s->items[reader].buf_slot_indices, s->items[reader].buf_slot_indices + s->items[reader].n_buf_slots);
@@ -2639,11 +2641,16 @@ void find_fused_groups(const PolySchedule *s, const std::vector<KernelGraph> &gr
   for (;;) {
     const std::vector<int> bad = fused_groups_out_of_order(s, graphs, *out);
     if (bad.empty()) break;
+    std::vector<int> partners;      // launch items of groups that go with a dropped one
     for (size_t i = bad.size(); i-- > 0;) {
       log_err("compile_schedule", "fused group at kernel %d (%zu kernels: %s) would launch out of order with a kernel it shares a buffer with: dropped",
               (*out)[(size_t)bad[i]].launch_item, (*out)[(size_t)bad[i]].items.size(), (*out)[(size_t)bad[i]].rk.strategy.substr(0, 60).c_str());
+      if ((*out)[(size_t)bad[i]].needs_group_at >= 0) partners.push_back((*out)[(size_t)bad[i]].needs_group_at);
       out->erase(out->begin() + bad[i]);
     }
+    for (int at : partners)
+      for (size_t i = out->size(); i-- > 0;)
+        if ((*out)[i].launch_item == at && (*out)[i].needs_group_at >= 0) out->erase(out->begin() + (long)i);
   }
 }
 

@@ -16,6 +16,10 @@ struct FusedGroup {
   RenderedKernel rk;
   // a row chain: the item it was grown from and the buffer its last kernel stores (-1: none)
   int row_chain_from = -1, row_chain_stores = -1;
+  // Two groups that only work together (a chain that stores bf16 values into an fp32 buffer
+  // and the product that reads them as such) name each other's launch item here: dropping
+  // one drops the other.
+  int needs_group_at = -1;
 };
 
 // Finds the fusable groups of a schedule.  graphs[k] is the analysed kernel of item k.
