@@ -295,9 +295,19 @@ int program_launch(Program *p, void **kernel_args, const LaunchSpec &ls) {
     if (hipEventCreate(&e0) != hipSuccess || hipEventCreate(&e1) != hipSuccess) { t->failed = true; return -1; }
     t->events.push_back((void *)e0);
     t->events.push_back((void *)e1);
-    // (this entry point takes the grid in threads, not in workgroups)
-    hipError_t e = hipExtModuleLaunchKernel(p->fn, ls.grid[0] * ls.block[0], ls.grid[1] * ls.block[1], ls.grid[2] * ls.block[2], ls.block[0], ls.block[1],
-                                            ls.block[2], ls.lds_bytes, stream, kernel_args, nullptr, e0, e1, 0);
+    // (this entry point takes the grid in threads, not in workgroups; a grid whose thread
+    // count does not fit its 32 bits is launched the usual way between the two events)
+    const unsigned long long tx = (unsigned long long)ls.grid[0] * ls.block[0], ty = (unsigned long long)ls.grid[1] * ls.block[1],
+                             tz = (unsigned long long)ls.grid[2] * ls.block[2];
+    hipError_t e;
+    if (tx <= 0xffffffffull && ty <= 0xffffffffull && tz <= 0xffffffffull) {
+      e = hipExtModuleLaunchKernel(p->fn, (uint32_t)tx, (uint32_t)ty, (uint32_t)tz, ls.block[0], ls.block[1], ls.block[2], ls.lds_bytes, stream,
+                                   kernel_args, nullptr, e0, e1, 0);
+    } else {
+      (void)hipEventRecord(e0, stream);
+      e = hipModuleLaunchKernel(p->fn, ls.grid[0], ls.grid[1], ls.grid[2], ls.block[0], ls.block[1], ls.block[2], ls.lds_bytes, stream, kernel_args, nullptr);
+      (void)hipEventRecord(e1, stream);
+    }
     if (!check(e, "hipExtModuleLaunchKernel")) { t->failed = true; return -1; }
     return 0;
   }
