@@ -353,7 +353,9 @@ def main():
                    "seq_len": extra.get("seq_len") if tokens else None, "parallelism": "single GPU",
                    "execution": "hipGraph replay of the compiled plan, inputs resident in HBM",
                    "parity": "against the reference CPU backend on the same seeded inputs (tests/, -m gpu): bit-exact for integer, "
-                             "index and movement kernels; rtol 1e-5 fp32 elementwise, 1e-4 fp32 reductions and matmul, 2e-2 bf16/fp16"},
+                             "index and movement kernels; rtol 1e-5 fp32 elementwise, 1e-4 fp32 reductions and matmul, 2e-2 bf16/fp16, with an "
+                             "absolute floor of 2e-2 of the tensor's scale on the T=1024 logits and residual stream (99.9 % of entries within "
+                             "2.5e-3 of it) and of 8e-3 on the one-pass attention form's output (2e-3 for the two-pass form)"},
         "roofline": roofline, "cpu_baseline": cpu, "detail": extra,
     }
     print(json.dumps(line), flush=True)
