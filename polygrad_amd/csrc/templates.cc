@@ -915,7 +915,7 @@ bool render_matmul(const MatmulMatch &mm, const MatmulEpilogue &ep, RenderedKern
   // GPT-2 small 682 -> 608 us, of GPT-2 medium 565 -> 509 us inside their plans (128x192:
   // 621 and 520; 128x128: 664; on 32-deep stages the same tiles are slower than 256x256, and
   // so is this one for K = 4096 and up or with a row-contiguous B).
-  if (!fixed_tile && !getenv("POLY_HIP_MM_TILE") && !getenv("POLY_HIP_NO_HEAD_TILE") && S == 1 && a_kc && b_kc && K <= 1536 && K % 64 == 0 && BM == 256 &&
+  if (!fixed_tile && !getenv("POLY_HIP_MM_TILE") && !getenv("POLY_HIP_NO_HEAD_TILE") && S == 1 && a_kc && b_kc && K >= 512 && K <= 1536 && K % 64 == 0 && BM == 256 &&
       BN == 256 && ((M + 255) / 256) * ((N + 255) / 256) * Z >= 1024) {
     Dma d{64, 2, 2, 2, 2};
     if (dma_for(192, 128, &d)) { BM = 192; BN = 128; WVM = WVN = 2; chosen = d; }
