@@ -910,13 +910,15 @@ bool render_matmul(const MatmulMatch &mm, const MatmulEpilogue &ep, RenderedKern
     }
   }
   // Many rounds of a short K loop with both operands contiguous along k (the 50 257-wide
-  // head: K = 768 or 1024, 6000 and 3000 tiles of 256x256): 192x128 tiles on 64-deep stages,
+  // head: K = 768 or 1024, 6000 and 3000 tiles of 256x256; from two rounds up: the head for
+  // one sequence, 788 tiles, 1.405 -> 1.362 ms for its plan; at 256 tiles a product with a
+  // table epilogue was 88 against 98 us the other way round): 192x128 tiles on 64-deep stages,
   // two workgroups to a CU, so that one's stores run under the other's K loop -- the head of
   // GPT-2 small 682 -> 608 us, of GPT-2 medium 565 -> 509 us inside their plans (128x192:
   // 621 and 520; 128x128: 664; on 32-deep stages the same tiles are slower than 256x256, and
   // so is this one for K = 4096 and up or with a row-contiguous B).
   if (!fixed_tile && !getenv("POLY_HIP_MM_TILE") && !getenv("POLY_HIP_NO_HEAD_TILE") && S == 1 && a_kc && b_kc && K >= 512 && K <= 1536 && K % 64 == 0 && BM == 256 &&
-      BN == 256 && ((M + 255) / 256) * ((N + 255) / 256) * Z >= 1024) {
+      BN == 256 && ((M + 255) / 256) * ((N + 255) / 256) * Z >= 512) {
     Dma d{64, 2, 2, 2, 2};
     if (dma_for(192, 128, &d)) { BM = 192; BN = 128; WVM = WVN = 2; chosen = d; }
   }
