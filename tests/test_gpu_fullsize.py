@@ -275,6 +275,35 @@ def test_gpt2_small_batch_elements_are_independent():
     assert float((diff > 0).float().mean()) < 1e-3, "same arithmetic per element: batch size must not change the logits"
 
 
+def test_head_product_on_two_workgroups_per_cu_changes_no_bit(monkeypatch):
+    """The 50 257-wide head of the B=1 plan (788 tiles of 256 x 256, both operands contiguous
+    along k, K = 768) runs on 192 x 128 tiles, 64 deep, two workgroups to a CU; the tile of
+    a product does not change the order of its sums, so the logits are those of the
+    256 x 256 tiles bit for bit (ragged on both sides: 1024 = 5 x 192 + 64 rows,
+    50257 = 392 x 128 + 81 columns)."""
+    import torch
+
+    def logits(switch_off):
+        if switch_off:
+            monkeypatch.setenv("POLY_HIP_NO_HEAD_TILE", "1")
+        else:
+            monkeypatch.delenv("POLY_HIP_NO_HEAD_TILE", raising=False)
+        plan = load("gpt2_small_bf16_b1_t1024")
+        data, names = gpt2_slot_tensors(plan, seed=3)
+        plan.run(data)
+        out = names["output"].clone()
+        descs = [k["desc"] for k in plan.kernel_info() if "N=50257" in k["desc"]]
+        plan.close()
+        return out, descs
+
+    new, d_new = logits(False)
+    old, d_old = logits(True)
+    assert len(d_new) == 1 and "tile 192x128x64" in d_new[0] and "2 per CU" in d_new[0], d_new
+    assert len(d_old) == 1 and "tile 256x256x32" in d_old[0], d_old
+    assert bool(torch.isfinite(new.float()).all()) and float(new.float().abs().max()) > 0
+    assert torch.equal(new.view(torch.uint8), old.view(torch.uint8))
+
+
 def test_gpt2_small_full_width_short_context_matches_reference():
     """GPT-2 small at its real width and depth (12 layers, d_model 768, vocab 50257) on one
     32-token sequence: the reference CPU backend finishes it in seconds.
