@@ -130,3 +130,36 @@ def test_24_layer_training_state_in_two_sets_of_buffers():
         assert not differing, differing[:10]
     assert bool(torch.isfinite(n0["loss"].float()).all())
     plan.close()
+
+
+def test_per_launch_times_add_up_to_the_step():
+    """poly_hip_plan_profile times every kernel with the events its own dispatch stamps at
+    start and end.  On the GPT-2 plan (one sequence) every launch gets a positive time, the
+    head product is the longest, and the sum of all of them lies a little under the time of
+    a replayed step (which also holds the gaps between kernels) -- not above it, as it did
+    when the time a launch waits in the queue was counted with it."""
+    import time
+    import torch
+    plan = load("gpt2_small_bf16_b1_t1024")
+    data, _ = gpt2_slot_tensors(plan, seed=3)
+    for _ in range(3):
+        plan.run(data)
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    steps = 20
+    for _ in range(steps):
+        plan.run(data, sync=False)
+    plan.sync()
+    step_ms = (time.perf_counter() - t0) / steps * 1e3
+    info = plan.kernel_info()
+    acc = [0.0] * len(info)
+    for _ in range(3):
+        plan.run(data, sync=False)
+        for i, ms in enumerate(plan.profile(data)):
+            acc[i] += ms / 3
+    plan.close()
+    assert all(ms > 0 for ms in acc), [k["desc"][:60] for k, ms in zip(info, acc) if ms <= 0]
+    longest = max(range(len(acc)), key=lambda i: acc[i])
+    assert "N=50257" in info[longest]["desc"], info[longest]["desc"]
+    total = sum(acc)
+    assert 0.6 * step_ms <= total <= 1.05 * step_ms, (total, step_ms)
