@@ -123,10 +123,15 @@ static_assert(POLY_BK == 32 || POLY_BK == 64, "K tile of 32 or 64");
 // bytes, four rows per 256) with the row number / 4.
 #define POLY_CH (POLY_BK / 8)
 __device__ __forceinline__ int poly_swz_k(int row) { return POLY_CH == 8 ? ((row ^ (row >> 3)) & 7) : ((row >> 2) & 3); }
-// Row-contiguous operand, [k][ROWS]: the transposing read of 16 lanes touches 4
-// consecutive k-rows x 32 bytes (32 lanes: 4 x 64 bytes), all at the same logical chunk;
-// the XOR term spreads the four rows over bits 0-1 and bits 1-2 of the chunk index.
-__device__ __forceinline__ int poly_swz_x(int k) { return (k & 3) | ((k & 1) << 2); }
+// Row-contiguous operand, [k][ROWS]: a transposing read is served 32 lanes at a time, which
+// touch 4 consecutive k-rows x 64 bytes (the same four logical chunks of each), 256 bytes in
+// all: the four k-rows have to land on the four different 64-byte groups of banks.  A k-row is
+// a multiple of 256 bytes long when ROWS is a multiple of 128, so without a swizzle they all
+// land on one; the chunk index is XORed with (k mod 4) * 4, which moves k-row k by k mod 4
+// groups.  (Other row counts -- 64, 192 -- keep a swizzle inside blocks of 8 chunks, which
+// pairs the four k-rows on two groups.)
+template <int ROWS>
+__device__ __forceinline__ int poly_swz_x(int k) { return (ROWS % 128 == 0) ? ((k & 3) << 2) : ((k & 3) | ((k & 1) << 2)); }
 
 // One LDS load: 16 bytes per lane from `base + voff` to LDS byte address lds_addr + 16 * lane.
 #ifdef POLY_HOST_ADDRESS_CHECK   // the kernel compiled for the host to check its indexing: lanes run one by one, LDS addresses count from the array
@@ -266,7 +271,7 @@ extern "C" __global__ void __launch_bounds__(POLY_NTHREADS) POLY_WAVES_ATTR poly
     a_off[q] = poly_a_row(m < POLY_M ? m : POLY_M - 1) + c * 8;
     a_kin[q] = 0;
 #else
-    const int kin = slot / (POLY_BM / 8), c = (slot % (POLY_BM / 8)) ^ poly_swz_x(kin);
+    const int kin = slot / (POLY_BM / 8), c = (slot % (POLY_BM / 8)) ^ poly_swz_x<POLY_BM>(kin);
     const int m = m0 + c * 8;
     a_off[q] = poly_a_row(m < POLY_M ? m : POLY_M - 8);
     a_kin[q] = kin;
@@ -281,7 +286,7 @@ extern "C" __global__ void __launch_bounds__(POLY_NTHREADS) POLY_WAVES_ATTR poly
     b_off[q] = poly_b_row(n < POLY_N ? n : POLY_N - 1) + c * 8;
     b_kin[q] = 0;
 #else
-    const int kin = slot / (POLY_BN / 8), c = (slot % (POLY_BN / 8)) ^ poly_swz_x(kin);
+    const int kin = slot / (POLY_BN / 8), c = (slot % (POLY_BN / 8)) ^ poly_swz_x<POLY_BN>(kin);
     const int n = n0 + c * 8;
     b_off[q] = poly_b_row(n < POLY_N ? n : POLY_N - 8);
     b_kin[q] = kin;
@@ -329,7 +334,7 @@ extern "C" __global__ void __launch_bounds__(POLY_NTHREADS) POLY_WAVES_ATTR poly
     a_fr[i] = r * (POLY_BK * 2); a_sw[i] = poly_swz_k(r);
 #else
     const int kl = 8 * (lane >> 5) + ((lane & 15) >> 2), x = wm + i * 32 + 16 * ((lane >> 4) & 1) + 4 * (lane & 3);
-    a_fr[i] = kl * (POLY_BM * 2) + (((x >> 3) ^ poly_swz_x(kl)) * 16) + (x & 7) * 2; a_sw[i] = 0;
+    a_fr[i] = kl * (POLY_BM * 2) + (((x >> 3) ^ poly_swz_x<POLY_BM>(kl)) * 16) + (x & 7) * 2; a_sw[i] = 0;
 #endif
   }
 #pragma unroll
@@ -339,7 +344,7 @@ extern "C" __global__ void __launch_bounds__(POLY_NTHREADS) POLY_WAVES_ATTR poly
     b_fr[j] = r * (POLY_BK * 2); b_sw[j] = poly_swz_k(r);
 #else
     const int kl = 8 * (lane >> 5) + ((lane & 15) >> 2), x = wn + j * 32 + 16 * ((lane >> 4) & 1) + 4 * (lane & 3);
-    b_fr[j] = kl * (POLY_BN * 2) + (((x >> 3) ^ poly_swz_x(kl)) * 16) + (x & 7) * 2; b_sw[j] = 0;
+    b_fr[j] = kl * (POLY_BN * 2) + (((x >> 3) ^ poly_swz_x<POLY_BN>(kl)) * 16) + (x & 7) * 2; b_sw[j] = 0;
 #endif
   }
   const int frag_col = lane >> 5;
