@@ -455,8 +455,9 @@ def test_gpt2_medium_24_layer_train_step_full_size():
     reference's scheduler (built with raised buffer caps; the stock reference stops at 256
     buffers), against the torch restatement of the same mixed-precision arithmetic.  Errors
     grow with the depth a gradient travels (every block rounds its activations to bf16 on
-    the way down): matrices are held to 5e-2 of their scale per element and 5e-3 on average,
-    vectors (sequential bf16 column sums over 4096 rows) to 1e-1 on average."""
+    the way down): matrices are held to 3e-2 of their scale per element and 4e-3 on average,
+    vectors (sequential bf16 column sums over 4096 rows) to 5e-2 on average (measured: 1.5e-2
+    and 2.3e-3 for the worst matrix, 2.4e-2 for the worst vector)."""
     import torch
     from polygrad_amd.inputs import block_train_slot_tensors
     path = os.path.join(PLANS, "gpt2_medium_train_24l_b4_t1024.polyplan")
@@ -485,9 +486,9 @@ def test_gpt2_medium_24_layer_train_step_full_size():
         kind = "matrix" if g.numel() > 8192 else "vector"
         worst[kind] = max(worst.get(kind, (0, 0)), (mean_e, max_e))
         if kind == "matrix":
-            assert mean_e <= 5e-3 and max_e <= 5e-2, (name, mean_e, max_e)
+            assert mean_e <= 4e-3 and max_e <= 3e-2, (name, mean_e, max_e)
         else:
-            assert mean_e <= 1e-1, (name, mean_e, max_e)
+            assert mean_e <= 5e-2, (name, mean_e, max_e)
         step = (t[name] - before[name]).float()
         big = want.abs() > 0.05 * s
         assert bool((torch.sign(step[big]) == -torch.sign(want[big])).float().mean() > 0.995), name
