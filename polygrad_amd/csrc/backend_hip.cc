@@ -140,7 +140,7 @@ int runner_use_variant(HipRunner *r, int idx) {
 }
 
 int runner_ensure_scratch(HipRunner *r) {
-  if (!r || r->pres.empty() || r->scratch) return 0;
+  if (!r || (r->pres.empty() && r->rk.scratch_bytes == 0) || r->scratch) return 0;
   r->scratch = runtime_alloc(r->rk.scratch_bytes);
   r->owns_scratch = true;
   return r->scratch ? 0 : -1;
@@ -198,7 +198,7 @@ int runner_launch(HipRunner *r, void **args, int n_args, void *scratch_from_call
     r->ptr_store[(size_t)(np + nv + t)] = r->tables[(size_t)t].get();
     r->arg_ptrs[(size_t)(np + nv + t)] = &r->ptr_store[(size_t)(np + nv + t)];
   }
-  if (!r->pres.empty()) {
+  if (!r->pres.empty() || r->rk.scratch_bytes > 0) {      // (scratch memory without a first stage: a product that leaves block maxima there)
     void *scratch = scratch_from_caller;
     if (!scratch) {
       if (runner_ensure_scratch(r) != 0) { log_err("execute", "%s: no scratch memory", r->name.c_str()); return -1; }

@@ -371,6 +371,12 @@ static std::string table_window_helpers(const std::vector<RenderedKernel::Table>
 
 // A matmul whose result only feeds a chain of pointwise kernels (bias/activation/residual
 // realised as kernels of their own): the chain becomes the matmul's epilogue.
+// Set around a second match of two groups that work together: the product whose output is
+// buffer `slot` leaves block maxima there (match_matmul_tail), and the attention group that
+// reads its keys from that buffer uses them (match_attention).
+static thread_local FusedGroup::KeyBounds g_block_maxima_hint;
+static thread_local int g_key_bounds_slot = -1;
+
 static bool match_matmul_tail(const Sched &sc, int s_item, const std::vector<char> &taken, FusedGroup *out) {
   const PolySchedule *s = sc.s;
   const KernelGraph &gS = sc.graphs[(size_t)s_item];
@@ -532,6 +538,31 @@ static bool match_matmul_tail(const Sched &sc, int s_item, const std::vector<cha
   {
     const int bs = sc.slot(s_item, mS.B.param);
     ep.b_from_hbm = !s->buf_slots[bs].is_intermediate && sc.writers[(size_t)bs].empty();
+  }
+  if (g_block_maxima_hint.slot == out_slot && ep.contiguous_n && mS.Z == 1) {
+    // the output as the reader sees it: row-major, `pitch` columns, from element 0 of the buffer
+    const FusedGroup::KeyBounds &h = g_block_maxima_hint;
+    const Member &m = members.back();
+    const KernelGraph &g = sc.graphs[(size_t)m.item];
+    const int li = g.n(g.n(g.stores[0].index).src[1]).lin;
+    Aff a;
+    bool plain = mS.M == h.rows && mS.N == h.pitch && m.range_expr.empty() && li >= 0 && lin_to_aff(g, g.lins[(size_t)li], m.rm, &a);
+    auto flat = [&](int64_t mm, int64_t nn) {
+      int64_t v = a.c0;
+      for (auto &kv : a.c) v += kv.second * matmul_range_value(mS, kv.first, mm, nn, 0);
+      return v;
+    };
+    for (int64_t mm = 0; plain && mm < mS.M; mm += 64)
+      for (int64_t nn = h.lo; plain && nn < h.hi; nn += 64)
+        plain = flat(mm, nn) == mm * h.pitch + nn && flat(mm, nn + 63) == mm * h.pitch + nn + 63 && flat(mm + 63, nn) == (mm + 63) * h.pitch + nn &&
+                flat(mm + 31, nn + 17) == (mm + 31) * h.pitch + nn + 17;
+    if (plain) {
+      ep.block_maxima.wanted = true;
+      ep.block_maxima.lo = h.lo;
+      ep.block_maxima.hi = h.hi;
+      ep.block_maxima.index = h.index;
+      ep.block_maxima.bytes = h.bytes;
+    }
   }
   if (!render_matmul(mS, ep, &out->rk)) return false;
   out->rk.tables = tables;
@@ -1679,6 +1710,7 @@ static bool match_attention(const Sched &sc, int s_item, const std::vector<char>
   };
   std::string v_expr = strf("%lld", (long long)aV.c0);
   for (auto &kv : aV.c) v_expr += strf(" + %lld * r%d", (long long)kv.second, kv.first);
+  int64_t k_pitch = 0;      // elements from one key to the next in the keys' buffer, when that is one number
   const char *off_name[3] = {"poly_q_off", "poly_k_off", "poly_v_off"};
   const std::string general[3] = {
       "__device__ __forceinline__ int poly_fa_q0(int z, int m) { return poly_fa_qz(z) + poly_fa_qm(m); }\n",
@@ -1695,6 +1727,7 @@ static bool match_attention(const Sched &sc, int s_item, const std::vector<char>
       for (int64_t x = 0; x < X; x++)
         if (eval_src(o, raw_off(o, z, x)) != base + x * step) { affine = false; break; }
     }
+    if (o == 1 && affine) k_pitch = step;
     if (affine)
       cfg += strf("__device__ __forceinline__ int %s(int z, int x) { return %s(%s(z, 0)) + x * %lld; }\n", off_name[o], src_name[o],
                   raw_name[o], (long long)step);
@@ -1703,6 +1736,46 @@ static bool match_attention(const Sched &sc, int s_item, const std::vector<char>
   }
   cfg += strf("#define POLY_SIGNATURE %s\n", sig.c_str());
   cfg += strf("#define POLY_FA_SKIP_DEAD_BLOCKS %d\n", p_is_term_over_sum ? 1 : 0);
+  // Do the keys lie in their buffer the way a row-major matrix product of `k_pitch` columns
+  // would have left them -- key block kb of z = (b, h) as the 64 x 64 block at row
+  // b * N + 64 kb, column c0 + 64 h?  Then that product can say how large the keys of every
+  // block are (key_bounds; find_fused_groups asks it to).
+  FusedGroup::KeyBounds kbnd;
+  if (k_pitch >= 64 && mS.N % 64 == 0 && mS.N / 64 <= 64 && mS.K == 64) {
+    const int64_t T = mS.N, NKB = T / 64, c0 = eval_src(1, raw_off(1, 0, 0)) % k_pitch;
+    // z counts (b, h) with either of the two running fastest
+    const bool heads_fastest = mS.Z > 1 && eval_src(1, raw_off(1, 1, 0)) % k_pitch != c0;
+    int64_t H = mS.Z, B = 1;
+    if (heads_fastest) {
+      for (int64_t z = 1; z < mS.Z; z++)
+        if (eval_src(1, raw_off(1, z, 0)) % k_pitch == c0) { H = z; break; }
+      B = mS.Z / H;
+    } else {
+      B = mS.Z;
+      for (int64_t z = 1; z < mS.Z; z++)
+        if (eval_src(1, raw_off(1, z, 0)) % k_pitch != c0) { B = z; break; }
+      H = mS.Z / B;
+    }
+    bool ok = c0 % 64 == 0 && B * H == mS.Z && c0 + H * 64 <= k_pitch;
+    for (int64_t z = 0; z < mS.Z && ok; z++)
+      for (int64_t kb = 0; kb < NKB && ok; kb++) {
+        const int64_t f = eval_src(1, raw_off(1, z, kb * 64));
+        const int64_t b = heads_fastest ? z / H : z % B, h = heads_fastest ? z % H : z / B;
+        ok = f / k_pitch == b * T + kb * 64 && f % k_pitch == c0 + h * 64;
+      }
+    if (ok) {
+      kbnd.possible = true;
+      kbnd.slot = folded[1].item >= 0 ? folded[1].src_slot : op_slot[1];
+      kbnd.pitch = k_pitch;
+      kbnd.rows = B * T;
+      kbnd.lo = c0;
+      kbnd.hi = c0 + H * 64;
+      const std::string zexpr = heads_fastest ? strf("((m) / %lld) * %lld + ((n) - %lld) / 64", (long long)T, (long long)H, (long long)c0)
+                                              : strf("(((n) - %lld) / 64) * %lld + (m) / %lld", (long long)c0, (long long)B, (long long)T);
+      kbnd.index = strf("(%s) * %lld + ((m) %% %lld) / 64", zexpr.c_str(), (long long)NKB, (long long)T);
+      kbnd.bytes = (size_t)(mS.Z * NKB) * sizeof(unsigned);
+    }
+  }
 
   // score: epilogue of S, then the pointwise chain
   {
@@ -1917,6 +1990,17 @@ static bool match_attention(const Sched &sc, int s_item, const std::vector<char>
     // the words depend on the mask buffer alone
     rk.pres_key = pre.source;
     rk.pre_reads.assign(1, mask_arg);
+    if (kbnd.possible && online) {
+      out->key_bounds = kbnd;
+      out->key_bounds.offset = (rk.scratch_bytes + 255) / 256 * 256;
+      if (g_key_bounds_slot == kbnd.slot) {
+        // the product that writes the keys leaves the block maxima behind the mask words
+        out->key_bounds.used = true;
+        cfg += strf("#define POLY_FA_KMAX_TABLE ((const unsigned int*)poly_scratch + %zu)\n", out->key_bounds.offset / sizeof(unsigned));
+        rk.scratch_bytes = out->key_bounds.offset + kbnd.bytes;
+        rk.pres_key += "// (scratch memory with key bounds)\n";     // shared only among launches that also get them
+      }
+    }
   }
   rk.source = std::string(hip_prelude()) + cfg + kAttentionTemplate;
   const std::string fa_cfg = cfg;
@@ -1928,6 +2012,7 @@ static bool match_attention(const Sched &sc, int s_item, const std::vector<char>
                      tin == DT_BF16 ? "bf16" : "f16", (long long)mS.Z, (long long)mS.M, (long long)mS.N,
                      cfg.find("#define POLY_FA_ONLINE 1") != std::string::npos ? "one pass, online softmax" : "two passes over keys, exact roundings");
   if (mask_table) rk.strategy += ", mask tiles classified by a first kernel";
+  if (out->key_bounds.used) rk.strategy += ", products of masked key blocks bounded by the block maxima the keys' product leaves";
   if (matmul_tuning_enabled()) {
     // the register budget (waves per SIMD) changes the schedule of the instructions, not
     // one value: candidates of the search that POLY_BEAM switches on
@@ -2574,6 +2659,7 @@ void find_fused_groups(const PolySchedule *s, const std::vector<KernelGraph> &gr
     if (taken[(size_t)k] || graphs[(size_t)k].reduces.size() != 1) continue;
     FusedGroup fg;
     if (!match_attention(sc, k, taken, &fg) && !match_matmul_tail(sc, k, taken, &fg) && !match_row_chain(sc, k, taken, &fg)) continue;
+    fg.matched_from = k;
     accept(fg, taken);
   }
   // what is left of the pointwise kernels, in runs over the same positions
@@ -2635,6 +2721,88 @@ void find_fused_groups(const PolySchedule *s, const std::vector<KernelGraph> &gr
     rg.launch_item = reader;
     rg.arg_slots.assign(s->items[reader].buf_slot_indices, s->items[reader].buf_slot_indices + s->items[reader].n_buf_slots);
     accept(rg, taken);
+  }
+  // An attention kernel that passes over masked key blocks must first compute their
+  // products, unless it knows how large the keys can be.  Where the keys are columns of a
+  // product's output (the q | k | v projection), that product's epilogue has every key in
+  // its registers: it leaves the largest magnitude of each block of 64 keys x 64 features
+  // in the attention kernel's scratch memory, and the attention kernel bounds the products
+  // of a block by that times the sum of |q|.  Both groups are matched once more, knowing of
+  // each other.
+  for (size_t gi = 0, n0 = out->size(); gi < n0 && !getenv("POLY_HIP_NO_KEY_BOUNDS"); gi++) {
+    const FusedGroup::KeyBounds kb = (*out)[gi].key_bounds;
+    if (!kb.possible || kb.used || (*out)[gi].matched_from < 0 || sc.writers[(size_t)kb.slot].size() != 1) continue;
+    size_t pj = n0;
+    for (size_t j = 0; j < n0; j++)
+      if (j != gi && (*out)[j].matched_from >= 0 && (*out)[j].rk.klass == KernelClass::MATMUL_MFMA && !(*out)[j].arg_slots.empty() &&
+          (*out)[j].arg_slots[0] == kb.slot && (*out)[j].rk.scratch_of_item < 0 && (*out)[j].needs_group_at < 0 &&
+          (*out)[j].launch_item == sc.writers[(size_t)kb.slot][0])
+        pj = j;
+    if ((*out)[gi].needs_group_at >= 0) continue;
+    const int w_item = sc.writers[(size_t)kb.slot][0];
+    if (pj == n0 && taken[(size_t)w_item]) continue;
+    int first_step = sc.step_of[(size_t)(*out)[gi].items[0]];
+    for (int it : (*out)[gi].items) first_step = std::min(first_step, sc.step_of[(size_t)it]);
+    if (sc.step_of[(size_t)w_item] >= first_step) continue;
+    std::vector<char> free_again = taken;
+    FusedGroup product;
+    bool writes = false;
+    if (pj < n0) {
+      // the product and the pointwise kernels in its epilogue
+      for (int it : (*out)[pj].items) free_again[(size_t)it] = 0;
+      g_block_maxima_hint = kb;
+      writes = match_matmul_tail(sc, (*out)[pj].matched_from, free_again, &product) && product.items == (*out)[pj].items &&
+               product.launch_item == (*out)[pj].launch_item;
+      g_block_maxima_hint = FusedGroup::KeyBounds();
+      product.matched_from = (*out)[pj].matched_from;
+    } else {
+      // a product by itself: lowered here as the plan would lower it, with the wish
+      const PolyExecItem &wi = s->items[w_item];
+      uint64_t inputs = 0;
+      for (int p = 0; p < wi.n_buf_slots && p < 64; p++) {
+        const int sl = wi.buf_slot_indices[p];
+        if (!s->buf_slots[sl].is_intermediate && sc.writers[(size_t)sl].empty()) inputs |= (uint64_t)1 << p;
+      }
+      MatmulEpilogue wish;
+      wish.block_maxima.wanted = true;
+      wish.block_maxima.lo = kb.lo;
+      wish.block_maxima.hi = kb.hi;
+      wish.block_maxima.index = kb.index;
+      wish.block_maxima.bytes = kb.bytes;
+      matmul_hint_input_params(inputs);
+      matmul_hint_param_kinds(matmul_param_kinds_of(s, graphs, w_item, {}));
+      matmul_hint_block_maxima(&wish, kb.rows, kb.pitch);
+      std::string err;
+      writes = render_kernel(graphs[(size_t)w_item], "poly_k", RenderOptions(), &product.rk, &err) && product.rk.klass == KernelClass::MATMUL_MFMA &&
+               product.rk.guards.empty() && product.rk.n_vars == 0 && product.rk.n_params == wi.n_buf_slots;
+      matmul_hint_block_maxima(nullptr, 0, 0);
+      matmul_hint_param_kinds({});
+      matmul_hint_input_params(0);
+      product.items = {w_item};
+      product.launch_item = w_item;
+      product.arg_slots.assign(wi.buf_slot_indices, wi.buf_slot_indices + wi.n_buf_slots);
+    }
+    writes = writes && product.rk.writes_block_maxima && product.rk.scratch_bytes == kb.bytes && product.rk.pres_key.empty();
+    if (!writes) continue;
+    free_again = taken;
+    for (int it : (*out)[gi].items) free_again[(size_t)it] = 0;
+    FusedGroup attention;
+    g_key_bounds_slot = kb.slot;
+    const bool reads = match_attention(sc, (*out)[gi].matched_from, free_again, &attention) && attention.items == (*out)[gi].items &&
+                       attention.launch_item == (*out)[gi].launch_item && attention.key_bounds.used && attention.key_bounds.bytes == kb.bytes;
+    g_key_bounds_slot = -1;
+    if (!reads) continue;
+    attention.matched_from = (*out)[gi].matched_from;
+    product.rk.scratch_of_item = attention.launch_item;
+    product.rk.scratch_offset = attention.key_bounds.offset;
+    product.needs_group_at = attention.launch_item;
+    attention.needs_group_at = product.launch_item;
+    if (getenv("POLY_HIP_DEBUG"))
+      fprintf(stderr, "polygrad: compile_schedule: the product at kernel %d leaves the block maxima of the keys for the attention kernel at kernel %d\n",
+              product.launch_item, attention.launch_item);
+    (*out)[gi] = std::move(attention);
+    if (pj < n0) (*out)[pj] = std::move(product);
+    else accept(product, taken);
   }
   // every pair of items that share a buffer keeps its order; a group that breaks one is
   // dropped and its kernels launch one by one at their own places

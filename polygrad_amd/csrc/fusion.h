@@ -1,5 +1,6 @@
 // Plan-level fusion of kernel groups (see fusion.cc).
 #pragma once
+#include <string>
 #include <vector>
 
 #include "polygrad_abi.h"
@@ -20,6 +21,18 @@ struct FusedGroup {
   // and the product that reads them as such) name each other's launch item here: dropping
   // one drops the other.
   int needs_group_at = -1;
+  int matched_from = -1;            // the item the matcher started from
+  // An attention group whose keys lie in the output of a product, in blocks of 64 keys x 64
+  // features that are blocks of 64 rows x 64 columns there (row-major, `pitch` columns,
+  // `rows` rows): what that product would have to leave for the kernel to bound the
+  // products of masked key blocks without computing them (MatmulEpilogue::block_maxima).
+  struct KeyBounds {
+    bool possible = false, used = false;
+    int slot = -1;
+    int64_t pitch = 0, rows = 0, lo = 0, hi = 0;
+    std::string index;
+    size_t bytes = 0, offset = 0;   // of the table, and where it lies in the kernel's scratch memory
+  } key_bounds;
 };
 
 // Finds the fusable groups of a schedule.  graphs[k] is the analysed kernel of item k.

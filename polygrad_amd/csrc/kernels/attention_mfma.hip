@@ -55,6 +55,13 @@
 //                                      not depend on z) pointer to the words that the
 //                                      classifying kernel below writes: the mask is then
 //                                      looked at once for all z instead of by every wave
+//   POLY_FA_KMAX_TABLE                 (optional, with POLY_FA_MASK_TABLE) pointer to one word per
+//                                      (z, block of 64 keys), [Z][N/64]: the bits of a float
+//                                      that no feature of any key of the block exceeds in
+//                                      magnitude (left there by the kernel that wrote the
+//                                      keys).  A tile whose mask entries are all one value
+//                                      is then passed over before its products when even
+//                                      the score of kmax * sum |q| is dead
 //   POLY_FA_CLASSIFY                   compile the classifying kernel instead of the
 //                                      attention kernel (same configuration block, the
 //                                      same arguments)
@@ -323,9 +330,10 @@ extern "C" __global__ void __launch_bounds__(FA_THREADS) __attribute__((amdgpu_w
     // entries of one query are consecutive in memory)
     const POLY_TIN *const mask_row = POLY_FA_MASK_PTR(mq, 4 * half, z);
 #endif
+    float q_l1 = 0.0f;   // (with POLY_FA_KMAX_TABLE) sum of |q| over the features of this lane's query, as staged
     // One 32 x 32 tile: tile t of key block kb, staged in LDS buffer cur.  With a mask,
     // `uniform` says that all its 32 x 32 entries hold the one value `cmask`.
-    auto tile = [&](int cur, int kb, int t, bool uniform, float cmask) {
+    auto tile = [&](int cur, int kb, int t, bool uniform, float cmask, float kmax) {
       // V^T fragment (A operand): feature row 32 dt + lq, the 8 keys of this lane's half
       // of the 16 keys 32t + 16u .., in the key order of the score registers
       auto v_frag = [&](int u, int dt) {
@@ -347,6 +355,22 @@ extern "C" __global__ void __launch_bounds__(FA_THREADS) __attribute__((amdgpu_w
       // non-finite product goes unseen here: its key is masked out for every query of
       // the tile, and would have made the unfused kernels' rows NaN.)
       if (uniform && cmask == -__builtin_inff()) return;
+#ifdef POLY_FA_KMAX_TABLE
+      // One value is added everywhere and no key of the block has a feature larger than
+      // kmax in magnitude: |product| <= kmax * sum |q| for every key (the factor covers
+      // the roundings of both sums).  If even the score of that bound has a term of exactly
+      // zero against the running maximum, for all 32 queries, the tile adds nothing and
+      // moves no maximum, and its products are not computed.  (A non-finite kmax or query
+      // makes the bound NaN or +inf, which is never dead.)
+      if (uniform && cmask != 0.0f) {
+        const int n0 = key_of(kb, t, 0);
+        const float bound = POLY_FA_MAXV(POLY_FA_SCORE_MASK(q_l1 * kmax * 1.001f, (POLY_TIN)cmask, mq, n0, z), mq, n0, z);
+        const bool early_dead = __builtin_amdgcn_exp2f((bound - m_run) * c) == 0.0f;
+        if (__builtin_amdgcn_ballot_w64(!early_dead) == 0) return;
+      }
+#else
+      (void)kmax;
+#endif
       asm volatile("" ::: "memory");   // (keeps the fragment reads and MFMAs below the test)
       fa_acc16 st;
       scores(cur, t, st);
@@ -481,16 +505,85 @@ extern "C" __global__ void __launch_bounds__(FA_THREADS) __attribute__((amdgpu_w
       store_v(0, rv);
     }
     __syncthreads();
+#if defined(POLY_FA_KMAX_TABLE) && POLY_FA_N / 32 <= 64
+    // lane l fetches the bound of key block l once (the bits of a float; whatever the
+    // keys' product has not written reads as NaN, which bounds nothing)
+    const unsigned my_kmax_bits = lane < FA_NKB ? (POLY_FA_KMAX_TABLE)[z * FA_NKB + lane] : 0xffffffffu;
+#pragma unroll
+    for (int ch = 0; ch < 8; ch++) {
+      const fa_in8 qf = *(const fa_in8 *)(q_row + ch * 8);
+#pragma unroll
+      for (int e = 0; e < 8; e++) q_l1 += __builtin_fabsf((float)qf[e]);
+    }
+    // When every tile that is left has one non-zero mask value for all four waves, the
+    // workgroup may be done before the last key block: each wave then tests the tiles left
+    // against its queries all at once (lane l: tile l, with the largest sum |q| and the
+    // smallest running maximum of the wave's queries), the waves tell each other through
+    // LDS in front of the block's barrier, and when all four say so the loop ends there --
+    // no load, store or barrier for the blocks behind.  Which blocks are left is the same
+    // for the four waves (the mask words of all four rows of tiles are looked at), so all
+    // of them take part in the same exchanges.
+    __shared__ int fa_rest_dead[2][4];
+    unsigned long long live_tiles, hard_tiles;
+    {
+      const unsigned *const wg_words = (const unsigned *)(POLY_FA_MASK_TABLE) + (m0 / 32) * (POLY_FA_N / 32);
+      bool one_value = lane < POLY_FA_N / 32;
+#pragma unroll
+      for (int w = 0; w < 4; w++) {
+        const unsigned u = lane < POLY_FA_N / 32 ? wg_words[w * (POLY_FA_N / 32) + lane] : 0u;
+        one_value = one_value && (u >> 16) != 0 && (u & 0x7fffu) != 0;
+      }
+      live_tiles = __builtin_amdgcn_ballot_w64(lane < POLY_FA_N / 32 && ((live_blocks >> (lane >> 1)) & 1ull) != 0);
+      hard_tiles = live_tiles & ~__builtin_amdgcn_ballot_w64(one_value);
+    }
+    const unsigned my_tile_kmax_bits = (unsigned)__builtin_amdgcn_ds_bpermute((lane >> 1) << 2, (int)my_kmax_bits);   // of the block of tile `lane`
+    unsigned q1max_bits = __builtin_bit_cast(unsigned, q_l1);      // (sums of magnitudes: ordered like their bits, a NaN above all)
+#pragma unroll
+    for (int sh = 1; sh < 64; sh <<= 1) {
+      const unsigned o = (unsigned)__builtin_amdgcn_ds_bpermute((lane ^ sh) << 2, (int)q1max_bits);
+      q1max_bits = q1max_bits < o ? o : q1max_bits;
+    }
+    int turn = 0;
+#endif
     while (kb < FA_NKB) {
       const int nb = next_block(kb + 1);
       if (nb < FA_NKB) { load_k(nb, rk); load_v(nb, rv); }
+#if defined(POLY_FA_KMAX_TABLE) && POLY_FA_N / 32 <= 64
+      const float kmax = __builtin_bit_cast(float, __builtin_amdgcn_readlane((int)my_kmax_bits, kb));
+#else
+      const float kmax = __builtin_inff();
+#endif
 #pragma unroll
       for (int t = 0; t < 2; t++) {
         const unsigned w = tile_word(2 * kb + t);
-        tile(cur, kb, t, (w >> 16) != 0, __builtin_bit_cast(float, w << 16));
+        tile(cur, kb, t, (w >> 16) != 0, __builtin_bit_cast(float, w << 16), kmax);
       }
+#if defined(POLY_FA_KMAX_TABLE) && POLY_FA_N / 32 <= 64
+      const unsigned long long rest = 2 * (kb + 1) < 64 ? (live_tiles & (~0ull << (2 * (kb + 1)))) : 0ull;
+      const bool exchange = rest != 0 && (hard_tiles & rest) == 0;      // (the same in all four waves)
+      if (exchange) {
+        float m_min = m_run;
+#pragma unroll
+        for (int sh = 1; sh < 64; sh <<= 1) m_min = __builtin_fminf(m_min, __builtin_bit_cast(float, __builtin_amdgcn_ds_bpermute((lane ^ sh) << 2, __builtin_bit_cast(int, m_min))));
+        const float ub = __builtin_bit_cast(float, q1max_bits) * __builtin_bit_cast(float, my_tile_kmax_bits) * 1.001f;
+        const POLY_TIN mk = __builtin_bit_cast(POLY_TIN, (unsigned short)(my_tile_word & 0xffffu));
+        const int n_of = 32 * (lane < POLY_FA_N / 32 ? lane : 0);
+        const float bound = POLY_FA_MAXV(POLY_FA_SCORE_MASK(ub, mk, mq, n_of, z), mq, n_of, z);
+        const bool lane_dead = __builtin_amdgcn_exp2f((bound - m_min) * c) == 0.0f;
+        const bool mine = ((rest >> lane) & 1ull) != 0;
+        const bool rest_dead = __builtin_amdgcn_ballot_w64(mine && !lane_dead) == 0;
+        if (lane == 0) fa_rest_dead[turn][wave] = rest_dead ? 1 : 0;
+      }
+#endif
       if (nb < FA_NKB) { store_k(cur ^ 1, rk); store_v(cur ^ 1, rv); }
       __syncthreads();
+#if defined(POLY_FA_KMAX_TABLE) && POLY_FA_N / 32 <= 64
+      if (exchange) {
+        const int all = fa_rest_dead[turn][0] & fa_rest_dead[turn][1] & fa_rest_dead[turn][2] & fa_rest_dead[turn][3];
+        if (all) break;
+      }
+      turn ^= 1;
+#endif
       kb = nb;
       cur ^= 1;
     }
@@ -533,13 +626,13 @@ extern "C" __global__ void __launch_bounds__(FA_THREADS) __attribute__((amdgpu_w
 #pragma unroll
           for (int j = 0; j < 4; j++) diff |= look[i][j] ^ s0;
         const bool uniform = __builtin_amdgcn_ballot_w64(diff != 0) == 0;
-        tile(cur, kb, t, uniform, __builtin_bit_cast(float, s0 << 16));
+        tile(cur, kb, t, uniform, __builtin_bit_cast(float, s0 << 16), __builtin_inff());
         look[0] = look_next[0];
         look[1] = look_next[1];
       }
 #else
-      tile(cur, kb, 0, false, 0.0f);
-      tile(cur, kb, 1, false, 0.0f);
+      tile(cur, kb, 0, false, 0.0f, __builtin_inff());
+      tile(cur, kb, 1, false, 0.0f, __builtin_inff());
 #endif
       if (kb + 1 < FA_NKB) { store_k(cur ^ 1, rk); store_v(cur ^ 1, rv); }
       __syncthreads();

@@ -26,6 +26,16 @@
 //                       into the first stage that the K loop no longer needs, during its
 //                       last iterations, so the window costs no LDS of its own
 //
+//   POLY_EP_BLOCKMAX_LO, POLY_EP_BLOCKMAX_HI, POLY_EP_BLOCKMAX_IDX(m, n), POLY_EP_BLOCKMAX_PTR
+//                       (optional, with POLY_EP_CONTIG and tiles of whole 64 x 64 blocks)
+//                       the columns [LO, HI) of the output, both multiples of 64, are read
+//                       by a later launch in blocks of 64 rows x 64 columns that wants a
+//                       bound on the magnitudes in each: the largest |stored value| of the
+//                       block whose first element is (m, n) goes, as the bits of the float,
+//                       to POLY_EP_BLOCKMAX_PTR[POLY_EP_BLOCKMAX_IDX(m, n)] (a NaN counts
+//                       as larger than everything).  Every block lies inside one
+//                       workgroup's tile: plain stores, nothing to clear beforehand
+//
 // Data path.  One global_load_lds_dwordx4 moves 16 bytes per lane from any global
 // address to LDS address M0 + 16 * lane: a wave fills 1024 consecutive bytes of LDS per
 // instruction, and which global chunk lands in which 16-byte slot is the lane's choice
@@ -211,6 +221,12 @@ extern "C" __global__ void __launch_bounds__(POLY_NTHREADS) POLY_WAVES_ATTR poly
   int bid = blockIdx.x - POLY_TOUCH_WGS;
 #else
   int bid = blockIdx.x;
+#endif
+#ifdef POLY_EP_BLOCKMAX_LO
+  static_assert(POLY_BM % 64 == 0 && POLY_BN % 64 == 0 && POLY_M % 64 == 0 && (POLY_EP_BLOCKMAX_LO) % 64 == 0 && (POLY_EP_BLOCKMAX_HI) % 64 == 0, "whole blocks per tile");
+  constexpr int BLK_N = POLY_BN / 64, BLK_COUNT = (POLY_BM / 64) * BLK_N;
+  __shared__ unsigned int poly_blk[BLK_COUNT];
+  if (threadIdx.x < BLK_COUNT) poly_blk[threadIdx.x] = 0u;      // (published by the K loop's barriers)
 #endif
   {
     constexpr int PER = NT / 8, REM = NT % 8;
@@ -498,6 +514,11 @@ extern "C" __global__ void __launch_bounds__(POLY_NTHREADS) POLY_WAVES_ATTR poly
       __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
       __builtin_amdgcn_wave_barrier();
       __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+#ifdef POLY_EP_BLOCKMAX_LO
+      typedef unsigned short poly_u16x8 __attribute__((ext_vector_type(8)));
+      poly_u16x8 tile_mag = (poly_u16x8)(0);      // largest magnitudes as 16-bit patterns (ordered like the values, a NaN above all)
+      const bool tile_counts = n0 + wn + j * 32 >= (POLY_EP_BLOCKMAX_LO) && n0 + wn + j * 32 < (POLY_EP_BLOCKMAX_HI);   // (wave-uniform)
+#endif
 #pragma unroll
       for (int h = 0; h < 2; h++) {
         const int row = (lane >> 2) + 16 * h, c0 = (lane & 3) * 8;
@@ -524,6 +545,9 @@ extern "C" __global__ void __launch_bounds__(POLY_NTHREADS) POLY_WAVES_ATTR poly
             const int ne = (POLY_N % 8 == 0 || n + e < POLY_N) ? n + e : n;
             o[e] = POLY_EP_VALUE(v[e], m, ne, z);
           }
+#ifdef POLY_EP_BLOCKMAX_LO
+          if (tile_counts) tile_mag = __builtin_elementwise_max(tile_mag, __builtin_bit_cast(poly_u16x8, o) & (poly_u16x8)(0x7fff));
+#endif
           if (POLY_N % 8 == 0 || n + 7 < POLY_N) {
 #ifdef POLY_EP_NT
             __builtin_nontemporal_store(o, (poly_out8_u *)POLY_EP_PTR(m, n, z));
@@ -546,6 +570,29 @@ extern "C" __global__ void __launch_bounds__(POLY_NTHREADS) POLY_WAVES_ATTR poly
       __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
       __builtin_amdgcn_wave_barrier();
       __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+#ifdef POLY_EP_BLOCKMAX_LO
+      if (tile_counts) {
+        unsigned int mag = tile_mag[0];
+#pragma unroll
+        for (int e = 1; e < 8; e++) mag = mag < tile_mag[e] ? (unsigned int)tile_mag[e] : mag;
+        // the largest of each row of 16 lanes (register exchanges only), then one LDS atomic per row
+#ifndef POLY_HOST_ADDRESS_CHECK
+#define POLY_ROW_MAX_STEP(CTRL) { const unsigned int o_ = (unsigned int)__builtin_amdgcn_update_dpp(0, (int)mag, CTRL, 0xf, 0xf, true); mag = mag < o_ ? o_ : mag; }
+        POLY_ROW_MAX_STEP(0xB1) POLY_ROW_MAX_STEP(0x4E) POLY_ROW_MAX_STEP(0x141) POLY_ROW_MAX_STEP(0x140)
+#undef POLY_ROW_MAX_STEP
+#endif
+        // (as the bits of the float of that magnitude)
+        const unsigned int tile_bits = __builtin_bit_cast(unsigned int, (float)__builtin_bit_cast(POLY_EP_TYPE, (unsigned short)mag));
+        if ((lane & 15) == 0) atomicMax(&poly_blk[((wm + i * 32) / 64) * BLK_N + (wn + j * 32) / 64], tile_bits);
+      }
+#endif
     }
+#ifdef POLY_EP_BLOCKMAX_LO
+  if (n0 < (POLY_EP_BLOCKMAX_HI) && n0 + POLY_BN > (POLY_EP_BLOCKMAX_LO)) __syncthreads();      // (the same for the whole workgroup)
+  if (threadIdx.x < BLK_COUNT) {
+    const int bm0 = m0 + ((int)threadIdx.x / BLK_N) * 64, bn0 = n0 + ((int)threadIdx.x % BLK_N) * 64;
+    if (bm0 < POLY_M && bn0 >= (POLY_EP_BLOCKMAX_LO) && bn0 < (POLY_EP_BLOCKMAX_HI)) (POLY_EP_BLOCKMAX_PTR)[POLY_EP_BLOCKMAX_IDX(bm0, bn0)] = poly_blk[threadIdx.x];
+  }
+#endif
 #endif
 }

@@ -434,7 +434,7 @@ PolyHipPlan *poly_hip_compile_schedule(PolyCtx *ctx, const PolySchedule *s) {
       const HipRunner *r = u.runner;
       // (several column sums as one launch are still a chain: up to 65 536 threads there)
       const uint64_t most = r->rk.klass == KernelClass::THREAD_REDUCE ? 65536 : 16384;
-      bool small = threads_of(r->rk.launch) <= most && r->guards.empty() && r->rk.variants.size() < 2 && r->rk.pres_key.empty();
+      bool small = threads_of(r->rk.launch) <= most && r->guards.empty() && r->rk.variants.size() < 2 && r->rk.pres_key.empty() && r->rk.scratch_of_item < 0;
       for (const RenderedKernel::Pre &pk : r->rk.pres) small = small && (r->rk.klass == KernelClass::THREAD_REDUCE || threads_of(pk.launch) <= 16384);
       int follows = 0;
       for (int sl : u.slots) if (!follows) follows = side_wrote[(size_t)sl];
@@ -536,8 +536,26 @@ PolyHipPlan *poly_hip_compile_schedule(PolyCtx *ctx, const PolySchedule *s) {
   // once: the first launch of such a family keeps its scratch memory to itself, the later
   // ones read it and skip their first stages.
   std::vector<char> keeps_scratch((size_t)n_units, 0);
+  // Launches that leave values in the scratch memory of a later launch (a product's block
+  // maxima for the attention kernel that reads its keys): writer_for[reader] = writer.
+  std::vector<int> writer_for((size_t)n_units, -1);
+  for (int ui = 0; ui < n_units; ui++) {
+    const RenderedKernel &rk = plan->units[(size_t)ui].runner->rk;
+    if (rk.scratch_of_item < 0) continue;
+    int reader = -1;
+    for (int r = ui + 1; r < n_units && reader < 0; r++)
+      if (plan->units[(size_t)r].item == rk.scratch_of_item) reader = r;
+    if (reader < 0 || plan->units[(size_t)reader].runner->rk.scratch_bytes < rk.scratch_offset + rk.scratch_bytes || plan->on_side[(size_t)ui] ||
+        plan->on_side[(size_t)reader]) {
+      log_err("compile_schedule", "launch %d leaves values for the launch of kernel %d, which is not a later launch of the main sequence with room for them", ui,
+              rk.scratch_of_item);
+      return nullptr;
+    }
+    writer_for[(size_t)reader] = ui;
+  }
   if (!getenv("POLY_HIP_NO_SHARED_FIRST_STAGE")) {
     std::map<std::pair<std::string, std::vector<int>>, int> leader_of;
+    std::map<std::pair<std::string, std::vector<int>>, int> last_member;      // the latest launch that reads a family's scratch memory
     for (int ui = 0; ui < n_units; ui++) {
       HipRunner *r = plan->units[(size_t)ui].runner;
       if (r->rk.pres_key.empty() || r->pres.empty()) continue;
@@ -554,6 +572,11 @@ PolyHipPlan *poly_hip_compile_schedule(PolyCtx *ctx, const PolySchedule *s) {
       for (int w = reuse ? it->second : ui; reuse && w < ui; w++)
         for (int sl : plan->units[(size_t)w].writes)
           if (std::find(read_slots.begin(), read_slots.end(), sl) != read_slots.end()) reuse = false;
+      // (values left by another launch arrive after the family's last reader is done, or this
+      // launch keeps scratch memory of its own)
+      if (reuse && writer_for[(size_t)ui] >= 0 && writer_for[(size_t)ui] < last_member[key]) reuse = false;
+      if (reuse && plan->units[(size_t)it->second].runner->rk.scratch_bytes < r->rk.scratch_bytes) reuse = false;
+      last_member[key] = ui;
       if (!reuse) { leader_of[key] = ui; continue; }
       HipRunner *lead = plan->units[(size_t)it->second].runner;
       if (runner_ensure_scratch(lead) != 0) return nullptr;
@@ -564,6 +587,21 @@ PolyHipPlan *poly_hip_compile_schedule(PolyCtx *ctx, const PolySchedule *s) {
       if (getenv("POLY_HIP_DEBUG"))
         fprintf(stderr, "polygrad: compile_schedule: launch %d reads what the first stage of launch %d leaves\n", ui, it->second);
     }
+  }
+  // (the writers get their readers' scratch memory, which starts as NaN bounds)
+  for (int ri = 0; ri < n_units; ri++) {
+    const int wi = writer_for[(size_t)ri];
+    if (wi < 0) continue;
+    HipRunner *reader = plan->units[(size_t)ri].runner, *writer = plan->units[(size_t)wi].runner;
+    if (!reader->scratch) {
+      if (runner_ensure_scratch(reader) != 0) return nullptr;
+      plan->kept_scratch_bytes += reader->rk.scratch_bytes;
+      keeps_scratch[(size_t)ri] = 1;
+    }
+    keeps_scratch[(size_t)wi] = 1;
+    void *at = (char *)reader->scratch + writer->rk.scratch_offset;
+    if (runtime_memset(at, 0xff, writer->rk.scratch_bytes) != 0) return nullptr;
+    runner_share_scratch(writer, at);
   }
   // What orders the two streams.
   if (plan->forked) {
@@ -1042,6 +1080,8 @@ int poly_hip_fused_groups(const PolySchedule *s, int index, char **source_out, i
                  pk.launch.block[0], groups[(size_t)index].rk.scratch_bytes);
         src += head + pk.source;
       }
+      if (groups[(size_t)index].rk.pres.empty() && groups[(size_t)index].rk.scratch_bytes > 0)     // scratch memory without a first stage
+        src += strf("\n// ---- scratch ---- bytes=%zu\n", groups[(size_t)index].rk.scratch_bytes);
       const std::vector<RenderedKernel::Variant> &vs = groups[(size_t)index].rk.variants;
       for (size_t i = 1; i < vs.size(); i++) src += "\n// ---- variant " + vs[i].label + "\n" + vs[i].source;
       *source_out = (char *)malloc(src.size() + 1);

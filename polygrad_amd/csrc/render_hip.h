@@ -72,6 +72,14 @@ struct RenderedKernel {
   // A matrix product whose own first workgroups read operand B into the memory-side cache
   // (the plan then launches nothing ahead of it for that).
   bool reads_b_ahead = false;
+  // A product that leaves the largest magnitude of every 64 x 64 block of some of its output
+  // columns in its scratch memory (MatmulEpilogue::block_maxima) -- and, set by the plan-level
+  // fusion, whose scratch memory that is: the launch that reads the bounds keeps them in its
+  // own scratch memory, `scratch_offset` bytes in, and the plan hands this kernel that
+  // address as its scratch pointer (`scratch_of_item`: the reader's launch item; -1: none).
+  bool writes_block_maxima = false;
+  int scratch_of_item = -1;
+  size_t scratch_offset = 0;
   // Kernels in two stages (reductions through partial results, matmuls whose operands are
   // prepared first): `pres` run first, in order, with the same arguments plus one more
   // pointer to `scratch_bytes` bytes of device memory that the runner owns; the main

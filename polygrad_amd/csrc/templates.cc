@@ -488,6 +488,39 @@ static bool epilogue_from_graph(const KernelGraph &g, const MatmulMatch &mm, Mat
   return true;
 }
 
+static thread_local MatmulEpilogue::BlockMaxima g_block_maxima;
+static thread_local int64_t g_block_maxima_rows = 0, g_block_maxima_pitch = 0;
+void matmul_hint_block_maxima(const MatmulEpilogue *e, int64_t rows, int64_t pitch) {
+  g_block_maxima = e ? e->block_maxima : MatmulEpilogue::BlockMaxima();
+  g_block_maxima_rows = rows;
+  g_block_maxima_pitch = pitch;
+}
+// Does the kernel store element (m, n) at m * pitch + n, for the blocks of 64 x 64 of the
+// columns [lo, hi)?  (checked at the corners and one inner point of every block)
+static bool store_is_row_major(const KernelGraph &g, const MatmulMatch &mm, int64_t pitch, int64_t lo, int64_t hi) {
+  const StoreInfo &st = g.stores[0];
+  const int li = g.n(g.n(st.index).src[1]).lin;
+  if (li < 0) return false;
+  const Lin &lin = g.lins[(size_t)li];
+  std::vector<std::pair<int, int64_t>> terms;
+  for (const auto &t : lin.terms) {
+    const Atom &a = g.atoms[(size_t)t.atom];
+    if (a.kind != Atom::RANGE) return false;
+    terms.push_back({g.range_ord.at(a.node), t.coef});
+  }
+  auto flat = [&](int64_t m, int64_t n) {
+    int64_t v = lin.c0;
+    for (auto &t : terms) v += t.second * matmul_range_value(mm, t.first, m, n, 0);
+    return v;
+  };
+  for (int64_t m = 0; m + 63 < mm.M; m += 64)
+    for (int64_t n = lo; n < hi; n += 64)
+      if (flat(m, n) != m * pitch + n || flat(m, n + 63) != m * pitch + n + 63 || flat(m + 63, n) != (m + 63) * pitch + n ||
+          flat(m + 31, n + 17) != (m + 31) * pitch + n + 17)
+        return false;
+  return true;
+}
+
 bool try_render_matmul(const KernelGraph &g, const std::string &fn, const RenderOptions &opt, RenderedKernel *out) {
   (void)fn; (void)opt;
   MatmulMatch mm;
@@ -495,6 +528,9 @@ bool try_render_matmul(const KernelGraph &g, const std::string &fn, const Render
   if (!match_matmul(g, &mm, &line)) return reject(line);
   MatmulEpilogue ep;
   if (!epilogue_from_graph(g, mm, &ep)) return false;
+  if (g_block_maxima.wanted && mm.Z == 1 && mm.M == g_block_maxima_rows && mm.N == g_block_maxima_pitch && mm.M % 64 == 0 &&
+      store_is_row_major(g, mm, g_block_maxima_pitch, g_block_maxima.lo, g_block_maxima.hi))
+    ep.block_maxima = g_block_maxima;
   ep.a_ptr = strf("data%d", mm.A.param);
   ep.b_ptr = strf("data%d", mm.B.param);
   ep.b_from_hbm = mm.B.param >= 0 && mm.B.param < 64 && ((g_input_params >> mm.B.param) & 1);
@@ -832,7 +868,15 @@ bool render_matmul(const MatmulMatch &mm, const MatmulEpilogue &ep, RenderedKern
     }
     cfg += matmul_k_fn("poly_a_k", ka, K);
     cfg += matmul_k_fn("poly_b_k", kb, K);
-    cfg += strf("#define POLY_SIGNATURE %s\n", signature.c_str());
+    // block maxima for a later launch (MatmulEpilogue::block_maxima): this template, one z, tiles of whole blocks
+    const bool block_maxima = ep.block_maxima.wanted && use_dma && S == 1 && Z == 1 && zd.empty() && bm % 64 == 0 && bn % 64 == 0 && M % 64 == 0 &&
+                              ep.contiguous_n && (ep.out_type == "__bf16" || ep.out_type == "_Float16") && ep.scratch_type.empty() &&
+                              ep.block_maxima.lo % 64 == 0 && ep.block_maxima.hi % 64 == 0 && ep.block_maxima.hi <= N &&
+                              !measurement_env("POLY_HIP_MM_NOEPI");
+    if (block_maxima)
+      cfg += strf("#define POLY_EP_BLOCKMAX_LO %lld\n#define POLY_EP_BLOCKMAX_HI %lld\n#define POLY_EP_BLOCKMAX_IDX(m, n) (%s)\n#define POLY_EP_BLOCKMAX_PTR poly_scratch\n",
+                  (long long)ep.block_maxima.lo, (long long)ep.block_maxima.hi, ep.block_maxima.index.c_str());
+    cfg += strf("#define POLY_SIGNATURE %s%s\n", signature.c_str(), block_maxima ? ", unsigned int* poly_scratch" : "");
     // LDS beside the operand tiles that an epilogue may use for the middle of its lookup tables
     if (S == 1 && !getenv("POLY_HIP_NO_LUT_WINDOW")) {
       if (!use_dma) cfg += strf("#define POLY_EP_WIN_ROOM %d\n", 163840 - 2 * (bm + bn) * BK * 2);
@@ -872,11 +916,15 @@ bool render_matmul(const MatmulMatch &mm, const MatmulEpilogue &ep, RenderedKern
     rk->launch.block[0] = (unsigned)(64 * wvm * wvn);
     rk->klass = KernelClass::MATMUL_MFMA;
     rk->reads_b_ahead = touch_wgs > 0;
+    rk->writes_block_maxima = block_maxima;
+    if (block_maxima) rk->scratch_bytes = ep.block_maxima.bytes;
     rk->strategy = strf("mfma 32x32x16 %s M=%lld N=%lld K=%lld Z=%lld tile %dx%dx%d A:%s B:%s", A.dt == DT_BF16 ? "bf16" : "f16",
                         (long long)M, (long long)N, (long long)K, (long long)Z, bm, bn, bk, a_kc ? "k-major" : "m-major",
                         b_kc ? "k-major" : "n-major");
     if (use_dma) rk->strategy += strf(", operands straight into LDS: %d waves, %d stages, %d per CU", wvm * wvn, dma.stages, dma.wg);
     if (touch_wgs) rk->strategy += strf(", %d workgroups read B ahead", touch_wgs);
+    if (block_maxima) rk->strategy += strf(", leaves the largest magnitude of every 64x64 block of columns [%lld, %lld) for the launch that reads them",
+                                           (long long)ep.block_maxima.lo, (long long)ep.block_maxima.hi);
     rk->n_params = ep.n_params;
     rk->n_vars = 0;
     rk->flops = 2.0 * (double)M * (double)N * (double)K * (double)Z;
@@ -972,11 +1020,12 @@ bool render_matmul(const MatmulMatch &mm, const MatmulEpilogue &ep, RenderedKern
       if (const char *ov = measurement_env("POLY_HIP_MM_TAIL_TILE"))    // "BM,BN,WVM,WVN": tuning experiments
         if (sscanf(ov, "%d,%d,%d,%d", &forced.bm, &forced.bn, &forced.wm, &forced.wn) == 4 && BN % forced.bn == 0) pick = &forced;
       RenderedKernel main, tail;
-      if (pick && emit(BM, BN, WVM, WVN, pipe, &main, 0, n_lo) && emit(pick->bm, pick->bn, pick->wm, pick->wn, 3, &tail, n_lo, N)) {
+      if (pick && emit(BM, BN, WVM, WVN, pipe, &main, 0, n_lo) && emit(pick->bm, pick->bn, pick->wm, pick->wn, 3, &tail, n_lo, N) &&
+          main.writes_block_maxima == out->writes_block_maxima && tail.writes_block_maxima == out->writes_block_maxima) {
         const std::string strategy = out->strategy;
         *out = main;
         out->pres.push_back({tail.source, tail.entry, tail.launch});
-        out->scratch_bytes = 256;      // (a kernel with a first stage owns scratch memory; this one uses none)
+        out->scratch_bytes = std::max<size_t>(256, main.scratch_bytes);      // (a kernel with a first stage owns scratch memory)
         out->strategy = strategy + strf(", columns from %lld on by a launch of %dx%d tiles ahead of it", (long long)n_lo, pick->bm, pick->bn);
         return true;
       }
@@ -992,7 +1041,7 @@ bool render_matmul(const MatmulMatch &mm, const MatmulEpilogue &ep, RenderedKern
     // the template with register staging
     for (const Shape &c : shapes) {
       RenderedKernel v;
-      if (emit(c.bm, c.bn, c.wm, c.wn, c.pp, &v, 0, -1, false) && v.source != out->source)
+      if (emit(c.bm, c.bn, c.wm, c.wn, c.pp, &v, 0, -1, false) && v.source != out->source && v.writes_block_maxima == out->writes_block_maxima)
         out->variants.push_back({strf("%dx%dw%dx%dp%d", c.bm, c.bn, c.wm, c.wn, c.pp), v.source, v.strategy, v.launch});
     }
     // the template that loads straight into LDS: tile, K tile, stages, workgroups per CU, waves
@@ -1005,7 +1054,8 @@ bool render_matmul(const MatmulMatch &mm, const MatmulEpilogue &ep, RenderedKern
     // on every product of the GPT-2 step)
     for (const DShape &c : dshapes) {
       RenderedKernel v;
-      if (emit(c.bm, c.bn, c.d.wvm, c.d.wvn, 3, &v, 0, -1, true, c.d) && v.source != out->source && v.strategy.find("straight into LDS") != std::string::npos)
+      if (emit(c.bm, c.bn, c.d.wvm, c.d.wvn, 3, &v, 0, -1, true, c.d) && v.source != out->source && v.strategy.find("straight into LDS") != std::string::npos &&
+          v.writes_block_maxima == out->writes_block_maxima)
         out->variants.push_back({strf("%dx%dx%dw%dx%ds%dg%d", c.bm, c.bn, c.d.bk, c.d.wvm, c.d.wvn, c.d.stages, c.d.wg), v.source, v.strategy, v.launch});
     }
   }

@@ -76,6 +76,18 @@ struct MatmulEpilogue {
   // Operand B is a buffer that nothing in the plan writes (weights): at the time of the
   // launch it is in HBM, not in the caches.
   bool b_from_hbm = false;
+  // A later launch reads the columns [lo, hi) of the output (row-major, one z) in blocks of
+  // 64 rows x 64 columns and wants the largest magnitude in each: the product then leaves
+  // it, as the bits of the float, in word `index` (C text in terms of the block's first
+  // row m and column n) of its scratch memory.  Only the template that loads straight into
+  // LDS does that, on tiles of whole blocks; RenderedKernel::writes_block_maxima says
+  // whether it did.
+  struct BlockMaxima {
+    bool wanted = false;
+    int64_t lo = 0, hi = 0;
+    std::string index;
+    size_t bytes = 0;      // of the table
+  } block_maxima;
 };
 // Set by the plan compiler around the lowering of one scheduled kernel: bit p says that
 // buffer parameter p is an input of the plan that none of its kernels writes.
@@ -88,6 +100,11 @@ void matmul_hint_input_params(uint64_t mask);
 // that takes the buffer as a plain operand can read that, and render_kernel refuses every
 // other use.
 void matmul_hint_param_kinds(const std::vector<int> &kinds);
+// Also set around a lowering: a later launch wants the block maxima of this product's
+// output, which it takes for a row-major matrix of `rows` x `pitch` elements from element 0
+// of the buffer (nullptr: no such wish).  The product grants it when its store is that.
+struct MatmulEpilogue;
+void matmul_hint_block_maxima(const MatmulEpilogue *with_block_maxima, int64_t rows, int64_t pitch);
 int matmul_param_kind(int param);
 // Is element (m, n + 1) of the kernel's output stored right after (m, n), for every n
 // that is not the last of an aligned group of 8?  (store index affine with coefficient 1

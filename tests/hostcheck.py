@@ -46,6 +46,7 @@ static poly_dim3 threadIdx, blockIdx, blockDim, gridDim;
 #define __builtin_amdgcn_sched_barrier(m) ((void)0)
 #define __builtin_amdgcn_exp2f(x) exp2f(x)
 template <class T> static T atomicAdd(T *p, T v) { T old = *p; *p += v; return old; }
+template <class T> static T atomicMax(T *p, T v) { T old = *p; if (old < v) *p = v; return old; }
 #define __builtin_amdgcn_mfma_f32_32x32x16_bf16(a, b, c, x, y, z) (c)
 #define __builtin_amdgcn_mfma_f32_32x32x16_f16(a, b, c, x, y, z) (c)
 #define __builtin_amdgcn_mfma_f32_32x32x2f32(a, b, c, x, y, z) (c)
@@ -177,6 +178,9 @@ def _jobs(lib, schedule, max_threads, only, groups):
         seen.add((main, sizes))
         scratch = 0
         for unit in text.split("\n// ---- ")[1:]:
+            m = re.match(r"scratch ---- bytes=(\d+)\n", unit)
+            if m:       # scratch memory without a first stage (a product that leaves values for a later launch)
+                scratch = int(m.group(1))
             m = re.match(r"first stage ---- grid=(\d+),(\d+) block=(\d+) scratch=(\d+)\n", unit)
             if m:
                 scratch = int(m.group(4))

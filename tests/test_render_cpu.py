@@ -144,20 +144,38 @@ def test_kernel_groups_of_the_gpt2_plan_fuse_and_compile(hiplib):
     """Needs no device: in the benchmark schedule the plan compiler recognises, per layer,
     one attention group (six scheduled kernels plus the three q/k/v copies), three matmuls followed by a pointwise
     kernel (residual add, GELU, residual add) and two LayerNorms of three kernels each
-    (plus the final LayerNorm); the generated sources compile."""
+    (plus the final LayerNorm); the generated sources compile.  The q | k | v product of a
+    layer is a launch of its own that leaves the largest magnitude of every block of keys
+    for the attention kernel behind it, which bounds the products of masked key blocks by
+    them (POLY_HIP_NO_KEY_BOUNDS=1: neither)."""
     from polygrad_amd import PlanFile
     pf = PlanFile(os.path.join(ROOT, "polygrad_amd", "plans", "gpt2_small_bf16_b8_t1024.polyplan"))
     count = hiplib.poly_hip_fused_groups(pf.schedule, -1, None, None)
-    assert count == 12 + 36 + 25
+    assert count == 12 + 36 + 25 + 12
     seen = {}
     for i in range(count):
         src, n = C.c_void_p(), C.c_int()
         hiplib.poly_hip_fused_groups(pf.schedule, i, C.byref(src), C.byref(n))
         text = _ffi.take_string(src.value)
-        kind = "attention" if "POLY_FA_M" in text else "rows" if "poly_row_p0" in text else "tail"
-        assert n.value == {"attention": 9, "tail": 2, "rows": 3}[kind]
+        kind = ("attention" if "POLY_FA_M" in text else "rows" if "poly_row_p0" in text else
+                "keys" if "#define POLY_EP_BLOCKMAX_LO 768" in text else "tail")
+        assert n.value == {"attention": 9, "tail": 2, "rows": 3, "keys": 1}[kind]
         seen.setdefault(kind, []).append(text)
-    assert len(seen["attention"]) == 12 and len(seen["tail"]) == 36 and len(seen["rows"]) == 25
+    assert len(seen["attention"]) == 12 and len(seen["tail"]) == 36 and len(seen["rows"]) == 25 and len(seen["keys"]) == 12
+    keys = seen["keys"][0]
+    # 8 sequences x 12 heads x 16 blocks of 64 keys, z counting the sequence fastest
+    assert "#define POLY_EP_BLOCKMAX_HI 1536" in keys and "(((n) - 768) / 64) * 8 + (m) / 1024) * 16 + ((m) % 1024) / 64" in keys
+    assert "unsigned int* poly_scratch" in keys and "\n// ---- scratch ---- bytes=6144\n" in keys
+    assert hiplib.poly_hip_compile_check(keys.split("\n// ---- ")[0].encode()) == 0
+    assert all("#define POLY_FA_KMAX_TABLE ((const unsigned int*)poly_scratch + " in a for a in seen["attention"])
+    os.environ["POLY_HIP_NO_KEY_BOUNDS"] = "1"
+    try:
+        assert hiplib.poly_hip_fused_groups(pf.schedule, -1, None, None) == 12 + 36 + 25
+        src = C.c_void_p()
+        hiplib.poly_hip_fused_groups(pf.schedule, 1, C.byref(src), None)
+        assert "POLY_FA_KMAX_TABLE ((" not in _ffi.take_string(src.value)
+    finally:
+        del os.environ["POLY_HIP_NO_KEY_BOUNDS"]
     assert hiplib.poly_hip_compile_check(seen["rows"][0].encode()) == 0
     att = seen["attention"][0]
     assert "poly_fa_term" in att and "__builtin_amdgcn_mfma_f32_32x32x16_bf16" in att
