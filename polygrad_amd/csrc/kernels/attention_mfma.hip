@@ -450,14 +450,30 @@ extern "C" __global__ void __launch_bounds__(FA_THREADS) __attribute__((amdgpu_w
             for (int r = 0; r < 16; r++) o[dt][r] = o[dt][r] * alpha;
         }
       }
-      const float mc = ((m_run == -__builtin_inff()) ? 0.0f : m_run) * c;
+      // The exponent (x - m) c as one fused multiply-add, x c - (m c): the rounding of m c
+      // puts 2^-24 |m c| into the exponent, which is nothing while the reference is of any
+      // ordinary size (|m| <= 4096: 3.5e-4 at most, a tenth of the 16-bit rounding of the
+      // term) and ruinous for scores of 1e9.  References beyond that (rare: one test per
+      // tile, the same for the whole wave) take the difference first, as the unfused
+      // kernels do.
+      const float m_ref = (m_run == -__builtin_inff()) ? 0.0f : m_run;
+      const float mc = m_ref * c;
       float sum = 0.0f;
       POLY_TIN p[16];
+      if (__builtin_amdgcn_ballot_w64(!(__builtin_fabsf(m_ref) <= 4096.0f)) == 0) {
 #pragma unroll
-      for (int r = 0; r < 16; r++) {
-        const float tt = __builtin_amdgcn_exp2f(__builtin_fmaf(x[r], c, -mc));
-        sum = sum + tt;
-        p[r] = (POLY_TIN)tt;
+        for (int r = 0; r < 16; r++) {
+          const float tt = __builtin_amdgcn_exp2f(__builtin_fmaf(x[r], c, -mc));
+          sum = sum + tt;
+          p[r] = (POLY_TIN)tt;
+        }
+      } else {
+#pragma unroll
+        for (int r = 0; r < 16; r++) {
+          const float tt = __builtin_amdgcn_exp2f((x[r] - m_ref) * c);
+          sum = sum + tt;
+          p[r] = (POLY_TIN)tt;
+        }
       }
       l_run = l_run + sum;
 #pragma unroll

@@ -100,3 +100,35 @@ def test_eight_sequences_same_bits_with_and_without_key_bounds():
     got = logits("gpt2_small_bf16_b8_t1024", nothing, True)
     want = logits("gpt2_small_bf16_b8_t1024", nothing, False)
     assert torch.equal(got.view(torch.int16), want.view(torch.int16))
+
+
+def test_scores_of_1e10_stay_finite_in_the_single_pass_form():
+    """Keys of a head around 1e10 give scores around 1e10, which the unfused kernels handle:
+    they subtract the row's maximum before anything is multiplied.  The single-pass kernel
+    forms its exponents as x c - m c while the reference m is small and as (x - m) c beyond
+    4096 (the fused form would put the rounding of m c, here around 1e3, into the exponent:
+    every term 0 or inf, rows of 0 / 0).  Wanted: finite logits, the same with and without
+    the bounds on the keys, and as close to the two-pass form (which keeps every rounding of
+    the unfused kernels) as on ordinary data."""
+    import torch
+
+    def tweak(names):
+        w, _ = k_columns(names, 0, 3)
+        w.mul_(2e10)
+
+    got = logits("gpt2_small_bf16_b1_t1024", tweak, True)
+    assert torch.equal(got.view(torch.int16), logits("gpt2_small_bf16_b1_t1024", tweak, False).view(torch.int16))
+    os.environ["POLY_HIP_EXACT_ATTENTION"] = "1"
+    try:
+        plan = HipPlan.from_file(os.path.join(PLANS, "gpt2_small_bf16_b1_t1024.polyplan"))
+    finally:
+        os.environ.pop("POLY_HIP_EXACT_ATTENTION", None)
+    data, names = gpt2_slot_tensors(plan, seed=3)
+    tweak(names)
+    plan.run(data)
+    want = names["output"].clone().float()
+    plan.close()
+    assert bool(torch.isfinite(got.float()).all()) and bool(torch.isfinite(want).all())
+    err = (got.float() - want).abs()
+    scale = float(want.abs().max())
+    assert float(err.mean()) <= 4e-3 * scale and float(err.max()) <= 4e-2 * scale, (float(err.mean()), float(err.max()), scale)
