@@ -154,7 +154,8 @@ def run_gpu(workload, steps, warmup):
                  flop_time_ms=round(total_flops / (PEAK_MFMA_TFLOPS * 1e12) * 1e3, 3),
                  byte_time_ms=round(total_bytes / (PEAK_HBM_GBS * 1e9) * 1e3, 3),
                  workspace_MiB=round(plan.workspace_bytes() / 2**20, 1), compile_s=round(compile_s, 1))
-    forms = sorted({"one pass, online softmax" if "one pass" in k["desc"] else "two passes, exact roundings"
+    forms = sorted({("one pass, online softmax" if "one pass" in k["desc"] else "two passes, exact roundings") +
+                    (", masked key blocks bounded by the keys' block maxima" if "bounded by the block maxima" in k["desc"] else "")
                     for k in info if k["klass"] == "attention-mfma"})
     if forms:
         extra["attention_form"] = "; ".join(forms)
