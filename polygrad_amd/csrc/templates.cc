@@ -389,34 +389,77 @@ static bool epilogue_from_graph(const KernelGraph &g, const MatmulMatch &mm, Mat
     visit(st.value);
   }
   MatmulEpilogue &ep0 = *epo;
-  std::vector<std::pair<int, int>> lut_of;       // (node, load) of table i
-  for (const Part &pt : parts) {
-    Emitter et(g);
-    Scope St;
-    St.indent = 1;
-    et.preset(pt.load, "x");
-    const std::string v = et.emit(pt.node, &St);
-    if (et.failed() || et.uses_threefry) continue;
-    const DT odt = g.n(pt.node).dt, idt = g.n(pt.load).dt;
-    RenderedKernel::Table t;
-    t.source = std::string(hip_prelude()) +
-               strf("extern \"C\" __global__ void __launch_bounds__(256) poly_lut_fill(%s* out) {\n"
-                    "  const unsigned int i = blockIdx.x * 256u + threadIdx.x;\n"
-                    "  const %s x = __builtin_bit_cast(%s, (unsigned short)i);\n",
-                    dt_cname(odt), dt_cname(idt), dt_cname(idt)) +
-               St.code + strf("  out[i] = %s;\n}\n", v.c_str());
-    t.entry = "poly_lut_fill";
-    t.bytes = (size_t)65536 * (size_t)dt_size(odt);
-    t.launch.grid[0] = 256;
-    t.launch.block[0] = 256;
-    ep0.tables.push_back(t);
-    lut_of.push_back({pt.node, pt.load});
+  // Parts of one load share a table: an entry holds the values of all of them (padded to a
+  // power of two), so an element costs one gather however many parts it has -- the address
+  // path serves two or three lanes a cycle, and three gathers per element of a 4096 x 4096
+  // output were 45 us of an 82 us launch.
+  struct Tab { int load; std::vector<int> nodes; std::string type; };
+  std::vector<Tab> tabs;
+  std::string lut_types;        // declarations of the packed entries
+  {
+    std::vector<Tab> wanted;
+    for (const Part &pt : parts) {
+      Tab *t = nullptr;
+      if (!getenv("POLY_HIP_NO_LUT_PACK"))
+        for (Tab &w : wanted) if (w.load == pt.load) t = &w;
+      if (!t) { wanted.push_back({pt.load, {}, ""}); t = &wanted.back(); }
+      t->nodes.push_back(pt.node);
+    }
+    for (Tab &t : wanted) {
+      // (fields by size, largest first: every one naturally aligned)
+      std::stable_sort(t.nodes.begin(), t.nodes.end(), [&](int x, int y) { return dt_size(g.n(x).dt) > dt_size(g.n(y).dt); });
+      Emitter et(g);
+      Scope St;
+      St.indent = 1;
+      et.preset(t.load, "x");
+      std::vector<std::string> vals;
+      size_t bytes = 0;
+      for (int node : t.nodes) { vals.push_back(et.emit(node, &St)); bytes += (size_t)dt_size(g.n(node).dt); }
+      if (et.failed() || et.uses_threefry) continue;
+      const DT idt = g.n(t.load).dt;
+      size_t entry = 2;
+      while (entry < bytes) entry *= 2;
+      std::string decl, stores;
+      if (t.nodes.size() == 1) {
+        t.type = dt_cname(g.n(t.nodes[0]).dt);
+        stores = strf("  out[i] = %s;\n", vals[0].c_str());
+      } else {
+        t.type = strf("poly_lutpack%zu_t", tabs.size());
+        decl = strf("struct __attribute__((aligned(%zu))) %s {", entry, t.type.c_str());
+        for (size_t j = 0; j < t.nodes.size(); j++) decl += strf(" %s v%zu;", dt_cname(g.n(t.nodes[j]).dt), j);
+        decl += " };\n";
+        // (the kernels take the table as a plain pointer: first stages share the signature without these declarations)
+        decl += strf("__device__ __forceinline__ %s poly_lutpack%zu_get(const void* __restrict__ t, unsigned short code) { return ((const %s*)t)[code]; }\n",
+                     t.type.c_str(), tabs.size(), t.type.c_str());
+        stores = strf("  %s e = {};\n", t.type.c_str());
+        for (size_t j = 0; j < t.nodes.size(); j++) stores += strf("  e.v%zu = %s;\n", j, vals[j].c_str());
+        stores += "  out[i] = e;\n";
+      }
+      RenderedKernel::Table rt;
+      rt.source = std::string(hip_prelude()) + decl +
+                  strf("extern \"C\" __global__ void __launch_bounds__(256) poly_lut_fill(%s* out) {\n"
+                       "  const unsigned int i = blockIdx.x * 256u + threadIdx.x;\n"
+                       "  const %s x = __builtin_bit_cast(%s, (unsigned short)i);\n",
+                       t.type.c_str(), dt_cname(idt), dt_cname(idt)) +
+                  St.code + stores + "}\n";
+      rt.entry = "poly_lut_fill";
+      rt.bytes = (size_t)65536 * (t.nodes.size() == 1 ? (size_t)dt_size(g.n(t.nodes[0]).dt) : entry);
+      rt.launch.grid[0] = 256;
+      rt.launch.block[0] = 256;
+      ep0.tables.push_back(rt);
+      lut_types += decl;
+      ep0.table_parts += (int)t.nodes.size();
+      tabs.push_back(t);
+    }
   }
   // (an emitter reads a table entry in place of the part: the load first, then the lookup)
   auto use_tables = [&](Emitter &e, Scope *S) {
-    for (size_t i = 0; i < lut_of.size(); i++) {
-      const std::string x = e.emit(lut_of[i].second, S);
-      e.preset(lut_of[i].first, strf("poly_lut%zu[__builtin_bit_cast(unsigned short, %s)]", i, x.c_str()));
+    for (size_t i = 0; i < tabs.size(); i++) {
+      const std::string x = e.emit(tabs[i].load, S);
+      if (tabs[i].nodes.size() == 1) e.preset(tabs[i].nodes[0], strf("poly_lut%zu[__builtin_bit_cast(unsigned short, %s)]", i, x.c_str()));
+      else
+        for (size_t j = 0; j < tabs[i].nodes.size(); j++)
+          e.preset(tabs[i].nodes[j], strf("poly_lutpack%zu_get(poly_lut%zu, __builtin_bit_cast(unsigned short, %s)).v%zu", i, i, x.c_str(), j));
     }
   };
   Emitter em(g);
@@ -440,11 +483,11 @@ static bool epilogue_from_graph(const KernelGraph &g, const MatmulMatch &mm, Mat
     params_call += strf("data%zu", i);
   }
   for (size_t i = 0; i < ep.tables.size(); i++) {
-    ep.signature += strf(", const %s* __restrict__ poly_lut%zu", dt_cname(g.n(lut_of[i].first).dt), i);
+    ep.signature += strf(", const %s* __restrict__ poly_lut%zu", tabs[i].nodes.size() == 1 ? tabs[i].type.c_str() : "void", i);
     params_call += strf(", poly_lut%zu", i);
   }
   ep.params_call = params_call;
-  ep.code = strf("__device__ __forceinline__ void poly_epilogue(float acc, int m, int n, int z, %s) {\n", ep.signature.c_str());
+  ep.code = lut_types + strf("__device__ __forceinline__ void poly_epilogue(float acc, int m, int n, int z, %s) {\n", ep.signature.c_str());
   ep.code += decomp + S0.code;
   ep.code += strf("  data%d[%s] = %s;\n}\n", pout, idx.c_str(), val.c_str());
   ep.call = strf("poly_epilogue(acc, m, n, z, %s)", params_call.c_str());
@@ -537,7 +580,7 @@ bool try_render_matmul(const KernelGraph &g, const std::string &fn, const Render
   if (!render_matmul(mm, ep, out)) return false;
   out->tables = ep.tables;
   if (!ep.tables.empty()) {
-    const std::string note = strf(", %zu parts of the epilogue as 16-bit lookup tables", ep.tables.size());
+    const std::string note = strf(", %d parts of the epilogue as 16-bit lookup tables (%zu, one per load)", ep.table_parts, ep.tables.size());
     out->strategy += note;
     for (RenderedKernel::Variant &v : out->variants) v.strategy += note;
   }
@@ -1658,7 +1701,7 @@ bool try_render_matmul_generic(const KernelGraph &g, const std::string &fn, cons
                              : in_place[0].ok && in_place[1].ok ? "; both read in place" : in_place[0].ok ? "; A read in place" : in_place[1].ok ? "; B read in place" : "") + out->strategy;
         out->narrow_loads = (in_place[0].ok && kind[0] == 2 ? 1 : 0) + (in_place[1].ok && kind[1] == 2 ? 1 : 0);
         out->tables = ep.tables;
-        if (!ep.tables.empty()) out->strategy += strf(", %zu parts of the epilogue as 16-bit lookup tables", ep.tables.size());
+        if (!ep.tables.empty()) out->strategy += strf(", %d parts of the epilogue as 16-bit lookup tables (%zu, one per load)", ep.table_parts, ep.tables.size());
         out->reads_planes_before = shared;
         if (!shared && !in_place[0].ok) out->a_planes = mine;
         for (RenderedKernel::Variant &v : out->variants) v.strategy = out->strategy;
@@ -1701,7 +1744,7 @@ bool try_render_matmul_generic(const KernelGraph &g, const std::string &fn, cons
     rk->flops = 2.0 * (double)M * (double)N * (double)K * (double)Z;
     rk->bytes = ep.bytes;
     rk->tables = ep.tables;
-    if (!ep.tables.empty()) rk->strategy += strf(", %zu parts of the epilogue as 16-bit lookup tables", ep.tables.size());
+    if (!ep.tables.empty()) rk->strategy += strf(", %d parts of the epilogue as 16-bit lookup tables (%zu, one per load)", ep.table_parts, ep.tables.size());
   };
   build(F32Shape{BM, BN, WVM, WVN}, out);
   f32_variants(M, N, F32Shape{BM, BN, WVM, WVN}, build, out);

@@ -72,6 +72,7 @@ struct MatmulEpilogue {
   // Lookup tables the epilogue reads (parameters `poly_lut<i>` at the end of `signature`,
   // in front of any scratch pointer), and the argument list that goes with `signature`.
   std::vector<RenderedKernel::Table> tables;
+  int table_parts = 0;     // parts of the epilogue that the tables stand for (parts of one load share a table)
   std::string params_call;
   // Operand B is a buffer that nothing in the plan writes (weights): at the time of the
   // launch it is in HBM, not in the caches.

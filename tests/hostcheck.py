@@ -115,9 +115,9 @@ def check_kernel(source, entry, grid, block, buf_sizes, block_stride=1, timeout=
     sanitizer's report on an out-of-bounds access."""
     types = _arg_types(source, entry)
     assert len(types) >= len(buf_sizes), (entry, types, buf_sizes)
-    # what follows the buffers: DEFINE_VAR ints (passed as 0) and lookup tables (65536 entries of at most 4 bytes)
+    # what follows the buffers: DEFINE_VAR ints (passed as 0) and lookup tables (65536 entries of at most 16 bytes)
     names = _arg_names(source, entry)
-    buf_sizes = list(buf_sizes) + [scratch_bytes if names[i] == "poly_scratch" else 65536 * 4
+    buf_sizes = list(buf_sizes) + [scratch_bytes if names[i] == "poly_scratch" else 65536 * 16
                                    for i, t in enumerate(types) if i >= len(buf_sizes) and "*" in t]
     args = ", ".join(f"({t})bufs[{i}]" if "*" in t else "0" for i, t in enumerate(types))
     tail = (DRIVER_TAIL.replace("GX", str(grid[0])).replace("GY", str(grid[1])).replace("GZ", str(grid[2]))

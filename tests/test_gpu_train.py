@@ -169,23 +169,32 @@ def test_epilogue_parts_of_one_16_bit_input_come_from_tables():
     """The backward product of the first MLP layer multiplies by the derivative of GELU at
     the saved bf16 pre-activation inside its epilogue; the parts of that expression that
     depend on the pre-activation alone are read from tables of 65 536 entries that the same
-    expression filled.  Bit for bit against the arithmetic (POLY_HIP_NO_LUT)."""
+    expression filled -- the three parts in one table whose entries hold all three values,
+    so that an element costs one gather.  Bit for bit against the arithmetic
+    (POLY_HIP_NO_LUT) and against a table per part (POLY_HIP_NO_LUT_PACK)."""
     import os
     B, T, D, H, V, lr = 1, 128, 128, 2, 97, 3e-4
     c = R.Ctx()
     bufs, sink = graphs.gpt2_block_train_step(c, B, T, D, H, V, lr=lr)
     arrays = graphs.gpt2_block_train_inputs(bufs, B, T, V)
     got, info = run_hip(c, sink, arrays)
-    assert any("parts of the epilogue as 16-bit lookup tables" in k["desc"] for k in info), [k["desc"] for k in info if "matmul" in k["desc"]]
+    assert any("3 parts of the epilogue as 16-bit lookup tables (1, one per load)" in k["desc"] for k in info), [k["desc"] for k in info if "matmul" in k["desc"]]
     os.environ["POLY_HIP_NO_LUT"] = "1"
     try:
         plain, info1 = run_hip(c, sink, arrays)
     finally:
         del os.environ["POLY_HIP_NO_LUT"]
+    os.environ["POLY_HIP_NO_LUT_PACK"] = "1"
+    try:
+        apart, info2 = run_hip(c, sink, arrays)
+    finally:
+        del os.environ["POLY_HIP_NO_LUT_PACK"]
     c.close()
     assert not any("lookup table" in k["desc"] for k in info1)
+    assert any("3 parts of the epilogue as 16-bit lookup tables (3, one per load)" in k["desc"] for k in info2)
     for name, t in bufs.items():
         assert got[t].tobytes() == plain[t].tobytes(), name
+        assert got[t].tobytes() == apart[t].tobytes(), name
 
 
 def test_ordered_column_sums_of_a_step_run_side_by_side():
