@@ -79,7 +79,43 @@ def huge_queries(names):
     w[:, 64 * 2:64 * 3].mul_(2e10)
 
 
-@pytest.mark.parametrize("tweak", [nothing, huge_keys, keys_not_finite, huge_queries], ids=lambda f: f.__name__)
+# The mask is data: the plan computes it as where(arange[i] < arange[j], -1e9, 0) from the
+# `arange` input (reference builder: gpt2.c:344-358), so other contents of that buffer give
+# other masks -- with the same plan, and the same inputs in both legs of the comparison.
+def mask_the_other_way(names):
+    """Keys BELOW the diagonal masked: the masked blocks of a query come before its live ones,
+    when it has no maximum yet."""
+    import torch
+    a = names["arange"]
+    a.copy_(torch.arange(a.numel() - 1, -1, -1, device=a.device).to(a.dtype))
+
+
+def mask_in_bands(names):
+    """arange in steps of 100 positions: a staircase whose tiles are mixed along every step,
+    blocks of 64 keys that are masked for some waves of a workgroup and live for others."""
+    import torch
+    a = names["arange"]
+    a.copy_((torch.arange(a.numel(), device=a.device) // 100).to(a.dtype))
+
+
+def mask_at_random(names):
+    """A random order of positions: hardly a tile with one value; with huge keys in one head."""
+    import torch
+    a = names["arange"]
+    g = torch.Generator(device=a.device)
+    g.manual_seed(5)
+    a.copy_(torch.randperm(a.numel(), generator=g, device=a.device).to(a.dtype))
+    w, _ = k_columns(names, 3, 1)
+    w.mul_(1e9)
+
+
+def no_mask(names):
+    """All positions equal: nothing is masked, every tile holds zeros."""
+    names["arange"].zero_()
+
+
+@pytest.mark.parametrize("tweak", [nothing, huge_keys, keys_not_finite, huge_queries, mask_the_other_way, mask_in_bands, mask_at_random, no_mask],
+                         ids=lambda f: f.__name__)
 def test_one_sequence_same_bits_with_and_without_key_bounds(tweak):
     import torch
     got = logits("gpt2_small_bf16_b1_t1024", tweak, True)
@@ -87,6 +123,9 @@ def test_one_sequence_same_bits_with_and_without_key_bounds(tweak):
     assert torch.equal(got.view(torch.int16), want.view(torch.int16))
     if tweak in (nothing, huge_keys):
         assert bool(torch.isfinite(got.float()).all())
+    if tweak in (mask_the_other_way, mask_in_bands, mask_at_random, no_mask):
+        # (the buffer does feed the mask: other logits than with the causal one)
+        assert not torch.equal(got.view(torch.int16), logits("gpt2_small_bf16_b1_t1024", nothing, True).view(torch.int16))
     if tweak is keys_not_finite:
         assert bool(torch.isnan(got.float()).any())
 
