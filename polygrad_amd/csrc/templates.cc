@@ -991,7 +991,15 @@ bool render_matmul(const MatmulMatch &mm, const MatmulEpilogue &ep, RenderedKern
     auto count = [&](int bm, int bn) { return ((M + bm - 1) / bm) * ((N + bn - 1) / bn) * Z * S; };   // workgroups of the launch
     const int64_t t = count(BM, BN);
     if (dma_for(BM, BN, &probe)) {
-      Dma p2{0, 0, 0, 0, 0}, p3{0, 0, 0, 0, 0};
+      Dma p2{0, 0, 0, 0, 0}, p3{0, 0, 0, 0, 0}, wide{64, 3, 1, 2, 4};
+      // Three quarters of a round of 128x256 tiles and more on a deep K, A along k and B along
+      // n (8192 x 768 x 3072 of the GPT-2 layer, 192 tiles): the tile stays, on 8 waves of
+      // 64x64 and three stages of 64, one workgroup per CU -- found by the tuner, inside the
+      // plan 43.5 -> 41.8 us against the 128x128 tiles below (step 3.22 -> 3.20 ms); at
+      // K = 768 the two are equal, with 128 tiles (4096 x 1024 x 4096) it loses by a third.
+      if (S == 1 && Z == 1 && BM == 128 && BN == 256 && t >= 192 && t <= 256 && a_kc && !b_kc && K >= 1536 && !getenv("POLY_HIP_NO_WIDE_SMALL_LAUNCH") &&
+          dma_for(128, 256, &wide)) { WVM = 2; WVN = 4; chosen = wide; }
+      else
       if (S == 1 && BM * BN == 128 * 256 && t <= 256 && M % 128 == 0 && dma_for(128, 128, &p2)) { BM = BN = 128; WVM = WVN = 2; }
       else if (S == 1 && BM * BN == 128 * 256 && t > 512 && t < 640 && N % 192 == 0 && count(128, 192) >= 768 && dma_for(128, 192, &p3)) { BM = 128; BN = 192; WVM = WVN = 2; }
       if (BM == 128 && BN == 128 && count(128, 128) <= 256) {
