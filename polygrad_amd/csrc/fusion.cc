@@ -1182,19 +1182,24 @@ static bool match_row_chain_impl(const Sched &sc, int a_item, const std::vector<
     }
     strat += strf("%s%s vec%d%s", pi ? ", " : "", ph.is_map ? "map" : "reduce", V, ragged ? " unaligned + tail" : "");
   }
-  std::string body = strf("extern \"C\" __global__ void __launch_bounds__(256) poly_k(%s) {\n", sig.c_str());
-  if (G == 64) {
-    body += "  const int lane = threadIdx.x & 63;\n  const long long row = (long long)blockIdx.x * 4 + (threadIdx.x >> 6);\n";
-    body += strf("  if (row < %lldll) {\n", (long long)rows);
-  } else if (G == 32) {
-    body += "  const int lane = threadIdx.x & 31;\n  const long long row = (long long)blockIdx.x * 8 + (threadIdx.x >> 5);\n";
-    body += strf("  if (row < %lldll) {\n", (long long)rows);
-  } else {
-    body += "  const int lane = threadIdx.x;\n  const long long row = blockIdx.x;\n  {\n";
-  }
-  for (size_t ci = 0; ci < cache.size(); ci++) body += strf("    %s c%zu[%d];\n", cache[ci].type.c_str(), ci, cache[ci].nit);
-  body += row_decls;
-  body += calls + "  }\n}\n";
+  // (threads: the workgroup's size; a row per wave or half wave means threads / G rows per workgroup)
+  auto body_for = [&](int threads) {
+    std::string b = strf("extern \"C\" __global__ void __launch_bounds__(%d) poly_k(%s) {\n", threads, sig.c_str());
+    if (G == 64) {
+      b += strf("  const int lane = threadIdx.x & 63;\n  const long long row = (long long)blockIdx.x * %d + (threadIdx.x >> 6);\n", threads / 64);
+      b += strf("  if (row < %lldll) {\n", (long long)rows);
+    } else if (G == 32) {
+      b += strf("  const int lane = threadIdx.x & 31;\n  const long long row = (long long)blockIdx.x * %d + (threadIdx.x >> 5);\n", threads / 32);
+      b += strf("  if (row < %lldll) {\n", (long long)rows);
+    } else {
+      b += "  const int lane = threadIdx.x;\n  const long long row = blockIdx.x;\n  {\n";
+    }
+    for (size_t ci = 0; ci < cache.size(); ci++) b += strf("    %s c%zu[%d];\n", cache[ci].type.c_str(), ci, cache[ci].nit);
+    b += row_decls;
+    b += calls + "  }\n}\n";
+    return b;
+  };
+  const std::string body = body_for(256);
 
   out->items = items;
   out->launch_item = last_item;
@@ -1222,6 +1227,20 @@ static bool match_row_chain_impl(const Sched &sc, int a_item, const std::vector<
   }
   rk.n_params = (int)arg_slots.size();
   rk.bytes = bytes - (narrow_stored ? (double)s->buf_slots[g_narrow_store_slot].nbytes / 2 : 0.0);      // (a buffer stored as bf16 values is half written)
+  // Candidates for on-device tuning: the same rows on smaller workgroups (fewer rows to a
+  // workgroup, more workgroups).  Which lanes add which elements of a row, and in what
+  // order, stays as it is -- the width of a row's group of lanes and of its loads would
+  // change that, so they are not candidates.
+  if (matmul_tuning_enabled() && G != 256) {
+    rk.variants.push_back({"default", rk.source, rk.strategy, rk.launch});
+    for (int threads : {128, 64}) {
+      LaunchSpec ls = rk.launch;
+      ls.grid[0] = (unsigned)std::ceil(rows / (double)(threads / G));
+      ls.block[0] = (unsigned)threads;
+      rk.variants.push_back({strf("rows_wg%d", threads), std::string(hip_prelude()) + code + body_for(threads),
+                             rk.strategy + strf(", workgroups of %d threads", threads), ls});
+    }
+  }
   return true;
 }
 

@@ -35,9 +35,10 @@ def known_label(l):
     """A decision names the winner: "256x256w4x2p2" (16-bit template that stages through
     registers), "128x256x32w2x2s3g2" (the one that loads straight into LDS), "f32_128x64w2x2"
     (fp32 template), "attn_occ2" (attention, waves per SIMD), "pw_vec2" (fused pointwise
-    kernels, elements per access), or keeps the default."""
+    kernels, elements per access), "rows_wg64" (row chains, threads per workgroup), or keeps
+    the default."""
     import re
-    return bool(re.fullmatch(r"default|\d+x\d+w\dx\dp\d|\d+x\d+x\d+w\dx\ds\dg\d|f32_\d+x\d+w\dx\d|attn_occ\d|pw_vec\d+", l))
+    return bool(re.fullmatch(r"default|\d+x\d+w\dx\dp\d|\d+x\d+x\d+w\dx\ds\dg\d|f32_\d+x\d+w\dx\d|attn_occ\d|pw_vec\d+|rows_wg\d+", l))
 
 
 @pytest.mark.parametrize("name,out_name", [("matmul_bf16_b16_1024x1024x1024", "C"), ("gpt2_small_bf16_b1_t1024", "output")])
@@ -56,8 +57,9 @@ def test_tuned_plan_is_bit_identical_and_remembered(name, out_name, tmp_path, mo
     decisions = [f for f in os.listdir(tmp_path / "cache") if f.endswith(".tune")]
     n_matmul_kinds = len({d.split(" ", 1)[1] for d in plain_descs if "matmul-mfma" in d})
     # (one decision per distinct set of candidates: every kind of matmul, and the attention
-    # and fused pointwise kernels, whose texts differ where their descriptions do not)
-    n_other = sum("attention" in d or "pointwise kernels over the same" in d for d in plain_descs)
+    # kernels, fused pointwise kernels and row chains, whose texts differ where their
+    # descriptions do not)
+    n_other = sum("attention" in d or "pointwise kernels over the same" in d or "row chain" in d for d in plain_descs)
     assert n_matmul_kinds <= len(decisions) <= n_matmul_kinds + n_other, (decisions, n_matmul_kinds, n_other)
     labels = {open(tmp_path / "cache" / f).read().strip() for f in decisions}
     assert all(known_label(l) for l in labels), labels

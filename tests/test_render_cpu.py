@@ -256,3 +256,21 @@ def test_tuning_candidates_render_and_compile(hiplib):
     shapes = set(re.findall(r"#define POLY_BM (\d+)\n#define POLY_BN (\d+)", tuned))
     assert shapes >= {("256", "256"), ("256", "128"), ("128", "256"), ("128", "128")}, shapes
     assert hiplib.poly_hip_compile_check(tuned.encode()) == 0
+    # a row chain (the LayerNorm of the GPT-2 plan) comes in smaller workgroups as well
+    gpt2 = PlanFile(os.path.join(ROOT, "polygrad_amd", "plans", "gpt2_small_bf16_b1_t1024.polyplan"))
+    os.environ["POLY_BEAM"] = "2"
+    try:
+        chains = []
+        for i in range(hiplib.poly_hip_fused_groups(gpt2.schedule, -1, None, None)):
+            src = C.c_void_p()
+            hiplib.poly_hip_fused_groups(gpt2.schedule, i, C.byref(src), None)
+            text = _ffi.take_string(src.value)
+            if "poly_row_p0" in text:
+                chains.append(text)
+    finally:
+        del os.environ["POLY_BEAM"]
+    assert chains and all(re.findall(r"// ---- variant (\S+)", t) == ["rows_wg128", "rows_wg64"] for t in chains)
+    units = chains[0].split("\n// ---- variant ")
+    assert "__launch_bounds__(256) poly_k" in units[0] and "__launch_bounds__(128) poly_k" in units[1] and "__launch_bounds__(64) poly_k" in units[2]
+    for u in units[1:]:
+        assert hiplib.poly_hip_compile_check(u[u.index("\n") + 1:].encode()) == 0
