@@ -394,13 +394,21 @@ static bool match_matmul_tail(const Sched &sc, int s_item, const std::vector<cha
   std::vector<Member> members;
   { Member m; m.item = s_item; m.rm = idS; members.push_back(m); }
   std::set<int> internal;
+  // One buffer on the way may have other readers than the chain (the pre-activation of a
+  // layer, which its backward pass reads much later): the launch then stores it as well.
+  int mid_slot = -1;
+  size_t mid_member = 0;      // the member whose store it is
   int cur = sc.slot(s_item, gS.param_slot(stS.param));
   while (members.size() < 4) {
-    if (!s->buf_slots[cur].is_intermediate || sc.writers[(size_t)cur].size() != 1 || sc.readers[(size_t)cur].size() != 1) break;
-    const int r = sc.readers[(size_t)cur][0];
+    if (!s->buf_slots[cur].is_intermediate || sc.writers[(size_t)cur].size() != 1 || sc.readers[(size_t)cur].empty()) break;
+    int r = sc.readers[(size_t)cur][0];
+    for (int o : sc.readers[(size_t)cur]) if (sc.step_of[(size_t)o] < sc.step_of[(size_t)r]) r = o;      // the first to read it
+    const bool shared = sc.readers[(size_t)cur].size() != 1;
+    if (shared && (mid_slot >= 0 || getenv("POLY_HIP_NO_STORED_MID"))) break;
     Member m;
     if (taken[(size_t)r] || !pointwise_member(sc, r, cur, aS, mext, "x", &m)) break;
-    internal.insert(cur);
+    if (shared) { mid_slot = cur; mid_member = members.size() - 1; }
+    else internal.insert(cur);
     members.push_back(m);
     const KernelGraph &g = sc.graphs[(size_t)r];
     cur = sc.slot(r, g.param_slot(g.stores[0].param));
@@ -410,11 +418,21 @@ static bool match_matmul_tail(const Sched &sc, int s_item, const std::vector<cha
   std::vector<int> items;
   for (const Member &m : members) items.push_back(m.item);
   std::set<int> inputs;
-  if (!group_is_schedulable(sc, items, s_item, last_item, internal, out_slot, &inputs)) FA_REJECT();
-  for (const Member &m : members) if (!internal_loads_replaced(sc, m, internal, -1)) FA_REJECT();
+  // (for the checks below the stored buffer counts as internal: members write and read it;
+  // what the others do with it is checked here)
+  std::set<int> inside = internal;
+  if (mid_slot >= 0) {
+    inside.insert(mid_slot);
+    if (mid_slot == out_slot) FA_REJECT();
+    for (int o : sc.readers[(size_t)mid_slot])
+      if (std::find(items.begin(), items.end(), o) == items.end() && sc.step_of[(size_t)o] <= sc.step_of[(size_t)last_item]) FA_REJECT();
+  }
+  if (!group_is_schedulable(sc, items, s_item, last_item, inside, out_slot, &inputs)) FA_REJECT();
+  for (const Member &m : members) if (!internal_loads_replaced(sc, m, inside, -1)) FA_REJECT();
 
   std::vector<int> arg_slots;
   arg_slots.push_back(out_slot);
+  if (mid_slot >= 0) arg_slots.push_back(mid_slot);
   for (int sl : inputs) arg_slots.push_back(sl);
   auto arg_of = [&](int sl) { return (int)(std::find(arg_slots.begin(), arg_slots.end(), sl) - arg_slots.begin()); };
   auto call_args = [&](int item) {
@@ -436,7 +454,7 @@ static bool match_matmul_tail(const Sched &sc, int s_item, const std::vector<cha
       if (p >= 0) dt = sc.graphs[(size_t)it].params[(size_t)p].dt;
     }
     if (j) ep.signature += ", ";
-    ep.signature += j == 0 ? strf("%s* fa%zu", dt_cname(dt), j) : strf("const %s* __restrict__ fa%zu", dt_cname(dt), j);
+    ep.signature += (j == 0 || arg_slots[j] == mid_slot) ? strf("%s* fa%zu", dt_cname(dt), j) : strf("const %s* __restrict__ fa%zu", dt_cname(dt), j);
     ep.bytes += (double)s->buf_slots[arg_slots[j]].nbytes;
   }
   const std::string master_decomp = matmul_decompose(mS, nullptr);
@@ -449,11 +467,14 @@ static bool match_matmul_tail(const Sched &sc, int s_item, const std::vector<cha
   std::map<size_t, std::string> lead_of, lut_arg_of, lookup_of;
   size_t win_bytes = 0;               // LDS windows of the tables so far
   bool windowed = false;              // some table takes bf16 codes: its lookups know the window
+  std::string mid_call;          // the value of the stored buffer on the way, in terms of acc
+  DT mid_dt = DT_VOID;
   for (size_t e = 1; e < members.size(); e++) {
     const Member &m = members[e];
     const KernelGraph &g = sc.graphs[(size_t)m.item];
     const bool last = e + 1 == members.size();
     const std::string fn = strf("poly_ep_e%zu", e);
+    if (mid_slot >= 0 && mid_member == e - 1) { mid_call = call; mid_dt = prev_dt; }
     std::string lead = strf("%s x", dt_cname(prev_dt));
     std::map<int, std::string> extra;
     RenderedKernel::Table tab;
@@ -529,9 +550,33 @@ static bool match_matmul_tail(const Sched &sc, int s_item, const std::vector<cha
         }
         ep.ptr_call = strf("poly_ep_ptr(m, n, z, %s)", call_args(m.item).c_str());
         ep.contiguous_n = true;
+        if (mid_slot >= 0) {
+          // the buffer stored on the way: same positions as the output (the same affine index
+          // in the product's ranges), its own element type
+          const Member &mm_ = members[mid_member];
+          const KernelGraph &gm = sc.graphs[(size_t)mm_.item];
+          const StoreInfo &sm = gm.stores[0];
+          const int lm = gm.n(gm.n(sm.index).src[1]).lin;
+          Aff am;
+          const bool same = mm_.range_expr.empty() && lm >= 0 && lin_to_aff(gm, gm.lins[(size_t)lm], mm_.rm, &am) && am == a &&
+                            gm.n(sm.value).dt == gm.n(sm.param).dt && gm.n(sm.value).dt == mid_dt && !mid_call.empty();
+          Emitter em2(gm);
+          Scope Sm;
+          Sm.indent = 1;
+          for (auto &kv : mm_.rm) { em2.bind_range(kv.first, strf("r%d", kv.second)); Sm.avail |= (uint64_t)1 << kv.first; }
+          const std::string midx = same ? em2.emit(gm.n(sm.index).src[1], &Sm) : std::string();
+          if (same && !em2.failed()) {
+            ep.mid_type = dt_cname(gm.n(sm.param).dt);
+            ep.code += strf("__device__ __forceinline__ %s* poly_ep_mid_ptr(int m, int n, int z, %s) {\n", ep.mid_type.c_str(), params_decl(gm).c_str());
+            ep.code += master_decomp + Sm.code + strf("  return data%d + %s;\n}\n", gm.param_slot(sm.param), midx.c_str());
+            ep.mid_value_call = mid_call;
+            ep.mid_ptr_call = strf("poly_ep_mid_ptr(m, n, z, %s)", call_args(mm_.item).c_str());
+          }
+        }
       }
     }
   }
+  if (mid_slot >= 0 && ep.mid_value_call.empty()) FA_REJECT();
   ep.a_ptr = strf("fa%d", arg_of(sc.slot(s_item, mS.A.param)));
   ep.b_ptr = strf("fa%d", arg_of(sc.slot(s_item, mS.B.param)));
   ep.n_params = (int)arg_slots.size();
@@ -568,6 +613,7 @@ static bool match_matmul_tail(const Sched &sc, int s_item, const std::vector<cha
   out->rk.tables = tables;
   std::string tail = strf(" + %zu pointwise kernel%s in the epilogue", members.size() - 1, members.size() > 2 ? "s" : "");
   if (!tables.empty()) tail += strf(" (%zu as a 16-bit lookup table)", tables.size());
+  if (mid_slot >= 0) tail += ", a value on the way stored as well";
   out->rk.strategy += tail;
   for (RenderedKernel::Variant &v : out->rk.variants) v.strategy += tail;
   out->items = items;

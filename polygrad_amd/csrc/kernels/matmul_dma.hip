@@ -26,6 +26,9 @@
 //                       into the first stage that the K loop no longer needs, during its
 //                       last iterations, so the window costs no LDS of its own
 //
+//   POLY_EP_MID_TYPE, POLY_EP_MID_VALUE(acc, m, n, z), POLY_EP_MID_PTR(m, n, z)
+//                       (optional, with POLY_EP_CONTIG) a second output with the layout of the
+//                       first: a value the epilogue passes through on its way, stored as well
 //   POLY_EP_BLOCKMAX_LO, POLY_EP_BLOCKMAX_HI, POLY_EP_BLOCKMAX_IDX(m, n), POLY_EP_BLOCKMAX_PTR
 //                       (optional, with POLY_EP_CONTIG and tiles of whole 64 x 64 blocks)
 //                       the columns [LO, HI) of the output, both multiples of 64, are read
@@ -559,6 +562,26 @@ extern "C" __global__ void __launch_bounds__(POLY_NTHREADS) POLY_WAVES_ATTR poly
             for (int e = 0; e < 8; e++)
               if (n + e < POLY_N) *POLY_EP_PTR(m, n + e, z) = o[e];
           }
+#ifdef POLY_EP_MID_VALUE
+          {
+            // a value on the way to the stored one that other kernels read as well: stored too
+            typedef POLY_EP_MID_TYPE poly_mid8 __attribute__((ext_vector_type(8)));
+            typedef poly_mid8 poly_mid8_u __attribute__((aligned(sizeof(POLY_EP_MID_TYPE))));
+            poly_mid8 mv;
+#pragma unroll
+            for (int e = 0; e < 8; e++) {
+              const int ne = (POLY_N % 8 == 0 || n + e < POLY_N) ? n + e : n;
+              mv[e] = POLY_EP_MID_VALUE(v[e], m, ne, z);
+            }
+            if (POLY_N % 8 == 0 || n + 7 < POLY_N) {
+              *(poly_mid8_u *)POLY_EP_MID_PTR(m, n, z) = mv;
+            } else {
+#pragma unroll
+              for (int e = 0; e < 8; e++)
+                if (n + e < POLY_N) *POLY_EP_MID_PTR(m, n + e, z) = mv[e];
+            }
+          }
+#endif
         }
 #else
         if (m < POLY_M && n < POLY_N) {

@@ -18,6 +18,10 @@
 //   POLY_EPILOGUE(acc, m, n, z)   stores one finished element (generated from the
 //                       UOps around the REDUCE: casts, bias, activation, index)
 //   POLY_KSPLIT         (optional) workgroups sharing the K tiles of one output tile
+//   POLY_EP_MID_TYPE, POLY_EP_MID_VALUE(acc, m, n, z), POLY_EP_MID_PTR(m, n, z)
+//                       (optional, with POLY_EP_CONTIG) a second output with the layout of the
+//                       first: a value the epilogue passes through on its way (the
+//                       pre-activation that a backward pass reads), stored as well
 //   POLY_EP_CONTIG      1 when consecutive n of a row are consecutive in memory; then
 //                       POLY_EP_TYPE, POLY_EP_VALUE(acc, m, n, z) and POLY_EP_PTR(m, n, z)
 //                       give the element type, value and address separately and the
@@ -577,6 +581,26 @@ extern "C" __global__ void __launch_bounds__(POLY_NTHREADS) poly_k(POLY_SIGNATUR
             for (int e = 0; e < 8; e++)
               if (n + e < POLY_N) *POLY_EP_PTR(m, n + e, z) = o[e];
           }
+#ifdef POLY_EP_MID_VALUE
+          {
+            // a value on the way to the stored one that other kernels read as well: stored too
+            typedef POLY_EP_MID_TYPE poly_mid8 __attribute__((ext_vector_type(8)));
+            typedef poly_mid8 poly_mid8_u __attribute__((aligned(sizeof(POLY_EP_MID_TYPE))));
+            poly_mid8 mv;
+#pragma unroll
+            for (int e = 0; e < 8; e++) {
+              const int ne = (POLY_N % 8 == 0 || n + e < POLY_N) ? n + e : n;
+              mv[e] = POLY_EP_MID_VALUE(v[e], m, ne, z);
+            }
+            if (POLY_N % 8 == 0 || n + 7 < POLY_N) {
+              *(poly_mid8_u *)POLY_EP_MID_PTR(m, n, z) = mv;
+            } else {
+#pragma unroll
+              for (int e = 0; e < 8; e++)
+                if (n + e < POLY_N) *POLY_EP_MID_PTR(m, n + e, z) = mv[e];
+            }
+          }
+#endif
         }
 #else
         if (m < POLY_M && n < POLY_N) {

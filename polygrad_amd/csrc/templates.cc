@@ -747,7 +747,7 @@ bool render_matmul(const MatmulMatch &mm, const MatmulEpilogue &ep, RenderedKern
   const KSplit &ka = mm.ka, &kb = mm.kb;
   const std::vector<Dim> &md = mm.md, &nd = mm.nd, &zd = mm.zd;
   if (M > 2147483647LL || N > 2147483647LL || Z > 65535) return reject(__LINE__);
-  if (A.dt == DT_F32) return render_matmul_f32(mm, ep, out);
+  if (A.dt == DT_F32) return ep.mid_value_call.empty() ? render_matmul_f32(mm, ep, out) : false;     // (no second output in the fp32 template)
   int BK = 64;
   if (const char *e = measurement_env("POLY_HIP_MM_BK")) BK = atoi(e) == 32 ? 32 : 64;
   // operand layout: contiguous along K, or along its row axis
@@ -944,6 +944,10 @@ bool render_matmul(const MatmulMatch &mm, const MatmulEpilogue &ep, RenderedKern
     cfg += strf("#define POLY_EPILOGUE(acc, m, n, z) %s\n", ep.call.c_str());
     const bool split = S == 1 && ep.contiguous_n && !measurement_env("POLY_HIP_MM_NOEPI") && (ep.out_type == "__bf16" || ep.out_type == "_Float16" || ep.out_type == "float");
     if (S == 1) cfg += strf("#define POLY_EP_CONTIG %d\n", split ? 1 : 0);
+    if (!ep.mid_value_call.empty() && !split) return false;      // (a second output only in the contiguous form)
+    if (split && !ep.mid_value_call.empty())
+      cfg += strf("#define POLY_EP_MID_TYPE %s\n#define POLY_EP_MID_VALUE(acc, m, n, z) %s\n#define POLY_EP_MID_PTR(m, n, z) %s\n", ep.mid_type.c_str(),
+                  ep.mid_value_call.c_str(), ep.mid_ptr_call.c_str());
     if (split) {
       cfg += strf("#define POLY_EP_TYPE %s\n", ep.out_type.c_str());
       cfg += strf("#define POLY_EP_VALUE(acc, m, n, z) %s\n", ep.value_call.c_str());

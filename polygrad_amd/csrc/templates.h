@@ -60,6 +60,10 @@ struct MatmulEpilogue {
   std::string value_call_win;   // the same value with table lookups served from LDS windows (sets poly_tmax), or empty
   std::string ptr_call;    // expression of type out_type*: uses m, n, z
   std::string out_type;
+  // A value the chain passes through that other kernels read as well (the pre-activation of
+  // a layer whose backward pass wants it): stored too, where the output is stored and with
+  // its layout (contiguous form only).  Value in terms of acc, m, n, z; address; element type.
+  std::string mid_value_call, mid_ptr_call, mid_type;
   bool out_16bit = false;  // the stored element is a 16-bit float, whatever the form of the store
   bool contiguous_n = false;
   int n_params = 0;

@@ -197,6 +197,30 @@ def test_epilogue_parts_of_one_16_bit_input_come_from_tables():
         assert got[t].tobytes() == apart[t].tobytes(), name
 
 
+def test_pre_activation_read_by_the_backward_pass_is_stored_by_the_product():
+    """The first MLP product's output (with its bias) feeds GELU and, much later, the backward
+    pass.  The product takes GELU into its epilogue all the same and stores both tensors --
+    the pre-activation where its own kernel would have, GELU's result where GELU's would --
+    instead of leaving GELU to a launch of its own that reads the pre-activation back.  Bit
+    for bit against the step with that launch (POLY_HIP_NO_STORED_MID)."""
+    import os
+    B, T, D, H, V, lr = 1, 128, 128, 2, 97, 3e-4
+    c = R.Ctx()
+    bufs, sink = graphs.gpt2_block_train_step(c, B, T, D, H, V, lr=lr)
+    arrays = graphs.gpt2_block_train_inputs(bufs, B, T, V)
+    got, info = run_hip(c, sink, arrays)
+    assert sum("a value on the way stored as well" in k["desc"] for k in info) == 1, [k["desc"] for k in info if "matmul" in k["desc"]]
+    os.environ["POLY_HIP_NO_STORED_MID"] = "1"
+    try:
+        apart, info1 = run_hip(c, sink, arrays)
+    finally:
+        del os.environ["POLY_HIP_NO_STORED_MID"]
+    c.close()
+    assert not any("stored as well" in k["desc"] for k in info1) and len(info1) == len(info) + 1
+    for name, t in bufs.items():
+        assert got[t].tobytes() == apart[t].tobytes(), name
+
+
 def test_ordered_column_sums_of_a_step_run_side_by_side():
     """The order-preserving bf16 column sums of the backward pass (bias and LayerNorm-parameter
     gradients: a terms kernel and an in-order adder each) that depend on nothing between
