@@ -637,6 +637,7 @@ struct RowPhase {
   Member m;
   bool is_map = false;
   bool keeps_row = false;           // a map whose output row only later phases read: kept in registers
+  bool is_copy = false;             // a kernel that copies the result before it, one value per row: another name for it
   int red = -1, own_red_ord = -1;   // REDUCE node and its range ordinal (reduce phases)
 };
 
@@ -770,7 +771,7 @@ static void collect_ref_loads(const Sched &sc, const Member &m, std::vector<std:
 // (set by find_fused_groups once it knows that the one reader of the buffer takes that)
 static thread_local int g_narrow_store_slot = -1;
 
-static bool match_row_chain_impl(const Sched &sc, int a_item, const std::vector<char> &taken, FusedGroup *out, bool allow_rows) {
+static bool match_row_chain_impl(const Sched &sc, int a_item, const std::vector<char> &taken, FusedGroup *out, bool allow_rows, bool allow_side = false) {
   const PolySchedule *s = sc.s;
   const KernelGraph &gA = sc.graphs[(size_t)a_item];
   auto reduce_shape = [&](const KernelGraph &g, int *red, int *ord) {
@@ -821,7 +822,7 @@ static bool match_row_chain_impl(const Sched &sc, int a_item, const std::vector<
   // grow: the readers of the latest result decide what comes next
   const bool exports_ok = !getenv("POLY_HIP_NO_ROW_CHAIN_EXPORTS");
   std::vector<char> row_result{0};   // per result: a whole row (kept in registers) instead of one value per row
-  int n_reduces = 1;
+  int n_reduces = 1, n_side = 0;
   for (;;) {
     const int cur = results.back().first;
     if (!s->buf_slots[cur].is_intermediate || sc.writers[(size_t)cur].size() != 1) return false;
@@ -855,6 +856,76 @@ static bool match_row_chain_impl(const Sched &sc, int a_item, const std::vector<
       continue;
     }
     if (next_reduce >= 0) return false;
+    // Side reductions.  The map may read one value per row that is a copy of the result of
+    // another reduction over the same rows, which reads nothing the chain makes (the
+    // derivative of a row maximum counts the elements equal to it: a reduction over the
+    // scores, whose row the chain holds anyway).  Such a reduction becomes a phase of its
+    // own in front of the map, and the copy another name for its result.
+    if (allow_side) {
+      const KernelGraph &gm = sc.graphs[(size_t)next_map];
+      const PolyExecItem &em_ = s->items[next_map];
+      for (int p = 0; p < em_.n_buf_slots && p < (int)gm.params.size() && phases.size() < 6; p++) {
+        const int sl = em_.buf_slot_indices[p];
+        if (gm.params[(size_t)p].written) continue;
+        bool known = false;
+        for (auto &rs : results) if (rs.first == sl) known = true;
+        if (known || !s->buf_slots[sl].is_intermediate || sc.writers[(size_t)sl].size() != 1 || sc.readers[(size_t)sl].size() != 1) continue;
+        const int w = sc.writers[(size_t)sl][0];
+        if (taken[(size_t)w] || sc.step_of[(size_t)w] <= sc.step_of[(size_t)a_item] || sc.step_of[(size_t)w] >= sc.step_of[(size_t)next_map]) continue;
+        // w: out[i] = in[i], nothing else
+        const KernelGraph &gw = sc.graphs[(size_t)w];
+        if (!gw.reduces.empty() || gw.stores.size() != 1 || gw.stores[0].gate >= 0 || !gw.vars.empty()) continue;
+        const KNode &cv = gw.n(gw.stores[0].value);
+        if (cv.op != POLY_OP_LOAD || cv.guard >= 0 || cv.dt != gw.n(gw.stores[0].param).dt) continue;
+        const KNode &cix = gw.n(cv.src[0]);
+        if (cix.src.size() != 2) continue;
+        const int l_ld = gw.n(cix.src[1]).lin, l_st = gw.n(gw.n(gw.stores[0].index).src[1]).lin;
+        RangeMap idw;
+        for (int r : gw.stores[0].ranges) idw[r] = r;
+        Aff a_ld, a_st;
+        if (l_ld < 0 || l_st < 0 || !lin_to_aff(gw, gw.lins[(size_t)l_ld], idw, &a_ld) || !lin_to_aff(gw, gw.lins[(size_t)l_st], idw, &a_st) || !(a_ld == a_st)) continue;
+        const int src = sc.slot(w, gw.param_slot(cix.src[0]));
+        if (!s->buf_slots[src].is_intermediate || sc.writers[(size_t)src].size() != 1 || sc.readers[(size_t)src].size() != 1 ||
+            s->buf_slots[src].numel != s->buf_slots[sl].numel) continue;
+        const int q = sc.writers[(size_t)src][0];
+        if (taken[(size_t)q] || sc.step_of[(size_t)q] <= sc.step_of[(size_t)a_item] || sc.step_of[(size_t)q] >= sc.step_of[(size_t)w]) continue;
+        RowPhase B;
+        const KernelGraph &gq = sc.graphs[(size_t)q];
+        if (!reduce_shape(gq, &B.red, &B.own_red_ord) || gq.ranges[(size_t)B.own_red_ord].extent != R) continue;
+        // (it reads nothing that a kernel of the chain writes, earlier results aside: map_phase names those)
+        bool independent = true;
+        for (int pi2 = 0; pi2 < s->items[q].n_buf_slots; pi2++) {
+          const int qs = s->items[q].buf_slot_indices[pi2];
+          bool is_res = false;
+          for (auto &rs : results) if (rs.first == qs) is_res = true;
+          if (is_res && qs != results[0].first) independent = false;     // (only the first result, a value per row, may feed it)
+        }
+        if (!independent) continue;
+        if (!map_phase(sc, q, mext, ref_loads, results, names, &B.m)) continue;
+        if (!B.m.rm.count(B.own_red_ord) || B.m.rm[B.own_red_ord] != red_master) continue;
+        bool mapped = true;
+        for (int r : gq.stores[0].ranges) if (!B.m.rm.count(r)) mapped = false;
+        Aff qa;
+        if (!mapped || !store_aff(B.m, &qa)) continue;
+        phases.push_back(B);
+        results.push_back({src, qa});
+        row_result.push_back(0);
+        names.push_back(strf("s%zu", results.size()));
+        internal.insert(src);
+        collect_ref_loads(sc, B.m, &ref_loads);
+        RowPhase Cp;
+        Cp.is_copy = true;
+        Cp.m.item = w;
+        for (int id = 0; id < (int)gw.nodes.size(); id++)
+          if (gw.n(id).op == POLY_OP_LOAD) Cp.m.preset[id] = names.back();
+        phases.push_back(Cp);
+        results.push_back({sl, qa});
+        row_result.push_back(0);
+        names.push_back(names.back());
+        internal.insert(sl);
+        n_side++;
+      }
+    }
     RowPhase C;
     C.is_map = true;
     const KernelGraph &g = sc.graphs[(size_t)next_map];
@@ -901,6 +972,7 @@ static bool match_row_chain_impl(const Sched &sc, int a_item, const std::vector<
       collect_ref_loads(sc, C.m, &ref_loads);
       continue;
     }
+    if (allow_side && n_side == 0) return false;      // (this attempt is for chains with side reductions; the plain ones follow)
     phases.push_back(C);
     break;
   }
@@ -997,6 +1069,7 @@ static bool match_row_chain_impl(const Sched &sc, int a_item, const std::vector<
   std::string row_decls;             // their declarations in the kernel body
   for (size_t pi = 0; pi < phases.size(); pi++) {
     const RowPhase &ph = phases[pi];
+    if (ph.is_copy) continue;        // (its value is the result before it, under the same name)
     const KernelGraph &g = sc.graphs[(size_t)ph.m.item];
     Emitter em(g);
     em.recip_div16 = true;
@@ -1292,7 +1365,9 @@ static bool match_row_chain_impl(const Sched &sc, int a_item, const std::vector<
 
 static bool match_row_chain(const Sched &sc, int a_item, const std::vector<char> &taken, FusedGroup *out) {
   fa_item = a_item;
-  // first with maps in the middle of the chain (their rows kept in registers), then the plain form
+  // first with side reductions, then with maps in the middle of the chain (their rows kept in
+  // registers), then the plain form
+  if (!getenv("POLY_HIP_NO_SIDE_REDUCE") && match_row_chain_impl(sc, a_item, taken, out, true, true)) return true;
   return match_row_chain_impl(sc, a_item, taken, out, true) || match_row_chain_impl(sc, a_item, taken, out, false);
 }
 
