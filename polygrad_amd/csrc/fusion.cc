@@ -1061,7 +1061,7 @@ static bool match_row_chain_impl(const Sched &sc, int a_item, const std::vector<
   // Short rows handled by one wave stay in registers between the phases: a vector load
   // that an earlier phase made from the same buffer at the same index is kept instead of
   // being repeated (the row is then read from memory once, not once per phase).
-  struct RowCache { std::string key, type; int nit; };
+  struct RowCache { std::string key, type; int nit; int V = 0; std::string what; };    // what: the key without the vector width
   std::vector<RowCache> cache;
   int n_cached_uses = 0, n_exported = 0;
   bool narrow_stored = false;
@@ -1102,6 +1102,21 @@ static bool match_row_chain_impl(const Sched &sc, int a_item, const std::vector<
       for (auto &kv : ph.m.preset) if (kv.second.find("[it]") != std::string::npos) reads_row = true;
       if (reads_row) V = row_V;   // positions must line up with the phase that made the row
       while (V > 1 && (R % V != 0 || R < (int64_t)G * V)) V /= 2;
+      // a reduction whose row an earlier phase keeps in narrower vectors walks it that way
+      // too, and takes the kept registers instead of reading the row again
+      if (!reads_row && !ph.is_map && !ph.keeps_row && V > 1) {
+        int kept = 0;
+        for (int i = 0; i < (int)g.nodes.size() && !kept; i++) {
+          if (!mark[(size_t)i] || g.n(i).op != POLY_OP_LOAD || ph.m.preset.count(i) || !(g.n(i).deps & ((uint64_t)1 << own_f))) continue;
+          const KNode &ix = g.n(g.n(i).src[0]);
+          Aff a;
+          if (ix.src.size() != 2 || g.n(ix.src[1]).lin < 0 || !lin_to_aff(g, g.lins[(size_t)g.n(ix.src[1]).lin], ph.m.rm, &a)) continue;
+          std::string what = strf("%d:%d:%lld", sc.slot(ph.m.item, g.param_slot(ix.src[0])), (int)g.n(i).dt, (long long)a.c0);
+          for (auto &kv : a.c) what += strf(",%d*%lld", kv.first, (long long)kv.second);
+          for (const RowCache &c : cache) if (c.what == what && c.V > 1 && c.V < V) kept = c.V;
+        }
+        if (kept) V = kept;
+      }
       // a row that half the vector width deals out evenly (768 = 3 x 64 x 4, against one
       // and a half steps of 64 x 8) is walked that way: no step with half the lanes idle
       // (LayerNorm of 8192 x 768: 12.3 -> 11.2 us)
@@ -1151,7 +1166,11 @@ static bool match_row_chain_impl(const Sched &sc, int a_item, const std::vector<
       for (size_t ci = 0; ci < cache.size(); ci++)
         if (cache[ci].key == key && cache[ci].nit == nit) { n_cached_uses++; return strf("c%zu[it]", ci); }
       if (pi + 1 == phases.size()) return ld;   // nobody comes after the last phase
-      cache.push_back({key, strf("poly_vec<%s,%d>", dt_cname(g.n(node).dt), V), nit});
+      {
+        std::string what = strf("%d:%d:%lld", sc.slot(ph.m.item, g.param_slot(ix.src[0])), (int)g.n(node).dt, (long long)a.c0);
+        for (auto &kv : a.c) what += strf(",%d*%lld", kv.first, (long long)kv.second);
+        cache.push_back({key, strf("poly_vec<%s,%d>", dt_cname(g.n(node).dt), V), nit, V, what});
+      }
       return strf("(c%zu[it] = %s)", cache.size() - 1, ld.c_str());
     };
     if (ragged && unrolled) FA_REJECT();
