@@ -28,11 +28,23 @@ typedef _Float16 poly_f16x4 __attribute__((ext_vector_type(4)));
 typedef _Float16 poly_f16x2 __attribute__((ext_vector_type(2)));
 
 template <typename T, int N> struct poly_vec { T v[N]; };
+// A kernel that streams through more data than the caches hold reads it with the
+// nontemporal hint (POLY_NT_LOADS, defined in front of this text for such a kernel), so
+// that what it reads once does not push out what it, or the next kernel, reads again.
+#ifdef POLY_NT_LOADS
+#define POLY_LD(...) __builtin_nontemporal_load(&(__VA_ARGS__))
+#else
+#define POLY_LD(...) (__VA_ARGS__)
+#endif
 template <typename T, int N>
 __device__ __forceinline__ poly_vec<T, N> poly_vload(const T *p) {
   typedef T vt __attribute__((ext_vector_type(N)));
   typedef vt uvt __attribute__((aligned(sizeof(T))));
+#ifdef POLY_NT_LOADS
+  vt x = __builtin_nontemporal_load((const uvt *)p);
+#else
   vt x = *(const uvt *)p;
+#endif
   poly_vec<T, N> r;
 #pragma unroll
   for (int i = 0; i < N; i++) r.v[i] = x[i];
@@ -45,7 +57,11 @@ __device__ __forceinline__ void poly_vstore(T *p, const poly_vec<T, N> &r) {
   vt x;
 #pragma unroll
   for (int i = 0; i < N; i++) x[i] = r.v[i];
+#ifdef POLY_NT_STORES
+  __builtin_nontemporal_store(x, (uvt *)p);
+#else
   *(uvt *)p = x;
+#endif
 }
 
 // ── wave64 reductions: DPP inside a row of 16 lanes, ds_swizzle across rows of
@@ -244,7 +260,7 @@ std::string Emitter::load_expr(int id, Scope *s) {
   const KNode &ix = g_.n(k.src[0]);
   int p = g_.param_slot(ix.src[0]);
   std::string idx = emit(ix.src[1], s);
-  std::string e = strf("data%d[%s]", p, idx.c_str());
+  std::string e = strf("POLY_LD(data%d[%s])", p, idx.c_str());
   std::string gate;
   if (ix.src.size() >= 3) gate = emit(ix.src[2], s);
   if (k.guard >= 0) {

@@ -1027,7 +1027,7 @@ static bool match_row_chain_impl(const Sched &sc, int a_item, const std::vector<
     return c;
   };
   std::string sig;
-  double bytes = 0;
+  double bytes = 0, bytes_written = 0;
   for (size_t j = 0; j < arg_slots.size(); j++) {
     DT dt = DT_VOID;
     for (int it : items) {
@@ -1037,6 +1037,7 @@ static bool match_row_chain_impl(const Sched &sc, int a_item, const std::vector<
     if (j) sig += ", ";
     sig += j == 0 || exported.count(arg_slots[j]) ? strf("%s* fa%zu", dt_cname(dt), j) : strf("const %s* __restrict__ fa%zu", dt_cname(dt), j);
     bytes += (double)s->buf_slots[arg_slots[j]].nbytes;
+    if (j == 0 || exported.count(arg_slots[j])) bytes_written += (double)s->buf_slots[arg_slots[j]].nbytes;
   }
   // master row decomposition: fastest row range = smallest stride in the first result
   std::string row_decomp;
@@ -1365,6 +1366,7 @@ static bool match_row_chain_impl(const Sched &sc, int a_item, const std::vector<
   }
   rk.n_params = (int)arg_slots.size();
   rk.bytes = bytes - (narrow_stored ? (double)s->buf_slots[g_narrow_store_slot].nbytes / 2 : 0.0);      // (a buffer stored as bf16 values is half written)
+  rk.bytes_written = bytes_written - (narrow_stored ? (double)s->buf_slots[g_narrow_store_slot].nbytes / 2 : 0.0);
   // Candidates for on-device tuning: the same rows on smaller workgroups (fewer rows to a
   // workgroup, more workgroups).  Which lanes add which elements of a row, and in what
   // order, stays as it is -- the width of a row's group of lanes and of its loads would
@@ -2321,7 +2323,7 @@ static bool match_pointwise_group(const Sched &sc, int a_item, const std::vector
   std::string code, body;
   std::map<int, std::string> value_of_slot;   // what the group has stored so far, by slot
   std::set<int> read_from_memory;
-  double bytes = 0;
+  double bytes = 0, bytes_written = 0;
   for (size_t mi = 0; mi < members.size(); mi++) {
     const Pw &pw = members[mi];
     const KernelGraph &g = sc.graphs[(size_t)pw.item];
@@ -2367,6 +2369,7 @@ static bool match_pointwise_group(const Sched &sc, int a_item, const std::vector
     else sig += strf("const %s* __restrict__ fa%zu", dt_cname(slot_dt[sl]), j);
     // (a buffer updated in place moves twice: in and out)
     bytes += (double)s->buf_slots[sl].nbytes * ((read_from_memory.count(sl) ? 1 : 0) + (written.count(sl) ? 1 : 0));
+    if (written.count(sl)) bytes_written += (double)s->buf_slots[sl].nbytes;
   }
   // the kernel for V positions per thread (the members themselves are per position)
   const auto kernel_for = [&](int V) {
@@ -2407,6 +2410,7 @@ static bool match_pointwise_group(const Sched &sc, int a_item, const std::vector
   rk.n_params = (int)arg_slots.size();
   rk.n_vars = 0;
   rk.bytes = bytes;
+  rk.bytes_written = bytes_written;
   rk.flops = 0;
   if (matmul_tuning_enabled()) {
     // other widths of a thread's accesses: candidates of the search that POLY_BEAM switches on

@@ -997,13 +997,15 @@ class Generic {
       }
     }
     for (const StoreInfo &st : g_.stores) touched[(size_t)g_.param_slot(st.param)] += distinct(g_.n(st.index).src[1]);
-    double bytes = 0;
+    double bytes = 0, stored = 0;
     for (size_t i = 0; i < g_.params.size(); i++) {
       double n = touched[i];
       if (g_.params[i].numel > 0) n = std::min(n, (double)g_.params[i].numel * ((g_.params[i].read && g_.params[i].written) ? 2 : 1));
       bytes += n * dt_size(g_.params[i].dt);
+      if (g_.params[i].written) stored += (g_.params[i].read ? n / 2 : n) * dt_size(g_.params[i].dt);
     }
     out->bytes = bytes;
+    out->bytes_written = stored;
   }
 };
 

@@ -101,6 +101,22 @@ def test_rowops_layernorm_full_size(rowops_inputs):
     assert float((got - want).abs().max()) < 1e-4
 
 
+@pytest.mark.parametrize("kind", ["softmax", "sum"])
+def test_streaming_hints_change_no_bit(rowops_inputs, kind, monkeypatch):
+    """A row kernel over 1 GiB of operands reads them with the nontemporal hint (a kernel that
+    moves more than the 256 MiB memory-side cache holds and reads nothing twice); the hint
+    is about where the lines are kept, so the result is that of plain loads bit for bit."""
+    import torch
+    inputs, _ = rowops_inputs
+    hinted, info = run_rowop(kind, inputs)
+    assert any("streaming loads" in k["desc"] for k in info), [k["desc"] for k in info]
+    monkeypatch.setenv("POLY_HIP_NO_STREAMING_HINTS", "1")
+    plain, info = run_rowop(kind, inputs)
+    assert not any("streaming" in k["desc"] for k in info), [k["desc"] for k in info]
+    assert bool(torch.isfinite(hinted).all())
+    assert torch.equal(hinted.view(torch.int32), plain.view(torch.int32))
+
+
 # ── config 3: bf16 matmul sweep at full size ─────────────────────────────────────────────
 
 SWEEP = [("matmul_bf16_4096x4096x4096", 4096, 4096, 4096, False, None),
