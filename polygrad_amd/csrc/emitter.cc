@@ -11,6 +11,7 @@
 #include <cstring>
 
 #include "render_hip.h"
+#include <functional>
 
 namespace polyhip {
 
@@ -62,6 +63,25 @@ __device__ __forceinline__ void poly_vstore(T *p, const poly_vec<T, N> &r) {
 #else
   *(uvt *)p = x;
 #endif
+}
+
+// x / d where many dividends share one divisor (a row's sum, a row's deviation): r = 1 / d
+// and `ok` (d finite and between 2^-100 and 2^100 in magnitude) are computed once per
+// divisor.  q = x r is within a unit or two of the quotient, the remainder x - q d is exact
+// in one fused multiply-add, and q + (x - q d) r is the correctly rounded quotient -- the
+// value x / d has -- whenever the remainder is representable, i.e. for |x| >= 2^-102
+// (checked on the host against x / d over all exponents and the awkward significands;
+// below that the result is within one unit in the last place, of a subnormal result:
+// 2^-149).  v_div_fixup gives a zero dividend the sign the quotient has.  Dividends beyond
+// 2^26, non-finite ones and every dividend of a divisor outside the range take the full
+// division.  Four instructions instead of eleven per quotient.
+__device__ __forceinline__ float poly_div_shared(float x, float d, float r, bool ok) {
+  if (ok && __builtin_fabsf(x) <= 0x1p+26f) {
+    const float q = x * r;
+    const float e = __builtin_fmaf(-q, d, x);
+    return __builtin_amdgcn_div_fixupf(__builtin_fmaf(e, r, q), d, x);
+  }
+  return x / d;
 }
 
 // ── wave64 reductions: DPP inside a row of 16 lanes, ds_swizzle across rows of
@@ -253,6 +273,48 @@ std::string Emitter::emit_lin(const Lin &l, Scope *s) {
   if (l.c0 > 0) e += strf("+%lld", (long long)l.c0);
   else if (l.c0 < 0) e += strf("%lld", (long long)l.c0);
   return "(" + e + ")";
+}
+
+// num / den in fp32 where den is shared by many values of num (it varies in fewer loops, or
+// is computed from per-row results alone): poly_div_shared with the reciprocal of den placed
+// where den is computed.  False when the division is not of that kind.
+bool Emitter::shared_division(DT dt, int num, int den, Scope *t, std::string *e) {
+  if (!shared_divisor || dt != DT_F32 || g_.n(num).dt != DT_F32 || g_.n(den).dt != DT_F32) return false;
+  const bool fewer_loops = (g_.n(den).deps & ~g_.n(num).deps) == 0 && g_.n(den).deps != g_.n(num).deps;
+  // (a divisor computed from shared presets and constants alone is as shared as they are)
+  std::function<bool(int, int)> from_shared = [&](int n, int depth) -> bool {
+    if (is_shared_preset(n)) return true;
+    if (is_preset(n) || depth > 16) return false;
+    const KNode &q = g_.n(n);
+    if (q.op == POLY_OP_CONST) return true;
+    if (q.op == POLY_OP_LOAD || q.op == POLY_OP_RANGE || q.op == POLY_OP_REDUCE || q.op == POLY_OP_DEFINE_VAR || q.src.empty()) return false;
+    for (int sN : q.src) if (!from_shared(sN, depth + 1)) return false;
+    return true;
+  };
+  const bool row_value = !shared_presets_.empty() && g_.n(den).op != POLY_OP_CONST && from_shared(den, 0) && !from_shared(num, 0);
+  if (!fewer_loops && !row_value) return false;
+  Scope *td = place(g_.n(den).deps, t);
+  if (row_value) while (td->parent) td = td->parent;
+  if (td == t) return false;
+  const int key = -2 - den, key_ok = -1000000 - den;
+  const std::string dv = emit(den, td);
+  std::string rc, ok;
+  auto f = td->names.find(key);
+  if (f != td->names.end()) rc = f->second;
+  else {
+    rc = strf("rcp%d", den);
+    stmt(td, strf("const float %s = 1.0f / %s;", rc.c_str(), dv.c_str()));
+    td->names[key] = rc;
+  }
+  auto fo = td->names.find(key_ok);
+  if (fo != td->names.end()) ok = fo->second;
+  else {
+    ok = strf("rok%d", den);
+    stmt(td, strf("const bool %s = __builtin_fabsf(%s) >= 0x1p-100f && __builtin_fabsf(%s) <= 0x1p+100f;", ok.c_str(), dv.c_str(), dv.c_str()));
+    td->names[key_ok] = ok;
+  }
+  *e = strf("poly_div_shared(%s, %s, %s, %s)", emit(num, t).c_str(), dv.c_str(), rc.c_str(), ok.c_str());
+  return true;
 }
 
 std::string Emitter::load_expr(int id, Scope *s) {
@@ -462,13 +524,15 @@ std::string Emitter::emit_raw(int id, Scope *s) {
       // (src/codegen.c:1867-1883; the reciprocal must be the second factor)
       const KNode &rb = g_.n(k.src[1]);
       if (dt_is_float(k.dt) && rb.op == POLY_OP_RECIPROCAL && rb.src.size() == 1) {
-        e = strf("(%s/%s)", S(0).c_str(), emit(rb.src[0], t).c_str());
+        if (is_preset(k.src[1]) || !shared_division(k.dt, k.src[0], rb.src[0], t, &e)) e = strf("(%s/%s)", S(0).c_str(), emit(rb.src[0], t).c_str());
         break;
       }
       e = strf("(%s*%s)", S(0).c_str(), S(1).c_str());
       break;
     }
-    case POLY_OP_FDIV: e = strf("(%s/%s)", S(0).c_str(), S(1).c_str()); break;
+    case POLY_OP_FDIV:
+      if (!shared_division(k.dt, k.src[0], k.src[1], t, &e)) e = strf("(%s/%s)", S(0).c_str(), S(1).c_str());
+      break;
     case POLY_OP_IDIV: e = strf("(%s/%s)", S(0).c_str(), S(1).c_str()); break;
     case POLY_OP_MOD: e = strf("(%s%%%s)", S(0).c_str(), S(1).c_str()); break;
     case POLY_OP_SHL: e = strf("(%s<<%s)", S(0).c_str(), S(1).c_str()); break;

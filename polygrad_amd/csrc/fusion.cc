@@ -1085,7 +1085,11 @@ static bool match_row_chain_impl(const Sched &sc, int a_item, const std::vector<
     std::string flat_base;           // flat phase: position of the row's first element
     for (auto &kv : ph.m.range_expr) { own_f = kv.first; flat_base = kv.second; }
     if (own_f < 0) FA_REJECT();
-    for (auto &kv : ph.m.preset) em.preset(kv.first, kv.second);
+    for (auto &kv : ph.m.preset) {
+      em.preset(kv.first, kv.second);
+      // (the results of earlier phases, s<n>, are one value per row)
+      if (kv.second.size() > 1 && kv.second[0] == 's' && kv.second.find_first_not_of("0123456789", 1) == std::string::npos) em.preset_shared(kv.first);
+    }
     const std::vector<int> roots{ph.is_map ? g.stores[0].value : g.n(ph.red).src[0]};
     // vector width along the row
     int V = 1;

@@ -6,6 +6,8 @@
 // per row with DPP/ds_swizzle wave reductions, and matmul-shaped reductions are
 // handed to the MFMA template.
 #pragma once
+#include <algorithm>
+#include <cstdlib>
 #include <functional>
 #include <string>
 #include <unordered_map>
@@ -182,6 +184,10 @@ class Emitter {
   void preset(int node, const std::string &expr) { preset_[node] = expr; }
   void clear_preset(int node) { preset_.erase(node); }
   bool is_preset(int node) const { return preset_.count(node) != 0; }
+  // a preset that holds one value for all positions the emitted code walks (a row's sum in
+  // a kernel that walks the row): what divides by it shares its reciprocal
+  void preset_shared(int node) { shared_presets_.push_back(node); }
+  bool is_shared_preset(int node) const { return std::find(shared_presets_.begin(), shared_presets_.end(), node) != shared_presets_.end(); }
   // Replaces the serial loop of a REDUCE node by caller-generated code; the
   // callback receives the scope the value is placed in and returns its C name.
   void custom_reduce(int node, std::function<std::string(Scope *)> fn) { custom_[node] = std::move(fn); }
@@ -211,8 +217,12 @@ class Emitter {
   // computed (outside the loops b does not depend on): the fp32 quotient may differ in its
   // last bit, which the 16-bit rounding hides except at rounding ties.
   bool recip_div16 = false;
+  // a / b in fp32 where b varies in fewer loops than a: poly_div_shared with the reciprocal
+  // of b placed where b is computed (the same quotient, four instructions instead of eleven)
+  bool shared_divisor = getenv("POLY_HIP_NO_SHARED_DIVISOR") == nullptr;
 
  private:
+  bool shared_division(DT dt, int num, int den, Scope *t, std::string *e);
   std::string emit_atom(int atom, Scope *s);
   bool light_body(int root, int ord) const;
   std::string emit_raw(int node, Scope *s);
@@ -220,6 +230,7 @@ class Emitter {
   const KernelGraph &g_;
   std::unordered_map<int, std::string> range_name_;
   std::unordered_map<int, std::string> preset_;
+  std::vector<int> shared_presets_;
   std::unordered_map<int, std::function<std::string(Scope *)>> custom_;
   int slice_node_ = -1, slice_ord_ = -1, slice_step_ = 1;
   std::string slice_first_;

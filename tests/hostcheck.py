@@ -45,6 +45,7 @@ static poly_dim3 threadIdx, blockIdx, blockDim, gridDim;
 #define __builtin_amdgcn_wave_barrier() ((void)0)
 #define __builtin_amdgcn_sched_barrier(m) ((void)0)
 #define __builtin_amdgcn_exp2f(x) exp2f(x)
+#define __builtin_amdgcn_div_fixupf(q, d, x) (q)
 template <class T> static T atomicAdd(T *p, T v) { T old = *p; *p += v; return old; }
 template <class T> static T atomicMax(T *p, T v) { T old = *p; if (old < v) *p = v; return old; }
 #define __builtin_amdgcn_mfma_f32_32x32x16_bf16(a, b, c, x, y, z) (c)

@@ -117,6 +117,21 @@ def test_streaming_hints_change_no_bit(rowops_inputs, kind, monkeypatch):
     assert torch.equal(hinted.view(torch.int32), plain.view(torch.int32))
 
 
+@pytest.mark.parametrize("kind", ["softmax", "layernorm"])
+def test_division_by_a_row_value_changes_no_bit(rowops_inputs, kind, monkeypatch):
+    """The last phase of these chains divides every element of a row by one value of the row
+    (the sum of the terms, the deviation); the generated code multiplies by that value's
+    reciprocal and corrects once with the exact remainder, which is the correctly rounded
+    quotient: the same bits as with the division itself."""
+    import torch
+    inputs, _ = rowops_inputs
+    shared, _ = run_rowop(kind, inputs)
+    monkeypatch.setenv("POLY_HIP_NO_SHARED_DIVISOR", "1")
+    divided, _ = run_rowop(kind, inputs)
+    assert bool(torch.isfinite(shared).all())
+    assert torch.equal(shared.view(torch.int32), divided.view(torch.int32))
+
+
 # ── config 3: bf16 matmul sweep at full size ─────────────────────────────────────────────
 
 SWEEP = [("matmul_bf16_4096x4096x4096", 4096, 4096, 4096, False, None),
