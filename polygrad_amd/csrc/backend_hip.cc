@@ -83,12 +83,16 @@ HipRunner *runner_create(const PolyUOp *root, const char *fn_name, int flags) {
 // the memory system serves the reads at a higher rate (three 256 MiB inputs and one output
 // of that size: 5.3 -> 6.3 TB/s; read-only rows: 6.1 -> 6.9 TB/s).  Its stores get the hint
 // too where the output alone exceeds that cache, so none of it could be found there by a
-// later kernel anyway (the AdamW update: 6.1 -> 6.4 TB/s).  Matmul, attention, gather and
+// later kernel anyway (the AdamW update: 6.1 -> 6.4 TB/s).  A kernel that reads its input
+// a second time keeps plain accesses.  Matmul, attention, gather and
 // copy kernels reuse what they read and are left alone.
 static void streaming_hints(RenderedKernel *rk) {
   if (rk->klass != KernelClass::ELEMENTWISE && rk->klass != KernelClass::ROW_REDUCE && rk->klass != KernelClass::THREAD_REDUCE) return;
   const double cache = 256.0 * 1048576.0;
-  bool loads = rk->bytes >= cache, stores = loads && rk->bytes_written > cache;
+  // (a row chain over rows too long for its registers reads them once per phase, the second
+  // time from the L2 that the first pass filled: 0.38 -> 0.45 ms with the hint on the
+  // derivative of the loss over 4096 rows of 50 257 logits)
+  bool loads = rk->bytes >= cache && !rk->rereads_inputs, stores = loads && rk->bytes_written > cache;
   if (getenv("POLY_HIP_NO_STREAMING_HINTS")) loads = stores = false;
   if (const char *mode = measurement_env("POLY_HIP_STREAM")) {
     const char *mb = measurement_env("POLY_HIP_STREAM_MB");

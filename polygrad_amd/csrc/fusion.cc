@@ -1066,6 +1066,7 @@ static bool match_row_chain_impl(const Sched &sc, int a_item, const std::vector<
   std::vector<RowCache> cache;
   int n_cached_uses = 0, n_exported = 0;
   bool narrow_stored = false;
+  int n_walked_phases = 0;          // phases that walk their row from memory in a loop (nothing kept for the next one)
   int row_V = 0, row_nit = 0;       // vector width and step count of the rows kept between phases
   std::string row_decls;             // their declarations in the kernel body
   for (size_t pi = 0; pi < phases.size(); pi++) {
@@ -1151,6 +1152,7 @@ static bool match_row_chain_impl(const Sched &sc, int a_item, const std::vector<
     const int nit = (int)((R + (int64_t)G * V - 1) / ((int64_t)G * V));
     // iterations as an unrolled loop over `it` (what is kept between phases is indexed by it)
     const bool unrolled = (G <= 64 && nit <= 4) || (G == 256 && nit <= 8);
+    if (!unrolled) n_walked_phases++;
     {
       bool reads_row = false;
       for (auto &kv : ph.m.preset) if (kv.second.find("[it]") != std::string::npos) reads_row = true;
@@ -1370,6 +1372,7 @@ static bool match_row_chain_impl(const Sched &sc, int a_item, const std::vector<
   }
   rk.n_params = (int)arg_slots.size();
   rk.bytes = bytes - (narrow_stored ? (double)s->buf_slots[g_narrow_store_slot].nbytes / 2 : 0.0);      // (a buffer stored as bf16 values is half written)
+  rk.rereads_inputs = n_walked_phases > 1;
   rk.bytes_written = bytes_written - (narrow_stored ? (double)s->buf_slots[g_narrow_store_slot].nbytes / 2 : 0.0);
   // Candidates for on-device tuning: the same rows on smaller workgroups (fewer rows to a
   // workgroup, more workgroups).  Which lanes add which elements of a row, and in what

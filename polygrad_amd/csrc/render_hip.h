@@ -44,6 +44,7 @@ struct RenderedKernel {
   // Algorithmic work of one launch, for roofline accounting.
   double bytes = 0;        // distinct buffer elements touched * element size
   double bytes_written = 0;   // the part of `bytes` that the kernel stores (0 where a renderer does not say)
+  bool rereads_inputs = false;   // a later phase of the kernel reads from memory what an earlier one read (rows too long to keep)
   double flops = 0;        // 2*M*N*K for matmul-shaped kernels, else 0
   // Guarded fast paths: a small check kernel must succeed for the fast kernel
   // to be valid; otherwise `fallback` runs (always the generic lowering).
