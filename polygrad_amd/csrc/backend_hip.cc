@@ -78,7 +78,7 @@ HipRunner *runner_create(const PolyUOp *root, const char *fn_name, int flags) {
 }
 
 // A kernel that only streams through its buffers and moves more bytes than the caches hold
-// (2 x 4 MiB of L2 per XCD pair aside, the memory-side cache is 256 MiB) reads with the
+// (the 4 MiB L2 of each XCD aside, the memory-side cache is 256 MiB) reads with the
 // nontemporal hint: what it reads once then leaves the caches to what is read again, and
 // the memory system serves the reads at a higher rate (three 256 MiB inputs and one output
 // of that size: 5.3 -> 6.3 TB/s; read-only rows: 6.1 -> 6.9 TB/s).  Its stores get the hint
