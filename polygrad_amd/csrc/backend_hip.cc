@@ -9,6 +9,7 @@
 
 #include "polygrad_hip.h"
 #include "runtime_hip.h"
+#include "templates.h"
 
 // Scratch memory of poly_hip_execute_static: stage-one results of a two-stage kernel go
 // here instead of into memory the runner allocates.  Every GPU the library runs on holds
@@ -93,20 +94,45 @@ static void streaming_hints(RenderedKernel *rk) {
   // time from the L2 that the first pass filled: 0.38 -> 0.45 ms with the hint on the
   // derivative of the loss over 4096 rows of 50 257 logits)
   bool loads = rk->bytes >= cache && !rk->rereads_inputs, stores = loads && rk->bytes_written > cache;
-  if (getenv("POLY_HIP_NO_STREAMING_HINTS")) loads = stores = false;
+  const bool off = getenv("POLY_HIP_NO_STREAMING_HINTS") != nullptr;
+  if (off) loads = stores = false;
+  bool forced = false;
   if (const char *mode = measurement_env("POLY_HIP_STREAM")) {
     const char *mb = measurement_env("POLY_HIP_STREAM_MB");
     const bool big = rk->bytes >= (mb ? atof(mb) : 256.0) * 1048576.0;
     loads = big && strchr(mode, 'L');
     stores = big && strchr(mode, 'S');
+    forced = true;
   }
-  if (!loads && !stores) return;
-  std::string defs;
-  if (loads) defs += "#define POLY_NT_LOADS 1\n";
-  if (stores) defs += "#define POLY_NT_STORES 1\n";
-  rk->source = defs + rk->source;
-  for (RenderedKernel::Variant &v : rk->variants) v.source = defs + v.source;
-  rk->strategy += loads && stores ? ", streaming loads and stores" : loads ? ", streaming loads" : ", streaming stores";
+  struct Form { bool loads, stores; const char *label, *defs, *text; };
+  static const Form forms[] = {{false, false, "nt_none", "", ""},
+                               {true, false, "nt_loads", "#define POLY_NT_LOADS 1\n", ", streaming loads"},
+                               {true, true, "nt_all", "#define POLY_NT_LOADS 1\n#define POLY_NT_STORES 1\n", ", streaming loads and stores"},
+                               {false, true, "nt_stores", "#define POLY_NT_STORES 1\n", ", streaming stores"}};
+  const Form *rule = &forms[0];
+  for (const Form &f : forms) if (f.loads == loads && f.stores == stores) rule = &f;
+  // With the search on, a kernel of a quarter of the cache's size and more also comes in the
+  // other forms (not the stores alone): which one is fastest depends on what the kernels
+  // around it leave in the caches and look for there, and that the timing on the plan's
+  // own buffers sees.  The hint changes no value.
+  std::vector<RenderedKernel::Variant> others;
+  // (a kernel that already carries its final symbol name has no candidates: they are named when chosen)
+  const bool unnamed = rk->source.find(" poly_k(") != std::string::npos;
+  if (matmul_tuning_enabled() && !off && !forced && unnamed && rk->bytes >= cache / 4 && !rk->rereads_inputs) {
+    if (rk->variants.empty()) rk->variants.push_back({"default", rk->source, rk->strategy, rk->launch});
+    for (int fi = 0; fi < 3; fi++) {
+      const Form &f = forms[fi];
+      if (&f == rule) continue;
+      for (const RenderedKernel::Variant &v : rk->variants)
+        others.push_back({v.label == "default" ? std::string(f.label) : v.label + "+" + f.label, f.defs + v.source, v.strategy + f.text, v.launch});
+    }
+  }
+  if (rule != &forms[0]) {
+    rk->source = rule->defs + rk->source;
+    for (RenderedKernel::Variant &v : rk->variants) { v.source = rule->defs + v.source; v.strategy += rule->text; }
+    rk->strategy += rule->text;
+  }
+  for (RenderedKernel::Variant &v : others) rk->variants.push_back(std::move(v));
 }
 
 HipRunner *runner_from_rendered(const RenderedKernel &rk, const char *fn_name, bool named) {

@@ -2,7 +2,7 @@
 src/render_c.c:839; its timing loop and disk cache are src/codegen.c:1012-1195).  The
 candidates: tile shapes and pipelines of the 16-bit matmul templates, tile shapes of the
 fp32 one, the register budget of the attention kernel, the access width of fused pointwise
-kernels.  A tuned plan must give bit-identical results -- no candidate changes the order
+kernels, the workgroup size of row chains, the streaming forms of large bandwidth-bound kernels.  A tuned plan must give bit-identical results -- no candidate changes the order
 in which a value's terms are added -- and remember its decisions."""
 import os
 
@@ -35,10 +35,12 @@ def known_label(l):
     """A decision names the winner: "256x256w4x2p2" (16-bit template that stages through
     registers), "128x256x32w2x2s3g2" (the one that loads straight into LDS), "f32_128x64w2x2"
     (fp32 template), "attn_occ2" (attention, waves per SIMD), "pw_vec2" (fused pointwise
-    kernels, elements per access), "rows_wg64" (row chains, threads per workgroup), or keeps
-    the default."""
+    kernels, elements per access), "rows_wg64" (row chains, threads per workgroup), "nt_loads"
+    (a streaming kernel's accesses, alone or behind one of the two before), or keeps the
+    default."""
     import re
-    return bool(re.fullmatch(r"default|\d+x\d+w\dx\dp\d|\d+x\d+x\d+w\dx\ds\dg\d|f32_\d+x\d+w\dx\d|attn_occ\d|pw_vec\d+|rows_wg\d+", l))
+    nt = r"nt_(none|loads|all)"      # a kernel that streams through a quarter of the memory-side cache and more: plain, nontemporal loads, loads and stores
+    return bool(re.fullmatch(r"default|\d+x\d+w\dx\dp\d|\d+x\d+x\d+w\dx\ds\dg\d|f32_\d+x\d+w\dx\d|attn_occ\d|(pw_vec\d+|rows_wg\d+)(\+%s)?|%s" % (nt, nt), l))
 
 
 @pytest.mark.parametrize("name,out_name", [("matmul_bf16_b16_1024x1024x1024", "C"), ("gpt2_small_bf16_b1_t1024", "output")])
@@ -101,3 +103,24 @@ def test_fp32_products_and_attention_are_tuned_too(tmp_path, monkeypatch):
         labels = [open(cache / f).read().strip() for f in os.listdir(cache) if f.endswith(".tune")]
         assert labels and all(known_label(l) for l in labels), labels
         assert any(l == "default" or l.startswith(prefix) for l in labels), labels
+
+
+def test_streaming_forms_are_candidates_and_change_no_bit(tmp_path, monkeypatch):
+    """The softmax over 8192 rows of 8192 (1 GiB moved) is timed with plain accesses, with
+    nontemporal loads and with nontemporal loads and stores; whichever wins, the result is
+    the untuned one bit for bit, and the decision is one of the three."""
+    import torch
+    name = "rowops_f32_8192_softmax"
+    make = lambda plan: random_slot_tensors(plan, seed=1)
+    monkeypatch.setenv("POLY_HIP_CACHE_DIR", str(tmp_path / "cache"))
+    monkeypatch.delenv("POLY_BEAM", raising=False)
+    want, descs = run_plan(name, make, "softmax")
+    assert any("streaming loads" in d for d in descs), descs
+    monkeypatch.setenv("POLY_BEAM", "1")
+    got, tuned = run_plan(name, make, "softmax")
+    assert torch.isfinite(want).all() and torch.equal(got.view(torch.uint8), want.view(torch.uint8))
+    labels = [open(tmp_path / "cache" / f).read().strip() for f in os.listdir(tmp_path / "cache") if f.endswith(".tune")]
+    assert len(labels) == 1 and (labels[0] == "default" or labels[0] in ("nt_none", "nt_all")), labels
+    again, again_descs = run_plan(name, make, "softmax")
+    assert torch.equal(again.view(torch.uint8), want.view(torch.uint8))
+    assert [d.split(" ", 1)[1] for d in again_descs] == [d.split(" ", 1)[1] for d in tuned]
