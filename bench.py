@@ -44,6 +44,11 @@ MEASURED_TRAFFIC = {
     "matmul-mfma: mfma 32x32x16 bf16 M=8192 N=768 K=3072 Z=1 tile 128x128x64 A:k-major B:n-major, operands straight into LDS: 4 waves, 2 stages, 2 per CU, 64 workgroups read B ahead": 103.8e6 + 12.8e6,
     "matmul-mfma: mfma 32x32x16 bf16 M=8192 N=768 K=768 Z=1 tile 128x128x64 A:k-major B:n-major, operands straight into LDS: 4 waves, 2 stages, 2 per CU, 32 workgroups read B ahead": 34.8e6 + 12.7e6,
     "matmul-mfma: mfma 32x32x16 bf16 M=8192 N=50257 K=768 Z=1 tile 192x128x64 A:k-major B:k-major, operands straight into LDS: 4 waves, 2 stages, 2 per CU, 64 workgroups read B ahead": 1106.5e6 + 849.1e6,
+    # the same two counters for `--workload rowops_f32_8192_{softmax,layernorm,sum,max} --steps 2 --warmup 1` and `--workload adamw_f32_355m`
+    # (sum and max are the same kernel but for the combining operation)
+    "row-reduce: row chain of 4 kernels (reduce vec4, map vec4, reduce vec4, map vec4) G=256 R=8192 rows=8192, 3 row loads kept in registers, intermediate rows kept in registers, streaming loads": 393310 * 2048.0 + 262144 * 1024.0,
+    "row-reduce: row-reduce G=256 vec4 R=8192 rows=8192, streaming loads": 393230 * 2048.0 + 257 * 1024.0,
+    "elementwise: 4 pointwise kernels over the same 354823168 positions as one, vec1, 1 buffers never written out, streaming loads and stores": 2772070 * 2048.0 + 4158090 * 1024.0,
     # the same two counters for `--workload gpt2_medium_train_24l_b4_t1024 --steps 1 --warmup 1`
     "row-reduce: row chain of 4 kernels (reduce vec4, map vec4, reduce vec4, map vec4) G=64 R=1024 rows=65536, 3 row loads kept in registers, intermediate rows kept in registers, result stored as the bf16 values that its fp32 values are casts of": 411.2e6 + 134.2e6,
 }
